@@ -1,0 +1,145 @@
+/*
+ * C ABI of the MI355X execution library for the vpux hot path: ACT-SHAVE software kernels and
+ * the NCE/DPU quantized convolution / matmul with the integer PPE.
+ *
+ * Every entry point takes plain pointers and sizes, is asynchronous on the caller's HIP stream
+ * (passed as void*, NULL = default stream), is safe to call from several host threads and owns
+ * no caller buffer.  Return values follow the reference's compiler C API
+ * (src/vpux_driver_compiler/include/npu_driver_compiler.h:94-103); the text of the last failure
+ * on the calling thread is available from vpx_get_last_error (the role of
+ * vclLogHandleGetString, npu_driver_compiler.h:287).
+ */
+#ifndef VPX_RUNTIME_H_
+#define VPX_RUNTIME_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "vpx_sw_params.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define VPX_API __attribute__((visibility("default")))
+#else
+#define VPX_API
+#endif
+
+/* Same numeric values as vcl_result_t (npu_driver_compiler.h:94-103). */
+typedef enum vpx_result_t {
+    VPX_RESULT_SUCCESS = 0,
+    VPX_RESULT_ERROR_OUT_OF_MEMORY = 0x70000002,
+    VPX_RESULT_ERROR_UNSUPPORTED_FEATURE = 0x78000003,
+    VPX_RESULT_ERROR_INVALID_ARGUMENT = 0x78000004,
+    VPX_RESULT_ERROR_INVALID_NULL_HANDLE = 0x78000005,
+    VPX_RESULT_ERROR_UNKNOWN = 0x7ffffffe
+} vpx_result_t;
+
+/* Text of the last error returned to the calling thread ("" when none). */
+VPX_API const char* vpx_get_last_error(void);
+
+/* Library version: major << 16 | minor. */
+VPX_API uint32_t vpx_get_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Boundary A: ACT-SHAVE software kernels.
+ *
+ * Replaces the firmware call `entry(paramsPtr)` made by the ACT-SHAVE management kernel for a
+ * VpuActKernelInvocation (src/vpux_compiler/src/dialect/VPUMI37XX/ops/act_kernel_invo.cpp:21-48).
+ * `entry` is the kernel's ELF stem as chosen by SwKernelOp::getKernelInfo
+ * (src/vpux_compiler/src/dialect/VPUIP/IR/ops/sw_kernel.cpp); `params` is the byte blob the
+ * compiler serialises for that kernel (layout in vpx_sw_params.h) and is read on the host during
+ * the call.  addrs[i] carries the 64-bit device address of memref i (inputs first, then outputs),
+ * which on the NPU firmware relocation would have patched into MemRefData::dataAddr.  dims and
+ * strides may be NULL: they are then read from the tail of the blob, where
+ * KernelParamsOp::serialize appends them (VPUMI37XX/ops/kernel_params.cpp:19-73).
+ * ------------------------------------------------------------------------------------------ */
+typedef struct vpx_memref_addr_t {
+    void* data;             /* device memory */
+    const int32_t* dims;    /* host memory, innermost first, or NULL */
+    const int64_t* strides; /* host memory, bits, innermost first, or NULL */
+} vpx_memref_addr_t;
+
+VPX_API int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_size,
+                                 const vpx_memref_addr_t* addrs, uint32_t num_addrs, void* stream);
+
+/* 1 when `entry` names a kernel this library implements, else 0. */
+VPX_API int vpx_sw_kernel_supported(const char* entry);
+
+/* Number of implemented entries; name of entry i (NULL when out of range). */
+VPX_API uint32_t vpx_sw_kernel_count(void);
+VPX_API const char* vpx_sw_kernel_name(uint32_t i);
+
+/* ------------------------------------------------------------------------------------------
+ * Boundary B: NCE cluster task (DPU).
+ *
+ * Replaces one VPUIP.NCEClusterTask of task_type CONV
+ * (src/vpux_compiler/tblgen/vpux/compiler/dialect/VPUIP/ops.td:651-750), the form
+ * VPU.NCE.Convolution and VPU.NCE.MatMul lower to (tblgen/.../VPU/ops.td:138-357).
+ *   input   NHWC  [N][H][W][IC]   u8 or i8
+ *   weights OYXI  [OC][KY][KX][IC] u8 or i8, one dense set per output channel
+ *   weight_table [OC][4] int32 as built by NCESparsity::getWeightsTable
+ *       (src/vpux_compiler/src/dialect/VPU/utils/nce_sparsity.cpp:195-231): word 2 holds
+ *       mult << 16 | shift << 8, word 3 the int32 bias
+ *       (src/vpux_compiler/src/NPU37XX/dialect/VPU/impl/nce_sparsity_converters.cpp:14-41);
+ *       words 0 and 1 (weight / sparsity pointers) are NPU addresses and are ignored
+ *   output  NHWC  [N][OH][OW][OC] u8 or i8
+ * A matmul A[M][K] x B[N][K] -> [M][N] is the task N=1, H=M, W=1, IC=K, OC=N, 1x1 kernel.
+ * Arithmetic: acc = sum (in - zp_in) * (w - zp_w) over the taps inside the image (padding adds 0),
+ * then the integer PPE in the order the compiler programs it
+ * (src/vpux_compiler/src/NPU40XX/dialect/VPUIPDPU/transforms/passes/expand_dpu_config/
+ * expand_dpu_config_invariant_ppe.cpp:322-380): t = (acc + bias) * mult; if t < 0 then
+ * t *= prelu_mult and shift += prelu_shift; r = round_half_even(t / 2^shift) + zp_out;
+ * clamp to [clamp_low, clamp_high]; saturate to the output type.
+ * ------------------------------------------------------------------------------------------ */
+
+/* VPUIP::NCETaskType (tblgen/.../VPUIP/attributes.td:56-70) */
+typedef enum vpx_nce_task_type_t { VPX_NCE_CONV = 0 } vpx_nce_task_type_t;
+
+/* VPU::PPEMode values used by the integer pipeline (tblgen/.../VPU/attributes.td:327-369) */
+typedef enum vpx_ppe_mode_t {
+    VPX_PPE_NOOP = 3,
+    VPX_PPE_LRELU = 13,
+    VPX_PPE_LRELUX = 14,
+    VPX_PPE_LPRELU = 15
+} vpx_ppe_mode_t;
+
+/* The PPEIntAttr fields the integer convolution path consumes (attributes.td:399-430). */
+typedef struct vpx_ppe_int_t {
+    int32_t mode; /* vpx_ppe_mode_t */
+    int32_t clamp_low;
+    int32_t clamp_high;
+    int32_t lrelu_mult;
+    int32_t lrelu_shift;
+} vpx_ppe_int_t;
+
+typedef struct vpx_nce_task_t {
+    int32_t task_type; /* vpx_nce_task_type_t */
+    const void* input;
+    const void* weights;
+    const int32_t* weight_table;
+    void* output;
+    int32_t input_type;   /* VPX_NN_U8 or VPX_NN_I8 */
+    int32_t weights_type; /* VPX_NN_U8 or VPX_NN_I8 */
+    int32_t output_type;  /* VPX_NN_U8 or VPX_NN_I8 */
+    int64_t N, H, W, IC;  /* input shape */
+    int64_t OC;
+    int32_t kernel_size[2];    /* KY, KX */
+    int32_t kernel_strides[2]; /* SY, SX */
+    int32_t kernel_padding[4]; /* left, right, top, bottom (VPU_PaddingAttr order) */
+    int32_t zp_in, zp_w, zp_out;
+    vpx_ppe_int_t ppe;
+} vpx_nce_task_t;
+
+VPX_API int vpx_nce_task(const vpx_nce_task_t* task, void* stream);
+
+/* Name of the device kernel the last successful vpx_nce_task on this thread dispatched to
+ * ("" before the first); for tests and profiles. */
+VPX_API const char* vpx_nce_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,289 @@
+"""ctypes view of the CPU oracle (oracle/vpx_oracle.c) -- TEST INFRASTRUCTURE ONLY.
+
+Only tests, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import
+this package.  The product package never does.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libvpx_oracle.so")
+_REF_PATH = os.path.join(_HERE, "_ref", "libref_float16.so")
+
+
+def build(force=False):
+    """Compile the oracle (and oracle/_ref when the reference checkout is present)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-B", "-C", _HERE, "all"])
+
+
+class _PPE(C.Structure):
+    _fields_ = [("prelu_mult", C.c_int32), ("prelu_shift", C.c_int32), ("zp_out", C.c_int32),
+                ("clamp_low", C.c_int32), ("clamp_high", C.c_int32)]
+
+
+class _Conv(C.Structure):
+    _fields_ = [(n, C.c_int64) for n in ("N", "H", "W", "IC", "OC", "KY", "KX", "stride_y", "stride_x", "pad_top",
+                                          "pad_left", "pad_bottom", "pad_right")] + \
+               [(n, C.c_int32) for n in ("in_signed", "w_signed", "out_signed", "zp_in", "zp_w")] + [("ppe", _PPE)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = C.CDLL(_LIB_PATH)
+        L.orc_f32_to_f16.restype = C.c_uint16
+        L.orc_f32_to_f16.argtypes = [C.c_float]
+        L.orc_f16_to_f32.restype = C.c_float
+        L.orc_f16_to_f32.argtypes = [C.c_uint16]
+        L.orc_fake_quantize.restype = C.c_float
+        L.orc_fake_quantize.argtypes = [C.c_float] * 6
+        L.orc_dequantize_value.restype = C.c_float
+        L.orc_dequantize_value.argtypes = [C.c_int64, C.c_double, C.c_int64]
+        L.orc_quantize_value.restype = C.c_int64
+        L.orc_quantize_value.argtypes = [C.c_double, C.c_double, C.c_int64, C.c_int64, C.c_int64]
+        L.orc_approximate.restype = C.c_int
+        L.orc_approximate.argtypes = [C.c_int, C.c_double] + [C.POINTER(C.c_int64)] * 3
+        L.orc_wt_pack_scale.restype = C.c_int32
+        L.orc_wt_pack_scale.argtypes = [C.c_uint8, C.c_int16]
+        L.orc_ppe_requant.restype = C.c_int32
+        L.orc_ppe_requant.argtypes = [C.c_int32] * 4 + [C.POINTER(_PPE)]
+        L.orc_num_threads.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def ref_lib():
+    """The reference's own float16.cpp compiled in place (None when it was not built)."""
+    if not os.path.exists(_REF_PATH):
+        return None
+    L = C.CDLL(_REF_PATH)
+    L.ref_f32_to_f16.restype = C.c_uint16
+    L.ref_f32_to_f16.argtypes = [C.c_float]
+    L.ref_f16_to_f32.restype = C.c_float
+    L.ref_f16_to_f32.argtypes = [C.c_uint16]
+    L.ref_f16_add.restype = C.c_uint16
+    L.ref_f16_add.argtypes = [C.c_uint16, C.c_uint16]
+    return L
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _i64(seq):
+    return (C.c_int64 * len(seq))(*[int(v) for v in seq])
+
+
+def set_num_threads(n):
+    lib().orc_set_num_threads(C.c_int(n))
+
+
+def num_threads():
+    return lib().orc_num_threads()
+
+
+# ---- fp16 ----------------------------------------------------------------------------------
+
+def f32_to_f16(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().orc_convert_f32_to_f16(_p(x), _p(out), C.c_size_t(x.size))
+    return out
+
+
+def f16_to_f32(h):
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, dtype=np.float32)
+    lib().orc_convert_f16_to_f32(_p(h), _p(out), C.c_size_t(h.size))
+    return out
+
+
+# ---- elementwise -----------------------------------------------------------------------------
+
+def fake_quantize_f16(x, in_lo, in_hi, out_lo, out_hi, levels):
+    """x and limits are uint16 (fp16 bit patterns) arrays of equal rank; limits broadcast NUMPY style."""
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    lims = [np.ascontiguousarray(l, dtype=np.uint16) for l in (in_lo, in_hi, out_lo, out_hi)]
+    rank = x.ndim
+    lims = [l.reshape((1,) * (rank - l.ndim) + l.shape) for l in lims]
+    y = np.empty_like(x)
+    ptrs = (C.c_void_p * 4)(*[l.ctypes.data for l in lims])
+    lim_dims = _i64([d for l in lims for d in l.shape])
+    lib().orc_fake_quantize_f16(_p(x), _p(y), C.c_int(rank), _i64(x.shape), ptrs, lim_dims, C.c_int64(levels))
+    return y
+
+
+def _axis_view(shape, axis):
+    if axis is None:
+        return 1, 1, int(np.prod(shape, dtype=np.int64))
+    outer = int(np.prod(shape[:axis], dtype=np.int64))
+    inner = int(np.prod(shape[axis + 1:], dtype=np.int64))
+    return outer, int(shape[axis]), inner
+
+
+def quantize(x, scales, zps, signed, qmin=None, qmax=None, axis=None):
+    """x: uint16 (fp16 bits) or float32 array -> int8/uint8 (createQuantizeFn semantics)."""
+    scales = np.atleast_1d(np.asarray(scales, dtype=np.float64))
+    zps = np.atleast_1d(np.asarray(zps, dtype=np.int64))
+    if qmin is None:
+        qmin = -128 if signed else 0
+    if qmax is None:
+        qmax = 127 if signed else 255
+    outer, ax, inner = _axis_view(x.shape, axis)
+    assert ax == scales.size == zps.size
+    q = np.empty(x.shape, dtype=np.int8 if signed else np.uint8)
+    if x.dtype == np.uint16:
+        fn = lib().orc_quantize_f16
+    else:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        fn = lib().orc_quantize_f32
+    x = np.ascontiguousarray(x)
+    fn(_p(x), _p(q), C.c_int(int(signed)), C.c_int64(outer), C.c_int64(ax), C.c_int64(inner), _p(scales), _p(zps),
+       C.c_int64(qmin), C.c_int64(qmax))
+    return q
+
+
+def dequantize(q, scales, zps, to_f16=True, axis=None):
+    scales = np.atleast_1d(np.asarray(scales, dtype=np.float64))
+    zps = np.atleast_1d(np.asarray(zps, dtype=np.int64))
+    q = np.ascontiguousarray(q)
+    signed = q.dtype == np.int8
+    outer, ax, inner = _axis_view(q.shape, axis)
+    assert ax == scales.size == zps.size
+    if to_f16:
+        y = np.empty(q.shape, dtype=np.uint16)
+        lib().orc_dequantize_f16(_p(q), C.c_int(int(signed)), _p(y), C.c_int64(outer), C.c_int64(ax), C.c_int64(inner),
+                                 _p(scales), _p(zps))
+    else:
+        y = np.empty(q.shape, dtype=np.float32)
+        lib().orc_dequantize_f32(_p(q), C.c_int(int(signed)), _p(y), C.c_int64(outer), C.c_int64(ax), C.c_int64(inner),
+                                 _p(scales), _p(zps))
+    return y
+
+
+ELT_OPS = {"add": 0, "sub": 1, "mul": 2, "min": 3, "max": 4, "div": 5}
+
+
+def eltwise_f16(op, a, b):
+    a = np.ascontiguousarray(a, dtype=np.uint16)
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    rank = max(a.ndim, b.ndim)
+    a = a.reshape((1,) * (rank - a.ndim) + a.shape)
+    b = b.reshape((1,) * (rank - b.ndim) + b.shape)
+    shape = tuple(max(x, y) for x, y in zip(a.shape, b.shape))
+    y = np.empty(shape, dtype=np.uint16)
+    lib().orc_eltwise_f16(C.c_int(ELT_OPS[op]), _p(a), _p(b), _p(y), C.c_int(rank), _i64(shape), _i64(a.shape),
+                          _i64(b.shape))
+    return y
+
+
+# ---- reductions --------------------------------------------------------------------------------
+
+def softmax_f16(x, axis, pad=0):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    outer, ax, inner = _axis_view(x.shape, axis % x.ndim)
+    y = np.empty_like(x)
+    lib().orc_softmax_f16(_p(x), _p(y), C.c_int64(outer), C.c_int64(ax), C.c_int64(inner), C.c_int64(pad))
+    return y
+
+
+def softmax_f32(x, axis, pad=0):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    outer, ax, inner = _axis_view(x.shape, axis % x.ndim)
+    y = np.empty_like(x)
+    lib().orc_softmax_f32(_p(x), _p(y), C.c_int64(outer), C.c_int64(ax), C.c_int64(inner), C.c_int64(pad))
+    return y
+
+
+def mvn_f16(x, across_channels, normalize_variance, eps, layout="NCHW"):
+    """x: uint16 array, 4-D in memory order given by layout ("NCHW" or "NHWC")."""
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    y = np.empty_like(x)
+    if layout == "NCHW":
+        N, Cc, H, W = x.shape
+        sn, sc, ss = Cc * H * W, H * W, 1
+    elif layout == "NHWC":
+        N, H, W, Cc = x.shape
+        sn, sc, ss = H * W * Cc, 1, Cc
+    else:
+        raise ValueError(layout)
+    lib().orc_mvn_f16(_p(x), _p(y), C.c_int64(N), C.c_int64(Cc), C.c_int64(H * W), C.c_int64(sn), C.c_int64(sc),
+                      C.c_int64(ss), C.c_int(int(across_channels)), C.c_int(int(normalize_variance)), C.c_float(eps))
+    return y
+
+
+# ---- integer path --------------------------------------------------------------------------------
+
+def approximate(bits, target):
+    m, s, p = C.c_int64(), C.c_int64(), C.c_int64()
+    rc = lib().orc_approximate(C.c_int(bits), C.c_double(target), C.byref(m), C.byref(s), C.byref(p))
+    if rc != 0:
+        raise OverflowError(target)
+    return m.value, s.value, p.value
+
+
+def wt_pack_scale(shift, mult):
+    return lib().orc_wt_pack_scale(C.c_uint8(shift), C.c_int16(mult))
+
+
+def make_weights_table(mults, shifts, biases, weight_step):
+    """[OC,4] int32 table as NCESparsity::getWeightsTable lays it out (nce_sparsity.cpp:195-231)."""
+    oc = len(mults)
+    wt = np.zeros((oc, 4), dtype=np.int32)
+    wt[:, 0] = np.arange(oc, dtype=np.int64) * weight_step
+    wt[:, 1] = 0xFFFFFF
+    wt[:, 2] = [wt_pack_scale(int(s), int(m)) for m, s in zip(mults, shifts)]
+    wt[:, 3] = biases
+    return wt
+
+
+def ppe(prelu_mult=1, prelu_shift=0, zp_out=0, clamp_low=-(2 ** 31), clamp_high=2 ** 31 - 1):
+    return _PPE(prelu_mult, prelu_shift, zp_out, clamp_low, clamp_high)
+
+
+def ppe_requant(acc, bias, mult, shift, p):
+    return lib().orc_ppe_requant(C.c_int32(acc), C.c_int32(bias), C.c_int32(mult), C.c_int32(shift), C.byref(p))
+
+
+def nce_conv(inp, w, wt, p, zp_in=0, zp_w=0, strides=(1, 1), pads=(0, 0, 0, 0), out_signed=False, rows=None,
+             want_acc=False):
+    """inp NHWC int8/uint8, w [OC,KY,KX,IC] int8/uint8, wt [OC,4] int32; pads = (top,left,bottom,right).
+
+    rows=(row0,nrows) computes only those flattened output rows (the rest of the result is zero)."""
+    inp = np.ascontiguousarray(inp)
+    w = np.ascontiguousarray(w)
+    wt = np.ascontiguousarray(wt, dtype=np.int32)
+    N, H, W, IC = inp.shape
+    OC, KY, KX, IC2 = w.shape
+    assert IC == IC2
+    d = _Conv(N, H, W, IC, OC, KY, KX, strides[0], strides[1], pads[0], pads[1], pads[2], pads[3],
+              int(inp.dtype == np.int8), int(w.dtype == np.int8), int(out_signed), zp_in, zp_w, p)
+    OH = (H + pads[0] + pads[2] - KY) // strides[0] + 1
+    OW = (W + pads[1] + pads[3] - KX) // strides[1] + 1
+    out = np.zeros((N, OH, OW, OC), dtype=np.int8 if out_signed else np.uint8)
+    acc = np.zeros((N, OH, OW, OC), dtype=np.int32) if want_acc else None
+    row0, nrows = rows if rows is not None else (0, N * OH * OW)
+    lib().orc_nce_conv_rows(C.byref(d), _p(inp), _p(w), _p(wt), _p(out), _p(acc) if want_acc else None,
+                            C.c_int64(row0), C.c_int64(nrows))
+    return (out, acc) if want_acc else out
+
+
+def nce_matmul(a, b_nk, wt, p, zp_a=0, zp_b=0, out_signed=True, rows=None, want_acc=False):
+    """A [M,K] x B stored [N,K] -> [M,N]: the 1x1-convolution form NCE.MatMul lowers to (ops.td:228-357)."""
+    M, K = a.shape
+    Nn, K2 = b_nk.shape
+    assert K == K2
+    r = nce_conv(a.reshape(1, M, 1, K), b_nk.reshape(Nn, 1, 1, K), wt, p, zp_in=zp_a, zp_w=zp_b,
+                 out_signed=out_signed, rows=rows, want_acc=want_acc)
+    if want_acc:
+        return r[0].reshape(M, Nn), r[1].reshape(M, Nn)
+    return r.reshape(M, Nn)

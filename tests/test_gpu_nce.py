@@ -1,0 +1,202 @@
+"""Bit-exact parity of the NCE task (int8 convolution / matmul + integer PPE) with the CPU oracle,
+through the C ABI, on a real MI355X."""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def dev_t(a, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0, zp_out=0, strides=(1, 1),
+             pads=(0, 0, 0, 0), out_signed=False, mode=None, force=None, rows=None):
+    """pads = (left, right, top, bottom).  Returns (gpu_out, oracle_out, kernel_name)."""
+    import torch
+    OC, KY, KX, IC = w.shape
+    wt = rt.make_weights_table(mults, shifts, bias, KY * KX * IC)
+    assert np.array_equal(wt, orc.make_weights_table(mults, shifts, bias, KY * KX * IC))
+    mode = mode if mode is not None else rt.PPE_NOOP
+    p = rt.PpeInt(mode, ppe_kw["clamp_low"], ppe_kw["clamp_high"], ppe_kw.get("lrelu_mult", 1), ppe_kw.get("lrelu_shift", 0))
+    pm, ps = {rt.PPE_NOOP: (1, 0), rt.PPE_LRELU: (0, 0), rt.PPE_LRELUX: (0, 0),
+              rt.PPE_LPRELU: (p.lrelu_mult, p.lrelu_shift)}[mode]
+    op = orc.ppe(pm, ps, zp_out, p.clamp_low, p.clamp_high)
+    N, H, W, _ = inp.shape
+    OH = (H + pads[2] + pads[3] - KY) // strides[0] + 1
+    OW = (W + pads[0] + pads[1] - KX) // strides[1] + 1
+    out = torch.full((N, OH, OW, OC), 77, dtype=torch.int8 if out_signed else torch.uint8, device=dev)
+    old = os.environ.pop("VPX_NCE_KERNEL", None)
+    if force:
+        os.environ["VPX_NCE_KERNEL"] = force
+    try:
+        rt.nce_task(dev_t(inp, dev), dev_t(w, dev), dev_t(wt, dev), out, p, zp_in=zp_in, zp_w=zp_w, zp_out=zp_out,
+                    strides=strides, pads=pads)
+        torch.cuda.synchronize()
+    finally:
+        os.environ.pop("VPX_NCE_KERNEL", None)
+        if old is not None:
+            os.environ["VPX_NCE_KERNEL"] = old
+    want = orc.nce_conv(inp, w, wt, op, zp_in=zp_in, zp_w=zp_w, strides=strides,
+                        pads=(pads[2], pads[0], pads[3], pads[1]), out_signed=out_signed, rows=rows)
+    return out.cpu().numpy(), want, rt.nce_last_kernel()
+
+
+def rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=True, w_u8=False, shift_lo=12, shift_hi=20):
+    inp = rng.integers(0, 256, (N, H, W, IC), dtype=np.uint8) if in_u8 else rng.integers(-128, 128, (N, H, W, IC)).astype(np.int8)
+    w = rng.integers(0, 256, (OC, KY, KX, IC), dtype=np.uint8) if w_u8 else rng.integers(-127, 128, (OC, KY, KX, IC)).astype(np.int8)
+    mults = rng.integers(2 ** 14, 2 ** 15, OC)
+    shifts = rng.integers(shift_lo, shift_hi, OC)
+    bias = rng.integers(-2 ** 15, 2 ** 15, OC).astype(np.int32)
+    return inp, w, mults, shifts, bias
+
+
+U8 = {"clamp_low": 0, "clamp_high": 255}
+I8 = {"clamp_low": -128, "clamp_high": 127}
+
+
+@pytest.mark.parametrize("force,expect", [(None, "nce_conv_mfma"), ("naive", "nce_conv_naive")])
+@pytest.mark.parametrize("geom", [
+    dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
+    dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)),
+    dict(N=3, H=8, W=5, IC=64, OC=70, KY=1, KX=3, strides=(1, 1), pads=(1, 0, 0, 0)),
+    dict(N=1, H=20, W=20, IC=64, OC=32, KY=5, KX=5, strides=(1, 2), pads=(2, 2, 2, 2)),
+])
+def test_conv_paths(rt, orc, dev, geom, force, expect):
+    g = dict(geom)
+    strides, pads = g.pop("strides"), g.pop("pads")
+    rng = np.random.default_rng(50 + g["H"])
+    for in_u8, zp_in, out_signed in ((True, 128, False), (True, 7, True), (False, -5, False), (False, 0, True)):
+        inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, **g)
+        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, I8 if out_signed else U8, zp_in=zp_in,
+                                   strides=strides, pads=pads, out_signed=out_signed, force=force)
+        assert name == expect
+        assert np.array_equal(got, want), "%s zp_in=%d: %d mismatches" % (name, zp_in, int((got != want).sum()))
+
+
+def test_naive_path_covers_odd_shapes_and_weight_zero_points(rt, orc, dev):
+    rng = np.random.default_rng(60)
+    inp, w, mults, shifts, bias = rand_case(rng, 2, 6, 7, 5, 9, 3, 2, in_u8=True, w_u8=True)
+    got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, U8, zp_in=100, zp_w=120, zp_out=10,
+                               strides=(1, 1), pads=(1, 0, 1, 0))
+    assert name == "nce_conv_naive" and np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("M,K,N", [(256, 64, 256), (300, 128, 520), (1, 64, 1), (513, 256, 77), (1024, 512, 768)])
+def test_matmul_gemm_path(rt, orc, dev, M, K, N):
+    rng = np.random.default_rng(70 + M)
+    for in_u8, zp in ((False, 3), (True, 128), (False, 0), (True, 11)):
+        a = rng.integers(0, 256, (M, K), dtype=np.uint8) if in_u8 else rng.integers(-128, 128, (M, K)).astype(np.int8)
+        b = rng.integers(-127, 128, (N, K)).astype(np.int8)
+        mults = rng.integers(2 ** 14, 2 ** 15, N)
+        shifts = rng.integers(18, 24, N)
+        bias = rng.integers(-2 ** 15, 2 ** 15, N).astype(np.int32)
+        kw = dict(I8, lrelu_mult=1638, lrelu_shift=14)
+        got, want, name = run_task(rt, orc, dev, a.reshape(1, M, 1, K), b.reshape(N, 1, 1, K), mults, shifts, bias, kw,
+                                   zp_in=zp, out_signed=True, mode=rt.PPE_LPRELU)
+        assert name == "nce_gemm_mfma"
+        assert np.array_equal(got, want), "M=%d K=%d N=%d zp=%d: %d mismatches" % (M, K, N, zp, int((got != want).sum()))
+
+
+@pytest.mark.parametrize("mode", ["NOOP", "LRELU", "LRELUX", "LPRELU"])
+def test_ppe_modes_and_rounding_edges(rt, orc, dev, mode):
+    """Accumulators chosen to land on ties, on both signs, with shifts from 0 to 40 and output zero points."""
+    rng = np.random.default_rng(80)
+    M, K, N = 256, 64, 256
+    a = rng.integers(-4, 5, (M, K)).astype(np.int8)
+    b = rng.integers(-4, 5, (N, K)).astype(np.int8)
+    mults = np.where(np.arange(N) % 3 == 0, 1 << 14, rng.integers(2 ** 14, 2 ** 15, N))
+    shifts = np.arange(N) % 41
+    bias = rng.integers(-64, 64, N).astype(np.int32)
+    md = getattr(rt, "PPE_" + mode)
+    kw = dict(clamp_low=-100, clamp_high=90, lrelu_mult=1638 if mode == "LPRELU" else 1, lrelu_shift=14 if mode == "LPRELU" else 0)
+    got, want, _ = run_task(rt, orc, dev, a.reshape(1, M, 1, K), b.reshape(N, 1, 1, K), mults, shifts, bias, kw, zp_in=1,
+                            zp_out=-7, out_signed=True, mode=md)
+    assert np.array_equal(got, want)
+    assert got.min() >= -100 and got.max() <= 90
+
+
+def test_conv_config_c4_full_size(rt, orc, dev):
+    from vpux_plugin_amd import configs
+    c = configs.c4_conv()
+    got, want, name = run_task(rt, orc, dev, c["input"], c["weights"], c["mult"], c["shift"], c["bias"],
+                               {"clamp_low": c["clamp"][0], "clamp_high": c["clamp"][1]}, zp_in=c["zp_in"],
+                               strides=c["strides"], pads=c["pads"])
+    assert name == "nce_conv_mfma"
+    assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
+    assert 0 < (got == 0).mean() < 0.9  # the ReLU clamp is active and the output is not saturated flat
+
+
+def test_matmul_config_c5_full_size_and_chain(rt, orc, dev):
+    """Full [4096x4096]x[4096x11008]: the MFMA result is compared bit for bit with the naive device path
+    over the whole tensor and with the CPU oracle on sampled rows; then Dequantize and the fp16 Add."""
+    import torch
+    from vpux_plugin_amd import configs
+    c = configs.c5_matmul()
+    M, K = c["a"].shape
+    N = c["b_nk"].shape[0]
+    wt = rt.make_weights_table(c["mult"], c["shift"], c["bias"], K)
+    p = rt.PpeInt(rt.PPE_LPRELU, c["clamp"][0], c["clamp"][1], c["lrelu_mult"], c["lrelu_shift"])
+    a, b, wtd = dev_t(c["a"], dev), dev_t(c["b_nk"], dev), dev_t(wt, dev)
+    out = torch.empty((M, N), dtype=torch.int8, device=dev)
+    rt.nce_matmul(a, b, wtd, out, p, zp_a=c["zp_a"], zp_out=c["zp_out"])
+    assert rt.nce_last_kernel() == "nce_gemm_mfma"
+    out2 = torch.empty_like(out)
+    os.environ["VPX_NCE_KERNEL"] = "naive"
+    try:
+        rt.nce_matmul(a, b, wtd, out2, p, zp_a=c["zp_a"], zp_out=c["zp_out"])
+        assert rt.nce_last_kernel() == "nce_conv_naive"
+    finally:
+        del os.environ["VPX_NCE_KERNEL"]
+    torch.cuda.synchronize()
+    assert bool((out == out2).all())
+    rows = np.sort(np.random.default_rng(90).choice(M, 24, replace=False))
+    op = orc.ppe(c["lrelu_mult"], c["lrelu_shift"], c["zp_out"], *c["clamp"])
+    want = orc.nce_matmul(np.ascontiguousarray(c["a"][rows]), c["b_nk"], wt, op, zp_a=c["zp_a"])
+    got = out.cpu().numpy()
+    assert np.array_equal(got[rows], want)
+    hist = np.bincount(got.astype(np.int64).ravel() + 128, minlength=256)
+    assert hist[0] / got.size < 0.05 and hist[255] / got.size < 0.05 and (hist > 0).sum() > 100  # spans i8
+    # C5 chain: Dequantize to fp16, then fp16 Add of the residual
+    deq = torch.empty((M, N), dtype=torch.float16, device=dev)
+    rt.dequantize(out, deq, c["deq_scale"], c["deq_zp"])
+    res = dev_t(c["residual"].view(np.float16), dev)
+    y = torch.empty_like(deq)
+    rt.eltwise("add", deq, res, y)
+    torch.cuda.synchronize()
+    shipped = float(orc.f16_to_f32(orc.f32_to_f16(np.array([c["deq_scale"]], np.float32)))[0])
+    wd = orc.dequantize(got[rows], shipped, c["deq_zp"])
+    assert np.array_equal(deq.cpu().numpy().view(np.uint16)[rows], wd)
+    wy = orc.eltwise_f16("add", wd, c["residual"][rows])
+    assert np.array_equal(y.cpu().numpy().view(np.uint16)[rows], wy)
+    # all 256 codes dequantize exactly as the oracle says, so the full tensor is pinned by the table
+    codes = np.arange(-128, 128, dtype=np.int8)
+    table = torch.from_numpy(orc.dequantize(codes, shipped, c["deq_zp"]).view(np.float16)).to(dev)
+    assert bool((deq == table[(out.long() + 128)]).all())
+
+
+def test_nce_rejects_bad_descriptors(rt, dev):
+    import torch
+    inp = torch.zeros((1, 4, 4, 16), dtype=torch.uint8, device=dev)
+    w = torch.zeros((8, 3, 3, 16), dtype=torch.int8, device=dev)
+    wt = torch.zeros((8, 4), dtype=torch.int32, device=dev)
+    out = torch.zeros((1, 2, 2, 8), dtype=torch.uint8, device=dev)
+    ok = rt.PpeInt(rt.PPE_NOOP, 0, 255, 1, 0)
+    with pytest.raises(rt.VpxError) as e:
+        rt.nce_task(inp, w, wt, out, rt.PpeInt(rt.PPE_NOOP, 10, 5, 1, 0))
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT and "clamp" in e.value.text
+    with pytest.raises(rt.VpxError) as e:
+        rt.nce_task(inp, w, wt, out, rt.PpeInt(5, 0, 255, 1, 0))  # ADD is not an integer-pipeline activation mode
+    assert e.value.code == rt.ERROR_UNSUPPORTED_FEATURE
+    with pytest.raises(rt.VpxError) as e:
+        rt.nce_task(inp, w, wt, out, rt.PpeInt(rt.PPE_LPRELU, 0, 255, 4096, 3))
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    with pytest.raises(rt.VpxError) as e:
+        rt.nce_task(inp.float(), w, wt, out, ok)
+    big_k = torch.zeros((8, 7, 7, 16), dtype=torch.int8, device=dev)
+    with pytest.raises(rt.VpxError) as e:
+        rt.nce_task(inp, big_k, wt, out, ok)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT and "fit" in e.value.text

@@ -1,0 +1,353 @@
+"""Pins the CPU oracle (oracle/vpx_oracle.c) before anything is compared against it:
+reference golden vectors, the reference's own compiled float16 (oracle/_ref, when built),
+closed forms and fp64 brute force.  No GPU."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "reference_goldens.json")) as f:
+    GOLD = json.load(f)
+
+
+def _bits(x):
+    return np.asarray(x, dtype=np.float32).view(np.uint32)
+
+
+def _interesting_f32(rng, n_random=2_000_000):
+    """fp32 bit patterns that stress fp32->fp16 rounding: every exponent near the half range with
+    mantissas on and around the round/tie boundaries, plus random bits."""
+    exps = np.arange(0, 256, dtype=np.uint32)
+    mant = []
+    for low in (0x0000, 0x0001, 0x0fff, 0x1000, 0x1001, 0x1fff, 0x2000, 0x2001, 0x2fff, 0x3000, 0x3001):
+        for hi in (0x000000, 0x7fc000, 0x7fe000, 0x400000, 0x002000, 0x7f8000, 0x555000 & ~0x3fff):
+            mant.append((hi | low) & 0x7fffff)
+    mant = np.unique(np.array(mant, dtype=np.uint32))
+    grid = (exps[:, None] << 23 | mant[None, :]).ravel()
+    # dense sweep of the subnormal-half range, exponents 102..113, coarse mantissa steps
+    e = np.arange(100, 115, dtype=np.uint32)
+    m = np.arange(0, 1 << 23, 509, dtype=np.uint32)
+    dense = (e[:, None] << 23 | m[None, :]).ravel()
+    rnd = rng.integers(0, 1 << 32, size=n_random, dtype=np.uint64).astype(np.uint32)
+    pos = np.concatenate([grid, dense, rnd & 0x7fffffff])
+    return np.concatenate([pos, pos | 0x80000000]).astype(np.uint32)
+
+
+# ---------------------------------------------------------------------------------- fp16
+
+def test_f16_reference_unit_test_vectors(orc):
+    g = GOLD["float16_values"]
+    for fbits, hbits in g["f32_bits_to_f16_bits"]:
+        x = np.array([int(fbits, 16)], dtype=np.uint32).view(np.float32)
+        assert int(orc.f32_to_f16(x)[0]) == int(hbits, 16), fbits
+    for val, hbits in g["double_to_f16_bits"]:
+        got = int(orc.f32_to_f16(np.array([np.float32(val)]))[0])
+        assert got == int(hbits, 16), (val, hex(got))
+    assert int(orc.f32_to_f16(np.array([np.inf], np.float32))[0]) == 0x7c00
+    assert int(orc.f32_to_f16(np.array([-np.inf], np.float32))[0]) == 0xfc00
+    for nan_bits in (0x7fc00000, 0x7f800001, 0xffc00000, 0x7fa00000):
+        h = int(orc.f32_to_f16(np.array([nan_bits], np.uint32).view(np.float32))[0])
+        assert (h & 0x7fff) > 0x7c00  # std::isnan(float16)
+
+
+def test_f16_widening_all_values_vs_numpy(orc):
+    h = np.arange(65536, dtype=np.uint16)
+    got = orc.f16_to_f32(h)
+    want = h.view(np.float16).astype(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+    assert np.all(np.isnan(got[nan]))
+    # round trip through the narrowing is the identity on every non-NaN half
+    back = orc.f32_to_f16(got)
+    assert np.array_equal(back[~nan], h[~nan])
+
+
+def test_f16_narrowing_vs_numpy_rne(orc):
+    rng = np.random.default_rng(1)
+    bits = _interesting_f32(rng)
+    x = bits.view(np.float32)
+    got = orc.f32_to_f16(x)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    nan = np.isnan(x)
+    # The reference's constructor doubles |v| < 2^-15 whose mantissa is >= 0x7ff000 before rounding
+    # (float16.cpp:74-107, the exponent bump of the first rounding leaks into the subnormal branch);
+    # everywhere else it is plain IEEE round-to-nearest-even.  fp32 subnormal inputs give zero,
+    # which is also what RNE gives.
+    e = (bits >> 23) & 0xff
+    quirk = (e >= 1) & (e <= 111) & ((bits & 0x7fffff) >= 0x7ff000)
+    ok = ~nan & ~quirk
+    assert np.array_equal(got[ok], want[ok])
+    with np.errstate(over="ignore"):
+        want2 = (x[quirk] * np.float32(2)).astype(np.float16).view(np.uint16)
+    assert np.array_equal(got[quirk], want2)
+
+
+def test_f16_matches_compiled_reference(orc):
+    ref = orc.ref_lib()
+    if ref is None:
+        pytest.skip("oracle/_ref not built (reference checkout absent)")
+    import ctypes as C
+    rng = np.random.default_rng(2)
+    bits = _interesting_f32(rng)
+    x = np.ascontiguousarray(bits.view(np.float32))
+    want = np.empty(x.size, dtype=np.uint16)
+    ref.ref_f32_to_f16_array(x.ctypes.data_as(C.c_void_p), want.ctypes.data_as(C.c_void_p), C.c_size_t(x.size))
+    got = orc.f32_to_f16(x)
+    assert np.array_equal(got, want)  # bit-exact, NaN payloads included
+    h = np.arange(65536, dtype=np.uint16)
+    wf = np.empty(65536, dtype=np.float32)
+    ref.ref_f16_to_f32_array(h.ctypes.data_as(C.c_void_p), wf.ctypes.data_as(C.c_void_p), C.c_size_t(65536))
+    assert np.array_equal(orc.f16_to_f32(h).view(np.uint32), wf.view(np.uint32))
+    # float16 operator+ of the reference against the oracle's eltwise add
+    a = rng.integers(0, 65536, size=200000).astype(np.uint16)
+    b = rng.integers(0, 65536, size=200000).astype(np.uint16)
+    ws = np.empty(a.size, dtype=np.uint16)
+    ref.ref_f16_add_array(a.ctypes.data_as(C.c_void_p), b.ctypes.data_as(C.c_void_p), ws.ctypes.data_as(C.c_void_p),
+                          C.c_size_t(a.size))
+    gs = orc.eltwise_f16("add", a, b)
+    nan = (ws & 0x7fff) > 0x7c00
+    assert np.array_equal(gs[~nan], ws[~nan])
+    assert np.all((gs[nan] & 0x7fff) > 0x7c00)
+
+
+# ---------------------------------------------------------------------------------- quantize / dequantize / FQ
+
+def test_dequantize_golden(orc):
+    g = GOLD["dequantize"]
+    q = np.array(g["q"], dtype=np.int8)
+    y = orc.dequantize(q, g["scale"], g["zero_point"], to_f16=False)
+    np.testing.assert_allclose(y, np.array(g["expected"], np.float32), rtol=4e-7)  # EXPECT_FLOAT_EQ = 4 ulp
+
+
+def test_quantize_golden(orc):
+    g = GOLD["quantize"]
+    x = np.array(g["x"], dtype=np.float32)
+    q = orc.quantize(x, g["scale"], g["zero_point"], signed=True, qmin=g["qmin"], qmax=g["qmax"])
+    assert q.tolist() == g["expected"]
+
+
+def test_quantize_per_axis_golden(orc):
+    g = GOLD["quantize_per_axis"]
+    x = np.array([g["x_row"], g["x_row"]], dtype=np.float32)
+    q = orc.quantize(x, g["scales"], g["zero_points"], signed=True, qmin=g["qmin"], qmax=g["qmax"], axis=0)
+    assert q.tolist() == g["expected"]
+
+
+def test_dequantize_quantize_round_trip(orc):
+    g = GOLD["dequantize_quantize_roundtrip"]
+    q = np.array(g["q"], dtype=np.int8)
+    x = orc.dequantize(q, g["scale"], g["zero_point"], to_f16=False)
+    back = orc.quantize(x, g["scale"], g["zero_point"], signed=True, qmin=g["qmin"], qmax=g["qmax"])
+    assert back.tolist() == g["q"]
+    # full storage range, several types
+    for signed, zp, scale in ((True, 0, 0.05), (True, -21, 0.003), (False, 128, 0.02), (False, 3, 1.0 / 255)):
+        allq = np.arange(-128, 128, dtype=np.int8) if signed else np.arange(0, 256, dtype=np.uint8)
+        x = orc.dequantize(allq, scale, zp, to_f16=False)
+        assert np.array_equal(orc.quantize(x, scale, zp, signed=signed), allq)
+
+
+def test_fake_quantize_properties(orc):
+    L = orc.lib()
+    # exact tie: x = 0 with limits +-4 and 256 levels sits at 127.5 -> rounds away from zero to level 128
+    want = np.float32(128.0) / np.float32(255.0) * np.float32(8.0) + np.float32(-4.0)
+    assert L.orc_fake_quantize(0.0, -4.0, 4.0, -4.0, 4.0, 256.0) == pytest.approx(float(want), abs=0)
+    assert L.orc_fake_quantize(-4.0, -4.0, 4.0, -1.0, 1.0, 256.0) == -1.0   # x <= in_lo
+    assert L.orc_fake_quantize(4.0001, -4.0, 4.0, -1.0, 1.0, 256.0) == 1.0  # x > in_hi
+    assert L.orc_fake_quantize(4.0, -4.0, 4.0, -1.0, 1.0, 256.0) == 1.0     # top level
+    rng = np.random.default_rng(3)
+    x = np.clip(rng.normal(0, 1.5, 20000), -6, 6).astype(np.float32)
+    xh = orc.f32_to_f16(x)
+    lim = lambda v: orc.f32_to_f16(np.array([v], np.float32)).reshape(1)
+    y = orc.fake_quantize_f16(xh, lim(-4), lim(4), lim(-4), lim(4), 256)
+    yf = orc.f16_to_f32(y).astype(np.float64)
+    # outputs lie on the 256-level grid (after fp16 rounding), are monotone in x and idempotent
+    k = np.round((yf + 4.0) / 8.0 * 255.0)
+    grid = orc.f16_to_f32(orc.f32_to_f16((k / 255.0 * 8.0 - 4.0).astype(np.float32)))
+    assert np.max(np.abs(grid - yf)) <= 2 ** -8  # within one fp16 ulp at |y| < 4
+    order = np.argsort(orc.f16_to_f32(xh), kind="stable")
+    assert np.all(np.diff(yf[order]) >= 0)
+    y2 = orc.fake_quantize_f16(y, lim(-4), lim(4), lim(-4), lim(4), 256)
+    assert np.max(np.abs(orc.f16_to_f32(y2) - orc.f16_to_f32(y))) <= 2 ** -8
+    # per-channel limits broadcast like numpy
+    xc = orc.f32_to_f16(rng.normal(0, 2, (2, 3, 4, 5)).astype(np.float32))
+    lo = orc.f32_to_f16(np.array([-1, -2, -3], np.float32)).reshape(1, 3, 1, 1)
+    hi = orc.f32_to_f16(np.array([1, 2, 3], np.float32)).reshape(1, 3, 1, 1)
+    yc = orc.fake_quantize_f16(xc, lo, hi, lo, hi, 16)
+    for c in range(3):
+        yc_c = orc.fake_quantize_f16(xc[:, c], lo[:, c].reshape(1), hi[:, c].reshape(1), lo[:, c].reshape(1),
+                                     hi[:, c].reshape(1), 16)
+        assert np.array_equal(yc[:, c], yc_c)
+
+
+# ---------------------------------------------------------------------------------- softmax / MVN
+
+def test_softmax_closed_forms(orc):
+    rng = np.random.default_rng(4)
+    x = rng.normal(0, 3, (7, 33, 19)).astype(np.float32)
+    for axis in (0, 1, 2):
+        y = orc.softmax_f32(x, axis)
+        np.testing.assert_allclose(y.sum(axis=axis), 1.0, rtol=2e-6)
+        # fp64 brute force
+        xd = x.astype(np.float64)
+        e = np.exp(xd - xd.max(axis=axis, keepdims=True))
+        np.testing.assert_allclose(y, e / e.sum(axis=axis, keepdims=True), rtol=3e-6, atol=1e-30)
+        # shift invariance
+        y2 = orc.softmax_f32(x + np.float32(5.0), axis)
+        np.testing.assert_allclose(y2, y, rtol=2e-5)
+    # all-equal row -> 1/n exactly representable for n = 512
+    eq = orc.softmax_f16(orc.f32_to_f16(np.full((3, 512), 1.25, np.float32)), 1)
+    assert np.all(eq == orc.f32_to_f16(np.array([1.0 / 512], np.float32))[0])
+    # masked entries (-60000) come out as exact zeros, the rest renormalises
+    xm = rng.normal(0, 3, (4, 512)).astype(np.float32)
+    mask = rng.random((4, 512)) < 0.05
+    xm[mask] = -60000.0
+    ym = orc.softmax_f16(orc.f32_to_f16(xm), 1)
+    assert np.all(ym[mask] == 0)
+    np.testing.assert_allclose(orc.f16_to_f32(ym).sum(axis=1), 1.0, atol=2e-3)
+    # padding: trailing entries ignored and zeroed
+    yp = orc.softmax_f32(x, 2, pad=4)
+    assert np.all(yp[..., -4:] == 0)
+    np.testing.assert_allclose(yp[..., :-4], orc.softmax_f32(np.ascontiguousarray(x[..., :-4]), 2), rtol=1e-6)
+
+
+def test_mvn_closed_forms(orc):
+    rng = np.random.default_rng(5)
+    x = (rng.uniform(-8, 8, (2, 6, 5, 7)) + rng.normal(0, 2, (1, 6, 1, 1))).astype(np.float32)
+    xh = orc.f32_to_f16(x)
+    xd = orc.f16_to_f32(xh).astype(np.float64)
+    for across in (True, False):
+        for nv in (True, False):
+            y = orc.f16_to_f32(orc.mvn_f16(xh, across, nv, 1e-9)).astype(np.float64)
+            ax = (1, 2, 3) if across else (2, 3)
+            mean = xd.mean(axis=ax, keepdims=True)
+            var = ((xd - mean) ** 2).mean(axis=ax, keepdims=True)
+            want = (xd - mean) / np.sqrt(var + 1e-9) if nv else xd - mean
+            np.testing.assert_allclose(y, want, rtol=1e-3, atol=2e-3)
+            assert np.max(np.abs(y.mean(axis=ax))) < 2e-3
+            if nv:
+                np.testing.assert_allclose(y.var(axis=ax), 1.0, rtol=5e-3)
+    # constant input -> zeros (eps keeps the division finite)
+    c = orc.f32_to_f16(np.full((1, 2, 3, 4), 3.5, np.float32))
+    assert np.all(orc.mvn_f16(c, True, True, 1e-9) == 0)
+    # NHWC memory layout gives the same numbers as NCHW on the transposed tensor
+    xn = np.ascontiguousarray(xh.transpose(0, 2, 3, 1))
+    for across in (True, False):
+        y1 = orc.mvn_f16(xh, across, True, 1e-9)
+        y2 = orc.mvn_f16(xn, across, True, 1e-9, layout="NHWC")
+        assert np.array_equal(y2, np.ascontiguousarray(y1.transpose(0, 2, 3, 1)))
+
+
+# ---------------------------------------------------------------------------------- integer path
+
+def test_approximate_goldens(orc):
+    for c in GOLD["approximate"]["cases"]:
+        m, s, p = orc.approximate(c["bits"], c["target"])
+        assert (m, s, p) == (c["mult"], c["shift"], 0), c
+    # multiplier range and reconstruction error of the 15-bit form
+    rng = np.random.default_rng(6)
+    for t in np.exp(rng.uniform(np.log(1e-9), np.log(100.0), 300)):
+        m, s, p = orc.approximate(15, float(t))
+        assert 2 ** 14 <= m < 2 ** 15 and p == 0
+        assert 0 <= t - m * 2.0 ** -s < t * 2.0 ** -14
+
+
+def test_weight_table_word(orc):
+    import ctypes as C
+    L = orc.lib()
+    for mult, shift in ((16384, 20), (32767, 24), (-19219, 31), (1, 0), (-32768, 63)):
+        w = orc.wt_pack_scale(shift, mult)
+        assert w == np.int32(np.uint32(((mult & 0xffff) << 16) | (shift << 8)))
+        m, s = C.c_int32(), C.c_int32()
+        L.orc_wt_unpack_scale(C.c_int32(w), C.byref(m), C.byref(s))
+        assert (m.value, s.value) == (mult, shift)
+
+
+def _rne_shift_exact(t, s):
+    """round_half_even(t / 2^s) with Python integers and fractions."""
+    from fractions import Fraction
+    if s <= 0:
+        return t
+    fr = Fraction(t, 1 << s)
+    fl = math.floor(fr)
+    rem = fr - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return fl
+
+
+def test_ppe_requant_properties(orc):
+    rng = np.random.default_rng(7)
+    noop = orc.ppe(1, 0, 0, -(2 ** 31), 2 ** 31 - 1)
+    # zero shift, unit multiplier: identity (plus bias)
+    for acc in (-5, 0, 7, 2 ** 30, -(2 ** 30)):
+        assert orc.ppe_requant(acc, 3, 1, 0, noop) == acc + 3
+    # ties go to even, on both signs
+    for acc, want in ((1, 0), (3, 2), (5, 2), (7, 4), (-1, 0), (-3, -2), (-5, -2), (6, 3), (-6, -3)):
+        assert orc.ppe_requant(acc, 0, 1, 1, noop) == want, acc
+    # exact-arithmetic cross-check, including LeakyReLU parameters and big shifts
+    lrelu = orc.ppe(1638, 14, 3, -128, 127)
+    for _ in range(3000):
+        acc = int(rng.integers(-2 ** 31, 2 ** 31))
+        bias = int(rng.integers(-2 ** 15, 2 ** 15))
+        mult = int(rng.integers(2 ** 14, 2 ** 15))
+        shift = int(rng.integers(0, 50))
+        for p, pm, ps, zp, lo, hi in ((noop, 1, 0, 0, -(2 ** 31), 2 ** 31 - 1), (lrelu, 1638, 14, 3, -128, 127)):
+            biased = (acc + bias + 2 ** 31) % 2 ** 32 - 2 ** 31
+            t = biased * mult
+            s = shift
+            if t < 0:
+                t *= pm
+                s += ps
+            want = min(max(_rne_shift_exact(t, s) + zp, lo), hi)
+            assert orc.ppe_requant(acc, bias, mult, shift, p) == want
+    # monotone in acc for a positive multiplier; clamp saturates; relu (prelu_mult 0) zeroes negatives
+    accs = np.sort(rng.integers(-10 ** 6, 10 ** 6, 500))
+    outs = [orc.ppe_requant(int(a), 0, 20000, 22, lrelu) for a in accs]
+    assert all(b >= a for a, b in zip(outs, outs[1:]))
+    assert orc.ppe_requant(2 ** 30, 0, 32767, 0, orc.ppe(1, 0, 0, 0, 255)) == 255
+    relu = orc.ppe(0, 0, 0, -128, 127)
+    assert orc.ppe_requant(-123456, 0, 20000, 10, relu) == 0
+    # LeakyReLU slope is 1638/16384 of the positive slope
+    wide = orc.ppe(1638, 14, 3, -2 ** 31, 2 ** 31 - 1)
+    pos = orc.ppe_requant(10 ** 6, 0, 16384, 14, wide) - 3
+    neg = orc.ppe_requant(-10 ** 6, 0, 16384, 14, wide) - 3
+    assert abs(neg / pos + 1638 / 16384) < 1e-5
+
+
+def test_nce_conv_against_brute_force(orc):
+    import torch
+    rng = np.random.default_rng(8)
+    N, H, W, IC, OC, KY, KX = 2, 7, 6, 16, 5, 3, 3
+    inp = rng.integers(0, 256, (N, H, W, IC), dtype=np.uint8)
+    w = rng.integers(-127, 128, (OC, KY, KX, IC)).astype(np.int8)
+    mults = rng.integers(2 ** 14, 2 ** 15, OC)
+    shifts = rng.integers(12, 16, OC)
+    bias = rng.integers(-2 ** 15, 2 ** 15, OC).astype(np.int32)
+    wt = orc.make_weights_table(mults, shifts, bias, KY * KX * IC)
+    p = orc.ppe(1, 0, 0, 0, 255)
+    for strides, pads in (((1, 1), (1, 1, 1, 1)), ((2, 2), (0, 1, 1, 0)), ((1, 2), (0, 0, 0, 0))):
+        out, acc = orc.nce_conv(inp, w, wt, p, zp_in=128, strides=strides, pads=pads, want_acc=True)
+        # independent integer reference: zero padding in the real domain == padding (in - zp) with 0
+        xi = torch.from_numpy(inp.astype(np.int64) - 128).permute(0, 3, 1, 2)
+        xi = torch.nn.functional.pad(xi, (pads[1], pads[3], pads[0], pads[2]))
+        wi = torch.from_numpy(w.astype(np.int64)).permute(0, 3, 1, 2)
+        ref = torch.nn.functional.conv2d(xi.double(), wi.double(), stride=strides).permute(0, 2, 3, 1).numpy()
+        assert np.array_equal(acc.astype(np.float64), ref)
+        want = np.empty_like(out)
+        for idx in np.ndindex(*acc.shape):
+            oc = idx[3]
+            want[idx] = orc.ppe_requant(int(acc[idx]), int(bias[oc]), int(mults[oc]), int(shifts[oc]), p)
+        assert np.array_equal(out, want)
+    # matmul form with an asymmetric activation zero point
+    A = rng.integers(-128, 128, (9, 32)).astype(np.int8)
+    B = rng.integers(-127, 128, (11, 32)).astype(np.int8)
+    wt2 = orc.make_weights_table([20000] * 11, [10] * 11, [0] * 11, 32)
+    out, acc = orc.nce_matmul(A, B, wt2, orc.ppe(1638, 14, 0, -128, 127), zp_a=3, want_acc=True)
+    assert np.array_equal(acc, (A.astype(np.int64) - 3) @ B.astype(np.int64).T)
+    # row-range evaluation equals the full evaluation on those rows
+    part = orc.nce_matmul(A, B, wt2, orc.ppe(1638, 14, 0, -128, 127), zp_a=3, rows=(2, 4))
+    assert np.array_equal(part[2:6], out[2:6])

@@ -1,0 +1,70 @@
+"""Seeded synthetic inputs of the five benchmark configurations (numpy, host side).
+
+Each generator takes a `scale` divisor so that tests can run the same distribution at a smaller
+size; scale=1 is the full configuration.  fp16 tensors are returned as uint16 bit patterns produced
+with numpy's IEEE round-to-nearest-even (inputs never fall in the range where the reference's
+float16 rounding differs from IEEE)."""
+import numpy as np
+
+
+def _f16_bits(x):
+    return np.asarray(x, dtype=np.float32).astype(np.float16).view(np.uint16)
+
+
+def c1_fake_quantize(seed=1, shape=(1, 64, 56, 56)):
+    """FakeQuantize fp16 NCHW, per-tensor, 256 levels, limits +-4; x ~ N(0,1.5) clipped to [-6,6]."""
+    rng = np.random.default_rng(seed)
+    x = np.clip(rng.normal(0.0, 1.5, shape), -6.0, 6.0)
+    lim = lambda v: _f16_bits(np.full((1, 1, 1, 1), v))
+    return {"x": _f16_bits(x), "in_lo": lim(-4.0), "in_hi": lim(4.0), "out_lo": lim(-4.0), "out_hi": lim(4.0),
+            "levels": 256}
+
+
+def c2_softmax(seed=2, shape=(8, 16, 512, 512)):
+    """Softmax over the last axis; logits ~ N(0,3), 5% of the entries set to -60000 (masking)."""
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal(shape, dtype=np.float32) * np.float32(3.0)
+    mask = rng.random(shape, dtype=np.float32) < 0.05
+    x[mask] = -60000.0
+    return {"x": _f16_bits(x), "axis": len(shape) - 1}
+
+
+def c3_mvn(seed=3, shape=(4, 256, 64, 64)):
+    """MVN across C,H,W, eps 1e-9 inside sqrt, normalize_variance; U(-8,8) + per-channel N(0,2)."""
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(-8.0, 8.0, shape).astype(np.float32)
+    x += rng.normal(0.0, 2.0, (1, shape[1], 1, 1)).astype(np.float32)
+    return {"x": _f16_bits(x), "across_channels": True, "normalize_variance": True, "eps": 1e-9}
+
+
+def c4_conv(seed=4, N=32, H=56, W=56, IC=64, OC=64):
+    """3x3 s1 p1 conv, NHWC u8 input zp 128, i8 symmetric weights, i32 bias, per-OC multiplier in
+    [2^14, 2^15) with shift 20..24, output zp 0, ReLU clamp [0,255]."""
+    rng = np.random.default_rng(seed)
+    return {
+        "input": rng.integers(0, 256, (N, H, W, IC), dtype=np.uint8),
+        "weights": rng.integers(-127, 128, (OC, 3, 3, IC)).astype(np.int8),
+        "bias": rng.integers(-2 ** 15, 2 ** 15, OC).astype(np.int32),
+        "mult": rng.integers(2 ** 14, 2 ** 15, OC).astype(np.int32),
+        "shift": rng.integers(20, 25, OC).astype(np.int32),
+        "zp_in": 128, "zp_out": 0, "clamp": (0, 255), "strides": (1, 1), "pads": (1, 1, 1, 1),
+    }
+
+
+def c5_matmul(seed=5, M=4096, K=4096, N=11008):
+    """A [M,K] i8 zp 3, B [N,K] i8 per-column symmetric; PPE per-column mult in [2^14,2^15), shift 27..28
+    (accumulator sigma ~3.5e5 * sqrt(K/4096) maps +-3 sigma onto the i8 range at K=4096), LeakyReLU 0.1
+    (1638 / 2^14), i8 output zp 0; then Dequantize (scale 0.05) to fp16 and an fp16 Add of N(0,1)."""
+    rng = np.random.default_rng(seed)
+    # keep the output spread comparable when a test shrinks K
+    shift_lo = 27 - int(round(np.log2(4096 / K) / 2)) if K < 4096 else 27
+    return {
+        "a": rng.integers(-128, 128, (M, K), dtype=np.int8),
+        "b_nk": rng.integers(-127, 128, (N, K)).astype(np.int8),
+        "bias": rng.integers(-2 ** 15, 2 ** 15, N).astype(np.int32),
+        "mult": rng.integers(2 ** 14, 2 ** 15, N).astype(np.int32),
+        "shift": rng.integers(shift_lo, shift_lo + 2, N).astype(np.int32),
+        "zp_a": 3, "zp_out": 0, "lrelu_mult": 1638, "lrelu_shift": 14, "clamp": (-128, 127),
+        "deq_scale": 0.05, "deq_zp": 0,
+        "residual": _f16_bits(rng.standard_normal((M, N), dtype=np.float32)),
+    }

@@ -1,0 +1,437 @@
+// C ABI of the execution library: blob parsing, validation, dispatch, error text, scratch memory.
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <utility>
+#include <vector>
+
+#include "vpx_common.h"
+
+namespace vpx {
+
+int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name);
+
+std::string& last_error() {
+    static thread_local std::string text;
+    return text;
+}
+
+int fail(int code, const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    last_error() = buf;
+    return code;
+}
+
+const char* dtype_name(uint32_t t) {
+    static const char* names[] = {"FP64", "FP32", "FP16", "FP8", "U64", "U32", "U16", "U8",  "I64",
+                                  "I32",  "I16",  "I8",   "I4",  "I2",  "BIN", "BF16", "UNDEFINED", "U4"};
+    return t < sizeof(names) / sizeof(names[0]) ? names[t] : "?";
+}
+
+// ---- scratch memory ---------------------------------------------------------------------------
+namespace {
+struct Scratch {
+    void* ptr = nullptr;
+    size_t size = 0;
+};
+std::mutex g_ws_mutex;
+std::map<std::pair<int, hipStream_t>, Scratch> g_ws;
+}  // namespace
+
+int get_workspace(hipStream_t stream, size_t bytes, void** out) {
+    int dev = 0;
+    VPX_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    Scratch& sc = g_ws[std::make_pair(dev, stream)];
+    if (sc.size < bytes) {
+        size_t want = 64 * 1024;
+        while (want < bytes) want *= 2;
+        void* p = nullptr;
+        VPX_HIP_CHECK(hipMalloc(&p, want));
+        // Work already queued on this stream may still use the old block, so it is kept until the
+        // process ends; sizes double, which bounds the total at twice the largest request.
+        sc.ptr = p;
+        sc.size = want;
+    }
+    *out = sc.ptr;
+    return VPX_RESULT_SUCCESS;
+}
+
+// ---- blob parsing -----------------------------------------------------------------------------
+namespace {
+
+struct Args {
+    std::vector<MemRef> mem;
+    const uint8_t* attrs = nullptr;
+    size_t attrs_size = 0;
+};
+
+bool is_compact(const MemRef& m) {
+    int64_t expect = 1;
+    for (int d = 0; d < m.nd; d++) {
+        if (m.dims[d] != 1 && m.strides[d] != expect) return false;
+        expect *= m.dims[d];
+    }
+    return true;
+}
+
+int parse_blob(const char* entry, int n_in, int n_out, const void* params, size_t params_size,
+               const vpx_memref_addr_t* addrs, uint32_t num_addrs, Args& a) {
+    const int n_mem = n_in + n_out;
+    VPX_REQUIRE((int)num_addrs == n_mem, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: expects %d memref addresses (%d in, %d out), got %u",
+                entry, n_mem, n_in, n_out, num_addrs);
+    VPX_REQUIRE(params_size >= (size_t)n_mem * sizeof(vpx_memref_data_t), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "%s: params blob of %zu bytes cannot hold %d MemRefData records", entry, params_size, n_mem);
+    const uint8_t* p = (const uint8_t*)params;
+    a.mem.resize(n_mem);
+    size_t tail = 0;
+    bool tail_needed = false;
+    for (int i = 0; i < n_mem; i++) {
+        vpx_memref_data_t md;
+        memcpy(&md, p + (size_t)i * sizeof(md), sizeof(md));
+        MemRef& m = a.mem[i];
+        VPX_REQUIRE(md.numDims >= 1 && md.numDims <= VPX_MAX_ND_DIMS, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: memref %d has %u dimensions (1..%d allowed)", entry, i, md.numDims, VPX_MAX_ND_DIMS);
+        m.nd = (int)md.numDims;
+        m.dtype = md.dataType;
+        m.order = md.dimsOrder;
+        m.elem_bits = dtype_bits(md.dataType);
+        VPX_REQUIRE(m.elem_bits > 0, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: memref %d has unsupported data type %s (%u)", entry, i,
+                    dtype_name(md.dataType), md.dataType);
+        VPX_REQUIRE(addrs[i].data != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "%s: memref %d has a null data address", entry, i);
+        VPX_REQUIRE((addrs[i].dims == nullptr) == (addrs[i].strides == nullptr), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: memref %d must give both dims and strides or neither", entry, i);
+        m.data = addrs[i].data;
+        tail += (size_t)m.nd * (sizeof(int32_t) + sizeof(int64_t));
+        if (addrs[i].dims == nullptr) tail_needed = true;
+    }
+    size_t body = params_size - (size_t)n_mem * sizeof(vpx_memref_data_t);
+    if (tail_needed) {
+        VPX_REQUIRE(body >= tail, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: params blob of %zu bytes has no room for the %zu bytes of dims/strides it must end with", entry,
+                    params_size, tail);
+        body -= tail;
+    }
+    a.attrs = p + (size_t)n_mem * sizeof(vpx_memref_data_t);
+    a.attrs_size = body;
+
+    // tail: input dims | input strides | output dims | output strides (kernel_params.cpp:56-71)
+    const uint8_t* t = a.attrs + body;
+    const uint8_t* in_dims = t;
+    size_t in_nd = 0, out_nd = 0;
+    for (int i = 0; i < n_in; i++) in_nd += a.mem[i].nd;
+    for (int i = n_in; i < n_mem; i++) out_nd += a.mem[i].nd;
+    const uint8_t* in_strides = in_dims + in_nd * 4;
+    const uint8_t* out_dims = in_strides + in_nd * 8;
+    const uint8_t* out_strides = out_dims + out_nd * 4;
+    size_t di = 0, dout = 0;
+    for (int i = 0; i < n_mem; i++) {
+        MemRef& m = a.mem[i];
+        const bool is_in = i < n_in;
+        size_t& cursor = is_in ? di : dout;
+        for (int d = 0; d < m.nd; d++) {
+            int32_t dim;
+            int64_t stride_bits;
+            if (addrs[i].dims) {
+                dim = addrs[i].dims[d];
+                stride_bits = addrs[i].strides[d];
+            } else {
+                memcpy(&dim, (is_in ? in_dims : out_dims) + (cursor + d) * 4, 4);
+                memcpy(&stride_bits, (is_in ? in_strides : out_strides) + (cursor + d) * 8, 8);
+            }
+            VPX_REQUIRE(dim >= 0, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: memref %d dimension %d is negative (%d)", entry, i, d, dim);
+            VPX_REQUIRE(stride_bits >= 0 && stride_bits % m.elem_bits == 0, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                        "%s: memref %d stride %lld bits is not a multiple of the %d-bit element", entry, i,
+                        (long long)stride_bits, m.elem_bits);
+            m.dims[d] = dim;
+            m.strides[d] = stride_bits / m.elem_bits;
+        }
+        cursor += m.nd;
+        m.compact = is_compact(m);
+    }
+    return VPX_RESULT_SUCCESS;
+}
+
+template <typename T>
+bool read_attr(const Args& a, size_t offset, T* out) {
+    if (offset + sizeof(T) > a.attrs_size) return false;
+    memcpy(out, a.attrs + offset, sizeof(T));
+    return true;
+}
+
+float half_bits_to_float(uint16_t h) {
+    const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+    float mag;
+    if (e == 0) mag = std::ldexp((float)m, -24);
+    else if (e == 31) mag = m ? NAN : INFINITY;
+    else mag = std::ldexp((float)(m | 0x400u), (int)e - 25);
+    return sign ? -mag : mag;
+}
+
+// quantize / dequantize attributes: int64 n, then n scales and n zero points, both as packed
+// floating-point values of the non-quantized operand's type (sw_kernel.cpp:97-163).
+int read_quant_params(const char* entry, const Args& a, uint32_t float_type, double* scale, int64_t* zp) {
+    int64_t n = 0;
+    VPX_REQUIRE(read_attr(a, 0, &n), VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: params blob has no quantization parameters", entry);
+    VPX_REQUIRE(n >= 1, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: quantization parameter count is %lld", entry, (long long)n);
+    VPX_REQUIRE(n == 1, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: per-axis quantization (%lld scales) is not implemented", entry,
+                (long long)n);
+    const int per_word = float_type == VPX_NN_FP16 ? 4 : 2;
+    const size_t words = (size_t)((n + per_word - 1) / per_word);
+    uint64_t sw = 0, zw = 0;
+    VPX_REQUIRE(read_attr(a, 8, &sw) && read_attr(a, 8 + words * 8, &zw), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "%s: params blob is too short for %lld scales and zero points", entry, (long long)n);
+    float zf;
+    if (float_type == VPX_NN_FP16) {
+        *scale = (double)half_bits_to_float((uint16_t)(sw & 0xffffu));
+        zf = half_bits_to_float((uint16_t)(zw & 0xffffu));
+    } else {
+        const uint32_t sb = (uint32_t)sw, zb = (uint32_t)zw;
+        float sf;
+        memcpy(&sf, &sb, 4);
+        memcpy(&zf, &zb, 4);
+        *scale = (double)sf;
+    }
+    *zp = (int64_t)std::llround(zf);
+    return VPX_RESULT_SUCCESS;
+}
+
+// Restatement of the compiler's softmax parameter packing for callers that pass the first form
+// (axis counted from the innermost memory dimension, padSize): drop unit dimensions, fuse
+// dimensions outer to the axis whose strides allow it (update_sw_kernel_params.cpp:73-101).
+void plan_from_memrefs(const MemRef& in, const MemRef& out, int64_t axis, int64_t pad, SoftmaxPlan& p) {
+    p.nd = 0;
+    int new_axis = 0;
+    for (int d = 0; d < in.nd; d++) {
+        if (in.dims[d] == 1 && d != axis && in.nd > 1) continue;
+        if (d == axis) new_axis = p.nd;
+        p.dims[p.nd] = in.dims[d];
+        p.in_stride[p.nd] = in.strides[d];
+        p.out_stride[p.nd] = out.strides[d];
+        p.nd++;
+    }
+    if (p.nd == 0) {
+        p.dims[0] = in.dims[0];
+        p.in_stride[0] = in.strides[0];
+        p.out_stride[0] = out.strides[0];
+        p.nd = 1;
+        new_axis = 0;
+    }
+    for (int i = p.nd - 2; i > new_axis; i--) {
+        if (p.in_stride[i + 1] == p.in_stride[i] * p.dims[i] && p.out_stride[i + 1] == p.out_stride[i] * p.dims[i]) {
+            p.dims[i] *= p.dims[i + 1];
+            for (int j = i + 1; j < p.nd - 1; j++) {
+                p.dims[j] = p.dims[j + 1];
+                p.in_stride[j] = p.in_stride[j + 1];
+                p.out_stride[j] = p.out_stride[j + 1];
+            }
+            p.nd--;
+        }
+    }
+    p.axis = new_axis;
+    p.pad = (int)pad;
+}
+
+int run_softmax(const char* entry, const Args& a, hipStream_t s) {
+    const MemRef& in = a.mem[0];
+    const MemRef& out = a.mem[1];
+    VPX_REQUIRE(in.dtype == out.dtype, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: input %s and output %s types differ", entry,
+                dtype_name(in.dtype), dtype_name(out.dtype));
+    const uint32_t want = strcmp(entry, "softmaxFp32") == 0 ? VPX_NN_FP32 : VPX_NN_FP16;
+    VPX_REQUIRE(in.dtype == want, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: expects %s tensors, got %s", entry, dtype_name(want),
+                dtype_name(in.dtype));
+    VPX_REQUIRE(in.nd == out.nd, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: input and output ranks differ", entry);
+    for (int d = 0; d < in.nd; d++)
+        VPX_REQUIRE(in.dims[d] == out.dims[d], VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: input and output shapes differ", entry);
+    uint64_t w0 = 0, w1 = 0;
+    VPX_REQUIRE(read_attr(a, 0, &w0) && read_attr(a, 8, &w1), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "%s: params blob has no axis / padSize attributes", entry);
+    SoftmaxPlan p{};
+    if ((w1 >> 32) == 0) {
+        // first form: int64 axis, int64 padSize
+        const int64_t axis = (int64_t)w0, pad = (int64_t)w1;
+        VPX_REQUIRE(axis >= 0 && axis < in.nd, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: axis %lld outside rank %d", entry,
+                    (long long)axis, in.nd);
+        VPX_REQUIRE(pad >= 0 && pad < in.dims[axis], VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: padSize %lld does not fit axis of %lld",
+                    entry, (long long)pad, (long long)in.dims[axis]);
+        plan_from_memrefs(in, out, axis, pad, p);
+    } else {
+        // packed form
+        const int64_t axis = (int64_t)(w0 & 0xffffffffu), pad = (int64_t)(w0 >> 32);
+        const int64_t mode = (int64_t)(w1 & 0xffffffffu), nd = (int64_t)(w1 >> 32);
+        VPX_REQUIRE(mode != VPX_SOFTMAX_DYNAMIC, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: dynamic-shape parameters are not supported", entry);
+        VPX_REQUIRE(mode >= 1 && mode <= 3, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: unknown mode %lld", entry, (long long)mode);
+        VPX_REQUIRE(nd >= 1 && nd <= VPX_MAX_ND_DIMS && axis < nd, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: packed parameters name axis %lld of %lld dimensions", entry, (long long)axis, (long long)nd);
+        p.nd = (int)nd;
+        p.axis = (int)axis;
+        p.pad = (int)pad;
+        int64_t count = 1;
+        for (int d = 0; d < p.nd; d++) {
+            uint64_t wd = 0, ws = 0;
+            VPX_REQUIRE(read_attr(a, 16 + (size_t)d * 16, &wd) && read_attr(a, 24 + (size_t)d * 16, &ws),
+                        VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: packed parameters end before dimension %d", entry, d);
+            p.dims[d] = (int64_t)(wd & 0xffffffffu);
+            p.in_stride[d] = (int64_t)(ws & 0xffffffffu);
+            p.out_stride[d] = (int64_t)(ws >> 32);
+            count *= p.dims[d];
+        }
+        VPX_REQUIRE(count == in.numel(), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: packed dimensions cover %lld elements but the tensor has %lld", entry, (long long)count,
+                    (long long)in.numel());
+        VPX_REQUIRE(pad >= 0 && pad < p.dims[p.axis], VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: padSize %lld does not fit axis of %lld",
+                    entry, (long long)pad, (long long)p.dims[p.axis]);
+    }
+    return launch_softmax(p, in.dtype, in.data, out.data, s);
+}
+
+struct Entry {
+    const char* name;
+    int n_in, n_out;
+    int kind;  // dispatch tag
+    int op;
+};
+
+enum { K_CONVERT, K_ELTWISE, K_FQ, K_QUANT, K_DEQUANT, K_MVN, K_SOFTMAX };
+
+const Entry kEntries[] = {
+        {"convert", 1, 1, K_CONVERT, 0},
+        {"eltwise_add", 2, 1, K_ELTWISE, ELT_ADD},
+        {"eltwise_sub", 2, 1, K_ELTWISE, ELT_SUB},
+        {"eltwise_mul", 2, 1, K_ELTWISE, ELT_MUL},
+        {"eltwise_min", 2, 1, K_ELTWISE, ELT_MIN},
+        {"eltwise_max", 2, 1, K_ELTWISE, ELT_MAX},
+        {"eltwise_div", 2, 1, K_ELTWISE, ELT_DIV},
+        {"fake_quantize", 5, 1, K_FQ, 0},
+        {"quantize", 1, 1, K_QUANT, 0},
+        {"dequantize", 1, 1, K_DEQUANT, 0},
+        {"mvn1", 1, 1, K_MVN, 0},
+        {"softmax", 1, 1, K_SOFTMAX, 0},
+        {"softmaxFp32", 1, 1, K_SOFTMAX, 0},
+};
+constexpr uint32_t kNumEntries = sizeof(kEntries) / sizeof(kEntries[0]);
+
+const Entry* find_entry(const char* name) {
+    for (uint32_t i = 0; i < kNumEntries; i++)
+        if (strcmp(kEntries[i].name, name) == 0) return &kEntries[i];
+    return nullptr;
+}
+
+thread_local const char* g_last_nce_kernel = "";
+
+}  // namespace
+}  // namespace vpx
+
+using namespace vpx;
+
+extern "C" {
+
+const char* vpx_get_last_error(void) {
+    return last_error().c_str();
+}
+
+uint32_t vpx_get_version(void) {
+    return (0u << 16) | 1u;
+}
+
+int vpx_sw_kernel_supported(const char* entry) {
+    return entry && find_entry(entry) ? 1 : 0;
+}
+
+uint32_t vpx_sw_kernel_count(void) {
+    return kNumEntries;
+}
+
+const char* vpx_sw_kernel_name(uint32_t i) {
+    return i < kNumEntries ? kEntries[i].name : nullptr;
+}
+
+int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_size, const vpx_memref_addr_t* addrs,
+                         uint32_t num_addrs, void* stream) {
+    last_error().clear();
+    VPX_REQUIRE(entry != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "kernel entry name is null");
+    VPX_REQUIRE(params != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "%s: params blob is null", entry);
+    VPX_REQUIRE(addrs != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "%s: memref address table is null", entry);
+    const Entry* e = find_entry(entry);
+    VPX_REQUIRE(e != nullptr, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "software kernel '%s' is not implemented", entry);
+    Args a;
+    int rc = parse_blob(entry, e->n_in, e->n_out, params, params_size, addrs, num_addrs, a);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (e->kind) {
+    case K_CONVERT: return launch_convert(a.mem[0], a.mem[1], s);
+    case K_ELTWISE: return launch_eltwise(e->op, a.mem[0], a.mem[1], a.mem[2], s);
+    case K_FQ: {
+        int64_t levels = 0;
+        VPX_REQUIRE(read_attr(a, 0, &levels), VPX_RESULT_ERROR_INVALID_ARGUMENT, "fake_quantize: params blob has no levels attribute");
+        return launch_fake_quantize(a.mem[0], &a.mem[1], a.mem[5], levels, s);
+    }
+    case K_QUANT: {
+        double scale;
+        int64_t zp;
+        rc = read_quant_params(entry, a, a.mem[0].dtype, &scale, &zp);
+        if (rc) return rc;
+        return launch_quantize(a.mem[0], a.mem[1], scale, zp, s);
+    }
+    case K_DEQUANT: {
+        double scale;
+        int64_t zp;
+        rc = read_quant_params(entry, a, a.mem[1].dtype, &scale, &zp);
+        if (rc) return rc;
+        return launch_dequantize(a.mem[0], a.mem[1], scale, zp, s);
+    }
+    case K_MVN: {
+        int64_t across = 0, normvar = 0;
+        float eps = 0.f;
+        VPX_REQUIRE(read_attr(a, 0, &across) && read_attr(a, 8, &normvar) && read_attr(a, 16, &eps),
+                    VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn1: params blob is too short for {acrossChannels, normalizeVariance, eps}");
+        VPX_REQUIRE(eps >= 0.f, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn1: eps must not be negative, got %g", (double)eps);
+        return launch_mvn(a.mem[0], a.mem[1], across != 0, normvar != 0, eps, s);
+    }
+    case K_SOFTMAX: return run_softmax(entry, a, s);
+    default: return fail(VPX_RESULT_ERROR_UNKNOWN, "%s: no dispatcher", entry);
+    }
+}
+
+int vpx_nce_task(const vpx_nce_task_t* t, void* stream) {
+    last_error().clear();
+    VPX_REQUIRE(t != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "NCE task descriptor is null");
+    VPX_REQUIRE(t->task_type == VPX_NCE_CONV, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "NCE task type %d is not implemented (CONV only)",
+                t->task_type);
+    VPX_REQUIRE(t->input && t->weights && t->weight_table && t->output, VPX_RESULT_ERROR_INVALID_NULL_HANDLE,
+                "NCE task: input, weights, weight_table and output must all be set");
+    const auto is8 = [](int32_t ty) { return ty == VPX_NN_U8 || ty == VPX_NN_I8; };
+    VPX_REQUIRE(is8(t->input_type) && is8(t->weights_type) && is8(t->output_type), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "NCE task: only U8/I8 input, weights and output are implemented (got %s, %s, %s)",
+                dtype_name((uint32_t)t->input_type), dtype_name((uint32_t)t->weights_type), dtype_name((uint32_t)t->output_type));
+    VPX_REQUIRE(t->N >= 0 && t->H >= 0 && t->W >= 0 && t->IC > 0 && t->OC >= 0, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "NCE task: invalid shape N=%lld H=%lld W=%lld IC=%lld OC=%lld", (long long)t->N, (long long)t->H,
+                (long long)t->W, (long long)t->IC, (long long)t->OC);
+    VPX_REQUIRE(t->kernel_size[0] >= 1 && t->kernel_size[1] >= 1 && t->kernel_strides[0] >= 1 && t->kernel_strides[1] >= 1,
+                VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: kernel size and strides must be positive");
+    for (int i = 0; i < 4; i++)
+        VPX_REQUIRE(t->kernel_padding[i] >= 0, VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: negative padding");
+    VPX_REQUIRE(t->ppe.clamp_low <= t->ppe.clamp_high, VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: clamp_low %d exceeds clamp_high %d",
+                t->ppe.clamp_low, t->ppe.clamp_high);
+    // prelu multiplier is an unsigned 11-bit field, prelu shift 5 bits (runtime_dpu_parser_imports.cpp.inc:411-417)
+    if (t->ppe.mode == VPX_PPE_LPRELU)
+        VPX_REQUIRE(t->ppe.lrelu_mult >= 0 && t->ppe.lrelu_mult < 2048 && t->ppe.lrelu_shift >= 0 && t->ppe.lrelu_shift < 32,
+                    VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: lrelu_mult %d / lrelu_shift %d outside the 11-bit / 5-bit fields",
+                    t->ppe.lrelu_mult, t->ppe.lrelu_shift);
+    const char* name = "";
+    const int rc = launch_nce(*t, (hipStream_t)stream, &name);
+    if (rc == VPX_RESULT_SUCCESS) g_last_nce_kernel = name;
+    return rc;
+}
+
+const char* vpx_nce_last_kernel(void) {
+    return g_last_nce_kernel;
+}
+
+}  // extern "C"

@@ -1,0 +1,282 @@
+// ACT-SHAVE `softmax` / `softmaxFp32`: y = exp(x - max) / sum(exp(x - max)) along one axis,
+// fp32 arithmetic inside, driven by the packed {axis, pad, dims, strides} parameters the compiler
+// writes (src/vpux_compiler/src/dialect/VPUIP/transforms/passes/update_sw_kernel_params.cpp:36-147).
+//
+// Three device paths:
+//   rows_wave  : reduction axis is the innermost, contiguous one and a row fits the registers of one
+//                wavefront (up to 4096 fp16 / 2048 fp32 values): one 64-lane wave owns a row, 128-bit
+//                loads, max and sum by DPP/swizzle butterflies, single pass over HBM.
+//   rows_block : innermost axis of any length or alignment: one workgroup per row, three passes.
+//   lines      : reduction over an outer (strided) axis: one lane per line, lanes adjacent along the
+//                innermost dimension so every step of the axis is a coalesced access.
+#include "vpx_common.h"
+
+namespace vpx {
+
+namespace {
+
+typedef _Float16 half_t;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct MaxOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+struct SumOp {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float v) {
+    const int i = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(i, i, CTRL, 0xf, 0xf, true));
+}
+
+// All-reduce over the 64 lanes of a wavefront; every lane returns the same value.
+template <class Op>
+__device__ __forceinline__ float wave_allreduce(float v, Op op) {
+    v = op(v, dpp<0xB1>(v));   // quad_perm [1,0,3,2]
+    v = op(v, dpp<0x4E>(v));   // quad_perm [2,3,0,1]
+    v = op(v, dpp<0x141>(v));  // row_half_mirror: the other quad of each 8 lanes
+    v = op(v, dpp<0x140>(v));  // row_mirror: the other half of each 16 lanes
+    v = op(v, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F)));  // lane ^ 16
+    const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    return op(lo, hi);
+}
+
+__device__ __forceinline__ float fast_exp(float x) {
+    return __builtin_amdgcn_exp2f(x * kLog2e);
+}
+
+struct RowMap {
+    int nd;                       // outer dimensions (all but the axis)
+    int64_t dims[VPX_MAX_ND_DIMS];
+    int64_t in_stride[VPX_MAX_ND_DIMS];
+    int64_t out_stride[VPX_MAX_ND_DIMS];
+};
+
+__device__ __forceinline__ void row_offsets(const RowMap& m, int64_t row, int64_t& in_off, int64_t& out_off) {
+    in_off = 0;
+    out_off = 0;
+    for (int d = 0; d < m.nd; d++) {
+        const int64_t q = row / m.dims[d];
+        const int64_t r = row - q * m.dims[d];
+        row = q;
+        in_off += r * m.in_stride[d];
+        out_off += r * m.out_stride[d];
+    }
+}
+
+template <typename T>
+struct VecTraits;
+template <>
+struct VecTraits<half_t> {
+    static constexpr int N = 8;
+};
+template <>
+struct VecTraits<float> {
+    static constexpr int N = 4;
+};
+
+// ---------------------------------------------------------------- rows_wave
+// NV 128-bit vectors per lane; ROWS rows per wave in flight.  `valid` = axis length minus padding.
+template <typename T, int NV, int ROWS>
+__global__ __launch_bounds__(256) void softmax_rows_wave(const T* __restrict__ in, T* __restrict__ out, RowMap map,
+                                                         int64_t rows, int len, int valid) {
+    constexpr int N = VecTraits<T>::N;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t row0 = wave * ROWS;
+    if (row0 >= rows) return;
+
+    float x[ROWS][NV][N];
+    int64_t ooff[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        const int64_t row = row0 + r < rows ? row0 + r : rows - 1;  // clamp: duplicates are not stored
+        int64_t ioff;
+        row_offsets(map, row, ioff, ooff[r]);
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int e0 = (j * 64 + lane) * N;
+            if (e0 < len) {
+                const u32x4 q = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + ioff + e0));
+                const T* p = reinterpret_cast<const T*>(&q);
+#pragma unroll
+                for (int k = 0; k < N; k++) x[r][j][k] = e0 + k < valid ? (float)p[k] : -INFINITY;
+            } else {
+#pragma unroll
+                for (int k = 0; k < N; k++) x[r][j][k] = -INFINITY;
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        float m = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+#pragma unroll
+            for (int k = 0; k < N; k++) m = fmaxf(m, x[r][j][k]);
+        m = wave_allreduce(m, MaxOp{});
+        const float mb = m * kLog2e;
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+#pragma unroll
+            for (int k = 0; k < N; k++) {
+                // exp(x - m) as exp2(x*log2e - m*log2e); padded slots hold -inf and give 0
+                const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(x[r][j][k], kLog2e, -mb));
+                x[r][j][k] = e;
+                s += e;
+            }
+        s = wave_allreduce(s, SumOp{});
+        const float inv = 1.0f / s;
+        if (row0 + r < rows) {
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const int e0 = (j * 64 + lane) * N;
+                if (e0 < len) {
+                    u32x4 q;
+                    T* p = reinterpret_cast<T*>(&q);
+#pragma unroll
+                    for (int k = 0; k < N; k++) p[k] = (T)(e0 + k < valid ? x[r][j][k] * inv : 0.f);
+                    __builtin_nontemporal_store(q, reinterpret_cast<u32x4*>(out + ooff[r] + e0));
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- rows_block
+__device__ __forceinline__ float block_allreduce_max(float v, float* smem) {
+    v = wave_allreduce(v, MaxOp{});
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) smem[w] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(smem[0], smem[1]), fmaxf(smem[2], smem[3]));
+}
+__device__ __forceinline__ float block_allreduce_sum(float v, float* smem) {
+    v = wave_allreduce(v, SumOp{});
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) smem[w] = v;
+    __syncthreads();
+    return (smem[0] + smem[1]) + (smem[2] + smem[3]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_rows_block(const T* __restrict__ in, T* __restrict__ out, RowMap map,
+                                                          int64_t len, int64_t valid, int64_t in_es, int64_t out_es) {
+    __shared__ float smem[4];
+    int64_t ioff, ooff;
+    row_offsets(map, blockIdx.x, ioff, ooff);
+    const T* px = in + ioff;
+    T* py = out + ooff;
+    float m = -INFINITY;
+    for (int64_t i = threadIdx.x; i < valid; i += 256) m = fmaxf(m, (float)px[i * in_es]);
+    m = block_allreduce_max(m, smem);
+    float s = 0.f;
+    for (int64_t i = threadIdx.x; i < valid; i += 256) s += fast_exp((float)px[i * in_es] - m);
+    s = block_allreduce_sum(s, smem);
+    const float inv = 1.0f / s;
+    for (int64_t i = threadIdx.x; i < len; i += 256)
+        py[i * out_es] = (T)(i < valid ? fast_exp((float)px[i * in_es] - m) * inv : 0.f);
+}
+
+// ---------------------------------------------------------------- lines (outer axis)
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_lines(const T* __restrict__ in, T* __restrict__ out, RowMap map,
+                                                     int64_t lines, int64_t len, int64_t valid, int64_t in_as,
+                                                     int64_t out_as) {
+    const int64_t line = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (line >= lines) return;
+    int64_t ioff, ooff;
+    row_offsets(map, line, ioff, ooff);
+    const T* px = in + ioff;
+    T* py = out + ooff;
+    // one pass keeps a running maximum and a sum rescaled whenever the maximum grows
+    float m = -INFINITY, s = 0.f;
+    for (int64_t a = 0; a < valid; a++) {
+        const float v = (float)px[a * in_as];
+        const float nm = fmaxf(m, v);
+        if (nm > -INFINITY) s = s * fast_exp(m - nm) + fast_exp(v - nm);
+        m = nm;
+    }
+    const float inv = 1.0f / s;
+    for (int64_t a = 0; a < len; a++)
+        py[a * out_as] = (T)(a < valid ? fast_exp((float)px[a * in_as] - m) * inv : 0.f);
+}
+
+template <typename T, int NV, int ROWS>
+void launch_rows_wave(const T* in, T* out, const RowMap& map, int64_t rows, int len, int valid, hipStream_t s) {
+    const int64_t waves = (rows + ROWS - 1) / ROWS;
+    const unsigned blocks = (unsigned)((waves + 3) / 4);
+    hipLaunchKernelGGL((softmax_rows_wave<T, NV, ROWS>), dim3(blocks), dim3(256), 0, s, in, out, map, rows, len, valid);
+}
+
+template <typename T>
+int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
+    constexpr int N = VecTraits<T>::N;
+    const int ax = p.axis;
+    const int64_t len = p.dims[ax];
+    const int64_t valid = len - p.pad;
+    VPX_REQUIRE(valid > 0, VPX_RESULT_ERROR_INVALID_ARGUMENT, "softmax: padSize %d leaves no element on an axis of %lld",
+                p.pad, (long long)len);
+    RowMap map{};
+    int64_t rows = 1;
+    for (int d = 0; d < p.nd; d++) {
+        if (d == ax) continue;
+        map.dims[map.nd] = p.dims[d];
+        map.in_stride[map.nd] = p.in_stride[d];
+        map.out_stride[map.nd] = p.out_stride[d];
+        map.nd++;
+        rows *= p.dims[d];
+    }
+    if (rows == 0 || len == 0) return VPX_RESULT_SUCCESS;
+    VPX_REQUIRE(rows < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "softmax: %lld rows exceed the launch limit",
+                (long long)rows);
+
+    const bool inner = ax == 0 && p.in_stride[0] == 1 && p.out_stride[0] == 1;
+    if (inner) {
+        bool vec_ok = len % N == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
+                      (reinterpret_cast<uintptr_t>(out) & 15) == 0 && len <= 64 * N * 8;
+        for (int d = 0; d < map.nd && vec_ok; d++)
+            vec_ok = map.dims[d] == 1 || (map.in_stride[d] % N == 0 && map.out_stride[d] % N == 0);
+        if (vec_ok) {
+            const int l = (int)len, v = (int)valid;
+            const int64_t per = 64 * N;
+            if (len <= per) launch_rows_wave<T, 1, 4>(in, out, map, rows, l, v, s);
+            else if (len <= 2 * per) launch_rows_wave<T, 2, 2>(in, out, map, rows, l, v, s);
+            else if (len <= 4 * per) launch_rows_wave<T, 4, 1>(in, out, map, rows, l, v, s);
+            else launch_rows_wave<T, 8, 1>(in, out, map, rows, l, v, s);
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
+    }
+    if (ax == 0) {
+        hipLaunchKernelGGL(softmax_rows_block<T>, dim3((unsigned)rows), dim3(256), 0, s, in, out, map, len, valid,
+                           p.in_stride[0], p.out_stride[0]);
+        VPX_HIP_CHECK(hipGetLastError());
+        return VPX_RESULT_SUCCESS;
+    }
+    const unsigned blocks = (unsigned)((rows + 255) / 256);
+    hipLaunchKernelGGL(softmax_lines<T>, dim3(blocks), dim3(256), 0, s, in, out, map, rows, len, valid, p.in_stride[ax],
+                       p.out_stride[ax]);
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
+}  // namespace
+
+int launch_softmax(const SoftmaxPlan& p, uint32_t dtype, const void* in, void* out, hipStream_t s) {
+    VPX_REQUIRE(p.nd >= 1 && p.nd <= VPX_MAX_ND_DIMS && p.axis >= 0 && p.axis < p.nd, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "softmax: axis %d outside a tensor of rank %d", p.axis, p.nd);
+    if (dtype == VPX_NN_FP16) return softmax_typed<half_t>(p, (const half_t*)in, (half_t*)out, s);
+    if (dtype == VPX_NN_FP32) return softmax_typed<float>(p, (const float*)in, (float*)out, s);
+    return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "softmax: element type %s is not implemented", dtype_name(dtype));
+}
+
+}  // namespace vpx

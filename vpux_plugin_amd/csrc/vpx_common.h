@@ -1,0 +1,106 @@
+// Shared host/device helpers of the execution library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+#include "vpx_runtime.h"
+
+namespace vpx {
+
+// ---- error channel -------------------------------------------------------------------------
+std::string& last_error();
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define VPX_HIP_CHECK(expr)                                                                              \
+    do {                                                                                                 \
+        hipError_t _e = (expr);                                                                          \
+        if (_e != hipSuccess)                                                                            \
+            return ::vpx::fail(_e == hipErrorOutOfMemory ? VPX_RESULT_ERROR_OUT_OF_MEMORY                \
+                                                         : VPX_RESULT_ERROR_UNKNOWN,                     \
+                               "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+    } while (0)
+
+#define VPX_REQUIRE(cond, code, ...)                   \
+    do {                                               \
+        if (!(cond)) return ::vpx::fail(code, __VA_ARGS__); \
+    } while (0)
+
+// ---- tensor views parsed from a params blob ---------------------------------------------------
+constexpr int kMaxDims = 8;  // deepest rank the strided kernels accept
+
+struct MemRef {
+    void* data = nullptr;
+    uint32_t dtype = VPX_NN_UNDEFINED;
+    uint64_t order = 0;
+    int nd = 0;
+    int64_t dims[VPX_MAX_ND_DIMS] = {};     // innermost first
+    int64_t strides[VPX_MAX_ND_DIMS] = {};  // in elements, innermost first
+    int elem_bits = 0;
+    bool compact = false;
+
+    int64_t numel() const {
+        int64_t n = 1;
+        for (int i = 0; i < nd; i++) n *= dims[i];
+        return n;
+    }
+};
+
+inline int dtype_bits(uint32_t t) {
+    switch (t) {
+    case VPX_NN_FP32:
+    case VPX_NN_I32:
+    case VPX_NN_U32: return 32;
+    case VPX_NN_FP16:
+    case VPX_NN_BF16:
+    case VPX_NN_I16:
+    case VPX_NN_U16: return 16;
+    case VPX_NN_U8:
+    case VPX_NN_I8: return 8;
+    case VPX_NN_FP64:
+    case VPX_NN_I64:
+    case VPX_NN_U64: return 64;
+    default: return 0;
+    }
+}
+
+const char* dtype_name(uint32_t t);
+
+// Device-side view for the generic strided kernels.
+struct NdIndex {
+    int nd;
+    int32_t dims[kMaxDims];     // output dims, innermost first
+    int64_t stride[4][kMaxDims];  // element strides of up to 4 operands (0 where broadcast)
+};
+
+// Library-owned scratch memory, one buffer per (device, stream): calls on one stream are ordered,
+// so they can share it; calls on different streams get different buffers.
+int get_workspace(hipStream_t stream, size_t bytes, void** out);
+
+// ---- kernel launchers (defined in the .hip files) ------------------------------------------
+int launch_convert(const MemRef& in, const MemRef& out, hipStream_t s);
+int launch_eltwise(int op, const MemRef& a, const MemRef& b, const MemRef& out, hipStream_t s);
+int launch_fake_quantize(const MemRef& in, const MemRef lims[4], const MemRef& out, int64_t levels, hipStream_t s);
+int launch_quantize(const MemRef& in, const MemRef& out, double scale, int64_t zp, hipStream_t s);
+int launch_dequantize(const MemRef& in, const MemRef& out, double scale, int64_t zp, hipStream_t s);
+
+struct SoftmaxPlan {
+    int axis;  // index into dims (innermost first)
+    int pad;
+    int nd;
+    int64_t dims[VPX_MAX_ND_DIMS];
+    int64_t in_stride[VPX_MAX_ND_DIMS];
+    int64_t out_stride[VPX_MAX_ND_DIMS];
+};
+int launch_softmax(const SoftmaxPlan& p, uint32_t dtype, const void* in, void* out, hipStream_t s);
+
+int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool normalize_variance, float eps,
+               hipStream_t s);
+
+enum EltOp { ELT_ADD = 0, ELT_SUB, ELT_MUL, ELT_MIN, ELT_MAX, ELT_DIV };
+
+}  // namespace vpx

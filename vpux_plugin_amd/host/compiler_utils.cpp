@@ -1,0 +1,419 @@
+// Host-side mirror of the reference compiler's parameter derivation for the hot path
+// (declarations and reference citations in include/vpx_compiler_utils.h).
+#include "vpx_compiler_utils.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <limits>
+#include <string>
+#include <vector>
+
+namespace vpx {
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+std::string& last_error();
+}  // namespace vpx
+
+namespace vpx {
+namespace host {
+
+// ---- fp16 ----------------------------------------------------------------------------------
+// Round to nearest even by adding the rounding constant to the bit pattern, then shifting.
+// Like vpux::type::float16 (src/vpux_utils/src/core/type/float16.cpp:74-107), a value below 2^-15
+// whose mantissa is at least 0x7ff000 is rounded as if it were twice as large: the reference's
+// first rounding step bumps the exponent and its subnormal branch then reuses the old mantissa.
+uint16_t floatToHalfBits(float v) {
+    uint32_t x;
+    std::memcpy(&x, &v, 4);
+    if ((x & 0x7f800000u) != 0 && (x & 0x7f800000u) <= (111u << 23) && (x & 0x7fffffu) >= 0x7ff000u) x += 1u << 23;
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    x &= 0x7fffffffu;
+    if (x >= 0x7f800000u) {  // Inf / NaN
+        if (x == 0x7f800000u) return (uint16_t)(sign | 0x7c00u);
+        const uint32_t payload = (x & 0x7fffffu) >> 13;
+        return (uint16_t)(sign | 0x7c00u | (payload ? payload : 1u));
+    }
+    if (x < 0x00800000u) return (uint16_t)sign;  // fp32 zero / subnormal
+    if (x >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);  // >= 65520 rounds to infinity
+    if (x >= 0x38800000u) {                                   // normal half
+        const uint32_t odd = (x >> 13) & 1u;
+        x += 0xfffu + odd;
+        return (uint16_t)(sign | ((x - 0x38000000u) >> 13));
+    }
+    if (x < 0x33000000u) return (uint16_t)sign;  // < 2^-25: underflow to zero
+    // subnormal half: align the mantissa so that one unit is 2^-24
+    const int e = (int)(x >> 23);
+    uint32_t m = (x & 0x7fffffu) | 0x800000u;
+    const int shift = 126 - e;  // 14 .. 24
+    const uint32_t rem_mask = (1u << shift) - 1u, half = 1u << (shift - 1);
+    const uint32_t rem = m & rem_mask;
+    m >>= shift;
+    if (rem > half || (rem == half && (m & 1u))) m++;
+    return (uint16_t)(sign | m);
+}
+
+float halfBitsToFloat(uint16_t h) {
+    const uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+    float mag;
+    if (e == 0) mag = std::ldexp((float)m, -24);
+    else if (e == 31) {
+        uint32_t bits = 0x7f800000u | (m << 13);
+        std::memcpy(&mag, &bits, 4);
+    } else mag = std::ldexp((float)(m | 0x400u), (int)e - 25);
+    return (h & 0x8000u) ? -mag : mag;
+}
+
+// ---- scale approximation ---------------------------------------------------------------------
+struct Approximation {
+    int64_t mult = 0, shift = 0, postShift = 0;
+};
+
+Approximation approximate(int bits, double target) {
+    int exponent = 0;
+    const double mantissa = std::frexp(target, &exponent);
+    Approximation a;
+    // floor: rounding could give 2^bits, which the multiplier register cannot hold
+    a.mult = (int64_t)std::floor(mantissa * std::pow(2.0, bits));
+    a.shift = exponent > bits ? 0 : bits - exponent;
+    a.postShift = exponent > bits ? bits - exponent : 0;
+    return a;
+}
+
+// ---- PPE attribute -----------------------------------------------------------------------------
+// absolute comparison at float epsilon (src/vpux_utils/include/vpux/utils/core/numeric.hpp:56-58)
+bool isFloatEqual(float a, float b) {
+    return std::fabs(a - b) <= std::numeric_limits<float>::epsilon();
+}
+
+}  // namespace host
+}  // namespace vpx
+
+using namespace vpx;
+using namespace vpx::host;
+
+extern "C" {
+
+uint16_t vpx_float_to_half_bits(float v) {
+    return floatToHalfBits(v);
+}
+float vpx_half_bits_to_float(uint16_t bits) {
+    return halfBitsToFloat(bits);
+}
+
+int vpx_approximate(int bits, double target, int64_t* mult, int64_t* shift, int64_t* post_shift) {
+    if (!mult || !shift || !post_shift) return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "approximate: null output");
+    if (bits < 1 || bits > 31 || !std::isfinite(target))
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "approximate: cannot approximate %g with %d bits", target, bits);
+    const Approximation a = approximate(bits, target);
+    *mult = a.mult;
+    *shift = a.shift;
+    *post_shift = a.postShift;
+    if (a.postShift != 0)
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "Encountered an attempt to approximate %g as mult = %lld, shift = %lld, postShift = %lld, but postShift is not supported",
+                    target, (long long)a.mult, (long long)a.shift, (long long)a.postShift);
+    return VPX_RESULT_SUCCESS;
+}
+
+int vpx_eltwise_quantization_approximation(double in1_scale, double in2_scale, double out_scale, int eltwise_type,
+                                           int64_t* in1_mult, int64_t* in2_mult, int64_t* out_mult, int64_t* out_shift) {
+    Approximation in1 = approximate(15, in1_scale), in2 = approximate(15, in2_scale), out = approximate(15, 1.0 / out_scale);
+    if (in1.postShift || in2.postShift || out.postShift)
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "eltwise approximation: postShift is not supported");
+    const int64_t minShift = std::min(in1.shift, in2.shift), maxShift = std::max(in1.shift, in2.shift);
+    const int64_t maxRegisterShift = 63;      // 6-bit shift register
+    const int64_t maxRegisterMult = 65535;    // unsigned 16-bit input multipliers
+    if (in1.mult < 0 || in2.mult < 0) {
+        const bool oneNegative = (in1.mult < 0) != (in2.mult < 0);
+        if (eltwise_type == 0 || eltwise_type == 1) {
+            if (oneNegative)
+                return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Unsupported case for ADD/SUB eltwise, just one negative scale %lld %lld.",
+                            (long long)in1.mult, (long long)in2.mult);
+            out.mult = -out.mult;
+        }
+        if (eltwise_type == 2 && oneNegative) out.mult = -out.mult;
+        in1.mult = (uint16_t)std::llabs(in1.mult);
+        in2.mult = (uint16_t)std::llabs(in2.mult);
+    }
+    const bool toMax = maxShift + out.shift <= maxRegisterShift && in1.mult <= (maxRegisterMult >> (maxShift - in1.shift)) &&
+                       in2.mult <= (maxRegisterMult >> (maxShift - in2.shift));
+    if (toMax) {
+        in1.mult = (uint16_t)(in1.mult << (maxShift - in1.shift));
+        in2.mult = (uint16_t)(in2.mult << (maxShift - in2.shift));
+        out.shift += maxShift;
+    } else if (minShift + out.shift < maxRegisterShift) {
+        in1.mult = (uint16_t)(in1.mult >> (in1.shift - minShift));
+        in2.mult = (uint16_t)(in2.mult >> (in2.shift - minShift));
+        out.shift += minShift;
+    } else {
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Elwise add input1_MULT/input2_MULT/output_SHIFT out of register range");
+    }
+    *in1_mult = in1.mult;
+    *in2_mult = in2.mult;
+    *out_mult = out.mult;
+    *out_shift = out.shift;
+    return VPX_RESULT_SUCCESS;
+}
+
+int32_t vpx_wt_get_scale(uint8_t shift, int16_t mult) {
+    const int32_t PPE_SHIFT_OFFSET = 8, PPE_MULT_OFFSET = 16;
+    return (int32_t)(((uint32_t)shift << PPE_SHIFT_OFFSET) | ((uint32_t)(int32_t)mult << PPE_MULT_OFFSET));
+}
+
+int vpx_wt_get_bias(double real_val, int32_t* bias) {
+    const double r = std::round(real_val);
+    if (!(r > (double)std::numeric_limits<int32_t>::min() && r < (double)std::numeric_limits<int32_t>::max()))
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Rescaled bias value is out of range");
+    *bias = (int32_t)r;
+    return VPX_RESULT_SUCCESS;
+}
+
+int vpx_get_weights_table(double in_scale, double out_scale, const double* weight_scales, size_t n_weight_scales,
+                          const double* bias, int64_t OC, int32_t weights_ptr, int32_t weights_ptr_step,
+                          int32_t sparsity_ptr, int32_t sparsity_ptr_step, int32_t* table) {
+    if (!weight_scales || !table) return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "getWeightsTable: null argument");
+    if (n_weight_scales != 1 && (int64_t)n_weight_scales != OC)
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "getWeightsTable: %zu weight scales cannot broadcast to %lld channels",
+                    n_weight_scales, (long long)OC);
+    for (int64_t oc = 0; oc < OC; oc++) {
+        const int32_t wptr = weights_ptr + (int32_t)oc * weights_ptr_step;
+        const int32_t sptr = sparsity_ptr + (int32_t)oc * sparsity_ptr_step;
+        if (wptr % 16 != 0) return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "weightsPtrs[%lld] must be multiple of 16, got %d", (long long)oc, wptr);
+        if (sptr != 0xFFFFFF && sptr % 16 != 0)
+            return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "sparsityPtrs[%lld] must be aligned to 16, got %d", (long long)oc, sptr);
+        const double ws = weight_scales[n_weight_scales == 1 ? 0 : oc];
+        const double rescale = (ws * in_scale) / out_scale;
+        const Approximation a = approximate(15, rescale);
+        if (a.postShift != 0)
+            return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                        "Encountered an attempt to approximate %g as mult = %lld, shift = %lld, postShift = %lld, but postShift is not supported",
+                        rescale, (long long)a.mult, (long long)a.shift, (long long)a.postShift);
+        if (a.shift > 255 || a.mult > 32767 || a.mult < -32768)
+            return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "scale %g does not fit the multiplier / shift fields", rescale);
+        int32_t b = 0;
+        if (bias) {
+            const int rc = vpx_wt_get_bias(bias[oc] / (ws * in_scale), &b);
+            if (rc) return rc;
+        }
+        table[oc * 4 + 0] = wptr;
+        table[oc * 4 + 1] = sptr;
+        table[oc * 4 + 2] = vpx_wt_get_scale((uint8_t)a.shift, (int16_t)a.mult);
+        table[oc * 4 + 3] = b;
+    }
+    return VPX_RESULT_SUCCESS;
+}
+
+int vpx_retrieve_ppe_int(int post_op, double param0, double param1, const vpx_quant_type_t* out_type, vpx_ppe_int_t* ppe) {
+    if (!out_type || !ppe) return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "retrievePPEAttribute: null argument");
+    // neutral values (VPU_PPEIntAttr description, tblgen/.../VPU/attributes.td:399-414)
+    ppe->mode = VPX_PPE_NOOP;
+    ppe->clamp_low = std::numeric_limits<int32_t>::min();
+    ppe->clamp_high = std::numeric_limits<int32_t>::max();
+    ppe->lrelu_mult = 1;
+    ppe->lrelu_shift = 0;
+    const bool q = out_type->is_quantized != 0;
+    switch (post_op) {
+    case VPX_POSTOP_NONE:
+        if (q) {
+            ppe->clamp_low = (int32_t)out_type->storage_min;
+            ppe->clamp_high = (int32_t)out_type->storage_max;
+        }
+        return VPX_RESULT_SUCCESS;
+    case VPX_POSTOP_RELU:
+        if (q) {
+            ppe->clamp_low = (int32_t)out_type->zero_point;
+            ppe->clamp_high = (int32_t)out_type->storage_max;
+        } else {
+            ppe->mode = VPX_PPE_LRELU;
+        }
+        return VPX_RESULT_SUCCESS;
+    case VPX_POSTOP_CLAMP: {
+        if (!q) return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "Clamp on a float output uses the fp PPE clamp, not the integer pipeline");
+        const int64_t zp = out_type->zero_point;
+        const int64_t qMin = (int64_t)std::round(param0 / out_type->scale) + zp;
+        const int64_t qMax = (int64_t)std::round(param1 / out_type->scale) + zp;
+        const int64_t lo = std::max(out_type->storage_min, qMin), hi = std::min(out_type->storage_max, qMax);
+        ppe->clamp_low = (int32_t)lo;
+        ppe->clamp_high = (int32_t)hi;
+        if (lo - zp == 0 && hi - zp < out_type->storage_max) ppe->mode = VPX_PPE_LRELUX;
+        return VPX_RESULT_SUCCESS;
+    }
+    case VPX_POSTOP_LEAKY_RELU: {
+        ppe->mode = VPX_PPE_LPRELU;
+        if (q) {
+            ppe->clamp_low = (int32_t)out_type->storage_min;
+            ppe->clamp_high = (int32_t)out_type->storage_max;
+        }
+        const double alpha = param0;
+        if (isFloatEqual((float)alpha, 0.0f)) {
+            ppe->lrelu_mult = 0;
+        } else if (!isFloatEqual((float)alpha, 1.0f)) {
+            const Approximation a = approximate(11, alpha);
+            if (a.postShift != 0)
+                return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                            "Encountered an attempt to approximate %g as mult = %lld, shift = %lld, postShift = %lld, but postShift is not supported",
+                            alpha, (long long)a.mult, (long long)a.shift, (long long)a.postShift);
+            ppe->lrelu_mult = (int32_t)a.mult;
+            ppe->lrelu_shift = (int32_t)a.shift;
+        }
+        return VPX_RESULT_SUCCESS;
+    }
+    default: return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Received unknown PPE PostOp: %d", post_op);
+    }
+}
+
+int vpx_generate_softmax_attr(uint32_t ndims_in, const int64_t* dims, const int64_t* in_strides_, const int64_t* out_strides_,
+                              int64_t axis, int64_t pad_size, uint64_t* words, uint32_t* n_words) {
+    if (!dims || !in_strides_ || !out_strides_ || !words || !n_words)
+        return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "generateVpuipSoftmaxAttr: null argument");
+    if (ndims_in < 1 || ndims_in > VPX_MAX_ND_DIMS || axis < 0 || axis >= (int64_t)ndims_in)
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "generateVpuipSoftmaxAttr: axis %lld outside rank %u", (long long)axis, ndims_in);
+    constexpr int MAXD = VPX_MAX_ND_DIMS + 1;
+    int64_t inDims[MAXD] = {}, inStrides[MAXD] = {}, outStrides[MAXD] = {};
+    int ndims = (int)ndims_in;
+    for (int i = 0; i < ndims; i++) {
+        inDims[i] = dims[i];
+        inStrides[i] = in_strides_[i];
+        outStrides[i] = out_strides_[i];
+    }
+    // unit dimensions other than the axis carry no information
+    for (int i = ndims - 1; i >= 0; i--) {
+        if (ndims <= 1) break;
+        if (inDims[i] == 1 && axis != i) {
+            for (int j = i; j < ndims - 1; j++) {
+                inDims[j] = inDims[j + 1];
+                inStrides[j] = inStrides[j + 1];
+                outStrides[j] = outStrides[j + 1];
+            }
+            if (axis > i) axis--;
+            ndims--;
+        }
+    }
+    // dimensions outer to the axis merge when both stride sets are contiguous across them
+    for (int i = ndims - 2; i > axis; i--) {
+        if (inStrides[i + 1] == inStrides[i] * inDims[i] && outStrides[i + 1] == outStrides[i] * inDims[i]) {
+            inDims[i] = inDims[i + 1] * inDims[i];
+            for (int j = i + 1; j < ndims - 1; j++) {
+                inDims[j] = inDims[j + 1];
+                inStrides[j] = inStrides[j + 1];
+                outStrides[j] = outStrides[j + 1];
+            }
+            ndims--;
+        }
+    }
+    // a strided innermost axis is handled as an outer axis over a unit inner dimension
+    if (axis == 0 && (inStrides[0] > 1 || outStrides[0] > 1)) {
+        for (int i = ndims; i >= 1; i--) {
+            inDims[i] = inDims[i - 1];
+            inStrides[i] = inStrides[i - 1];
+            outStrides[i] = outStrides[i - 1];
+        }
+        inDims[0] = 1;
+        ndims++;
+        axis = 1;
+    }
+    if (ndims < 3) {
+        for (int i = ndims; i < 3; i++) {
+            inStrides[i] = inStrides[ndims - 1] * inDims[ndims - 1];
+            outStrides[i] = outStrides[ndims - 1] * inDims[ndims - 1];
+            inDims[i] = 1;
+        }
+        ndims = 3;
+    }
+    int64_t mode;
+    if (axis == 0) {
+        const bool hardcoded = (inDims[0] == 2 || inDims[0] == 4) && pad_size == 0 && inStrides[2] == outStrides[2] &&
+                               inDims[0] == inStrides[1];
+        mode = hardcoded ? VPX_SOFTMAX_INNER_HARDCODED : VPX_SOFTMAX_INNER;
+    } else {
+        mode = VPX_SOFTMAX_OUTER;
+    }
+    auto pack = [](int64_t lo, int64_t hi) { return ((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo; };
+    uint32_t n = 0;
+    words[n++] = pack(axis, pad_size);
+    words[n++] = pack(mode, ndims);
+    for (int i = 0; i < ndims; i++) {
+        words[n++] = pack(inDims[i], inDims[i]);
+        words[n++] = pack(inStrides[i], outStrides[i]);
+    }
+    *n_words = n;
+    return VPX_RESULT_SUCCESS;
+}
+
+int vpx_get_quant_params_attr(const double* scales, const int64_t* zero_points, uint32_t n, uint32_t float_type,
+                              uint64_t* words, uint32_t* n_words) {
+    if (!scales || !zero_points || !words || !n_words) return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "getQuantParamsAttr: null argument");
+    if (float_type != VPX_NN_FP16 && float_type != VPX_NN_FP32)
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Supported non-quantized type : f16/f32");
+    const uint32_t per = float_type == VPX_NN_FP16 ? 4 : 2, width = 64 / per;
+    uint32_t w = 0;
+    words[w++] = n;
+    auto pack = [&](auto value_at) {
+        for (uint32_t i = 0; i < n; i += per) {
+            uint64_t word = 0;
+            for (uint32_t k = 0; k < per && i + k < n; k++) {
+                const float f = (float)value_at(i + k);
+                uint64_t bits;
+                if (float_type == VPX_NN_FP16) {
+                    bits = floatToHalfBits(f);
+                } else {
+                    uint32_t b;
+                    std::memcpy(&b, &f, 4);
+                    bits = b;
+                }
+                word |= bits << (width * k);
+            }
+            words[w++] = word;
+        }
+    };
+    pack([&](uint32_t i) { return scales[i]; });
+    pack([&](uint32_t i) { return (double)zero_points[i]; });
+    *n_words = w;
+    return VPX_RESULT_SUCCESS;
+}
+
+int vpx_create_kernel_params(const vpx_tensor_desc_t* inputs, uint32_t n_inputs, const vpx_tensor_desc_t* outputs,
+                             uint32_t n_outputs, const void* attrs, size_t attrs_size, void* blob, size_t* blob_size) {
+    if (!blob_size || (n_inputs && !inputs) || (n_outputs && !outputs) || (attrs_size && !attrs))
+        return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "createKernelParams: null argument");
+    std::vector<uint8_t> v;
+    auto append = [&](const void* p, size_t n) {
+        const uint8_t* b = (const uint8_t*)p;
+        v.insert(v.end(), b, b + n);
+    };
+    auto add_memref = [&](const vpx_tensor_desc_t& t) {
+        vpx_memref_data_t m;
+        std::memset(&m, 0, sizeof(m));
+        m.numDims = t.num_dims;
+        m.dimsOrder = t.dims_order;
+        m.dataType = t.data_type;
+        m.location = t.location;
+        m.isStatic = 1;
+        append(&m, sizeof(m));
+    };
+    for (uint32_t i = 0; i < n_inputs; i++) add_memref(inputs[i]);
+    for (uint32_t i = 0; i < n_outputs; i++) add_memref(outputs[i]);
+    append(attrs, attrs_size);
+    auto add_dims = [&](const vpx_tensor_desc_t* t, uint32_t n) {
+        for (uint32_t i = 0; i < n; i++) append(t[i].dims, sizeof(int32_t) * t[i].num_dims);
+    };
+    auto add_strides = [&](const vpx_tensor_desc_t* t, uint32_t n) {
+        for (uint32_t i = 0; i < n; i++) append(t[i].strides, sizeof(int64_t) * t[i].num_dims);
+    };
+    add_dims(inputs, n_inputs);
+    add_strides(inputs, n_inputs);
+    add_dims(outputs, n_outputs);
+    add_strides(outputs, n_outputs);
+    if (blob) {
+        if (*blob_size < v.size()) {
+            *blob_size = v.size();
+            return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "createKernelParams: buffer too small, %zu bytes needed", v.size());
+        }
+        std::memcpy(blob, v.data(), v.size());
+    }
+    *blob_size = v.size();
+    return VPX_RESULT_SUCCESS;
+}
+
+}  // extern "C"

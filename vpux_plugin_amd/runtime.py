@@ -1,0 +1,346 @@
+"""ctypes binding of libvpx_amd.so and thin operator wrappers over torch device tensors.
+
+torch is used for device memory and streams only; every computation goes through the C ABI
+declared in include/vpx_runtime.h.  There is no fallback: a missing library raises at import of
+this module's `lib()`.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libvpx_amd.so")
+
+# sw_params::DataType codes (include/vpx_sw_params.h)
+NN_FP32, NN_FP16, NN_U8, NN_I32, NN_I8 = 1, 2, 7, 9, 11
+ORDER = {"NCHW": 0x4321, "NHWC": 0x2431, "NCWH": 0x3421, "NWHC": 0x2341, "CHW": 0x321, "HWC": 0x132, "NC": 0x21, "C": 0x1}
+LOC_DDR = 1
+
+SUCCESS = 0
+ERROR_OUT_OF_MEMORY = 0x70000002
+ERROR_UNSUPPORTED_FEATURE = 0x78000003
+ERROR_INVALID_ARGUMENT = 0x78000004
+ERROR_INVALID_NULL_HANDLE = 0x78000005
+ERROR_UNKNOWN = 0x7FFFFFFE
+
+PPE_NOOP, PPE_LRELU, PPE_LRELUX, PPE_LPRELU = 3, 13, 14, 15
+POSTOP_NONE, POSTOP_RELU, POSTOP_CLAMP, POSTOP_LEAKY_RELU = 0, 1, 2, 3
+
+
+class VpxError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__("vpx error 0x%x: %s" % (code & 0xFFFFFFFF, text))
+        self.code = code
+        self.text = text
+
+
+class MemRefAddr(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("dims", C.POINTER(C.c_int32)), ("strides", C.POINTER(C.c_int64))]
+
+
+class TensorDesc(C.Structure):
+    _fields_ = [("num_dims", C.c_uint32), ("dims", C.POINTER(C.c_int32)), ("strides", C.POINTER(C.c_int64)),
+                ("data_type", C.c_uint32), ("dims_order", C.c_uint64), ("location", C.c_uint32)]
+
+
+class PpeInt(C.Structure):
+    _fields_ = [("mode", C.c_int32), ("clamp_low", C.c_int32), ("clamp_high", C.c_int32), ("lrelu_mult", C.c_int32),
+                ("lrelu_shift", C.c_int32)]
+
+
+class QuantType(C.Structure):
+    _fields_ = [("is_quantized", C.c_int32), ("scale", C.c_double), ("zero_point", C.c_int64),
+                ("storage_min", C.c_int64), ("storage_max", C.c_int64)]
+
+
+class NceTask(C.Structure):
+    _fields_ = [("task_type", C.c_int32), ("input", C.c_void_p), ("weights", C.c_void_p), ("weight_table", C.c_void_p),
+                ("output", C.c_void_p), ("input_type", C.c_int32), ("weights_type", C.c_int32),
+                ("output_type", C.c_int32), ("N", C.c_int64), ("H", C.c_int64), ("W", C.c_int64), ("IC", C.c_int64),
+                ("OC", C.c_int64), ("kernel_size", C.c_int32 * 2), ("kernel_strides", C.c_int32 * 2),
+                ("kernel_padding", C.c_int32 * 4), ("zp_in", C.c_int32), ("zp_w", C.c_int32), ("zp_out", C.c_int32),
+                ("ppe", PpeInt)]
+
+
+# every symbol include/vpx_runtime.h and include/vpx_compiler_utils.h declare
+EXPORTS = ["vpx_get_last_error", "vpx_get_version", "vpx_sw_kernel_launch", "vpx_sw_kernel_supported",
+           "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_approximate",
+           "vpx_eltwise_quantization_approximation", "vpx_wt_get_scale", "vpx_wt_get_bias", "vpx_get_weights_table",
+           "vpx_retrieve_ppe_int", "vpx_generate_softmax_attr", "vpx_get_quant_params_attr", "vpx_create_kernel_params",
+           "vpx_float_to_half_bits", "vpx_half_bits_to_float"]
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("%s is missing: build it with `python -m vpux_plugin_amd.build` "
+                               "(there is no CPU fallback)" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        L.vpx_get_last_error.restype = C.c_char_p
+        L.vpx_get_version.restype = C.c_uint32
+        L.vpx_sw_kernel_name.restype = C.c_char_p
+        L.vpx_sw_kernel_name.argtypes = [C.c_uint32]
+        L.vpx_sw_kernel_count.restype = C.c_uint32
+        L.vpx_sw_kernel_supported.argtypes = [C.c_char_p]
+        L.vpx_nce_last_kernel.restype = C.c_char_p
+        L.vpx_sw_kernel_launch.argtypes = [C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(MemRefAddr), C.c_uint32,
+                                           C.c_void_p]
+        L.vpx_nce_task.argtypes = [C.POINTER(NceTask), C.c_void_p]
+        L.vpx_approximate.argtypes = [C.c_int, C.c_double] + [C.POINTER(C.c_int64)] * 3
+        L.vpx_eltwise_quantization_approximation.argtypes = [C.c_double] * 3 + [C.c_int] + [C.POINTER(C.c_int64)] * 4
+        L.vpx_wt_get_scale.restype = C.c_int32
+        L.vpx_wt_get_scale.argtypes = [C.c_uint8, C.c_int16]
+        L.vpx_wt_get_bias.argtypes = [C.c_double, C.POINTER(C.c_int32)]
+        L.vpx_get_weights_table.argtypes = [C.c_double, C.c_double, C.c_void_p, C.c_size_t, C.c_void_p, C.c_int64,
+                                            C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
+        L.vpx_retrieve_ppe_int.argtypes = [C.c_int, C.c_double, C.c_double, C.POINTER(QuantType), C.POINTER(PpeInt)]
+        L.vpx_generate_softmax_attr.argtypes = [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
+                                                C.c_void_p, C.POINTER(C.c_uint32)]
+        L.vpx_get_quant_params_attr.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_void_p,
+                                                C.POINTER(C.c_uint32)]
+        L.vpx_create_kernel_params.argtypes = [C.POINTER(TensorDesc), C.c_uint32, C.POINTER(TensorDesc), C.c_uint32,
+                                               C.c_void_p, C.c_size_t, C.c_void_p, C.POINTER(C.c_size_t)]
+        L.vpx_float_to_half_bits.restype = C.c_uint16
+        L.vpx_float_to_half_bits.argtypes = [C.c_float]
+        L.vpx_half_bits_to_float.restype = C.c_float
+        L.vpx_half_bits_to_float.argtypes = [C.c_uint16]
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != SUCCESS:
+        raise VpxError(rc, lib().vpx_get_last_error().decode())
+
+
+# ---- host-side helpers (compile-time arithmetic) ---------------------------------------------------
+
+def approximate(bits, target):
+    m, s, p = C.c_int64(), C.c_int64(), C.c_int64()
+    check(lib().vpx_approximate(bits, target, C.byref(m), C.byref(s), C.byref(p)))
+    return m.value, s.value, p.value
+
+
+def eltwise_quantization_approximation(in1, in2, out, eltwise_type=0):
+    v = [C.c_int64() for _ in range(4)]
+    check(lib().vpx_eltwise_quantization_approximation(in1, in2, out, eltwise_type, *[C.byref(x) for x in v]))
+    return tuple(x.value for x in v)
+
+
+def get_weights_table(in_scale, out_scale, weight_scales, bias, OC, weights_ptr=0, weights_ptr_step=16,
+                      sparsity_ptr=0xFFFFFF, sparsity_ptr_step=0):
+    ws = np.ascontiguousarray(np.atleast_1d(weight_scales), dtype=np.float64)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float64)
+    table = np.zeros((OC, 4), dtype=np.int32)
+    check(lib().vpx_get_weights_table(in_scale, out_scale, ws.ctypes.data, ws.size, None if b is None else b.ctypes.data,
+                                      OC, weights_ptr, weights_ptr_step, sparsity_ptr, sparsity_ptr_step,
+                                      table.ctypes.data))
+    return table
+
+
+def make_weights_table(mults, shifts, biases, weights_ptr_step=16):
+    """[OC,4] int32 table from explicit per-channel multiplier / shift / int32 bias."""
+    oc = len(mults)
+    t = np.zeros((oc, 4), dtype=np.int32)
+    t[:, 0] = (np.arange(oc, dtype=np.int64) * weights_ptr_step).astype(np.int32)
+    t[:, 1] = 0xFFFFFF
+    t[:, 2] = [lib().vpx_wt_get_scale(int(s), int(m)) for m, s in zip(mults, shifts)]
+    t[:, 3] = biases
+    return t
+
+
+def retrieve_ppe_int(post_op, out_type=None, param0=0.0, param1=0.0):
+    """out_type: None (float output) or (scale, zero_point, storage_min, storage_max)."""
+    q = QuantType(0, 1.0, 0, 0, 0) if out_type is None else QuantType(1, *out_type)
+    p = PpeInt()
+    check(lib().vpx_retrieve_ppe_int(post_op, param0, param1, C.byref(q), C.byref(p)))
+    return p
+
+
+def generate_softmax_attr(dims, in_strides, out_strides, axis, pad_size=0):
+    """dims/strides innermost first (strides in elements); returns the packed uint64 words."""
+    d = np.ascontiguousarray(dims, dtype=np.int64)
+    si = np.ascontiguousarray(in_strides, dtype=np.int64)
+    so = np.ascontiguousarray(out_strides, dtype=np.int64)
+    words = np.zeros(2 + 2 * 16, dtype=np.uint64)
+    n = C.c_uint32()
+    check(lib().vpx_generate_softmax_attr(d.size, d.ctypes.data, si.ctypes.data, so.ctypes.data, axis, pad_size,
+                                          words.ctypes.data, C.byref(n)))
+    return words[:n.value].copy()
+
+
+def get_quant_params_attr(scales, zero_points, float_type):
+    s = np.ascontiguousarray(np.atleast_1d(scales), dtype=np.float64)
+    z = np.ascontiguousarray(np.atleast_1d(zero_points), dtype=np.int64)
+    words = np.zeros(1 + 2 * ((s.size + 1) // 2) + 2, dtype=np.uint64)
+    n = C.c_uint32()
+    check(lib().vpx_get_quant_params_attr(s.ctypes.data, z.ctypes.data, s.size, float_type, words.ctypes.data,
+                                          C.byref(n)))
+    return words[:n.value].copy()
+
+
+def half_bits(v):
+    return lib().vpx_float_to_half_bits(C.c_float(v))
+
+
+def half_to_float(bits):
+    return lib().vpx_half_bits_to_float(C.c_uint16(bits))
+
+
+# ---- kernel parameter blobs ------------------------------------------------------------------------
+
+def _torch_dtype_code(t):
+    import torch
+    return {torch.float16: NN_FP16, torch.float32: NN_FP32, torch.uint8: NN_U8, torch.int8: NN_I8,
+            torch.int32: NN_I32}[t.dtype]
+
+
+class Operand:
+    """A device tensor seen as a memref: `t` is indexed in MEMORY order (outermost first); its torch
+    strides may describe a sub-view.  `order` is the NDOrder code / name of the logical layout."""
+
+    def __init__(self, t, order=None):
+        self.t = t
+        nd = t.dim()
+        if order is None:
+            order = {4: "NCHW", 3: "CHW", 2: "NC", 1: "C"}.get(nd, None)
+            order = ORDER[order] if order else int("".join("%x" % (nd - i) for i in range(nd)), 16)
+        elif isinstance(order, str):
+            order = ORDER[order]
+        self.order = order
+        bits = t.element_size() * 8
+        self.dims = (C.c_int32 * nd)(*[int(s) for s in reversed(t.shape)])
+        self.strides = (C.c_int64 * nd)(*[int(s) * bits for s in reversed(t.stride())])
+        self.desc = TensorDesc(nd, self.dims, self.strides, _torch_dtype_code(t), order, LOC_DDR)
+
+
+def create_kernel_params(inputs, outputs, attrs=b""):
+    ins = (TensorDesc * len(inputs))(*[o.desc for o in inputs])
+    outs = (TensorDesc * len(outputs))(*[o.desc for o in outputs])
+    size = C.c_size_t(0)
+    check(lib().vpx_create_kernel_params(ins, len(inputs), outs, len(outputs), attrs, len(attrs), None, C.byref(size)))
+    buf = C.create_string_buffer(size.value)
+    check(lib().vpx_create_kernel_params(ins, len(inputs), outs, len(outputs), attrs, len(attrs), buf, C.byref(size)))
+    return buf.raw[:size.value]
+
+
+def _stream_handle(stream):
+    import torch
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return C.c_void_p(stream.cuda_stream)
+
+
+def sw_kernel_launch(entry, blob, operands, stream=None, side_dims=False):
+    """Launch `entry` with the serialized blob; operands supply the device addresses.  With
+    side_dims=True dims/strides travel in the address table instead of the blob tail."""
+    addrs = (MemRefAddr * len(operands))()
+    for i, o in enumerate(operands):
+        addrs[i].data = o.t.data_ptr()
+        if side_dims:
+            addrs[i].dims = C.cast(o.dims, C.POINTER(C.c_int32))
+            addrs[i].strides = C.cast(o.strides, C.POINTER(C.c_int64))
+    check(lib().vpx_sw_kernel_launch(entry.encode(), blob, len(blob), addrs, len(operands), _stream_handle(stream)))
+
+
+def _i64(*vals):
+    return np.asarray(vals, dtype=np.int64).tobytes()
+
+
+# ---- operator wrappers (VPU op -> kernel entry + attributes, as SwKernelOp::getKernelInfo does) -------
+
+def convert(x, out, order=None, stream=None):
+    ops = [Operand(x, order), Operand(out, order)]
+    sw_kernel_launch("convert", create_kernel_params(ops[:1], ops[1:]), ops, stream)
+    return out
+
+
+def eltwise(kind, a, b, out, order=None, stream=None):
+    ops = [Operand(a, order), Operand(b, order), Operand(out, order)]
+    sw_kernel_launch("eltwise_" + kind, create_kernel_params(ops[:2], ops[2:]), ops, stream)
+    return out
+
+
+def fake_quantize(x, in_lo, in_hi, out_lo, out_hi, levels, out, order=None, stream=None):
+    ops = [Operand(t, order) for t in (x, in_lo, in_hi, out_lo, out_hi, out)]
+    sw_kernel_launch("fake_quantize", create_kernel_params(ops[:5], ops[5:], _i64(levels)), ops, stream)
+    return out
+
+
+def quantize(x, out, scale, zero_point, order=None, stream=None):
+    ops = [Operand(x, order), Operand(out, order)]
+    attrs = get_quant_params_attr(scale, zero_point, _torch_dtype_code(x)).tobytes()
+    sw_kernel_launch("quantize", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    return out
+
+
+def dequantize(q, out, scale, zero_point, order=None, stream=None):
+    ops = [Operand(q, order), Operand(out, order)]
+    attrs = get_quant_params_attr(scale, zero_point, _torch_dtype_code(out)).tobytes()
+    sw_kernel_launch("dequantize", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    return out
+
+
+def mvn(x, out, across_channels, normalize_variance, eps, order="NCHW", stream=None):
+    ops = [Operand(x, order), Operand(out, order)]
+    # a true boolean attribute serialises as int64 -1 (sign-extended i1)
+    attrs = _i64(-1 if across_channels else 0, -1 if normalize_variance else 0) + np.float32(eps).tobytes()
+    sw_kernel_launch("mvn1", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    return out
+
+
+def softmax(x, out, axis, pad_size=0, order=None, packed=True, stream=None):
+    """axis indexes x in memory order (outermost first), like a torch dim."""
+    nd = x.dim()
+    axis = axis % nd
+    ops = [Operand(x, order), Operand(out, order)]
+    rev_axis = nd - 1 - axis
+    if packed:
+        bits = x.element_size() * 8
+        dims = [int(d) for d in ops[0].dims]
+        si = [int(s) // bits for s in ops[0].strides]
+        so = [int(s) // bits for s in ops[1].strides]
+        attrs = generate_softmax_attr(dims, si, so, rev_axis, pad_size).tobytes()
+    else:
+        attrs = _i64(rev_axis, pad_size)
+    entry = "softmaxFp32" if _torch_dtype_code(x) == NN_FP32 else "softmax"
+    sw_kernel_launch(entry, create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    return out
+
+
+def nce_task(inp, weights, weight_table, out, ppe, zp_in=0, zp_w=0, zp_out=0, strides=(1, 1),
+             pads=(0, 0, 0, 0), stream=None):
+    """inp NHWC, weights [OC,KY,KX,IC], weight_table [OC,4] int32 (device), out NHWC.
+    pads = (left, right, top, bottom)."""
+    N, H, W, IC = inp.shape
+    OC, KY, KX, IC2 = weights.shape
+    assert IC == IC2
+    t = NceTask()
+    t.task_type = 0
+    t.input, t.weights, t.weight_table, t.output = inp.data_ptr(), weights.data_ptr(), weight_table.data_ptr(), out.data_ptr()
+    t.input_type, t.weights_type, t.output_type = (_torch_dtype_code(x) for x in (inp, weights, out))
+    t.N, t.H, t.W, t.IC, t.OC = N, H, W, IC, OC
+    t.kernel_size[0], t.kernel_size[1] = KY, KX
+    t.kernel_strides[0], t.kernel_strides[1] = strides
+    for i in range(4):
+        t.kernel_padding[i] = pads[i]
+    t.zp_in, t.zp_w, t.zp_out = zp_in, zp_w, zp_out
+    t.ppe = ppe
+    check(lib().vpx_nce_task(C.byref(t), _stream_handle(stream)))
+    return out
+
+
+def nce_matmul(a, b_nk, weight_table, out, ppe, zp_a=0, zp_b=0, zp_out=0, stream=None):
+    """A [M,K] x B stored [N,K] -> out [M,N]: NCE.MatMul as the 1x1 convolution task."""
+    M, K = a.shape
+    Nn, _ = b_nk.shape
+    return nce_task(a.view(1, M, 1, K), b_nk.view(Nn, 1, 1, K), weight_table, out.view(1, M, 1, Nn), ppe, zp_in=zp_a,
+                    zp_w=zp_b, zp_out=zp_out, stream=stream)
+
+
+def nce_last_kernel():
+    return lib().vpx_nce_last_kernel().decode()
