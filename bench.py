@@ -1,0 +1,357 @@
+#!/usr/bin/env python3
+"""Benchmark of the vpux hot path on one MI355X.
+
+A step is one pass of the selected configuration's hot path over one batch of synthetic input that
+is already resident in HBM.  The default workload is BASELINE configuration 2 (softmax fp16
+[8,16,512,512]); `--workload` selects another one and `--all` appends a short measurement of every
+configuration to the same JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2_softmax] [--all] [--no-cpu]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E, published
+I8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA, published
+
+METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
+
+
+def _dev(a, f16=False):
+    import torch
+    a = np.ascontiguousarray(a)
+    if f16:
+        a = a.view(np.float16)
+    return torch.from_numpy(a).cuda()
+
+
+class Workload:
+    """name, description, a zero-argument `step` that enqueues one pass on the current stream,
+    algorithmic bytes and ops per step, roofline bound and the CPU-oracle sample runner."""
+
+    def __init__(self, name, desc, step, bytes_per_step, ops_per_step, bound, dtype, kernel, cpu_sample=None):
+        self.name, self.desc, self.step = name, desc, step
+        self.bytes, self.ops, self.bound, self.dtype, self.kernel = bytes_per_step, ops_per_step, bound, dtype, kernel
+        self.cpu_sample = cpu_sample
+
+
+def _prebuilt_sw_launch(rt, entry, blob, operands):
+    """Bind everything once so that a step is a single foreign call."""
+    import torch
+    L = rt.lib()
+    addrs = (rt.MemRefAddr * len(operands))()
+    for i, o in enumerate(operands):
+        addrs[i].data = o.t.data_ptr()
+    name = entry.encode()
+    n = len(operands)
+    size = len(blob)
+
+    def step():
+        rc = L.vpx_sw_kernel_launch(name, blob, size, addrs, n, C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        if rc:
+            rt.check(rc)
+    step.keep = (addrs, operands, blob)
+    return step
+
+
+def make_c1(rt):
+    import torch
+    from vpux_plugin_amd import configs
+    c = configs.c1_fake_quantize()
+    x = _dev(c["x"], True)
+    out = torch.empty_like(x)
+    ops = [rt.Operand(t) for t in (x, *[_dev(c[k], True) for k in ("in_lo", "in_hi", "out_lo", "out_hi")], out)]
+    blob = rt.create_kernel_params(ops[:5], ops[5:], np.int64(c["levels"]).tobytes())
+    n = x.numel()
+
+    def cpu(orc, frac):
+        return lambda: orc.fake_quantize_f16(c["x"], c["in_lo"], c["in_hi"], c["out_lo"], c["out_hi"], 256), n * 4
+    return Workload("c1_fake_quantize", "FakeQuantize fp16 NCHW [1,64,56,56], per-tensor, 256 levels, +-4",
+                    _prebuilt_sw_launch(rt, "fake_quantize", blob, ops), n * 4, 0, "hbm", "f16", "stream_kernel<FqFn>", cpu)
+
+
+def make_c2(rt):
+    import torch
+    from vpux_plugin_amd import configs
+    c = configs.c2_softmax()
+    x = _dev(c["x"], True)
+    out = torch.empty_like(x)
+    ops = [rt.Operand(x), rt.Operand(out)]
+    dims = [int(d) for d in ops[0].dims]
+    st = [int(s) // 16 for s in ops[0].strides]
+    attrs = rt.generate_softmax_attr(dims, st, st, 0, 0).tobytes()
+    blob = rt.create_kernel_params(ops[:1], ops[1:], attrs)
+    n = x.numel()
+
+    def cpu(orc, rows):
+        xs = np.ascontiguousarray(c["x"].reshape(-1, 512)[:rows])
+        return lambda: orc.softmax_f16(xs, 1), xs.size * 4
+    return Workload("c2_softmax", "Softmax fp16 last axis [8,16,512,512], 5% of logits masked to -60000",
+                    _prebuilt_sw_launch(rt, "softmax", blob, ops), n * 4, 0, "hbm", "f16", "softmax_rows_wave", cpu)
+
+
+def make_c3(rt):
+    import torch
+    from vpux_plugin_amd import configs
+    c = configs.c3_mvn()
+    x = _dev(c["x"], True)
+    out = torch.empty_like(x)
+    ops = [rt.Operand(x, "NCHW"), rt.Operand(out, "NCHW")]
+    attrs = np.asarray([-1, -1], dtype=np.int64).tobytes() + np.float32(c["eps"]).tobytes()
+    blob = rt.create_kernel_params(ops[:1], ops[1:], attrs)
+    n = x.numel()
+
+    def cpu(orc, groups):
+        xs = np.ascontiguousarray(c["x"][:groups])
+        return lambda: orc.mvn_f16(xs, True, True, c["eps"]), xs.size * 4
+    return Workload("c3_mvn", "MVN fp16 across C,H,W [4,256,64,64], eps 1e-9, normalize_variance",
+                    _prebuilt_sw_launch(rt, "mvn1", blob, ops), n * 4, 0, "hbm", "f16", "mvn_chunk_kernel", cpu)
+
+
+def _nce_step(rt, task):
+    import torch
+    L = rt.lib()
+
+    def step():
+        rc = L.vpx_nce_task(C.byref(task), C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        if rc:
+            rt.check(rc)
+    return step
+
+
+def _nce_task(rt, inp, w, wt, out, ppe, zp_in, zp_out, strides, pads):
+    N, H, W, IC = inp.shape
+    OC, KY, KX, _ = w.shape
+    t = rt.NceTask()
+    t.task_type = 0
+    t.input, t.weights, t.weight_table, t.output = inp.data_ptr(), w.data_ptr(), wt.data_ptr(), out.data_ptr()
+    t.input_type, t.weights_type, t.output_type = (rt._torch_dtype_code(v) for v in (inp, w, out))
+    t.N, t.H, t.W, t.IC, t.OC = N, H, W, IC, OC
+    t.kernel_size[0], t.kernel_size[1] = KY, KX
+    t.kernel_strides[0], t.kernel_strides[1] = strides
+    for i in range(4):
+        t.kernel_padding[i] = pads[i]
+    t.zp_in, t.zp_w, t.zp_out = zp_in, 0, zp_out
+    t.ppe = ppe
+    return t
+
+
+def make_c4(rt):
+    import torch
+    from vpux_plugin_amd import configs
+    c = configs.c4_conv()
+    inp, w = _dev(c["input"]), _dev(c["weights"])
+    wt_h = rt.make_weights_table(c["mult"], c["shift"], c["bias"], 9 * 64)
+    wt = _dev(wt_h)
+    out = torch.empty((32, 56, 56, 64), dtype=torch.uint8, device="cuda")
+    ppe = rt.PpeInt(rt.PPE_NOOP, c["clamp"][0], c["clamp"][1], 1, 0)
+    task = _nce_task(rt, inp, w, wt, out, ppe, c["zp_in"], c["zp_out"], c["strides"], c["pads"])
+    step = _nce_step(rt, task)
+    step.keep = (inp, w, wt, out, task)
+    ops = 2 * 32 * 56 * 56 * 64 * 9 * 64
+    nbytes = inp.numel() + out.numel() + w.numel() + wt.numel() * 4
+
+    def cpu(orc, rows):
+        p = orc.ppe(1, 0, 0, 0, 255)
+        return lambda: orc.nce_conv(c["input"], c["weights"], wt_h, p, zp_in=128, pads=(1, 1, 1, 1), rows=(0, rows)), \
+            2 * rows * 64 * 9 * 64
+    return Workload("c4_conv", "int8 Conv 3x3 s1 p1 NHWC [32,56,56,64] u8 zp128 x [64,3,3,64] i8, PPE ReLU clamp [0,255]",
+                    step, nbytes, ops, "mfma", "int8", "nce_conv_mfma", cpu)
+
+
+def make_c5(rt, part="matmul"):
+    import torch
+    from vpux_plugin_amd import configs
+    c = configs.c5_matmul()
+    M, K = c["a"].shape
+    N = c["b_nk"].shape[0]
+    if part == "matmul":
+        a, b = _dev(c["a"]), _dev(c["b_nk"])
+        wt_h = rt.make_weights_table(c["mult"], c["shift"], c["bias"], K)
+        wt = _dev(wt_h)
+        out = torch.empty((M, N), dtype=torch.int8, device="cuda")
+        ppe = rt.PpeInt(rt.PPE_LPRELU, c["clamp"][0], c["clamp"][1], c["lrelu_mult"], c["lrelu_shift"])
+        task = _nce_task(rt, a.view(1, M, 1, K), b.view(N, 1, 1, K), wt, out.view(1, M, 1, N), ppe, c["zp_a"],
+                         c["zp_out"], (1, 1), (0, 0, 0, 0))
+        step = _nce_step(rt, task)
+        step.keep = (a, b, wt, out, task)
+
+        def cpu(orc, rows):
+            p = orc.ppe(c["lrelu_mult"], c["lrelu_shift"], 0, -128, 127)
+            a_s = np.ascontiguousarray(c["a"][:rows])
+            return lambda: orc.nce_matmul(a_s, c["b_nk"], wt_h, p, zp_a=c["zp_a"]), 2 * rows * K * N
+        return Workload("c5_matmul", "int8 MatMul A[4096,4096] zp3 x B[4096,11008], PPE per-column + LeakyReLU 0.1 -> i8",
+                        step, M * K + N * K + M * N + N * 16, 2 * M * K * N, "mfma", "int8", "nce_gemm_mfma", cpu)
+    q = torch.randint(-128, 128, (M, N), dtype=torch.int8, device="cuda")
+    deq = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    if part == "dequant":
+        ops = [rt.Operand(q), rt.Operand(deq)]
+        blob = rt.create_kernel_params(ops[:1], ops[1:], rt.get_quant_params_attr(c["deq_scale"], c["deq_zp"], rt.NN_FP16).tobytes())
+        return Workload("c5_dequantize", "Dequantize i8 -> fp16 [4096,11008], per-tensor",
+                        _prebuilt_sw_launch(rt, "dequantize", blob, ops), M * N * 3, 0, "hbm", "f16", "stream_kernel<DequantFn>")
+    res = _dev(c["residual"], True)
+    y = torch.empty_like(deq)
+    deq.normal_()
+    ops = [rt.Operand(deq), rt.Operand(res), rt.Operand(y)]
+    blob = rt.create_kernel_params(ops[:2], ops[2:])
+    return Workload("c5_eltwise_add", "Eltwise Add fp16 [4096,11008] + residual",
+                    _prebuilt_sw_launch(rt, "eltwise_add", blob, ops), M * N * 6, 0, "hbm", "f16", "stream_kernel<EltFn add>")
+
+
+MAKERS = {
+    "c1_fake_quantize": make_c1,
+    "c2_softmax": make_c2,
+    "c3_mvn": make_c3,
+    "c4_conv": make_c4,
+    "c5_matmul": lambda rt: make_c5(rt, "matmul"),
+    "c5_dequantize": lambda rt: make_c5(rt, "dequant"),
+    "c5_eltwise_add": lambda rt: make_c5(rt, "add"),
+}
+
+
+def time_steps(step, steps, warmup, graph=False):
+    """Returns (wall ms per step, device ms per step from events on the launch stream)."""
+    import torch
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    if graph:
+        g = torch.cuda.CUDAGraph()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            step()  # first use of a stream may size the library's scratch buffer: not allowed while capturing
+        s.synchronize()
+        with torch.cuda.stream(s):
+            with torch.cuda.graph(g, stream=s):
+                for _ in range(steps):
+                    step()
+        torch.cuda.current_stream().wait_stream(s)
+        g.replay()
+        torch.cuda.synchronize()
+        run = g.replay
+    else:
+        def run():
+            for _ in range(steps):
+                step()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    run()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
+
+
+def roofline(w, dev_ms):
+    if w.bound == "hbm":
+        achieved = w.bytes / (dev_ms * 1e-3) / 1e9
+        return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": w.kernel}
+    achieved = w.ops / (dev_ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": round(achieved, 2), "peak": I8_PEAK_TOPS, "unit": "TOP/s",
+            "frac": round(achieved / I8_PEAK_TOPS, 4), "traffic": None, "kernel": w.kernel}
+
+
+def value_of(w, ms):
+    if w.bound == "hbm":
+        return w.bytes / (ms * 1e-3) / 1e9, "GB/s"
+    return w.ops / (ms * 1e-3) / 1e12, "TOP/s"
+
+
+def cpu_baseline(w, budget_s=12.0):
+    """Times the CPU oracle on a bounded sample of the same workload, all host threads."""
+    import oracle
+    if w.cpu_sample is None:
+        return None
+    cores = min(oracle.num_threads(), int(os.environ.get("OMP_NUM_THREADS", "1024")))
+    units = {"c1_fake_quantize": 1, "c2_softmax": 2048, "c3_mvn": 1, "c4_conv": 3136, "c5_matmul": 8}[w.name]
+    full = {"c1_fake_quantize": 1, "c2_softmax": 65536, "c3_mvn": 4, "c4_conv": 100352, "c5_matmul": 4096}[w.name]
+    fn, work = w.cpu_sample(oracle, units)
+    t0 = time.perf_counter()
+    fn()
+    dt = time.perf_counter() - t0
+    # grow the sample towards the time budget (at most the full workload), then time it once more
+    scale = int(min(full // units, max(1, budget_s / max(dt, 1e-4))))
+    reps = 1
+    if scale > 1:
+        units *= scale
+        fn, work = w.cpu_sample(oracle, units)
+    else:
+        reps = int(max(1, min(2000, budget_s / max(dt, 1e-5))))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    dt = (time.perf_counter() - t0) / reps
+    if w.bound == "hbm":
+        val, unit = work / dt / 1e9, "GB/s"
+    else:
+        val, unit = work / dt / 1e12, "TOP/s"
+    what = {"c1_fake_quantize": "full tensor", "c2_softmax": "%d of 65536 rows" % units, "c3_mvn": "%d of 4 batch elements" % units,
+            "c4_conv": "%d of 100352 output positions" % units, "c5_matmul": "%d of 4096 rows of A" % units}[w.name]
+    return {"value": round(val, 4), "unit": unit, "cores": cores, "kind": "port",
+            "sample": "%s, %d repetition(s), %.1f s of CPU time per repetition" % (what, reps, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2_softmax", choices=sorted(MAKERS))
+    ap.add_argument("--all", action="store_true", help="also measure every other configuration (short runs)")
+    ap.add_argument("--graph", action="store_true", help="replay the timed steps from one HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this path runs on one GPU only (every kernel shards without exchange; see DESIGN.md); "
+                 "run it with --gpus 1")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    from vpux_plugin_amd import runtime as rt
+    rt.lib()
+    torch.cuda.set_device(0)
+
+    w = MAKERS[args.workload](rt)
+    wall_ms, dev_ms = time_steps(w.step, args.steps, args.warmup, graph=args.graph)
+    value, unit = value_of(w, wall_ms)
+    line = {
+        "metric": METRIC, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": w.dtype, "data": "synthetic",
+        "config": {"workload": w.name, "description": w.desc, "launch": "hip graph" if args.graph else "eager"},
+        "device_ms_per_step": round(dev_ms, 6),
+        "roofline": roofline(w, dev_ms),
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(w)
+    if args.all:
+        others = {}
+        for name in sorted(MAKERS):
+            if name == args.workload:
+                continue
+            del w
+            torch.cuda.empty_cache()
+            w = MAKERS[name](rt)
+            steps = 50 if name == "c5_matmul" else 200
+            wall, dev = time_steps(w.step, steps, 10, graph=False)
+            _, gdev = time_steps(w.step, steps, 2, graph=True)
+            v, u = value_of(w, wall)
+            others[name] = {"value": round(v, 2), "unit": u, "ms_per_step": round(wall, 6),
+                            "device_ms_per_step": round(dev, 6), "graph_device_ms_per_step": round(gdev, 6),
+                            "roofline": roofline(w, min(dev, gdev))}
+        line["other_configs"] = others
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -37,7 +37,7 @@ void orc_set_num_threads(int n) {
  * first (:74-80) and, when that carries, bumps the exponent even if the result is subnormal; the
  * subnormal branch (:92-107) then re-reads the ORIGINAL mantissa with the bumped exponent.  For
  * |v| < 2^-15 with mantissa >= 0x7ff000 the result is therefore the rounding of 2*v. */
-uint16_t orc_f32_to_f16(float v) {
+static uint16_t f32_to_f16_impl(float v, int reference_quirk) {
     uint32_t bits;
     memcpy(&bits, &v, 4);
     const uint16_t sign = (uint16_t)((bits >> 16) & 0x8000u);
@@ -59,7 +59,7 @@ uint16_t orc_f32_to_f16(float v) {
         if (h >= 0x7c00u) h = 0x7c00u;
         return (uint16_t)(sign | h);
     }
-    if (man >= 0x7ff000u) {
+    if (reference_quirk && man >= 0x7ff000u) {
         e++; /* the carry of the first rounding, see above */
         if (e > 0) return (uint16_t)(sign | 0x0400u);
     }
@@ -72,6 +72,17 @@ uint16_t orc_f32_to_f16(float v) {
     const uint32_t half = 1u << (sh - 1);
     if (rem > half || (rem == half && (h & 1u))) h++;
     return (uint16_t)(sign | h);
+}
+
+uint16_t orc_f32_to_f16(float v) {
+    return f32_to_f16_impl(v, 1);
+}
+
+/* Plain IEEE-754 round-to-nearest-even narrowing, without the deviation above.  Used for the
+ * results of softmax and MVN, whose semantics come from the operator definitions rather than
+ * from the reference's float16 class. */
+uint16_t orc_f32_to_f16_ieee(float v) {
+    return f32_to_f16_impl(v, 0);
 }
 
 /* exact widening, src/vpux_utils/src/core/type/float16.cpp:118-144 */
@@ -275,7 +286,7 @@ void orc_softmax_f16(const uint16_t* x, uint16_t* y, int64_t outer, int64_t axis
             for (int64_t a = 0; a < valid; a++) sum += (double)expf(orc_f16_to_f32(px[a * inner]) - mx);
             for (int64_t a = 0; a < valid; a++) {
                 const double e = (double)expf(orc_f16_to_f32(px[a * inner]) - mx);
-                py[a * inner] = orc_f32_to_f16((float)(e / sum));
+                py[a * inner] = orc_f32_to_f16_ieee((float)(e / sum));
             }
             for (int64_t a = valid; a < axis; a++) py[a * inner] = 0;
         }
@@ -311,7 +322,7 @@ void orc_mvn_f16(const uint16_t* x, uint16_t* y, int64_t N, int64_t C, int64_t S
         for (int64_t c = 0; c < gc; c++)
             for (int64_t s = 0; s < S; s++) {
                 const int64_t off = base + c * stride_c + s * stride_s;
-                y[off] = orc_f32_to_f16((float)(((double)orc_f16_to_f32(x[off]) - mean) * inv));
+                y[off] = orc_f32_to_f16_ieee((float)(((double)orc_f16_to_f32(x[off]) - mean) * inv));
             }
     }
 }

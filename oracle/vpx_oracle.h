@@ -35,7 +35,8 @@ extern "C" {
 #endif
 
 /* ---- fp16 (src/vpux_utils/src/core/type/float16.cpp:30-144) ---- */
-uint16_t orc_f32_to_f16(float v);
+uint16_t orc_f32_to_f16(float v);      /* bit-exact with the reference class, its subnormal-range deviation included */
+uint16_t orc_f32_to_f16_ieee(float v); /* plain IEEE RNE; rounds softmax / MVN results */
 float orc_f16_to_f32(uint16_t h);
 void orc_convert_f32_to_f16(const float* in, uint16_t* out, size_t n);
 void orc_convert_f16_to_f32(const uint16_t* in, float* out, size_t n);

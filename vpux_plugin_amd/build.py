@@ -35,7 +35,10 @@ def build(verbose=True, jobs=8):
         if len(procs) >= jobs:
             _drain(procs, verbose)
     _drain(procs, verbose)
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    # -no-hip-rt: no DT_NEEDED on a particular libamdhip64.  A process must hold exactly one HIP
+    # runtime; the host application (or vpux_plugin_amd.runtime, which picks the copy torch ships)
+    # provides it before this library is loaded.
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-no-hip-rt", "-o", LIB] + objs
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

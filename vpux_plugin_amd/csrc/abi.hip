@@ -103,7 +103,6 @@ int parse_blob(const char* entry, int n_in, int n_out, const void* params, size_
         m.elem_bits = dtype_bits(md.dataType);
         VPX_REQUIRE(m.elem_bits > 0, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: memref %d has unsupported data type %s (%u)", entry, i,
                     dtype_name(md.dataType), md.dataType);
-        VPX_REQUIRE(addrs[i].data != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "%s: memref %d has a null data address", entry, i);
         VPX_REQUIRE((addrs[i].dims == nullptr) == (addrs[i].strides == nullptr), VPX_RESULT_ERROR_INVALID_ARGUMENT,
                     "%s: memref %d must give both dims and strides or neither", entry, i);
         m.data = addrs[i].data;
@@ -153,6 +152,8 @@ int parse_blob(const char* entry, int n_in, int n_out, const void* params, size_
         }
         cursor += m.nd;
         m.compact = is_compact(m);
+        VPX_REQUIRE(m.data != nullptr || m.numel() == 0, VPX_RESULT_ERROR_INVALID_NULL_HANDLE,
+                    "%s: memref %d has a null data address", entry, i);
     }
     return VPX_RESULT_SUCCESS;
 }

@@ -73,12 +73,30 @@ EXPORTS = ["vpx_get_last_error", "vpx_get_version", "vpx_sw_kernel_launch", "vpx
 _lib = None
 
 
+def _load_hip_runtime():
+    """libvpx_amd.so leaves the HIP runtime symbols undefined so that it binds to whichever single
+    runtime the process holds.  Under Python that is the copy bundled with torch (a second,
+    system-wide copy in the same process does not see the GPU); without torch, the ROCm install."""
+    candidates = []
+    try:
+        import torch
+        candidates.append(os.path.join(os.path.dirname(torch.__file__), "lib", "libamdhip64.so"))
+    except ImportError:
+        pass
+    candidates += [os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib", "libamdhip64.so")]
+    for path in candidates:
+        if os.path.exists(path):
+            return C.CDLL(path, mode=C.RTLD_GLOBAL)
+    raise RuntimeError("no libamdhip64.so found (looked in %s)" % ", ".join(candidates))
+
+
 def lib():
     global _lib
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise RuntimeError("%s is missing: build it with `python -m vpux_plugin_amd.build` "
                                "(there is no CPU fallback)" % LIB_PATH)
+        _load_hip_runtime()
         L = C.CDLL(LIB_PATH)
         L.vpx_get_last_error.restype = C.c_char_p
         L.vpx_get_version.restype = C.c_uint32
