@@ -3,8 +3,9 @@
 //
 // Device paths (chosen by vpx_nce_task):
 //   nce_gemm_mfma  : 1x1 kernel, stride 1, no padding (this is how NCE.MatMul arrives): a plain
-//                    A[M][K] x B[N][K]^T GEMM.  256x256 output tile per workgroup, K staged through
-//                    double-buffered, XOR-swizzled LDS, v_mfma_i32_32x32x32_i8, 128x128 per wave.
+//                    A[M][K] x B[N][K]^T GEMM.  256x256 output tile per workgroup, 128x128 per wave,
+//                    v_mfma_i32_32x32x32_i8.  K panels go from global memory straight into
+//                    XOR-swizzled LDS (global_load_lds, no register staging), two stages.
 //   nce_conv_mfma  : general KYxKX / stride / padding with IC a multiple of 32: implicit GEMM, the
 //                    activation fragments are gathered from the NHWC tensor (no im2col buffer),
 //                    the weights of the tile sit in LDS.
@@ -16,6 +17,7 @@
 // zero point so they contribute exactly 0, as the MPE does (runtime_dpu_parser_imports.cpp.inc:872-879).
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 #include "vpx_common.h"
 
@@ -32,14 +34,14 @@ struct Ppe {
     int prelu_mult, prelu_shift, zp_out, clamp_lo, clamp_hi;
 };
 
-// Per output channel, unpacked from weight-table words 2 and 3 with the zero-point term folded in.
+// Raw per-channel PPE parameters, unpacked from weight-table words 2 and 3.
 struct ChanParams {
-    int bias, mult, shift, pad;
+    int bias, mult, shift;
 };
 
 // Integer PPE in the order the compiler programs it (expand_dpu_config_invariant_ppe.cpp:322-380):
 // bias add, scale multiply, [prelu multiply on negatives], one round-half-even over the combined
-// right shift, zero point, clamp.
+// right shift, zero point, clamp.  64-bit integer arithmetic; the general, slow form.
 __device__ __forceinline__ int ppe_requant(int acc, ChanParams c, Ppe p) {
     const int biased = (int)((unsigned)acc + (unsigned)c.bias);
     long long t = (long long)biased * (long long)c.mult;
@@ -66,15 +68,77 @@ __device__ __forceinline__ int ppe_requant(int acc, ChanParams c, Ppe p) {
 }
 
 template <bool OUT_SIGNED>
+__device__ __forceinline__ int saturate8i(int r) {
+    if (OUT_SIGNED) return r < -128 ? -128 : (r > 127 ? 127 : r);
+    return r < 0 ? 0 : (r > 255 ? 255 : r);
+}
+template <bool OUT_SIGNED>
 __device__ __forceinline__ uint8_t saturate8(int r) {
-    if (OUT_SIGNED) return (uint8_t)(int8_t)(r < -128 ? -128 : (r > 127 ? 127 : r));
-    return (uint8_t)(r < 0 ? 0 : (r > 255 ? 255 : r));
+    return (uint8_t)saturate8i<OUT_SIGNED>(r);
+}
+
+// Per-channel parameters prepared for the fast epilogue.  With f = mult * 2^-shift (exactly
+// representable), one double-precision fused multiply-add b * f + 1.5 * 2^52 rounds the exact
+// product to an integer, ties to even, in a single step: that IS the round-half-even shift of the
+// integer pipeline, for every 32-bit b and every multiplier / shift the weight table can hold.
+// The integer then sits in the low dword of the sum.  f_pos serves t >= 0 and
+// f_neg = mult * prelu_mult * 2^-(shift + prelu_shift) serves t < 0.
+struct ChanPrep {
+    double f_pos;
+    double f_neg;
+    int bias;      // weight-table bias with the zero-point term folded in
+    int sgn;       // -1 when mult < 0, else 0: t < 0  <=>  (b ^ sgn) < 0 for b != 0
+    int bmax_pos;  // |b| beyond these makes |b * f| exceed 2^30: such b are clipped first, which
+    int bmax_neg;  // cannot change a result that saturates anyway; INT_MAX when |f| <= 1/2
+};
+static_assert(sizeof(ChanPrep) == 32, "ChanPrep layout");
+
+struct PpeFast {
+    int zp_out, lo, hi;  // clamp bounds already intersected with the storage range
+};
+
+__device__ __forceinline__ int ppe_bmax(double f) {
+    const double a = __builtin_fabs(f);
+    return a <= 0.5 ? 0x7fffffff : (int)(1073741824.0 / a);
+}
+
+__device__ __forceinline__ ChanPrep ppe_prepare(int mult, int shift, int bias, int prelu_mult, int prelu_shift) {
+    ChanPrep c;
+    c.bias = bias;
+    c.sgn = mult < 0 ? -1 : 0;
+    c.f_pos = __builtin_ldexp((double)mult, -shift);
+    c.f_neg = __builtin_ldexp((double)((long long)mult * (long long)prelu_mult), -(shift + prelu_shift));
+    c.bmax_pos = ppe_bmax(c.f_pos);
+    c.bmax_neg = ppe_bmax(c.f_neg);
+    return c;
+}
+
+// CLIP = false may be used when both bmax are INT_MAX (no clipping needed).
+template <bool CLIP>
+__device__ __forceinline__ int ppe_fast(int acc, const ChanPrep& c, const PpeFast& p) {
+    int b = (int)((unsigned)acc + (unsigned)c.bias);
+    const bool neg = (b ^ c.sgn) < 0;
+    const double f = neg ? c.f_neg : c.f_pos;
+    if (CLIP) {
+        const int bm = neg ? c.bmax_neg : c.bmax_pos;
+        b = b > bm ? bm : (b < -bm ? -bm : b);
+    }
+    // (double)b without a conversion instruction: the bit pattern of 2^52 + (b + 2^31), minus that offset
+    const double bd = __builtin_bit_cast(double, 0x4330000000000000ull | (unsigned long long)((unsigned)b ^ 0x80000000u)) -
+                      4503601774854144.0;
+    constexpr double kMagic = 6755399441055744.0;  // 1.5 * 2^52
+    const double y = __builtin_fma(bd, f, kMagic);
+    const int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, y) + p.zp_out;
+    const int t = q > p.lo ? q : p.lo;
+    return t < p.hi ? t : p.hi;
 }
 
 // ---------------------------------------------------------------- per-channel parameter fold
-// params[oc] = {bias + corr * sum_k w[oc][k], mult, shift}; one wavefront per output channel.
+// One wavefront per output channel: sum of the channel's weights (for the zero-point term) and the
+// prepared epilogue parameters.
 __global__ __launch_bounds__(256) void nce_fold_kernel(const int8_t* __restrict__ w, const int32_t* __restrict__ wt,
-                                                       ChanParams* __restrict__ params, int64_t OC, int64_t K, int corr) {
+                                                       ChanPrep* __restrict__ prep, int64_t OC, int64_t K, int corr,
+                                                       Ppe ppe) {
     const int lane = threadIdx.x & 63;
     const int64_t oc = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (oc >= OC) return;
@@ -94,13 +158,43 @@ __global__ __launch_bounds__(256) void nce_fold_kernel(const int8_t* __restrict_
     }
     if (lane == 0) {
         const uint32_t w2 = (uint32_t)wt[oc * 4 + 2];
-        ChanParams c;
-        c.bias = (int)((unsigned)wt[oc * 4 + 3] + (unsigned)(corr * sum));
-        c.mult = (int)(int16_t)(w2 >> 16);
-        c.shift = (int)((w2 >> 8) & 0xffu);
-        c.pad = 0;
-        params[oc] = c;
+        const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+                                       (int)((unsigned)wt[oc * 4 + 3] + (unsigned)(corr * sum)), ppe.prelu_mult, ppe.prelu_shift);
+        prep[oc] = c;
     }
+}
+
+// sum_k w[oc][k] alone (the GEMM path unpacks the weight table itself); one wavefront per channel,
+// four 128-bit loads in flight per lane.
+__global__ __launch_bounds__(256) void nce_colsum_kernel(const int8_t* __restrict__ w, int32_t* __restrict__ colsum,
+                                                         int64_t OC, int64_t K) {
+    const int lane = threadIdx.x & 63;
+    const int64_t oc = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (oc >= OC) return;
+    const int8_t* row = w + oc * K;
+    int s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+    int64_t k = (int64_t)lane * 16;
+    for (; k + 3 * 1024 < K; k += 4 * 1024) {
+        const i32x4 q0 = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(row + k));
+        const i32x4 q1 = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(row + k + 1024));
+        const i32x4 q2 = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(row + k + 2048));
+        const i32x4 q3 = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(row + k + 3072));
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            s0 = __builtin_amdgcn_sdot4(q0[j], 0x01010101, s0, false);
+            s1 = __builtin_amdgcn_sdot4(q1[j], 0x01010101, s1, false);
+            s2 = __builtin_amdgcn_sdot4(q2[j], 0x01010101, s2, false);
+            s3 = __builtin_amdgcn_sdot4(q3[j], 0x01010101, s3, false);
+        }
+    }
+    for (; k < K; k += 1024) {
+        const i32x4 q = *reinterpret_cast<const i32x4*>(row + k);
+#pragma unroll
+        for (int j = 0; j < 4; j++) s0 = __builtin_amdgcn_sdot4(q[j], 0x01010101, s0, false);
+    }
+    int sum = (s0 + s1) + (s2 + s3);
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    if (lane == 0) colsum[oc] = sum;
 }
 
 // ---------------------------------------------------------------- naive path
@@ -137,34 +231,95 @@ __global__ __launch_bounds__(256) void nce_conv_naive(const uint8_t* __restrict_
         }
     }
     const uint32_t w2 = (uint32_t)wt[oc * 4 + 2];
-    ChanParams c{wt[oc * 4 + 3], (int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu), 0};
+    ChanParams c{wt[oc * 4 + 3], (int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu)};
     out[idx] = saturate8<OUT_SIGNED>(ppe_requant(acc, c, ppe));
 }
 
 // ---------------------------------------------------------------- GEMM path
 // LDS tile of ROWS x BK bytes; the 16-byte chunk c of row r is kept at chunk slot c ^ swz(r) so
-// that the 16 lanes served together by a 128-bit LDS read hit 16 different bank groups.
+// that the lanes served together by a 128-bit LDS read hit different bank groups.
+template <int BK>
+__device__ __forceinline__ int lds_swz(int row) {
+    constexpr int CPR = BK / 16;   // chunks per row
+    constexpr int RPW = 16 / CPR;  // rows per 256-byte bank wrap
+    return (row / RPW) % CPR;
+}
 template <int BK>
 __device__ __forceinline__ int lds_offset(int row, int chunk) {
-    constexpr int CPR = BK / 16;        // chunks per row
-    constexpr int RPW = 16 / CPR;       // rows per 256-byte bank wrap
-    return row * BK + ((chunk ^ ((row / RPW) % CPR)) << 4);
+    return row * BK + ((chunk ^ lds_swz<BK>(row)) << 4);
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool IN_U8, bool OUT_SIGNED>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void nce_gemm_mfma(
-        const int8_t* __restrict__ A, const int8_t* __restrict__ B, const ChanParams* __restrict__ params,
-        uint8_t* __restrict__ out, int64_t M, int64_t N, int64_t K, int tiles_m, int tiles_n, Ppe ppe) {
-    constexpr int NT = (BM / WM) * (BN / WN) * 64;
-    constexpr int CPR = BK / 16;
-    constexpr int A_CHUNKS = BM * CPR / NT;  // 16-byte chunks per lane per K step
-    constexpr int B_CHUNKS = BN * CPR / NT;
-    constexpr int TM = WM / 32, TN = WN / 32;
-    static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "tile does not split evenly over the lanes");
+// 16 bytes per lane from global memory straight into LDS: the wave's 64 lanes fill the 1 KiB that
+// starts at the wave-uniform LDS byte address `lds_addr`, lane l at +16*l.  Issued as assembly so
+// that the compiler keeps managing only the counter of the LDS reads; completion of these loads is
+// awaited explicitly with dma_wait_all_and_barrier().
+__device__ __forceinline__ void dma16(const void* gptr, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
+}
+// same, the source given as a wave-uniform base plus a 32-bit per-lane byte offset
+__device__ __forceinline__ void dma16(const void* gbase, unsigned goff, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(goff), "s"(gbase) : "memory");
+}
+__device__ __forceinline__ void dma_wait_all_and_barrier() {
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <typename T>
+__device__ __forceinline__ unsigned lds_address(T* p) {
+    return (unsigned)(size_t)(__attribute__((address_space(3))) char*)(p);
+}
+
+template <int CTRL>
+__device__ __forceinline__ unsigned dpp_u32(unsigned v) {
+    return (unsigned)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, 0xf, 0xf, true);
+}
+
+// Each lane of a quad holds one dword = 4 bytes of ONE column (rows R..R+3).  Afterwards lane t of
+// the quad holds row R+t of the quad's FOUR columns, i.e. 4 bytes that are adjacent in memory.
+__device__ __forceinline__ unsigned quad_transpose_bytes(unsigned w, int lane) {
+    const unsigned p = dpp_u32<0xB1>(w);  // lane ^ 1
+    // even lane: [w.b0, p.b0, w.b2, p.b2]   odd lane: [p.b1, w.b1, p.b3, w.b3]
+    // (v_perm_b32 selector bytes: 0-3 pick from the second source, 4-7 from the first)
+    const unsigned sel1 = (lane & 1) ? 0x03070105u : 0x06020400u;
+    const unsigned a = __builtin_amdgcn_perm(p, w, sel1);
+    const unsigned q = dpp_u32<0x4E>(a);  // lane ^ 2
+    // lanes 0,1: [a.b0, a.b1, q.b0, q.b1]   lanes 2,3: [q.b2, q.b3, a.b2, a.b3]
+    const unsigned sel2 = (lane & 2) ? 0x03020706u : 0x05040100u;
+    return __builtin_amdgcn_perm(q, a, sel2);
+}
+
+constexpr int kOutStride = 288;  // bytes per row of the 256-column output staging tile in LDS
+
+struct GemmPpe {
+    int prelu_mult, prelu_shift;  // applied to negative scaled values (1,0 = none; 0,0 = ReLU)
+    int corr;                     // zero-point term: acc_true = acc_raw + corr * sum_k B[n][k]
+    int zp_out, lo, hi;           // clamp bounds already intersected with the storage range
+};
+
+// A[M][K] x B[N][K]^T with the PPE fused; see the file header.  K must be a multiple of 64.
+//
+// Pipeline.  K is walked in panels of 64 bytes; a panel of A and B (32 KiB) goes from global memory
+// straight into one of four LDS buffers.  In iteration kt the waves multiply panel kt, fetch panel
+// kt+3 (8 DMA instructions per wave, spread between the MFMAs) and read the fragments one sub-step
+// ahead; the only wait is for panel kt+1, which was requested two iterations earlier, and it sits
+// with the workgroup barrier in the middle of the iteration, between the two sub-steps,
+// so that the MFMAs of the second sub-step cover the first fragment reads of panel kt+1.  The column sums of B that the zero-point
+// term needs come from nce_colsum_kernel (only when that term is not zero), and the per-column PPE
+// parameters are unpacked from the weight table in the epilogue.
+template <bool IN_U8, bool OUT_SIGNED>
+__global__ __launch_bounds__(256) void nce_gemm_mfma(const int8_t* __restrict__ A, const int8_t* __restrict__ B,
+                                                     const int32_t* __restrict__ wt, const int32_t* __restrict__ colsum,
+                                                     uint8_t* __restrict__ out,
+                                                     int64_t M, int64_t N, int64_t K, int tiles_m, int tiles_n,
+                                                     GemmPpe ppe) {
+    constexpr int BM = 256, BN = 256, BK = 64, WM = 128, WN = 128, TM = 4, TN = 4;
+    constexpr int NS = 4;                             // LDS panel buffers
+    constexpr int CPR = BK / 16;                      // 16-byte chunks per tile row
+    constexpr int RPI = 64 / CPR;                     // tile rows one 1 KiB DMA instruction covers
+    constexpr int DMA_PER_WAVE = BM * BK / 1024 / 4;  // per operand, per panel: 4
+    constexpr int STAGE = (BM + BN) * BK;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    uint8_t* sA = smem;                  // [2][BM][BK]
-    uint8_t* sB = smem + 2 * BM * BK;    // [2][BN][BK]
 
     // Workgroup ids are dealt round-robin to the 8 XCDs.  Give each XCD a contiguous run of tile
     // ids and walk tiles in groups of 4 tile-rows, so that workgroups resident on one XCD at the
@@ -182,28 +337,37 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void nce_gemm_mfma(
     const int tn = in_group / gsz;
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm0 = (wave / (BN / WN)) * WM, wn0 = (wave % (BN / WN)) * WN;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
 
-    const int8_t* ga[A_CHUNKS];
-    const int8_t* gb[B_CHUNKS];
-    int la[A_CHUNKS], lb[B_CHUNKS];
+    // Source addresses of this lane's DMA chunks.  Instruction q of a panel fills LDS bytes
+    // [q*1024, q*1024+1024) of the operand's tile = rows q*RPI .. ; the lane sitting at chunk slot p
+    // of row r fetches source chunk p ^ swz(r), which is what puts the swizzle in place.
+    unsigned oa[DMA_PER_WAVE], ob[DMA_PER_WAVE];  // byte offsets from the tile's first row
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; i++) {
-        const int cid = tid + NT * i, row = cid / CPR, c = cid % CPR;
-        int64_t m = m0 + row;
+    for (int i = 0; i < DMA_PER_WAVE; i++) {
+        const int q = wave + 4 * i;
+        const int r = q * RPI + lane / CPR, p = lane % CPR;
+        const int c = p ^ lds_swz<BK>(r);
+        int64_t m = m0 + r, n = n0 + r;
         m = m < M ? m : M - 1;  // rows past the edge repeat the last one; their outputs are not stored
-        ga[i] = A + m * K + c * 16;
-        la[i] = lds_offset<BK>(row, c);
-    }
-#pragma unroll
-    for (int i = 0; i < B_CHUNKS; i++) {
-        const int cid = tid + NT * i, row = cid / CPR, c = cid % CPR;
-        int64_t n = n0 + row;
         n = n < N ? n : N - 1;
-        gb[i] = B + n * K + c * 16;
-        lb[i] = lds_offset<BK>(row, c);
+        oa[i] = (unsigned)((m - m0) * K + c * 16);
+        ob[i] = (unsigned)((n - n0) * K + c * 16);
     }
+    const int8_t* abase = A + m0 * K;
+    const int8_t* bbase = B + n0 * K;
+    const unsigned lds0 = lds_address(smem);
+    const int nk = (int)(K / BK);
+    // d-th DMA instruction (0..3 A, 4..7 B) of panel p; panels past the end re-fetch the last one into a
+    // buffer nobody reads, which keeps the number of loads in flight the same in every iteration
+    auto dma_one = [&](int p, int d) {
+        const unsigned base = lds0 + (unsigned)((p & (NS - 1)) * STAGE);
+        const int64_t k0 = (int64_t)(p < nk ? p : nk - 1) * BK;
+        if (d < DMA_PER_WAVE) dma16(abase + k0, oa[d], base + (unsigned)((wave + 4 * d) * 1024));
+        else dma16(bbase + k0, ob[d - DMA_PER_WAVE], base + (unsigned)(BM * BK + (wave + 4 * (d - DMA_PER_WAVE)) * 1024));
+    };
 
     i32x16 acc[TM][TN];
 #pragma unroll
@@ -213,65 +377,101 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void nce_gemm_mfma(
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
-    i32x4 ra[A_CHUNKS], rb[B_CHUNKS];
-    auto load_global = [&](int64_t k0) {
-#pragma unroll
-        for (int i = 0; i < A_CHUNKS; i++) {
-            ra[i] = *reinterpret_cast<const i32x4*>(ga[i] + k0);
-            if (IN_U8) ra[i] ^= (int32_t)0x80808080;
-        }
-#pragma unroll
-        for (int i = 0; i < B_CHUNKS; i++) rb[i] = *reinterpret_cast<const i32x4*>(gb[i] + k0);
+    i32x4 fa[2][TM], fb[2][TN];
+    auto load_frag = [&](const uint8_t* pa, int kk, int slot, int n) {
+        const int chunk = kk * 2 + (lane >> 5);
+        if (n == 0) fa[slot][0] = *reinterpret_cast<const i32x4*>(pa + lds_offset<BK>(wm0 + (lane & 31), chunk));
+        else if (n <= TN) fb[slot][n - 1] = *reinterpret_cast<const i32x4*>(pa + BM * BK + lds_offset<BK>(wn0 + (n - 1) * 32 + (lane & 31), chunk));
+        else fa[slot][n - TN] = *reinterpret_cast<const i32x4*>(pa + lds_offset<BK>(wm0 + (n - TN) * 32 + (lane & 31), chunk));
     };
-    auto store_lds = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < A_CHUNKS; i++) *reinterpret_cast<i32x4*>(sA + buf * BM * BK + la[i]) = ra[i];
-#pragma unroll
-        for (int i = 0; i < B_CHUNKS; i++) *reinterpret_cast<i32x4*>(sB + buf * BN * BK + lb[i]) = rb[i];
-    };
-
-    const int nk = (int)(K / BK);
-    load_global(0);
-    store_lds(0);
-    __syncthreads();
-    for (int kt = 0; kt < nk; kt++) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) load_global((int64_t)(kt + 1) * BK);
-        const uint8_t* pa = sA + buf * BM * BK;
-        const uint8_t* pb = sB + buf * BN * BK;
-#pragma unroll
-        for (int kk = 0; kk < BK / 32; kk++) {
-            i32x4 fa[TM], fb[TN];
-            const int chunk = kk * 2 + (lane >> 5);
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-                fa[i] = *reinterpret_cast<const i32x4*>(pa + lds_offset<BK>(wm0 + i * 32 + (lane & 31), chunk));
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-                fb[j] = *reinterpret_cast<const i32x4*>(pb + lds_offset<BK>(wn0 + j * 32 + (lane & 31), chunk));
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) store_lds(buf ^ 1);
-        __syncthreads();
-    }
-
-    // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const int64_t n = n0 + wn0 + j * 32 + (lane & 31);
-        if (n >= N) continue;
-        const ChanParams cp = params[n];
+    // One sub-step: 16 MFMAs on fragment slot `cur`; between them, the 8 fragment reads of the next
+    // sub-step (panel at pnext, sub-step knext) into the other slot, DMA instructions dma0..dma0+3 of
+    // panel dma_p, and the column-sum update.
+    auto substep = [&](int cur, const uint8_t* pnext, int knext, int dma_p, int dma0) {
 #pragma unroll
         for (int i = 0; i < TM; i++) {
+            i32x4 a = fa[cur][i];
+            if (IN_U8) a ^= (int32_t)0x80808080;  // u8 -> s8 (value - 128)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int64_t m = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                if (m < M) out[m * N + n] = saturate8<OUT_SIGNED>(ppe_requant(acc[i][j][r], cp, ppe));
+            for (int j = 0; j < TN; j++) {
+                const int idx = i * TN + j;
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, fb[cur][j], acc[i][j], 0, 0, 0);
+                if (idx < TM + TN) load_frag(pnext, knext, cur ^ 1, idx);  // early: all back before the barrier
+                if ((idx & 3) == 3) dma_one(dma_p, dma0 + (idx >> 2));
+                __builtin_amdgcn_sched_barrier(0);
             }
+        }
+    };
+
+#pragma unroll
+    for (int p = 0; p < NS - 1; p++)
+#pragma unroll
+        for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
+    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");  // panel 0 is in
+#pragma unroll
+    for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
+    for (int kt = 0; kt < nk; kt++) {
+        const uint8_t* pcur = smem + (kt & (NS - 1)) * STAGE;
+        const uint8_t* pnxt = smem + ((kt + 1) & (NS - 1)) * STAGE;
+        substep(0, pcur, 1, kt + NS - 1, 0);
+        // Loads in flight here, oldest first: panel kt+1 (8), panel kt+2 (8), half of panel kt+3 (4).
+        // Behind the barrier panel kt+1 is complete for every wave and nobody reads panel kt-1 any
+        // more, whose buffer panel kt+3 is being written to.
+        asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        substep(1, pnxt, 0, kt + NS - 1, DMA_PER_WAVE);
+    }
+    dma_wait_all_and_barrier();  // every wave is done with the panels: LDS becomes the output staging tile
+
+    // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
+    ChanPrep cp[TN];
+    bool clip = false;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        int64_t n = n0 + wn0 + j * 32 + (lane & 31);
+        n = n < N ? n : N - 1;
+        const int csum = colsum ? colsum[n] : 0;  // sum_k B[n][k], present when the zero-point term is not 0
+        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        cp[j] = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+                            (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * csum)), ppe.prelu_mult, ppe.prelu_shift);
+        clip = clip || cp[j].bmax_pos != 0x7fffffff || cp[j].bmax_neg != 0x7fffffff;
+        // keep the prepared factors in registers: without this the compiler re-derives them per element
+        asm volatile("" : "+v"(cp[j].f_pos), "+v"(cp[j].f_neg));
+    }
+    const PpeFast pf{ppe.zp_out, ppe.lo, ppe.hi};
+    auto requant_tile = [&](auto clip_c) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col4 = wn0 + j * 32 + ((lane & 31) & ~3);
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    unsigned w = 0;
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        w |= (unsigned)(ppe_fast<decltype(clip_c)::value>(acc[i][j][g * 4 + r], cp[j], pf) & 0xff) << (8 * r);
+                    w = quad_transpose_bytes(w, lane);
+                    const int row = wm0 + i * 32 + 8 * g + 4 * (lane >> 5) + (lane & 3);
+                    *reinterpret_cast<unsigned*>(smem + row * kOutStride + col4) = w;
+                }
+            }
+        }
+    };
+    // scale factors above 1/2 are rare (shift < 15): only then is the clipping variant needed
+    if (__builtin_amdgcn_ballot_w64(clip) != 0) requant_tile(std::true_type{});
+    else requant_tile(std::false_type{});
+    __syncthreads();
+    const bool vec_ok = (N & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    for (int it = 0; it < BM * (BN / 16) / 256; it++) {
+        const int cid = tid + 256 * it;
+        const int row = cid >> 4, c16 = cid & 15;
+        const int64_t m = m0 + row, n = n0 + c16 * 16;
+        if (m >= M || n >= N) continue;
+        const i32x4 v = *reinterpret_cast<const i32x4*>(smem + row * kOutStride + c16 * 16);
+        if (vec_ok && n + 16 <= N) {
+            __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(out + m * N + n));
+        } else {
+            for (int e = 0; e < 16 && n + e < N; e++) out[m * N + n + e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
         }
     }
 }
@@ -279,11 +479,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void nce_gemm_mfma(
 // ---------------------------------------------------------------- implicit-GEMM convolution path
 // Workgroup: BM output positions (flattened n, oy, ox) x BN output channels, 4 waves split BM.
 // The weights of the BN channels, all taps, sit in LDS as [BN][KY*KX*IC] rows (swizzle as above
-// on 64-byte granules, applied when a row is a whole number of them); activation fragments come straight from global memory, 16 bytes per lane.
+// on 64-byte granules, applied when a row is a whole number of them); activation fragments come
+// straight from global memory, 16 bytes per lane.
 template <int BM, int BN, bool IN_U8, bool OUT_SIGNED>
 __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
-                                                     const ChanParams* __restrict__ params, uint8_t* __restrict__ out,
-                                                     ConvGeom g, int pad_byte, int swz, Ppe ppe) {
+                                                     const ChanPrep* __restrict__ prep, uint8_t* __restrict__ out,
+                                                     ConvGeom g, int pad_byte, int swz, PpeFast ppe) {
     constexpr int WM = BM / 4;
     constexpr int TM = WM / 32, TN = BN / 32;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // [BN][Ktot]
@@ -309,12 +510,10 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
     // positions of this lane's rows
     int64_t base_n[TM];
     int oy[TM], ox[TM];
-    bool live[TM];
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         int64_t m = m0 + wave * WM + i * 32 + (lane & 31);
-        live[i] = m < Mtot;
-        m = live[i] ? m : Mtot - 1;
+        m = m < Mtot ? m : Mtot - 1;
         ox[i] = (int)(m % g.OW);
         oy[i] = (int)((m / g.OW) % g.OH);
         base_n[i] = (m / (g.OW * g.OH)) * g.H * g.W * g.IC;
@@ -371,13 +570,13 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
     for (int j = 0; j < TN; j++) {
         const int64_t oc = oc0 + j * 32 + (lane & 31);
         if (oc >= g.OC) continue;
-        const ChanParams cp = params[oc];
+        const ChanPrep cp = prep[oc];
 #pragma unroll
         for (int i = 0; i < TM; i++) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t m = m0 + wave * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                if (m < Mtot) out[m * g.OC + oc] = saturate8<OUT_SIGNED>(ppe_requant(acc[i][j][r], cp, ppe));
+                if (m < Mtot) out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(acc[i][j][r], cp, ppe);
             }
         }
     }
@@ -424,7 +623,9 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     if (Mtot == 0 || g.OC == 0) return VPX_RESULT_SUCCESS;
 
     const bool zp_in_ok = in_u8 ? (t.zp_in >= 0 && t.zp_in <= 255) : (t.zp_in >= -128 && t.zp_in <= 127);
-    const bool mfma_ok = !w_u8 && t.zp_w == 0 && zp_in_ok && Mtot < (1ll << 31) && g.OC < (1ll << 31);
+    // the fast epilogue adds the output zero point after limiting the scaled value to +-2^30
+    const bool zp_out_ok = t.zp_out >= -(1 << 20) && t.zp_out <= (1 << 20);
+    const bool mfma_ok = !w_u8 && t.zp_w == 0 && zp_in_ok && zp_out_ok && Mtot < (1ll << 31) && g.OC < (1ll << 31);
     const bool is_gemm = g.KY == 1 && g.KX == 1 && g.SY == 1 && g.SX == 1 && t.kernel_padding[0] == 0 &&
                          t.kernel_padding[1] == 0 && t.kernel_padding[2] == 0 && t.kernel_padding[3] == 0;
     const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights)) & 15) == 0;
@@ -434,30 +635,42 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const bool allow_gemm = !force || !*force;
     const bool allow_mfma = allow_gemm || std::strcmp(force, "conv") == 0;
 
-    const bool use_gemm = allow_gemm && is_gemm && g.IC % 64 == 0;
+    const bool use_gemm = allow_gemm && is_gemm && g.IC % 64 == 0 && g.IC < (1 << 24);
     if (allow_mfma && mfma_ok && aligned && (use_gemm || (g.IC % 32 == 0 && 64 * Ktot <= 128 * 1024))) {
-        void* ws = nullptr;
-        int rc = get_workspace(s, sizeof(ChanParams) * (size_t)g.OC, &ws);
-        if (rc) return rc;
-        ChanParams* params = (ChanParams*)ws;
+        int rc = VPX_RESULT_SUCCESS;
         const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
-        hipLaunchKernelGGL(nce_fold_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s, (const int8_t*)t.weights,
-                           t.weight_table, params, g.OC, Ktot, corr);
-        VPX_HIP_CHECK(hipGetLastError());
+        PpeFast pf;
+        pf.zp_out = t.zp_out;
+        const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
+        pf.lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin;
+        pf.hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
+        if (pf.lo > tmax) pf.lo = tmax;  // clamp window entirely above / below the storage range
+        if (pf.hi < tmin) pf.hi = tmin;
 
         if (use_gemm) {
-            constexpr int BM = 256, BN = 256, BK = 64, WM = 128, WN = 128;
+            constexpr int BM = 256, BN = 256;
             const int tiles_m = (int)((Mtot + BM - 1) / BM), tiles_n = (int)((g.OC + BN - 1) / BN);
             const int per_xcd = (tiles_m * tiles_n + 7) / 8;
-            const size_t lds = 2 * (BM + BN) * BK;
-            const dim3 grid((unsigned)(per_xcd * 8)), block((BM / WM) * (BN / WN) * 64);
+            const dim3 grid((unsigned)(per_xcd * 8)), block(256);
+            const size_t lds = 4 * (BM + BN) * 64;  // four K panels; the output staging tile reuses them
+            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi};
+            int32_t* colsum = nullptr;
+            if (corr != 0) {
+                void* ws = nullptr;
+                rc = get_workspace(s, sizeof(int32_t) * (size_t)g.OC, &ws);
+                if (rc) return rc;
+                colsum = (int32_t*)ws;
+                hipLaunchKernelGGL(nce_colsum_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s,
+                                   (const int8_t*)t.weights, colsum, g.OC, Ktot);
+                VPX_HIP_CHECK(hipGetLastError());
+            }
 #define VPX_GEMM(U8, SGN)                                                                                            \
     do {                                                                                                             \
-        auto kern = nce_gemm_mfma<BM, BN, BK, WM, WN, U8, SGN>;                                                      \
+        auto kern = nce_gemm_mfma<U8, SGN>;                                                                        \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
-        hipLaunchKernelGGL(kern, grid, block, lds, s, (const int8_t*)t.input, (const int8_t*)t.weights, params,      \
-                           (uint8_t*)t.output, Mtot, g.OC, g.IC, tiles_m, tiles_n, ppe);                            \
+        hipLaunchKernelGGL(kern, grid, block, lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,              \
+                           t.weight_table, colsum, (uint8_t*)t.output, Mtot, g.OC, g.IC, tiles_m, tiles_n, gp);             \
     } while (0)
             if (in_u8 && out_signed) VPX_GEMM(true, true);
             else if (in_u8) VPX_GEMM(true, false);
@@ -469,6 +682,15 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             return VPX_RESULT_SUCCESS;
         }
 
+        // the convolution path takes its per-channel parameters from a small preparation kernel
+        void* ws = nullptr;
+        rc = get_workspace(s, sizeof(ChanPrep) * (size_t)g.OC, &ws);
+        if (rc) return rc;
+        ChanPrep* prep = (ChanPrep*)ws;
+        hipLaunchKernelGGL(nce_fold_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s, (const int8_t*)t.weights,
+                           t.weight_table, prep, g.OC, Ktot, corr, ppe);
+        VPX_HIP_CHECK(hipGetLastError());
+
         constexpr int BM = 256, BN = 64;
         const size_t lds = (size_t)BN * Ktot;
         const dim3 grid((unsigned)((Mtot + BM - 1) / BM), (unsigned)((g.OC + BN - 1) / BN));
@@ -479,8 +701,8 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         auto kern = nce_conv_mfma<BM, BN, U8, SGN>;                                                                  \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights, params,  \
-                           (uint8_t*)t.output, g, pad_byte, swz, ppe);                                                  \
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights, prep,    \
+                           (uint8_t*)t.output, g, pad_byte, swz, pf);                                                \
     } while (0)
         if (in_u8 && out_signed) VPX_CONV(true, true);
         else if (in_u8) VPX_CONV(true, false);
