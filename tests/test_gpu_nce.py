@@ -58,16 +58,20 @@ U8 = {"clamp_low": 0, "clamp_high": 255}
 I8 = {"clamp_low": -128, "clamp_high": 127}
 
 
-@pytest.mark.parametrize("force,expect", [(None, "nce_conv_mfma"), ("naive", "nce_conv_naive")])
+@pytest.mark.parametrize("force", [None, "gather", "naive"])
 @pytest.mark.parametrize("geom", [
     dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
     dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)),
     dict(N=3, H=8, W=5, IC=64, OC=70, KY=1, KX=3, strides=(1, 1), pads=(1, 0, 0, 0)),
     dict(N=1, H=20, W=20, IC=64, OC=32, KY=5, KX=5, strides=(1, 2), pads=(2, 2, 2, 2)),
+    dict(N=2, H=30, W=40, IC=128, OC=96, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
+    dict(N=1, H=33, W=70, IC=64, OC=16, KY=3, KX=2, strides=(2, 1), pads=(0, 1, 2, 0)),
 ])
-def test_conv_paths(rt, orc, dev, geom, force, expect):
+def test_conv_paths(rt, orc, dev, geom, force):
     g = dict(geom)
     strides, pads = g.pop("strides"), g.pop("pads")
+    expect = {None: "nce_conv_patch" if g["IC"] % 64 == 0 else "nce_conv_mfma", "gather": "nce_conv_mfma",
+              "naive": "nce_conv_naive"}[force]
     rng = np.random.default_rng(50 + g["H"])
     for in_u8, zp_in, out_signed in ((True, 128, False), (True, 7, True), (False, -5, False), (False, 0, True)):
         inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, **g)
@@ -75,6 +79,21 @@ def test_conv_paths(rt, orc, dev, geom, force, expect):
                                    strides=strides, pads=pads, out_signed=out_signed, force=force)
         assert name == expect
         assert np.array_equal(got, want), "%s zp_in=%d: %d mismatches" % (name, zp_in, int((got != want).sum()))
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3, 5])
+def test_conv_patch_tile_heights(rt, orc, dev, rows):
+    """The patch kernel with its tile height forced: tiles that end past the last output row, one-row tiles."""
+    rng = np.random.default_rng(55 + rows)
+    inp, w, mults, shifts, bias = rand_case(rng, 2, 13, 24, 64, 80, 3, 3)
+    os.environ["VPX_CONV_ROWS"] = str(rows)
+    try:
+        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, U8, zp_in=121, zp_out=3,
+                                   strides=(1, 1), pads=(1, 1, 1, 1))
+    finally:
+        del os.environ["VPX_CONV_ROWS"]
+    assert name == "nce_conv_patch"
+    assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
 
 
 def test_naive_path_covers_odd_shapes_and_weight_zero_points(rt, orc, dev):
@@ -125,7 +144,7 @@ def test_conv_config_c4_full_size(rt, orc, dev):
     got, want, name = run_task(rt, orc, dev, c["input"], c["weights"], c["mult"], c["shift"], c["bias"],
                                {"clamp_low": c["clamp"][0], "clamp_high": c["clamp"][1]}, zp_in=c["zp_in"],
                                strides=c["strides"], pads=c["pads"])
-    assert name == "nce_conv_mfma"
+    assert name == "nce_conv_patch"
     assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
     assert 0 < (got == 0).mean() < 0.9  # the ReLU clamp is active and the output is not saturated flat
 

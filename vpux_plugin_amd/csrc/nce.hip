@@ -582,6 +582,233 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
     }
 }
 
+// ---------------------------------------------------------------- convolution with the input patch in LDS
+// Workgroup: `R` whole output rows of one image x 64 output channels.  The (R-1)*SY+KY input rows
+// the tile needs are copied to LDS once, padding materialised with the zero-point byte and u8
+// re-biased to s8 on the way, so every tap of every output position is an LDS read; the weights of
+// the 64 channels sit beside them.  One launch does everything: the per-channel weight sums of the
+// zero-point term come from the LDS copy of the weights and the PPE parameters are unpacked from
+// the weight table in the epilogue.
+//
+// LDS layouts (16-byte chunks):
+//   weights [64][Ktot]      chunk c of row r at c ^ ((r >> 2) & 3) when Ktot is a multiple of 64
+//   patch   [PH*PW][IC]     chunk c of pixel p at c ^ ((p >> 2) & 3)   (IC is a multiple of 64)
+// Lanes 0-31 of a fragment read walk consecutive rows / pixels at one chunk index; the xor spreads
+// them over all banks.
+//
+// Waves: the tile has MT = ceil(R*OW / 32) row blocks of 32 positions and one or two column blocks
+// of 32 channels; wave w takes column block w % nt and row blocks w / nt, w / nt + 4 / nt, ...
+struct PatchGeom {
+    int R;       // output rows per workgroup
+    int PH, PW;  // patch size in input pixels
+    int tiles_y; // workgroups per image
+    int MT;      // row blocks of 32 output positions per workgroup
+    int nt;      // column blocks of 32 channels in use (1 or 2)
+    int w_swz;   // weights rows are swizzled
+};
+
+constexpr int kPatchMaxMT = 14;
+constexpr int kPatchOutStride = 80;  // bytes per output position in the staging tile
+
+template <bool IN_U8>
+__global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
+                                                      const int32_t* __restrict__ wt, uint8_t* __restrict__ out,
+                                                      ConvGeom g, PatchGeom pg, int pad_byte, GemmPpe ppe) {
+    constexpr int BN = 64;
+    constexpr int TMW = kPatchMaxMT / 2;  // most row blocks per wave
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int Ktot = g.KY * g.KX * (int)g.IC;
+    const int IC = (int)g.IC;
+    uint8_t* const wlds = smem;                                 // [64][Ktot]
+    uint8_t* const patch = smem + BN * Ktot;                    // [PH*PW][IC], later the output staging tile
+    __shared__ int csum[BN];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int img = blockIdx.x / pg.tiles_y;
+    const int oy0 = (blockIdx.x % pg.tiles_y) * pg.R;
+    const int oc0 = blockIdx.y * BN;
+
+    // ---- weights -> LDS.  cid walks (row, chunk) pairs; 256 = dr * cpr + dc advances both without a division.
+    {
+        const int cpr = Ktot / 16;
+        const int dr = 256 / cpr, dc = 256 % cpr;
+        int row = tid / cpr, c = tid % cpr;
+        constexpr int UNR = 4;
+        while (row < BN) {
+            i32x4 q[UNR];
+            int dst[UNR];
+#pragma unroll
+            for (int u = 0; u < UNR; u++) {
+                dst[u] = -1;
+                if (row < BN) {
+                    int64_t oc = oc0 + row;
+                    oc = oc < g.OC ? oc : g.OC - 1;
+                    q[u] = *reinterpret_cast<const i32x4*>(w + oc * Ktot + c * 16);
+                    const int cs = pg.w_swz ? ((c & ~3) | ((c ^ (row >> 2)) & 3)) : c;
+                    dst[u] = row * Ktot + cs * 16;
+                }
+                row += dr;
+                c += dc;
+                if (c >= cpr) {
+                    c -= cpr;
+                    row++;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNR; u++)
+                if (dst[u] >= 0) *reinterpret_cast<i32x4*>(wlds + dst[u]) = q[u];
+        }
+    }
+
+    // ---- input patch -> LDS.  A unit is 64 consecutive chunks of one patch row; units go round the waves.
+    {
+        const int cpp = IC / 16;                  // chunks per pixel
+        const int row_chunks = pg.PW * cpp;
+        const int upr = (row_chunks + 63) / 64;   // units per patch row
+        const int units = pg.PH * upr;
+        const int pad32 = (pad_byte & 0xff) * 0x01010101;
+        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
+        constexpr int UNR = 4;
+        for (int u0 = wave; u0 < units; u0 += 4 * UNR) {
+            i32x4 q[UNR];
+            int dst[UNR];
+#pragma unroll
+            for (int u = 0; u < UNR; u++) {
+                const int unit = u0 + 4 * u;
+                dst[u] = -1;
+                if (unit < units) {
+                    const int py = unit / upr;  // wave-uniform
+                    const int qi = (unit - py * upr) * 64 + lane;
+                    if (qi < row_chunks) {
+                        const int px = (int)((unsigned)qi / (unsigned)cpp), c = qi - px * cpp;
+                        const int iy = oy0 * g.SY - g.PT + py, ix = px - g.PL;
+                        const bool inside = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+                        i32x4 v = i32x4{pad32, pad32, pad32, pad32};
+                        if (inside) v = *reinterpret_cast<const i32x4*>(img_base + ((int64_t)iy * g.W + ix) * IC + c * 16);
+                        if (IN_U8) v ^= (int32_t)0x80808080;
+                        q[u] = v;
+                        const int pp = py * pg.PW + px;
+                        dst[u] = pp * IC + (((c & ~3) | ((c ^ (pp >> 2)) & 3)) << 4);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UNR; u++)
+                if (dst[u] >= 0) *reinterpret_cast<i32x4*>(patch + dst[u]) = q[u];
+        }
+    }
+    __syncthreads();
+
+    // ---- per-channel weight sums from the LDS copy (chunk order within a row does not matter)
+    if (ppe.corr != 0) {
+        const int row = tid >> 2, part = tid & 3;
+        int sum = 0;
+        for (int c = part; c < Ktot / 16; c += 4) {
+            const i32x4 q = *reinterpret_cast<const i32x4*>(wlds + row * Ktot + c * 16);
+#pragma unroll
+            for (int j = 0; j < 4; j++) sum = __builtin_amdgcn_sdot4(q[j], 0x01010101, sum, false);
+        }
+        sum += (int)dpp_u32<0xB1>((unsigned)sum);
+        sum += (int)dpp_u32<0x4E>((unsigned)sum);
+        if (part == 0) csum[row] = sum;
+    }
+
+    // ---- main loop
+    const int nj = wave % pg.nt;               // column block of this wave
+    const int mi0 = wave / pg.nt, mstep = 4 / pg.nt;
+    const int npos = pg.R * (int)g.OW;         // output positions of a full tile
+    int pp0[TMW];
+#pragma unroll
+    for (int i = 0; i < TMW; i++) {
+        int p = (mi0 + i * mstep) * 32 + (lane & 31);
+        p = p < npos ? p : 0;
+        const int r = (int)((unsigned)p / (unsigned)g.OW), ox = p - r * (int)g.OW;
+        pp0[i] = r * g.SY * pg.PW + ox * g.SX;
+    }
+    i32x16 acc[TMW];
+#pragma unroll
+    for (int i = 0; i < TMW; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0;
+
+    const int kgroup = lane >> 5;
+    const int brow = nj * 32 + (lane & 31);
+    const uint8_t* const bbase = wlds + brow * Ktot;
+    const int bsw = pg.w_swz ? (brow >> 2) & 3 : 0;
+    for (int ky = 0; ky < g.KY; ky++) {
+        for (int kx = 0; kx < g.KX; kx++) {
+            const int tap_pp = ky * pg.PW + kx;
+            const int ctap = (ky * g.KX + kx) * (IC / 16);
+            int abase[TMW], asw[TMW];
+#pragma unroll
+            for (int i = 0; i < TMW; i++) {
+                const int pp = pp0[i] + tap_pp;
+                abase[i] = pp * IC;
+                asw[i] = (pp >> 2) & 3;
+            }
+            for (int ic = 0; ic < IC; ic += 32) {
+                const int c = ic / 16 + kgroup;
+                const int cb = ctap + c;
+                const i32x4 fb = *reinterpret_cast<const i32x4*>(bbase + (((cb & ~3) | ((cb ^ bsw) & 3)) << 4));
+                i32x4 fa[TMW];
+#pragma unroll
+                for (int i = 0; i < TMW; i++)
+                    if (mi0 + i * mstep < pg.MT)
+                        fa[i] = *reinterpret_cast<const i32x4*>(patch + abase[i] + (((c & ~3) | ((c ^ asw[i]) & 3)) << 4));
+#pragma unroll
+                for (int i = 0; i < TMW; i++)
+                    if (mi0 + i * mstep < pg.MT)
+                        acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb, acc[i], 0, 0, 0);
+            }
+        }
+    }
+    __syncthreads();  // all waves are done with the patch: its LDS becomes the output staging tile
+
+    // ---- epilogue
+    {
+        int64_t n = oc0 + brow;
+        n = n < g.OC ? n : g.OC - 1;
+        const int cs = ppe.corr != 0 ? csum[brow] : 0;
+        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        ChanPrep cp = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+                                  (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
+        asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));
+        const PpeFast pf{ppe.zp_out, ppe.lo, ppe.hi};
+        const int col4 = nj * 32 + ((lane & 31) & ~3);
+#pragma unroll
+        for (int i = 0; i < TMW; i++) {
+            if (mi0 + i * mstep >= pg.MT) continue;
+#pragma unroll
+            for (int gq = 0; gq < 4; gq++) {
+                unsigned v = 0;
+#pragma unroll
+                for (int r = 0; r < 4; r++) v |= (unsigned)(ppe_fast<true>(acc[i][gq * 4 + r], cp, pf) & 0xff) << (8 * r);
+                v = quad_transpose_bytes(v, lane);
+                const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
+                *reinterpret_cast<unsigned*>(patch + row * kPatchOutStride + col4) = v;
+            }
+        }
+    }
+    __syncthreads();
+    const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
+    const int valid = rows_here * (int)g.OW;
+    const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
+    const bool vec_ok = (g.OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    for (int cid = tid; cid < valid * 4; cid += 256) {
+        const int row = cid >> 2, c16 = cid & 3;
+        const int64_t n = oc0 + c16 * 16;
+        if (n >= g.OC) continue;
+        const i32x4 v = *reinterpret_cast<const i32x4*>(patch + row * kPatchOutStride + c16 * 16);
+        uint8_t* dst = out + (pos0 + row) * g.OC + n;
+        if (vec_ok && n + 16 <= g.OC) {
+            __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
+        } else {
+            for (int e = 0; e < 16 && n + e < g.OC; e++) dst[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+        }
+    }
+}
+
 template <class KernelT>
 int set_dyn_lds(KernelT kernel, size_t bytes) {
     if (bytes > 64 * 1024) {
@@ -629,11 +856,12 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const bool is_gemm = g.KY == 1 && g.KX == 1 && g.SY == 1 && g.SX == 1 && t.kernel_padding[0] == 0 &&
                          t.kernel_padding[1] == 0 && t.kernel_padding[2] == 0 && t.kernel_padding[3] == 0;
     const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights)) & 15) == 0;
-    // VPX_NCE_KERNEL=naive|conv restricts the choice to the slower, more general paths (used by tests
+    // VPX_NCE_KERNEL=naive|gather|conv restricts the choice to the slower, more general paths (used by tests
     // to check the device paths against each other).
     const char* force = std::getenv("VPX_NCE_KERNEL");
     const bool allow_gemm = !force || !*force;
-    const bool allow_mfma = allow_gemm || std::strcmp(force, "conv") == 0;
+    const bool allow_patch = allow_gemm || std::strcmp(force, "conv") == 0;
+    const bool allow_mfma = allow_patch || std::strcmp(force, "gather") == 0;
 
     const bool use_gemm = allow_gemm && is_gemm && g.IC % 64 == 0 && g.IC < (1 << 24);
     if (allow_mfma && mfma_ok && aligned && (use_gemm || (g.IC % 32 == 0 && 64 * Ktot <= 128 * 1024))) {
@@ -682,7 +910,55 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             return VPX_RESULT_SUCCESS;
         }
 
-        // the convolution path takes its per-channel parameters from a small preparation kernel
+        // Preferred: input patch and weights in LDS, one launch.  R = output rows per workgroup.
+        if (allow_patch && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20)) {
+            PatchGeom pg{};
+            const size_t lds_max = 160 * 1024 - 512;
+            auto lds_need = [&](int R) {
+                const size_t patch = (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)g.IC;
+                const size_t stage = (size_t)((R * g.OW + 31) / 32) * 32 * kPatchOutStride;
+                return 64 * (size_t)Ktot + (patch > stage ? patch : stage);
+            };
+            int R = (int)(32 * kPatchMaxMT / g.OW);
+            if (R > g.OH) R = (int)g.OH;
+            while (R > 1 && lds_need(R) > lds_max) R--;
+            if (lds_need(R) <= lds_max) {
+                const int64_t ocb = (g.OC + 63) / 64;
+                // enough workgroups to fill the device twice, as long as a tile keeps at least 4 row blocks
+                while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 512 && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
+                if (const char* e = std::getenv("VPX_CONV_ROWS")) {
+                    const int v = std::atoi(e);
+                    if (v >= 1 && v <= R) R = v;
+                }
+                pg.tiles_y = (int)((g.OH + R - 1) / R);
+                pg.R = (int)((g.OH + pg.tiles_y - 1) / pg.tiles_y);
+                pg.PH = (pg.R - 1) * g.SY + g.KY;
+                pg.PW = (int)(g.OW - 1) * g.SX + g.KX;
+                pg.MT = (int)((pg.R * g.OW + 31) / 32);
+                pg.nt = g.OC <= 32 ? 1 : 2;
+                pg.w_swz = Ktot % 64 == 0 ? 1 : 0;
+                const size_t lds = lds_need(pg.R);
+                const dim3 grid((unsigned)(g.N * pg.tiles_y), (unsigned)ocb);
+                GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi};
+                const int pad_byte = t.zp_in & 0xff;
+                if (in_u8) {
+                    rc = set_dyn_lds(nce_conv_patch<true>, lds);
+                    if (rc) return rc;
+                    hipLaunchKernelGGL(nce_conv_patch<true>, grid, dim3(256), lds, s, (const int8_t*)t.input,
+                                       (const int8_t*)t.weights, t.weight_table, (uint8_t*)t.output, g, pg, pad_byte, gp);
+                } else {
+                    rc = set_dyn_lds(nce_conv_patch<false>, lds);
+                    if (rc) return rc;
+                    hipLaunchKernelGGL(nce_conv_patch<false>, grid, dim3(256), lds, s, (const int8_t*)t.input,
+                                       (const int8_t*)t.weights, t.weight_table, (uint8_t*)t.output, g, pg, pad_byte, gp);
+                }
+                VPX_HIP_CHECK(hipGetLastError());
+                *kernel_name = "nce_conv_patch";
+                return VPX_RESULT_SUCCESS;
+            }
+        }
+        // Fallback: activation fragments gathered from global memory; per-channel parameters come
+        // from a small preparation kernel.
         void* ws = nullptr;
         rc = get_workspace(s, sizeof(ChanPrep) * (size_t)g.OC, &ws);
         if (rc) return rc;

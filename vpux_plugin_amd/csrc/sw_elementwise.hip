@@ -13,24 +13,36 @@ typedef _Float16 half_t;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-// N elements of T held as whole 128-bit words, the unit every global access of the flat path moves.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+template <int BYTES>
+struct Words;
+template <>
+struct Words<4> {
+    typedef uint32_t type;
+};
+template <>
+struct Words<8> {
+    typedef u32x2 type;
+};
+template <>
+struct Words<16> {
+    typedef u32x4 type;
+};
+
+// N elements of T moved by one 32/64/128-bit access per lane.  Adjacent lanes touch adjacent
+// words, so a wavefront's access is one contiguous run; the wider operand of a kernel gets the
+// 128-bit form.  Stores are non-temporal (results are not re-read); loads are ordinary, which
+// measures faster than non-temporal loads on this memory system.
 template <typename T, int N>
 struct Pack {
-    static_assert((sizeof(T) * N) % 16 == 0, "a pack is a whole number of 128-bit words");
-    static constexpr int WORDS = sizeof(T) * N / 16;
-    u32x4 q[WORDS];
-    __device__ __forceinline__ T get(int k) const { return reinterpret_cast<const T*>(q)[k]; }
-    __device__ __forceinline__ void set(int k, T v) { reinterpret_cast<T*>(q)[k] = v; }
-    // streaming data is touched once: keep it out of the caches' way
-    __device__ __forceinline__ void load(const T* base, int64_t v) {
-        const u32x4* p = reinterpret_cast<const u32x4*>(base) + v * WORDS;
-#pragma unroll
-        for (int w = 0; w < WORDS; w++) q[w] = __builtin_nontemporal_load(p + w);
-    }
+    typedef typename Words<sizeof(T) * N>::type W;
+    W q;
+    __device__ __forceinline__ T get(int k) const { return reinterpret_cast<const T*>(&q)[k]; }
+    __device__ __forceinline__ void set(int k, T v) { reinterpret_cast<T*>(&q)[k] = v; }
+    __device__ __forceinline__ void load(const T* base, int64_t v) { q = reinterpret_cast<const W*>(base)[v]; }
     __device__ __forceinline__ void store(T* base, int64_t v) const {
-        u32x4* p = reinterpret_cast<u32x4*>(base) + v * WORDS;
-#pragma unroll
-        for (int w = 0; w < WORDS; w++) __builtin_nontemporal_store(q[w], p + w);
+        __builtin_nontemporal_store(q, reinterpret_cast<W*>(base) + v);
     }
 };
 
@@ -75,14 +87,14 @@ __device__ __forceinline__ float narrow<float>(float r) {
 
 // ---------------------------------------------------------------- flat streaming skeleton
 // F provides: static constexpr int VEC; void vec(int64_t v) (elements [v*VEC, v*VEC+VEC)); void one(int64_t i).
-template <class F>
-__global__ __launch_bounds__(kBlock) void stream_kernel(F f, int64_t n_vec, int64_t n) {
-    const int64_t block0 = (int64_t)blockIdx.x * (kBlock * kUnroll);
-    if (block0 + kBlock * kUnroll <= n_vec) {
-        f.template vecs<kUnroll>(block0 + threadIdx.x, kBlock);
+template <class F, int BLOCK, int UNROLL>
+__global__ __launch_bounds__(BLOCK) void stream_kernel(F f, int64_t n_vec, int64_t n) {
+    const int64_t block0 = (int64_t)blockIdx.x * (BLOCK * UNROLL);
+    if (block0 + BLOCK * UNROLL <= n_vec) {
+        f.template vecs<UNROLL>(block0 + threadIdx.x, BLOCK);
     } else {
-        for (int u = 0; u < kUnroll; u++) {
-            const int64_t v = block0 + u * kBlock + threadIdx.x;
+        for (int u = 0; u < UNROLL; u++) {
+            const int64_t v = block0 + u * BLOCK + threadIdx.x;
             if (v < n_vec) f.template vecs<1>(v, 0);
         }
     }
@@ -97,11 +109,18 @@ template <class F>
 int launch_stream(const F& f, int64_t n, hipStream_t s) {
     if (n <= 0) return VPX_RESULT_SUCCESS;
     const int64_t n_vec = n / F::VEC;
-    int64_t blocks = (n_vec + kBlock * kUnroll - 1) / (kBlock * kUnroll);
+    // A tensor too small to give every compute unit several full-size workgroups is latency-bound:
+    // fewer vectors per lane, and in the end single-wave workgroups, spread it over more units.
+    const int tier = n_vec >= (int64_t)kBlock * kUnroll * 2048 ? 2 : (n_vec >= (int64_t)kBlock * 1024 ? 1 : 0);
+    const int64_t per_block = tier == 2 ? kBlock * kUnroll : (tier == 1 ? kBlock : 64);
+    int64_t blocks = (n_vec + per_block - 1) / per_block;
     if (blocks < 1) blocks = 1;
     VPX_REQUIRE(blocks < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "tensor of %lld elements is too large",
                 (long long)n);
-    hipLaunchKernelGGL(stream_kernel<F>, dim3((unsigned)blocks), dim3(kBlock), 0, s, f, n_vec, n);
+    const dim3 grid((unsigned)blocks);
+    if (tier == 2) hipLaunchKernelGGL((stream_kernel<F, kBlock, kUnroll>), grid, dim3(kBlock), 0, s, f, n_vec, n);
+    else if (tier == 1) hipLaunchKernelGGL((stream_kernel<F, kBlock, 1>), grid, dim3(kBlock), 0, s, f, n_vec, n);
+    else hipLaunchKernelGGL((stream_kernel<F, 64, 1>), grid, dim3(64), 0, s, f, n_vec, n);
     VPX_HIP_CHECK(hipGetLastError());
     return VPX_RESULT_SUCCESS;
 }
@@ -208,12 +227,16 @@ struct QuantFn {
 };
 
 // vpux::dequantize, include/vpux/compiler/utils/quantization.hpp:208-210: double product -> float
-template <typename TQ, typename TO>
+// PLAIN: every nonzero result is at least 2^-14 in magnitude and finite, where the reference's
+// float16 rounding is plain round-to-nearest-even, one conversion instruction.
+template <typename TQ, typename TO, bool PLAIN>
 struct DequantFn {
     double scale;
     int zp;
     __device__ __forceinline__ TO operator()(TQ q) const {
-        return narrow<TO>((float)((double)((int)q - zp) * scale));
+        const float r = (float)((double)((int)q - zp) * scale);
+        if (PLAIN) return (TO)r;
+        return narrow<TO>(r);
     }
 };
 
@@ -310,7 +333,7 @@ template <typename TI, typename TO, class Fn>
 static int convert_impl(const MemRef& in, const MemRef& out, Fn fn, hipStream_t s) {
     const int64_t n = out.numel();
     if (in.compact && out.compact && aligned16(in.data) && aligned16(out.data)) {
-        constexpr int VEC = 16 / (sizeof(TI) < sizeof(TO) ? sizeof(TI) : sizeof(TO));
+        constexpr int VEC = 16 / (sizeof(TI) > sizeof(TO) ? sizeof(TI) : sizeof(TO));
         UnaryMap<TI, TO, VEC, Fn> f{(const TI*)in.data, (TO*)out.data, fn};
         return launch_stream(f, n, s);
     }
@@ -460,14 +483,17 @@ int launch_quantize(const MemRef& in, const MemRef& out, double scale, int64_t z
 int launch_dequantize(const MemRef& in, const MemRef& out, double scale, int64_t zp, hipStream_t s) {
     VPX_REQUIRE(same_shape(in, out), VPX_RESULT_ERROR_INVALID_ARGUMENT, "dequantize: input and output shapes differ");
     const int z = (int)zp;
+    const bool plain = __builtin_isfinite(scale) && __builtin_fabs(scale) >= 0x1p-14 && __builtin_fabs(scale) < 64.0;
     if (in.dtype == VPX_NN_U8 && out.dtype == VPX_NN_FP16)
-        return convert_impl<uint8_t, half_t>(in, out, DequantFn<uint8_t, half_t>{scale, z}, s);
+        return plain ? convert_impl<uint8_t, half_t>(in, out, DequantFn<uint8_t, half_t, true>{scale, z}, s)
+                     : convert_impl<uint8_t, half_t>(in, out, DequantFn<uint8_t, half_t, false>{scale, z}, s);
     if (in.dtype == VPX_NN_I8 && out.dtype == VPX_NN_FP16)
-        return convert_impl<int8_t, half_t>(in, out, DequantFn<int8_t, half_t>{scale, z}, s);
+        return plain ? convert_impl<int8_t, half_t>(in, out, DequantFn<int8_t, half_t, true>{scale, z}, s)
+                     : convert_impl<int8_t, half_t>(in, out, DequantFn<int8_t, half_t, false>{scale, z}, s);
     if (in.dtype == VPX_NN_U8 && out.dtype == VPX_NN_FP32)
-        return convert_impl<uint8_t, float>(in, out, DequantFn<uint8_t, float>{scale, z}, s);
+        return convert_impl<uint8_t, float>(in, out, DequantFn<uint8_t, float, true>{scale, z}, s);
     if (in.dtype == VPX_NN_I8 && out.dtype == VPX_NN_FP32)
-        return convert_impl<int8_t, float>(in, out, DequantFn<int8_t, float>{scale, z}, s);
+        return convert_impl<int8_t, float>(in, out, DequantFn<int8_t, float, true>{scale, z}, s);
     return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "dequantize: %s -> %s is not implemented", dtype_name(in.dtype),
                 dtype_name(out.dtype));
 }

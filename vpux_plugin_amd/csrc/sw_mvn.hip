@@ -62,13 +62,23 @@ __device__ __forceinline__ float wave_sum(float v) {
     return lane_bcast(v, 0) + lane_bcast(v, 32);
 }
 
-// Sum over the 256 lanes of the workgroup, same value in every lane.
-__device__ __forceinline__ float block_sum(float v, float* smem) {
-    v = wave_sum(v);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
-    __syncthreads();
-    return (smem[0] + smem[1]) + (smem[2] + smem[3]);
+template <class Shuffle>
+__device__ __forceinline__ Moments merge_with(Moments m, Shuffle sh) {
+    return merge(m, Moments{sh(m.n), sh(m.mean), sh(m.m2)});
+}
+
+// Combines the moments held by the 64 lanes of a wavefront in a fixed butterfly order.  The
+// pairwise update is not exactly commutative, so lanes may end a few ulps apart: lane 0's value
+// is taken for all.
+__device__ __forceinline__ Moments wave_merge(Moments m) {
+    m = merge_with(m, [](float v) { return dppf<0xB1>(v); });
+    m = merge_with(m, [](float v) { return dppf<0x4E>(v); });
+    m = merge_with(m, [](float v) { return dppf<0x141>(v); });
+    m = merge_with(m, [](float v) { return dppf<0x140>(v); });
+    m = merge_with(m, [](float v) { return swz16(v); });
+    const Moments lo{lane_bcast(m.n, 0), lane_bcast(m.mean, 0), lane_bcast(m.m2, 0)};
+    const Moments hi{lane_bcast(m.n, 32), lane_bcast(m.mean, 32), lane_bcast(m.m2, 32)};
+    return merge(lo, hi);
 }
 
 struct Chunk {
@@ -99,16 +109,17 @@ __device__ __forceinline__ void load_chunk(const half_t* __restrict__ g, int64_t
     }
 }
 
-// chunk statistics; padded slots hold 0 and are excluded through the counts
-__device__ __forceinline__ Moments chunk_moments(const Chunk& c, int64_t base, int64_t size, float* smem) {
+// Chunk statistics.  Each wavefront finds the mean and centred sum of squares of its own 1024
+// elements with lane shuffles only; the four results meet in local memory once and every lane
+// merges them in the same order.  Padded slots hold 0 and are excluded through the counts.
+__device__ __forceinline__ Moments chunk_moments(const Chunk& c, int64_t base, int64_t size, Moments* smem) {
     float s = 0.f;
 #pragma unroll
     for (int j = 0; j < kVecPerThread; j++)
 #pragma unroll
         for (int k = 0; k < 8; k++) s += c.x[j][k];
-    const int64_t left = size - base;
-    const float n = (float)(left < kChunk ? left : kChunk);
-    const float mean = block_sum(s, smem) / n;
+    const float n = wave_sum((float)c.cnt);
+    const float mean = n > 0.f ? wave_sum(s) / n : 0.f;
     float q = 0.f;
 #pragma unroll
     for (int j = 0; j < kVecPerThread; j++)
@@ -118,7 +129,10 @@ __device__ __forceinline__ Moments chunk_moments(const Chunk& c, int64_t base, i
             const float d = c.x[j][k] - mean;
             q += e < size ? d * d : 0.f;
         }
-    return Moments{n, mean, block_sum(q, smem)};
+    q = wave_sum(q);
+    if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = Moments{n, mean, q};
+    __syncthreads();
+    return merge(merge(smem[0], smem[1]), merge(smem[2], smem[3]));
 }
 
 template <bool ALIGNED>
@@ -145,7 +159,21 @@ __device__ __forceinline__ float inv_std(Moments m, bool normalize_variance, flo
     return normalize_variance ? 1.0f / __builtin_sqrtf(m.m2 / m.n + eps) : 1.0f;
 }
 
-// Fixed-order tree merge of `count` (<= 256) partials, one per lane; every lane returns the total.
+// Fixed-order merge of up to 256 published partials of one group.  Every wavefront does the
+// whole merge on its own (four partials per lane in sequence, then the butterfly), so no
+// exchange through local memory is needed and all wavefronts of all workgroups get the same bits.
+__device__ __forceinline__ Moments merge_partials(const Moments* __restrict__ partial, int chunks) {
+    const int lane = threadIdx.x & 63;
+    Moments acc{0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < kMergeInKernel / 64; k++) {
+        const int i = lane * (kMergeInKernel / 64) + k;
+        if (i < chunks) acc = merge(acc, partial[i]);
+    }
+    return wave_merge(acc);
+}
+
+// Fixed-order tree merge of one partial per lane of the workgroup; every lane returns the total.
 __device__ __forceinline__ Moments block_merge(Moments m, Moments* smem) {
     __syncthreads();
     smem[threadIdx.x] = m;
@@ -164,8 +192,7 @@ template <int MODE, bool ALIGNED>
 __global__ __launch_bounds__(kThreads) void mvn_chunk_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
                                                              int64_t group_size, int chunks, Moments* partial,
                                                              const Moments* merged, int normalize_variance, float eps) {
-    __shared__ float red[4];
-    __shared__ Moments tree[MODE == 2 ? kThreads : 1];
+    __shared__ Moments red[4];
     const int64_t group = blockIdx.x / chunks;
     const int chunk = blockIdx.x % chunks;
     const int64_t base = (int64_t)chunk * kChunk;
@@ -179,14 +206,7 @@ __global__ __launch_bounds__(kThreads) void mvn_chunk_kernel(const half_t* __res
         const Moments m = chunk_moments(c, base, group_size, red);
         if (threadIdx.x == 0) partial[blockIdx.x] = m;
     } else {
-        Moments total;
-        if (merged) {
-            total = merged[group];
-        } else {
-            Moments mine{0.f, 0.f, 0.f};
-            if ((int)threadIdx.x < chunks) mine = partial[group * chunks + threadIdx.x];
-            total = block_merge(mine, tree);
-        }
+        const Moments total = merged ? merged[group] : merge_partials(partial + group * chunks, chunks);
         store_chunk<ALIGNED>(out + group * group_size, base, group_size, c, total.mean,
                              inv_std(total, normalize_variance, eps));
     }

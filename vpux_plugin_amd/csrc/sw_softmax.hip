@@ -57,15 +57,21 @@ struct RowMap {
     int64_t out_stride[VPX_MAX_ND_DIMS];
 };
 
+// The outermost dimension needs no division, and the host merges dimensions that are contiguous
+// in both operands, so a compact tensor costs one multiplication per row.
 __device__ __forceinline__ void row_offsets(const RowMap& m, int64_t row, int64_t& in_off, int64_t& out_off) {
     in_off = 0;
     out_off = 0;
-    for (int d = 0; d < m.nd; d++) {
+    for (int d = 0; d + 1 < m.nd; d++) {
         const int64_t q = row / m.dims[d];
         const int64_t r = row - q * m.dims[d];
         row = q;
         in_off += r * m.in_stride[d];
         out_off += r * m.out_stride[d];
+    }
+    if (m.nd > 0) {
+        in_off += row * m.in_stride[m.nd - 1];
+        out_off += row * m.out_stride[m.nd - 1];
     }
 }
 
@@ -87,7 +93,8 @@ __global__ __launch_bounds__(256) void softmax_rows_wave(const T* __restrict__ i
                                                          int64_t rows, int len, int valid) {
     constexpr int N = VecTraits<T>::N;
     const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    // wave-uniform, so the row addressing below runs on the scalar unit
+    const int64_t wave = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t row0 = wave * ROWS;
     if (row0 >= rows) return;
 
@@ -102,7 +109,7 @@ __global__ __launch_bounds__(256) void softmax_rows_wave(const T* __restrict__ i
         for (int j = 0; j < NV; j++) {
             const int e0 = (j * 64 + lane) * N;
             if (e0 < len) {
-                const u32x4 q = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + ioff + e0));
+                const u32x4 q = *reinterpret_cast<const u32x4*>(in + ioff + e0);
                 const T* p = reinterpret_cast<const T*>(&q);
 #pragma unroll
                 for (int k = 0; k < N; k++) x[r][j][k] = e0 + k < valid ? (float)p[k] : -INFINITY;
@@ -229,11 +236,18 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
     int64_t rows = 1;
     for (int d = 0; d < p.nd; d++) {
         if (d == ax) continue;
+        rows *= p.dims[d];
+        if (p.dims[d] == 1) continue;
+        const int k = map.nd - 1;
+        if (k >= 0 && p.in_stride[d] == map.dims[k] * map.in_stride[k] &&
+            p.out_stride[d] == map.dims[k] * map.out_stride[k]) {
+            map.dims[k] *= p.dims[d];  // contiguous with the previous one in both operands: one dimension
+            continue;
+        }
         map.dims[map.nd] = p.dims[d];
         map.in_stride[map.nd] = p.in_stride[d];
         map.out_stride[map.nd] = p.out_stride[d];
         map.nd++;
-        rows *= p.dims[d];
     }
     if (rows == 0 || len == 0) return VPX_RESULT_SUCCESS;
     VPX_REQUIRE(rows < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "softmax: %lld rows exceed the launch limit",
