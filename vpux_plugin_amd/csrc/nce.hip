@@ -597,56 +597,92 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
 // them over all banks.
 //
 // Waves: the tile has MT = ceil(R*OW / 32) row blocks of 32 positions and one or two column blocks
-// of 32 channels; wave w takes column block w % nt and row blocks w / nt, w / nt + 4 / nt, ...
+// of 32 channels; wave w takes column block w % nt and the TMW row blocks w / nt + i * (4 / nt).
+// Row blocks past MT are computed on position 0 and dropped: the main loop has no branches, and
+// the fragments of K step s+1 are read while the MFMAs of step s run.
+//
+// At the sizes this kernel serves a whole launch lasts a few microseconds, so index arithmetic
+// counts: divisions by launch constants use multiply-high reciprocals prepared on the host.
+struct FastDiv {
+    uint32_t d, m;  // m = ceil(2^32 / d); exact for numerators below 2^32 / d
+};
+__device__ __forceinline__ int fdiv(int a, FastDiv f) {
+    return f.d == 1 ? a : (int)__umulhi((unsigned)a, f.m);
+}
+
 struct PatchGeom {
     int R;       // output rows per workgroup
     int PH, PW;  // patch size in input pixels
-    int tiles_y; // workgroups per image
     int MT;      // row blocks of 32 output positions per workgroup
     int nt;      // column blocks of 32 channels in use (1 or 2)
     int w_swz;   // weights rows are swizzled
+    FastDiv tiles_y, cpr, cpp, upr, ow;  // workgroups per image, chunks per weight row / pixel, units per patch row, OW
 };
 
 constexpr int kPatchMaxMT = 14;
 constexpr int kPatchOutStride = 80;  // bytes per output position in the staging tile
 
-template <bool IN_U8>
+// SAME_F: the PPE treats both signs alike (no PReLU stage), which drops the per-value sign test.
+template <bool SAME_F, bool CLIP>
+__device__ __forceinline__ int ppe_fast2(int acc, const ChanPrep& c, const PpeFast& p) {
+    if (!SAME_F) return ppe_fast<CLIP>(acc, c, p);
+    int b = (int)((unsigned)acc + (unsigned)c.bias);
+    if (CLIP) b = b > c.bmax_pos ? c.bmax_pos : (b < -c.bmax_pos ? -c.bmax_pos : b);
+    const double bd = __builtin_bit_cast(double, 0x4330000000000000ull | (unsigned long long)((unsigned)b ^ 0x80000000u)) -
+                      4503601774854144.0;
+    const double y = __builtin_fma(bd, c.f_pos, 6755399441055744.0);
+    const int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, y) + p.zp_out;
+    const int t = q > p.lo ? q : p.lo;
+    return t < p.hi ? t : p.hi;
+}
+
+template <bool IN_U8, int TMW, bool SAME_F>
 __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                       const int32_t* __restrict__ wt, uint8_t* __restrict__ out,
                                                       ConvGeom g, PatchGeom pg, int pad_byte, GemmPpe ppe) {
     constexpr int BN = 64;
-    constexpr int TMW = kPatchMaxMT / 2;  // most row blocks per wave
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int Ktot = g.KY * g.KX * (int)g.IC;
     const int IC = (int)g.IC;
-    uint8_t* const wlds = smem;                                 // [64][Ktot]
-    uint8_t* const patch = smem + BN * Ktot;                    // [PH*PW][IC], later the output staging tile
+    uint8_t* const wlds = smem;               // [64][Ktot]
+    uint8_t* const patch = smem + BN * Ktot;  // [PH*PW][IC], later the output staging tile
     __shared__ int csum[BN];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int img = blockIdx.x / pg.tiles_y;
-    const int oy0 = (blockIdx.x % pg.tiles_y) * pg.R;
+    const int img = fdiv(blockIdx.x, pg.tiles_y);
+    const int oy0 = (blockIdx.x - img * (int)pg.tiles_y.d) * pg.R;
     const int oc0 = blockIdx.y * BN;
 
-    // ---- weights -> LDS.  cid walks (row, chunk) pairs; 256 = dr * cpr + dc advances both without a division.
+    // ---- weights and input patch -> LDS.  All loads of a round are issued before its first LDS
+    // store so that one memory latency covers them.
     {
-        const int cpr = Ktot / 16;
-        const int dr = 256 / cpr, dc = 256 % cpr;
-        int row = tid / cpr, c = tid % cpr;
-        constexpr int UNR = 4;
-        while (row < BN) {
-            i32x4 q[UNR];
-            int dst[UNR];
+        // weights: (row, chunk) pairs; 256 = dr * cpr + dc advances both without a division
+        const int cpr = (int)pg.cpr.d;
+        const int dr = fdiv(256, pg.cpr), dc = 256 - dr * cpr;
+        int row = fdiv(tid, pg.cpr), c = tid - row * cpr;
+        // patch: a unit is 64 consecutive chunks of one patch row; units go round the waves
+        const int cpp = (int)pg.cpp.d;
+        const int row_chunks = pg.PW * cpp;
+        const int upr = (int)pg.upr.d;
+        const int units = pg.PH * upr;
+        const int pad32 = (pad_byte & 0xff) * 0x01010101;
+        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
+        const int iy0 = oy0 * g.SY - g.PT;
+        int unit = wave;
+        constexpr int UW = 9, UP = 6;
+        while (row < BN || unit < units) {
+            i32x4 qw[UW], qp[UP];
+            int dw[UW], dp[UP];
 #pragma unroll
-            for (int u = 0; u < UNR; u++) {
-                dst[u] = -1;
+            for (int u = 0; u < UW; u++) {
+                dw[u] = -1;
                 if (row < BN) {
                     int64_t oc = oc0 + row;
                     oc = oc < g.OC ? oc : g.OC - 1;
-                    q[u] = *reinterpret_cast<const i32x4*>(w + oc * Ktot + c * 16);
-                    const int cs = pg.w_swz ? ((c & ~3) | ((c ^ (row >> 2)) & 3)) : c;
-                    dst[u] = row * Ktot + cs * 16;
+                    qw[u] = *reinterpret_cast<const i32x4*>(w + oc * Ktot + c * 16);
+                    const int cs = pg.w_swz ? c ^ ((row >> 2) & 3) : c;
+                    dw[u] = row * Ktot + cs * 16;
                 }
                 row += dr;
                 c += dc;
@@ -656,46 +692,33 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
                 }
             }
 #pragma unroll
-            for (int u = 0; u < UNR; u++)
-                if (dst[u] >= 0) *reinterpret_cast<i32x4*>(wlds + dst[u]) = q[u];
-        }
-    }
-
-    // ---- input patch -> LDS.  A unit is 64 consecutive chunks of one patch row; units go round the waves.
-    {
-        const int cpp = IC / 16;                  // chunks per pixel
-        const int row_chunks = pg.PW * cpp;
-        const int upr = (row_chunks + 63) / 64;   // units per patch row
-        const int units = pg.PH * upr;
-        const int pad32 = (pad_byte & 0xff) * 0x01010101;
-        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
-        constexpr int UNR = 4;
-        for (int u0 = wave; u0 < units; u0 += 4 * UNR) {
-            i32x4 q[UNR];
-            int dst[UNR];
-#pragma unroll
-            for (int u = 0; u < UNR; u++) {
-                const int unit = u0 + 4 * u;
-                dst[u] = -1;
+            for (int u = 0; u < UP; u++) {
+                dp[u] = -1;
                 if (unit < units) {
-                    const int py = unit / upr;  // wave-uniform
+                    const int py = fdiv(unit, pg.upr);  // wave-uniform
                     const int qi = (unit - py * upr) * 64 + lane;
                     if (qi < row_chunks) {
-                        const int px = (int)((unsigned)qi / (unsigned)cpp), c = qi - px * cpp;
-                        const int iy = oy0 * g.SY - g.PT + py, ix = px - g.PL;
+                        const int px = fdiv(qi, pg.cpp), cc = qi - px * cpp;
+                        const int iy = iy0 + py, ix = px - g.PL;
                         const bool inside = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
                         i32x4 v = i32x4{pad32, pad32, pad32, pad32};
-                        if (inside) v = *reinterpret_cast<const i32x4*>(img_base + ((int64_t)iy * g.W + ix) * IC + c * 16);
-                        if (IN_U8) v ^= (int32_t)0x80808080;
-                        q[u] = v;
+                        if (inside) v = *reinterpret_cast<const i32x4*>(img_base + ((int64_t)iy * g.W + ix) * IC + cc * 16);
+                        qp[u] = v;
                         const int pp = py * pg.PW + px;
-                        dst[u] = pp * IC + (((c & ~3) | ((c ^ (pp >> 2)) & 3)) << 4);
+                        dp[u] = pp * IC + ((cc ^ ((pp >> 2) & 3)) << 4);
                     }
                 }
+                unit += 4;
             }
 #pragma unroll
-            for (int u = 0; u < UNR; u++)
-                if (dst[u] >= 0) *reinterpret_cast<i32x4*>(patch + dst[u]) = q[u];
+            for (int u = 0; u < UW; u++)
+                if (dw[u] >= 0) *reinterpret_cast<i32x4*>(wlds + dw[u]) = qw[u];
+#pragma unroll
+            for (int u = 0; u < UP; u++)
+                if (dp[u] >= 0) {
+                    if (IN_U8) qp[u] ^= (int32_t)0x80808080;
+                    *reinterpret_cast<i32x4*>(patch + dp[u]) = qp[u];
+                }
         }
     }
     __syncthreads();
@@ -704,7 +727,7 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
     if (ppe.corr != 0) {
         const int row = tid >> 2, part = tid & 3;
         int sum = 0;
-        for (int c = part; c < Ktot / 16; c += 4) {
+        for (int c = part; c < (int)pg.cpr.d; c += 4) {
             const i32x4 q = *reinterpret_cast<const i32x4*>(wlds + row * Ktot + c * 16);
 #pragma unroll
             for (int j = 0; j < 4; j++) sum = __builtin_amdgcn_sdot4(q[j], 0x01010101, sum, false);
@@ -715,15 +738,15 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
     }
 
     // ---- main loop
-    const int nj = wave % pg.nt;               // column block of this wave
-    const int mi0 = wave / pg.nt, mstep = 4 / pg.nt;
+    const int nj = pg.nt == 2 ? wave & 1 : 0;  // column block of this wave
+    const int mi0 = pg.nt == 2 ? wave >> 1 : wave, mstep = pg.nt == 2 ? 2 : 4;
     const int npos = pg.R * (int)g.OW;         // output positions of a full tile
     int pp0[TMW];
 #pragma unroll
     for (int i = 0; i < TMW; i++) {
         int p = (mi0 + i * mstep) * 32 + (lane & 31);
         p = p < npos ? p : 0;
-        const int r = (int)((unsigned)p / (unsigned)g.OW), ox = p - r * (int)g.OW;
+        const int r = fdiv(p, pg.ow), ox = p - r * (int)g.OW;
         pp0[i] = r * g.SY * pg.PW + ox * g.SX;
     }
     i32x16 acc[TMW];
@@ -736,32 +759,53 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
     const int brow = nj * 32 + (lane & 31);
     const uint8_t* const bbase = wlds + brow * Ktot;
     const int bsw = pg.w_swz ? (brow >> 2) & 3 : 0;
-    for (int ky = 0; ky < g.KY; ky++) {
-        for (int kx = 0; kx < g.KX; kx++) {
-            const int tap_pp = ky * pg.PW + kx;
-            const int ctap = (ky * g.KX + kx) * (IC / 16);
-            int abase[TMW], asw[TMW];
+
+    // K walk state: tap (ky, kx) and the 32-channel step `ic` inside it
+    int ky = 0, kx = 0, ic = 0, ctap = 0;
+    int abase[TMW], asw[TMW];
+    auto set_tap = [&]() {
+        const int tap_pp = ky * pg.PW + kx;
 #pragma unroll
-            for (int i = 0; i < TMW; i++) {
-                const int pp = pp0[i] + tap_pp;
-                abase[i] = pp * IC;
-                asw[i] = (pp >> 2) & 3;
-            }
-            for (int ic = 0; ic < IC; ic += 32) {
-                const int c = ic / 16 + kgroup;
-                const int cb = ctap + c;
-                const i32x4 fb = *reinterpret_cast<const i32x4*>(bbase + (((cb & ~3) | ((cb ^ bsw) & 3)) << 4));
-                i32x4 fa[TMW];
-#pragma unroll
-                for (int i = 0; i < TMW; i++)
-                    if (mi0 + i * mstep < pg.MT)
-                        fa[i] = *reinterpret_cast<const i32x4*>(patch + abase[i] + (((c & ~3) | ((c ^ asw[i]) & 3)) << 4));
-#pragma unroll
-                for (int i = 0; i < TMW; i++)
-                    if (mi0 + i * mstep < pg.MT)
-                        acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb, acc[i], 0, 0, 0);
-            }
+        for (int i = 0; i < TMW; i++) {
+            const int pp = pp0[i] + tap_pp;
+            abase[i] = pp * IC;
+            asw[i] = (pp >> 2) & 3;
         }
+    };
+    auto read_frags = [&](i32x4(&fa)[TMW], i32x4& fb) {
+        const int c = (ic >> 4) + kgroup;
+        fb = *reinterpret_cast<const i32x4*>(bbase + (((ctap + c) ^ bsw) << 4));
+#pragma unroll
+        for (int i = 0; i < TMW; i++) fa[i] = *reinterpret_cast<const i32x4*>(patch + abase[i] + ((c ^ asw[i]) << 4));
+    };
+    auto advance = [&]() {
+        ic += 32;
+        if (ic == IC) {
+            ic = 0;
+            ctap += IC >> 4;
+            kx++;
+            if (kx == g.KX) {
+                kx = 0;
+                ky++;
+            }
+            set_tap();
+        }
+    };
+    const int steps = g.KY * g.KX * (IC >> 5);  // even: IC is a multiple of 64
+    i32x4 fa0[TMW], fa1[TMW], fb0, fb1;
+    set_tap();
+    read_frags(fa0, fb0);
+    for (int s = 0; s < steps; s += 2) {
+        advance();
+        read_frags(fa1, fb1);
+#pragma unroll
+        for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0[i], fb0, acc[i], 0, 0, 0);
+        if (s + 2 < steps) {
+            advance();
+            read_frags(fa0, fb0);
+        }
+#pragma unroll
+        for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1[i], fb1, acc[i], 0, 0, 0);
     }
     __syncthreads();  // all waves are done with the patch: its LDS becomes the output staging tile
 
@@ -773,22 +817,28 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
         const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
         ChanPrep cp = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
                                   (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
+        const bool clip = cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff;
         asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));
         const PpeFast pf{ppe.zp_out, ppe.lo, ppe.hi};
         const int col4 = nj * 32 + ((lane & 31) & ~3);
+        auto requant = [&](auto clip_c) {
 #pragma unroll
-        for (int i = 0; i < TMW; i++) {
-            if (mi0 + i * mstep >= pg.MT) continue;
+            for (int i = 0; i < TMW; i++) {
+                if (mi0 + i * mstep >= pg.MT) continue;
 #pragma unroll
-            for (int gq = 0; gq < 4; gq++) {
-                unsigned v = 0;
+                for (int gq = 0; gq < 4; gq++) {
+                    unsigned v = 0;
 #pragma unroll
-                for (int r = 0; r < 4; r++) v |= (unsigned)(ppe_fast<true>(acc[i][gq * 4 + r], cp, pf) & 0xff) << (8 * r);
-                v = quad_transpose_bytes(v, lane);
-                const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
-                *reinterpret_cast<unsigned*>(patch + row * kPatchOutStride + col4) = v;
+                    for (int r = 0; r < 4; r++)
+                        v |= (unsigned)(ppe_fast2<SAME_F, decltype(clip_c)::value>(acc[i][gq * 4 + r], cp, pf) & 0xff) << (8 * r);
+                    v = quad_transpose_bytes(v, lane);
+                    const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
+                    *reinterpret_cast<unsigned*>(patch + row * kPatchOutStride + col4) = v;
+                }
             }
-        }
+        };
+        if (__builtin_amdgcn_ballot_w64(clip) != 0) requant(std::true_type{});
+        else requant(std::false_type{});
     }
     __syncthreads();
     const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
@@ -911,7 +961,8 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         }
 
         // Preferred: input patch and weights in LDS, one launch.  R = output rows per workgroup.
-        if (allow_patch && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20)) {
+        if (allow_patch && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20) &&
+            g.IC < (1 << 14) && g.W * g.SX < (1 << 14) && g.N * g.OH * g.OH < (1ll << 32)) {
             PatchGeom pg{};
             const size_t lds_max = 160 * 1024 - 512;
             auto lds_need = [&](int R) {
@@ -930,28 +981,46 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     const int v = std::atoi(e);
                     if (v >= 1 && v <= R) R = v;
                 }
-                pg.tiles_y = (int)((g.OH + R - 1) / R);
-                pg.R = (int)((g.OH + pg.tiles_y - 1) / pg.tiles_y);
+                const int tiles_y = (int)((g.OH + R - 1) / R);
+                auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
+                pg.R = (int)((g.OH + tiles_y - 1) / tiles_y);
                 pg.PH = (pg.R - 1) * g.SY + g.KY;
                 pg.PW = (int)(g.OW - 1) * g.SX + g.KX;
                 pg.MT = (int)((pg.R * g.OW + 31) / 32);
                 pg.nt = g.OC <= 32 ? 1 : 2;
                 pg.w_swz = Ktot % 64 == 0 ? 1 : 0;
+                pg.tiles_y = fd(tiles_y);
+                pg.cpr = fd(Ktot / 16);
+                pg.cpp = fd(g.IC / 16);
+                pg.upr = fd((pg.PW * (g.IC / 16) + 63) / 64);
+                pg.ow = fd(g.OW);
                 const size_t lds = lds_need(pg.R);
-                const dim3 grid((unsigned)(g.N * pg.tiles_y), (unsigned)ocb);
+                const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
                 GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi};
                 const int pad_byte = t.zp_in & 0xff;
-                if (in_u8) {
-                    rc = set_dyn_lds(nce_conv_patch<true>, lds);
-                    if (rc) return rc;
-                    hipLaunchKernelGGL(nce_conv_patch<true>, grid, dim3(256), lds, s, (const int8_t*)t.input,
-                                       (const int8_t*)t.weights, t.weight_table, (uint8_t*)t.output, g, pg, pad_byte, gp);
-                } else {
-                    rc = set_dyn_lds(nce_conv_patch<false>, lds);
-                    if (rc) return rc;
-                    hipLaunchKernelGGL(nce_conv_patch<false>, grid, dim3(256), lds, s, (const int8_t*)t.input,
-                                       (const int8_t*)t.weights, t.weight_table, (uint8_t*)t.output, g, pg, pad_byte, gp);
-                }
+                const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
+                const int per_wave = (pg.MT + 4 / pg.nt - 1) / (4 / pg.nt);  // row blocks the busiest wave owns
+#define VPX_PATCH(U8, TMW, SAME)                                                                                     \
+    do {                                                                                                             \
+        auto kern = nce_conv_patch<U8, TMW, SAME>;                                                                   \
+        rc = set_dyn_lds(kern, lds);                                                                                 \
+        if (rc) return rc;                                                                                           \
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,          \
+                           t.weight_table, (uint8_t*)t.output, g, pg, pad_byte, gp);                                 \
+    } while (0)
+#define VPX_PATCH_T(TMW)                                                                                             \
+    do {                                                                                                             \
+        if (in_u8 && same_f) VPX_PATCH(true, TMW, true);                                                             \
+        else if (in_u8) VPX_PATCH(true, TMW, false);                                                                 \
+        else if (same_f) VPX_PATCH(false, TMW, true);                                                                \
+        else VPX_PATCH(false, TMW, false);                                                                           \
+    } while (0)
+                if (per_wave <= 1) VPX_PATCH_T(1);
+                else if (per_wave <= 2) VPX_PATCH_T(2);
+                else if (per_wave <= 4) VPX_PATCH_T(4);
+                else VPX_PATCH_T(7);
+#undef VPX_PATCH_T
+#undef VPX_PATCH
                 VPX_HIP_CHECK(hipGetLastError());
                 *kernel_name = "nce_conv_patch";
                 return VPX_RESULT_SUCCESS;

@@ -262,8 +262,9 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
         if (vec_ok) {
             const int l = (int)len, v = (int)valid;
             const int64_t per = 64 * N;
-            if (len <= per) launch_rows_wave<T, 1, 4>(in, out, map, rows, l, v, s);
-            else if (len <= 2 * per) launch_rows_wave<T, 2, 2>(in, out, map, rows, l, v, s);
+            // one row per wave measures fastest: more, shorter-lived waves keep more loads in flight
+            if (len <= per) launch_rows_wave<T, 1, 1>(in, out, map, rows, l, v, s);
+            else if (len <= 2 * per) launch_rows_wave<T, 2, 1>(in, out, map, rows, l, v, s);
             else if (len <= 4 * per) launch_rows_wave<T, 4, 1>(in, out, map, rows, l, v, s);
             else launch_rows_wave<T, 8, 1>(in, out, map, rows, l, v, s);
             VPX_HIP_CHECK(hipGetLastError());
