@@ -5,10 +5,14 @@
 // Three device paths:
 //   rows_wave  : reduction axis is the innermost, contiguous one and a row fits the registers of one
 //                wavefront (up to 4096 fp16 / 2048 fp32 values): one 64-lane wave owns a row, 128-bit
-//                loads, max and sum by DPP/swizzle butterflies, single pass over HBM.
+//                loads, max and sum by DPP/swizzle butterflies, single pass over HBM.  fp16 rows
+//                without padding take rows_wave_f16, the same scheme with about half the
+//                instructions (packed-half maximum, mixed-precision fma).
 //   rows_block : innermost axis of any length or alignment: one workgroup per row, three passes.
 //   lines      : reduction over an outer (strided) axis: one lane per line, lanes adjacent along the
 //                innermost dimension so every step of the axis is a coalesced access.
+#include <type_traits>
+
 #include "vpx_common.h"
 
 namespace vpx {
@@ -60,6 +64,11 @@ struct RowMap {
 // The outermost dimension needs no division, and the host merges dimensions that are contiguous
 // in both operands, so a compact tensor costs one multiplication per row.
 __device__ __forceinline__ void row_offsets(const RowMap& m, int64_t row, int64_t& in_off, int64_t& out_off) {
+    if (m.nd == 1) {
+        in_off = row * m.in_stride[0];
+        out_off = row * m.out_stride[0];
+        return;
+    }
     in_off = 0;
     out_off = 0;
     for (int d = 0; d + 1 < m.nd; d++) {
@@ -149,6 +158,94 @@ __global__ __launch_bounds__(256) void softmax_rows_wave(const T* __restrict__ i
                     T* p = reinterpret_cast<T*>(&q);
 #pragma unroll
                     for (int k = 0; k < N; k++) p[k] = (T)(e0 + k < valid ? x[r][j][k] * inv : 0.f);
+                    __builtin_nontemporal_store(q, reinterpret_cast<u32x4*>(out + ooff[r] + e0));
+                }
+            }
+        }
+    }
+}
+
+// fp16 rows without padding: the variant that serves the common case with the fewest
+// instructions, because at one row per wave the kernel is otherwise bound by instruction issue,
+// not by memory.  The maximum is taken on packed halves (exact); x*log2(e) - m*log2(e) is one
+// mixed-precision fma that reads the half directly; the scaled result is rounded to half once.
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
+template <int CTRL>
+__device__ __forceinline__ half2_t dpp_h2(half2_t v) {
+    const int i = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(half2_t, __builtin_amdgcn_update_dpp(i, i, CTRL, 0xf, 0xf, true));
+}
+
+template <int NV, int ROWS>
+__global__ __launch_bounds__(256) void softmax_rows_wave_f16(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                             RowMap map, int64_t rows, int len) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row0 = ((int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) * ROWS;
+    if (row0 >= rows) return;
+
+    half8_t h[ROWS][NV];
+    int64_t ooff[ROWS];
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        const int64_t row = row0 + r < rows ? row0 + r : rows - 1;  // clamp: duplicates are not stored
+        int64_t ioff;
+        row_offsets(map, row, ioff, ooff[r]);
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int e0 = (j * 64 + lane) * 8;
+            if (e0 < len) {
+                h[r][j] = *reinterpret_cast<const half8_t*>(in + ioff + e0);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; k++) h[r][j][k] = (half_t)-INFINITY;
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) {
+        half8_t m8 = h[r][0];
+#pragma unroll
+        for (int j = 1; j < NV; j++) m8 = __builtin_elementwise_max(m8, h[r][j]);
+        const half4_t m4 = __builtin_elementwise_max(__builtin_shufflevector(m8, m8, 0, 1, 2, 3),
+                                                     __builtin_shufflevector(m8, m8, 4, 5, 6, 7));
+        half2_t m2 = __builtin_elementwise_max(__builtin_shufflevector(m4, m4, 0, 1), __builtin_shufflevector(m4, m4, 2, 3));
+        m2 = __builtin_elementwise_max(m2, dpp_h2<0xB1>(m2));
+        m2 = __builtin_elementwise_max(m2, dpp_h2<0x4E>(m2));
+        m2 = __builtin_elementwise_max(m2, dpp_h2<0x141>(m2));
+        m2 = __builtin_elementwise_max(m2, dpp_h2<0x140>(m2));
+        m2 = __builtin_elementwise_max(
+                m2, __builtin_bit_cast(half2_t, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, m2), 0x401F)));
+        const half2_t lo = __builtin_bit_cast(half2_t, __builtin_amdgcn_readlane(__builtin_bit_cast(int, m2), 0));
+        const half2_t hi = __builtin_bit_cast(half2_t, __builtin_amdgcn_readlane(__builtin_bit_cast(int, m2), 32));
+        m2 = __builtin_elementwise_max(lo, hi);
+        const float m = fmaxf((float)m2[0], (float)m2[1]);
+        const float nmb = -m * kLog2e;
+
+        float e[NV][8];
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                e[j][k] = __builtin_amdgcn_exp2f(__builtin_fmaf((float)h[r][j][k], kLog2e, nmb));
+                s += e[j][k];
+            }
+        s = wave_allreduce(s, SumOp{});
+        const float inv = __builtin_amdgcn_rcpf(s);  // 1 ulp, far inside the tolerance of the fp16 result
+        if (row0 + r < rows) {
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const int e0 = (j * 64 + lane) * 8;
+                if (e0 < len) {
+                    u32x4 q;
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        const half2_t v = {(half_t)(e[j][2 * k] * inv), (half_t)(e[j][2 * k + 1] * inv)};
+                        q[k] = __builtin_bit_cast(uint32_t, v);
+                    }
                     __builtin_nontemporal_store(q, reinterpret_cast<u32x4*>(out + ooff[r] + e0));
                 }
             }
@@ -262,8 +359,21 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
         if (vec_ok) {
             const int l = (int)len, v = (int)valid;
             const int64_t per = 64 * N;
-            // one row per wave measures fastest: more, shorter-lived waves keep more loads in flight
-            if (len <= per) launch_rows_wave<T, 1, 1>(in, out, map, rows, l, v, s);
+            if (std::is_same<T, half_t>::value && valid == len) {
+                const half_t* hin = reinterpret_cast<const half_t*>(in);
+                half_t* hout = reinterpret_cast<half_t*>(out);
+                const dim3 block(256);
+                const dim3 grid((unsigned)((rows + 3) / 4));
+                // short rows, many of them: two rows per wave keep more bytes in flight (measured best)
+                if (len <= per && rows >= 16384)
+                    hipLaunchKernelGGL((softmax_rows_wave_f16<1, 2>), dim3((unsigned)((rows + 7) / 8)), block, 0, s, hin, hout, map, rows, l);
+                else if (len <= per) hipLaunchKernelGGL((softmax_rows_wave_f16<1, 1>), grid, block, 0, s, hin, hout, map, rows, l);
+                else if (len <= 2 * per) hipLaunchKernelGGL((softmax_rows_wave_f16<2, 1>), grid, block, 0, s, hin, hout, map, rows, l);
+                else if (len <= 4 * per) hipLaunchKernelGGL((softmax_rows_wave_f16<4, 1>), grid, block, 0, s, hin, hout, map, rows, l);
+                else hipLaunchKernelGGL((softmax_rows_wave_f16<8, 1>), grid, block, 0, s, hin, hout, map, rows, l);
+            }
+            // general form (fp32, padded axis)
+            else if (len <= per) launch_rows_wave<T, 1, 1>(in, out, map, rows, l, v, s);
             else if (len <= 2 * per) launch_rows_wave<T, 2, 1>(in, out, map, rows, l, v, s);
             else if (len <= 4 * per) launch_rows_wave<T, 4, 1>(in, out, map, rows, l, v, s);
             else launch_rows_wave<T, 8, 1>(in, out, map, rows, l, v, s);
