@@ -133,6 +133,54 @@ __device__ __forceinline__ int ppe_fast(int acc, const ChanPrep& c, const PpeFas
     return t < p.hi ? t : p.hi;
 }
 
+// Four results of one output channel as four bytes.  Same arithmetic as ppe_fast with the tail
+// shortened: the even part of the output zero point (plus 128 for signed storage) is folded into
+// the rounding constant -- an odd offset there would flip which way ties round --, the clamp is
+// one float median (all values involved are small integers, exact in fp32; anything larger lies
+// outside the window on the correct side), and the byte is produced by the saturating
+// convert-and-pack instruction.  Signed storage flips the top bits afterwards.
+// GENERAL adds what few layers need: clipping of inputs whose product would leave the +-2^30
+// range, and the odd unit of the zero point.
+struct PpePack {
+    double magic;      // 1.5 * 2^52 + the even part of (zp_out + 128 when the output is signed)
+    float odd;         // the remaining 0 or 1
+    float lo_f, hi_f;  // clamp window in the same shifted domain, inside [0, 255]
+    unsigned flip;     // 0x80808080 for signed storage, else 0
+};
+
+__device__ __forceinline__ PpePack make_ppe_pack(int zp_out, int lo, int hi, bool out_signed) {
+    const int off = out_signed ? 128 : 0;
+    const int z = zp_out + off;
+    return PpePack{6755399441055744.0 + (double)(z & ~1), (float)(z & 1), (float)(lo + off), (float)(hi + off),
+                   out_signed ? 0x80808080u : 0u};
+}
+
+template <bool SAME_F, bool GENERAL>
+__device__ __forceinline__ unsigned ppe_pack4(int a0, int a1, int a2, int a3, const ChanPrep& c, const PpePack& p) {
+    const int a[4] = {a0, a1, a2, a3};
+    unsigned w = 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        int b = (int)((unsigned)a[r] + (unsigned)c.bias);
+        double f = c.f_pos;
+        int bm = c.bmax_pos;
+        if (!SAME_F) {
+            const bool neg = (b ^ c.sgn) < 0;
+            f = neg ? c.f_neg : c.f_pos;
+            if (GENERAL) bm = neg ? c.bmax_neg : c.bmax_pos;
+        }
+        if (GENERAL) b = b > bm ? bm : (b < -bm ? -bm : b);
+        const double bd =
+                __builtin_bit_cast(double, 0x4330000000000000ull | (unsigned long long)((unsigned)b ^ 0x80000000u)) -
+                4503601774854144.0;
+        const double y = __builtin_fma(bd, f, p.magic);
+        float q = (float)(int)(unsigned)__builtin_bit_cast(unsigned long long, y);
+        if (GENERAL) q += p.odd;
+        w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(q, p.lo_f, p.hi_f), r, w);
+    }
+    return w ^ p.flip;
+}
+
 // ---------------------------------------------------------------- per-channel parameter fold
 // One wavefront per output channel: sum of the channel's weights (for the zero-point term) and the
 // prepared epilogue parameters.
@@ -294,6 +342,7 @@ struct GemmPpe {
     int prelu_mult, prelu_shift;  // applied to negative scaled values (1,0 = none; 0,0 = ReLU)
     int corr;                     // zero-point term: acc_true = acc_raw + corr * sum_k B[n][k]
     int zp_out, lo, hi;           // clamp bounds already intersected with the storage range
+    int out_signed;               // output storage is i8
 };
 
 // A[M][K] x B[N][K]^T with the PPE fused; see the file header.  K must be a multiple of 64.
@@ -306,17 +355,20 @@ struct GemmPpe {
 // so that the MFMAs of the second sub-step cover the first fragment reads of panel kt+1.  The column sums of B that the zero-point
 // term needs come from nce_colsum_kernel (only when that term is not zero), and the per-column PPE
 // parameters are unpacked from the weight table in the epilogue.
-template <bool IN_U8, bool OUT_SIGNED>
-__global__ __launch_bounds__(256) void nce_gemm_mfma(const int8_t* __restrict__ A, const int8_t* __restrict__ B,
+template <bool IN_U8, bool OUT_SIGNED, int NW>
+__global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restrict__ A, const int8_t* __restrict__ B,
                                                      const int32_t* __restrict__ wt, const int32_t* __restrict__ colsum,
                                                      uint8_t* __restrict__ out,
                                                      int64_t M, int64_t N, int64_t K, int tiles_m, int tiles_n,
                                                      GemmPpe ppe) {
-    constexpr int BM = 256, BN = 256, BK = 64, WM = 128, WN = 128, TM = 4, TN = 4;
+    // NW = 4: waves 2 x 2, 128 x 128 each, one per SIMD.  NW = 8: waves 2 x 4, 128 x 64 each, two per SIMD,
+    // so that one wave's loads and address arithmetic issue while the other's MFMAs run.
+    constexpr int BM = 256, BN = 256, BK = 64, WM = 128, WN = NW == 4 ? 128 : 64, TM = 4, TN = WN / 32;
+    constexpr int NT = 64 * NW;
     constexpr int NS = 4;                             // LDS panel buffers
     constexpr int CPR = BK / 16;                      // 16-byte chunks per tile row
     constexpr int RPI = 64 / CPR;                     // tile rows one 1 KiB DMA instruction covers
-    constexpr int DMA_PER_WAVE = BM * BK / 1024 / 4;  // per operand, per panel: 4
+    constexpr int DMA_PER_WAVE = BM * BK / 1024 / NW;  // per operand, per panel
     constexpr int STAGE = (BM + BN) * BK;
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -339,7 +391,7 @@ __global__ __launch_bounds__(256) void nce_gemm_mfma(const int8_t* __restrict__ 
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+    const int wm0 = NW == 4 ? (wave >> 1) * WM : (wave >> 2) * WM, wn0 = NW == 4 ? (wave & 1) * WN : (wave & 3) * WN;
 
     // Source addresses of this lane's DMA chunks.  Instruction q of a panel fills LDS bytes
     // [q*1024, q*1024+1024) of the operand's tile = rows q*RPI .. ; the lane sitting at chunk slot p
@@ -347,7 +399,7 @@ __global__ __launch_bounds__(256) void nce_gemm_mfma(const int8_t* __restrict__ 
     unsigned oa[DMA_PER_WAVE], ob[DMA_PER_WAVE];  // byte offsets from the tile's first row
 #pragma unroll
     for (int i = 0; i < DMA_PER_WAVE; i++) {
-        const int q = wave + 4 * i;
+        const int q = wave + NW * i;
         const int r = q * RPI + lane / CPR, p = lane % CPR;
         const int c = p ^ lds_swz<BK>(r);
         int64_t m = m0 + r, n = n0 + r;
@@ -365,8 +417,8 @@ __global__ __launch_bounds__(256) void nce_gemm_mfma(const int8_t* __restrict__ 
     auto dma_one = [&](int p, int d) {
         const unsigned base = lds0 + (unsigned)((p & (NS - 1)) * STAGE);
         const int64_t k0 = (int64_t)(p < nk ? p : nk - 1) * BK;
-        if (d < DMA_PER_WAVE) dma16(abase + k0, oa[d], base + (unsigned)((wave + 4 * d) * 1024));
-        else dma16(bbase + k0, ob[d - DMA_PER_WAVE], base + (unsigned)(BM * BK + (wave + 4 * (d - DMA_PER_WAVE)) * 1024));
+        if (d < DMA_PER_WAVE) dma16(abase + k0, oa[d], base + (unsigned)((wave + NW * d) * 1024));
+        else dma16(bbase + k0, ob[d - DMA_PER_WAVE], base + (unsigned)(BM * BK + (wave + NW * (d - DMA_PER_WAVE)) * 1024));
     };
 
     i32x16 acc[TM][TN];
@@ -403,21 +455,33 @@ __global__ __launch_bounds__(256) void nce_gemm_mfma(const int8_t* __restrict__ 
         }
     };
 
+    // per-column PPE words, fetched now so that the epilogue does not start with a memory round trip
+    int w2r[TN], w3r[TN], csr[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        int64_t n = n0 + wn0 + j * 32 + (lane & 31);
+        n = n < N ? n : N - 1;
+        csr[j] = colsum ? colsum[n] : 0;  // sum_k B[n][k], present when the zero-point term is not 0
+        w2r[j] = wt[n * 4 + 2];
+        w3r[j] = wt[n * 4 + 3];
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // keeps the count of loads in flight below exact
+
 #pragma unroll
     for (int p = 0; p < NS - 1; p++)
 #pragma unroll
         for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
-    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");  // panel 0 is in
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * DMA_PER_WAVE) : "memory");  // panel 0 is in
 #pragma unroll
     for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
     for (int kt = 0; kt < nk; kt++) {
         const uint8_t* pcur = smem + (kt & (NS - 1)) * STAGE;
         const uint8_t* pnxt = smem + ((kt + 1) & (NS - 1)) * STAGE;
         substep(0, pcur, 1, kt + NS - 1, 0);
-        // Loads in flight here, oldest first: panel kt+1 (8), panel kt+2 (8), half of panel kt+3 (4).
+        // Loads in flight here, oldest first: panel kt+1, panel kt+2 (2 * DMA_PER_WAVE each), half of panel kt+3.
         // Behind the barrier panel kt+1 is complete for every wave and nobody reads panel kt-1 any
         // more, whose buffer panel kt+3 is being written to.
-        asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * DMA_PER_WAVE) : "memory");
         substep(1, pnxt, 0, kt + NS - 1, DMA_PER_WAVE);
     }
     dma_wait_all_and_barrier();  // every wave is done with the panels: LDS becomes the output staging tile
@@ -427,17 +491,14 @@ __global__ __launch_bounds__(256) void nce_gemm_mfma(const int8_t* __restrict__ 
     bool clip = false;
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-        int64_t n = n0 + wn0 + j * 32 + (lane & 31);
-        n = n < N ? n : N - 1;
-        const int csum = colsum ? colsum[n] : 0;  // sum_k B[n][k], present when the zero-point term is not 0
-        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        const uint32_t w2 = (uint32_t)w2r[j];
         cp[j] = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
-                            (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * csum)), ppe.prelu_mult, ppe.prelu_shift);
+                            (int)((unsigned)w3r[j] + (unsigned)(ppe.corr * csr[j])), ppe.prelu_mult, ppe.prelu_shift);
         clip = clip || cp[j].bmax_pos != 0x7fffffff || cp[j].bmax_neg != 0x7fffffff;
         // keep the prepared factors in registers: without this the compiler re-derives them per element
         asm volatile("" : "+v"(cp[j].f_pos), "+v"(cp[j].f_neg));
     }
-    const PpeFast pf{ppe.zp_out, ppe.lo, ppe.hi};
+    const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, OUT_SIGNED);
     auto requant_tile = [&](auto clip_c) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
@@ -446,10 +507,8 @@ __global__ __launch_bounds__(256) void nce_gemm_mfma(const int8_t* __restrict__ 
             for (int i = 0; i < TM; i++) {
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    unsigned w = 0;
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        w |= (unsigned)(ppe_fast<decltype(clip_c)::value>(acc[i][j][g * 4 + r], cp[j], pf) & 0xff) << (8 * r);
+                    unsigned w = ppe_pack4<false, decltype(clip_c)::value>(acc[i][j][g * 4], acc[i][j][g * 4 + 1],
+                                                                           acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3], cp[j], pk);
                     w = quad_transpose_bytes(w, lane);
                     const int row = wm0 + i * 32 + 8 * g + 4 * (lane >> 5) + (lane & 3);
                     *reinterpret_cast<unsigned*>(smem + row * kOutStride + col4) = w;
@@ -458,12 +517,12 @@ __global__ __launch_bounds__(256) void nce_gemm_mfma(const int8_t* __restrict__ 
         }
     };
     // scale factors above 1/2 are rare (shift < 15): only then is the clipping variant needed
-    if (__builtin_amdgcn_ballot_w64(clip) != 0) requant_tile(std::true_type{});
+    if (__builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0.f) requant_tile(std::true_type{});
     else requant_tile(std::false_type{});
     __syncthreads();
     const bool vec_ok = (N & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
-    for (int it = 0; it < BM * (BN / 16) / 256; it++) {
-        const int cid = tid + 256 * it;
+    for (int it = 0; it < BM * (BN / 16) / NT; it++) {
+        const int cid = tid + NT * it;
         const int row = cid >> 4, c16 = cid & 15;
         const int64_t m = m0 + row, n = n0 + c16 * 16;
         if (m >= M || n >= N) continue;
@@ -623,19 +682,6 @@ constexpr int kPatchMaxMT = 14;
 constexpr int kPatchOutStride = 80;  // bytes per output position in the staging tile
 
 // SAME_F: the PPE treats both signs alike (no PReLU stage), which drops the per-value sign test.
-template <bool SAME_F, bool CLIP>
-__device__ __forceinline__ int ppe_fast2(int acc, const ChanPrep& c, const PpeFast& p) {
-    if (!SAME_F) return ppe_fast<CLIP>(acc, c, p);
-    int b = (int)((unsigned)acc + (unsigned)c.bias);
-    if (CLIP) b = b > c.bmax_pos ? c.bmax_pos : (b < -c.bmax_pos ? -c.bmax_pos : b);
-    const double bd = __builtin_bit_cast(double, 0x4330000000000000ull | (unsigned long long)((unsigned)b ^ 0x80000000u)) -
-                      4503601774854144.0;
-    const double y = __builtin_fma(bd, c.f_pos, 6755399441055744.0);
-    const int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, y) + p.zp_out;
-    const int t = q > p.lo ? q : p.lo;
-    return t < p.hi ? t : p.hi;
-}
-
 template <bool IN_U8, int TMW, bool SAME_F>
 __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                       const int32_t* __restrict__ wt, uint8_t* __restrict__ out,
@@ -819,7 +865,7 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
                                   (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
         const bool clip = cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff;
         asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));
-        const PpeFast pf{ppe.zp_out, ppe.lo, ppe.hi};
+        const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
         const int col4 = nj * 32 + ((lane & 31) & ~3);
         auto requant = [&](auto clip_c) {
 #pragma unroll
@@ -827,17 +873,15 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
                 if (mi0 + i * mstep >= pg.MT) continue;
 #pragma unroll
                 for (int gq = 0; gq < 4; gq++) {
-                    unsigned v = 0;
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        v |= (unsigned)(ppe_fast2<SAME_F, decltype(clip_c)::value>(acc[i][gq * 4 + r], cp, pf) & 0xff) << (8 * r);
+                    unsigned v = ppe_pack4<SAME_F, decltype(clip_c)::value>(acc[i][gq * 4], acc[i][gq * 4 + 1], acc[i][gq * 4 + 2],
+                                                                            acc[i][gq * 4 + 3], cp, pk);
                     v = quad_transpose_bytes(v, lane);
                     const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
                     *reinterpret_cast<unsigned*>(patch + row * kPatchOutStride + col4) = v;
                 }
             }
         };
-        if (__builtin_amdgcn_ballot_w64(clip) != 0) requant(std::true_type{});
+        if (__builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0.f) requant(std::true_type{});
         else requant(std::false_type{});
     }
     __syncthreads();
@@ -924,14 +968,19 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         pf.hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
         if (pf.lo > tmax) pf.lo = tmax;  // clamp window entirely above / below the storage range
         if (pf.hi < tmin) pf.hi = tmin;
+        if (pf.lo > pf.hi) pf.lo = pf.hi;  // inverted window: max-then-min always ends at the upper bound
 
         if (use_gemm) {
             constexpr int BM = 256, BN = 256;
             const int tiles_m = (int)((Mtot + BM - 1) / BM), tiles_n = (int)((g.OC + BN - 1) / BN);
             const int per_xcd = (tiles_m * tiles_n + 7) / 8;
-            const dim3 grid((unsigned)(per_xcd * 8)), block(256);
+            // Eight waves (two per SIMD) overlap the PPE epilogue better and win up to K = 4096; beyond
+            // that the lower LDS traffic of four 128x128 waves wins.  VPX_GEMM_WAVES=4|8 overrides.
+            const char* wenv = std::getenv("VPX_GEMM_WAVES");
+            const int nw = wenv && *wenv ? (std::atoi(wenv) == 4 ? 4 : 8) : (g.IC > 4096 ? 4 : 8);
+            const dim3 grid((unsigned)(per_xcd * 8)), block(64 * nw);
             const size_t lds = 4 * (BM + BN) * 64;  // four K panels; the output staging tile reuses them
-            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi};
+            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
             int32_t* colsum = nullptr;
             if (corr != 0) {
                 void* ws = nullptr;
@@ -942,19 +991,25 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                                    (const int8_t*)t.weights, colsum, g.OC, Ktot);
                 VPX_HIP_CHECK(hipGetLastError());
             }
-#define VPX_GEMM(U8, SGN)                                                                                            \
+#define VPX_GEMM_W(U8, SGN, NW)                                                                                      \
     do {                                                                                                             \
-        auto kern = nce_gemm_mfma<U8, SGN>;                                                                        \
+        auto kern = nce_gemm_mfma<U8, SGN, NW>;                                                                      \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
         hipLaunchKernelGGL(kern, grid, block, lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,              \
-                           t.weight_table, colsum, (uint8_t*)t.output, Mtot, g.OC, g.IC, tiles_m, tiles_n, gp);             \
+                           t.weight_table, colsum, (uint8_t*)t.output, Mtot, g.OC, g.IC, tiles_m, tiles_n, gp);      \
+    } while (0)
+#define VPX_GEMM(U8, SGN)                                                                                            \
+    do {                                                                                                             \
+        if (nw == 4) VPX_GEMM_W(U8, SGN, 4);                                                                         \
+        else VPX_GEMM_W(U8, SGN, 8);                                                                                 \
     } while (0)
             if (in_u8 && out_signed) VPX_GEMM(true, true);
             else if (in_u8) VPX_GEMM(true, false);
             else if (out_signed) VPX_GEMM(false, true);
             else VPX_GEMM(false, false);
 #undef VPX_GEMM
+#undef VPX_GEMM_W
             VPX_HIP_CHECK(hipGetLastError());
             *kernel_name = "nce_gemm_mfma";
             return VPX_RESULT_SUCCESS;
@@ -996,7 +1051,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 pg.ow = fd(g.OW);
                 const size_t lds = lds_need(pg.R);
                 const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
-                GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi};
+                GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
                 const int pad_byte = t.zp_in & 0xff;
                 const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
                 const int per_wave = (pg.MT + 4 / pg.nt - 1) / (4 / pg.nt);  // row blocks the busiest wave owns
