@@ -104,8 +104,16 @@ def test_naive_path_covers_odd_shapes_and_weight_zero_points(rt, orc, dev):
     assert name == "nce_conv_naive" and np.array_equal(got, want)
 
 
+@pytest.fixture(params=["8", "4"])
+def gemm_waves(request):
+    """Both shapes of the matmul kernel: two waves per SIMD (64 x 128 each) and one (128 x 128)."""
+    os.environ["VPX_GEMM_WAVES"] = request.param
+    yield request.param
+    del os.environ["VPX_GEMM_WAVES"]
+
+
 @pytest.mark.parametrize("M,K,N", [(256, 64, 256), (300, 128, 520), (1, 64, 1), (513, 256, 77), (1024, 512, 768)])
-def test_matmul_gemm_path(rt, orc, dev, M, K, N):
+def test_matmul_gemm_path(rt, orc, dev, gemm_waves, M, K, N):
     rng = np.random.default_rng(70 + M)
     for in_u8, zp in ((False, 3), (True, 128), (False, 0), (True, 11)):
         a = rng.integers(0, 256, (M, K), dtype=np.uint8) if in_u8 else rng.integers(-128, 128, (M, K)).astype(np.int8)

@@ -97,9 +97,11 @@ struct PpeFast {
     int zp_out, lo, hi;  // clamp bounds already intersected with the storage range
 };
 
+// Any bound between the largest |b| whose result can still lie inside a clamp window and 2^30 / |f|
+// serves; single precision is plenty.
 __device__ __forceinline__ int ppe_bmax(double f) {
-    const double a = __builtin_fabs(f);
-    return a <= 0.5 ? 0x7fffffff : (int)(1073741824.0 / a);
+    const float a = __builtin_fabsf((float)f);
+    return a <= 0.5f ? 0x7fffffff : (int)(1.0e9f * __builtin_amdgcn_rcpf(a));
 }
 
 __device__ __forceinline__ ChanPrep ppe_prepare(int mult, int shift, int bias, int prelu_mult, int prelu_shift) {
@@ -142,43 +144,59 @@ __device__ __forceinline__ int ppe_fast(int acc, const ChanPrep& c, const PpeFas
 // GENERAL adds what few layers need: clipping of inputs whose product would leave the +-2^30
 // range, and the odd unit of the zero point.
 struct PpePack {
-    double magic;      // 1.5 * 2^52 + the even part of (zp_out + 128 when the output is signed)
-    float odd;         // the remaining 0 or 1
-    float lo_f, hi_f;  // clamp window in the same shifted domain, inside [0, 255]
-    unsigned flip;     // 0x80808080 for signed storage, else 0
+    double magic;  // 1.5 * 2^52 + the even part of (zp_out + 128 when the output is signed)
+    int odd;       // the remaining 0 or 1
+    int lo, hi;    // clamp window in the same shifted domain, inside [0, 255]
+    unsigned flip; // 0x80808080 for signed storage, else 0
 };
 
 __device__ __forceinline__ PpePack make_ppe_pack(int zp_out, int lo, int hi, bool out_signed) {
     const int off = out_signed ? 128 : 0;
     const int z = zp_out + off;
-    return PpePack{6755399441055744.0 + (double)(z & ~1), (float)(z & 1), (float)(lo + off), (float)(hi + off),
-                   out_signed ? 0x80808080u : 0u};
+    return PpePack{6755399441055744.0 + (double)(z & ~1), z & 1, lo + off, hi + off, out_signed ? 0x80808080u : 0u};
 }
 
+__device__ __forceinline__ int med3_i32(int v, int lo, int hi) {
+    int r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
+    return r;
+}
+
+// `c.bias` must already carry the +2^31 that turns the int -> double bit trick's sign flip into part
+// of the bias addition (see ppe_prepare_packed).
 template <bool SAME_F, bool GENERAL>
 __device__ __forceinline__ unsigned ppe_pack4(int a0, int a1, int a2, int a3, const ChanPrep& c, const PpePack& p) {
     const int a[4] = {a0, a1, a2, a3};
     unsigned w = 0;
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        int b = (int)((unsigned)a[r] + (unsigned)c.bias);
+        unsigned bu = (unsigned)a[r] + (unsigned)c.bias;  // (acc + bias) ^ 0x80000000
         double f = c.f_pos;
         int bm = c.bmax_pos;
         if (!SAME_F) {
-            const bool neg = (b ^ c.sgn) < 0;
+            const bool neg = (int)(bu ^ (unsigned)c.sgn) >= 0;  // flipped domain: top bit clear means negative
             f = neg ? c.f_neg : c.f_pos;
             if (GENERAL) bm = neg ? c.bmax_neg : c.bmax_pos;
         }
-        if (GENERAL) b = b > bm ? bm : (b < -bm ? -bm : b);
-        const double bd =
-                __builtin_bit_cast(double, 0x4330000000000000ull | (unsigned long long)((unsigned)b ^ 0x80000000u)) -
-                4503601774854144.0;
+        if (GENERAL) {
+            int b = (int)(bu ^ 0x80000000u);
+            b = b > bm ? bm : (b < -bm ? -bm : b);
+            bu = (unsigned)b ^ 0x80000000u;
+        }
+        const double bd = __builtin_bit_cast(double, 0x4330000000000000ull | (unsigned long long)bu) - 4503601774854144.0;
         const double y = __builtin_fma(bd, f, p.magic);
-        float q = (float)(int)(unsigned)__builtin_bit_cast(unsigned long long, y);
+        int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, y);
         if (GENERAL) q += p.odd;
-        w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_amdgcn_fmed3f(q, p.lo_f, p.hi_f), r, w);
+        w |= (unsigned)med3_i32(q, p.lo, p.hi) << (8 * r);
     }
     return w ^ p.flip;
+}
+
+// ChanPrep for ppe_pack4: the bias carries the sign flip.
+__device__ __forceinline__ ChanPrep ppe_prepare_packed(int mult, int shift, int bias, int prelu_mult, int prelu_shift) {
+    ChanPrep c = ppe_prepare(mult, shift, bias, prelu_mult, prelu_shift);
+    c.bias = (int)((unsigned)c.bias + 0x80000000u);
+    return c;
 }
 
 // ---------------------------------------------------------------- per-channel parameter fold
@@ -492,8 +510,8 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const uint32_t w2 = (uint32_t)w2r[j];
-        cp[j] = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
-                            (int)((unsigned)w3r[j] + (unsigned)(ppe.corr * csr[j])), ppe.prelu_mult, ppe.prelu_shift);
+        cp[j] = ppe_prepare_packed((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+                                   (int)((unsigned)w3r[j] + (unsigned)(ppe.corr * csr[j])), ppe.prelu_mult, ppe.prelu_shift);
         clip = clip || cp[j].bmax_pos != 0x7fffffff || cp[j].bmax_neg != 0x7fffffff;
         // keep the prepared factors in registers: without this the compiler re-derives them per element
         asm volatile("" : "+v"(cp[j].f_pos), "+v"(cp[j].f_neg));
@@ -517,7 +535,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
         }
     };
     // scale factors above 1/2 are rare (shift < 15): only then is the clipping variant needed
-    if (__builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0.f) requant_tile(std::true_type{});
+    if (__builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0) requant_tile(std::true_type{});
     else requant_tile(std::false_type{});
     __syncthreads();
     const bool vec_ok = (N & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
@@ -642,16 +660,25 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
 }
 
 // ---------------------------------------------------------------- convolution with the input patch in LDS
-// Workgroup: `R` whole output rows of one image x 64 output channels.  The (R-1)*SY+KY input rows
-// the tile needs are copied to LDS once, padding materialised with the zero-point byte and u8
-// re-biased to s8 on the way, so every tap of every output position is an LDS read; the weights of
-// the 64 channels sit beside them.  One launch does everything: the per-channel weight sums of the
+// A tile is `R` whole output rows of one image x 64 output channels.  The (R-1)*SY+KY input rows a
+// tile needs are copied to LDS once, padding materialised with the zero-point byte and u8 re-biased
+// to s8 on the way, so every tap of every output position is an LDS read; the weights of the 64
+// channels sit beside them.  One launch does everything: the per-channel weight sums of the
 // zero-point term come from the LDS copy of the weights and the PPE parameters are unpacked from
-// the weight table in the epilogue.
+// the weight table.
+//
+// Workgroups are persistent: each loads the weights and prepares the PPE parameters once, then
+// walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...  The global loads of tile t+1's patch are
+// issued before the MFMA loop of tile t and land in registers while it runs; they are written to
+// LDS after it, next to the PPE of tile t, whose bytes go through a separate staging area:
+//
+//     issue loads(t+1) | MFMA loop(t) | barrier | patch(t+1) -> LDS, PPE(t) -> staging | barrier |
+//     staging -> global (asynchronous) | next tile
 //
 // LDS layouts (16-byte chunks):
 //   weights [64][Ktot]      chunk c of row r at c ^ ((r >> 2) & 3) when Ktot is a multiple of 64
 //   patch   [PH*PW][IC]     chunk c of pixel p at c ^ ((p >> 2) & 3)   (IC is a multiple of 64)
+//   staging [MT*32][80]     output bytes of the tile, 64 per position
 // Lanes 0-31 of a fragment read walk consecutive rows / pixels at one chunk index; the xor spreads
 // them over all banks.
 //
@@ -670,66 +697,99 @@ __device__ __forceinline__ int fdiv(int a, FastDiv f) {
 }
 
 struct PatchGeom {
-    int R;       // output rows per workgroup
-    int PH, PW;  // patch size in input pixels
-    int MT;      // row blocks of 32 output positions per workgroup
-    int nt;      // column blocks of 32 channels in use (1 or 2)
-    int w_swz;   // weights rows are swizzled
-    FastDiv tiles_y, cpr, cpp, upr, ow;  // workgroups per image, chunks per weight row / pixel, units per patch row, OW
+    int R;        // output rows per tile
+    int PH, PW;   // patch size in input pixels
+    int MT;       // row blocks of 32 output positions per tile
+    int nt;       // column blocks of 32 channels in use (1 or 2)
+    int w_swz;    // weights rows are swizzled
+    int ntiles;   // tiles per 64-channel block: N * tiles_y
+    int patch_bytes;
+    FastDiv tiles_y, cpr, cpp, upr, ow;  // tiles per image, chunks per weight row / pixel, units per patch row, OW
 };
 
 constexpr int kPatchMaxMT = 14;
 constexpr int kPatchOutStride = 80;  // bytes per output position in the staging tile
+constexpr int kPatchPrefetch = 6;    // 16-byte patch chunks per lane fetched ahead of the MFMA loop
 
 // SAME_F: the PPE treats both signs alike (no PReLU stage), which drops the per-value sign test.
 template <bool IN_U8, int TMW, bool SAME_F>
-__global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
+__global__ __launch_bounds__(256, TMW <= 4 ? 2 : 1) void nce_conv_patch(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                       const int32_t* __restrict__ wt, uint8_t* __restrict__ out,
                                                       ConvGeom g, PatchGeom pg, int pad_byte, GemmPpe ppe) {
     constexpr int BN = 64;
+    constexpr int UP = kPatchPrefetch;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int Ktot = g.KY * g.KX * (int)g.IC;
     const int IC = (int)g.IC;
-    uint8_t* const wlds = smem;               // [64][Ktot]
-    uint8_t* const patch = smem + BN * Ktot;  // [PH*PW][IC], later the output staging tile
+    uint8_t* const wlds = smem;                      // [64][Ktot]
+    uint8_t* const patch = smem + BN * Ktot;         // [PH*PW][IC]
+    uint8_t* const stage = patch + pg.patch_bytes;   // [MT*32][kPatchOutStride]
     __shared__ int csum[BN];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int img = fdiv(blockIdx.x, pg.tiles_y);
-    const int oy0 = (blockIdx.x - img * (int)pg.tiles_y.d) * pg.R;
     const int oc0 = blockIdx.y * BN;
 
-    // ---- weights and input patch -> LDS.  All loads of a round are issued before its first LDS
-    // store so that one memory latency covers them.
+    // patch transfer: a unit is 64 consecutive chunks of one patch row; units go round the waves
+    const int cpp = (int)pg.cpp.d;
+    const int row_chunks = pg.PW * cpp;
+    const int upr = (int)pg.upr.d;
+    const int units = pg.PH * upr;
+    const int pad32 = (pad_byte & 0xff) * 0x01010101;
+    // loads units unit0 + wave + 4u (u < UP) of tile `tile` into registers; dst < 0 marks an unused slot
+    auto patch_issue = [&](int tile, int unit0, i32x4(&q)[UP], int(&dst)[UP]) {
+        const int img = fdiv(tile, pg.tiles_y);
+        const int iy0 = (tile - img * (int)pg.tiles_y.d) * pg.R * g.SY - g.PT;
+        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
+        // branch-free: a slot without work loads from a valid dummy address and is marked by dst < 0
+#pragma unroll
+        for (int u = 0; u < UP; u++) {
+            const int unit = unit0 + wave + 4 * u;
+            const int py = fdiv(unit, pg.upr);  // wave-uniform
+            const int qi = (unit - py * upr) * 64 + lane;
+            const bool ok = unit < units && qi < row_chunks;
+            const int px = fdiv(qi, pg.cpp), cc = qi - px * cpp;
+            const int iy = iy0 + py, ix = px - g.PL;
+            const bool inside = ok && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+            const int64_t off = inside ? ((int64_t)iy * g.W + ix) * IC + cc * 16 : 0;
+            const i32x4 v = *reinterpret_cast<const i32x4*>(img_base + off);
+            q[u] = inside ? v : i32x4{pad32, pad32, pad32, pad32};
+            const int pp = py * pg.PW + px;
+            dst[u] = ok ? pp * IC + ((cc ^ ((pp >> 2) & 3)) << 4) : -1;
+        }
+    };
+    auto patch_commit = [&](i32x4(&q)[UP], int(&dst)[UP]) {
+#pragma unroll
+        for (int u = 0; u < UP; u++)
+            if (dst[u] >= 0) {
+                if (IN_U8) q[u] ^= (int32_t)0x80808080;
+                *reinterpret_cast<i32x4*>(patch + dst[u]) = q[u];
+            }
+    };
+
+    int tile = blockIdx.x;
+    i32x4 pq[UP];
+    int pdst[UP];
+    patch_issue(tile, 0, pq, pdst);  // in flight together with the weights
+
+    // ---- weights -> LDS, once.  (row, chunk) pairs; 256 = dr * cpr + dc advances both without a division.
     {
-        // weights: (row, chunk) pairs; 256 = dr * cpr + dc advances both without a division
         const int cpr = (int)pg.cpr.d;
         const int dr = fdiv(256, pg.cpr), dc = 256 - dr * cpr;
         int row = fdiv(tid, pg.cpr), c = tid - row * cpr;
-        // patch: a unit is 64 consecutive chunks of one patch row; units go round the waves
-        const int cpp = (int)pg.cpp.d;
-        const int row_chunks = pg.PW * cpp;
-        const int upr = (int)pg.upr.d;
-        const int units = pg.PH * upr;
-        const int pad32 = (pad_byte & 0xff) * 0x01010101;
-        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
-        const int iy0 = oy0 * g.SY - g.PT;
-        int unit = wave;
-        constexpr int UW = 9, UP = 6;
-        while (row < BN || unit < units) {
-            i32x4 qw[UW], qp[UP];
-            int dw[UW], dp[UP];
+        constexpr int UW = 9;
+        while (row < BN) {
+            i32x4 qw[UW];
+            int dw[UW];
 #pragma unroll
             for (int u = 0; u < UW; u++) {
-                dw[u] = -1;
-                if (row < BN) {
-                    int64_t oc = oc0 + row;
-                    oc = oc < g.OC ? oc : g.OC - 1;
-                    qw[u] = *reinterpret_cast<const i32x4*>(w + oc * Ktot + c * 16);
-                    const int cs = pg.w_swz ? c ^ ((row >> 2) & 3) : c;
-                    dw[u] = row * Ktot + cs * 16;
-                }
+                const bool ok = row < BN;
+                const int rr = ok ? row : BN - 1;
+                int64_t oc = oc0 + rr;
+                oc = oc < g.OC ? oc : g.OC - 1;
+                qw[u] = *reinterpret_cast<const i32x4*>(w + oc * Ktot + c * 16);
+                const int cs = pg.w_swz ? c ^ ((rr >> 2) & 3) : c;
+                dw[u] = ok ? rr * Ktot + cs * 16 : -1;
                 row += dr;
                 c += dc;
                 if (c >= cpr) {
@@ -738,34 +798,14 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
                 }
             }
 #pragma unroll
-            for (int u = 0; u < UP; u++) {
-                dp[u] = -1;
-                if (unit < units) {
-                    const int py = fdiv(unit, pg.upr);  // wave-uniform
-                    const int qi = (unit - py * upr) * 64 + lane;
-                    if (qi < row_chunks) {
-                        const int px = fdiv(qi, pg.cpp), cc = qi - px * cpp;
-                        const int iy = iy0 + py, ix = px - g.PL;
-                        const bool inside = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-                        i32x4 v = i32x4{pad32, pad32, pad32, pad32};
-                        if (inside) v = *reinterpret_cast<const i32x4*>(img_base + ((int64_t)iy * g.W + ix) * IC + cc * 16);
-                        qp[u] = v;
-                        const int pp = py * pg.PW + px;
-                        dp[u] = pp * IC + ((cc ^ ((pp >> 2) & 3)) << 4);
-                    }
-                }
-                unit += 4;
-            }
-#pragma unroll
             for (int u = 0; u < UW; u++)
                 if (dw[u] >= 0) *reinterpret_cast<i32x4*>(wlds + dw[u]) = qw[u];
-#pragma unroll
-            for (int u = 0; u < UP; u++)
-                if (dp[u] >= 0) {
-                    if (IN_U8) qp[u] ^= (int32_t)0x80808080;
-                    *reinterpret_cast<i32x4*>(patch + dp[u]) = qp[u];
-                }
         }
+    }
+    patch_commit(pq, pdst);
+    for (int unit0 = 4 * UP; unit0 < units; unit0 += 4 * UP) {  // patches larger than the prefetch window
+        patch_issue(tile, unit0, pq, pdst);
+        patch_commit(pq, pdst);
     }
     __syncthreads();
 
@@ -781,9 +821,10 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
         sum += (int)dpp_u32<0xB1>((unsigned)sum);
         sum += (int)dpp_u32<0x4E>((unsigned)sum);
         if (part == 0) csum[row] = sum;
+        __syncthreads();
     }
 
-    // ---- main loop
+    // ---- per-wave constants: tile geometry, B addressing, PPE parameters of this lane's channel
     const int nj = pg.nt == 2 ? wave & 1 : 0;  // column block of this wave
     const int mi0 = pg.nt == 2 ? wave >> 1 : wave, mstep = pg.nt == 2 ? 2 : 4;
     const int npos = pg.R * (int)g.OW;         // output positions of a full tile
@@ -795,110 +836,131 @@ __global__ __launch_bounds__(256) void nce_conv_patch(const int8_t* __restrict__
         const int r = fdiv(p, pg.ow), ox = p - r * (int)g.OW;
         pp0[i] = r * g.SY * pg.PW + ox * g.SX;
     }
-    i32x16 acc[TMW];
-#pragma unroll
-    for (int i = 0; i < TMW; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[i][r] = 0;
-
     const int kgroup = lane >> 5;
     const int brow = nj * 32 + (lane & 31);
     const uint8_t* const bbase = wlds + brow * Ktot;
     const int bsw = pg.w_swz ? (brow >> 2) & 3 : 0;
 
-    // K walk state: tap (ky, kx) and the 32-channel step `ic` inside it
-    int ky = 0, kx = 0, ic = 0, ctap = 0;
-    int abase[TMW], asw[TMW];
-    auto set_tap = [&]() {
-        const int tap_pp = ky * pg.PW + kx;
-#pragma unroll
-        for (int i = 0; i < TMW; i++) {
-            const int pp = pp0[i] + tap_pp;
-            abase[i] = pp * IC;
-            asw[i] = (pp >> 2) & 3;
-        }
-    };
-    auto read_frags = [&](i32x4(&fa)[TMW], i32x4& fb) {
-        const int c = (ic >> 4) + kgroup;
-        fb = *reinterpret_cast<const i32x4*>(bbase + (((ctap + c) ^ bsw) << 4));
-#pragma unroll
-        for (int i = 0; i < TMW; i++) fa[i] = *reinterpret_cast<const i32x4*>(patch + abase[i] + ((c ^ asw[i]) << 4));
-    };
-    auto advance = [&]() {
-        ic += 32;
-        if (ic == IC) {
-            ic = 0;
-            ctap += IC >> 4;
-            kx++;
-            if (kx == g.KX) {
-                kx = 0;
-                ky++;
-            }
-            set_tap();
-        }
-    };
-    const int steps = g.KY * g.KX * (IC >> 5);  // even: IC is a multiple of 64
-    i32x4 fa0[TMW], fa1[TMW], fb0, fb1;
-    set_tap();
-    read_frags(fa0, fb0);
-    for (int s = 0; s < steps; s += 2) {
-        advance();
-        read_frags(fa1, fb1);
-#pragma unroll
-        for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0[i], fb0, acc[i], 0, 0, 0);
-        if (s + 2 < steps) {
-            advance();
-            read_frags(fa0, fb0);
-        }
-#pragma unroll
-        for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1[i], fb1, acc[i], 0, 0, 0);
-    }
-    __syncthreads();  // all waves are done with the patch: its LDS becomes the output staging tile
-
-    // ---- epilogue
+    ChanPrep cp;
     {
         int64_t n = oc0 + brow;
         n = n < g.OC ? n : g.OC - 1;
         const int cs = ppe.corr != 0 ? csum[brow] : 0;
         const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
-        ChanPrep cp = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
-                                  (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
-        const bool clip = cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff;
-        asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));
-        const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
-        const int col4 = nj * 32 + ((lane & 31) & ~3);
-        auto requant = [&](auto clip_c) {
+        cp = ppe_prepare_packed((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+                                (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
+    }
+    asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));  // keep the factors in registers instead of re-deriving them per value
+    const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
+    const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 ||
+                         pk.odd != 0;
+    const int col4 = nj * 32 + ((lane & 31) & ~3);
+    const bool vec_ok = (g.OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    const int steps = g.KY * g.KX * (IC >> 5);  // even: IC is a multiple of 64
+
+    for (; tile < pg.ntiles; tile += gridDim.x) {
+        const int next = tile + gridDim.x;
+        const bool has_next = next < pg.ntiles;
+        if (has_next) patch_issue(next, 0, pq, pdst);
+
+        // ---- MFMA loop over taps and channels
+        i32x16 acc[TMW];
+#pragma unroll
+        for (int i = 0; i < TMW; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][r] = 0;
+        int ky = 0, kx = 0, ic = 0, ctap = 0;
+        int abase[TMW], asw[TMW];
+        auto set_tap = [&]() {
+            const int tap_pp = ky * pg.PW + kx;
+#pragma unroll
+            for (int i = 0; i < TMW; i++) {
+                const int pp = pp0[i] + tap_pp;
+                abase[i] = pp * IC;
+                asw[i] = (pp >> 2) & 3;
+            }
+        };
+        auto read_frags = [&](i32x4(&fa)[TMW], i32x4& fb) {
+            const int c = (ic >> 4) + kgroup;
+            fb = *reinterpret_cast<const i32x4*>(bbase + (((ctap + c) ^ bsw) << 4));
+#pragma unroll
+            for (int i = 0; i < TMW; i++) fa[i] = *reinterpret_cast<const i32x4*>(patch + abase[i] + ((c ^ asw[i]) << 4));
+        };
+        auto advance = [&]() {
+            ic += 32;
+            if (ic == IC) {
+                ic = 0;
+                ctap += IC >> 4;
+                kx++;
+                if (kx == g.KX) {
+                    kx = 0;
+                    ky++;
+                }
+                set_tap();
+            }
+        };
+        i32x4 fa0[TMW], fa1[TMW], fb0, fb1;
+        set_tap();
+        read_frags(fa0, fb0);
+        for (int s = 0; s < steps; s += 2) {
+            advance();
+            read_frags(fa1, fb1);
+#pragma unroll
+            for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0[i], fb0, acc[i], 0, 0, 0);
+            if (s + 2 < steps) {
+                advance();
+                read_frags(fa0, fb0);
+            }
+#pragma unroll
+            for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1[i], fb1, acc[i], 0, 0, 0);
+        }
+        __syncthreads();  // every wave is done reading this tile's patch (and the previous tile's staging bytes)
+
+        // ---- next tile's patch -> LDS
+        if (has_next) {
+            patch_commit(pq, pdst);
+            for (int unit0 = 4 * UP; unit0 < units; unit0 += 4 * UP) {
+                patch_issue(next, unit0, pq, pdst);
+                patch_commit(pq, pdst);
+            }
+        }
+
+        // ---- PPE of this tile -> staging
+        auto requant = [&](auto general_c) {
 #pragma unroll
             for (int i = 0; i < TMW; i++) {
                 if (mi0 + i * mstep >= pg.MT) continue;
 #pragma unroll
                 for (int gq = 0; gq < 4; gq++) {
-                    unsigned v = ppe_pack4<SAME_F, decltype(clip_c)::value>(acc[i][gq * 4], acc[i][gq * 4 + 1], acc[i][gq * 4 + 2],
-                                                                            acc[i][gq * 4 + 3], cp, pk);
+                    unsigned v = ppe_pack4<SAME_F, decltype(general_c)::value>(acc[i][gq * 4], acc[i][gq * 4 + 1],
+                                                                               acc[i][gq * 4 + 2], acc[i][gq * 4 + 3], cp, pk);
                     v = quad_transpose_bytes(v, lane);
                     const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
-                    *reinterpret_cast<unsigned*>(patch + row * kPatchOutStride + col4) = v;
+                    *reinterpret_cast<unsigned*>(stage + row * kPatchOutStride + col4) = v;
                 }
             }
         };
-        if (__builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0.f) requant(std::true_type{});
+        if (general) requant(std::true_type{});
         else requant(std::false_type{});
-    }
-    __syncthreads();
-    const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
-    const int valid = rows_here * (int)g.OW;
-    const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
-    const bool vec_ok = (g.OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
-    for (int cid = tid; cid < valid * 4; cid += 256) {
-        const int row = cid >> 2, c16 = cid & 3;
-        const int64_t n = oc0 + c16 * 16;
-        if (n >= g.OC) continue;
-        const i32x4 v = *reinterpret_cast<const i32x4*>(patch + row * kPatchOutStride + c16 * 16);
-        uint8_t* dst = out + (pos0 + row) * g.OC + n;
-        if (vec_ok && n + 16 <= g.OC) {
-            __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
-        } else {
-            for (int e = 0; e < 16 && n + e < g.OC; e++) dst[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+        __syncthreads();
+
+        // ---- staging -> global
+        const int img = fdiv(tile, pg.tiles_y);
+        const int oy0 = (tile - img * (int)pg.tiles_y.d) * pg.R;
+        const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
+        const int valid = rows_here * (int)g.OW;
+        const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
+        for (int cid = tid; cid < valid * 4; cid += 256) {
+            const int row = cid >> 2, c16 = cid & 3;
+            const int64_t n = oc0 + c16 * 16;
+            if (n >= g.OC) continue;
+            const i32x4 v = *reinterpret_cast<const i32x4*>(stage + row * kPatchOutStride + c16 * 16);
+            uint8_t* dst = out + (pos0 + row) * g.OC + n;
+            if (vec_ok && n + 16 <= g.OC) {
+                __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
+            } else {
+                for (int e = 0; e < 16 && n + e < g.OC; e++) dst[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+            }
         }
     }
 }
@@ -1020,21 +1082,25 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             g.IC < (1 << 14) && g.W * g.SX < (1 << 14) && g.N * g.OH * g.OH < (1ll << 32)) {
             PatchGeom pg{};
             const size_t lds_max = 160 * 1024 - 512;
+            auto patch_need = [&](int R) {
+                return (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)g.IC;
+            };
             auto lds_need = [&](int R) {
-                const size_t patch = (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)g.IC;
-                const size_t stage = (size_t)((R * g.OW + 31) / 32) * 32 * kPatchOutStride;
-                return 64 * (size_t)Ktot + (patch > stage ? patch : stage);
+                return 64 * (size_t)Ktot + patch_need(R) + (size_t)((R * g.OW + 31) / 32) * 32 * kPatchOutStride;
             };
             int R = (int)(32 * kPatchMaxMT / g.OW);
             if (R > g.OH) R = (int)g.OH;
             while (R > 1 && lds_need(R) > lds_max) R--;
             if (lds_need(R) <= lds_max) {
                 const int64_t ocb = (g.OC + 63) / 64;
-                // enough workgroups to fill the device twice, as long as a tile keeps at least 4 row blocks
-                while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 512 && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
+                int cus = 0, devid = 0;
+                VPX_HIP_CHECK(hipGetDevice(&devid));
+                VPX_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, devid));
+                // enough tiles to fill the device twice, as long as a tile keeps at least 4 row blocks
+                while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 2ll * cus && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
                 if (const char* e = std::getenv("VPX_CONV_ROWS")) {
                     const int v = std::atoi(e);
-                    if (v >= 1 && v <= R) R = v;
+                    if (v >= 1 && lds_need(v) <= lds_max && v * g.OW <= 32 * kPatchMaxMT) R = v;
                 }
                 const int tiles_y = (int)((g.OH + R - 1) / R);
                 auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
@@ -1044,13 +1110,19 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 pg.MT = (int)((pg.R * g.OW + 31) / 32);
                 pg.nt = g.OC <= 32 ? 1 : 2;
                 pg.w_swz = Ktot % 64 == 0 ? 1 : 0;
+                pg.ntiles = (int)(g.N * tiles_y);
+                pg.patch_bytes = (int)patch_need(pg.R);
                 pg.tiles_y = fd(tiles_y);
                 pg.cpr = fd(Ktot / 16);
                 pg.cpp = fd(g.IC / 16);
                 pg.upr = fd((pg.PW * (g.IC / 16) + 63) / 64);
                 pg.ow = fd(g.OW);
                 const size_t lds = lds_need(pg.R);
-                const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
+                const int per_cu = lds <= 80 * 1024 ? 2 : 1;
+                int64_t blocks = (int64_t)cus * per_cu / ocb;
+                if (blocks < 1) blocks = 1;
+                if (blocks > pg.ntiles) blocks = pg.ntiles;
+                const dim3 grid((unsigned)blocks, (unsigned)ocb);
                 GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
                 const int pad_byte = t.zp_in & 0xff;
                 const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
