@@ -3,6 +3,8 @@
 Bars: convert / eltwise / fake_quantize / quantize / dequantize bit-exact (any NaN matches any NaN
 where arithmetic produced it); softmax and MVN within relative 2e-3, or one fp16 subnormal step
 (2^-24) in absolute terms for results that small."""
+import os
+
 import numpy as np
 import pytest
 

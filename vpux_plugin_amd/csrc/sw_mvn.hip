@@ -10,6 +10,12 @@
 // (MVN1Sum -> MVN1MeanVar -> MVN1Normalize,
 // src/vpux_compiler/src/NPU37XX/dialect/VPU/transforms/passes/decompose_mvn.cpp:82-129), with
 // centred partial sums instead of raw sum / sum of squares.
+//
+// Two launches on purpose.  A single launch whose workgroups keep their chunk in registers and
+// meet at a device-wide barrier (arrival counter + bounded wait) was built and measured: on this
+// part the barrier alone costs about 30 us (device-scope atomics from 1024 workgroups on 8 dies
+// meet in memory, not in a cache), against about 3 us for a launch boundary, and the second read
+// of the input comes from L2 / Infinity Cache anyway.
 #include "vpx_common.h"
 
 namespace vpx {
@@ -28,12 +34,20 @@ struct Moments {
     float n, mean, m2;
 };
 
+// A published record: 16 bytes, so that it moves as one access.
+struct __attribute__((aligned(16))) Record {
+    float n, mean, m2, pad;
+};
+__device__ __forceinline__ Moments unpack(const Record& r) {
+    return Moments{r.n, r.mean, r.m2};
+}
+
 // Chan/Golub/LeVeque pairwise combination of two sample sets.
 __device__ __forceinline__ Moments merge(Moments a, Moments b) {
     const float n = a.n + b.n;
     if (n == 0.f) return Moments{0.f, 0.f, 0.f};
     const float d = b.mean - a.mean;
-    const float w = b.n / n;
+    const float w = b.n * __builtin_amdgcn_rcpf(n);  // 1 ulp; the same everywhere, so still deterministic
     Moments r;
     r.n = n;
     r.mean = a.mean + d * w;
@@ -160,15 +174,17 @@ __device__ __forceinline__ float inv_std(Moments m, bool normalize_variance, flo
 }
 
 // Fixed-order merge of up to 256 published partials of one group.  Every wavefront does the
-// whole merge on its own (four partials per lane in sequence, then the butterfly), so no
-// exchange through local memory is needed and all wavefronts of all workgroups get the same bits.
-__device__ __forceinline__ Moments merge_partials(const Moments* __restrict__ partial, int chunks) {
+// whole merge on its own (lane l folds partials l, l+64, l+128, l+192 in sequence -- a wave reads
+// 64 consecutive records at a time --, then the butterfly), so all wavefronts of all workgroups get
+// the same bits.  `get(i)` returns partial i.
+template <class Get>
+__device__ __forceinline__ Moments merge_partials(Get get, int chunks) {
     const int lane = threadIdx.x & 63;
     Moments acc{0.f, 0.f, 0.f};
 #pragma unroll
     for (int k = 0; k < kMergeInKernel / 64; k++) {
-        const int i = lane * (kMergeInKernel / 64) + k;
-        if (i < chunks) acc = merge(acc, partial[i]);
+        const int i = k * 64 + lane;
+        if (i < chunks) acc = merge(acc, get(i));
     }
     return wave_merge(acc);
 }
@@ -190,8 +206,8 @@ __device__ __forceinline__ Moments block_merge(Moments m, Moments* smem) {
 // when `merged` is null, else read the finished result) and normalise.
 template <int MODE, bool ALIGNED>
 __global__ __launch_bounds__(kThreads) void mvn_chunk_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
-                                                             int64_t group_size, int chunks, Moments* partial,
-                                                             const Moments* merged, int normalize_variance, float eps) {
+                                                             int64_t group_size, int chunks, Record* partial,
+                                                             const Record* merged, int normalize_variance, float eps) {
     __shared__ Moments red[4];
     const int64_t group = blockIdx.x / chunks;
     const int chunk = blockIdx.x % chunks;
@@ -204,23 +220,24 @@ __global__ __launch_bounds__(kThreads) void mvn_chunk_kernel(const half_t* __res
         store_chunk<ALIGNED>(out + group * group_size, base, group_size, c, m.mean, inv_std(m, normalize_variance, eps));
     } else if (MODE == 1) {
         const Moments m = chunk_moments(c, base, group_size, red);
-        if (threadIdx.x == 0) partial[blockIdx.x] = m;
+        if (threadIdx.x == 0) partial[blockIdx.x] = Record{m.n, m.mean, m.m2, 0.f};
     } else {
-        const Moments total = merged ? merged[group] : merge_partials(partial + group * chunks, chunks);
+        const Record* mine = partial + group * chunks;
+        const Moments total = merged ? unpack(merged[group]) : merge_partials([&](int i) { return unpack(mine[i]); }, chunks);
         store_chunk<ALIGNED>(out + group * group_size, base, group_size, c, total.mean,
                              inv_std(total, normalize_variance, eps));
     }
 }
 
 // Groups with more than kMergeInKernel chunks: one workgroup per group folds its partials.
-__global__ __launch_bounds__(kThreads) void mvn_merge_kernel(const Moments* partial, Moments* merged, int chunks) {
+__global__ __launch_bounds__(kThreads) void mvn_merge_kernel(const Record* partial, Record* merged, int chunks) {
     __shared__ Moments tree[kThreads];
     const int64_t group = blockIdx.x;
     Moments acc{0.f, 0.f, 0.f};
     // lane t folds chunks t, t+256, ... in order, then the lanes are merged by the fixed tree
-    for (int c = threadIdx.x; c < chunks; c += kThreads) acc = merge(acc, partial[group * chunks + c]);
+    for (int c = threadIdx.x; c < chunks; c += kThreads) acc = merge(acc, unpack(partial[group * chunks + c]));
     const Moments total = block_merge(acc, tree);
-    if (threadIdx.x == 0) merged[group] = total;
+    if (threadIdx.x == 0) merged[group] = Record{total.n, total.mean, total.m2, 0.f};
 }
 
 // Per-channel statistics of a channel-minor layout (NHWC / NWHC): element (n,s,c) at
@@ -274,20 +291,21 @@ int launch_groups(const half_t* in, half_t* out, int64_t groups, int64_t group_s
     const unsigned blocks = (unsigned)(groups * chunks);
     if (chunks == 1) {
         hipLaunchKernelGGL((mvn_chunk_kernel<0, ALIGNED>), dim3(blocks), dim3(kThreads), 0, s, in, out, group_size, 1,
-                           (Moments*)nullptr, (const Moments*)nullptr, nv, eps);
+                           (Record*)nullptr, (const Record*)nullptr, nv, eps);
         VPX_HIP_CHECK(hipGetLastError());
         return VPX_RESULT_SUCCESS;
     }
     void* ws = nullptr;
-    const size_t need = sizeof(Moments) * ((size_t)blocks + (size_t)groups);
+    const size_t need = sizeof(Record) * ((size_t)blocks + (size_t)groups);
     int rc = get_workspace(s, need, &ws);
     if (rc) return rc;
-    Moments* partial = (Moments*)ws;
-    Moments* merged = partial + blocks;
+    Record* partial = (Record*)ws;
+    Record* merged = partial + blocks;
+
     hipLaunchKernelGGL((mvn_chunk_kernel<1, ALIGNED>), dim3(blocks), dim3(kThreads), 0, s, in, out, group_size, chunks,
-                       partial, (const Moments*)nullptr, nv, eps);
+                       partial, (const Record*)nullptr, nv, eps);
     VPX_HIP_CHECK(hipGetLastError());
-    const Moments* use_merged = nullptr;
+    const Record* use_merged = nullptr;
     if (chunks > kMergeInKernel) {
         hipLaunchKernelGGL(mvn_merge_kernel, dim3((unsigned)groups), dim3(kThreads), 0, s, partial, merged, chunks);
         VPX_HIP_CHECK(hipGetLastError());
