@@ -22,6 +22,13 @@ I8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA, published
 
 METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
 
+# Bytes moved through L2 per step, from rocprofv3 FETCH_SIZE / WRITE_SIZE counters scaled by a plain
+# copy of known size (profiles/<workload>__*.md hold the runs these come from).
+MEASURED_TRAFFIC = {
+    "c1_fake_quantize": 880465, "c2_softmax": 134240024, "c3_mvn": 12725340, "c4_conv": 16426621,
+    "c5_matmul": 384896480, "c5_dequantize": 135343006, "c5_eltwise_add": 270488016,
+}
+
 
 def _dev(a, f16=False):
     import torch
@@ -269,10 +276,10 @@ def roofline(w, dev_ms):
     if w.bound == "hbm":
         achieved = w.bytes / (dev_ms * 1e-3) / 1e9
         return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": w.kernel}
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(w.name), "kernel": w.kernel}
     achieved = w.ops / (dev_ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": round(achieved, 2), "peak": I8_PEAK_TOPS, "unit": "TOP/s",
-            "frac": round(achieved / I8_PEAK_TOPS, 4), "traffic": None, "kernel": w.kernel}
+            "frac": round(achieved / I8_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC.get(w.name), "kernel": w.kernel}
 
 
 def value_of(w, ms):
