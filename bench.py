@@ -25,7 +25,7 @@ METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
 # Bytes moved through L2 per step, from rocprofv3 FETCH_SIZE / WRITE_SIZE counters scaled by a plain
 # copy of known size (profiles/<workload>__*.md hold the runs these come from).
 MEASURED_TRAFFIC = {
-    "c1_fake_quantize": 880465, "c2_softmax": 134240024, "c3_mvn": 12725340, "c4_conv": 16426621,
+    "c1_fake_quantize": 880465, "c2_softmax": 134240024, "c3_mvn": 25450680, "c4_conv": 16426621,
     "c5_matmul": 384896480, "c5_dequantize": 135343006, "c5_eltwise_add": 270488016,
 }
 
