@@ -196,6 +196,23 @@ def make_c5(rt, part="matmul"):
         return Workload("c5_matmul", "int8 MatMul A[4096,4096] zp3 x B[4096,11008], PPE per-column + LeakyReLU 0.1 -> i8",
                         step, M * K + N * K + M * N + N * 16, 2 * M * K * N, "mfma", "int8", "nce_gemm_mfma", cpu)
     q = torch.randint(-128, 128, (M, N), dtype=torch.int8, device="cuda")
+    if part == "nce_eltwise":
+        # the quantized form of the same residual add: i8 + i8 -> i8 on the NCE eltwise path
+        res_q = torch.randint(-128, 128, (M, N), dtype=torch.int8, device="cuda")
+        out_q = torch.empty_like(q)
+        m1, m2, mo, so = rt.eltwise_quantization_approximation(0.05, 0.04, 0.07, 0)
+        t = rt.NceTask()
+        t.task_type, t.eltwise_type = rt.NCE_ELTWISE, rt.ELTWISE_ADD
+        t.input, t.weights, t.weight_table, t.output = q.data_ptr(), res_q.data_ptr(), None, out_q.data_ptr()
+        t.input_type = t.weights_type = t.output_type = rt.NN_I8
+        t.N, t.H, t.W, t.IC, t.OC = 1, M, 1, N, N
+        t.kernel_size[0] = t.kernel_size[1] = t.kernel_strides[0] = t.kernel_strides[1] = 1
+        t.zp_in, t.zp_w, t.zp_out = 3, -2, 0
+        t.ppe = rt.PpeInt(rt.PPE_NOOP, -128, 127, 1, 0, mo, so, m1, m2)
+        step = _nce_step(rt, t)
+        step.keep = (q, res_q, out_q, t)
+        return Workload("c5_nce_eltwise", "NCE eltwise add i8 + i8 -> i8 [4096,11008] (quantized residual; not a BASELINE config)",
+                        step, M * N * 3, 0, "hbm", "int8", "nce_eltwise_kernel")
     deq = torch.empty((M, N), dtype=torch.float16, device="cuda")
     if part == "dequant":
         ops = [rt.Operand(q), rt.Operand(deq)]
@@ -233,6 +250,7 @@ MAKERS = {
     "c5_matmul": lambda rt: make_c5(rt, "matmul"),
     "c5_dequantize": lambda rt: make_c5(rt, "dequant"),
     "c5_eltwise_add": lambda rt: make_c5(rt, "add"),
+    "c5_nce_eltwise": lambda rt: make_c5(rt, "nce_eltwise"),
 }
 
 

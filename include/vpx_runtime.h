@@ -87,6 +87,12 @@ VPX_API const char* vpx_sw_kernel_name(uint32_t i);
  *       words 0 and 1 (weight / sparsity pointers) are NPU addresses and are ignored
  *   output  NHWC  [N][OH][OW][OC] u8 or i8
  * A matmul A[M][K] x B[N][K] -> [M][N] is the task N=1, H=M, W=1, IC=K, OC=N, 1x1 kernel.
+ *
+ * task_type ELTWISE (the quantized residual add of a network): `weights` is the second input,
+ * same shape and layout as `input`, zero point zp_w; OC = IC; weight_table, kernel_* are not used.
+ *   acc = (in1 - zp_in) * in1_quant_mult +/- (in2 - zp_w) * in2_quant_mult       (int32)
+ *   t = acc * quant_mult, PReLU stage as above, r = round_half_even(t / 2^quant_shift) + zp_out, clamp
+ * ("input1 * MULT1 --> + --> * MULT_OUT >> SHIFT_OUT", quantization.cpp:461-462).
  * Arithmetic: acc = sum (in - zp_in) * (w - zp_w) over the taps inside the image (padding adds 0),
  * then the integer PPE in the order the compiler programs it
  * (src/vpux_compiler/src/NPU40XX/dialect/VPUIPDPU/transforms/passes/expand_dpu_config/
@@ -96,7 +102,10 @@ VPX_API const char* vpx_sw_kernel_name(uint32_t i);
  * ------------------------------------------------------------------------------------------ */
 
 /* VPUIP::NCETaskType (tblgen/.../VPUIP/attributes.td:56-70) */
-typedef enum vpx_nce_task_type_t { VPX_NCE_CONV = 0 } vpx_nce_task_type_t;
+typedef enum vpx_nce_task_type_t { VPX_NCE_CONV = 0, VPX_NCE_ELTWISE = 4 } vpx_nce_task_type_t;
+
+/* VPU::EltwiseType values the ELTWISE task implements (tblgen/.../VPU/attributes.td:237-252) */
+typedef enum vpx_eltwise_type_t { VPX_ELTWISE_ADD = 0, VPX_ELTWISE_SUBTRACT = 1 } vpx_eltwise_type_t;
 
 /* VPU::PPEMode values used by the integer pipeline (tblgen/.../VPU/attributes.td:327-369) */
 typedef enum vpx_ppe_mode_t {
@@ -113,6 +122,13 @@ typedef struct vpx_ppe_int_t {
     int32_t clamp_high;
     int32_t lrelu_mult;
     int32_t lrelu_shift;
+    /* ELTWISE tasks only (a CONV task takes its scale from the weight table and ignores these):
+     * the per-tensor output and input multipliers EltwiseQuantizationApproximation produces
+     * (src/vpux_compiler/src/utils/quantization.cpp:455-516, ppe_factory.cpp:300-310) */
+    int32_t quant_mult;
+    int32_t quant_shift;
+    int32_t in1_quant_mult;
+    int32_t in2_quant_mult;
 } vpx_ppe_int_t;
 
 typedef struct vpx_nce_task_t {
@@ -131,6 +147,7 @@ typedef struct vpx_nce_task_t {
     int32_t kernel_padding[4]; /* left, right, top, bottom (VPU_PaddingAttr order) */
     int32_t zp_in, zp_w, zp_out;
     vpx_ppe_int_t ppe;
+    int32_t eltwise_type; /* vpx_eltwise_type_t, ELTWISE tasks only */
 } vpx_nce_task_t;
 
 VPX_API int vpx_nce_task(const vpx_nce_task_t* task, void* stream);

@@ -448,3 +448,21 @@ void orc_nce_conv(const orc_conv_t* d, const void* in, const void* w, const int3
     const int64_t OW = (d->W + d->pad_left + d->pad_right - d->KX) / d->stride_x + 1;
     orc_nce_conv_rows(d, in, w, wt, out, acc_out, 0, d->N * OH * OW);
 }
+
+void orc_nce_eltwise(const void* a, int a_signed, const void* b, int b_signed, void* out, int out_signed, int64_t n,
+                     int32_t zp_a, int32_t zp_b, int32_t mult_a, int32_t mult_b, int subtract, int32_t out_mult,
+                     int32_t out_shift, const orc_ppe_t* ppe) {
+    const uint8_t* pa = (const uint8_t*)a;
+    const uint8_t* pb = (const uint8_t*)b;
+    uint8_t* po = (uint8_t*)out;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        const int32_t va = (a_signed ? (int32_t)(int8_t)pa[i] : (int32_t)pa[i]) - zp_a;
+        const int32_t vb = (b_signed ? (int32_t)(int8_t)pb[i] : (int32_t)pb[i]) - zp_b;
+        const int32_t acc = va * mult_a + (subtract ? -1 : 1) * vb * mult_b;
+        int32_t r = orc_ppe_requant(acc, 0, out_mult, out_shift, ppe);
+        if (out_signed) r = r < -128 ? -128 : (r > 127 ? 127 : r);
+        else r = r < 0 ? 0 : (r > 255 ? 255 : r);
+        po[i] = (uint8_t)r;
+    }
+}

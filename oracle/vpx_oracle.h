@@ -114,6 +114,13 @@ void orc_nce_conv(const orc_conv_t* d, const void* in, const void* w, const int3
 void orc_nce_conv_rows(const orc_conv_t* d, const void* in, const void* w, const int32_t* wt, void* out,
                        int32_t* acc_out, int64_t row0, int64_t nrows);
 
+/* ---- NCE eltwise add / subtract (EltwiseQuantizationApproximation, utils/quantization.cpp:455-516) ----
+ * acc = (a - zp_a) * mult_a +/- (b - zp_b) * mult_b, then the integer PPE with bias 0 and the
+ * per-tensor out_mult / out_shift.  "parity unpinned" against silicon like orc_ppe_requant. */
+void orc_nce_eltwise(const void* a, int a_signed, const void* b, int b_signed, void* out, int out_signed, int64_t n,
+                     int32_t zp_a, int32_t zp_b, int32_t mult_a, int32_t mult_b, int subtract, int32_t out_mult,
+                     int32_t out_shift, const orc_ppe_t* ppe);
+
 int orc_num_threads(void);
 void orc_set_num_threads(int n);
 

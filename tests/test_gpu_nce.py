@@ -205,6 +205,52 @@ def test_matmul_config_c5_full_size_and_chain(rt, orc, dev):
     assert bool((deq == table[(out.long() + 128)]).all())
 
 
+@pytest.mark.parametrize("subtract", [False, True])
+@pytest.mark.parametrize("mode", ["NOOP", "LPRELU"])
+def test_nce_eltwise(rt, orc, dev, subtract, mode):
+    """Quantized residual add / subtract: every combination of operand signedness, odd and even output
+    zero points, partial clamp windows, ragged sizes and an unaligned view."""
+    import torch
+    rng = np.random.default_rng(95)
+    in1_mult, in2_mult, out_mult, out_shift = rt.eltwise_quantization_approximation(0.02, 0.035, 0.05, 1 if subtract else 0)
+    md = getattr(rt, "PPE_" + mode)
+    pm, ps = (1638, 14) if mode == "LPRELU" else (1, 0)
+    for a_signed, b_signed, out_signed, zp1, zp2, zpo, clamp, shape in (
+            (False, True, False, 128, -3, 7, (0, 255), (2, 9, 11, 64)),
+            (True, True, True, 0, 5, 0, (-128, 127), (1, 7, 5, 33)),
+            (True, False, True, -7, 100, -20, (-100, 90), (3, 4, 4, 16)),
+            (False, False, False, 3, 250, 128, (128, 255), (1, 1, 1, 5))):
+        a = rng.integers(-128, 128, shape).astype(np.int8) if a_signed else rng.integers(0, 256, shape, dtype=np.uint8)
+        b = rng.integers(-128, 128, shape).astype(np.int8) if b_signed else rng.integers(0, 256, shape, dtype=np.uint8)
+        ppe = rt.PpeInt(md, clamp[0], clamp[1], pm, ps, out_mult, out_shift, in1_mult, in2_mult)
+        out = torch.full(shape, 99, dtype=torch.int8 if out_signed else torch.uint8, device=dev)
+        rt.nce_eltwise(dev_t(a, dev), dev_t(b, dev), out, ppe, zp1, zp2, zpo, subtract=subtract)
+        torch.cuda.synchronize()
+        assert rt.nce_last_kernel() == "nce_eltwise_kernel"
+        want = orc.nce_eltwise(a, b, orc.ppe(pm if mode == "LPRELU" else 1, ps, zpo, clamp[0], clamp[1]), zp1, zp2, in1_mult,
+                               in2_mult, out_mult, out_shift, subtract=subtract, out_signed=out_signed)
+        got = out.cpu().numpy()
+        assert np.array_equal(got, want), "%s: %d mismatches" % (shape, int((got != want).sum()))
+
+
+def test_nce_eltwise_full_size_residual(rt, orc, dev):
+    """[4096, 11008] i8 + i8 -> i8, the quantized form of the C5 residual add, whole tensor against the oracle."""
+    import torch
+    rng = np.random.default_rng(96)
+    shape = (1, 4096, 1, 11008)
+    a = rng.integers(-128, 128, shape).astype(np.int8)
+    b = rng.integers(-128, 128, shape).astype(np.int8)
+    in1_mult, in2_mult, out_mult, out_shift = rt.eltwise_quantization_approximation(0.05, 0.04, 0.07, 0)
+    ppe = rt.PpeInt(rt.PPE_NOOP, -128, 127, 1, 0, out_mult, out_shift, in1_mult, in2_mult)
+    out = torch.empty(shape, dtype=torch.int8, device=dev)
+    rt.nce_eltwise(dev_t(a, dev), dev_t(b, dev), out, ppe, 3, -2, 0)
+    torch.cuda.synchronize()
+    want = orc.nce_eltwise(a, b, orc.ppe(1, 0, 0, -128, 127), 3, -2, in1_mult, in2_mult, out_mult, out_shift, out_signed=True)
+    got = out.cpu().numpy()
+    assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
+    assert 0.001 < (np.abs(got.astype(np.int32)) == 127).mean() + (got == -128).mean() < 0.5
+
+
 def test_nce_rejects_bad_descriptors(rt, dev):
     import torch
     inp = torch.zeros((1, 4, 4, 16), dtype=torch.uint8, device=dev)

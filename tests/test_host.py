@@ -63,8 +63,10 @@ def test_error_codes_without_gpu(rt):
     assert L.vpx_nce_task(None, None) == rt.ERROR_INVALID_NULL_HANDLE
     t = rt.NceTask()
     assert L.vpx_nce_task(C.byref(t), None) == rt.ERROR_INVALID_NULL_HANDLE  # null buffers
-    t.task_type = 4  # ELTWISE
+    t.task_type = 1  # DWCONV
     assert L.vpx_nce_task(C.byref(t), None) == rt.ERROR_UNSUPPORTED_FEATURE
+    t.task_type = 4  # ELTWISE: implemented, so the null buffers are what is refused
+    assert L.vpx_nce_task(C.byref(t), None) == rt.ERROR_INVALID_NULL_HANDLE
 
 
 def test_half_conversion_matches_oracle(rt, orc):

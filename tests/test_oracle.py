@@ -351,3 +351,36 @@ def test_nce_conv_against_brute_force(orc):
     # row-range evaluation equals the full evaluation on those rows
     part = orc.nce_matmul(A, B, wt2, orc.ppe(1638, 14, 0, -128, 127), zp_a=3, rows=(2, 4))
     assert np.array_equal(part[2:6], out[2:6])
+
+
+def test_nce_eltwise_against_exact_integers_and_real_arithmetic(orc):
+    """The eltwise restatement against Python integers (round half even with fractions) and, loosely,
+    against the real-valued sum it approximates; multipliers from the reference's golden case
+    (tests/unit/vpux_compiler/utils/quantization_tests.cpp style: scales 0.02 / 0.035 -> 0.05)."""
+    from fractions import Fraction
+    rng = np.random.default_rng(90)
+    a = rng.integers(0, 256, 4000, dtype=np.uint8)
+    b = rng.integers(-128, 128, 4000).astype(np.int8)
+    s1, s2, so = 0.02, 0.035, 0.05
+    m1, sh1, _ = orc.approximate(15, s1)
+    m2, sh2, _ = orc.approximate(15, s2)
+    mo, sho, _ = orc.approximate(15, 1.0 / so)
+    shift_in = max(sh1, sh2)
+    m1a, m2a = m1 << (shift_in - sh1), m2 << (shift_in - sh2)
+    assert m1a < 65536 and m2a < 65536
+    zp_a, zp_b, zp_o = 128, -3, 7
+    for subtract in (False, True):
+        p = orc.ppe(1, 0, zp_o, 0, 255)
+        got = orc.nce_eltwise(a, b, p, zp_a, zp_b, m1a, m2a, mo, sho + shift_in, subtract=subtract)
+        sign = -1 if subtract else 1
+        want = np.empty_like(got)
+        real = np.empty(a.size)
+        for i in range(a.size):
+            acc = (int(a[i]) - zp_a) * m1a + sign * (int(b[i]) - zp_b) * m2a
+            t = Fraction(acc * mo, 1 << (sho + shift_in))
+            r = round(t)  # Python rounds halves to even
+            want[i] = min(255, max(0, r + zp_o))
+            real[i] = ((int(a[i]) - zp_a) * s1 + sign * (int(b[i]) - zp_b) * s2) / so + zp_o
+        assert np.array_equal(got, want)
+        unsat = (real > 1) & (real < 254)
+        assert np.abs(got[unsat].astype(np.float64) - real[unsat]).max() <= 1.0

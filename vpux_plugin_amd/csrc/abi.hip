@@ -403,10 +403,27 @@ int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_si
 int vpx_nce_task(const vpx_nce_task_t* t, void* stream) {
     last_error().clear();
     VPX_REQUIRE(t != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "NCE task descriptor is null");
-    VPX_REQUIRE(t->task_type == VPX_NCE_CONV, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "NCE task type %d is not implemented (CONV only)",
-                t->task_type);
-    VPX_REQUIRE(t->input && t->weights && t->weight_table && t->output, VPX_RESULT_ERROR_INVALID_NULL_HANDLE,
-                "NCE task: input, weights, weight_table and output must all be set");
+    VPX_REQUIRE(t->task_type == VPX_NCE_CONV || t->task_type == VPX_NCE_ELTWISE, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "NCE task type %d is not implemented (CONV and ELTWISE only)", t->task_type);
+    const bool eltwise = t->task_type == VPX_NCE_ELTWISE;
+    VPX_REQUIRE(t->input && t->weights && (eltwise || t->weight_table) && t->output, VPX_RESULT_ERROR_INVALID_NULL_HANDLE,
+                "NCE task: input, weights%s and output must all be set", eltwise ? " (second input)" : ", weight_table");
+    if (eltwise) {
+        VPX_REQUIRE(t->eltwise_type == VPX_ELTWISE_ADD || t->eltwise_type == VPX_ELTWISE_SUBTRACT, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                    "NCE eltwise type %d is not implemented (ADD and SUBTRACT only)", t->eltwise_type);
+        VPX_REQUIRE(t->OC == t->IC, VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE eltwise: OC %lld differs from IC %lld",
+                    (long long)t->OC, (long long)t->IC);
+        // input multipliers are unsigned 16-bit registers, the output shift has 6 bits (quantization.cpp:466-473)
+        VPX_REQUIRE(t->ppe.in1_quant_mult >= 0 && t->ppe.in1_quant_mult <= 65535 && t->ppe.in2_quant_mult >= 0 &&
+                            t->ppe.in2_quant_mult <= 65535 && t->ppe.quant_shift >= 0 && t->ppe.quant_shift <= 63 &&
+                            t->ppe.quant_mult >= -32768 && t->ppe.quant_mult <= 32767,
+                    VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "NCE eltwise: multipliers %d, %d, %d / shift %d outside the register ranges", t->ppe.in1_quant_mult,
+                    t->ppe.in2_quant_mult, t->ppe.quant_mult, t->ppe.quant_shift);
+        VPX_REQUIRE(t->zp_in >= -128 && t->zp_in <= 255 && t->zp_w >= -128 && t->zp_w <= 255 && t->zp_out >= -(1 << 20) &&
+                            t->zp_out <= (1 << 20),
+                    VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE eltwise: zero point out of range");
+    }
     const auto is8 = [](int32_t ty) { return ty == VPX_NN_U8 || ty == VPX_NN_I8; };
     VPX_REQUIRE(is8(t->input_type) && is8(t->weights_type) && is8(t->output_type), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
                 "NCE task: only U8/I8 input, weights and output are implemented (got %s, %s, %s)",

@@ -15,6 +15,7 @@
 // the top bit) and add the missing term to the bias: acc_true = acc_raw + k * sum_k w[oc][k] with
 // k = 128 - zp_in (u8) or -zp_in (i8); padded taps are filled with the byte that stands for the
 // zero point so they contribute exactly 0, as the MPE does (runtime_dpu_parser_imports.cpp.inc:872-879).
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
 #include <type_traits>
@@ -965,12 +966,119 @@ __global__ __launch_bounds__(256, TMW <= 4 ? 2 : 1) void nce_conv_patch(const in
     }
 }
 
+// ---------------------------------------------------------------- NCE eltwise (quantized add / subtract)
+// out = PPE((a - zp_a) * m1 +/- (b - zp_b) * m2): a streaming kernel, 16 bytes of each operand per
+// lane.  The zero points are folded into the bias (acc = a * m1 +/- b * m2 - (zp_a * m1 +/- zp_b * m2)),
+// which leaves two 24-bit multiply-adds per value in front of the shared PPE tail.
+struct EltParams {
+    int m1, m2;  // m2 negated for a subtraction
+    ChanPrep cp;
+    PpePack pk;
+    int general;
+};
+
+template <bool A_SIGNED, bool B_SIGNED, bool SAME_F>
+__global__ __launch_bounds__(256) void nce_eltwise_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                                                          uint8_t* __restrict__ out, int64_t n_vec, int64_t n,
+                                                          EltParams e) {
+    auto val = [](unsigned word, int k, bool sgn) {
+        return sgn ? (int)(int8_t)(word >> (8 * k)) : (int)((word >> (8 * k)) & 0xffu);
+    };
+    auto four = [&](unsigned wa, unsigned wb, auto general_c) {
+        int acc[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) acc[k] = val(wa, k, A_SIGNED) * e.m1 + val(wb, k, B_SIGNED) * e.m2;
+        return ppe_pack4<SAME_F, decltype(general_c)::value>(acc[0], acc[1], acc[2], acc[3], e.cp, e.pk);
+    };
+    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (v < n_vec) {
+        const i32x4 qa = reinterpret_cast<const i32x4*>(a)[v];
+        const i32x4 qb = reinterpret_cast<const i32x4*>(b)[v];
+        i32x4 r;
+        if (e.general) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) r[j] = (int)four((unsigned)qa[j], (unsigned)qb[j], std::true_type{});
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) r[j] = (int)four((unsigned)qa[j], (unsigned)qb[j], std::false_type{});
+        }
+        __builtin_nontemporal_store(r, reinterpret_cast<i32x4*>(out) + v);
+    }
+    // ragged tail (fewer than 16 bytes) and unaligned tensors: one value per lane
+    if (blockIdx.x == gridDim.x - 1) {
+        for (int64_t i = n_vec * 16 + threadIdx.x; i < n; i += 256) {
+            const int acc = val(a[i], 0, A_SIGNED) * e.m1 + val(b[i], 0, B_SIGNED) * e.m2;
+            out[i] = (uint8_t)ppe_pack4<SAME_F, true>(acc, 0, 0, 0, e.cp, e.pk);
+        }
+    }
+}
+
 template <class KernelT>
 int set_dyn_lds(KernelT kernel, size_t bytes) {
     if (bytes > 64 * 1024) {
         VPX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
     }
+    return VPX_RESULT_SUCCESS;
+}
+
+// PPE of one eltwise value on the host: decides which device variant is needed
+int launch_nce_eltwise(const vpx_nce_task_t& t, const Ppe& ppe, hipStream_t s, const char** kernel_name) {
+    const bool a_signed = t.input_type == VPX_NN_I8, b_signed = t.weights_type == VPX_NN_I8, out_signed = t.output_type == VPX_NN_I8;
+    const int64_t n = t.N * t.H * t.W * t.IC;
+    *kernel_name = "nce_eltwise_kernel";
+    if (n == 0) return VPX_RESULT_SUCCESS;
+    const int sign = t.eltwise_type == VPX_ELTWISE_SUBTRACT ? -1 : 1;
+    const long long bias = -((long long)t.zp_in * t.ppe.in1_quant_mult + (long long)sign * t.zp_w * t.ppe.in2_quant_mult);
+    VPX_REQUIRE(bias > -(1ll << 30) && bias < (1ll << 30), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "NCE eltwise: zero points and input multipliers do not fit the 32-bit accumulator");
+    const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
+    int lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin, hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
+    if (lo > tmax) lo = tmax;
+    if (hi < tmin) hi = tmin;
+    if (lo > hi) lo = hi;
+    EltParams e{};
+    e.m1 = t.ppe.in1_quant_mult;
+    e.m2 = sign * t.ppe.in2_quant_mult;
+    // host copy of ppe_prepare_packed / make_ppe_pack
+    const double f_pos = std::ldexp((double)t.ppe.quant_mult, -t.ppe.quant_shift);
+    const double f_neg = std::ldexp((double)((long long)t.ppe.quant_mult * (long long)ppe.prelu_mult), -(t.ppe.quant_shift + ppe.prelu_shift));
+    auto bmax = [](double f) {
+        const float a = std::fabs((float)f);
+        return a <= 0.5f ? 0x7fffffff : (int)(1.0e9f / a);
+    };
+    e.cp.f_pos = f_pos;
+    e.cp.f_neg = f_neg;
+    e.cp.bias = (int)((unsigned)(int)bias + 0x80000000u);
+    e.cp.sgn = t.ppe.quant_mult < 0 ? -1 : 0;
+    e.cp.bmax_pos = bmax(f_pos);
+    e.cp.bmax_neg = bmax(f_neg);
+    const int off = out_signed ? 128 : 0, z = t.zp_out + off;
+    e.pk = PpePack{6755399441055744.0 + (double)(z & ~1), z & 1, lo + off, hi + off, out_signed ? 0x80808080u : 0u};
+    e.general = (e.cp.bmax_pos != 0x7fffffff || e.cp.bmax_neg != 0x7fffffff || (z & 1)) ? 1 : 0;
+    const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
+    const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights) |
+                           reinterpret_cast<uintptr_t>(t.output)) & 15) == 0;
+    const int64_t n_vec = aligned ? n / 16 : 0;
+    const int64_t blocks64 = n_vec > 0 ? (n_vec + 255) / 256 : 1;
+    VPX_REQUIRE(blocks64 < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "NCE eltwise: tensor of %lld elements is too large", (long long)n);
+    const dim3 grid((unsigned)blocks64), block(256);
+#define VPX_ELT(AS, BS, SF)                                                                                            \
+    hipLaunchKernelGGL((nce_eltwise_kernel<AS, BS, SF>), grid, block, 0, s, (const uint8_t*)t.input,                   \
+                       (const uint8_t*)t.weights, (uint8_t*)t.output, n_vec, n, e)
+    const int sel = (a_signed ? 4 : 0) | (b_signed ? 2 : 0) | (same_f ? 1 : 0);
+    switch (sel) {
+    case 0: VPX_ELT(false, false, false); break;
+    case 1: VPX_ELT(false, false, true); break;
+    case 2: VPX_ELT(false, true, false); break;
+    case 3: VPX_ELT(false, true, true); break;
+    case 4: VPX_ELT(true, false, false); break;
+    case 5: VPX_ELT(true, false, true); break;
+    case 6: VPX_ELT(true, true, false); break;
+    default: VPX_ELT(true, true, true); break;
+    }
+#undef VPX_ELT
+    VPX_HIP_CHECK(hipGetLastError());
     return VPX_RESULT_SUCCESS;
 }
 
@@ -1000,6 +1108,8 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     case VPX_PPE_LPRELU: ppe.prelu_mult = t.ppe.lrelu_mult; ppe.prelu_shift = t.ppe.lrelu_shift; break;
     default: return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "NCE task: PPE mode %d is not an integer-pipeline mode", t.ppe.mode);
     }
+
+    if (t.task_type == VPX_NCE_ELTWISE) return launch_nce_eltwise(t, ppe, s, kernel_name);
 
     const int64_t Mtot = g.N * g.OH * g.OW;
     const int64_t Ktot = (int64_t)g.KY * g.KX * g.IC;

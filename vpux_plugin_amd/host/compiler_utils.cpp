@@ -212,6 +212,10 @@ int vpx_retrieve_ppe_int(int post_op, double param0, double param1, const vpx_qu
     ppe->clamp_high = std::numeric_limits<int32_t>::max();
     ppe->lrelu_mult = 1;
     ppe->lrelu_shift = 0;
+    ppe->quant_mult = 1;  // the eltwise-only fields: neutral
+    ppe->quant_shift = 0;
+    ppe->in1_quant_mult = 1;
+    ppe->in2_quant_mult = 1;
     const bool q = out_type->is_quantized != 0;
     switch (post_op) {
     case VPX_POSTOP_NONE:

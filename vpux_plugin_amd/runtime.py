@@ -46,7 +46,8 @@ class TensorDesc(C.Structure):
 
 class PpeInt(C.Structure):
     _fields_ = [("mode", C.c_int32), ("clamp_low", C.c_int32), ("clamp_high", C.c_int32), ("lrelu_mult", C.c_int32),
-                ("lrelu_shift", C.c_int32)]
+                ("lrelu_shift", C.c_int32), ("quant_mult", C.c_int32), ("quant_shift", C.c_int32),
+                ("in1_quant_mult", C.c_int32), ("in2_quant_mult", C.c_int32)]
 
 
 class QuantType(C.Structure):
@@ -60,7 +61,11 @@ class NceTask(C.Structure):
                 ("output_type", C.c_int32), ("N", C.c_int64), ("H", C.c_int64), ("W", C.c_int64), ("IC", C.c_int64),
                 ("OC", C.c_int64), ("kernel_size", C.c_int32 * 2), ("kernel_strides", C.c_int32 * 2),
                 ("kernel_padding", C.c_int32 * 4), ("zp_in", C.c_int32), ("zp_w", C.c_int32), ("zp_out", C.c_int32),
-                ("ppe", PpeInt)]
+                ("ppe", PpeInt), ("eltwise_type", C.c_int32)]
+
+
+NCE_CONV, NCE_ELTWISE = 0, 4
+ELTWISE_ADD, ELTWISE_SUBTRACT = 0, 1
 
 
 # every symbol include/vpx_runtime.h and include/vpx_compiler_utils.h declare
@@ -347,6 +352,24 @@ def nce_task(inp, weights, weight_table, out, ppe, zp_in=0, zp_w=0, zp_out=0, st
     for i in range(4):
         t.kernel_padding[i] = pads[i]
     t.zp_in, t.zp_w, t.zp_out = zp_in, zp_w, zp_out
+    t.ppe = ppe
+    check(lib().vpx_nce_task(C.byref(t), _stream_handle(stream)))
+    return out
+
+
+def nce_eltwise(in1, in2, out, ppe, zp_in1=0, zp_in2=0, zp_out=0, subtract=False, stream=None):
+    """Quantized add / subtract of two NHWC 8-bit tensors of one shape (NCE ELTWISE task); `ppe` carries
+    quant_mult / quant_shift / in1_quant_mult / in2_quant_mult."""
+    assert in1.shape == in2.shape == out.shape and in1.dim() == 4
+    N, H, W, IC = in1.shape
+    t = NceTask()
+    t.task_type = NCE_ELTWISE
+    t.eltwise_type = ELTWISE_SUBTRACT if subtract else ELTWISE_ADD
+    t.input, t.weights, t.weight_table, t.output = in1.data_ptr(), in2.data_ptr(), None, out.data_ptr()
+    t.input_type, t.weights_type, t.output_type = (_torch_dtype_code(x) for x in (in1, in2, out))
+    t.N, t.H, t.W, t.IC, t.OC = N, H, W, IC, IC
+    t.kernel_size[0] = t.kernel_size[1] = t.kernel_strides[0] = t.kernel_strides[1] = 1
+    t.zp_in, t.zp_w, t.zp_out = zp_in1, zp_in2, zp_out
     t.ppe = ppe
     check(lib().vpx_nce_task(C.byref(t), _stream_handle(stream)))
     return out
