@@ -100,7 +100,7 @@ def make_c2(rt):
         xs = np.ascontiguousarray(c["x"].reshape(-1, 512)[:rows])
         return lambda: orc.softmax_f16(xs, 1), xs.size * 4
     return Workload("c2_softmax", "Softmax fp16 last axis [8,16,512,512], 5% of logits masked to -60000",
-                    _prebuilt_sw_launch(rt, "softmax", blob, ops), n * 4, 0, "hbm", "f16", "softmax_rows_wave_f16", cpu)
+                    _prebuilt_sw_launch(rt, "softmax", blob, ops), n * 4, 0, "hbm", "f16", "softmax_rows_f16", cpu)
 
 
 def make_c3(rt):

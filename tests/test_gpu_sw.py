@@ -252,7 +252,11 @@ def _softmax(rt, dev, x_bits, axis, pad=0, packed=True, f32=False):
 
 @pytest.mark.parametrize("shape,axis", [((64, 512), 1), ((3, 5, 1024), 2), ((7, 2048), 1), ((5, 4096), 1), ((33, 40), 1),
                                         ((9, 1000), 1), ((4, 8200), 1), ((2, 3, 4, 4), 3), ((6, 32, 4, 4), 1),
-                                        ((5, 17, 300), 1), ((17, 64), 0), ((2, 3, 50, 7), 2)])
+                                        ((5, 17, 300), 1), ((17, 64), 0), ((2, 3, 50, 7), 2),
+                                        # rows that are not 16-byte aligned, long rows (one workgroup per row), and beyond
+                                        ((65, 500), 1), ((7, 511), 1), ((130, 197), 1), ((3, 1023), 1), ((9, 4099), 1),
+                                        ((3, 32768), 1), ((5, 20000), 1), ((6, 8191), 1), ((2, 33000), 1), ((2, 40001), 1),
+                                        ((20000, 8), 1), ((17000, 509), 1)])
 def test_softmax_shapes_and_axes(rt, orc, dev, shape, axis):
     rng = np.random.default_rng(hash((shape, axis)) % 2 ** 32)
     x = rng.normal(0, 3, shape).astype(np.float32)

@@ -6,8 +6,9 @@
 //   rows_wave  : reduction axis is the innermost, contiguous one and a row fits the registers of one
 //                wavefront (up to 4096 fp16 / 2048 fp32 values): one 64-lane wave owns a row, 128-bit
 //                loads, max and sum by DPP/swizzle butterflies, single pass over HBM.  fp16 rows
-//                without padding take rows_wave_f16, the same scheme with about half the
-//                instructions (packed-half maximum, mixed-precision fma).
+//                without padding take rows_f16, the same scheme with about half the
+//                instructions (packed-half maximum, mixed-precision fma); it also serves rows of
+//                up to 32768 values (one workgroup per row) and rows that are not 16-byte aligned.
 //   rows_block : innermost axis of any length or alignment: one workgroup per row, three passes.
 //   lines      : reduction over an outer (strided) axis: one lane per line, lanes adjacent along the
 //                innermost dimension so every step of the axis is a coalesced access.
@@ -179,25 +180,43 @@ __device__ __forceinline__ half2_t dpp_h2(half2_t v) {
     return __builtin_bit_cast(half2_t, __builtin_amdgcn_update_dpp(i, i, CTRL, 0xf, 0xf, true));
 }
 
-template <int NV, int ROWS>
-__global__ __launch_bounds__(256) void softmax_rows_wave_f16(const half_t* __restrict__ in, half_t* __restrict__ out,
-                                                             RowMap map, int64_t rows, int len) {
-    const int lane = threadIdx.x & 63;
-    const int64_t row0 = ((int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) * ROWS;
+// LANES = 64: a wave owns ROWS rows (4 waves of a workgroup work independently);
+// LANES = 256: the workgroup owns one row (rows of up to 32768 values), reductions cross LDS.
+// MISALIGNED: rows start anywhere (odd lengths); the row is read through 16-byte-aligned vectors
+// that may stick out at both ends -- those slots are masked to -inf, which makes them 0 after the
+// exponential -- and the two ragged ends are stored value by value.  Input and output rows must
+// be misaligned by the same amount.
+template <int NV, int ROWS, int LANES, bool MISALIGNED>
+__global__ __launch_bounds__(256) void softmax_rows_f16(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                        RowMap map, int64_t rows, int len) {
+    static_assert(LANES == 64 || (LANES == 256 && ROWS == 1), "a workgroup-wide row comes alone");
+    __shared__ float red[2][4];
+    const int lane = LANES == 64 ? (threadIdx.x & 63) : threadIdx.x;
+    const int64_t unit = LANES == 64 ? (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : blockIdx.x;
+    const int64_t row0 = unit * ROWS;
     if (row0 >= rows) return;
 
     half8_t h[ROWS][NV];
     int64_t ooff[ROWS];
+    int mis[ROWS];
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
         const int64_t row = row0 + r < rows ? row0 + r : rows - 1;  // clamp: duplicates are not stored
         int64_t ioff;
         row_offsets(map, row, ioff, ooff[r]);
+        mis[r] = MISALIGNED ? (int)((reinterpret_cast<uintptr_t>(in + ioff) >> 1) & 7) : 0;
+        const half_t* src = in + ioff - mis[r];
+        const int end = len + mis[r];
 #pragma unroll
         for (int j = 0; j < NV; j++) {
-            const int e0 = (j * 64 + lane) * 8;
-            if (e0 < len) {
-                h[r][j] = *reinterpret_cast<const half8_t*>(in + ioff + e0);
+            const int e0 = (j * LANES + lane) * 8;
+            if (e0 < end) {
+                h[r][j] = *reinterpret_cast<const half8_t*>(src + e0);
+                if (MISALIGNED && (e0 < mis[r] || e0 + 8 > end)) {
+#pragma unroll
+                    for (int k = 0; k < 8; k++)
+                        if (e0 + k < mis[r] || e0 + k >= end) h[r][j][k] = (half_t)-INFINITY;
+                }
             } else {
 #pragma unroll
                 for (int k = 0; k < 8; k++) h[r][j][k] = (half_t)-INFINITY;
@@ -221,7 +240,12 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_f16(const half_t* __res
         const half2_t lo = __builtin_bit_cast(half2_t, __builtin_amdgcn_readlane(__builtin_bit_cast(int, m2), 0));
         const half2_t hi = __builtin_bit_cast(half2_t, __builtin_amdgcn_readlane(__builtin_bit_cast(int, m2), 32));
         m2 = __builtin_elementwise_max(lo, hi);
-        const float m = fmaxf((float)m2[0], (float)m2[1]);
+        float m = fmaxf((float)m2[0], (float)m2[1]);
+        if (LANES == 256) {
+            if ((threadIdx.x & 63) == 0) red[0][threadIdx.x >> 6] = m;
+            __syncthreads();
+            m = fmaxf(fmaxf(red[0][0], red[0][1]), fmaxf(red[0][2], red[0][3]));
+        }
         const float nmb = -m * kLog2e;
 
         float e[NV][8];
@@ -234,19 +258,33 @@ __global__ __launch_bounds__(256) void softmax_rows_wave_f16(const half_t* __res
                 s += e[j][k];
             }
         s = wave_allreduce(s, SumOp{});
+        if (LANES == 256) {
+            if ((threadIdx.x & 63) == 0) red[1][threadIdx.x >> 6] = s;
+            __syncthreads();
+            s = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+        }
         const float inv = __builtin_amdgcn_rcpf(s);  // 1 ulp, far inside the tolerance of the fp16 result
         if (row0 + r < rows) {
+            half_t* dst = out + ooff[r] - mis[r];
+            const int end = len + mis[r];
 #pragma unroll
             for (int j = 0; j < NV; j++) {
-                const int e0 = (j * 64 + lane) * 8;
-                if (e0 < len) {
+                const int e0 = (j * LANES + lane) * 8;
+                if (e0 < end) {
                     u32x4 q;
+                    half_t* qh = reinterpret_cast<half_t*>(&q);
 #pragma unroll
                     for (int k = 0; k < 4; k++) {
                         const half2_t v = {(half_t)(e[j][2 * k] * inv), (half_t)(e[j][2 * k + 1] * inv)};
                         q[k] = __builtin_bit_cast(uint32_t, v);
                     }
-                    __builtin_nontemporal_store(q, reinterpret_cast<u32x4*>(out + ooff[r] + e0));
+                    if (!MISALIGNED || (e0 >= mis[r] && e0 + 8 <= end)) {
+                        __builtin_nontemporal_store(q, reinterpret_cast<u32x4*>(dst + e0));
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < 8; k++)
+                            if (e0 + k >= mis[r] && e0 + k < end) dst[e0 + k] = qh[k];
+                    }
                 }
             }
         }
@@ -351,6 +389,43 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
                 (long long)rows);
 
     const bool inner = ax == 0 && p.in_stride[0] == 1 && p.out_stride[0] == 1;
+    if (inner && std::is_same<T, half_t>::value && valid == len && len <= 256 * 8 * 16) {
+        // fp16 rows without padding: registers hold the row; rows need not be 16-byte aligned as long as
+        // input and output rows are misaligned alike
+        const half_t* hin = reinterpret_cast<const half_t*>(in);
+        half_t* hout = reinterpret_cast<half_t*>(out);
+        bool aligned = len % 8 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+        bool same_mis = ((reinterpret_cast<uintptr_t>(in) ^ reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+        for (int d = 0; d < map.nd; d++) {
+            if (map.dims[d] == 1) continue;
+            aligned = aligned && map.in_stride[d] % 8 == 0 && map.out_stride[d] % 8 == 0;
+            same_mis = same_mis && (map.in_stride[d] - map.out_stride[d]) % 8 == 0;
+        }
+        if (aligned || same_mis) {
+            const int l = (int)len;
+            const int span = aligned ? l : l + 7;  // aligned vectors a misaligned row can touch
+            const dim3 block(256);
+            const dim3 gw((unsigned)((rows + 3) / 4)), gb((unsigned)rows);
+#define VPX_SM(NV, ROWS, LANES, GRID)                                                                                 \
+    do {                                                                                                              \
+        if (aligned) hipLaunchKernelGGL((softmax_rows_f16<NV, ROWS, LANES, false>), GRID, block, 0, s, hin, hout, map, rows, l); \
+        else hipLaunchKernelGGL((softmax_rows_f16<NV, ROWS, LANES, true>), GRID, block, 0, s, hin, hout, map, rows, l);         \
+    } while (0)
+            // short rows, many of them: two rows per wave keep more bytes in flight (measured best)
+            if (span <= 512 && rows >= 16384) VPX_SM(1, 2, 64, dim3((unsigned)((rows + 7) / 8)));
+            else if (span <= 512) VPX_SM(1, 1, 64, gw);
+            else if (span <= 1024) VPX_SM(2, 1, 64, gw);
+            else if (span <= 2048) VPX_SM(4, 1, 64, gw);
+            else if (span <= 4096 && rows >= 1024) VPX_SM(8, 1, 64, gw);
+            else if (span <= 4096) VPX_SM(2, 1, 256, gb);
+            else if (span <= 8192) VPX_SM(4, 1, 256, gb);
+            else if (span <= 16384) VPX_SM(8, 1, 256, gb);
+            else VPX_SM(16, 1, 256, gb);
+#undef VPX_SM
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
+    }
     if (inner) {
         bool vec_ok = len % N == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
                       (reinterpret_cast<uintptr_t>(out) & 15) == 0 && len <= 64 * N * 8;
@@ -359,21 +434,8 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
         if (vec_ok) {
             const int l = (int)len, v = (int)valid;
             const int64_t per = 64 * N;
-            if (std::is_same<T, half_t>::value && valid == len) {
-                const half_t* hin = reinterpret_cast<const half_t*>(in);
-                half_t* hout = reinterpret_cast<half_t*>(out);
-                const dim3 block(256);
-                const dim3 grid((unsigned)((rows + 3) / 4));
-                // short rows, many of them: two rows per wave keep more bytes in flight (measured best)
-                if (len <= per && rows >= 16384)
-                    hipLaunchKernelGGL((softmax_rows_wave_f16<1, 2>), dim3((unsigned)((rows + 7) / 8)), block, 0, s, hin, hout, map, rows, l);
-                else if (len <= per) hipLaunchKernelGGL((softmax_rows_wave_f16<1, 1>), grid, block, 0, s, hin, hout, map, rows, l);
-                else if (len <= 2 * per) hipLaunchKernelGGL((softmax_rows_wave_f16<2, 1>), grid, block, 0, s, hin, hout, map, rows, l);
-                else if (len <= 4 * per) hipLaunchKernelGGL((softmax_rows_wave_f16<4, 1>), grid, block, 0, s, hin, hout, map, rows, l);
-                else hipLaunchKernelGGL((softmax_rows_wave_f16<8, 1>), grid, block, 0, s, hin, hout, map, rows, l);
-            }
             // general form (fp32, padded axis)
-            else if (len <= per) launch_rows_wave<T, 1, 1>(in, out, map, rows, l, v, s);
+            if (len <= per) launch_rows_wave<T, 1, 1>(in, out, map, rows, l, v, s);
             else if (len <= 2 * per) launch_rows_wave<T, 2, 1>(in, out, map, rows, l, v, s);
             else if (len <= 4 * per) launch_rows_wave<T, 4, 1>(in, out, map, rows, l, v, s);
             else launch_rows_wave<T, 8, 1>(in, out, map, rows, l, v, s);
