@@ -256,7 +256,11 @@ def _softmax(rt, dev, x_bits, axis, pad=0, packed=True, f32=False):
                                         # rows that are not 16-byte aligned, long rows (one workgroup per row), and beyond
                                         ((65, 500), 1), ((7, 511), 1), ((130, 197), 1), ((3, 1023), 1), ((9, 4099), 1),
                                         ((3, 32768), 1), ((5, 20000), 1), ((6, 8191), 1), ((2, 33000), 1), ((2, 40001), 1),
-                                        ((20000, 8), 1), ((17000, 509), 1)])
+                                        ((20000, 8), 1), ((17000, 509), 1),
+                                        # outer axis with contiguous inner dimensions: every slab shape (steps x columns x waves)
+                                        ((3, 12, 64), 1), ((2, 50, 8, 24), 1), ((2, 200, 520), 1), ((3, 21, 36), 1),
+                                        ((2, 100, 4, 5), 1), ((1, 400, 132), 1), ((2, 40, 6), 1), ((1, 200, 30), 1),
+                                        ((1, 1000, 66), 1), ((1, 1024, 2, 64), 1), ((1, 1100, 64), 1), ((2, 2, 512, 512), 2)])
 def test_softmax_shapes_and_axes(rt, orc, dev, shape, axis):
     rng = np.random.default_rng(hash((shape, axis)) % 2 ** 32)
     x = rng.normal(0, 3, shape).astype(np.float32)

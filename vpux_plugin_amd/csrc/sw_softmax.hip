@@ -2,7 +2,7 @@
 // fp32 arithmetic inside, driven by the packed {axis, pad, dims, strides} parameters the compiler
 // writes (src/vpux_compiler/src/dialect/VPUIP/transforms/passes/update_sw_kernel_params.cpp:36-147).
 //
-// Three device paths:
+// Device paths:
 //   rows_wave  : reduction axis is the innermost, contiguous one and a row fits the registers of one
 //                wavefront (up to 4096 fp16 / 2048 fp32 values): one 64-lane wave owns a row, 128-bit
 //                loads, max and sum by DPP/swizzle butterflies, single pass over HBM.  fp16 rows
@@ -10,8 +10,10 @@
 //                instructions (packed-half maximum, mixed-precision fma); it also serves rows of
 //                up to 32768 values (one workgroup per row) and rows that are not 16-byte aligned.
 //   rows_block : innermost axis of any length or alignment: one workgroup per row, three passes.
-//   lines      : reduction over an outer (strided) axis: one lane per line, lanes adjacent along the
-//                innermost dimension so every step of the axis is a coalesced access.
+//   slabs      : fp16 reduction over an outer axis of up to 1024 steps with contiguous inner
+//                dimensions: the whole [axis x 512 columns] slab of a workgroup sits in registers.
+//   lines      : any other reduction over an outer (strided) axis: one lane per line, lanes adjacent
+//                along the innermost dimension so every step of the axis is a coalesced access.
 #include <type_traits>
 
 #include "vpx_common.h"
@@ -352,6 +354,93 @@ __global__ __launch_bounds__(256) void softmax_lines(const T* __restrict__ in, T
         py[a * out_as] = (T)(a < valid ? fast_exp((float)px[a * in_as] - m) * inv : 0.f);
 }
 
+// ---------------------------------------------------------------- slabs (outer axis, fp16)
+// Reduction over an outer axis whose inner dimensions are contiguous: the tensor is
+// [outer][axis L][inner I].  A tile is every step of the axis x 64*VEC adjacent inner positions of
+// one outer index; lane l owns VEC adjacent columns, so each step of the axis is one contiguous
+// access of the wave.  KW waves share a tile, wave w taking steps w, w+KW, ...; all values of the
+// tile stay in registers (packed halves) between the single read and the single write, column
+// maxima and sums of the KW waves meet in LDS.  The exponential is evaluated twice (for the sum and
+// for the result) instead of keeping fp32 copies, which would not fit the registers.
+template <int VEC, int KW, int SMAX>
+__global__ __launch_bounds__(KW == 1 ? 256 : 64 * KW) void softmax_slab_f16(const half_t* __restrict__ in,
+                                                                           half_t* __restrict__ out, RowMap outer_map,
+                                                                           int64_t tiles, int tiles_per_outer, int L, int I,
+                                                                           int64_t in_as, int64_t out_as) {
+    typedef _Float16 hvec __attribute__((ext_vector_type(VEC)));
+    typedef float fvec __attribute__((ext_vector_type(VEC)));
+    __shared__ hvec smax[KW == 1 ? 1 : KW][64];
+    __shared__ fvec ssum[KW == 1 ? 1 : KW][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t tile = KW == 1 ? (int64_t)blockIdx.x * 4 + wave : blockIdx.x;
+    if (tile >= tiles) return;
+    const int kw = KW == 1 ? 0 : wave;  // which share of the axis this wave takes
+    const int64_t outer = tile / tiles_per_outer;
+    const int col = (int)(tile - outer * tiles_per_outer) * 64 * VEC + lane * VEC;
+    int64_t ioff, ooff;
+    row_offsets(outer_map, outer, ioff, ooff);
+    const bool live = col < I;
+    const half_t* src = in + ioff + col;
+    half_t* dst = out + ooff + col;
+
+    hvec h[SMAX];
+    hvec m;
+#pragma unroll
+    for (int k = 0; k < VEC; k++) m[k] = (half_t)-INFINITY;
+#pragma unroll
+    for (int i = 0; i < SMAX; i++) {
+        const int a = kw + KW * i;
+        h[i] = m;  // -inf
+        if (live && a < L) h[i] = *reinterpret_cast<const hvec*>(src + a * in_as);
+    }
+#pragma unroll
+    for (int i = 0; i < SMAX; i++) m = __builtin_elementwise_max(m, h[i]);
+    if (KW > 1) {
+        smax[kw][lane] = m;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < KW; w++) m = __builtin_elementwise_max(m, smax[w][lane]);
+    }
+    fvec nmb, sum;
+#pragma unroll
+    for (int k = 0; k < VEC; k++) {
+        nmb[k] = -(float)m[k] * kLog2e;
+        sum[k] = 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < SMAX; i++)
+#pragma unroll
+        for (int k = 0; k < VEC; k++) sum[k] += __builtin_amdgcn_exp2f(__builtin_fmaf((float)h[i][k], kLog2e, nmb[k]));
+    if (KW > 1) {
+        ssum[kw][lane] = sum;
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < VEC; k++) sum[k] = 0.f;
+#pragma unroll
+        for (int w = 0; w < KW; w++) sum += ssum[w][lane];  // same order in every wave
+    }
+    fvec inv;
+#pragma unroll
+    for (int k = 0; k < VEC; k++) {
+        inv[k] = __builtin_amdgcn_rcpf(sum[k]);
+        // hide the value's origin: otherwise the exponents of the summation pass are kept for reuse, one
+        // fp32 register per value, which is exactly what does not fit
+        asm volatile("" : "+v"(nmb[k]));
+    }
+#pragma unroll
+    for (int i = 0; i < SMAX; i++) {
+        const int a = kw + KW * i;
+        if (live && a < L) {
+            hvec r;
+#pragma unroll
+            for (int k = 0; k < VEC; k++)
+                r[k] = (half_t)(__builtin_amdgcn_exp2f(__builtin_fmaf((float)h[i][k], kLog2e, nmb[k])) * inv[k]);
+            __builtin_nontemporal_store(r, reinterpret_cast<hvec*>(dst + a * out_as));
+        }
+    }
+}
+
 template <typename T, int NV, int ROWS>
 void launch_rows_wave(const T* in, T* out, const RowMap& map, int64_t rows, int len, int valid, hipStream_t s) {
     const int64_t waves = (rows + ROWS - 1) / ROWS;
@@ -448,6 +537,62 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
                            p.in_stride[0], p.out_stride[0]);
         VPX_HIP_CHECK(hipGetLastError());
         return VPX_RESULT_SUCCESS;
+    }
+    // fp16, outer axis, contiguous inner dimension: register-resident slabs
+    if (std::is_same<T, half_t>::value && valid == len && len <= 1024 && p.in_stride[0] == 1 && p.out_stride[0] == 1) {
+        // inner = the dimensions below the axis, which must form one contiguous run in both operands
+        int64_t inner = 1;
+        bool ok = true;
+        for (int d = 0; d < ax && ok; d++) {
+            ok = p.dims[d] == 1 || (p.in_stride[d] == inner && p.out_stride[d] == inner);
+            inner *= p.dims[d];
+        }
+        RowMap om{};
+        int64_t outer = 1;
+        for (int d = ax + 1; d < p.nd; d++) {
+            outer *= p.dims[d];
+            if (p.dims[d] == 1) continue;
+            om.dims[om.nd] = p.dims[d];
+            om.in_stride[om.nd] = p.in_stride[d];
+            om.out_stride[om.nd] = p.out_stride[d];
+            om.nd++;
+        }
+        const int64_t in_as = p.in_stride[ax], out_as = p.out_stride[ax];
+        auto aligned_to = [&](int vec) {
+            bool a = inner % vec == 0 && in_as % vec == 0 && out_as % vec == 0 &&
+                     (reinterpret_cast<uintptr_t>(in) % (2 * vec)) == 0 && (reinterpret_cast<uintptr_t>(out) % (2 * vec)) == 0;
+            for (int d = 0; d < om.nd; d++) a = a && om.in_stride[d] % vec == 0 && om.out_stride[d] % vec == 0;
+            return a;
+        };
+        // 128 halves per lane (64 registers): 16, 32 or 64 steps of 8, 4 or 2 columns, times 1, 4 or 16 waves
+        int vec = 0;
+        if (len <= 256 && aligned_to(8)) vec = 8;
+        else if (len <= 512 && aligned_to(4)) vec = 4;
+        else if (aligned_to(2)) vec = 2;
+        if (ok && vec != 0 && inner < (1ll << 31)) {
+            const half_t* hin = reinterpret_cast<const half_t*>(in);
+            half_t* hout = reinterpret_cast<half_t*>(out);
+            const int tpo = (int)((inner + 64 * vec - 1) / (64 * vec));
+            const int64_t tiles = outer * tpo;
+            VPX_REQUIRE(tiles < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "softmax: %lld tiles exceed the launch limit",
+                        (long long)tiles);
+            const int L = (int)len, I = (int)inner;
+#define VPX_SLAB(VEC, KW, SMAX, GRID, BLOCK)                                                                          \
+    hipLaunchKernelGGL((softmax_slab_f16<VEC, KW, SMAX>), dim3((unsigned)(GRID)), dim3(BLOCK), 0, s, hin, hout, om,     \
+                       tiles, tpo, L, I, in_as, out_as)
+            if (vec == 8 && L <= 16) VPX_SLAB(8, 1, 16, (tiles + 3) / 4, 256);
+            else if (vec == 8 && L <= 64) VPX_SLAB(8, 4, 16, tiles, 256);
+            else if (vec == 8) VPX_SLAB(8, 16, 16, tiles, 1024);
+            else if (vec == 4 && L <= 32) VPX_SLAB(4, 1, 32, (tiles + 3) / 4, 256);
+            else if (vec == 4 && L <= 128) VPX_SLAB(4, 4, 32, tiles, 256);
+            else if (vec == 4) VPX_SLAB(4, 16, 32, tiles, 1024);
+            else if (L <= 64) VPX_SLAB(2, 1, 64, (tiles + 3) / 4, 256);
+            else if (L <= 256) VPX_SLAB(2, 4, 64, tiles, 256);
+            else VPX_SLAB(2, 16, 64, tiles, 1024);
+#undef VPX_SLAB
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
     }
     const unsigned blocks = (unsigned)((rows + 255) / 256);
     hipLaunchKernelGGL(softmax_lines<T>, dim3(blocks), dim3(256), 0, s, in, out, map, rows, len, valid, p.in_stride[ax],
