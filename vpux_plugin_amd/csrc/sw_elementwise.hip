@@ -74,6 +74,28 @@ __device__ __forceinline__ float fq_f32(float x, float ilo, float ihi, float olo
     return x <= ilo ? olo : (x > ihi ? ohi : q);
 }
 
+// a / c, correctly rounded, from r = RN(1 / c): q = RN(a r) is within an ulp, the residual
+// a - q c is exact in one fma, and the corrected q + residual * r rounds to the true quotient
+// (Markstein).  Three operations instead of the dozen of an IEEE division; valid away from
+// overflow and underflow, where the operands of a FakeQuantize live.
+__device__ __forceinline__ float div_const(float a, float c, float r) {
+    const float q = a * r;
+    const float rem = __builtin_fmaf(-q, c, a);
+    return __builtin_fmaf(rem, r, q);
+}
+
+// Per-tensor FakeQuantize prepared on the host: ranges and their correctly rounded reciprocals.
+struct FqConst {
+    float ilo, ihi, olo, ohi, lm1;
+    float irange, r_irange;  // ihi - ilo and RN(1 / (ihi - ilo))
+    float r_lm1;             // RN(1 / lm1)
+    float orange;            // ohi - olo
+};
+__device__ __forceinline__ float fq_f32_const(float x, const FqConst& c) {
+    const float q = div_const(roundf(div_const(x - c.ilo, c.irange, c.r_irange) * c.lm1), c.lm1, c.r_lm1) * c.orange + c.olo;
+    return x <= c.ilo ? c.olo : (x > c.ihi ? c.ohi : q);
+}
+
 template <typename T>
 __device__ __forceinline__ T narrow(float r);
 template <>
@@ -206,14 +228,87 @@ struct EltFn {
     }
 };
 
-struct FqFn {
+// Narrows N fp32 results to fp16 as vpux::type::float16 would.  The reference deviates from IEEE
+// only for nonzero magnitudes below 2^-15; a wave that holds no such value -- nearly always --
+// takes the plain conversion instruction, the others the exact emulation.
+template <int N>
+__device__ __forceinline__ void narrow_vec(const float (&r)[N], half_t (&h)[N]) {
+    bool zone = false;
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+        const uint32_t mag = __builtin_bit_cast(uint32_t, r[k]) & 0x7fffffffu;
+        zone = zone || (mag - 1u) < 0x37ffffffu || mag > 0x7f800000u;  // 0 < |r| < 2^-15, or NaN (payload rule)
+    }
+    if (__builtin_amdgcn_ballot_w64(zone) != 0) {
+#pragma unroll
+        for (int k = 0; k < N; k++) h[k] = f32_to_f16(r[k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < N; k++) h[k] = (half_t)r[k];
+    }
+}
+
+// Per-tensor FakeQuantize as a flat streaming map.  The four limits are device tensors of one
+// element; every lane turns them into the constants of fq_f32_const once (two IEEE divisions per
+// lane instead of two per value).
+struct FqMap {
+    static constexpr int VEC = 8;
+    const half_t* __restrict__ in;
+    half_t* __restrict__ out;
     const half_t* ilo;
     const half_t* ihi;
     const half_t* olo;
     const half_t* ohi;
     float lm1;
-    __device__ __forceinline__ half_t operator()(half_t x) const {
-        return f32_to_f16(fq_f32((float)x, (float)*ilo, (float)*ihi, (float)*olo, (float)*ohi, lm1));
+    __device__ __forceinline__ FqConst prep() const {
+        FqConst c;
+        c.ilo = (float)*ilo;
+        c.ihi = (float)*ihi;
+        c.olo = (float)*olo;
+        c.ohi = (float)*ohi;
+        c.lm1 = lm1;
+        c.irange = c.ihi - c.ilo;
+        c.r_irange = 1.0f / c.irange;
+        c.r_lm1 = 1.0f / lm1;
+        c.orange = c.ohi - c.olo;
+        return c;
+    }
+    template <int U>
+    __device__ __forceinline__ void vecs(int64_t v0, int64_t step) const {
+        const FqConst c = prep();
+        Pack<half_t, VEC> x[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) x[u].load(in, v0 + u * step);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float r[VEC];
+            half_t h[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) r[k] = fq_f32_const((float)x[u].get(k), c);
+            narrow_vec(r, h);
+            Pack<half_t, VEC> y;
+#pragma unroll
+            for (int k = 0; k < VEC; k++) y.set(k, h[k]);
+            y.store(out, v0 + u * step);
+        }
+    }
+    __device__ __forceinline__ void one(int64_t i) const {
+        out[i] = f32_to_f16(fq_f32_const((float)in[i], prep()));
+    }
+};
+
+// FakeQuantize with limits that vary between values (vnd_kernel functor): plain fq_f32 per value.
+struct FqVecFn {
+    float lm1;
+    __device__ __forceinline__ void operator()(const Pack<half_t, 8> (&x)[5], Pack<half_t, 8>& y) const {
+        float r[8];
+        half_t h[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            r[k] = fq_f32((float)x[0].get(k), (float)x[1].get(k), (float)x[2].get(k), (float)x[3].get(k), (float)x[4].get(k), lm1);
+        narrow_vec(r, h);
+#pragma unroll
+        for (int k = 0; k < 8; k++) y.set(k, h[k]);
     }
 };
 
@@ -284,6 +379,119 @@ __global__ __launch_bounds__(kBlock) void nd_fq_kernel(const half_t* in, half_t*
     nd_offsets<4>(lim, i, lo);
     out[off[1]] = f32_to_f16(fq_f32((float)in[off[0]], (float)ilo[lo[0]], (float)ihi[lo[1]], (float)olo[lo[2]],
                                     (float)ohi[lo[3]], lm1));
+}
+
+// ---------------------------------------------------------------- vectorised broadcast path
+// Same-type maps over operands that broadcast or are strided in the outer dimensions but are, along
+// the innermost (merged) dimension, either contiguous or constant.  Work is dealt out in vectors of
+// VEC elements of the innermost dimension; a lane finds its row by divisions with reciprocals
+// prepared on the host, loads a vector from each contiguous operand and one element from each
+// constant one.  NOPS operands, the last one is the output.
+struct VndIndex {
+    int nd;                          // row dimensions (all but the innermost)
+    uint32_t vec_per_row;            // vectors along the innermost dimension
+    uint64_t m_vec_per_row;          // ceil(2^64 / vec_per_row)
+    uint32_t dims[kMaxDims];         // row dimensions, innermost first
+    uint64_t m_dims[kMaxDims];
+    int64_t stride[6][kMaxDims];     // element strides of the row dimensions
+    int inner_stride[6];             // 1 or 0
+};
+
+__device__ __forceinline__ uint32_t fdiv64(uint32_t a, uint32_t d, uint64_t m) {
+    return d == 1 ? a : (uint32_t)__umul64hi((uint64_t)a, m);
+}
+
+template <typename T, int NOPS, class Fn>
+__global__ __launch_bounds__(kBlock) void vnd_kernel(const T* p0, const T* p1, const T* p2, const T* p3, const T* p4, T* pout,
+                                                     Fn fn, VndIndex ix, uint32_t total_vec) {
+    constexpr int VEC = 16 / sizeof(T);
+    const uint32_t v = blockIdx.x * kBlock + threadIdx.x;
+    if (v >= total_vec) return;
+    uint32_t row = fdiv64(v, ix.vec_per_row, ix.m_vec_per_row);
+    const uint32_t iv = v - row * ix.vec_per_row;
+    int64_t off[NOPS];
+#pragma unroll
+    for (int o = 0; o < NOPS; o++) off[o] = (int64_t)iv * VEC * ix.inner_stride[o];
+    for (int d = 0; d < ix.nd; d++) {
+        const uint32_t q = fdiv64(row, ix.dims[d], ix.m_dims[d]);
+        const uint32_t r = row - q * ix.dims[d];
+        row = q;
+#pragma unroll
+        for (int o = 0; o < NOPS; o++) off[o] += (int64_t)r * ix.stride[o][d];
+    }
+    const T* src[5] = {p0, p1, p2, p3, p4};
+    Pack<T, VEC> x[NOPS - 1];
+#pragma unroll
+    for (int o = 0; o < NOPS - 1; o++) {
+        if (ix.inner_stride[o]) {
+            x[o].load(src[o] + off[o], 0);
+        } else {
+            const T e = src[o][off[o]];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) x[o].set(k, e);
+        }
+    }
+    Pack<T, VEC> y;
+    fn(x, y);
+    y.store(pout + off[NOPS - 1], 0);
+}
+
+// Host side: merges dimensions that every operand walks contiguously or not at all, then checks
+// what vnd_kernel needs.  `ops` are NOPS memrefs broadcastable to the last one.  Returns false when
+// the shape does not qualify (the caller falls back to the one-element-per-lane kernels).
+template <typename T, int NOPS>
+bool make_vnd(const MemRef* const (&ops)[NOPS], VndIndex& ix, uint32_t& total_vec) {
+    constexpr int VEC = 16 / sizeof(T);
+    const MemRef& out = *ops[NOPS - 1];
+    if (out.nd > kMaxDims || out.nd < 1) return false;
+    int64_t dims[kMaxDims], st[NOPS][kMaxDims];
+    int nd = 0;
+    for (int d = 0; d < out.nd; d++) {
+        if (out.dims[d] == 1) continue;
+        int64_t cur[NOPS];
+        for (int o = 0; o < NOPS; o++) {
+            const MemRef& m = *ops[o];
+            const bool scalar = m.numel() == 1;
+            if (!scalar && m.nd != out.nd) return false;
+            cur[o] = scalar || m.dims[d] == 1 ? 0 : m.strides[d];
+            if (!scalar && m.dims[d] != 1 && m.dims[d] != out.dims[d]) return false;
+        }
+        bool merge = nd > 0;
+        for (int o = 0; o < NOPS && merge; o++) merge = cur[o] == st[o][nd - 1] * dims[nd - 1];
+        if (merge) {
+            dims[nd - 1] *= out.dims[d];
+        } else {
+            dims[nd] = out.dims[d];
+            for (int o = 0; o < NOPS; o++) st[o][nd] = cur[o];
+            nd++;
+        }
+    }
+    if (nd == 0) return false;  // a single element: not worth a vector path
+    if (dims[0] % VEC != 0 || dims[0] / VEC >= (1ll << 32)) return false;
+    ix = VndIndex{};
+    for (int o = 0; o < NOPS; o++) {
+        if (st[o][0] != 0 && st[o][0] != 1) return false;
+        if (o == NOPS - 1 && st[o][0] != 1) return false;
+        ix.inner_stride[o] = (int)st[o][0];
+        if ((reinterpret_cast<uintptr_t>(ops[o]->data) & 15) != 0 && st[o][0] == 1) return false;
+        for (int d = 1; d < nd; d++)
+            if (st[o][0] == 1 && st[o][d] % VEC != 0) return false;
+    }
+    auto magic = [](uint64_t d) { return d == 1 ? 0ull : (~0ull) / d + 1ull; };
+    ix.vec_per_row = (uint32_t)(dims[0] / VEC);
+    ix.m_vec_per_row = magic(ix.vec_per_row);
+    ix.nd = nd - 1;
+    int64_t total = dims[0] / VEC;
+    for (int d = 1; d < nd; d++) {
+        if (dims[d] >= (1ll << 32)) return false;
+        ix.dims[d - 1] = (uint32_t)dims[d];
+        ix.m_dims[d - 1] = magic((uint64_t)dims[d]);
+        for (int o = 0; o < NOPS; o++) ix.stride[o][d - 1] = st[o][d];
+        total *= dims[d];
+        if (total >= (1ll << 32)) return false;
+    }
+    total_vec = (uint32_t)total;
+    return total > 0;
 }
 
 int grid_1d(int64_t n, unsigned* blocks) {
@@ -373,6 +581,25 @@ static int eltwise_impl(const MemRef& a, const MemRef& b, const MemRef& out, hip
         BinaryMap<T, 16 / sizeof(T), Fn> f{(const T*)a.data, (const T*)b.data, (T*)out.data, Fn{}};
         return launch_stream(f, n, s);
     }
+    {
+        struct VecFn {
+            __device__ __forceinline__ void operator()(const Pack<T, 16 / sizeof(T)> (&x)[2], Pack<T, 16 / sizeof(T)>& y) const {
+                Fn f;
+#pragma unroll
+                for (int k = 0; k < (int)(16 / sizeof(T)); k++) y.set(k, f(x[0].get(k), x[1].get(k)));
+            }
+        };
+        const MemRef* const ops[3] = {&a, &b, &out};
+        VndIndex vx;
+        uint32_t total_vec = 0;
+        if (make_vnd<T, 3>(ops, vx, total_vec)) {
+            hipLaunchKernelGGL((vnd_kernel<T, 3, VecFn>), dim3((total_vec + kBlock - 1) / kBlock), dim3(kBlock), 0, s,
+                               (const T*)a.data, (const T*)b.data, (const T*)nullptr, (const T*)nullptr, (const T*)nullptr,
+                               (T*)out.data, VecFn{}, vx, total_vec);
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
+    }
     NdIndex ix{};
     int rc = fill_index(ix, 0, a, out, "eltwise input 1");
     if (rc) return rc;
@@ -430,10 +657,23 @@ int launch_fake_quantize(const MemRef& in, const MemRef lims[4], const MemRef& o
     const bool per_tensor =
             lims[0].numel() == 1 && lims[1].numel() == 1 && lims[2].numel() == 1 && lims[3].numel() == 1;
     if (per_tensor && in.compact && out.compact && aligned16(in.data) && aligned16(out.data)) {
-        FqFn fn{(const half_t*)lims[0].data, (const half_t*)lims[1].data, (const half_t*)lims[2].data,
-                (const half_t*)lims[3].data, lm1};
-        UnaryMap<half_t, half_t, 8, FqFn> f{(const half_t*)in.data, (half_t*)out.data, fn};
+        FqMap f{(const half_t*)in.data, (half_t*)out.data, (const half_t*)lims[0].data, (const half_t*)lims[1].data,
+                (const half_t*)lims[2].data, (const half_t*)lims[3].data, lm1};
         return launch_stream(f, n, s);
+    }
+    {
+        // limits that broadcast (per channel and the like): five inputs, vectors along the innermost run
+        const MemRef* const ops[6] = {&in, &lims[0], &lims[1], &lims[2], &lims[3], &out};
+        VndIndex vx;
+        uint32_t total_vec = 0;
+        if (make_vnd<half_t, 6>(ops, vx, total_vec)) {
+            hipLaunchKernelGGL((vnd_kernel<half_t, 6, FqVecFn>), dim3((total_vec + kBlock - 1) / kBlock), dim3(kBlock), 0, s,
+                               (const half_t*)in.data, (const half_t*)lims[0].data, (const half_t*)lims[1].data,
+                               (const half_t*)lims[2].data, (const half_t*)lims[3].data, (half_t*)out.data, FqVecFn{lm1}, vx,
+                               total_vec);
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
     }
     NdIndex io{}, lim{};
     int rc = fill_index(io, 0, in, out, "fake_quantize input");
