@@ -3,6 +3,8 @@
 // All of them are HBM-bound maps.  The fast path views compact operands as flat arrays and moves
 // 128 bits per lane per access, several independent accesses in flight per lane; a strided /
 // broadcasting path covers sub-views and NUMPY broadcast one element per lane.
+#include <type_traits>
+
 #include "vpx_common.h"
 
 namespace vpx {
@@ -107,6 +109,33 @@ __device__ __forceinline__ float narrow<float>(float r) {
     return r;
 }
 
+// Narrows N fp32 results to fp16 as vpux::type::float16 would.  The reference deviates from IEEE
+// only for nonzero magnitudes below 2^-15; a wave that holds no such value -- nearly always --
+// takes the plain conversion instruction, the others the exact emulation.
+template <int N>
+__device__ __forceinline__ void narrow_vec(const float (&r)[N], half_t (&h)[N]) {
+    bool zone = false;
+#pragma unroll
+    for (int k = 0; k < N; k++) {
+        const uint32_t mag = __builtin_bit_cast(uint32_t, r[k]) & 0x7fffffffu;
+        zone = zone || (mag - 1u) < 0x37ffffffu || mag > 0x7f800000u;  // 0 < |r| < 2^-15, or NaN (payload rule)
+    }
+    if (__builtin_amdgcn_ballot_w64(zone) != 0) {
+#pragma unroll
+        for (int k = 0; k < N; k++) h[k] = f32_to_f16(r[k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < N; k++) h[k] = (half_t)r[k];
+    }
+}
+
+// A functor may expose `f32(...)`, the fp32 value that still has to be narrowed to fp16; the maps
+// then narrow a whole vector at once (narrow_vec) instead of value by value.
+template <class Fn, class = void>
+struct HasF32 : std::false_type {};
+template <class Fn>
+struct HasF32<Fn, std::void_t<decltype(Fn::kF32)>> : std::true_type {};
+
 // ---------------------------------------------------------------- flat streaming skeleton
 // F provides: static constexpr int VEC; void vec(int64_t v) (elements [v*VEC, v*VEC+VEC)); void one(int64_t i).
 template <class F, int BLOCK, int UNROLL>
@@ -162,8 +191,18 @@ struct UnaryMap {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             Pack<TO, VEC> y;
+            if constexpr (HasF32<Fn>::value && std::is_same<TO, half_t>::value) {
+                float r[VEC];
+                half_t h[VEC];
 #pragma unroll
-            for (int k = 0; k < VEC; k++) y.set(k, fn(x[u].get(k)));
+                for (int k = 0; k < VEC; k++) r[k] = fn.f32(x[u].get(k));
+                narrow_vec(r, h);
+#pragma unroll
+                for (int k = 0; k < VEC; k++) y.set(k, h[k]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; k++) y.set(k, fn(x[u].get(k)));
+            }
             y.store(out, v0 + u * step);
         }
     }
@@ -190,8 +229,18 @@ struct BinaryMap {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             Pack<T, VEC> r;
+            if constexpr (HasF32<Fn>::value && std::is_same<T, half_t>::value) {
+                float f[VEC];
+                half_t h[VEC];
 #pragma unroll
-            for (int k = 0; k < VEC; k++) r.set(k, fn(x[u].get(k), y[u].get(k)));
+                for (int k = 0; k < VEC; k++) f[k] = fn.f32(x[u].get(k), y[u].get(k));
+                narrow_vec(f, h);
+#pragma unroll
+                for (int k = 0; k < VEC; k++) r.set(k, h[k]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; k++) r.set(k, fn(x[u].get(k), y[u].get(k)));
+            }
             r.store(out, v0 + u * step);
         }
     }
@@ -205,6 +254,8 @@ struct CvtF16F32 {
     __device__ __forceinline__ float operator()(half_t h) const { return (float)h; }
 };
 struct CvtF32F16 {
+    static constexpr bool kF32 = true;
+    __device__ __forceinline__ float f32(float f) const { return f; }
     __device__ __forceinline__ half_t operator()(float f) const { return f32_to_f16(f); }
 };
 template <typename T>
@@ -215,38 +266,18 @@ struct Copy {
 // float16 arithmetic = fp32 operation, then one rounding (include/vpux/utils/core/type/float16.hpp:123-150)
 template <typename T, int OP>
 struct EltFn {
-    __device__ __forceinline__ T operator()(T x, T y) const {
+    static constexpr bool kF32 = true;
+    __device__ __forceinline__ float f32(T x, T y) const {
         const float a = (float)x, b = (float)y;
-        float r;
-        if (OP == ELT_ADD) r = a + b;
-        else if (OP == ELT_SUB) r = a - b;
-        else if (OP == ELT_MUL) r = a * b;
-        else if (OP == ELT_MIN) r = fminf(a, b);
-        else if (OP == ELT_MAX) r = fmaxf(a, b);
-        else r = a / b;
-        return narrow<T>(r);
+        if (OP == ELT_ADD) return a + b;
+        if (OP == ELT_SUB) return a - b;
+        if (OP == ELT_MUL) return a * b;
+        if (OP == ELT_MIN) return fminf(a, b);
+        if (OP == ELT_MAX) return fmaxf(a, b);
+        return a / b;
     }
+    __device__ __forceinline__ T operator()(T x, T y) const { return narrow<T>(f32(x, y)); }
 };
-
-// Narrows N fp32 results to fp16 as vpux::type::float16 would.  The reference deviates from IEEE
-// only for nonzero magnitudes below 2^-15; a wave that holds no such value -- nearly always --
-// takes the plain conversion instruction, the others the exact emulation.
-template <int N>
-__device__ __forceinline__ void narrow_vec(const float (&r)[N], half_t (&h)[N]) {
-    bool zone = false;
-#pragma unroll
-    for (int k = 0; k < N; k++) {
-        const uint32_t mag = __builtin_bit_cast(uint32_t, r[k]) & 0x7fffffffu;
-        zone = zone || (mag - 1u) < 0x37ffffffu || mag > 0x7f800000u;  // 0 < |r| < 2^-15, or NaN (payload rule)
-    }
-    if (__builtin_amdgcn_ballot_w64(zone) != 0) {
-#pragma unroll
-        for (int k = 0; k < N; k++) h[k] = f32_to_f16(r[k]);
-    } else {
-#pragma unroll
-        for (int k = 0; k < N; k++) h[k] = (half_t)r[k];
-    }
-}
 
 // Per-tensor FakeQuantize as a flat streaming map.  The four limits are device tensors of one
 // element; every lane turns them into the constants of fq_f32_const once (two IEEE divisions per
@@ -585,8 +616,19 @@ static int eltwise_impl(const MemRef& a, const MemRef& b, const MemRef& out, hip
         struct VecFn {
             __device__ __forceinline__ void operator()(const Pack<T, 16 / sizeof(T)> (&x)[2], Pack<T, 16 / sizeof(T)>& y) const {
                 Fn f;
+                constexpr int V = (int)(16 / sizeof(T));
+                if constexpr (std::is_same<T, half_t>::value) {
+                    float r[V];
+                    half_t h[V];
 #pragma unroll
-                for (int k = 0; k < (int)(16 / sizeof(T)); k++) y.set(k, f(x[0].get(k), x[1].get(k)));
+                    for (int k = 0; k < V; k++) r[k] = f.f32(x[0].get(k), x[1].get(k));
+                    narrow_vec(r, h);
+#pragma unroll
+                    for (int k = 0; k < V; k++) y.set(k, h[k]);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < V; k++) y.set(k, f(x[0].get(k), x[1].get(k)));
+                }
             }
         };
         const MemRef* const ops[3] = {&a, &b, &out};
