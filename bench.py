@@ -337,8 +337,23 @@ def cpu_baseline(w, budget_s=12.0):
         val, unit = work / dt / 1e12, "TOP/s"
     what = {"c1_fake_quantize": "full tensor", "c2_softmax": "%d of 65536 rows" % units, "c3_mvn": "%d of 4 batch elements" % units,
             "c4_conv": "%d of 100352 output positions" % units, "c5_matmul": "%d of 4096 rows of A" % units}[w.name]
+    # a sample sized for about four seconds on one thread
+    units1 = max(1, int(units * min(1.0, 4.0 / max(dt * cores, 1e-6))))
+    fn1, work1 = w.cpu_sample(oracle, units1)
+    oracle.set_num_threads(1)
+    try:
+        t0 = time.perf_counter()
+        n1 = 0
+        while n1 < reps and (n1 == 0 or time.perf_counter() - t0 < 4.0):
+            fn1()
+            n1 += 1
+        dt1 = (time.perf_counter() - t0) / n1
+    finally:
+        oracle.set_num_threads(cores)
+    val1 = work1 / dt1 / (1e9 if w.bound == "hbm" else 1e12)
     return {"value": round(val, 4), "unit": unit, "cores": cores, "kind": "port",
-            "sample": "%s, %d repetition(s), %.3f s per repetition, %.1f s in total" % (what, reps, dt, reps * dt)}
+            "sample": "%s, %d repetition(s), %.3f s per repetition, %.1f s in total" % (what, reps, dt, reps * dt),
+            "value_one_thread": round(val1, 4)}
 
 
 def main():
