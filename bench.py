@@ -365,6 +365,9 @@ def main():
     ap.add_argument("--all", action="store_true", help="also measure every other configuration (short runs)")
     ap.add_argument("--graph", action="store_true", help="replay the timed steps from one HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--rotate", type=int, default=1, metavar="N",
+                    help="cycle through N separate buffer sets so that a step does not find its operands in the 256 MB "
+                         "Infinity Cache left there by the previous one (default 1: same buffers every step)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on one GPU only (every kernel shards without exchange; see DESIGN.md); "
@@ -377,13 +380,22 @@ def main():
     torch.cuda.set_device(0)
 
     w = MAKERS[args.workload](rt)
-    wall_ms, dev_ms = time_steps(w.step, args.steps, args.warmup, graph=args.graph)
+    step = w.step
+    if args.rotate > 1:
+        sets = [w] + [MAKERS[args.workload](rt) for _ in range(args.rotate - 1)]
+        counter = [0]
+
+        def step():
+            sets[counter[0] % len(sets)].step()
+            counter[0] += 1
+    wall_ms, dev_ms = time_steps(step, args.steps, args.warmup, graph=args.graph)
     value, unit = value_of(w, wall_ms)
     line = {
         "metric": METRIC, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": w.dtype, "data": "synthetic",
-        "config": {"workload": w.name, "description": w.desc, "launch": "hip graph" if args.graph else "eager"},
+        "config": {"workload": w.name, "description": w.desc, "launch": "hip graph" if args.graph else "eager",
+                   "buffer_sets": args.rotate},
         "device_ms_per_step": round(dev_ms, 6),
         "roofline": roofline(w, dev_ms),
     }
