@@ -232,12 +232,39 @@ def test_quantize_dequantize(rt, orc, dev, signed, scale, zp):
     assert np.array_equal(q32.cpu().numpy(), orc.quantize(x32, f32scale, zp, signed))
 
 
-def test_quantize_per_axis_is_refused(rt, dev):
+@pytest.mark.parametrize("shape,axis,order", [((2, 6, 5, 7), 1, "NCHW"), ((3, 300, 4, 4), 1, "NCHW"), ((2, 5, 7, 6), 3, "NHWC"),
+                                              ((8, 8, 3, 3), 1, "NCHW"), ((16, 64), 1, None), ((700, 3), 0, None)])
+def test_quantize_dequantize_per_axis(rt, orc, dev, shape, axis, order):
+    """One scale / zero point per slice of `axis`.  The blob does not name the axis: it is the dimension
+    whose size equals the parameter count, and the channel dimension when several have it ((8, 8, 3, 3))."""
     import torch
-    x = torch.zeros((2, 4), dtype=torch.float16, device=dev)
+    rng = np.random.default_rng(28 + len(shape) + axis)
+    n = shape[axis]
+    scales = rng.uniform(0.004, 0.08, n)
+    zps = rng.integers(-20, 21, n)
+    shipped = orc.f16_to_f32(orc.f32_to_f16(scales.astype(np.float32))).astype(np.float64)
+    x = orc.f32_to_f16(rng.normal(0, 3, shape).astype(np.float32))
+    q = torch.empty(shape, dtype=torch.int8, device=dev)
+    rt.quantize(to_dev(x, dev, True), q, scales, zps, order=order)
+    want = orc.quantize(x, shipped, zps, True, axis=axis)
+    assert np.array_equal(q.cpu().numpy(), want)
+    y = torch.empty(shape, dtype=torch.float16, device=dev)
+    rt.dequantize(q, y, scales, zps, order=order)
+    assert_f16_exact(f16_bits(y).reshape(-1), orc.dequantize(want, shipped, zps, axis=axis).reshape(-1), "per-axis dequantize")
+    y32 = torch.empty(shape, dtype=torch.float32, device=dev)
+    rt.dequantize(q, y32, scales, zps, order=order)
+    f32scales = scales.astype(np.float32).astype(np.float64)
+    assert np.array_equal(y32.cpu().numpy(), orc.dequantize(want, f32scales, zps, to_f16=False, axis=axis))
+
+
+def test_quantize_per_axis_ambiguous_axis_is_refused(rt, dev):
+    import torch
+    x = torch.zeros((4, 2, 4), dtype=torch.float16, device=dev)  # two dimensions of size 4, neither is the channel
     with pytest.raises(rt.VpxError) as e:
-        rt.quantize(x, torch.empty((2, 4), dtype=torch.int8, device=dev), [0.1, 0.2], [0, 1])
-    assert e.value.code == rt.ERROR_UNSUPPORTED_FEATURE
+        rt.quantize(x, torch.empty((4, 2, 4), dtype=torch.int8, device=dev), [0.1] * 4, [0] * 4)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    with pytest.raises(rt.VpxError):
+        rt.quantize(x, torch.empty((4, 2, 4), dtype=torch.int8, device=dev), [0.1] * 3, [0] * 3)  # no dimension of size 3
 
 
 # ---------------------------------------------------------------------------------- softmax

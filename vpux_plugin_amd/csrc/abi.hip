@@ -177,29 +177,33 @@ float half_bits_to_float(uint16_t h) {
 
 // quantize / dequantize attributes: int64 n, then n scales and n zero points, both as packed
 // floating-point values of the non-quantized operand's type (sw_kernel.cpp:97-163).
-int read_quant_params(const char* entry, const Args& a, uint32_t float_type, double* scale, int64_t* zp) {
+int read_quant_params(const char* entry, const Args& a, uint32_t float_type, std::vector<double>& scales,
+                      std::vector<int64_t>& zps) {
     int64_t n = 0;
     VPX_REQUIRE(read_attr(a, 0, &n), VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: params blob has no quantization parameters", entry);
-    VPX_REQUIRE(n >= 1, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: quantization parameter count is %lld", entry, (long long)n);
-    VPX_REQUIRE(n == 1, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: per-axis quantization (%lld scales) is not implemented", entry,
+    VPX_REQUIRE(n >= 1 && n <= (1 << 24), VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: quantization parameter count is %lld", entry,
                 (long long)n);
     const int per_word = float_type == VPX_NN_FP16 ? 4 : 2;
     const size_t words = (size_t)((n + per_word - 1) / per_word);
-    uint64_t sw = 0, zw = 0;
-    VPX_REQUIRE(read_attr(a, 8, &sw) && read_attr(a, 8 + words * 8, &zw), VPX_RESULT_ERROR_INVALID_ARGUMENT,
-                "%s: params blob is too short for %lld scales and zero points", entry, (long long)n);
-    float zf;
-    if (float_type == VPX_NN_FP16) {
-        *scale = (double)half_bits_to_float((uint16_t)(sw & 0xffffu));
-        zf = half_bits_to_float((uint16_t)(zw & 0xffffu));
-    } else {
-        const uint32_t sb = (uint32_t)sw, zb = (uint32_t)zw;
-        float sf;
-        memcpy(&sf, &sb, 4);
-        memcpy(&zf, &zb, 4);
-        *scale = (double)sf;
+    scales.resize((size_t)n);
+    zps.resize((size_t)n);
+    for (int64_t i = 0; i < n; i++) {
+        uint64_t sw = 0, zw = 0;
+        const size_t word = (size_t)(i / per_word), slot = (size_t)(i % per_word);
+        VPX_REQUIRE(read_attr(a, 8 + word * 8, &sw) && read_attr(a, 8 + (words + word) * 8, &zw), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: params blob is too short for %lld scales and zero points", entry, (long long)n);
+        float sf, zf;
+        if (float_type == VPX_NN_FP16) {
+            sf = half_bits_to_float((uint16_t)((sw >> (16 * slot)) & 0xffffu));
+            zf = half_bits_to_float((uint16_t)((zw >> (16 * slot)) & 0xffffu));
+        } else {
+            const uint32_t sb = (uint32_t)(sw >> (32 * slot)), zb = (uint32_t)(zw >> (32 * slot));
+            memcpy(&sf, &sb, 4);
+            memcpy(&zf, &zb, 4);
+        }
+        scales[(size_t)i] = (double)sf;
+        zps[(size_t)i] = (int64_t)std::llround(zf);
     }
-    *zp = (int64_t)std::llround(zf);
     return VPX_RESULT_SUCCESS;
 }
 
@@ -374,18 +378,20 @@ int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_si
         return launch_fake_quantize(a.mem[0], &a.mem[1], a.mem[5], levels, s);
     }
     case K_QUANT: {
-        double scale;
-        int64_t zp;
-        rc = read_quant_params(entry, a, a.mem[0].dtype, &scale, &zp);
+        std::vector<double> scales;
+        std::vector<int64_t> zps;
+        rc = read_quant_params(entry, a, a.mem[0].dtype, scales, zps);
         if (rc) return rc;
-        return launch_quantize(a.mem[0], a.mem[1], scale, zp, s);
+        if (scales.size() == 1) return launch_quantize(a.mem[0], a.mem[1], scales[0], zps[0], s);
+        return launch_quantize_per_axis(a.mem[0], a.mem[1], scales.data(), zps.data(), (int64_t)scales.size(), s);
     }
     case K_DEQUANT: {
-        double scale;
-        int64_t zp;
-        rc = read_quant_params(entry, a, a.mem[1].dtype, &scale, &zp);
+        std::vector<double> scales;
+        std::vector<int64_t> zps;
+        rc = read_quant_params(entry, a, a.mem[1].dtype, scales, zps);
         if (rc) return rc;
-        return launch_dequantize(a.mem[0], a.mem[1], scale, zp, s);
+        if (scales.size() == 1) return launch_dequantize(a.mem[0], a.mem[1], scales[0], zps[0], s);
+        return launch_dequantize_per_axis(a.mem[0], a.mem[1], scales.data(), zps.data(), (int64_t)scales.size(), s);
     }
     case K_MVN: {
         int64_t across = 0, normvar = 0;

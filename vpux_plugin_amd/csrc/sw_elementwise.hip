@@ -4,6 +4,7 @@
 // 128 bits per lane per access, several independent accesses in flight per lane; a strided /
 // broadcasting path covers sub-views and NUMPY broadcast one element per lane.
 #include <type_traits>
+#include <vector>
 
 #include "vpx_common.h"
 
@@ -776,6 +777,167 @@ int launch_dequantize(const MemRef& in, const MemRef& out, double scale, int64_t
         return convert_impl<uint8_t, float>(in, out, DequantFn<uint8_t, float, true>{scale, z}, s);
     if (in.dtype == VPX_NN_I8 && out.dtype == VPX_NN_FP32)
         return convert_impl<int8_t, float>(in, out, DequantFn<int8_t, float, true>{scale, z}, s);
+    return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "dequantize: %s -> %s is not implemented", dtype_name(in.dtype),
+                dtype_name(out.dtype));
+}
+
+// ---------------------------------------------------------------- per-axis quantize / dequantize
+// The params blob ships n scales and zero points but not the axis they run along
+// (getQuantParamsAttr, sw_kernel.cpp:130-163), so it is taken to be the one dimension of size n;
+// when several dimensions have that size, the channel dimension (logical dimension 1 of the
+// memref's order) if it is among them.  Operands must be compact.
+namespace {
+
+struct AxisChunk {
+    float a[256];
+    float b[256];
+};
+
+// Kernel arguments are the one path from host to device memory that a caller's graph capture can
+// record: the per-channel table goes to the workspace 256 entries per launch.
+__global__ __launch_bounds__(256) void fill_axis_table(float2* table, AxisChunk c, int count) {
+    if ((int)threadIdx.x < count) table[threadIdx.x] = float2{c.a[threadIdx.x], c.b[threadIdx.x]};
+}
+
+struct AxisGeom {
+    uint32_t inner, count;
+    uint64_t m_inner, m_count;
+};
+__device__ __forceinline__ uint32_t axis_channel(uint32_t i, const AxisGeom& g) {
+    const uint32_t q = fdiv64(i, g.inner, g.m_inner);
+    return q - fdiv64(q, g.count, g.m_count) * g.count;
+}
+
+// table entry: {in_min, in_max} of the channel's quantizer (quantize.cpp:91-96)
+template <typename TI, typename TQ>
+__global__ __launch_bounds__(kBlock) void quantize_axis_kernel(const TI* __restrict__ in, TQ* __restrict__ out,
+                                                               const float2* __restrict__ table, AxisGeom g, uint32_t n,
+                                                               float qmin, float qmax, float lm1) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const float2 p = table[axis_channel(i, g)];
+    out[i] = (TQ)(int)fq_f32((float)in[i], p.x, p.y, qmin, qmax, lm1);
+}
+
+// table entry: {scale, zero point as a float (an integer of at most 9 bits)}
+template <typename TQ, typename TO>
+__global__ __launch_bounds__(kBlock) void dequantize_axis_kernel(const TQ* __restrict__ in, TO* __restrict__ out,
+                                                                 const float2* __restrict__ table, AxisGeom g, uint32_t n) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    const float2 p = table[axis_channel(i, g)];
+    out[i] = narrow<TO>((float)((double)((int)in[i] - (int)p.y) * (double)p.x));
+}
+
+int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t n, const float* a, const float* b, hipStream_t s,
+               AxisGeom& g, float2** table) {
+    VPX_REQUIRE(ref.compact && other.compact, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: per-axis form needs compact operands", what);
+    VPX_REQUIRE(ref.numel() < (1ll << 32), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: tensor of %lld elements is too large", what,
+                (long long)ref.numel());
+    int axis = -1, hits = 0;
+    for (int d = 0; d < ref.nd; d++)
+        if (ref.dims[d] == n) {
+            axis = d;
+            hits++;
+        }
+    VPX_REQUIRE(hits >= 1, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: no dimension has the size of the %lld quantization parameters", what,
+                (long long)n);
+    if (hits > 1) {
+        // memory position (innermost = 0) of logical dimension 1
+        int pc = -1;
+        for (int i = 0; i < ref.nd; i++)
+            if ((int)((ref.order >> (4 * i)) & 0xf) == 2) pc = ref.nd - 1 - i;
+        VPX_REQUIRE(pc >= 0 && ref.dims[pc] == n, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: %d dimensions have size %lld and the channel dimension is not one of them: the axis is ambiguous", what, hits,
+                    (long long)n);
+        axis = pc;
+    }
+    int64_t inner = 1;
+    for (int d = 0; d < axis; d++) inner *= ref.dims[d];
+    auto magic = [](uint64_t d) { return d == 1 ? 0ull : (~0ull) / d + 1ull; };
+    g.inner = (uint32_t)inner;
+    g.count = (uint32_t)n;
+    g.m_inner = magic((uint64_t)inner);
+    g.m_count = magic((uint64_t)n);
+    void* ws = nullptr;
+    int rc = get_workspace(s, sizeof(float2) * (size_t)n, &ws);
+    if (rc) return rc;
+    *table = (float2*)ws;
+    for (int64_t c0 = 0; c0 < n; c0 += 256) {
+        AxisChunk ch;
+        const int cnt = (int)(n - c0 < 256 ? n - c0 : 256);
+        for (int k = 0; k < cnt; k++) {
+            ch.a[k] = a[c0 + k];
+            ch.b[k] = b[c0 + k];
+        }
+        for (int k = cnt; k < 256; k++) ch.a[k] = ch.b[k] = 0.f;
+        hipLaunchKernelGGL(fill_axis_table, dim3(1), dim3(256), 0, s, *table + c0, ch, cnt);
+        VPX_HIP_CHECK(hipGetLastError());
+    }
+    return VPX_RESULT_SUCCESS;
+}
+
+template <typename TI, typename TQ>
+int quantize_axis_impl(const MemRef& in, const MemRef& out, const double* scales, const int64_t* zps, int64_t n, int64_t qmin,
+                       int64_t qmax, hipStream_t s) {
+    std::vector<float> lo((size_t)n), hi((size_t)n);
+    for (int64_t c = 0; c < n; c++) {
+        VPX_REQUIRE(scales[c] > 0.0, VPX_RESULT_ERROR_INVALID_ARGUMENT, "quantize: scale %lld must be positive, got %g", (long long)c,
+                    scales[c]);
+        lo[(size_t)c] = (float)((double)(qmin - zps[c]) * scales[c]);
+        hi[(size_t)c] = (float)((double)(qmax - zps[c]) * scales[c]);
+    }
+    AxisGeom g;
+    float2* table = nullptr;
+    int rc = axis_setup("quantize", in, out, n, lo.data(), hi.data(), s, g, &table);
+    if (rc) return rc;
+    const uint32_t total = (uint32_t)in.numel();
+    if (total == 0) return VPX_RESULT_SUCCESS;
+    hipLaunchKernelGGL((quantize_axis_kernel<TI, TQ>), dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (const TI*)in.data,
+                       (TQ*)out.data, table, g, total, (float)qmin, (float)qmax, (float)(qmax - qmin + 1) - 1.0f);
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
+template <typename TQ, typename TO>
+int dequantize_axis_impl(const MemRef& in, const MemRef& out, const double* scales, const int64_t* zps, int64_t n, hipStream_t s) {
+    std::vector<float> sc((size_t)n), zp((size_t)n);
+    for (int64_t c = 0; c < n; c++) {
+        sc[(size_t)c] = (float)scales[c];  // exact: the blob ships scales as fp16 or fp32
+        zp[(size_t)c] = (float)zps[c];
+    }
+    AxisGeom g;
+    float2* table = nullptr;
+    int rc = axis_setup("dequantize", out, in, n, sc.data(), zp.data(), s, g, &table);
+    if (rc) return rc;
+    const uint32_t total = (uint32_t)in.numel();
+    if (total == 0) return VPX_RESULT_SUCCESS;
+    hipLaunchKernelGGL((dequantize_axis_kernel<TQ, TO>), dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (const TQ*)in.data,
+                       (TO*)out.data, table, g, total);
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
+}  // namespace
+
+int launch_quantize_per_axis(const MemRef& in, const MemRef& out, const double* scales, const int64_t* zps, int64_t n,
+                             hipStream_t s) {
+    VPX_REQUIRE(same_shape(in, out), VPX_RESULT_ERROR_INVALID_ARGUMENT, "quantize: input and output shapes differ");
+    if (in.dtype == VPX_NN_FP16 && out.dtype == VPX_NN_U8) return quantize_axis_impl<half_t, uint8_t>(in, out, scales, zps, n, 0, 255, s);
+    if (in.dtype == VPX_NN_FP16 && out.dtype == VPX_NN_I8) return quantize_axis_impl<half_t, int8_t>(in, out, scales, zps, n, -128, 127, s);
+    if (in.dtype == VPX_NN_FP32 && out.dtype == VPX_NN_U8) return quantize_axis_impl<float, uint8_t>(in, out, scales, zps, n, 0, 255, s);
+    if (in.dtype == VPX_NN_FP32 && out.dtype == VPX_NN_I8) return quantize_axis_impl<float, int8_t>(in, out, scales, zps, n, -128, 127, s);
+    return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "quantize: %s -> %s is not implemented", dtype_name(in.dtype),
+                dtype_name(out.dtype));
+}
+
+int launch_dequantize_per_axis(const MemRef& in, const MemRef& out, const double* scales, const int64_t* zps, int64_t n,
+                               hipStream_t s) {
+    VPX_REQUIRE(same_shape(in, out), VPX_RESULT_ERROR_INVALID_ARGUMENT, "dequantize: input and output shapes differ");
+    if (in.dtype == VPX_NN_U8 && out.dtype == VPX_NN_FP16) return dequantize_axis_impl<uint8_t, half_t>(in, out, scales, zps, n, s);
+    if (in.dtype == VPX_NN_I8 && out.dtype == VPX_NN_FP16) return dequantize_axis_impl<int8_t, half_t>(in, out, scales, zps, n, s);
+    if (in.dtype == VPX_NN_U8 && out.dtype == VPX_NN_FP32) return dequantize_axis_impl<uint8_t, float>(in, out, scales, zps, n, s);
+    if (in.dtype == VPX_NN_I8 && out.dtype == VPX_NN_FP32) return dequantize_axis_impl<int8_t, float>(in, out, scales, zps, n, s);
     return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "dequantize: %s -> %s is not implemented", dtype_name(in.dtype),
                 dtype_name(out.dtype));
 }

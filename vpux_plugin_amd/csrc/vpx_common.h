@@ -87,6 +87,11 @@ int launch_eltwise(int op, const MemRef& a, const MemRef& b, const MemRef& out, 
 int launch_fake_quantize(const MemRef& in, const MemRef lims[4], const MemRef& out, int64_t levels, hipStream_t s);
 int launch_quantize(const MemRef& in, const MemRef& out, double scale, int64_t zp, hipStream_t s);
 int launch_dequantize(const MemRef& in, const MemRef& out, double scale, int64_t zp, hipStream_t s);
+// per-axis forms: n scales / zero points along the dimension of size n (see the definition for how it is chosen)
+int launch_quantize_per_axis(const MemRef& in, const MemRef& out, const double* scales, const int64_t* zps, int64_t n,
+                             hipStream_t s);
+int launch_dequantize_per_axis(const MemRef& in, const MemRef& out, const double* scales, const int64_t* zps, int64_t n,
+                               hipStream_t s);
 
 struct SoftmaxPlan {
     int axis;  // index into dims (innermost first)
