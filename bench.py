@@ -169,7 +169,7 @@ def make_c4(rt):
         return lambda: orc.nce_conv(c["input"], c["weights"], wt_h, p, zp_in=128, pads=(1, 1, 1, 1), rows=(0, rows)), \
             2 * rows * 64 * 9 * 64
     return Workload("c4_conv", "int8 Conv 3x3 s1 p1 NHWC [32,56,56,64] u8 zp128 x [64,3,3,64] i8, PPE ReLU clamp [0,255]",
-                    step, nbytes, ops, "mfma", "int8", "nce_conv_patch", cpu)
+                    step, nbytes, ops, "mfma", "int8", "nce_conv_tile", cpu)
 
 
 def make_c5(rt, part="matmul"):

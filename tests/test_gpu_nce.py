@@ -30,7 +30,9 @@ def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0,
     OW = (W + pads[0] + pads[1] - KX) // strides[1] + 1
     out = torch.full((N, OH, OW, OC), 77, dtype=torch.int8 if out_signed else torch.uint8, device=dev)
     old = os.environ.pop("VPX_NCE_KERNEL", None)
-    if force:
+    if force == "patch":  # the persistent patch kernel instead of the one-tile-per-workgroup one
+        os.environ["VPX_CONV_TILE"] = "0"
+    elif force:
         os.environ["VPX_NCE_KERNEL"] = force
     try:
         rt.nce_task(dev_t(inp, dev), dev_t(w, dev), dev_t(wt, dev), out, p, zp_in=zp_in, zp_w=zp_w, zp_out=zp_out,
@@ -38,6 +40,7 @@ def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0,
         torch.cuda.synchronize()
     finally:
         os.environ.pop("VPX_NCE_KERNEL", None)
+        os.environ.pop("VPX_CONV_TILE", None)
         if old is not None:
             os.environ["VPX_NCE_KERNEL"] = old
     want = orc.nce_conv(inp, w, wt, op, zp_in=zp_in, zp_w=zp_w, strides=strides,
@@ -58,7 +61,7 @@ U8 = {"clamp_low": 0, "clamp_high": 255}
 I8 = {"clamp_low": -128, "clamp_high": 127}
 
 
-@pytest.mark.parametrize("force", [None, "gather", "naive"])
+@pytest.mark.parametrize("force", [None, "patch", "gather", "naive"])
 @pytest.mark.parametrize("geom", [
     dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
     dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)),
@@ -70,8 +73,9 @@ I8 = {"clamp_low": -128, "clamp_high": 127}
 def test_conv_paths(rt, orc, dev, geom, force):
     g = dict(geom)
     strides, pads = g.pop("strides"), g.pop("pads")
-    expect = {None: "nce_conv_patch" if g["IC"] % 64 == 0 else "nce_conv_mfma", "gather": "nce_conv_mfma",
-              "naive": "nce_conv_naive"}[force]
+    lds = g["IC"] % 64 == 0
+    expect = {None: "nce_conv_tile" if lds else "nce_conv_mfma", "patch": "nce_conv_patch" if lds else "nce_conv_mfma",
+              "gather": "nce_conv_mfma", "naive": "nce_conv_naive"}[force]
     rng = np.random.default_rng(50 + g["H"])
     for in_u8, zp_in, out_signed in ((True, 128, False), (True, 7, True), (False, -5, False), (False, 0, True)):
         inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, **g)
@@ -82,17 +86,18 @@ def test_conv_paths(rt, orc, dev, geom, force):
 
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 5])
-def test_conv_patch_tile_heights(rt, orc, dev, rows):
-    """The patch kernel with its tile height forced: tiles that end past the last output row, one-row tiles."""
+@pytest.mark.parametrize("force,kernel", [(None, "nce_conv_tile"), ("patch", "nce_conv_patch")])
+def test_conv_patch_tile_heights(rt, orc, dev, rows, force, kernel):
+    """Both LDS-patch kernels with the tile height forced: tiles that end past the last output row, one-row tiles."""
     rng = np.random.default_rng(55 + rows)
     inp, w, mults, shifts, bias = rand_case(rng, 2, 13, 24, 64, 80, 3, 3)
     os.environ["VPX_CONV_ROWS"] = str(rows)
     try:
         got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, U8, zp_in=121, zp_out=3,
-                                   strides=(1, 1), pads=(1, 1, 1, 1))
+                                   strides=(1, 1), pads=(1, 1, 1, 1), force=force)
     finally:
         del os.environ["VPX_CONV_ROWS"]
-    assert name == "nce_conv_patch"
+    assert name == kernel
     assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
 
 
@@ -152,7 +157,7 @@ def test_conv_config_c4_full_size(rt, orc, dev):
     got, want, name = run_task(rt, orc, dev, c["input"], c["weights"], c["mult"], c["shift"], c["bias"],
                                {"clamp_low": c["clamp"][0], "clamp_high": c["clamp"][1]}, zp_in=c["zp_in"],
                                strides=c["strides"], pads=c["pads"])
-    assert name == "nce_conv_patch"
+    assert name == "nce_conv_tile"
     assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
     assert 0 < (got == 0).mean() < 0.9  # the ReLU clamp is active and the output is not saturated flat
 

@@ -966,6 +966,216 @@ __global__ __launch_bounds__(256, TMW <= 4 ? 2 : 1) void nce_conv_patch(const in
     }
 }
 
+// ---------------------------------------------------------------- patch convolution, one tile per workgroup
+// The same tiling as nce_conv_patch with everything shaped for few instructions, which is what
+// bounds a convolution of a few microseconds: LDS rows are padded by 16 bytes instead of
+// xor-swizzled (pixel stride IC + 16, weight-row stride Ktot + 16: with IC a multiple of 64 the 16
+// lanes an LDS pass serves fall on 16 different 4-bank groups), so a fragment address is one add of
+// a per-tap scalar to a per-lane constant and the K steps inside a tap are immediate offsets;
+// one workgroup computes one tile; fragments of tap t+1 are read while the MFMAs of tap t run.
+// ICS = IC / 64.
+template <bool IN_U8, int TMW, bool SAME_F, int ICS, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce_conv_tile(const int8_t* __restrict__ in,
+                                                                      const int8_t* __restrict__ w,
+                                                                      const int32_t* __restrict__ wt,
+                                                                      uint8_t* __restrict__ out, ConvGeom g, PatchGeom pg,
+                                                                      int pad_byte, GemmPpe ppe) {
+    constexpr int BN = 64, IC = ICS * 64, KS = ICS * 2, PS = IC + 16, NT = 64 * NW;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int Ktot = g.KY * g.KX * IC, WS = Ktot + 16;
+    uint8_t* const wlds = smem;             // [64][Ktot + 16]
+    uint8_t* const patch = smem + BN * WS;  // [PH*PW][IC + 16], later the output staging tile
+    __shared__ int csum[BN];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int img = fdiv(blockIdx.x, pg.tiles_y);
+    const int oy0 = (blockIdx.x - img * (int)pg.tiles_y.d) * pg.R;
+    const int oc0 = blockIdx.y * BN;
+
+    // ---- weights and patch -> LDS; every load is issued before the first LDS store
+    {
+        constexpr int UW = NW == 8 ? 5 : 9, UP = NW == 8 ? 3 : 6;
+        const int cpr = (int)pg.cpr.d;                 // 16-byte chunks per weight row
+        const int wchunks = BN * cpr;
+        constexpr int cpp = IC / 16;
+        const int row_chunks = pg.PW * cpp;
+        const int upr = (int)pg.upr.d, units = pg.PH * upr;
+        const int pad32 = (pad_byte & 0xff) * 0x01010101;
+        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
+        const int iy0 = oy0 * g.SY - g.PT;
+        const bool full_rows = oc0 + BN <= g.OC;       // the 64 weight rows are one contiguous run
+        for (int q0 = 0, u0 = 0; q0 < wchunks || u0 < units; q0 += NT * UW, u0 += NW * UP) {
+            i32x4 qw[UW], qp[UP];
+            int dw[UW], dp[UP];
+#pragma unroll
+            for (int u = 0; u < UW; u++) {
+                const int q = q0 + u * NT + tid;
+                const bool ok = q < wchunks;
+                const int qq = ok ? q : 0;
+                const int row = fdiv(qq, pg.cpr);
+                int64_t src = (int64_t)qq * 16;
+                if (!full_rows) {
+                    const int64_t oc = oc0 + row < g.OC ? row : g.OC - 1 - oc0;
+                    src = oc * Ktot + (int64_t)(qq - row * cpr) * 16;
+                }
+                qw[u] = *reinterpret_cast<const i32x4*>(w + (int64_t)oc0 * Ktot + src);
+                dw[u] = ok ? (qq + row) * 16 : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < UP; u++) {
+                const int unit = u0 + wave + NW * u;
+                const int py = fdiv(unit, pg.upr);  // wave-uniform
+                const int qi = (unit - py * upr) * 64 + lane;
+                const bool ok = unit < units && qi < row_chunks;
+                const int px = qi / cpp, cc = qi % cpp;
+                const int iy = iy0 + py, ix = px - g.PL;
+                const bool inside = ok && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+                const int64_t off = inside ? ((int64_t)iy * g.W + ix) * IC + cc * 16 : 0;
+                const i32x4 v = *reinterpret_cast<const i32x4*>(img_base + off);
+                qp[u] = inside ? v : i32x4{pad32, pad32, pad32, pad32};
+                dp[u] = ok ? (py * pg.PW + px) * PS + cc * 16 : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < UW; u++)
+                if (dw[u] >= 0) *reinterpret_cast<i32x4*>(wlds + dw[u]) = qw[u];
+#pragma unroll
+            for (int u = 0; u < UP; u++)
+                if (dp[u] >= 0) {
+                    if (IN_U8) qp[u] ^= (int32_t)0x80808080;
+                    *reinterpret_cast<i32x4*>(patch + dp[u]) = qp[u];
+                }
+        }
+    }
+    __syncthreads();
+
+    // ---- per-channel weight sums from the LDS copy
+    if (ppe.corr != 0 && tid < 256) {
+        const int row = tid >> 2, part = tid & 3;
+        int sum = 0;
+        for (int c = part; c < (int)pg.cpr.d; c += 4) {
+            const i32x4 q = *reinterpret_cast<const i32x4*>(wlds + row * WS + c * 16);
+#pragma unroll
+            for (int j = 0; j < 4; j++) sum = __builtin_amdgcn_sdot4(q[j], 0x01010101, sum, false);
+        }
+        sum += (int)dpp_u32<0xB1>((unsigned)sum);
+        sum += (int)dpp_u32<0x4E>((unsigned)sum);
+        if (part == 0) csum[row] = sum;
+    }
+
+    // ---- main loop
+    const int nj = pg.nt == 2 ? wave & 1 : 0;
+    const int mi0 = pg.nt == 2 ? wave >> 1 : wave, mstep = pg.nt == 2 ? NW / 2 : NW;
+    const int npos = pg.R * (int)g.OW;
+    const int kgroup = lane >> 5;
+    int abase[TMW];
+#pragma unroll
+    for (int i = 0; i < TMW; i++) {
+        int p = (mi0 + i * mstep) * 32 + (lane & 31);
+        p = p < npos ? p : 0;
+        const int r = fdiv(p, pg.ow), ox = p - r * (int)g.OW;
+        abase[i] = (r * g.SY * pg.PW + ox * g.SX) * PS + kgroup * 16;
+    }
+    const int brow = nj * 32 + (lane & 31);
+    const int bbase = brow * WS + kgroup * 16;
+
+    i32x4 fa[2][KS][TMW], fb[2][KS];
+    auto read_tap = [&](auto buf_c, int soff_a, int soff_b) {
+        constexpr int buf = decltype(buf_c)::value;
+        const uint8_t* pb = wlds + bbase + soff_b;
+#pragma unroll
+        for (int k = 0; k < KS; k++) fb[buf][k] = *reinterpret_cast<const i32x4*>(pb + k * 32);
+#pragma unroll
+        for (int i = 0; i < TMW; i++) {
+            const uint8_t* pa = patch + abase[i] + soff_a;
+#pragma unroll
+            for (int k = 0; k < KS; k++) fa[buf][k][i] = *reinterpret_cast<const i32x4*>(pa + k * 32);
+        }
+    };
+    i32x16 acc[TMW];
+#pragma unroll
+    for (int i = 0; i < TMW; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0;
+    auto mfma_tap = [&](auto buf_c) {
+        constexpr int buf = decltype(buf_c)::value;
+#pragma unroll
+        for (int k = 0; k < KS; k++)
+#pragma unroll
+            for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][k][i], fb[buf][k], acc[i], 0, 0, 0);
+    };
+    const int taps = g.KY * g.KX;
+    int ky = 0, kx = 0, tap = 0;
+    auto next_tap = [&]() {  // advances (ky, kx, tap); returns false past the last one
+        tap++;
+        kx++;
+        if (kx == g.KX) {
+            kx = 0;
+            ky++;
+        }
+        return tap < taps;
+    };
+    read_tap(std::integral_constant<int, 0>{}, 0, 0);
+    for (;;) {
+        const bool more1 = next_tap();
+        if (more1) read_tap(std::integral_constant<int, 1>{}, (ky * pg.PW + kx) * PS, tap * IC);
+        mfma_tap(std::integral_constant<int, 0>{});
+        if (!more1) break;
+        const bool more0 = next_tap();
+        if (more0) read_tap(std::integral_constant<int, 0>{}, (ky * pg.PW + kx) * PS, tap * IC);
+        mfma_tap(std::integral_constant<int, 1>{});
+        if (!more0) break;
+    }
+    __syncthreads();  // all waves are done with the patch: its LDS becomes the output staging tile
+
+    // ---- epilogue
+    {
+        int64_t n = oc0 + brow;
+        n = n < g.OC ? n : g.OC - 1;
+        const int cs = ppe.corr != 0 ? csum[brow] : 0;
+        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        ChanPrep cp = ppe_prepare_packed((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+                                         (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
+        asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));
+        const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
+        const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 || pk.odd != 0;
+        const int col4 = nj * 32 + ((lane & 31) & ~3);
+        auto requant = [&](auto general_c) {
+#pragma unroll
+            for (int i = 0; i < TMW; i++) {
+                if (mi0 + i * mstep >= pg.MT) continue;
+#pragma unroll
+                for (int gq = 0; gq < 4; gq++) {
+                    unsigned v = ppe_pack4<SAME_F, decltype(general_c)::value>(acc[i][gq * 4], acc[i][gq * 4 + 1],
+                                                                               acc[i][gq * 4 + 2], acc[i][gq * 4 + 3], cp, pk);
+                    v = quad_transpose_bytes(v, lane);
+                    const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
+                    *reinterpret_cast<unsigned*>(patch + row * kPatchOutStride + col4) = v;
+                }
+            }
+        };
+        if (general) requant(std::true_type{});
+        else requant(std::false_type{});
+    }
+    __syncthreads();
+    const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
+    const int valid = rows_here * (int)g.OW;
+    const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
+    const bool vec_ok = (g.OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    for (int cid = tid; cid < valid * 4; cid += NT) {
+        const int row = cid >> 2, c16 = cid & 3;
+        const int64_t n = oc0 + c16 * 16;
+        if (n >= g.OC) continue;
+        const i32x4 v = *reinterpret_cast<const i32x4*>(patch + row * kPatchOutStride + c16 * 16);
+        uint8_t* dst = out + (pos0 + row) * g.OC + n;
+        if (vec_ok && n + 16 <= g.OC) {
+            __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
+        } else {
+            for (int e = 0; e < 16 && n + e < g.OC; e++) dst[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+        }
+    }
+}
+
 // ---------------------------------------------------------------- NCE eltwise (quantized add / subtract)
 // out = PPE((a - zp_a) * m1 +/- (b - zp_b) * m2): a streaming kernel, 16 bytes of each operand per
 // lane.  The zero points are folded into the bias (acc = a * m1 +/- b * m2 - (zp_a * m1 +/- zp_b * m2)),
@@ -1190,6 +1400,86 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         // Preferred: input patch and weights in LDS, one launch.  R = output rows per workgroup.
         if (allow_patch && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20) &&
             g.IC < (1 << 14) && g.W * g.SX < (1 << 14) && g.N * g.OH * g.OH < (1ll << 32)) {
+            // IC of 64 or 128: the one-tile-per-workgroup kernel with padded LDS rows (a tap's fragments of more
+            // channels do not fit the registers twice)
+            const char* tile_env = std::getenv("VPX_CONV_TILE");
+            if ((g.IC == 64 || g.IC == 128) && !(tile_env && *tile_env == '0')) {
+                PatchGeom pg{};
+                const int64_t PS = g.IC + 16, WS = Ktot + 16;
+                auto need = [&](int R) {
+                    const size_t patch = (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)PS;
+                    const size_t stage = (size_t)((R * g.OW + 31) / 32) * 32 * kPatchOutStride;
+                    return 64 * (size_t)WS + (patch > stage ? patch : stage);
+                };
+                int R = (int)(32 * kPatchMaxMT / g.OW);
+                if (R > g.OH) R = (int)g.OH;
+                while (R > 1 && need(R) > 160 * 1024 - 512) R--;
+                if (need(R) <= 160 * 1024 - 512) {
+                    const int64_t ocb = (g.OC + 63) / 64;
+                    while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 512 && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
+                    if (const char* e = std::getenv("VPX_CONV_ROWS")) {
+                        const int v = std::atoi(e);
+                        if (v >= 1 && v <= R) R = v;
+                    }
+                    const int tiles_y = (int)((g.OH + R - 1) / R);
+                    auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
+                    pg.R = (int)((g.OH + tiles_y - 1) / tiles_y);
+                    pg.PH = (pg.R - 1) * g.SY + g.KY;
+                    pg.PW = (int)(g.OW - 1) * g.SX + g.KX;
+                    pg.MT = (int)((pg.R * g.OW + 31) / 32);
+                    pg.nt = g.OC <= 32 ? 1 : 2;
+                    pg.ntiles = (int)(g.N * tiles_y);
+                    pg.tiles_y = fd(tiles_y);
+                    pg.cpr = fd(Ktot / 16);
+                    pg.cpp = fd(g.IC / 16);
+                    pg.upr = fd((pg.PW * (g.IC / 16) + 63) / 64);
+                    pg.ow = fd(g.OW);
+                    const size_t lds = need(pg.R);
+                    const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
+                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
+                    const int pad_byte = t.zp_in & 0xff;
+                    const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
+                    const char* cw = std::getenv("VPX_CONV_WAVES");
+                    const int nw = cw && std::atoi(cw) == 4 ? 4 : 8;
+                    const int per_wave = (pg.MT + nw / pg.nt - 1) / (nw / pg.nt);
+                    const int ics = (int)(g.IC / 64);
+#define VPX_TILE_W(U8, TMW, SAME, ICS, NW)                                                                            \
+    do {                                                                                                              \
+        auto kern = nce_conv_tile<U8, TMW, SAME, ICS, NW>;                                                            \
+        rc = set_dyn_lds(kern, lds);                                                                                  \
+        if (rc) return rc;                                                                                            \
+        hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,       \
+                           t.weight_table, (uint8_t*)t.output, g, pg, pad_byte, gp);                                  \
+    } while (0)
+#define VPX_TILE(U8, TMW, SAME, ICS)                                                                                  \
+    do {                                                                                                              \
+        if (nw == 8 && TMW <= 4) VPX_TILE_W(U8, (TMW <= 4 ? TMW : 4), SAME, ICS, 8);                                  \
+        else VPX_TILE_W(U8, TMW, SAME, ICS, 4);                                                                       \
+    } while (0)
+#define VPX_TILE_I(U8, TMW, SAME)                                                                                     \
+    do {                                                                                                              \
+        if (ics == 1) VPX_TILE(U8, TMW, SAME, 1);                                                                     \
+        else VPX_TILE(U8, TMW, SAME, 2);                                                                              \
+    } while (0)
+#define VPX_TILE_T(TMW)                                                                                               \
+    do {                                                                                                              \
+        if (in_u8 && same_f) VPX_TILE_I(true, TMW, true);                                                             \
+        else if (in_u8) VPX_TILE_I(true, TMW, false);                                                                 \
+        else if (same_f) VPX_TILE_I(false, TMW, true);                                                                \
+        else VPX_TILE_I(false, TMW, false);                                                                           \
+    } while (0)
+                    if (per_wave <= 2) VPX_TILE_T(2);
+                    else if (per_wave <= 4) VPX_TILE_T(4);
+                    else VPX_TILE_T(7);
+#undef VPX_TILE_T
+#undef VPX_TILE_I
+#undef VPX_TILE
+#undef VPX_TILE_W
+                    VPX_HIP_CHECK(hipGetLastError());
+                    *kernel_name = "nce_conv_tile";
+                    return VPX_RESULT_SUCCESS;
+                }
+            }
             PatchGeom pg{};
             const size_t lds_max = 160 * 1024 - 512;
             auto patch_need = [&](int R) {
