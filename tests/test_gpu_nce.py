@@ -278,3 +278,14 @@ def test_nce_rejects_bad_descriptors(rt, dev):
     with pytest.raises(rt.VpxError) as e:
         rt.nce_task(inp, big_k, wt, out, ok)
     assert e.value.code == rt.ERROR_INVALID_ARGUMENT and "fit" in e.value.text
+
+
+def test_c_abi_host_example(rt):
+    """The C++ host example drives softmax, an NCE matmul + PPE and dequantize through the C ABI alone
+    (its own process, the system HIP runtime, no Python in the loop) and checks them against host arithmetic."""
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(rt.__file__)), "examples", "c_abi_host")
+    assert os.path.exists(exe), "build the library first (vpux_plugin_amd/build.py)"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "OK" in r.stdout and "0 mismatches" in r.stdout
