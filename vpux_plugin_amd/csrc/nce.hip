@@ -562,28 +562,19 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
 template <int BM, int BN, bool IN_U8, bool OUT_SIGNED>
 __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                      const ChanPrep* __restrict__ prep, uint8_t* __restrict__ out,
-                                                     ConvGeom g, int pad_byte, int swz, PpeFast ppe) {
+                                                     ConvGeom g, int pad_byte, int swz, int tc, int icc, PpeFast ppe) {
     constexpr int WM = BM / 4;
     constexpr int TM = WM / 32, TN = BN / 32;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // [BN][Ktot]
+    // Weights are staged a slice of K at a time: `tc` taps x `icc` channels of each of the BN rows
+    // (the whole of K when it fits).  Slice row stride KC = tc * icc bytes.
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // [BN][KC]
     const int64_t Ktot = (int64_t)g.KY * g.KX * g.IC;
     const int64_t Mtot = g.N * g.OH * g.OW;
     const int64_t m0 = (int64_t)blockIdx.x * BM;
     const int64_t oc0 = (int64_t)blockIdx.y * BN;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-
-    // stage the weights: row = local output channel, 16-byte chunks, chunk index xor-ed with (row>>2)&3
-    const int64_t chunks_per_row = Ktot / 16;
-    for (int64_t cid = tid; cid < BN * chunks_per_row; cid += 256) {
-        const int row = (int)(cid / chunks_per_row);
-        const int64_t c = cid % chunks_per_row;
-        int64_t oc = oc0 + row;
-        oc = oc < g.OC ? oc : g.OC - 1;
-        const i32x4 q = *reinterpret_cast<const i32x4*>(w + oc * Ktot + c * 16);
-        const int64_t cs = swz ? ((c & ~3ll) | ((c ^ (row >> 2)) & 3)) : c;
-        *reinterpret_cast<i32x4*>(smem + row * Ktot + cs * 16) = q;
-    }
-    __syncthreads();
+    const int taps = g.KY * g.KX;
+    const int KC = tc * icc;
 
     // positions of this lane's rows
     int64_t base_n[TM];
@@ -607,39 +598,60 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
     const int kgroup = lane >> 5;  // which 16-byte half of a 32-wide K step this lane feeds
-    for (int ky = 0; ky < g.KY; ky++) {
-        for (int kx = 0; kx < g.KX; kx++) {
-            const int8_t* pin[TM];
-            bool inside[TM];
-#pragma unroll
-            for (int i = 0; i < TM; i++) {
-                const int iy = oy[i] * g.SY + ky - g.PT;
-                const int ix = ox[i] * g.SX + kx - g.PL;
-                inside[i] = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-                pin[i] = in + base_n[i] + ((int64_t)(inside[i] ? iy : 0) * g.W + (inside[i] ? ix : 0)) * g.IC + kgroup * 16;
+    for (int tap0 = 0; tap0 < taps; tap0 += tc) {
+        const int ntap = taps - tap0 < tc ? taps - tap0 : tc;
+        for (int ic0 = 0; ic0 < (int)g.IC; ic0 += icc) {
+            const int icn = (int)g.IC - ic0 < icc ? (int)g.IC - ic0 : icc;
+            // stage the slice: 16-byte chunks, chunk index xor-ed with (row>>2)&3 inside 64-byte granules
+            const int cpt = icn / 16;  // chunks per tap of this slice
+            const int chunks_per_row = ntap * cpt;
+            __syncthreads();           // everybody is done with the previous slice
+            for (int cid = tid; cid < BN * chunks_per_row; cid += 256) {
+                const int row = cid / chunks_per_row;
+                const int c = cid - row * chunks_per_row;
+                const int tl = c / cpt, cc = c - tl * cpt;
+                int64_t oc = oc0 + row;
+                oc = oc < g.OC ? oc : g.OC - 1;
+                const i32x4 q = *reinterpret_cast<const i32x4*>(w + oc * Ktot + (int64_t)(tap0 + tl) * g.IC + ic0 + cc * 16);
+                const int lc = tl * (icc / 16) + cc;  // chunk position in the slice row
+                const int cs = swz ? ((lc & ~3) | ((lc ^ (row >> 2)) & 3)) : lc;
+                *reinterpret_cast<i32x4*>(smem + row * KC + cs * 16) = q;
             }
-            const int64_t ktap = (int64_t)(ky * g.KX + kx) * g.IC;
-            for (int64_t ic = 0; ic < g.IC; ic += 32) {
-                i32x4 fa[TM], fb[TN];
+            __syncthreads();
+            for (int tl = 0; tl < ntap; tl++) {
+                const int tap = tap0 + tl;
+                const int ky = tap / g.KX, kx = tap - ky * g.KX;
+                const int8_t* pin[TM];
+                bool inside[TM];
 #pragma unroll
                 for (int i = 0; i < TM; i++) {
-                    i32x4 q = *reinterpret_cast<const i32x4*>(pin[i] + ic);
-                    if (!inside[i]) q = i32x4{pad32, pad32, pad32, pad32};
-                    if (IN_U8) q ^= (int32_t)0x80808080;
-                    fa[i] = q;
+                    const int iy = oy[i] * g.SY + ky - g.PT;
+                    const int ix = ox[i] * g.SX + kx - g.PL;
+                    inside[i] = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+                    pin[i] = in + base_n[i] + ((int64_t)(inside[i] ? iy : 0) * g.W + (inside[i] ? ix : 0)) * g.IC + ic0 + kgroup * 16;
                 }
-                const int64_t c = (ktap + ic) / 16 + kgroup;
+                for (int ic = 0; ic < icn; ic += 32) {
+                    i32x4 fa[TM], fb[TN];
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int row = j * 32 + (lane & 31);
-                    const int64_t cs = swz ? ((c & ~3ll) | ((c ^ (row >> 2)) & 3)) : c;
-                    fb[j] = *reinterpret_cast<const i32x4*>(smem + row * Ktot + cs * 16);
+                    for (int i = 0; i < TM; i++) {
+                        i32x4 q = *reinterpret_cast<const i32x4*>(pin[i] + ic);
+                        if (!inside[i]) q = i32x4{pad32, pad32, pad32, pad32};
+                        if (IN_U8) q ^= (int32_t)0x80808080;
+                        fa[i] = q;
+                    }
+                    const int c = tl * (icc / 16) + ic / 16 + kgroup;
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const int row = j * 32 + (lane & 31);
+                        const int cs = swz ? ((c & ~3) | ((c ^ (row >> 2)) & 3)) : c;
+                        fb[j] = *reinterpret_cast<const i32x4*>(smem + row * KC + cs * 16);
+                    }
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
                 }
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
             }
         }
     }
@@ -1339,8 +1351,10 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const bool allow_patch = allow_gemm || std::strcmp(force, "conv") == 0;
     const bool allow_mfma = allow_patch || std::strcmp(force, "gather") == 0;
 
-    const bool use_gemm = allow_gemm && is_gemm && g.IC % 64 == 0 && g.IC < (1 << 24);
-    if (allow_mfma && mfma_ok && aligned && (use_gemm || (g.IC % 32 == 0 && 64 * Ktot <= 128 * 1024))) {
+    // A 256-column matmul tile wastes three quarters of its MFMAs on 64 output channels: such 1x1 layers go
+    // to the convolution kernels, whose tiles are 64 channels wide (measured 7 us against 18 us at [100352 x 64 x 64]).
+    const bool use_gemm = allow_gemm && is_gemm && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || Mtot < 1024);
+    if (allow_mfma && mfma_ok && aligned && (use_gemm || g.IC % 32 == 0)) {
         int rc = VPX_RESULT_SUCCESS;
         const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
         PpeFast pf;
@@ -1564,17 +1578,21 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         VPX_HIP_CHECK(hipGetLastError());
 
         constexpr int BM = 256, BN = 64;
-        const size_t lds = (size_t)BN * Ktot;
+        // weight slice per staging round: whole taps while 64 rows of them fit 64 KiB, else 1024 channels of one tap
+        const int icc = g.IC <= 1024 ? (int)g.IC : 1024;
+        int tc = g.IC <= 1024 ? (int)(1024 / g.IC) : 1;
+        if (tc > g.KY * g.KX) tc = g.KY * g.KX;
+        const size_t lds = (size_t)BN * tc * icc;
         const dim3 grid((unsigned)((Mtot + BM - 1) / BM), (unsigned)((g.OC + BN - 1) / BN));
         const int pad_byte = t.zp_in & 0xff;
-        const int swz = Ktot % 64 == 0 ? 1 : 0;
+        const int swz = icc % 64 == 0 ? 1 : 0;
 #define VPX_CONV(U8, SGN)                                                                                            \
     do {                                                                                                             \
         auto kern = nce_conv_mfma<BM, BN, U8, SGN>;                                                                  \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
         hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights, prep,    \
-                           (uint8_t*)t.output, g, pad_byte, swz, pf);                                                \
+                           (uint8_t*)t.output, g, pad_byte, swz, tc, icc, pf);                                       \
     } while (0)
         if (in_u8 && out_signed) VPX_CONV(true, true);
         else if (in_u8) VPX_CONV(true, false);
