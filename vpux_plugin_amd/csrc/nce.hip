@@ -1188,6 +1188,212 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
     }
 }
 
+// ---------------------------------------------------------------- patch convolution with streamed weights
+// For layers whose weights do not fit LDS next to the input patch (many input channels): the patch
+// stays resident, the weights pass through two small LDS buffers a slice at a time -- one tap x KSL
+// channels of the 64 output channels (KSL = 64, 128 or 256, a divisor of IC).  The global loads of
+// slice s+1 are issued before the MFMAs of slice s and written to the other buffer after them;
+// one barrier per slice.  Same padded LDS rows and addressing as nce_conv_tile; IC is a run-time
+// multiple of 64.
+struct StreamGeom {
+    int ksl;       // channels per weight slice
+    int spt;       // slices per tap = IC / ksl
+};
+
+template <bool IN_U8, int TMW, bool SAME_F, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(const int8_t* __restrict__ in,
+                                                                           const int8_t* __restrict__ w,
+                                                                           const int32_t* __restrict__ wt,
+                                                                           const int32_t* __restrict__ colsum,
+                                                                           uint8_t* __restrict__ out, ConvGeom g,
+                                                                           PatchGeom pg, StreamGeom sg, int pad_byte,
+                                                                           GemmPpe ppe) {
+    constexpr int BN = 64, NT = 64 * NW, UWS = 256 * BN / 16 / NT;  // chunks of a 256-channel slice per thread
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int IC = (int)g.IC, PS = IC + 16;
+    const int Ktot = g.KY * g.KX * IC;
+    const int KSL = sg.ksl, WS = KSL + 16;
+    uint8_t* const wbuf = smem;                 // [2][64][KSL + 16]
+    uint8_t* const patch = smem + 2 * BN * WS;  // [PH*PW][IC + 16], later the output staging tile
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int img = fdiv(blockIdx.x, pg.tiles_y);
+    const int oy0 = (blockIdx.x - img * (int)pg.tiles_y.d) * pg.R;
+    const int oc0 = blockIdx.y * BN;
+
+    // weight slice transfer: chunk q of a slice = (row q / cps, chunk q % cps), cps = KSL / 16 (4, 8 or 16)
+    const int cps_shift = KSL == 64 ? 2 : (KSL == 128 ? 3 : 4);
+    const int slice_chunks = BN << cps_shift;
+    auto slice_issue = [&](int sl, i32x4(&q)[UWS]) {
+        const int tap = sl / sg.spt, ic0 = (sl - tap * sg.spt) * KSL;
+#pragma unroll
+        for (int u = 0; u < UWS; u++) {
+            const int qi = u * NT + tid;
+            const int qq = qi < slice_chunks ? qi : 0;
+            const int row = qq >> cps_shift, c = qq & ((1 << cps_shift) - 1);
+            int64_t oc = oc0 + row;
+            oc = oc < g.OC ? oc : g.OC - 1;
+            q[u] = *reinterpret_cast<const i32x4*>(w + oc * Ktot + (int64_t)tap * IC + ic0 + c * 16);
+        }
+    };
+    auto slice_commit = [&](int buf, const i32x4(&q)[UWS]) {
+#pragma unroll
+        for (int u = 0; u < UWS; u++) {
+            const int qi = u * NT + tid;
+            if (qi < slice_chunks) {
+                const int row = qi >> cps_shift, c = qi & ((1 << cps_shift) - 1);
+                *reinterpret_cast<i32x4*>(wbuf + buf * BN * WS + row * WS + c * 16) = q[u];
+            }
+        }
+    };
+
+    // ---- patch and the first weight slice -> LDS
+    i32x4 wq[UWS];
+    slice_issue(0, wq);
+    {
+        constexpr int UP = NW == 8 ? 4 : 6;
+        const int cpp = IC / 16;
+        const int row_chunks = pg.PW * cpp;
+        const int upr = (int)pg.upr.d, units = pg.PH * upr;
+        const int pad32 = (pad_byte & 0xff) * 0x01010101;
+        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
+        const int iy0 = oy0 * g.SY - g.PT;
+        for (int u0 = 0; u0 < units; u0 += NW * UP) {
+            i32x4 qp[UP];
+            int dp[UP];
+#pragma unroll
+            for (int u = 0; u < UP; u++) {
+                const int unit = u0 + wave + NW * u;
+                const int py = fdiv(unit, pg.upr);  // wave-uniform
+                const int qi = (unit - py * upr) * 64 + lane;
+                const bool ok = unit < units && qi < row_chunks;
+                const int px = fdiv(qi, pg.cpp), cc = qi - px * cpp;
+                const int iy = iy0 + py, ix = px - g.PL;
+                const bool inside = ok && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+                const int64_t off = inside ? ((int64_t)iy * g.W + ix) * IC + cc * 16 : 0;
+                const i32x4 v = *reinterpret_cast<const i32x4*>(img_base + off);
+                qp[u] = inside ? v : i32x4{pad32, pad32, pad32, pad32};
+                dp[u] = ok ? (py * pg.PW + px) * PS + cc * 16 : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < UP; u++)
+                if (dp[u] >= 0) {
+                    if (IN_U8) qp[u] ^= (int32_t)0x80808080;
+                    *reinterpret_cast<i32x4*>(patch + dp[u]) = qp[u];
+                }
+        }
+    }
+    slice_commit(0, wq);
+    __syncthreads();
+
+    // ---- main loop
+    const int nj = pg.nt == 2 ? wave & 1 : 0;
+    const int mi0 = pg.nt == 2 ? wave >> 1 : wave, mstep = pg.nt == 2 ? NW / 2 : NW;
+    const int npos = pg.R * (int)g.OW;
+    const int kgroup = lane >> 5;
+    int abase[TMW];
+#pragma unroll
+    for (int i = 0; i < TMW; i++) {
+        int p = (mi0 + i * mstep) * 32 + (lane & 31);
+        p = p < npos ? p : 0;
+        const int r = fdiv(p, pg.ow), ox = p - r * (int)g.OW;
+        abase[i] = (r * g.SY * pg.PW + ox * g.SX) * PS + kgroup * 16;
+    }
+    const int brow = nj * 32 + (lane & 31);
+    const int bbase = brow * WS + kgroup * 16;
+
+    i32x16 acc[TMW];
+#pragma unroll
+    for (int i = 0; i < TMW; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0;
+
+    const int slices = g.KY * g.KX * sg.spt;
+    const int ksteps = KSL / 32;
+    int ky = 0, kx = 0, sub = 0;  // position of the current slice
+    for (int sl = 0; sl < slices; sl++) {
+        const int buf = sl & 1;
+        const bool more = sl + 1 < slices;
+        if (more) slice_issue(sl + 1, wq);
+        const uint8_t* pa0 = patch + (ky * pg.PW + kx) * PS + sub * KSL;
+        const uint8_t* pb = wbuf + buf * BN * WS + bbase;
+        i32x4 fa[2][TMW], fb[2];
+        auto read_frags = [&](int slot, int k) {
+            fb[slot] = *reinterpret_cast<const i32x4*>(pb + k * 32);
+#pragma unroll
+            for (int i = 0; i < TMW; i++) fa[slot][i] = *reinterpret_cast<const i32x4*>(pa0 + abase[i] + k * 32);
+        };
+        read_frags(0, 0);
+        for (int k = 0; k < ksteps; k += 2) {  // ksteps is even
+            read_frags(1, k + 1);
+#pragma unroll
+            for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][i], fb[0], acc[i], 0, 0, 0);
+            if (k + 2 < ksteps) read_frags(0, k + 2);
+#pragma unroll
+            for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[1][i], fb[1], acc[i], 0, 0, 0);
+        }
+        if (more) slice_commit(buf ^ 1, wq);
+        __syncthreads();  // slice sl+1 is visible; nobody reads buffer `buf` any more
+        sub++;
+        if (sub == sg.spt) {
+            sub = 0;
+            kx++;
+            if (kx == g.KX) {
+                kx = 0;
+                ky++;
+            }
+        }
+    }
+
+    // ---- epilogue (the last barrier of the loop has freed the patch)
+    {
+        int64_t n = oc0 + brow;
+        n = n < g.OC ? n : g.OC - 1;
+        const int cs = colsum ? colsum[n] : 0;
+        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        ChanPrep cp = ppe_prepare_packed((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+                                         (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
+        asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));
+        const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
+        const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 || pk.odd != 0;
+        const int col4 = nj * 32 + ((lane & 31) & ~3);
+        auto requant = [&](auto general_c) {
+#pragma unroll
+            for (int i = 0; i < TMW; i++) {
+                if (mi0 + i * mstep >= pg.MT) continue;
+#pragma unroll
+                for (int gq = 0; gq < 4; gq++) {
+                    unsigned v = ppe_pack4<SAME_F, decltype(general_c)::value>(acc[i][gq * 4], acc[i][gq * 4 + 1],
+                                                                               acc[i][gq * 4 + 2], acc[i][gq * 4 + 3], cp, pk);
+                    v = quad_transpose_bytes(v, lane);
+                    const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
+                    *reinterpret_cast<unsigned*>(patch + row * kPatchOutStride + col4) = v;
+                }
+            }
+        };
+        if (general) requant(std::true_type{});
+        else requant(std::false_type{});
+    }
+    __syncthreads();
+    const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
+    const int valid = rows_here * (int)g.OW;
+    const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
+    const bool vec_ok = (g.OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    for (int cid = tid; cid < valid * 4; cid += NT) {
+        const int row = cid >> 2, c16 = cid & 3;
+        const int64_t n = oc0 + c16 * 16;
+        if (n >= g.OC) continue;
+        const i32x4 v = *reinterpret_cast<const i32x4*>(patch + row * kPatchOutStride + c16 * 16);
+        uint8_t* dst = out + (pos0 + row) * g.OC + n;
+        if (vec_ok && n + 16 <= g.OC) {
+            __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
+        } else {
+            for (int e = 0; e < 16 && n + e < g.OC; e++) dst[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+        }
+    }
+}
+
 // ---------------------------------------------------------------- NCE eltwise (quantized add / subtract)
 // out = PPE((a - zp_a) * m1 +/- (b - zp_b) * m2): a streaming kernel, 16 bytes of each operand per
 // lane.  The zero points are folded into the bias (acc = a * m1 +/- b * m2 - (zp_a * m1 +/- zp_b * m2)),
@@ -1416,8 +1622,10 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             g.IC < (1 << 14) && g.W * g.SX < (1 << 14) && g.N * g.OH * g.OH < (1ll << 32)) {
             // IC of 64 or 128: the one-tile-per-workgroup kernel with padded LDS rows (a tap's fragments of more
             // channels do not fit the registers twice)
-            const char* tile_env = std::getenv("VPX_CONV_TILE");
-            if ((g.IC == 64 || g.IC == 128) && !(tile_env && *tile_env == '0')) {
+            // VPX_CONV_KERNEL=stream|patch starts the choice below the faster kernels (tests compare them)
+            const char* ck = std::getenv("VPX_CONV_KERNEL");
+            const int first = !ck || !*ck ? 0 : (std::strcmp(ck, "stream") == 0 ? 1 : (std::strcmp(ck, "patch") == 0 ? 2 : 0));
+            if ((g.IC == 64 || g.IC == 128) && first <= 0) {
                 PatchGeom pg{};
                 const int64_t PS = g.IC + 16, WS = Ktot + 16;
                 auto need = [&](int R) {
@@ -1491,6 +1699,81 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
 #undef VPX_TILE_W
                     VPX_HIP_CHECK(hipGetLastError());
                     *kernel_name = "nce_conv_tile";
+                    return VPX_RESULT_SUCCESS;
+                }
+            }
+            // any IC that is a multiple of 64: resident patch, weights streamed a slice at a time
+            if (first <= 1) {
+                PatchGeom pg{};
+                StreamGeom sg{};
+                sg.ksl = g.IC % 256 == 0 ? 256 : (g.IC % 128 == 0 ? 128 : 64);
+                sg.spt = (int)(g.IC / sg.ksl);
+                const int64_t PS = g.IC + 16;
+                auto need = [&](int R) {
+                    const size_t patch = (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)PS;
+                    const size_t stage = (size_t)((R * g.OW + 31) / 32) * 32 * kPatchOutStride;
+                    return 2 * 64 * (size_t)(sg.ksl + 16) + (patch > stage ? patch : stage);
+                };
+                int R = (int)(32 * kPatchMaxMT / g.OW);
+                if (R > g.OH) R = (int)g.OH;
+                while (R > 1 && need(R) > 160 * 1024 - 512) R--;
+                if (need(R) <= 160 * 1024 - 512) {
+                    const int64_t ocb = (g.OC + 63) / 64;
+                    while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 512 && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
+                    if (const char* e = std::getenv("VPX_CONV_ROWS")) {
+                        const int v = std::atoi(e);
+                        if (v >= 1 && v <= R) R = v;
+                    }
+                    const int tiles_y = (int)((g.OH + R - 1) / R);
+                    auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
+                    pg.R = (int)((g.OH + tiles_y - 1) / tiles_y);
+                    pg.PH = (pg.R - 1) * g.SY + g.KY;
+                    pg.PW = (int)(g.OW - 1) * g.SX + g.KX;
+                    pg.MT = (int)((pg.R * g.OW + 31) / 32);
+                    pg.nt = g.OC <= 32 ? 1 : 2;
+                    pg.ntiles = (int)(g.N * tiles_y);
+                    pg.tiles_y = fd(tiles_y);
+                    pg.cpr = fd(Ktot / 16);
+                    pg.cpp = fd(g.IC / 16);
+                    pg.upr = fd((pg.PW * (g.IC / 16) + 63) / 64);
+                    pg.ow = fd(g.OW);
+                    const size_t lds = need(pg.R);
+                    const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
+                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
+                    const int pad_byte = t.zp_in & 0xff;
+                    const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
+                    int32_t* colsum = nullptr;
+                    if (corr != 0) {
+                        void* ws = nullptr;
+                        rc = get_workspace(s, sizeof(int32_t) * (size_t)g.OC, &ws);
+                        if (rc) return rc;
+                        colsum = (int32_t*)ws;
+                        hipLaunchKernelGGL(nce_colsum_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s,
+                                           (const int8_t*)t.weights, colsum, g.OC, Ktot);
+                        VPX_HIP_CHECK(hipGetLastError());
+                    }
+                    const int per_wave = (pg.MT + 8 / pg.nt - 1) / (8 / pg.nt);  // eight waves: at most 4 row blocks each
+#define VPX_STREAM_W(U8, TMW, SAME, NW)                                                                               \
+    do {                                                                                                              \
+        auto kern = nce_conv_stream<U8, TMW, SAME, NW>;                                                               \
+        rc = set_dyn_lds(kern, lds);                                                                                  \
+        if (rc) return rc;                                                                                            \
+        hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,       \
+                           t.weight_table, colsum, (uint8_t*)t.output, g, pg, sg, pad_byte, gp);                      \
+    } while (0)
+#define VPX_STREAM(TMW, NW)                                                                                           \
+    do {                                                                                                              \
+        if (in_u8 && same_f) VPX_STREAM_W(true, TMW, true, NW);                                                       \
+        else if (in_u8) VPX_STREAM_W(true, TMW, false, NW);                                                           \
+        else if (same_f) VPX_STREAM_W(false, TMW, true, NW);                                                          \
+        else VPX_STREAM_W(false, TMW, false, NW);                                                                     \
+    } while (0)
+                    if (per_wave <= 2) VPX_STREAM(2, 8);
+                    else VPX_STREAM(4, 8);
+#undef VPX_STREAM
+#undef VPX_STREAM_W
+                    VPX_HIP_CHECK(hipGetLastError());
+                    *kernel_name = "nce_conv_stream";
                     return VPX_RESULT_SUCCESS;
                 }
             }
