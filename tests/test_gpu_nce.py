@@ -30,7 +30,7 @@ def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0,
     OW = (W + pads[0] + pads[1] - KX) // strides[1] + 1
     out = torch.full((N, OH, OW, OC), 77, dtype=torch.int8 if out_signed else torch.uint8, device=dev)
     old = os.environ.pop("VPX_NCE_KERNEL", None)
-    if force in ("patch", "stream"):  # start the choice of LDS-patch kernel below the fastest one
+    if force == "stream":  # start the choice of LDS-patch kernel below the fastest one
         os.environ["VPX_CONV_KERNEL"] = force
     elif force:
         os.environ["VPX_NCE_KERNEL"] = force
@@ -61,7 +61,7 @@ U8 = {"clamp_low": 0, "clamp_high": 255}
 I8 = {"clamp_low": -128, "clamp_high": 127}
 
 
-@pytest.mark.parametrize("force", [None, "stream", "patch", "gather", "naive"])
+@pytest.mark.parametrize("force", [None, "stream", "gather", "naive"])
 @pytest.mark.parametrize("geom", [
     dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
     dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)),
@@ -76,27 +76,22 @@ I8 = {"clamp_low": -128, "clamp_high": 127}
 def test_conv_paths(rt, orc, dev, geom, force):
     g = dict(geom)
     strides, pads = g.pop("strides"), g.pop("pads")
-    big_k = 64 * g["KY"] * g["KX"] * g["IC"] > 140 * 1024  # weights alone (nearly) fill the LDS
     tile = g["IC"] in (64, 128)
     lds = g["IC"] % 64 == 0
     expect = {None: "nce_conv_tile" if tile else ("nce_conv_stream" if lds else "nce_conv_mfma"),
               "stream": "nce_conv_stream" if lds else "nce_conv_mfma",
-              "patch": "nce_conv_patch" if lds and not big_k else "nce_conv_mfma",
               "gather": "nce_conv_mfma", "naive": "nce_conv_naive"}[force]
     rng = np.random.default_rng(50 + g["H"])
     for in_u8, zp_in, out_signed in ((True, 128, False), (True, 7, True), (False, -5, False), (False, 0, True)):
         inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, **g)
         got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, I8 if out_signed else U8, zp_in=zp_in,
                                    strides=strides, pads=pads, out_signed=out_signed, force=force)
-        if big_k and force == "patch":
-            assert name in ("nce_conv_patch", "nce_conv_mfma")  # whichever the LDS budget allows, never the naive one
-        else:
-            assert name == expect
+        assert name == expect
         assert np.array_equal(got, want), "%s zp_in=%d: %d mismatches" % (name, zp_in, int((got != want).sum()))
 
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 5])
-@pytest.mark.parametrize("force,kernel", [(None, "nce_conv_tile"), ("stream", "nce_conv_stream"), ("patch", "nce_conv_patch")])
+@pytest.mark.parametrize("force,kernel", [(None, "nce_conv_tile"), ("stream", "nce_conv_stream")])
 def test_conv_patch_tile_heights(rt, orc, dev, rows, force, kernel):
     """Both LDS-patch kernels with the tile height forced: tiles that end past the last output row, one-row tiles."""
     rng = np.random.default_rng(55 + rows)

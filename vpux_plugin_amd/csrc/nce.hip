@@ -2,14 +2,18 @@
 // units and the integer PPE fused into the epilogue.
 //
 // Device paths (chosen by vpx_nce_task):
-//   nce_gemm_mfma  : 1x1 kernel, stride 1, no padding (this is how NCE.MatMul arrives): a plain
-//                    A[M][K] x B[N][K]^T GEMM.  256x256 output tile per workgroup, 128x128 per wave,
-//                    v_mfma_i32_32x32x32_i8.  K panels go from global memory straight into
-//                    XOR-swizzled LDS (global_load_lds, no register staging), two stages.
-//   nce_conv_mfma  : general KYxKX / stride / padding with IC a multiple of 32: implicit GEMM, the
-//                    activation fragments are gathered from the NHWC tensor (no im2col buffer),
-//                    the weights of the tile sit in LDS.
-//   nce_conv_naive : any shape and any zero points, one output per lane.
+//   nce_gemm_mfma   : 1x1 kernel, stride 1, no padding, more than 64 output channels (this is how
+//                     NCE.MatMul arrives): a plain A[M][K] x B[N][K]^T GEMM.  256x256 output tile per
+//                     workgroup, v_mfma_i32_32x32x32_i8, K panels from global memory straight into
+//                     XOR-swizzled LDS (global_load_lds, no register staging), four buffers.
+//   nce_conv_tile   : KYxKX / stride / padding with 64 or 128 input channels: the input rows of a tile
+//                     and the weights of 64 output channels sit in LDS, every tap is an LDS read.
+//   nce_conv_stream : the same with any multiple of 64 input channels: the weights pass through LDS a
+//                     slice at a time.
+//   nce_conv_mfma   : IC a multiple of 32, any size: activation fragments gathered from global
+//                     memory, weights staged a K slice at a time.
+//   nce_eltwise_kernel : task type ELTWISE (quantized add / subtract).
+//   nce_conv_naive  : any shape and any zero points, one output per lane.
 //
 // Zero points: the MFMA paths multiply raw bytes (u8 activations are re-biased to s8 by flipping
 // the top bit) and add the missing term to the bias: acc_true = acc_raw + k * sum_k w[oc][k] with
@@ -672,35 +676,15 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
     }
 }
 
-// ---------------------------------------------------------------- convolution with the input patch in LDS
+// ---------------------------------------------------------------- convolutions with the input patch in LDS
 // A tile is `R` whole output rows of one image x 64 output channels.  The (R-1)*SY+KY input rows a
 // tile needs are copied to LDS once, padding materialised with the zero-point byte and u8 re-biased
-// to s8 on the way, so every tap of every output position is an LDS read; the weights of the 64
-// channels sit beside them.  One launch does everything: the per-channel weight sums of the
-// zero-point term come from the LDS copy of the weights and the PPE parameters are unpacked from
-// the weight table.
+// to s8 on the way, so every tap of every output position is an LDS read.  The tile has
+// MT = ceil(R*OW / 32) row blocks of 32 positions and one or two column blocks of 32 channels; wave
+// w takes column block w % nt and the TMW row blocks w / nt + i * (waves / nt).  Row blocks past MT
+// are computed on position 0 and dropped: the main loops have no branches.
 //
-// Workgroups are persistent: each loads the weights and prepares the PPE parameters once, then
-// walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...  The global loads of tile t+1's patch are
-// issued before the MFMA loop of tile t and land in registers while it runs; they are written to
-// LDS after it, next to the PPE of tile t, whose bytes go through a separate staging area:
-//
-//     issue loads(t+1) | MFMA loop(t) | barrier | patch(t+1) -> LDS, PPE(t) -> staging | barrier |
-//     staging -> global (asynchronous) | next tile
-//
-// LDS layouts (16-byte chunks):
-//   weights [64][Ktot]      chunk c of row r at c ^ ((r >> 2) & 3) when Ktot is a multiple of 64
-//   patch   [PH*PW][IC]     chunk c of pixel p at c ^ ((p >> 2) & 3)   (IC is a multiple of 64)
-//   staging [MT*32][80]     output bytes of the tile, 64 per position
-// Lanes 0-31 of a fragment read walk consecutive rows / pixels at one chunk index; the xor spreads
-// them over all banks.
-//
-// Waves: the tile has MT = ceil(R*OW / 32) row blocks of 32 positions and one or two column blocks
-// of 32 channels; wave w takes column block w % nt and the TMW row blocks w / nt + i * (4 / nt).
-// Row blocks past MT are computed on position 0 and dropped: the main loop has no branches, and
-// the fragments of K step s+1 are read while the MFMAs of step s run.
-//
-// At the sizes this kernel serves a whole launch lasts a few microseconds, so index arithmetic
+// At the sizes these kernels serve a whole launch lasts a few microseconds, so index arithmetic
 // counts: divisions by launch constants use multiply-high reciprocals prepared on the host.
 struct FastDiv {
     uint32_t d, m;  // m = ceil(2^32 / d); exact for numerators below 2^32 / d
@@ -722,264 +706,12 @@ struct PatchGeom {
 
 constexpr int kPatchMaxMT = 14;
 constexpr int kPatchOutStride = 80;  // bytes per output position in the staging tile
-constexpr int kPatchPrefetch = 6;    // 16-byte patch chunks per lane fetched ahead of the MFMA loop
 
-// SAME_F: the PPE treats both signs alike (no PReLU stage), which drops the per-value sign test.
-template <bool IN_U8, int TMW, bool SAME_F>
-__global__ __launch_bounds__(256, TMW <= 4 ? 2 : 1) void nce_conv_patch(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
-                                                      const int32_t* __restrict__ wt, uint8_t* __restrict__ out,
-                                                      ConvGeom g, PatchGeom pg, int pad_byte, GemmPpe ppe) {
-    constexpr int BN = 64;
-    constexpr int UP = kPatchPrefetch;
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const int Ktot = g.KY * g.KX * (int)g.IC;
-    const int IC = (int)g.IC;
-    uint8_t* const wlds = smem;                      // [64][Ktot]
-    uint8_t* const patch = smem + BN * Ktot;         // [PH*PW][IC]
-    uint8_t* const stage = patch + pg.patch_bytes;   // [MT*32][kPatchOutStride]
-    __shared__ int csum[BN];
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int oc0 = blockIdx.y * BN;
-
-    // patch transfer: a unit is 64 consecutive chunks of one patch row; units go round the waves
-    const int cpp = (int)pg.cpp.d;
-    const int row_chunks = pg.PW * cpp;
-    const int upr = (int)pg.upr.d;
-    const int units = pg.PH * upr;
-    const int pad32 = (pad_byte & 0xff) * 0x01010101;
-    // loads units unit0 + wave + 4u (u < UP) of tile `tile` into registers; dst < 0 marks an unused slot
-    auto patch_issue = [&](int tile, int unit0, i32x4(&q)[UP], int(&dst)[UP]) {
-        const int img = fdiv(tile, pg.tiles_y);
-        const int iy0 = (tile - img * (int)pg.tiles_y.d) * pg.R * g.SY - g.PT;
-        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
-        // branch-free: a slot without work loads from a valid dummy address and is marked by dst < 0
-#pragma unroll
-        for (int u = 0; u < UP; u++) {
-            const int unit = unit0 + wave + 4 * u;
-            const int py = fdiv(unit, pg.upr);  // wave-uniform
-            const int qi = (unit - py * upr) * 64 + lane;
-            const bool ok = unit < units && qi < row_chunks;
-            const int px = fdiv(qi, pg.cpp), cc = qi - px * cpp;
-            const int iy = iy0 + py, ix = px - g.PL;
-            const bool inside = ok && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-            const int64_t off = inside ? ((int64_t)iy * g.W + ix) * IC + cc * 16 : 0;
-            const i32x4 v = *reinterpret_cast<const i32x4*>(img_base + off);
-            q[u] = inside ? v : i32x4{pad32, pad32, pad32, pad32};
-            const int pp = py * pg.PW + px;
-            dst[u] = ok ? pp * IC + ((cc ^ ((pp >> 2) & 3)) << 4) : -1;
-        }
-    };
-    auto patch_commit = [&](i32x4(&q)[UP], int(&dst)[UP]) {
-#pragma unroll
-        for (int u = 0; u < UP; u++)
-            if (dst[u] >= 0) {
-                if (IN_U8) q[u] ^= (int32_t)0x80808080;
-                *reinterpret_cast<i32x4*>(patch + dst[u]) = q[u];
-            }
-    };
-
-    int tile = blockIdx.x;
-    i32x4 pq[UP];
-    int pdst[UP];
-    patch_issue(tile, 0, pq, pdst);  // in flight together with the weights
-
-    // ---- weights -> LDS, once.  (row, chunk) pairs; 256 = dr * cpr + dc advances both without a division.
-    {
-        const int cpr = (int)pg.cpr.d;
-        const int dr = fdiv(256, pg.cpr), dc = 256 - dr * cpr;
-        int row = fdiv(tid, pg.cpr), c = tid - row * cpr;
-        constexpr int UW = 9;
-        while (row < BN) {
-            i32x4 qw[UW];
-            int dw[UW];
-#pragma unroll
-            for (int u = 0; u < UW; u++) {
-                const bool ok = row < BN;
-                const int rr = ok ? row : BN - 1;
-                int64_t oc = oc0 + rr;
-                oc = oc < g.OC ? oc : g.OC - 1;
-                qw[u] = *reinterpret_cast<const i32x4*>(w + oc * Ktot + c * 16);
-                const int cs = pg.w_swz ? c ^ ((rr >> 2) & 3) : c;
-                dw[u] = ok ? rr * Ktot + cs * 16 : -1;
-                row += dr;
-                c += dc;
-                if (c >= cpr) {
-                    c -= cpr;
-                    row++;
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < UW; u++)
-                if (dw[u] >= 0) *reinterpret_cast<i32x4*>(wlds + dw[u]) = qw[u];
-        }
-    }
-    patch_commit(pq, pdst);
-    for (int unit0 = 4 * UP; unit0 < units; unit0 += 4 * UP) {  // patches larger than the prefetch window
-        patch_issue(tile, unit0, pq, pdst);
-        patch_commit(pq, pdst);
-    }
-    __syncthreads();
-
-    // ---- per-channel weight sums from the LDS copy (chunk order within a row does not matter)
-    if (ppe.corr != 0) {
-        const int row = tid >> 2, part = tid & 3;
-        int sum = 0;
-        for (int c = part; c < (int)pg.cpr.d; c += 4) {
-            const i32x4 q = *reinterpret_cast<const i32x4*>(wlds + row * Ktot + c * 16);
-#pragma unroll
-            for (int j = 0; j < 4; j++) sum = __builtin_amdgcn_sdot4(q[j], 0x01010101, sum, false);
-        }
-        sum += (int)dpp_u32<0xB1>((unsigned)sum);
-        sum += (int)dpp_u32<0x4E>((unsigned)sum);
-        if (part == 0) csum[row] = sum;
-        __syncthreads();
-    }
-
-    // ---- per-wave constants: tile geometry, B addressing, PPE parameters of this lane's channel
-    const int nj = pg.nt == 2 ? wave & 1 : 0;  // column block of this wave
-    const int mi0 = pg.nt == 2 ? wave >> 1 : wave, mstep = pg.nt == 2 ? 2 : 4;
-    const int npos = pg.R * (int)g.OW;         // output positions of a full tile
-    int pp0[TMW];
-#pragma unroll
-    for (int i = 0; i < TMW; i++) {
-        int p = (mi0 + i * mstep) * 32 + (lane & 31);
-        p = p < npos ? p : 0;
-        const int r = fdiv(p, pg.ow), ox = p - r * (int)g.OW;
-        pp0[i] = r * g.SY * pg.PW + ox * g.SX;
-    }
-    const int kgroup = lane >> 5;
-    const int brow = nj * 32 + (lane & 31);
-    const uint8_t* const bbase = wlds + brow * Ktot;
-    const int bsw = pg.w_swz ? (brow >> 2) & 3 : 0;
-
-    ChanPrep cp;
-    {
-        int64_t n = oc0 + brow;
-        n = n < g.OC ? n : g.OC - 1;
-        const int cs = ppe.corr != 0 ? csum[brow] : 0;
-        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
-        cp = ppe_prepare_packed((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
-                                (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
-    }
-    asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));  // keep the factors in registers instead of re-deriving them per value
-    const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
-    const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 ||
-                         pk.odd != 0;
-    const int col4 = nj * 32 + ((lane & 31) & ~3);
-    const bool vec_ok = (g.OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
-    const int steps = g.KY * g.KX * (IC >> 5);  // even: IC is a multiple of 64
-
-    for (; tile < pg.ntiles; tile += gridDim.x) {
-        const int next = tile + gridDim.x;
-        const bool has_next = next < pg.ntiles;
-        if (has_next) patch_issue(next, 0, pq, pdst);
-
-        // ---- MFMA loop over taps and channels
-        i32x16 acc[TMW];
-#pragma unroll
-        for (int i = 0; i < TMW; i++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][r] = 0;
-        int ky = 0, kx = 0, ic = 0, ctap = 0;
-        int abase[TMW], asw[TMW];
-        auto set_tap = [&]() {
-            const int tap_pp = ky * pg.PW + kx;
-#pragma unroll
-            for (int i = 0; i < TMW; i++) {
-                const int pp = pp0[i] + tap_pp;
-                abase[i] = pp * IC;
-                asw[i] = (pp >> 2) & 3;
-            }
-        };
-        auto read_frags = [&](i32x4(&fa)[TMW], i32x4& fb) {
-            const int c = (ic >> 4) + kgroup;
-            fb = *reinterpret_cast<const i32x4*>(bbase + (((ctap + c) ^ bsw) << 4));
-#pragma unroll
-            for (int i = 0; i < TMW; i++) fa[i] = *reinterpret_cast<const i32x4*>(patch + abase[i] + ((c ^ asw[i]) << 4));
-        };
-        auto advance = [&]() {
-            ic += 32;
-            if (ic == IC) {
-                ic = 0;
-                ctap += IC >> 4;
-                kx++;
-                if (kx == g.KX) {
-                    kx = 0;
-                    ky++;
-                }
-                set_tap();
-            }
-        };
-        i32x4 fa0[TMW], fa1[TMW], fb0, fb1;
-        set_tap();
-        read_frags(fa0, fb0);
-        for (int s = 0; s < steps; s += 2) {
-            advance();
-            read_frags(fa1, fb1);
-#pragma unroll
-            for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa0[i], fb0, acc[i], 0, 0, 0);
-            if (s + 2 < steps) {
-                advance();
-                read_frags(fa0, fb0);
-            }
-#pragma unroll
-            for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa1[i], fb1, acc[i], 0, 0, 0);
-        }
-        __syncthreads();  // every wave is done reading this tile's patch (and the previous tile's staging bytes)
-
-        // ---- next tile's patch -> LDS
-        if (has_next) {
-            patch_commit(pq, pdst);
-            for (int unit0 = 4 * UP; unit0 < units; unit0 += 4 * UP) {
-                patch_issue(next, unit0, pq, pdst);
-                patch_commit(pq, pdst);
-            }
-        }
-
-        // ---- PPE of this tile -> staging
-        auto requant = [&](auto general_c) {
-#pragma unroll
-            for (int i = 0; i < TMW; i++) {
-                if (mi0 + i * mstep >= pg.MT) continue;
-#pragma unroll
-                for (int gq = 0; gq < 4; gq++) {
-                    unsigned v = ppe_pack4<SAME_F, decltype(general_c)::value>(acc[i][gq * 4], acc[i][gq * 4 + 1],
-                                                                               acc[i][gq * 4 + 2], acc[i][gq * 4 + 3], cp, pk);
-                    v = quad_transpose_bytes(v, lane);
-                    const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
-                    *reinterpret_cast<unsigned*>(stage + row * kPatchOutStride + col4) = v;
-                }
-            }
-        };
-        if (general) requant(std::true_type{});
-        else requant(std::false_type{});
-        __syncthreads();
-
-        // ---- staging -> global
-        const int img = fdiv(tile, pg.tiles_y);
-        const int oy0 = (tile - img * (int)pg.tiles_y.d) * pg.R;
-        const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
-        const int valid = rows_here * (int)g.OW;
-        const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
-        for (int cid = tid; cid < valid * 4; cid += 256) {
-            const int row = cid >> 2, c16 = cid & 3;
-            const int64_t n = oc0 + c16 * 16;
-            if (n >= g.OC) continue;
-            const i32x4 v = *reinterpret_cast<const i32x4*>(stage + row * kPatchOutStride + c16 * 16);
-            uint8_t* dst = out + (pos0 + row) * g.OC + n;
-            if (vec_ok && n + 16 <= g.OC) {
-                __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
-            } else {
-                for (int e = 0; e < 16 && n + e < g.OC; e++) dst[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
-            }
-        }
-    }
-}
+// SAME_F (template parameter of the kernels below): the PPE treats both signs alike (no PReLU stage),
+// which drops the per-value sign test.
 
 // ---------------------------------------------------------------- patch convolution, one tile per workgroup
-// The same tiling as nce_conv_patch with everything shaped for few instructions, which is what
+// Everything here is shaped for few instructions, which is what
 // bounds a convolution of a few microseconds: LDS rows are padded by 16 bytes instead of
 // xor-swizzled (pixel stride IC + 16, weight-row stride Ktot + 16: with IC a multiple of 64 the 16
 // lanes an LDS pass serves fall on 16 different 4-bank groups), so a fragment address is one add of
@@ -1554,8 +1286,8 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     // to check the device paths against each other).
     const char* force = std::getenv("VPX_NCE_KERNEL");
     const bool allow_gemm = !force || !*force;
-    const bool allow_patch = allow_gemm || std::strcmp(force, "conv") == 0;
-    const bool allow_mfma = allow_patch || std::strcmp(force, "gather") == 0;
+    const bool allow_lds = allow_gemm || std::strcmp(force, "conv") == 0;
+    const bool allow_mfma = allow_lds || std::strcmp(force, "gather") == 0;
 
     // A 256-column matmul tile wastes three quarters of its MFMAs on 64 output channels: such 1x1 layers go
     // to the convolution kernels, whose tiles are 64 channels wide (measured 7 us against 18 us at [100352 x 64 x 64]).
@@ -1617,14 +1349,14 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             return VPX_RESULT_SUCCESS;
         }
 
-        // Preferred: input patch and weights in LDS, one launch.  R = output rows per workgroup.
-        if (allow_patch && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20) &&
+        // Preferred: input patch in LDS, one launch.  R = output rows per workgroup.
+        if (allow_lds && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20) &&
             g.IC < (1 << 14) && g.W * g.SX < (1 << 14) && g.N * g.OH * g.OH < (1ll << 32)) {
             // IC of 64 or 128: the one-tile-per-workgroup kernel with padded LDS rows (a tap's fragments of more
             // channels do not fit the registers twice)
-            // VPX_CONV_KERNEL=stream|patch starts the choice below the faster kernels (tests compare them)
+            // VPX_CONV_KERNEL=stream starts the choice below the tile kernel (tests compare them)
             const char* ck = std::getenv("VPX_CONV_KERNEL");
-            const int first = !ck || !*ck ? 0 : (std::strcmp(ck, "stream") == 0 ? 1 : (std::strcmp(ck, "patch") == 0 ? 2 : 0));
+            const int first = ck && std::strcmp(ck, "stream") == 0 ? 1 : 0;
             if ((g.IC == 64 || g.IC == 128) && first <= 0) {
                 PatchGeom pg{};
                 const int64_t PS = g.IC + 16, WS = Ktot + 16;
@@ -1776,78 +1508,6 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     *kernel_name = "nce_conv_stream";
                     return VPX_RESULT_SUCCESS;
                 }
-            }
-            PatchGeom pg{};
-            const size_t lds_max = 160 * 1024 - 512;
-            auto patch_need = [&](int R) {
-                return (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)g.IC;
-            };
-            auto lds_need = [&](int R) {
-                return 64 * (size_t)Ktot + patch_need(R) + (size_t)((R * g.OW + 31) / 32) * 32 * kPatchOutStride;
-            };
-            int R = (int)(32 * kPatchMaxMT / g.OW);
-            if (R > g.OH) R = (int)g.OH;
-            while (R > 1 && lds_need(R) > lds_max) R--;
-            if (lds_need(R) <= lds_max) {
-                const int64_t ocb = (g.OC + 63) / 64;
-                int cus = 0, devid = 0;
-                VPX_HIP_CHECK(hipGetDevice(&devid));
-                VPX_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, devid));
-                // enough tiles to fill the device twice, as long as a tile keeps at least 4 row blocks
-                while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 2ll * cus && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
-                if (const char* e = std::getenv("VPX_CONV_ROWS")) {
-                    const int v = std::atoi(e);
-                    if (v >= 1 && lds_need(v) <= lds_max && v * g.OW <= 32 * kPatchMaxMT) R = v;
-                }
-                const int tiles_y = (int)((g.OH + R - 1) / R);
-                auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
-                pg.R = (int)((g.OH + tiles_y - 1) / tiles_y);
-                pg.PH = (pg.R - 1) * g.SY + g.KY;
-                pg.PW = (int)(g.OW - 1) * g.SX + g.KX;
-                pg.MT = (int)((pg.R * g.OW + 31) / 32);
-                pg.nt = g.OC <= 32 ? 1 : 2;
-                pg.w_swz = Ktot % 64 == 0 ? 1 : 0;
-                pg.ntiles = (int)(g.N * tiles_y);
-                pg.patch_bytes = (int)patch_need(pg.R);
-                pg.tiles_y = fd(tiles_y);
-                pg.cpr = fd(Ktot / 16);
-                pg.cpp = fd(g.IC / 16);
-                pg.upr = fd((pg.PW * (g.IC / 16) + 63) / 64);
-                pg.ow = fd(g.OW);
-                const size_t lds = lds_need(pg.R);
-                const int per_cu = lds <= 80 * 1024 ? 2 : 1;
-                int64_t blocks = (int64_t)cus * per_cu / ocb;
-                if (blocks < 1) blocks = 1;
-                if (blocks > pg.ntiles) blocks = pg.ntiles;
-                const dim3 grid((unsigned)blocks, (unsigned)ocb);
-                GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
-                const int pad_byte = t.zp_in & 0xff;
-                const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
-                const int per_wave = (pg.MT + 4 / pg.nt - 1) / (4 / pg.nt);  // row blocks the busiest wave owns
-#define VPX_PATCH(U8, TMW, SAME)                                                                                     \
-    do {                                                                                                             \
-        auto kern = nce_conv_patch<U8, TMW, SAME>;                                                                   \
-        rc = set_dyn_lds(kern, lds);                                                                                 \
-        if (rc) return rc;                                                                                           \
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,          \
-                           t.weight_table, (uint8_t*)t.output, g, pg, pad_byte, gp);                                 \
-    } while (0)
-#define VPX_PATCH_T(TMW)                                                                                             \
-    do {                                                                                                             \
-        if (in_u8 && same_f) VPX_PATCH(true, TMW, true);                                                             \
-        else if (in_u8) VPX_PATCH(true, TMW, false);                                                                 \
-        else if (same_f) VPX_PATCH(false, TMW, true);                                                                \
-        else VPX_PATCH(false, TMW, false);                                                                           \
-    } while (0)
-                if (per_wave <= 1) VPX_PATCH_T(1);
-                else if (per_wave <= 2) VPX_PATCH_T(2);
-                else if (per_wave <= 4) VPX_PATCH_T(4);
-                else VPX_PATCH_T(7);
-#undef VPX_PATCH_T
-#undef VPX_PATCH
-                VPX_HIP_CHECK(hipGetLastError());
-                *kernel_name = "nce_conv_patch";
-                return VPX_RESULT_SUCCESS;
             }
         }
         // Fallback: activation fragments gathered from global memory; per-channel parameters come
