@@ -72,15 +72,19 @@ I8 = {"clamp_low": -128, "clamp_high": 127}
     # K too large for the weights of 64 channels to sit in LDS at once: staged a slice at a time
     dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
     dict(N=1, H=8, W=8, IC=1536, OC=32, KY=1, KX=1, strides=(2, 2), pads=(0, 0, 0, 0)),
+    # channel counts that are a multiple of 16 only (stem layers): two taps can share an MFMA step, odd tap counts
+    dict(N=2, H=30, W=30, IC=16, OC=64, KY=7, KX=7, strides=(2, 2), pads=(3, 3, 3, 3)),
+    dict(N=1, H=10, W=12, IC=48, OC=40, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
 ])
 def test_conv_paths(rt, orc, dev, geom, force):
     g = dict(geom)
     strides, pads = g.pop("strides"), g.pop("pads")
     tile = g["IC"] in (64, 128)
     lds = g["IC"] % 64 == 0
-    expect = {None: "nce_conv_tile" if tile else ("nce_conv_stream" if lds else "nce_conv_mfma"),
-              "stream": "nce_conv_stream" if lds else "nce_conv_mfma",
-              "gather": "nce_conv_mfma", "naive": "nce_conv_naive"}[force]
+    gather = "nce_conv_mfma" if g["IC"] % 32 == 0 else "nce_conv_mfma16"
+    expect = {None: "nce_conv_tile" if tile else ("nce_conv_stream" if lds else gather),
+              "stream": "nce_conv_stream" if lds else gather,
+              "gather": gather, "naive": "nce_conv_naive"}[force]
     rng = np.random.default_rng(50 + g["H"])
     for in_u8, zp_in, out_signed in ((True, 128, False), (True, 7, True), (False, -5, False), (False, 0, True)):
         inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, **g)

@@ -12,6 +12,7 @@
 //                     slice at a time.
 //   nce_conv_mfma   : IC a multiple of 32, any size: activation fragments gathered from global
 //                     memory, weights staged a K slice at a time.
+//   nce_conv_mfma16 : IC a multiple of 16 only (stem layers), K up to 1008: two taps may share an MFMA step.
 //   nce_eltwise_kernel : task type ELTWISE (quantized add / subtract).
 //   nce_conv_naive  : any shape and any zero points, one output per lane.
 //
@@ -1173,6 +1174,97 @@ __global__ __launch_bounds__(256) void nce_eltwise_kernel(const uint8_t* __restr
     }
 }
 
+// ---------------------------------------------------------------- gather convolution, IC a multiple of 16
+// Stem layers (3 or 4 image channels padded to 16) and other channel counts that are a multiple of
+// 16 but not of 32.  K = KY*KX*IC is walked as a flat run of 16-byte chunks, two per MFMA step:
+// lanes 0-31 feed chunk 2j, lanes 32-63 chunk 2j+1, which may belong to different taps.  All
+// weights of the 64 output channels (K rounded up to 32, zero-filled) sit in LDS.
+template <bool IN_U8>
+__global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
+                                                       const ChanPrep* __restrict__ prep, uint8_t* __restrict__ out,
+                                                       ConvGeom g, int pad_byte, PpeFast ppe) {
+    constexpr int BM = 256, BN = 64, WM = BM / 4, TM = WM / 32, TN = BN / 32;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];  // [BN][K32 + 16]
+    const int Ktot = g.KY * g.KX * (int)g.IC;
+    const int K32 = (Ktot + 31) & ~31, WS = K32 + 16;
+    const int64_t Mtot = g.N * g.OH * g.OW;
+    const int64_t m0 = (int64_t)blockIdx.x * BM;
+    const int64_t oc0 = (int64_t)blockIdx.y * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cpr = K32 / 16, cpt = (int)g.IC / 16;
+
+    for (int cid = tid; cid < BN * cpr; cid += 256) {
+        const int row = cid / cpr, c = cid - row * cpr;
+        int64_t oc = oc0 + row;
+        oc = oc < g.OC ? oc : g.OC - 1;
+        i32x4 q = i32x4{0, 0, 0, 0};
+        if (c * 16 < Ktot) q = *reinterpret_cast<const i32x4*>(w + oc * Ktot + c * 16);
+        *reinterpret_cast<i32x4*>(smem + row * WS + c * 16) = q;
+    }
+    __syncthreads();
+
+    int64_t base_n[TM];
+    int oy[TM], ox[TM];
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        int64_t m = m0 + wave * WM + i * 32 + (lane & 31);
+        m = m < Mtot ? m : Mtot - 1;
+        ox[i] = (int)(m % g.OW) * g.SX - g.PL;
+        oy[i] = (int)((m / g.OW) % g.OH) * g.SY - g.PT;
+        base_n[i] = (m / (g.OW * g.OH)) * g.H * g.W * g.IC;
+    }
+    const int pad32 = (pad_byte & 0xff) * 0x01010101;
+    i32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+    const int kgroup = lane >> 5;
+    const int last_tap = g.KY * g.KX - 1;
+    for (int c = kgroup; c < cpr; c += 2) {  // this lane's chunk of every step
+        int tap = c / cpt;
+        const int cc = c - tap * cpt;
+        const bool real = tap <= last_tap;   // the zero-filled tail of K: any finite activation will do
+        tap = real ? tap : last_tap;
+        const int ky = tap / g.KX, kx = tap - ky * g.KX;
+        i32x4 fa[TM], fb[TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int iy = oy[i] + ky, ix = ox[i] + kx;
+            const bool inside = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
+            const int64_t off = inside ? ((int64_t)iy * g.W + ix) * g.IC + cc * 16 : 0;
+            i32x4 q = *reinterpret_cast<const i32x4*>(in + base_n[i] + off);
+            if (!inside) q = i32x4{pad32, pad32, pad32, pad32};
+            if (IN_U8) q ^= (int32_t)0x80808080;
+            fa[i] = q;
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[j] = *reinterpret_cast<const i32x4*>(smem + (j * 32 + (lane & 31)) * WS + c * 16);
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int64_t oc = oc0 + j * 32 + (lane & 31);
+        if (oc >= g.OC) continue;
+        const ChanPrep cp = prep[oc];
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t m = m0 + wave * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                if (m < Mtot) out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(acc[i][j][r], cp, ppe);
+            }
+        }
+    }
+}
+
 template <class KernelT>
 int set_dyn_lds(KernelT kernel, size_t bytes) {
     if (bytes > 64 * 1024) {
@@ -1544,6 +1636,35 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
 #undef VPX_CONV
         VPX_HIP_CHECK(hipGetLastError());
         *kernel_name = "nce_conv_mfma";
+        return VPX_RESULT_SUCCESS;
+    }
+
+    if (allow_mfma && mfma_ok && aligned && g.IC % 16 == 0 && g.IC % 32 != 0 && ((Ktot + 31) / 32 * 32 + 16) * 64 <= 64 * 1024) {
+        const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
+        PpeFast pf;
+        pf.zp_out = t.zp_out;
+        const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
+        pf.lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin;
+        pf.hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
+        if (pf.lo > tmax) pf.lo = tmax;
+        if (pf.hi < tmin) pf.hi = tmin;
+        if (pf.lo > pf.hi) pf.lo = pf.hi;
+        void* ws = nullptr;
+        int rc = get_workspace(s, sizeof(ChanPrep) * (size_t)g.OC, &ws);
+        if (rc) return rc;
+        ChanPrep* prep = (ChanPrep*)ws;
+        hipLaunchKernelGGL(nce_fold_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s, (const int8_t*)t.weights,
+                           t.weight_table, prep, g.OC, Ktot, corr, ppe);
+        VPX_HIP_CHECK(hipGetLastError());
+        const size_t lds = (size_t)64 * ((Ktot + 31) / 32 * 32 + 16);
+        const dim3 grid((unsigned)((Mtot + 255) / 256), (unsigned)((g.OC + 63) / 64));
+        const int pad_byte = t.zp_in & 0xff;
+        if (in_u8) hipLaunchKernelGGL(nce_conv_mfma16<true>, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,
+                                      prep, (uint8_t*)t.output, g, pad_byte, pf);
+        else hipLaunchKernelGGL(nce_conv_mfma16<false>, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,
+                                prep, (uint8_t*)t.output, g, pad_byte, pf);
+        VPX_HIP_CHECK(hipGetLastError());
+        *kernel_name = "nce_conv_mfma16";
         return VPX_RESULT_SUCCESS;
     }
 
