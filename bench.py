@@ -25,8 +25,8 @@ METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
 # Bytes moved through L2 per step, from rocprofv3 FETCH_SIZE / WRITE_SIZE counters scaled by a plain
 # copy of known size (profiles/<workload>__*.md hold the runs these come from).
 MEASURED_TRAFFIC = {
-    "c1_fake_quantize": 880465, "c2_softmax": 134240024, "c3_mvn": 25450680, "c4_conv": 16426621,
-    "c5_matmul": 384896480, "c5_dequantize": 135343006, "c5_eltwise_add": 270488016,
+    "c1_fake_quantize": 871101, "c2_softmax": 134269999, "c3_mvn": 25451430, "c4_conv": 16264736,
+    "c5_matmul": 384962929, "c5_dequantize": 135336726, "c5_eltwise_add": 270546244,
 }
 
 
@@ -80,7 +80,7 @@ def make_c1(rt):
     def cpu(orc, frac):
         return lambda: orc.fake_quantize_f16(c["x"], c["in_lo"], c["in_hi"], c["out_lo"], c["out_hi"], 256), n * 4
     return Workload("c1_fake_quantize", "FakeQuantize fp16 NCHW [1,64,56,56], per-tensor, 256 levels, +-4",
-                    _prebuilt_sw_launch(rt, "fake_quantize", blob, ops), n * 4, 0, "hbm", "f16", "stream_kernel<FqFn>", cpu)
+                    _prebuilt_sw_launch(rt, "fake_quantize", blob, ops), n * 4, 0, "hbm", "f16", "stream_kernel<FqMap>", cpu)
 
 
 def make_c2(rt):
