@@ -170,7 +170,25 @@ def dequantize(q, scales, zps, to_f16=True, axis=None):
     return y
 
 
-ELT_OPS = {"add": 0, "sub": 1, "mul": 2, "min": 3, "max": 4, "div": 5}
+ELT_OPS = {"add": 0, "sub": 1, "mul": 2, "min": 3, "max": 4, "div": 5, "prelu": 6}
+
+ACT_OPS = {name: i for i, name in enumerate(
+    ["relu", "leaky_relu", "clamp", "negative", "abs", "hswish", "hsigmoid", "hardsigmoid", "sigmoid", "tanh", "exp",
+     "sqrt", "log", "floor", "ceil", "sign", "elu", "selu", "swish", "mish", "softplus", "gelu", "erf"])}
+
+
+def activation_f16(op, x, p0=0.0, p1=0.0):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    y = np.empty_like(x)
+    lib().orc_activation_f16(C.c_int(ACT_OPS[op]), C.c_float(p0), C.c_float(p1), _p(x), _p(y), C.c_int64(x.size))
+    return y
+
+
+def activation_f32(op, x, p0=0.0, p1=0.0):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty_like(x)
+    lib().orc_activation_f32(C.c_int(ACT_OPS[op]), C.c_float(p0), C.c_float(p1), _p(x), _p(y), C.c_int64(x.size))
+    return y
 
 
 def eltwise_f16(op, a, b):
@@ -219,6 +237,72 @@ def mvn_f16(x, across_channels, normalize_variance, eps, layout="NCHW"):
     lib().orc_mvn_f16(_p(x), _p(y), C.c_int64(N), C.c_int64(Cc), C.c_int64(H * W), C.c_int64(sn), C.c_int64(sc),
                       C.c_int64(ss), C.c_int(int(across_channels)), C.c_int(int(normalize_variance)), C.c_float(eps))
     return y
+
+
+# The three-step decomposition of MVN-1 (decompose_mvn.cpp:82-129; ops.td:3659-3845), in numpy.  Tensors are
+# logical [N,C,H,W] arrays; statistics tensors are in their memory order [N, parts, 2 or 1, C or 1].
+# "parity unpinned" like mvn_f16: the reference holds no vectors for these kernels.  Pinned by the tests through
+# hand-computed cases and through mvn1_norm(mvn1_mean_var(mvn1_sum(x))) == mvn_f16(x).
+
+def mvn1_sum(x_bits, across_channels, normalize_variance):
+    """{sum, sum of squares} per group, accumulated in double and rounded to float32; one part."""
+    x = f16_to_f32(np.asarray(x_bits, dtype=np.uint16)).astype(np.float64)
+    axes = (1, 2, 3) if across_channels else (2, 3)
+    terms = [x.sum(axis=axes)] + ([(x * x).sum(axis=axes)] if normalize_variance else [])
+    out = np.stack([t.reshape(x.shape[0], -1) for t in terms], axis=1)  # [N, W, C]
+    return out[:, None].astype(np.float32)
+
+
+def mvn1_mean_var(sums, orig_shape, across_channels, normalize_variance, eps, group_c=1, out_dtype=np.float32):
+    """sums: float32 [N, parts, 2 or 1, C or 1] -> {mean, 1/sqrt(var + eps)} [N, 1, 2 or 1, C or 1]; channels are
+    pooled in consecutive groups of group_c (the op's internal reshape)."""
+    s = np.asarray(sums, dtype=np.float32).astype(np.float64).sum(axis=1)  # [N, W, Cin]
+    N, Cc, H, W = orig_shape
+    if across_channels:
+        pooled = s.sum(axis=2, keepdims=True)
+        count = float(Cc * H * W)
+    else:
+        g = s.reshape(s.shape[0], s.shape[1], Cc // group_c, group_c).sum(axis=3, keepdims=True)
+        pooled = np.broadcast_to(g, g.shape[:3] + (group_c,)).reshape(s.shape[0], s.shape[1], Cc)
+        count = float(group_c * H * W)
+    mean = pooled[:, 0] / count
+    rows = [mean]
+    if normalize_variance:
+        var = np.maximum(pooled[:, 1] / count - mean * mean, 0.0)
+        with np.errstate(divide="ignore"):
+            rows.append(1.0 / np.sqrt(var + np.float64(np.float32(eps))))
+    out = np.stack(rows, axis=1)[:, None].astype(np.float32)
+    return out.astype(out_dtype)
+
+
+def mvn1_norm(x_bits, mean_var, across_channels, normalize_variance):
+    """(x - mean) * inv in float32, rounded to fp16 (IEEE); mean_var [N, 1, 2 or 1, C or 1] of fp16 or fp32."""
+    x = f16_to_f32(np.asarray(x_bits, dtype=np.uint16))
+    mv = np.asarray(mean_var).astype(np.float32)
+    mean = mv[:, 0, 0, :, None, None]
+    inv = mv[:, 0, 1, :, None, None] if normalize_variance else np.float32(1.0)
+    with np.errstate(all="ignore"):
+        return ((x - mean) * inv).astype(np.float32).astype(np.float16).view(np.uint16)
+
+
+def mvn6_f16(x_bits, axes, normalize_variance, eps, eps_mode, scale_bits=None, bias_bits=None):
+    """OpenVINO MVN-6 over `axes` of an array indexed in memory order: y = (x - mean) / sqrt(var + eps) (eps_mode 0,
+    INSIDE_SQRT) or (x - mean) / (sqrt(var) + eps) (1, OUTSIDE_SQRT), then the fused y * scale + bias with NUMPY
+    broadcast (fuse_mvn6_scale_bias.cpp); double statistics, one rounding to fp16 (IEEE)."""
+    x = f16_to_f32(np.asarray(x_bits, dtype=np.uint16)).astype(np.float64)
+    axes = tuple(int(a) % x.ndim for a in axes)
+    mean = x.mean(axis=axes, keepdims=True)
+    y = x - mean
+    if normalize_variance:
+        var = (y * y).mean(axis=axes, keepdims=True)
+        e = np.float64(np.float32(eps))
+        y = y / (np.sqrt(var + e) if eps_mode == 0 else np.sqrt(var) + e)
+    if scale_bits is not None:
+        y = y * f16_to_f32(np.asarray(scale_bits, dtype=np.uint16)).astype(np.float64)
+    if bias_bits is not None:
+        y = y + f16_to_f32(np.asarray(bias_bits, dtype=np.uint16)).astype(np.float64)
+    with np.errstate(all="ignore"):
+        return y.astype(np.float32).astype(np.float16).view(np.uint16)
 
 
 # ---- integer path --------------------------------------------------------------------------------

@@ -233,6 +233,7 @@ static float elt_apply(int op, float a, float b) {
     case ORC_ELT_MIN: return fminf(a, b);
     case ORC_ELT_MAX: return fmaxf(a, b);
     case ORC_ELT_DIV: return a / b;
+    case ORC_ELT_PRELU: return a < 0.0f ? a * b : a;
     default: return 0.0f;
     }
 }
@@ -250,6 +251,50 @@ void orc_eltwise_f16(int op, const uint16_t* a, const uint16_t* b, uint16_t* y, 
         const float fb = orc_f16_to_f32(b[bcast_offset(rank, idx, b_dims)]);
         y[i] = orc_f32_to_f16(elt_apply(op, fa, fb));
     }
+}
+
+/* ------------------------------------------------------------------ Activations */
+
+/* OpenVINO operator definitions of the unary VPU ops that lower to the activation kernels
+ * (src/vpux_compiler/src/dialect/VPUIP/IR/ops/sw_kernel.cpp:650-941, 1266-1285, 1689-1845);
+ * fp32 arithmetic, one rounding. */
+float orc_activation(int op, float x, float p0, float p1) {
+    switch (op) {
+    case ORC_ACT_RELU: return x > 0.0f ? x : 0.0f;
+    case ORC_ACT_LEAKY_RELU: return x < 0.0f ? x * p0 : x;
+    case ORC_ACT_CLAMP: return x < p0 ? p0 : (x > p1 ? p1 : x);
+    case ORC_ACT_NEGATIVE: return -x;
+    case ORC_ACT_ABS: return fabsf(x);
+    case ORC_ACT_HSWISH: return x * fminf(fmaxf(x + 3.0f, 0.0f), 6.0f) / 6.0f;
+    case ORC_ACT_HSIGMOID: return fminf(fmaxf(x + 3.0f, 0.0f), 6.0f) / 6.0f;
+    case ORC_ACT_HARDSIGMOID: return fmaxf(0.0f, fminf(1.0f, p0 * x + p1));
+    case ORC_ACT_SIGMOID: return 1.0f / (1.0f + expf(-x));
+    case ORC_ACT_TANH: return tanhf(x);
+    case ORC_ACT_EXP: return expf(x);
+    case ORC_ACT_SQRT: return sqrtf(x);
+    case ORC_ACT_LOG: return logf(x);
+    case ORC_ACT_FLOOR: return floorf(x);
+    case ORC_ACT_CEIL: return ceilf(x);
+    case ORC_ACT_SIGN: return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : x);
+    case ORC_ACT_ELU: return x < 0.0f ? p0 * (expf(x) - 1.0f) : x;
+    case ORC_ACT_SELU: return x > 0.0f ? p1 * x : p0 * p1 * (expf(x) - 1.0f);
+    case ORC_ACT_SWISH: return x / (1.0f + expf(-p0 * x));
+    case ORC_ACT_MISH: return x * tanhf(x < 20.0f ? log1pf(expf(x)) : x);
+    case ORC_ACT_SOFTPLUS: return x < 20.0f ? log1pf(expf(x)) : x;
+    case ORC_ACT_GELU: return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+    case ORC_ACT_ERF: return erff(x);
+    default: return 0.0f;
+    }
+}
+
+void orc_activation_f16(int op, float p0, float p1, const uint16_t* x, uint16_t* y, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) y[i] = orc_f32_to_f16(orc_activation(op, orc_f16_to_f32(x[i]), p0, p1));
+}
+
+void orc_activation_f32(int op, float p0, float p1, const float* x, float* y, int64_t n) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) y[i] = orc_activation(op, x[i], p0, p1);
 }
 
 /* ------------------------------------------------------------------ Softmax */

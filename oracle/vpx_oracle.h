@@ -63,7 +63,21 @@ void orc_dequantize_f32(const void* q, int in_is_signed, float* y, int64_t outer
                         const double* scales, const int64_t* zps);
 
 /* ---- Eltwise fp16 (float16.hpp:123-126: fp32 op then RNE) ---- */
-enum { ORC_ELT_ADD = 0, ORC_ELT_SUB = 1, ORC_ELT_MUL = 2, ORC_ELT_MIN = 3, ORC_ELT_MAX = 4, ORC_ELT_DIV = 5 };
+enum { ORC_ELT_ADD = 0, ORC_ELT_SUB = 1, ORC_ELT_MUL = 2, ORC_ELT_MIN = 3, ORC_ELT_MAX = 4, ORC_ELT_DIV = 5,
+       ORC_ELT_PRELU = 6 /* a < 0 ? a * b : a */ };
+
+/* Unary activations (OpenVINO operator definitions; p0, p1 = the op's float attributes in the
+ * order the compiler serialises them).  "parity unpinned" against the SHAVE kernels, whose sources
+ * are not public; pinned by special values and an independent fp64 evaluation in the tests. */
+enum {
+    ORC_ACT_RELU = 0, ORC_ACT_LEAKY_RELU, ORC_ACT_CLAMP, ORC_ACT_NEGATIVE, ORC_ACT_ABS, ORC_ACT_HSWISH,
+    ORC_ACT_HSIGMOID, ORC_ACT_HARDSIGMOID, ORC_ACT_SIGMOID, ORC_ACT_TANH, ORC_ACT_EXP, ORC_ACT_SQRT,
+    ORC_ACT_LOG, ORC_ACT_FLOOR, ORC_ACT_CEIL, ORC_ACT_SIGN, ORC_ACT_ELU, ORC_ACT_SELU, ORC_ACT_SWISH,
+    ORC_ACT_MISH, ORC_ACT_SOFTPLUS, ORC_ACT_GELU, ORC_ACT_ERF
+};
+float orc_activation(int op, float x, float p0, float p1);
+void orc_activation_f16(int op, float p0, float p1, const uint16_t* x, uint16_t* y, int64_t n);
+void orc_activation_f32(int op, float p0, float p1, const float* x, float* y, int64_t n);
 /* NUMPY broadcast: a_dims/b_dims entries are 1 or dims[] */
 void orc_eltwise_f16(int op, const uint16_t* a, const uint16_t* b, uint16_t* y, int rank, const int64_t* dims,
                      const int64_t* a_dims, const int64_t* b_dims);

@@ -148,6 +148,86 @@ def test_eltwise_add_f32(rt, dev):
     assert np.array_equal(out.cpu().numpy(), a + b)
 
 
+# ---------------------------------------------------------------------------------- activations
+
+def _act_cases():
+    from test_oracle import ACT_CASES
+    return ACT_CASES
+
+
+@pytest.mark.parametrize("op,params", _act_cases(), ids=[c[0] for c in _act_cases()])
+def test_activation_every_f16_value_and_f32(rt, orc, dev, op, params):
+    """Piecewise-linear activations bit-exact; the ones built on exp / tanh / log / erf within one fp16
+    step (device and host libm differ in the last fp32 bits), outside the range below 2^-14 where the
+    float16 class's own rounding can double such a difference."""
+    import torch
+    from test_oracle import ACT_EXACT, f16_ulp_distance
+    h = np.tile(np.arange(65536, dtype=np.uint16), 5)[:300_001]  # ragged tail, every value several times
+    x = to_dev(h, dev, True)
+    out = torch.empty_like(x)
+    rt.activation(op, x, out, *params)
+    got, want = f16_bits(out), orc.activation_f16(op, h, *params)
+    nan = is_nan16(want)
+    if op in ACT_EXACT:
+        assert_f16_exact(got, want, op)
+    else:
+        assert np.array_equal(is_nan16(got), nan), op
+        with np.errstate(invalid="ignore"):
+            w = np.abs(orc.f16_to_f32(want).astype(np.float64))
+        check = ~nan & (w >= 2.0 ** -14)
+        d = f16_ulp_distance(got[check], want[check])
+        assert d.max() <= 1, (op, d.max(), hex(h[check][np.argmax(d)]))
+        tiny = ~nan & ~check
+        assert np.all(np.abs(orc.f16_to_f32(got[tiny])) <= 2.0 ** -13), op
+    # fp32 tensors
+    rng = np.random.default_rng(31)
+    xf = np.concatenate([rng.normal(0, 3, 70_001), rng.uniform(-12, 12, 30_000), [0.0, -0.0, 1.0, -1.0]]).astype(np.float32)
+    of = torch.empty(xf.shape, dtype=torch.float32, device=dev)
+    rt.activation(op, to_dev(xf, dev), of, *params)
+    gf, wf = of.cpu().numpy(), orc.activation_f32(op, xf, *params)
+    if op in ACT_EXACT:
+        ok = ~np.isnan(wf)
+        assert np.array_equal(np.isnan(gf), np.isnan(wf)) and np.array_equal(gf[ok].view(np.uint32), wf[ok].view(np.uint32)), op
+    else:
+        assert np.allclose(gf, wf, rtol=3e-6, atol=3e-7, equal_nan=True), (op, np.nanmax(np.abs(gf - wf)))
+
+
+def test_activation_4d_views_and_errors(rt, orc, dev):
+    import torch
+    rng = np.random.default_rng(32)
+    a = orc.f32_to_f16(rng.normal(0, 2, (2, 6, 5, 8)).astype(np.float32))
+    big = to_dev(a, dev, True)
+    out = torch.zeros_like(big)
+    rt.activation("leaky_relu", big[:, 1:4], out[:, 2:5], 0.1)
+    want = np.zeros_like(a)
+    want[:, 2:5] = orc.activation_f16("leaky_relu", np.ascontiguousarray(a[:, 1:4]), 0.1)
+    assert_f16_exact(f16_bits(out), want, "strided views")
+    nhwc = big.permute(0, 2, 3, 1).contiguous().permute(0, 3, 1, 2)
+    o2 = torch.empty_like(nhwc)
+    rt.activation("clamp", nhwc, o2, -1.0, 1.0, order="NHWC")
+    assert_f16_exact(f16_bits(o2.contiguous()), orc.activation_f16("clamp", a, -1.0, 1.0), "NHWC")
+    with pytest.raises(rt.VpxError) as e:
+        rt.activation("clamp", big, out, 2.0, 1.0)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    with pytest.raises(rt.VpxError) as e:
+        rt.activation("relu", big, torch.empty((2, 6, 5, 8), dtype=torch.float32, device=dev))
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    rt.activation("relu", torch.empty((0, 4), dtype=torch.float16, device=dev), torch.empty((0, 4), dtype=torch.float16, device=dev))
+
+
+def test_prelu_per_channel_slope(rt, orc, dev):
+    import torch
+    rng = np.random.default_rng(33)
+    a = orc.f32_to_f16(rng.normal(0, 2, (3, 16, 9, 24)).astype(np.float32))
+    slope = orc.f32_to_f16(rng.uniform(0.01, 0.5, (1, 16, 1, 1)).astype(np.float32))
+    out = torch.empty((3, 16, 9, 24), dtype=torch.float16, device=dev)
+    rt.prelu(to_dev(a, dev, True), to_dev(slope, dev, True), out)
+    assert_f16_exact(f16_bits(out), orc.eltwise_f16("prelu", a, slope), "per-channel slope")
+    one = orc.f32_to_f16(np.full((1, 1, 1, 1), 0.25, np.float32))
+    rt.prelu(to_dev(a, dev, True), to_dev(one, dev, True), out)
+    assert_f16_exact(f16_bits(out), orc.activation_f16("leaky_relu", a, 0.25), "scalar slope equals leaky relu")
+
+
 # ---------------------------------------------------------------------------------- fake_quantize
 
 def _run_fq(rt, dev, c, order=None):
@@ -265,6 +345,189 @@ def test_quantize_per_axis_ambiguous_axis_is_refused(rt, dev):
     assert e.value.code == rt.ERROR_INVALID_ARGUMENT
     with pytest.raises(rt.VpxError):
         rt.quantize(x, torch.empty((4, 2, 4), dtype=torch.int8, device=dev), [0.1] * 3, [0] * 3)  # no dimension of size 3
+
+
+# ---------------------------------------------------------------------------------- MVN decomposition
+
+def _mvn_input(orc, rng, shape):
+    x = rng.uniform(-8, 8, shape) + rng.normal(0, 2, (1, shape[1], 1, 1))
+    return orc.f32_to_f16(x.astype(np.float32))
+
+
+def _to_layout(a, layout):
+    """logical NCHW numpy array -> array in the layout's memory order"""
+    return a if layout == "NCHW" else np.ascontiguousarray(a.transpose(0, 2, 3, 1))
+
+
+@pytest.mark.parametrize("layout", ["NCHW", "NHWC"])
+@pytest.mark.parametrize("across", [False, True])
+@pytest.mark.parametrize("shape,parts", [((2, 5, 9, 7), 1), ((1, 64, 56, 56), 1), ((3, 40, 33, 31), 3), ((1, 16, 128, 96), 2)])
+def test_mvn1_sum(rt, orc, dev, layout, across, shape, parts):
+    import torch
+    rng = np.random.default_rng(51)
+    x = _mvn_input(orc, rng, shape)
+    xm = to_dev(_to_layout(x, layout), dev, True)
+    for nv in (True, False):
+        out_c, out_w = (1 if across else shape[1]), (2 if nv else 1)
+        out = torch.full((shape[0], parts, out_w, out_c), float("nan"), dtype=torch.float32, device=dev)
+        rt.mvn1_sum(xm, out, across, nv, order=layout)
+        got = out.cpu().numpy().astype(np.float64)
+        want = orc.mvn1_sum(x, across, nv).astype(np.float64)
+        assert not np.isnan(got).any()
+        # fp32 accumulation in a fixed tree against double: relative to the sum of magnitudes
+        xf = np.abs(orc.f16_to_f32(x).astype(np.float64))
+        axes = (1, 2, 3) if across else (2, 3)
+        scale = np.stack([xf.sum(axis=axes).reshape(shape[0], -1)] + ([(xf * xf).sum(axis=axes).reshape(shape[0], -1)] if nv else []), axis=1)
+        assert np.all(np.abs(got.sum(axis=1) - want[:, 0]) <= 2e-6 * scale), (layout, across, nv)
+
+
+@pytest.mark.parametrize("out_dtype", ["float32", "float16"])
+def test_mvn1_mean_var(rt, orc, dev, out_dtype):
+    import torch
+    rng = np.random.default_rng(52)
+    tdt = getattr(torch, out_dtype)
+    ndt = getattr(np, out_dtype)
+    for (N, Cc, H, W), across, parts, group_c in (((2, 12, 9, 7), False, 1, 1), ((2, 12, 9, 7), True, 4, 1),
+                                                   ((3, 12, 5, 5), False, 2, 4), ((1, 300, 8, 8), False, 3, 1)):
+        x = rng.normal(0.5, 2, (N, Cc, H, W))
+        c_in = 1 if across else Cc
+        axes = (1, 2, 3) if across else (2, 3)
+        total = np.stack([x.sum(axis=axes).reshape(N, c_in), (x * x).sum(axis=axes).reshape(N, c_in)], axis=1)  # [N, 2, Cin]
+        w = rng.dirichlet(np.ones(parts), size=(N, 2, c_in)).transpose(0, 3, 1, 2)  # split every sum into parts
+        sums = (total[:, None] * w).astype(np.float32)
+        for nv in (True, False):
+            out = torch.empty((N, 1, 2 if nv else 1, c_in if across else Cc), dtype=tdt, device=dev)
+            rt.mvn1_mean_var(to_dev(sums[:, :, :2 if nv else 1].copy(), dev), out, (N, Cc, H, W), across, nv, 1e-6, group_c)
+            got = out.cpu().numpy().astype(np.float64)
+            want = orc.mvn1_mean_var(sums[:, :, :2 if nv else 1], (N, Cc, H, W), across, nv, 1e-6, group_c, ndt).astype(np.float64)
+            tol = 2e-6 if out_dtype == "float32" else 1e-3
+            assert np.all(np.abs(got - want) <= tol * np.abs(want) + 1e-7), (across, nv, group_c)
+
+
+@pytest.mark.parametrize("layout", ["NCHW", "NHWC"])
+@pytest.mark.parametrize("across", [False, True])
+@pytest.mark.parametrize("stat_dtype", ["float32", "float16"])
+def test_mvn1_norm_exact(rt, orc, dev, layout, across, stat_dtype):
+    import torch
+    rng = np.random.default_rng(53)
+    for shape in ((2, 5, 9, 7), (2, 24, 16, 40), (1, 3, 64, 100)):
+        x = _mvn_input(orc, rng, shape)
+        xm = to_dev(_to_layout(x, layout), dev, True)
+        for nv in (True, False):
+            c = 1 if across else shape[1]
+            mv = np.stack([rng.normal(0, 2, (shape[0], c))] + ([rng.uniform(0.1, 3, (shape[0], c))] if nv else []), axis=1)[:, None]
+            mv = mv.astype(getattr(np, stat_dtype))
+            out = torch.empty_like(xm)
+            rt.mvn1_norm(xm, to_dev(mv, dev), out, across, nv, order=layout)
+            want = _to_layout(orc.mvn1_norm(x, mv, across, nv), layout)
+            assert_f16_exact(f16_bits(out), want, "%s %s %s" % (layout, across, nv))
+
+
+@pytest.mark.parametrize("layout", ["NCHW", "NHWC"])
+@pytest.mark.parametrize("across", [False, True])
+def test_mvn1_three_steps_match_the_single_kernel(rt, orc, dev, layout, across):
+    import torch
+    rng = np.random.default_rng(54)
+    shape = (2, 32, 48, 40)
+    x = _mvn_input(orc, rng, shape)
+    xm = to_dev(_to_layout(x, layout), dev, True)
+    c = 1 if across else shape[1]
+    sums = torch.empty((shape[0], 2, 2, c), dtype=torch.float32, device=dev)
+    mv = torch.empty((shape[0], 1, 2, c), dtype=torch.float32, device=dev)
+    out = torch.empty_like(xm)
+    rt.mvn1_sum(xm, sums, across, True, order=layout)
+    rt.mvn1_mean_var(sums, mv, shape, across, True, 1e-9)
+    rt.mvn1_norm(xm, mv, out, across, True, order=layout)
+    want = _to_layout(orc.mvn_f16(x, across, True, 1e-9), layout)
+    # values next to zero carry the absolute error of the fp32 mean (x - mean cancels): absolute floor
+    _assert_mvn6_close(f16_bits(out), want, orc, "three steps vs oracle mvn")
+    single = torch.empty_like(xm)
+    rt.mvn(xm, single, across, True, 1e-9, order=layout)
+    _assert_mvn6_close(f16_bits(out), f16_bits(single), orc, "three steps vs mvn1 kernel")
+
+
+def test_mvn1_decomposition_errors(rt, dev):
+    import torch
+    x = torch.zeros((2, 4, 8, 8), dtype=torch.float16, device=dev)
+    with pytest.raises(rt.VpxError) as e:
+        rt.mvn1_sum(x, torch.empty((2, 1, 2, 3), dtype=torch.float32, device=dev), False, True)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    with pytest.raises(rt.VpxError) as e:
+        rt.mvn1_sum(x, torch.empty((2, 1, 2, 4), dtype=torch.float16, device=dev), False, True)
+    assert e.value.code == rt.ERROR_UNSUPPORTED_FEATURE
+    with pytest.raises(rt.VpxError) as e:
+        rt.mvn1_mean_var(torch.zeros((2, 1, 2, 4), dtype=torch.float32, device=dev),
+                         torch.empty((2, 1, 2, 4), dtype=torch.float32, device=dev), (2, 4, 8, 8), False, True, 1e-6, group_c=3)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    with pytest.raises(rt.VpxError) as e:
+        rt.mvn1_norm(x, torch.zeros((2, 1, 2, 1), dtype=torch.float32, device=dev), torch.empty_like(x), False, True)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+
+
+# ---------------------------------------------------------------------------------- MVN-6
+
+def _assert_mvn6_close(got_bits, want_bits, orc, what):
+    g = orc.f16_to_f32(got_bits).astype(np.float64)
+    w = orc.f16_to_f32(want_bits).astype(np.float64)
+    bad = np.argwhere(~(np.abs(g - w) <= REL_TOL * np.abs(w) + 2e-5))
+    assert len(bad) == 0, "%s: %d outside tolerance, first %s got %r want %r" % (what, len(bad), bad[0], g[tuple(bad[0])], w[tuple(bad[0])])
+
+
+MVN6_CASES = [
+    # shape, axes, scale shape, bias shape
+    ((8, 128, 768), (2,), (1, 1, 768), (1, 1, 768)),      # LayerNorm, one wavefront per row
+    ((4, 77, 512), (-1,), None, None),
+    ((4, 16, 2048), (2,), (1, 1, 2048), None),            # one workgroup per row
+    ((2, 8, 8192), (2,), None, (1, 1, 8192)),
+    ((2, 6, 4096), (2,), (1, 6, 1), (2, 6, 4096)),        # scale constant along the row, bias of full shape
+    ((3, 5, 16, 24), (2, 3), (1, 1, 16, 24), (1, 5, 1, 1)),  # two innermost axes
+    ((5, 7, 30), (2,), (1, 1, 30), (1, 1, 30)),           # row not a multiple of 8: generic
+    ((4, 6, 10), (1,), (1, 6, 1), None),                  # middle axis: generic
+    ((2, 3, 4, 5), (1, 3), (1, 3, 1, 5), (1, 1, 1, 5)),   # split axes
+    ((2, 20000), (1,), None, None),                       # long row
+    ((6, 1, 64), (1, 2), None, None),                     # unit dimension among the axes
+]
+
+
+@pytest.mark.parametrize("shape,axes,sc_shape,bi_shape", MVN6_CASES, ids=[str(c[0]) + str(c[1]) for c in MVN6_CASES])
+def test_mvn6(rt, orc, dev, shape, axes, sc_shape, bi_shape):
+    import torch
+    rng = np.random.default_rng(55)
+    x = orc.f32_to_f16(rng.normal(0.5, 2, shape).astype(np.float32))
+    sc = orc.f32_to_f16(rng.uniform(0.5, 2, sc_shape).astype(np.float32)) if sc_shape else None
+    bi = orc.f32_to_f16(rng.normal(0, 1, bi_shape).astype(np.float32)) if bi_shape else None
+    xd = to_dev(x, dev, True)
+    for nv, eps, mode in ((True, 1e-5, 0), (True, 1e-2, 1), (False, 0.0, 0)):
+        out = torch.empty_like(xd)
+        rt.mvn6(xd, out, axes, nv, eps, mode, scale=None if sc is None else to_dev(sc, dev, True),
+                bias=None if bi is None else to_dev(bi, dev, True))
+        _assert_mvn6_close(f16_bits(out), orc.mvn6_f16(x, axes, nv, eps, mode, sc, bi), orc, "%s nv=%s mode=%d" % (shape, nv, mode))
+
+
+def test_mvn6_strided_rows_and_errors(rt, orc, dev):
+    import torch
+    rng = np.random.default_rng(56)
+    x = orc.f32_to_f16(rng.normal(0, 2, (4, 10, 256)).astype(np.float32))
+    xd = to_dev(x, dev, True)
+    out = torch.zeros_like(xd)
+    rt.mvn6(xd[:, 2:7], out[:, 3:8], (2,), True, 1e-5, 0)  # rows keep their alignment, outer strides differ
+    want = np.zeros_like(x)
+    want[:, 3:8] = orc.mvn6_f16(np.ascontiguousarray(x[:, 2:7]), (2,), True, 1e-5, 0)
+    _assert_mvn6_close(f16_bits(out), want, orc, "row views")
+    out.zero_()
+    rt.mvn6(xd[:, :, 3:131], out[:, :, 5:133], (2,), True, 1e-5, 0)  # misaligned rows: generic kernel
+    want = np.zeros_like(x)
+    want[:, :, 5:133] = orc.mvn6_f16(np.ascontiguousarray(x[:, :, 3:131]), (2,), True, 1e-5, 0)
+    _assert_mvn6_close(f16_bits(out), want, orc, "misaligned views")
+    with pytest.raises(rt.VpxError) as e:
+        rt.mvn6(xd, out, (2, 2), True, 1e-5, 0)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    with pytest.raises(rt.VpxError) as e:
+        rt.mvn6(xd, out, (2,), True, 1e-5, 0, scale=torch.ones((1, 1, 7), dtype=torch.float16, device=dev))
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    with pytest.raises(rt.VpxError) as e:
+        rt.mvn6(xd, out, (2,), True, 1e-5, 2)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
 
 
 # ---------------------------------------------------------------------------------- softmax

@@ -384,3 +384,149 @@ def test_nce_eltwise_against_exact_integers_and_real_arithmetic(orc):
         assert np.array_equal(got, want)
         unsat = (real > 1) & (real < 254)
         assert np.abs(got[unsat].astype(np.float64) - real[unsat]).max() <= 1.0
+
+
+# ---------------------------------------------------------------------------------- activations
+
+def _activation_fp64(op, x, p0, p1):
+    """Independent evaluation in fp64 with numpy / scipy (not a retyping of the oracle's branches where a
+    smooth closed form exists)."""
+    from scipy import special
+    x = x.astype(np.float64)
+    with np.errstate(all="ignore"):
+        return {
+            "relu": lambda: np.maximum(x, 0.0),
+            "leaky_relu": lambda: np.where(x < 0, x * np.float64(np.float32(p0)), x),
+            "clamp": lambda: np.clip(x, np.float32(p0), np.float32(p1)),
+            "negative": lambda: -x,
+            "abs": lambda: np.abs(x),
+            "hswish": lambda: x * np.clip(x + 3.0, 0.0, 6.0) / 6.0,
+            "hsigmoid": lambda: np.clip(x + 3.0, 0.0, 6.0) / 6.0,
+            "hardsigmoid": lambda: np.clip(np.float64(np.float32(p0)) * x + np.float64(np.float32(p1)), 0.0, 1.0),
+            "sigmoid": lambda: special.expit(x),
+            "tanh": lambda: np.tanh(x),
+            "exp": lambda: np.exp(x),
+            "sqrt": lambda: np.sqrt(x),
+            "log": lambda: np.log(x),
+            "floor": lambda: np.floor(x),
+            "ceil": lambda: np.ceil(x),
+            "sign": lambda: np.sign(x),
+            "elu": lambda: np.where(x < 0, np.float64(np.float32(p0)) * np.expm1(x), x),
+            "selu": lambda: np.float64(np.float32(p1)) * np.where(x > 0, x, np.float64(np.float32(p0)) * np.expm1(x)),
+            "swish": lambda: x * special.expit(np.float64(np.float32(p0)) * x),
+            "mish": lambda: x * np.tanh(np.logaddexp(0.0, x)),
+            "softplus": lambda: np.logaddexp(0.0, x),
+            "gelu": lambda: x * special.ndtr(x),
+            "erf": lambda: special.erf(x),
+        }[op]()
+
+
+ACT_CASES = [("relu", ()), ("leaky_relu", (0.1,)), ("clamp", (-1.5, 6.0)), ("negative", ()), ("abs", ()), ("hswish", ()),
+             ("hsigmoid", ()), ("hardsigmoid", (0.2, 0.5)), ("sigmoid", ()), ("tanh", ()), ("exp", ()), ("sqrt", ()),
+             ("log", ()), ("floor", ()), ("ceil", ()), ("sign", ()), ("elu", (1.0,)), ("selu", (1.67326, 1.0507)),
+             ("swish", (1.0,)), ("mish", ()), ("softplus", ()), ("gelu", ()), ("erf", ())]
+ACT_EXACT = {"relu", "leaky_relu", "clamp", "negative", "abs", "hsigmoid", "hardsigmoid", "floor", "ceil", "sign", "sqrt"}
+
+
+def f16_ulp_distance(a_bits, b_bits):
+    """Distance in representable fp16 values (sign-magnitude folded onto a line)."""
+    def line(b):
+        b = b.astype(np.int32)
+        return np.where(b & 0x8000, -(b & 0x7fff), b & 0x7fff)
+    return np.abs(line(a_bits) - line(b_bits))
+
+
+@pytest.mark.parametrize("op,params", ACT_CASES, ids=[c[0] for c in ACT_CASES])
+def test_activation_every_f16_value_against_fp64(orc, op, params):
+    h = np.arange(65536, dtype=np.uint16)
+    h = h[(h & 0x7fff) <= 0x7c00]  # drop NaNs
+    p = tuple(params) + (0.0,) * (2 - len(params))
+    got = orc.activation_f16(op, h, *p)
+    x = orc.f16_to_f32(h)
+    want64 = _activation_fp64(op, x, *p)
+    # the fp64 result narrowed fp64 -> fp32 -> fp16 with the float16 class's own rounding (pinned by the
+    # float16 tests above), so only the activation arithmetic is under test here
+    with np.errstate(all="ignore"):
+        want = orc.f32_to_f16(want64.astype(np.float32))
+    nan = np.isnan(want64)
+    assert np.array_equal(((got & 0x7fff) > 0x7c00), nan)
+    ok = ~nan
+    d = f16_ulp_distance(got[ok], want[ok])
+    # one step where fp32 arithmetic and the fp64 evaluation fall on different sides of a rounding
+    # boundary; below 2^-14 the float16 class doubles some magnitudes (float16.cpp:74-107), which turns
+    # such a difference into a factor of two there
+    tiny = np.abs(want64[ok]) < 2.0 ** -14
+    if op in ACT_EXACT:
+        assert d.max() == 0, (op, d.max())
+    assert d[~tiny].max() <= 1, (op, d[~tiny].max(), h[ok][~tiny][np.argmax(d[~tiny])])
+
+
+def test_activation_special_values(orc):
+    f = lambda v: orc.f32_to_f16(np.asarray(v, dtype=np.float32))
+    val = lambda op, v, *p: orc.f16_to_f32(orc.activation_f16(op, f(v), *p))
+    assert val("relu", [-1.0, -0.0, 0.0, 2.5]).tolist() == [0.0, 0.0, 0.0, 2.5]
+    assert val("clamp", [-9.0, 0.25, 9.0], -1.0, 6.0).tolist() == [-1.0, 0.25, 6.0]
+    assert val("leaky_relu", [-2.0, 3.0], 0.25).tolist() == [-0.5, 3.0]
+    assert val("hswish", [-3.0, 0.0, 3.0, 6.0]).tolist() == [0.0, 0.0, 3.0, 6.0]
+    assert val("hsigmoid", [-3.0, 0.0, 3.0]).tolist() == [0.0, 0.5, 1.0]
+    assert val("sigmoid", [0.0]).tolist() == [0.5]
+    assert val("exp", [0.0]).tolist() == [1.0]
+    assert val("tanh", [0.0]).tolist() == [0.0]
+    assert val("sign", [-4.0, 0.0, 7.0]).tolist() == [-1.0, 0.0, 1.0]
+    assert val("erf", [0.0]).tolist() == [0.0]
+    assert val("softplus", [0.0])[0] == np.float32(np.float16(np.log(2.0)))
+    # prelu is the binary form of leaky relu
+    a = f([-2.0, 3.0, -8.0])
+    b = f([0.25, 0.25, 0.5])
+    assert orc.f16_to_f32(orc.eltwise_f16("prelu", a, b)).tolist() == [-0.5, 3.0, -4.0]
+
+
+# ---------------------------------------------------------------------------------- MVN decomposition, MVN-6
+
+def test_mvn1_decomposition_hand_case_and_chain(orc):
+    x = orc.f32_to_f16(np.array([1, 2, 3, 4, 10, 10, 10, 10], np.float32).reshape(1, 2, 2, 2))
+    s = orc.mvn1_sum(x, False, True)
+    assert s.shape == (1, 1, 2, 2) and s[0, 0].tolist() == [[10.0, 40.0], [30.0, 400.0]]
+    assert orc.mvn1_sum(x, True, False)[0, 0].tolist() == [[50.0]]
+    mv = orc.mvn1_mean_var(s, (1, 2, 2, 2), False, True, 0.0)
+    assert mv[0, 0, 0].tolist() == [2.5, 10.0]
+    assert mv[0, 0, 1, 0] == np.float32(1.0 / np.sqrt(1.25)) and np.isinf(mv[0, 0, 1, 1])
+    mv = orc.mvn1_mean_var(s, (1, 2, 2, 2), False, True, 1e-2)
+    y = orc.f16_to_f32(orc.mvn1_norm(x, mv, False, True))
+    assert np.allclose(y[0, 0].ravel(), (np.array([1, 2, 3, 4]) - 2.5) / np.sqrt(1.25 + 1e-2), rtol=1e-3)
+    assert np.all(y[0, 1] == 0)
+    # pooled channel groups: two channels of one group share the statistics of their union
+    mvg = orc.mvn1_mean_var(s, (1, 2, 2, 2), False, True, 0.0, group_c=2)
+    assert mvg[0, 0, 0].tolist() == [6.25, 6.25]
+    assert np.allclose(mvg[0, 0, 1], 1.0 / np.sqrt(430.0 / 8 - 6.25 ** 2))
+    # partial sums split over parts add up
+    two = np.concatenate([0.25 * s, 0.75 * s], axis=1)
+    assert np.array_equal(orc.mvn1_mean_var(two, (1, 2, 2, 2), False, True, 1e-2), orc.mvn1_mean_var(s, (1, 2, 2, 2), False, True, 1e-2))
+    # the three steps reproduce the one-kernel MVN (two-pass, double) on random data
+    rng = np.random.default_rng(41)
+    xr = orc.f32_to_f16((rng.normal(0, 2, (2, 5, 9, 7)) + rng.normal(0, 3, (1, 5, 1, 1))).astype(np.float32))
+    for across in (False, True):
+        for nv in (False, True):
+            mv = orc.mvn1_mean_var(orc.mvn1_sum(xr, across, nv), xr.shape, across, nv, 1e-9)
+            got = orc.f16_to_f32(orc.mvn1_norm(xr, mv, across, nv)).astype(np.float64)
+            want = orc.f16_to_f32(orc.mvn_f16(xr, across, nv, 1e-9)).astype(np.float64)
+            assert np.all(np.abs(got - want) <= 2e-3 * np.abs(want) + 1e-5), (across, nv)
+
+
+def test_mvn6_against_mvn1_and_hand_cases(orc):
+    rng = np.random.default_rng(42)
+    x = orc.f32_to_f16(rng.normal(1, 2, (2, 5, 9, 7)).astype(np.float32))
+    for axes, across in (((1, 2, 3), True), ((2, 3), False)):
+        got = orc.f16_to_f32(orc.mvn6_f16(x, axes, True, 1e-6, 0)).astype(np.float64)
+        want = orc.f16_to_f32(orc.mvn_f16(x, across, True, 1e-6)).astype(np.float64)
+        assert np.all(np.abs(got - want) <= 1e-3 * np.abs(want) + 1e-6)
+    row = orc.f32_to_f16(np.array([[1, 2, 3, 4]], np.float32))
+    inside = orc.f16_to_f32(orc.mvn6_f16(row, (1,), True, 0.75, 0))[0]
+    outside = orc.f16_to_f32(orc.mvn6_f16(row, (1,), True, 0.75, 1))[0]
+    assert np.allclose(inside, (np.array([1, 2, 3, 4]) - 2.5) / np.sqrt(2.0), rtol=1e-3)          # var 1.25 + 0.75
+    assert np.allclose(outside, (np.array([1, 2, 3, 4]) - 2.5) / (np.sqrt(1.25) + 0.75), rtol=1e-3)
+    assert orc.f16_to_f32(orc.mvn6_f16(row, (1,), False, 0.75, 0))[0].tolist() == [-1.5, -0.5, 0.5, 1.5]
+    sc = orc.f32_to_f16(np.array([[2, 2, 0, -1]], np.float32))
+    bi = orc.f32_to_f16(np.array([[1]], np.float32))
+    assert orc.f16_to_f32(orc.mvn6_f16(row, (1,), False, 0.0, 0, sc, bi))[0].tolist() == [-2.0, 0.0, 1.0, -0.5]
+

@@ -301,9 +301,10 @@ struct Entry {
     int n_in, n_out;
     int kind;  // dispatch tag
     int op;
+    int n_float_attrs;  // K_ACT: 32-bit float attributes that follow the memrefs
 };
 
-enum { K_CONVERT, K_ELTWISE, K_FQ, K_QUANT, K_DEQUANT, K_MVN, K_SOFTMAX };
+enum { K_CONVERT, K_ELTWISE, K_FQ, K_QUANT, K_DEQUANT, K_MVN, K_SOFTMAX, K_ACT, K_MVN_SUM, K_MVN_MEAN_VAR, K_MVN_NORM, K_MVN6 };
 
 const Entry kEntries[] = {
         {"convert", 1, 1, K_CONVERT, 0},
@@ -317,8 +318,37 @@ const Entry kEntries[] = {
         {"quantize", 1, 1, K_QUANT, 0},
         {"dequantize", 1, 1, K_DEQUANT, 0},
         {"mvn1", 1, 1, K_MVN, 0},
+        {"mvn1_sum", 1, 1, K_MVN_SUM, 0},
+        {"mvn1_mean_var", 1, 1, K_MVN_MEAN_VAR, 0},
+        {"mvn1_norm", 2, 1, K_MVN_NORM, 0},
+        {"mvn6", -1, 1, K_MVN6, 0},  // input, optional scale, optional bias; the memref list ends at an INT64_MIN word
         {"softmax", 1, 1, K_SOFTMAX, 0},
         {"softmaxFp32", 1, 1, K_SOFTMAX, 0},
+        // activations (sw_kernel.cpp:650-941, 1266-1285, 1689-1845); float attributes in serialisation order
+        {"prelu_fp16", 2, 1, K_ELTWISE, ELT_PRELU},
+        {"activation_relu", 1, 1, K_ACT, ACT_RELU, 0},
+        {"leaky_relu_fp16", 1, 1, K_ACT, ACT_LEAKY_RELU, 1},
+        {"activation_clamp", 1, 1, K_ACT, ACT_CLAMP, 2},
+        {"activation_negative", 1, 1, K_ACT, ACT_NEGATIVE, 0},
+        {"activation_abs", 1, 1, K_ACT, ACT_ABS, 0},
+        {"activation_hswish", 1, 1, K_ACT, ACT_HSWISH, 0},
+        {"activation_hsigmoid", 1, 1, K_ACT, ACT_HSIGMOID, 0},
+        {"activation_hardsigmoid", 1, 1, K_ACT, ACT_HARDSIGMOID, 2},
+        {"activation_sigmoid", 1, 1, K_ACT, ACT_SIGMOID, 0},
+        {"activation_tanh", 1, 1, K_ACT, ACT_TANH, 0},
+        {"activation_exp", 1, 1, K_ACT, ACT_EXP, 0},
+        {"activation_sqrt", 1, 1, K_ACT, ACT_SQRT, 0},
+        {"activation_log", 1, 1, K_ACT, ACT_LOG, 0},
+        {"activation_floor", 1, 1, K_ACT, ACT_FLOOR, 0},
+        {"activation_ceil", 1, 1, K_ACT, ACT_CEIL, 0},
+        {"activation_sign", 1, 1, K_ACT, ACT_SIGN, 0},
+        {"activation_elu", 1, 1, K_ACT, ACT_ELU, 1},
+        {"activation_selu", 1, 1, K_ACT, ACT_SELU, 2},
+        {"activation_swish", 1, 1, K_ACT, ACT_SWISH, 1},
+        {"activation_mish", 1, 1, K_ACT, ACT_MISH, 0},
+        {"activation_softplus", 1, 1, K_ACT, ACT_SOFTPLUS, 0},
+        {"activation_gelu", 1, 1, K_ACT, ACT_GELU, 0},
+        {"activation_erf", 1, 1, K_ACT, ACT_ERF, 0},
 };
 constexpr uint32_t kNumEntries = sizeof(kEntries) / sizeof(kEntries[0]);
 
@@ -366,7 +396,21 @@ int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_si
     const Entry* e = find_entry(entry);
     VPX_REQUIRE(e != nullptr, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "software kernel '%s' is not implemented", entry);
     Args a;
-    int rc = parse_blob(entry, e->n_in, e->n_out, params, params_size, addrs, num_addrs, a);
+    int n_in = e->n_in;
+    if (n_in < 0) {
+        // optional operands: count MemRefData records up to the marker word (sw_kernel.cpp:164-185)
+        int n_mem = 0;
+        int64_t head = 0;
+        while ((size_t)(n_mem + 1) * sizeof(vpx_memref_data_t) <= params_size && n_mem <= 4) {
+            memcpy(&head, (const uint8_t*)params + (size_t)n_mem * sizeof(vpx_memref_data_t), 8);
+            if (head == INT64_MIN) break;
+            n_mem++;
+        }
+        VPX_REQUIRE(head == INT64_MIN && n_mem >= 2 && n_mem <= 4, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: the memref list must hold 2..4 records and end at the marker word", entry);
+        n_in = n_mem - e->n_out;
+    }
+    int rc = parse_blob(entry, n_in, e->n_out, params, params_size, addrs, num_addrs, a);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
     switch (e->kind) {
@@ -401,7 +445,54 @@ int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_si
         VPX_REQUIRE(eps >= 0.f, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn1: eps must not be negative, got %g", (double)eps);
         return launch_mvn(a.mem[0], a.mem[1], across != 0, normvar != 0, eps, s);
     }
+    case K_MVN_SUM:
+    case K_MVN_NORM: {
+        // {acrossChannels, normalizeVariance} (sw_kernel.cpp:964-968, 982-986)
+        int64_t across = 0, normvar = 0;
+        VPX_REQUIRE(read_attr(a, 0, &across) && read_attr(a, 8, &normvar), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: params blob is too short for {acrossChannels, normalizeVariance}", entry);
+        if (e->kind == K_MVN_SUM) return launch_mvn_sum(a.mem[0], a.mem[1], across != 0, normvar != 0, s);
+        return launch_mvn_norm(a.mem[0], a.mem[1], a.mem[2], across != 0, normvar != 0, s);
+    }
+    case K_MVN_MEAN_VAR: {
+        // {origShape[4], acrossChannels, normalizeVariance, groupC, eps} (sw_kernel.cpp:969-981)
+        int64_t shape[4] = {0, 0, 0, 0}, across = 0, normvar = 0, group_c = 0;
+        float eps = 0.f;
+        bool ok = true;
+        for (int i = 0; i < 4; i++) ok = ok && read_attr(a, (size_t)i * 8, &shape[i]);
+        ok = ok && read_attr(a, 32, &across) && read_attr(a, 40, &normvar) && read_attr(a, 48, &group_c) && read_attr(a, 56, &eps);
+        VPX_REQUIRE(ok, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "mvn1_mean_var: params blob is too short for {origShape[4], acrossChannels, normalizeVariance, groupC, eps}");
+        return launch_mvn_mean_var(a.mem[0], a.mem[1], shape, across != 0, normvar != 0, group_c, eps, s);
+    }
+    case K_MVN6: {
+        // {marker, io mask}, normalizeVariance, epsMode, eps, numAxes, memAxes[numAxes] (sw_kernel.cpp:987-1004)
+        int64_t marker = 0, mask = 0, normvar = 0, eps_mode = 0, n_axes = 0;
+        float eps = 0.f;
+        VPX_REQUIRE(read_attr(a, 0, &marker) && read_attr(a, 8, &mask) && read_attr(a, 16, &normvar) && read_attr(a, 24, &eps_mode) &&
+                            read_attr(a, 32, &eps) && read_attr(a, 36, &n_axes),
+                    VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: params blob is too short for its attributes");
+        VPX_REQUIRE((mask & 9) == 9 && (mask & ~15ll) == 0 && 2 + ((mask >> 1) & 1) + ((mask >> 2) & 1) == (int64_t)a.mem.size(),
+                    VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: operand mask 0x%llx does not describe %zu memrefs",
+                    (unsigned long long)mask, a.mem.size());
+        VPX_REQUIRE(n_axes >= 1 && n_axes <= VPX_MAX_ND_DIMS, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: %lld axes", (long long)n_axes);
+        int64_t axes[VPX_MAX_ND_DIMS];
+        for (int64_t i = 0; i < n_axes; i++)
+            VPX_REQUIRE(read_attr(a, 44 + (size_t)i * 8, &axes[i]), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                        "mvn6: params blob ends before axis %lld", (long long)i);
+        int next = 1;
+        const MemRef* scale = (mask & 2) ? &a.mem[next++] : nullptr;
+        const MemRef* bias = (mask & 4) ? &a.mem[next++] : nullptr;
+        return launch_mvn6(a.mem[0], scale, bias, a.mem[next], normvar != 0, (int)eps_mode, eps, axes, (int)n_axes, s);
+    }
     case K_SOFTMAX: return run_softmax(entry, a, s);
+    case K_ACT: {
+        float p[2] = {0.f, 0.f};
+        for (int i = 0; i < e->n_float_attrs; i++)
+            VPX_REQUIRE(read_attr(a, (size_t)i * 4, &p[i]), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                        "%s: params blob is too short for %d float attributes", entry, e->n_float_attrs);
+        return launch_activation(e->op, p[0], p[1], a.mem[0], a.mem[1], s);
+    }
     default: return fail(VPX_RESULT_ERROR_UNKNOWN, "%s: no dispatcher", entry);
     }
 }

@@ -275,9 +275,46 @@ struct EltFn {
         if (OP == ELT_MUL) return a * b;
         if (OP == ELT_MIN) return fminf(a, b);
         if (OP == ELT_MAX) return fmaxf(a, b);
+        if (OP == ELT_PRELU) return a < 0.f ? a * b : a;
         return a / b;
     }
     __device__ __forceinline__ T operator()(T x, T y) const { return narrow<T>(f32(x, y)); }
+};
+
+// Unary activations with the OpenVINO operator definitions the VPU ops carry over (operator list:
+// src/vpux_compiler/src/dialect/VPUIP/IR/ops/sw_kernel.cpp:650-941,1266-1285,1689-1845): fp32 arithmetic,
+// one rounding to the storage type.
+template <typename T, int OP>
+struct ActFn {
+    static constexpr bool kF32 = true;
+    float p0, p1;
+    __device__ __forceinline__ float f32(T v) const {
+        const float x = (float)v;
+        if (OP == ACT_RELU) return x > 0.f ? x : 0.f;
+        if (OP == ACT_LEAKY_RELU) return x < 0.f ? x * p0 : x;
+        if (OP == ACT_CLAMP) return x < p0 ? p0 : (x > p1 ? p1 : x);
+        if (OP == ACT_NEGATIVE) return -x;
+        if (OP == ACT_ABS) return fabsf(x);
+        if (OP == ACT_HSWISH) return x * fminf(fmaxf(x + 3.f, 0.f), 6.f) / 6.f;
+        if (OP == ACT_HSIGMOID) return fminf(fmaxf(x + 3.f, 0.f), 6.f) / 6.f;
+        if (OP == ACT_HARDSIGMOID) return fmaxf(0.f, fminf(1.f, p0 * x + p1));
+        if (OP == ACT_SIGMOID) return 1.f / (1.f + expf(-x));
+        if (OP == ACT_TANH) return tanhf(x);
+        if (OP == ACT_EXP) return expf(x);
+        if (OP == ACT_SQRT) return sqrtf(x);
+        if (OP == ACT_LOG) return logf(x);
+        if (OP == ACT_FLOOR) return floorf(x);
+        if (OP == ACT_CEIL) return ceilf(x);
+        if (OP == ACT_SIGN) return x > 0.f ? 1.f : (x < 0.f ? -1.f : x);
+        if (OP == ACT_ELU) return x < 0.f ? p0 * (expf(x) - 1.f) : x;
+        if (OP == ACT_SELU) return x > 0.f ? p1 * x : p0 * p1 * (expf(x) - 1.f);
+        if (OP == ACT_SWISH) return x / (1.f + expf(-p0 * x));
+        if (OP == ACT_MISH) return x * tanhf(x < 20.f ? log1pf(expf(x)) : x);
+        if (OP == ACT_SOFTPLUS) return x < 20.f ? log1pf(expf(x)) : x;
+        if (OP == ACT_GELU) return 0.5f * x * (1.f + erff(x * 0.70710678118654752440f));
+        return erff(x);
+    }
+    __device__ __forceinline__ T operator()(T v) const { return narrow<T>(f32(v)); }
 };
 
 // Per-tensor FakeQuantize as a flat streaming map.  The four limits are device tensors of one
@@ -603,6 +640,25 @@ int launch_convert(const MemRef& in, const MemRef& out, hipStream_t s) {
                 dtype_name(out.dtype));
 }
 
+// ---------------------------------------------------------------- activations
+template <typename T, int OP>
+static int activation_impl(int op, float p0, float p1, const MemRef& in, const MemRef& out, hipStream_t s) {
+    if (op == OP) return convert_impl<T, T>(in, out, ActFn<T, OP>{p0, p1}, s);
+    if constexpr (OP + 1 < ACT_COUNT) return activation_impl<T, OP + 1>(op, p0, p1, in, out, s);
+    return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "activation: unknown operation %d", op);
+}
+
+int launch_activation(int op, float p0, float p1, const MemRef& in, const MemRef& out, hipStream_t s) {
+    VPX_REQUIRE(same_shape(in, out), VPX_RESULT_ERROR_INVALID_ARGUMENT, "activation: input and output shapes differ");
+    VPX_REQUIRE(in.dtype == out.dtype, VPX_RESULT_ERROR_INVALID_ARGUMENT, "activation: input %s and output %s types differ",
+                dtype_name(in.dtype), dtype_name(out.dtype));
+    if (op == ACT_CLAMP)
+        VPX_REQUIRE(p0 <= p1, VPX_RESULT_ERROR_INVALID_ARGUMENT, "activation_clamp: min %g exceeds max %g", (double)p0, (double)p1);
+    if (in.dtype == VPX_NN_FP16) return activation_impl<half_t, 0>(op, p0, p1, in, out, s);
+    if (in.dtype == VPX_NN_FP32) return activation_impl<float, 0>(op, p0, p1, in, out, s);
+    return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "activation: element type %s is not implemented", dtype_name(in.dtype));
+}
+
 // ---------------------------------------------------------------- eltwise
 template <typename T, int OP>
 static int eltwise_impl(const MemRef& a, const MemRef& b, const MemRef& out, hipStream_t s) {
@@ -669,6 +725,7 @@ static int eltwise_dispatch(int op, const MemRef& a, const MemRef& b, const MemR
     case ELT_MIN: return eltwise_impl<T, ELT_MIN>(a, b, out, s);
     case ELT_MAX: return eltwise_impl<T, ELT_MAX>(a, b, out, s);
     case ELT_DIV: return eltwise_impl<T, ELT_DIV>(a, b, out, s);
+    case ELT_PRELU: return eltwise_impl<T, ELT_PRELU>(a, b, out, s);
     default: return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "eltwise: unknown operation %d", op);
     }
 }

@@ -317,6 +317,413 @@ int launch_groups(const half_t* in, half_t* out, int64_t groups, int64_t group_s
     return VPX_RESULT_SUCCESS;
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// The compiler's three-step decomposition of MVN-1 for tensors that do not fit local memory
+// (src/vpux_compiler/src/NPU37XX/dialect/VPU/transforms/passes/decompose_mvn.cpp:82-129;
+// operator definitions src/vpux_compiler/tblgen/vpux/compiler/dialect/VPU/ops.td:3659-3845):
+//   mvn1_sum      x[N,C,H,W] -> f32 {sum, sum of squares} [N, C or 1, parts, 2 or 1], channel-minor
+//   mvn1_mean_var those partial sums -> {mean, 1/sqrt(var + eps)} [N, C or 1, 1, 2 or 1]
+//   mvn1_norm     x, {mean, 1/std} -> (x - mean) * 1/std
+// `parts` (the output height of mvn1_sum) is the number of partial sums per group; a single call
+// here splits the group's elements into that many consecutive ranges, so that their sum is the
+// group's total whatever the count.
+
+// fp32 value -> fp16, round to nearest even.  The empty asm keeps the compiler from folding the preceding
+// multiply into a mixed-precision multiply that rounds the exact product once: the result is defined as
+// the fp32 product rounded again.
+__device__ __forceinline__ half_t round_f16(float v) {
+    asm volatile("" : "+v"(v));
+    return (half_t)v;
+}
+
+struct SumOut {
+    float* out;
+    int parts, out_w;
+    int64_t out_c;
+    __device__ __forceinline__ void put(int64_t group, int part, float s, float q) const {
+        const int64_t n = group / out_c, c = group % out_c;
+        float* o = out + ((n * parts + part) * out_w) * out_c + c;
+        o[0] = s;
+        if (out_w == 2) o[out_c] = q;
+    }
+};
+
+__device__ __forceinline__ float2 add2(float2 a, float2 b) {
+    return float2{a.x + b.x, a.y + b.y};
+}
+
+// One workgroup per (group, chunk) of a contiguous group: raw fp32 sum and sum of squares.
+template <bool ALIGNED>
+__global__ __launch_bounds__(kThreads) void mvn_sum_chunk_kernel(const half_t* __restrict__ in, int64_t group_size,
+                                                                 int chunks, float2* __restrict__ partial, SumOut o,
+                                                                 int direct) {
+    __shared__ float2 red[4];
+    const int64_t group = blockIdx.x / chunks;
+    const int chunk = blockIdx.x % chunks;
+    Chunk c;
+    load_chunk<ALIGNED>(in + group * group_size, (int64_t)chunk * kChunk, group_size, c);
+    float sum = 0.f, sq = 0.f;
+#pragma unroll
+    for (int j = 0; j < kVecPerThread; j++)
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            sum += c.x[j][k];
+            sq += c.x[j][k] * c.x[j][k];
+        }
+    sum = wave_sum(sum);
+    sq = wave_sum(sq);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = float2{sum, sq};
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float2 t = add2(add2(red[0], red[1]), add2(red[2], red[3]));
+        if (direct) o.put(group, 0, t.x, t.y);
+        else partial[blockIdx.x] = t;
+    }
+}
+
+// One workgroup per (group, part): folds that part's chunk sums in a fixed order.
+__global__ __launch_bounds__(kThreads) void mvn_sum_finish_kernel(const float2* __restrict__ partial, int chunks, SumOut o) {
+    __shared__ float2 tree[kThreads];
+    const int64_t group = blockIdx.x / o.parts;
+    const int part = blockIdx.x % o.parts;
+    const int c0 = (int)((int64_t)part * chunks / o.parts), c1 = (int)((int64_t)(part + 1) * chunks / o.parts);
+    float2 acc{0.f, 0.f};
+    for (int c = c0 + threadIdx.x; c < c1; c += kThreads) acc = add2(acc, partial[group * chunks + c]);
+    tree[threadIdx.x] = acc;
+    __syncthreads();
+    for (int step = kThreads / 2; step > 0; step >>= 1) {
+        if ((int)threadIdx.x < step) tree[threadIdx.x] = add2(tree[threadIdx.x], tree[threadIdx.x + step]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) o.put(group, part, tree[0].x, tree[0].y);
+}
+
+// Per-channel sums of a channel-minor layout: a workgroup takes 64 channels of one spatial range
+// of one batch element (lane (r, c) walks positions r, r+4, ...).
+__global__ __launch_bounds__(kThreads) void mvn_sum_cminor_kernel(const half_t* __restrict__ in, int64_t S, int64_t C,
+                                                                  int subparts, int64_t cpad, float2* __restrict__ partial) {
+    __shared__ float2 red[4][64];
+    const int cl = threadIdx.x & 63, r = threadIdx.x >> 6;
+    const int64_t ctiles = cpad / 64;
+    const int64_t ct = blockIdx.x % ctiles;
+    const int sp = (int)((blockIdx.x / ctiles) % subparts);
+    const int64_t n = blockIdx.x / (ctiles * subparts);
+    const int64_t s0 = sp * S / subparts, s1 = (sp + 1) * S / subparts;
+    const int64_t c = ct * 64 + cl;
+    float sum = 0.f, sq = 0.f;
+    if (c < C) {
+        const half_t* px = in + n * S * C + c;
+        for (int64_t i = s0 + r; i < s1; i += 4) {
+            const float x = (float)px[i * C];
+            sum += x;
+            sq += x * x;
+        }
+    }
+    red[r][cl] = float2{sum, sq};
+    __syncthreads();
+    if (r == 0) partial[(n * subparts + sp) * cpad + c] = add2(add2(red[0][cl], red[1][cl]), add2(red[2][cl], red[3][cl]));
+}
+
+__global__ __launch_bounds__(kThreads) void mvn_sum_cminor_finish_kernel(const float2* __restrict__ partial, int64_t total,
+                                                                         int64_t C, int64_t cpad, int subparts, int isplit,
+                                                                         SumOut o) {
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t c = idx % C;
+    const int part = (int)((idx / C) % o.parts);
+    const int64_t n = idx / (C * o.parts);
+    float2 acc{0.f, 0.f};
+    for (int j = 0; j < isplit; j++) acc = add2(acc, partial[(n * subparts + part * isplit + j) * cpad + c]);
+    o.put(n * C + c, part, acc.x, acc.y);
+}
+
+// One lane per output statistic; the handful of partial sums is folded in double.
+template <typename TO>
+__global__ __launch_bounds__(kThreads) void mvn_mean_var_kernel(const float* __restrict__ sum, TO* __restrict__ out, int64_t N,
+                                                                int64_t c_in, int parts, int in_w, int64_t out_c, int out_w,
+                                                                int across, int64_t group_c, double count, float eps) {
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= N * out_c) return;
+    const int64_t n = idx / out_c, c = idx % out_c;
+    int64_t c0 = 0, c1 = c_in;
+    if (!across) {
+        c0 = (c / group_c) * group_c;
+        c1 = c0 + group_c < c_in ? c0 + group_c : c_in;
+    }
+    double s = 0.0, q = 0.0;
+    for (int p = 0; p < parts; p++) {
+        const float* row = sum + ((n * parts + p) * in_w) * c_in;
+        for (int64_t ci = c0; ci < c1; ci++) {
+            s += (double)row[ci];
+            if (in_w == 2) q += (double)row[c_in + ci];
+        }
+    }
+    const double mean = s / count;
+    out[(n * out_w) * out_c + c] = (TO)(float)mean;
+    if (out_w == 2) {
+        double var = q / count - mean * mean;
+        var = var > 0.0 ? var : 0.0;
+        out[(n * out_w + 1) * out_c + c] = (TO)(float)(1.0 / __builtin_sqrt(var + (double)eps));
+    }
+}
+
+// x and y in runs of `run` elements that share one statistic (a (n,c) plane, or a whole batch
+// element when across channels): one workgroup per 2048-element piece of a run.
+template <typename TS, bool ALIGNED>
+__global__ __launch_bounds__(kThreads) void mvn_norm_runs_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                                 const TS* __restrict__ mv, int64_t run, int pieces,
+                                                                 int64_t rows_per_n, int64_t out_c, int out_w) {
+    const int64_t row = blockIdx.x / pieces;
+    const int piece = blockIdx.x % pieces;
+    const int64_t n = row / rows_per_n, c = row % rows_per_n;  // rows_per_n = 1 when across channels
+    const float mean = (float)mv[(n * out_w) * out_c + c];
+    const float inv = out_w == 2 ? (float)mv[(n * out_w + 1) * out_c + c] : 1.0f;
+    const int64_t e0 = (int64_t)piece * (kThreads * 8) + threadIdx.x * 8;
+    const half_t* gi = in + row * run;
+    half_t* go = out + row * run;
+    if (ALIGNED && e0 + 8 <= run) {
+        const u32x4 q = *reinterpret_cast<const u32x4*>(gi + e0);
+        const half_t* p = reinterpret_cast<const half_t*>(&q);
+        u32x4 y;
+        half_t* py = reinterpret_cast<half_t*>(&y);
+#pragma unroll
+        for (int k = 0; k < 8; k++) py[k] = round_f16(((float)p[k] - mean) * inv);
+        __builtin_nontemporal_store(y, reinterpret_cast<u32x4*>(go + e0));
+    } else {
+        for (int k = 0; k < 8; k++)
+            if (e0 + k < run) go[e0 + k] = round_f16(((float)gi[e0 + k] - mean) * inv);
+    }
+}
+
+// Channel-minor layout with per-channel statistics: element e of batch element n has channel e % C.
+template <typename TS>
+__global__ __launch_bounds__(kThreads) void mvn_norm_cminor_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                                   const TS* __restrict__ mv, int64_t per_n, int64_t C,
+                                                                   int pieces, int out_w) {
+    const int64_t n = blockIdx.x / pieces;
+    const int64_t e0 = (int64_t)(blockIdx.x % pieces) * (kThreads * 8) + threadIdx.x * 8;
+    const TS* mean = mv + (n * out_w) * C;
+    const TS* inv = mean + C;
+    const half_t* gi = in + n * per_n;
+    half_t* go = out + n * per_n;
+    uint32_t c = (uint32_t)(e0 % C);
+    for (int k = 0; k < 8; k++) {
+        if (e0 + k < per_n) {
+            const float i = out_w == 2 ? (float)inv[c] : 1.0f;
+            go[e0 + k] = round_f16(((float)gi[e0 + k] - (float)mean[c]) * i);
+        }
+        c = c + 1 == (uint32_t)C ? 0 : c + 1;
+    }
+}
+
+struct MvnShape {
+    int64_t N, C, S;
+    bool channel_minor;
+};
+
+int mvn_shape(const char* what, const MemRef& in, MvnShape& sh) {
+    VPX_REQUIRE(in.nd == 4, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: expects a 4-D tensor, got rank %d", what, in.nd);
+    VPX_REQUIRE(in.order == VPX_ORDER_NCHW || in.order == VPX_ORDER_NCWH || in.order == VPX_ORDER_NHWC ||
+                        in.order == VPX_ORDER_NWHC,
+                VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: unsupported order 0x%llx", what, (unsigned long long)in.order);
+    VPX_REQUIRE(in.compact, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: only compact tensors are supported", what);
+    const int pn = mem_pos_of(in.order, 4, 0), pc = mem_pos_of(in.order, 4, 1);
+    VPX_REQUIRE(pn == 3, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: batch must be the outermost dimension", what);
+    sh.N = in.dims[pn];
+    sh.C = in.dims[pc];
+    sh.S = sh.N * sh.C ? in.numel() / (sh.N * sh.C) : 0;
+    sh.channel_minor = pc != 2;
+    return VPX_RESULT_SUCCESS;
+}
+
+// Logical [N, C, H, W] of a 4-D channel-minor (NHWC) statistics tensor.
+int stats_shape(const char* what, const MemRef& m, int64_t dims[4]) {
+    VPX_REQUIRE(m.nd == 4 && m.order == VPX_ORDER_NHWC && m.compact, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "%s: the statistics tensor must be a compact 4-D NHWC tensor", what);
+    for (int l = 0; l < 4; l++) dims[l] = m.dims[mem_pos_of(m.order, 4, l)];
+    return VPX_RESULT_SUCCESS;
+}
+
+
+// ------------------------------------------------------------------------------------------------
+// mvn6: OpenVINO MVN-6 over an arbitrary set of axes with the eps inside or outside the square
+// root, and the compiler's fused `* scale + bias` (VPU.MVN6,
+// src/vpux_compiler/tblgen/vpux/compiler/dialect/VPU/ops.td:3850-3900;
+// src/vpux_compiler/src/dialect/IE/transforms/passes/fuse_mvn6_scale_bias.cpp).  A row is one
+// combination of the kept (not normalised) coordinates.
+
+struct Mvn6Geom {
+    int nk, nr;
+    int32_t kdim[kMaxDims], rdim[kMaxDims];
+    int64_t k_in[kMaxDims], k_out[kMaxDims], k_sc[kMaxDims], k_bi[kMaxDims];
+    int64_t r_in[kMaxDims], r_out[kMaxDims], r_sc[kMaxDims], r_bi[kMaxDims];
+    int64_t rows;
+    uint32_t row_len;
+    int sc_along_row, bi_along_row;  // contiguous-row kernels: 1 = the operand has the row's elements, 0 = one value per row
+};
+
+struct RowBase {
+    int64_t in, out, sc, bi;
+};
+
+__device__ __forceinline__ RowBase row_base(const Mvn6Geom& g, int64_t row) {
+    RowBase b{0, 0, 0, 0};
+    for (int d = 0; d < g.nk; d++) {
+        const int64_t c = row % g.kdim[d];
+        row /= g.kdim[d];
+        b.in += c * g.k_in[d];
+        b.out += c * g.k_out[d];
+        b.sc += c * g.k_sc[d];
+        b.bi += c * g.k_bi[d];
+    }
+    return b;
+}
+
+__device__ __forceinline__ float mvn6_inv(float var, int normalize_variance, int eps_mode, float eps) {
+    if (!normalize_variance) return 1.0f;
+    return eps_mode == 0 ? 1.0f / __builtin_sqrtf(var + eps) : 1.0f / (__builtin_sqrtf(var) + eps);
+}
+
+// Sum over the TEAM = 64 * WPR lanes that share a row (one wavefront, or the whole workgroup).
+template <int WPR>
+__device__ __forceinline__ float team_sum(float v, float* smem) {
+    v = wave_sum(v);
+    if (WPR == 1) return v;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (smem[0] + smem[1]) + (smem[2] + smem[3]);
+}
+
+// Rows that are contiguous in memory and a multiple of 8 long: the row lives in the registers of one
+// wavefront (WPR = 1, four rows per workgroup) or of the workgroup (WPR = 4).
+template <int WPR, int VPT>
+__global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                             const half_t* __restrict__ sc, const half_t* __restrict__ bi,
+                                                             Mvn6Geom g, int normalize_variance, int eps_mode, float eps) {
+    __shared__ float red[4];
+    constexpr int TEAM = 64 * WPR;
+    const int t = WPR == 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
+    int64_t row = WPR == 1 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
+    const bool live = row < g.rows;  // uniform per team; dead teams of a WPR == 1 workgroup skip memory only
+    if (!live) row = 0;
+    const RowBase b = row_base(g, row);
+    float x[VPT][8];
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; j++) {
+        const uint32_t e0 = (uint32_t)(j * TEAM + t) * 8;
+        if (live && e0 < g.row_len) {
+            const u32x4 q = *reinterpret_cast<const u32x4*>(in + b.in + e0);
+            const half_t* p = reinterpret_cast<const half_t*>(&q);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                x[j][k] = (float)p[k];
+                sum += x[j][k];
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) x[j][k] = 0.f;
+        }
+    }
+    const float n = (float)g.row_len;
+    const float mean = team_sum<WPR>(sum, red) / n;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < VPT; j++) {
+        const uint32_t e0 = (uint32_t)(j * TEAM + t) * 8;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float d = x[j][k] - mean;
+            q += e0 < g.row_len ? d * d : 0.f;
+        }
+    }
+    const float var = team_sum<WPR>(q, red) / n;
+    const float inv = mvn6_inv(var, normalize_variance, eps_mode, eps);
+    const float sc_row = sc && !g.sc_along_row ? (float)sc[b.sc] : 1.0f;
+    const float bi_row = bi && !g.bi_along_row ? (float)bi[b.bi] : 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPT; j++) {
+        const uint32_t e0 = (uint32_t)(j * TEAM + t) * 8;
+        if (!(live && e0 < g.row_len)) continue;
+        float y[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) y[k] = (x[j][k] - mean) * inv;
+        if (sc) {
+            if (g.sc_along_row) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(sc + b.sc + e0);
+                const half_t* p = reinterpret_cast<const half_t*>(&v);
+#pragma unroll
+                for (int k = 0; k < 8; k++) y[k] *= (float)p[k];
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; k++) y[k] *= sc_row;
+            }
+        }
+        if (bi) {
+            if (g.bi_along_row) {
+                const u32x4 v = *reinterpret_cast<const u32x4*>(bi + b.bi + e0);
+                const half_t* p = reinterpret_cast<const half_t*>(&v);
+#pragma unroll
+                for (int k = 0; k < 8; k++) y[k] += (float)p[k];
+            } else {
+#pragma unroll
+                for (int k = 0; k < 8; k++) y[k] += bi_row;
+            }
+        }
+        u32x4 o;
+        half_t* po = reinterpret_cast<half_t*>(&o);
+#pragma unroll
+        for (int k = 0; k < 8; k++) po[k] = (half_t)y[k];
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out + b.out + e0));
+    }
+}
+
+struct ElemOff {
+    int64_t in, out, sc, bi;
+};
+__device__ __forceinline__ ElemOff elem_off(const Mvn6Geom& g, uint32_t e) {
+    ElemOff o{0, 0, 0, 0};
+    for (int d = 0; d < g.nr; d++) {
+        const uint32_t c = e % (uint32_t)g.rdim[d];
+        e /= (uint32_t)g.rdim[d];
+        o.in += c * g.r_in[d];
+        o.out += c * g.r_out[d];
+        o.sc += c * g.r_sc[d];
+        o.bi += c * g.r_bi[d];
+    }
+    return o;
+}
+
+// Any layout, any row length: one workgroup per row, three passes over the row (the second and
+// third come from cache).
+__global__ __launch_bounds__(kThreads) void mvn6_generic_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                                const half_t* __restrict__ sc, const half_t* __restrict__ bi,
+                                                                Mvn6Geom g, int normalize_variance, int eps_mode, float eps) {
+    __shared__ float red[4];
+    const RowBase b = row_base(g, blockIdx.x);
+    float sum = 0.f;
+    for (uint32_t e = threadIdx.x; e < g.row_len; e += kThreads) sum += (float)in[b.in + elem_off(g, e).in];
+    const float n = (float)g.row_len;
+    const float mean = team_sum<4>(sum, red) / n;
+    float q = 0.f;
+    if (normalize_variance)
+        for (uint32_t e = threadIdx.x; e < g.row_len; e += kThreads) {
+            const float d = (float)in[b.in + elem_off(g, e).in] - mean;
+            q += d * d;
+        }
+    const float var = team_sum<4>(q, red) / n;
+    const float inv = mvn6_inv(var, normalize_variance, eps_mode, eps);
+    for (uint32_t e = threadIdx.x; e < g.row_len; e += kThreads) {
+        const ElemOff o = elem_off(g, e);
+        float y = ((float)in[b.in + o.in] - mean) * inv;
+        if (sc) y *= (float)sc[b.sc + o.sc];
+        if (bi) y += (float)bi[b.bi + o.bi];
+        out[b.out + o.out] = (half_t)y;
+    }
+}
+
 }  // namespace
 
 int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool normalize_variance, float eps,
@@ -362,6 +769,291 @@ int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool n
                          (reinterpret_cast<uintptr_t>(po) & 15) == 0;
     return aligned ? launch_groups<true>(pi, po, groups, group_size, nv, eps, s)
                    : launch_groups<false>(pi, po, groups, group_size, nv, eps, s);
+}
+
+int launch_mvn_sum(const MemRef& in, const MemRef& out, bool across_channels, bool normalize_variance, hipStream_t s) {
+    VPX_REQUIRE(in.dtype == VPX_NN_FP16 && out.dtype == VPX_NN_FP32, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "mvn1_sum: FP16 input and FP32 sums are implemented, got %s -> %s", dtype_name(in.dtype), dtype_name(out.dtype));
+    MvnShape sh;
+    int rc = mvn_shape("mvn1_sum", in, sh);
+    if (rc) return rc;
+    int64_t od[4];
+    rc = stats_shape("mvn1_sum", out, od);
+    if (rc) return rc;
+    const int64_t out_c = across_channels ? 1 : sh.C;
+    const int out_w = normalize_variance ? 2 : 1;
+    VPX_REQUIRE(od[0] == sh.N && od[1] == out_c && od[2] >= 1 && od[3] == out_w, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "mvn1_sum: output shape [%lld,%lld,%lld,%lld] does not match [%lld,%lld,parts,%d]", (long long)od[0],
+                (long long)od[1], (long long)od[2], (long long)od[3], (long long)sh.N, (long long)out_c, out_w);
+    VPX_REQUIRE(od[2] <= 4096, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "mvn1_sum: %lld partial sums per group", (long long)od[2]);
+    if (in.numel() == 0) return VPX_RESULT_SUCCESS;
+    const SumOut o{(float*)out.data, (int)od[2], out_w, out_c};
+    const half_t* pi = (const half_t*)in.data;
+
+    if (!across_channels && sh.channel_minor) {
+        const int64_t ctiles = (sh.C + 63) / 64, cpad = ctiles * 64;
+        // enough spatial ranges to spread over the device, at least 64 positions each
+        int64_t isplit = (1024 + sh.N * ctiles * o.parts - 1) / (sh.N * ctiles * o.parts);
+        const int64_t most = sh.S / (64 * (int64_t)o.parts);
+        if (isplit > most) isplit = most;
+        if (isplit < 1) isplit = 1;
+        const int64_t subparts = isplit * o.parts;
+        const int64_t blocks = sh.N * subparts * ctiles, total = sh.N * o.parts * sh.C;
+        VPX_REQUIRE(blocks < (1ll << 31) && total < (1ll << 31) * kThreads, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                    "mvn1_sum: tensor exceeds the launch limit");
+        void* ws = nullptr;
+        rc = get_workspace(s, sizeof(float2) * (size_t)(sh.N * subparts * cpad), &ws);
+        if (rc) return rc;
+        hipLaunchKernelGGL(mvn_sum_cminor_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, s, pi, sh.S, sh.C, (int)subparts,
+                           cpad, (float2*)ws);
+        VPX_HIP_CHECK(hipGetLastError());
+        hipLaunchKernelGGL(mvn_sum_cminor_finish_kernel, dim3((unsigned)((total + kThreads - 1) / kThreads)), dim3(kThreads), 0,
+                           s, (const float2*)ws, total, sh.C, cpad, (int)subparts, (int)isplit, o);
+        VPX_HIP_CHECK(hipGetLastError());
+        return VPX_RESULT_SUCCESS;
+    }
+
+    const int64_t groups = across_channels ? sh.N : sh.N * sh.C;
+    const int64_t group_size = across_channels ? sh.C * sh.S : sh.S;
+    const int64_t chunks64 = (group_size + kChunk - 1) / kChunk;
+    VPX_REQUIRE(chunks64 * groups < (1ll << 31) && groups * o.parts < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "mvn1_sum: %lld groups of %lld elements exceed the launch limit", (long long)groups, (long long)group_size);
+    const int chunks = (int)chunks64;
+    const bool direct = chunks == 1 && o.parts == 1;
+    void* ws = nullptr;
+    if (!direct) {
+        rc = get_workspace(s, sizeof(float2) * (size_t)(groups * chunks), &ws);
+        if (rc) return rc;
+    }
+    const bool aligned = group_size % 8 == 0 && (reinterpret_cast<uintptr_t>(pi) & 15) == 0;
+    const dim3 grid((unsigned)(groups * chunks));
+    if (aligned)
+        hipLaunchKernelGGL((mvn_sum_chunk_kernel<true>), grid, dim3(kThreads), 0, s, pi, group_size, chunks, (float2*)ws, o,
+                           direct ? 1 : 0);
+    else
+        hipLaunchKernelGGL((mvn_sum_chunk_kernel<false>), grid, dim3(kThreads), 0, s, pi, group_size, chunks, (float2*)ws, o,
+                           direct ? 1 : 0);
+    VPX_HIP_CHECK(hipGetLastError());
+    if (!direct) {
+        hipLaunchKernelGGL(mvn_sum_finish_kernel, dim3((unsigned)(groups * o.parts)), dim3(kThreads), 0, s, (const float2*)ws,
+                           chunks, o);
+        VPX_HIP_CHECK(hipGetLastError());
+    }
+    return VPX_RESULT_SUCCESS;
+}
+
+int launch_mvn_mean_var(const MemRef& sum, const MemRef& out, const int64_t orig_shape[4], bool across_channels,
+                        bool normalize_variance, int64_t group_c, float eps, hipStream_t s) {
+    VPX_REQUIRE(sum.dtype == VPX_NN_FP32 && (out.dtype == VPX_NN_FP16 || out.dtype == VPX_NN_FP32),
+                VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "mvn1_mean_var: FP32 sums and FP16/FP32 output are implemented, got %s -> %s",
+                dtype_name(sum.dtype), dtype_name(out.dtype));
+    int64_t id[4], od[4];
+    int rc = stats_shape("mvn1_mean_var", sum, id);
+    if (rc) return rc;
+    rc = stats_shape("mvn1_mean_var", out, od);
+    if (rc) return rc;
+    for (int i = 0; i < 4; i++)
+        VPX_REQUIRE(orig_shape[i] >= 1, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn1_mean_var: orig_shape[%d] = %lld", i,
+                    (long long)orig_shape[i]);
+    const int64_t N = orig_shape[0], C = orig_shape[1];
+    const int64_t out_c = across_channels ? 1 : C;
+    const int out_w = normalize_variance ? 2 : 1;
+    VPX_REQUIRE(id[0] == N && id[3] >= out_w && id[3] <= 2 && id[1] == out_c, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "mvn1_mean_var: sums of shape [%lld,%lld,%lld,%lld] do not fit the original shape [%lld,%lld,..] (%s channels)",
+                (long long)id[0], (long long)id[1], (long long)id[2], (long long)id[3], (long long)N, (long long)C,
+                across_channels ? "across" : "per");
+    VPX_REQUIRE(od[0] == N && od[1] == out_c && od[2] == 1 && od[3] == out_w, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "mvn1_mean_var: output shape [%lld,%lld,%lld,%lld] does not match [%lld,%lld,1,%d]", (long long)od[0],
+                (long long)od[1], (long long)od[2], (long long)od[3], (long long)N, (long long)out_c, out_w);
+    VPX_REQUIRE(group_c >= 1 && C % group_c == 0, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "mvn1_mean_var: %lld channels per group does not divide %lld channels", (long long)group_c, (long long)C);
+    VPX_REQUIRE(eps >= 0.f, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn1_mean_var: eps must not be negative, got %g", (double)eps);
+    const double count = (double)orig_shape[2] * (double)orig_shape[3] * (double)(across_channels ? C : group_c);
+    const dim3 grid((unsigned)((N * out_c + kThreads - 1) / kThreads));
+    if (out.dtype == VPX_NN_FP16)
+        hipLaunchKernelGGL((mvn_mean_var_kernel<half_t>), grid, dim3(kThreads), 0, s, (const float*)sum.data, (half_t*)out.data, N,
+                           id[1], (int)id[2], (int)id[3], out_c, out_w, across_channels ? 1 : 0, group_c, count, eps);
+    else
+        hipLaunchKernelGGL((mvn_mean_var_kernel<float>), grid, dim3(kThreads), 0, s, (const float*)sum.data, (float*)out.data, N,
+                           id[1], (int)id[2], (int)id[3], out_c, out_w, across_channels ? 1 : 0, group_c, count, eps);
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
+template <typename TS>
+static int mvn_norm_impl(const MemRef& in, const MemRef& mv, const MemRef& out, const MvnShape& sh, bool across_channels, int out_w,
+                         hipStream_t s) {
+    const half_t* pi = (const half_t*)in.data;
+    half_t* po = (half_t*)out.data;
+    const TS* pm = (const TS*)mv.data;
+    const int64_t piece = kThreads * 8;
+    if (!across_channels && sh.channel_minor) {
+        const int64_t per_n = sh.S * sh.C;
+        const int64_t pieces = (per_n + piece - 1) / piece;
+        VPX_REQUIRE(sh.N * pieces < (1ll << 31) && sh.C < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                    "mvn1_norm: tensor exceeds the launch limit");
+        hipLaunchKernelGGL((mvn_norm_cminor_kernel<TS>), dim3((unsigned)(sh.N * pieces)), dim3(kThreads), 0, s, pi, po, pm, per_n,
+                           sh.C, (int)pieces, out_w);
+        VPX_HIP_CHECK(hipGetLastError());
+        return VPX_RESULT_SUCCESS;
+    }
+    const int64_t rows = across_channels ? sh.N : sh.N * sh.C;
+    const int64_t run = across_channels ? sh.C * sh.S : sh.S;
+    const int64_t pieces = (run + piece - 1) / piece;
+    VPX_REQUIRE(rows * pieces < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "mvn1_norm: tensor exceeds the launch limit");
+    const bool aligned = run % 8 == 0 && (reinterpret_cast<uintptr_t>(pi) & 15) == 0 && (reinterpret_cast<uintptr_t>(po) & 15) == 0;
+    const int64_t rows_per_n = across_channels ? 1 : sh.C;
+    const int64_t out_c = across_channels ? 1 : sh.C;
+    const dim3 grid((unsigned)(rows * pieces));
+    if (aligned)
+        hipLaunchKernelGGL((mvn_norm_runs_kernel<TS, true>), grid, dim3(kThreads), 0, s, pi, po, pm, run, (int)pieces, rows_per_n,
+                           out_c, out_w);
+    else
+        hipLaunchKernelGGL((mvn_norm_runs_kernel<TS, false>), grid, dim3(kThreads), 0, s, pi, po, pm, run, (int)pieces, rows_per_n,
+                           out_c, out_w);
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
+int launch_mvn_norm(const MemRef& in, const MemRef& mean_var, const MemRef& out, bool across_channels, bool normalize_variance,
+                    hipStream_t s) {
+    VPX_REQUIRE(in.dtype == VPX_NN_FP16 && out.dtype == VPX_NN_FP16, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "mvn1_norm: only FP16 input/output is implemented, got %s -> %s", dtype_name(in.dtype), dtype_name(out.dtype));
+    VPX_REQUIRE(mean_var.dtype == VPX_NN_FP16 || mean_var.dtype == VPX_NN_FP32, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "mvn1_norm: statistics must be FP16 or FP32, got %s", dtype_name(mean_var.dtype));
+    MvnShape sh;
+    int rc = mvn_shape("mvn1_norm", in, sh);
+    if (rc) return rc;
+    VPX_REQUIRE(out.nd == 4 && out.order == in.order && out.compact, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "mvn1_norm: output must be a compact tensor of the input's layout");
+    for (int d = 0; d < 4; d++)
+        VPX_REQUIRE(in.dims[d] == out.dims[d], VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn1_norm: input and output shapes differ");
+    int64_t md[4];
+    rc = stats_shape("mvn1_norm", mean_var, md);
+    if (rc) return rc;
+    const int out_w = normalize_variance ? 2 : 1;
+    VPX_REQUIRE(md[0] == sh.N && md[1] == (across_channels ? 1 : sh.C) && md[2] == 1 && md[3] == out_w,
+                VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn1_norm: statistics of shape [%lld,%lld,%lld,%lld] do not match [%lld,%lld,1,%d]",
+                (long long)md[0], (long long)md[1], (long long)md[2], (long long)md[3], (long long)sh.N,
+                (long long)(across_channels ? 1 : sh.C), out_w);
+    if (in.numel() == 0) return VPX_RESULT_SUCCESS;
+    if (mean_var.dtype == VPX_NN_FP16) return mvn_norm_impl<half_t>(in, mean_var, out, sh, across_channels, out_w, s);
+    return mvn_norm_impl<float>(in, mean_var, out, sh, across_channels, out_w, s);
+}
+
+namespace {
+
+// How an optional operand varies along a row whose reduced dimensions have element strides `stride`:
+// 1 = laid out like the contiguous row, 0 = constant along the row, -1 = neither.
+int along_row(bool present, const int32_t* rdim, const int64_t* stride, int nr) {
+    if (!present) return 0;
+    bool constant = true, full = true;
+    int64_t expect = 1;
+    for (int d = 0; d < nr; d++) {
+        if (stride[d] != 0) constant = false;
+        if (stride[d] != expect) full = false;
+        expect *= rdim[d];
+    }
+    return constant ? 0 : (full ? 1 : -1);
+}
+
+bool aligned_rows(const void* p, const int64_t* kstride, int nk) {
+    if (reinterpret_cast<uintptr_t>(p) & 15) return false;
+    for (int d = 0; d < nk; d++)
+        if (kstride[d] % 8 != 0) return false;
+    return true;
+}
+
+}  // namespace
+
+int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const MemRef& out, bool normalize_variance, int eps_mode,
+                float eps, const int64_t* mem_axes, int n_axes, hipStream_t s) {
+    VPX_REQUIRE(in.dtype == VPX_NN_FP16 && out.dtype == VPX_NN_FP16, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "mvn6: only FP16 input/output is implemented, got %s -> %s", dtype_name(in.dtype), dtype_name(out.dtype));
+    VPX_REQUIRE(in.nd == out.nd && in.nd <= kMaxDims, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: ranks %d / %d (at most %d)", in.nd,
+                out.nd, kMaxDims);
+    for (int d = 0; d < in.nd; d++)
+        VPX_REQUIRE(in.dims[d] == out.dims[d], VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: input and output shapes differ");
+    VPX_REQUIRE(eps_mode == 0 || eps_mode == 1, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: unknown eps mode %d", eps_mode);
+    VPX_REQUIRE(eps >= 0.f, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: eps must not be negative, got %g", (double)eps);
+    VPX_REQUIRE(n_axes >= 1 && n_axes <= in.nd, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: %d axes for rank %d", n_axes, in.nd);
+    bool reduced[kMaxDims] = {};
+    for (int i = 0; i < n_axes; i++) {
+        VPX_REQUIRE(mem_axes[i] >= 0 && mem_axes[i] < in.nd && !reduced[mem_axes[i]], VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "mvn6: axis %lld is outside rank %d or repeated", (long long)mem_axes[i], in.nd);
+        reduced[mem_axes[i]] = true;
+    }
+    const MemRef* extra[2] = {scale, bias};
+    for (const MemRef* m : extra) {
+        if (!m) continue;
+        VPX_REQUIRE(m->dtype == VPX_NN_FP16 && m->nd == in.nd, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "mvn6: scale / bias must be FP16 tensors of the input's rank");
+        for (int d = 0; d < in.nd; d++)
+            VPX_REQUIRE(m->dims[d] == in.dims[d] || m->dims[d] == 1, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                        "mvn6: scale / bias dimension %d is %lld, input has %lld", d, (long long)m->dims[d], (long long)in.dims[d]);
+    }
+    if (in.numel() == 0) return VPX_RESULT_SUCCESS;
+
+    Mvn6Geom g{};
+    int64_t row_len = 1;
+    g.rows = 1;
+    bool innermost = true;  // the reduced dimensions are the innermost ones
+    for (int d = 0; d < in.nd; d++) {
+        if (in.dims[d] == 1) continue;
+        const int64_t ssc = scale && scale->dims[d] != 1 ? scale->strides[d] : 0;
+        const int64_t sbi = bias && bias->dims[d] != 1 ? bias->strides[d] : 0;
+        if (reduced[d]) {
+            if (g.nk > 0) innermost = false;
+            g.rdim[g.nr] = (int32_t)in.dims[d];
+            g.r_in[g.nr] = in.strides[d];
+            g.r_out[g.nr] = out.strides[d];
+            g.r_sc[g.nr] = ssc;
+            g.r_bi[g.nr] = sbi;
+            g.nr++;
+            row_len *= in.dims[d];
+        } else {
+            g.kdim[g.nk] = (int32_t)in.dims[d];
+            g.k_in[g.nk] = in.strides[d];
+            g.k_out[g.nk] = out.strides[d];
+            g.k_sc[g.nk] = ssc;
+            g.k_bi[g.nk] = sbi;
+            g.nk++;
+            g.rows *= in.dims[d];
+        }
+    }
+    VPX_REQUIRE(row_len < (1ll << 31) && g.rows < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "mvn6: %lld rows of %lld elements exceed the launch limit", (long long)g.rows, (long long)row_len);
+    g.row_len = (uint32_t)row_len;
+    const half_t* pi = (const half_t*)in.data;
+    half_t* po = (half_t*)out.data;
+    const half_t* ps = scale ? (const half_t*)scale->data : nullptr;
+    const half_t* pb = bias ? (const half_t*)bias->data : nullptr;
+    const int nv = normalize_variance ? 1 : 0;
+
+    bool fast = innermost && row_len % 8 == 0 && row_len <= 8192;
+    if (fast) {
+        fast = along_row(true, g.rdim, g.r_in, g.nr) == 1 && along_row(true, g.rdim, g.r_out, g.nr) == 1;
+        g.sc_along_row = along_row(scale != nullptr, g.rdim, g.r_sc, g.nr);
+        g.bi_along_row = along_row(bias != nullptr, g.rdim, g.r_bi, g.nr);
+        fast = fast && g.sc_along_row >= 0 && g.bi_along_row >= 0 && aligned_rows(pi, g.k_in, g.nk) && aligned_rows(po, g.k_out, g.nk);
+        if (fast && scale && g.sc_along_row) fast = aligned_rows(ps, g.k_sc, g.nk);
+        if (fast && bias && g.bi_along_row) fast = aligned_rows(pb, g.k_bi, g.nk);
+    }
+    if (fast) {
+        const dim3 wave_rows((unsigned)((g.rows + 3) / 4)), block_rows((unsigned)g.rows);
+#define VPX_MVN6_ROWS(WPR, VPT, GRID) \
+    hipLaunchKernelGGL((mvn6_rows_kernel<WPR, VPT>), GRID, dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps)
+        if (row_len <= 512) VPX_MVN6_ROWS(1, 1, wave_rows);
+        else if (row_len <= 1024) VPX_MVN6_ROWS(1, 2, wave_rows);
+        else if (row_len <= 2048) VPX_MVN6_ROWS(4, 1, block_rows);
+        else if (row_len <= 4096) VPX_MVN6_ROWS(4, 2, block_rows);
+        else VPX_MVN6_ROWS(4, 4, block_rows);
+#undef VPX_MVN6_ROWS
+    } else {
+        hipLaunchKernelGGL(mvn6_generic_kernel, dim3((unsigned)g.rows), dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps);
+    }
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
 }
 
 }  // namespace vpx

@@ -106,6 +106,46 @@ int launch_softmax(const SoftmaxPlan& p, uint32_t dtype, const void* in, void* o
 int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool normalize_variance, float eps,
                hipStream_t s);
 
-enum EltOp { ELT_ADD = 0, ELT_SUB, ELT_MUL, ELT_MIN, ELT_MAX, ELT_DIV };
+// MVN-1 decomposition (mvn1_sum -> mvn1_mean_var -> mvn1_norm)
+int launch_mvn_sum(const MemRef& in, const MemRef& out, bool across_channels, bool normalize_variance, hipStream_t s);
+int launch_mvn_mean_var(const MemRef& sum, const MemRef& out, const int64_t orig_shape[4], bool across_channels,
+                        bool normalize_variance, int64_t group_c, float eps, hipStream_t s);
+int launch_mvn_norm(const MemRef& in, const MemRef& mean_var, const MemRef& out, bool across_channels, bool normalize_variance,
+                    hipStream_t s);
+
+// mem_axes: normalised dimensions counted from the innermost memory dimension; scale / bias may be null
+int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const MemRef& out, bool normalize_variance, int eps_mode,
+                float eps, const int64_t* mem_axes, int n_axes, hipStream_t s);
+
+enum EltOp { ELT_ADD = 0, ELT_SUB, ELT_MUL, ELT_MIN, ELT_MAX, ELT_DIV, ELT_PRELU };
+
+// Unary activations; p0 / p1 are the kernel's float attributes in the order the compiler serialises them.
+enum ActOp {
+    ACT_RELU = 0,
+    ACT_LEAKY_RELU,   // p0 = negative slope
+    ACT_CLAMP,        // p0 = min, p1 = max
+    ACT_NEGATIVE,
+    ACT_ABS,
+    ACT_HSWISH,
+    ACT_HSIGMOID,
+    ACT_HARDSIGMOID,  // p0 = alpha, p1 = beta
+    ACT_SIGMOID,
+    ACT_TANH,
+    ACT_EXP,
+    ACT_SQRT,
+    ACT_LOG,
+    ACT_FLOOR,
+    ACT_CEIL,
+    ACT_SIGN,
+    ACT_ELU,          // p0 = alpha
+    ACT_SELU,         // p0 = alpha, p1 = lambda
+    ACT_SWISH,        // p0 = beta
+    ACT_MISH,
+    ACT_SOFTPLUS,
+    ACT_GELU,
+    ACT_ERF,
+    ACT_COUNT
+};
+int launch_activation(int op, float p0, float p1, const MemRef& in, const MemRef& out, hipStream_t s);
 
 }  // namespace vpx

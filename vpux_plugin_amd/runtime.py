@@ -288,6 +288,35 @@ def eltwise(kind, a, b, out, order=None, stream=None):
     return out
 
 
+# kernel entry and number of float attributes of each unary activation (sw_kernel.cpp getKernelInfo)
+ACTIVATIONS = {
+    "relu": ("activation_relu", 0), "leaky_relu": ("leaky_relu_fp16", 1), "clamp": ("activation_clamp", 2),
+    "negative": ("activation_negative", 0), "abs": ("activation_abs", 0), "hswish": ("activation_hswish", 0),
+    "hsigmoid": ("activation_hsigmoid", 0), "hardsigmoid": ("activation_hardsigmoid", 2),
+    "sigmoid": ("activation_sigmoid", 0), "tanh": ("activation_tanh", 0), "exp": ("activation_exp", 0),
+    "sqrt": ("activation_sqrt", 0), "log": ("activation_log", 0), "floor": ("activation_floor", 0),
+    "ceil": ("activation_ceil", 0), "sign": ("activation_sign", 0), "elu": ("activation_elu", 1),
+    "selu": ("activation_selu", 2), "swish": ("activation_swish", 1), "mish": ("activation_mish", 0),
+    "softplus": ("activation_softplus", 0), "gelu": ("activation_gelu", 0), "erf": ("activation_erf", 0),
+}
+
+
+def activation(kind, x, out, *params, order=None, stream=None):
+    entry, n_attrs = ACTIVATIONS[kind]
+    if len(params) != n_attrs:
+        raise ValueError(f"{kind} takes {n_attrs} attributes, got {len(params)}")
+    ops = [Operand(x, order), Operand(out, order)]
+    attrs = np.asarray(params, dtype=np.float32).tobytes()
+    sw_kernel_launch(entry, create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    return out
+
+
+def prelu(x, slope, out, order=None, stream=None):
+    ops = [Operand(x, order), Operand(slope, order), Operand(out, order)]
+    sw_kernel_launch("prelu_fp16", create_kernel_params(ops[:2], ops[2:]), ops, stream)
+    return out
+
+
 def fake_quantize(x, in_lo, in_hi, out_lo, out_hi, levels, out, order=None, stream=None):
     ops = [Operand(t, order) for t in (x, in_lo, in_hi, out_lo, out_hi, out)]
     sw_kernel_launch("fake_quantize", create_kernel_params(ops[:5], ops[5:], _i64(levels)), ops, stream)
@@ -313,6 +342,47 @@ def mvn(x, out, across_channels, normalize_variance, eps, order="NCHW", stream=N
     # a true boolean attribute serialises as int64 -1 (sign-extended i1)
     attrs = _i64(-1 if across_channels else 0, -1 if normalize_variance else 0) + np.float32(eps).tobytes()
     sw_kernel_launch("mvn1", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    return out
+
+
+def _bool_attr(v):
+    return -1 if v else 0
+
+
+def mvn1_sum(x, out, across_channels, normalize_variance, order="NCHW", stream=None):
+    """out: float32 statistics tensor in memory order [N, parts, 2 or 1, C or 1] (the NHWC storage of the
+    op's logical [N, C or 1, parts, 2 or 1] result)."""
+    ops = [Operand(x, order), Operand(out, "NHWC")]
+    attrs = _i64(_bool_attr(across_channels), _bool_attr(normalize_variance))
+    sw_kernel_launch("mvn1_sum", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    return out
+
+
+def mvn1_mean_var(sums, out, orig_shape, across_channels, normalize_variance, eps, group_c=1, stream=None):
+    ops = [Operand(sums, "NHWC"), Operand(out, "NHWC")]
+    attrs = _i64(*orig_shape, _bool_attr(across_channels), _bool_attr(normalize_variance), group_c) + np.float32(eps).tobytes()
+    sw_kernel_launch("mvn1_mean_var", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    return out
+
+
+def mvn1_norm(x, mean_var, out, across_channels, normalize_variance, order="NCHW", stream=None):
+    ops = [Operand(x, order), Operand(mean_var, "NHWC"), Operand(out, order)]
+    attrs = _i64(_bool_attr(across_channels), _bool_attr(normalize_variance))
+    sw_kernel_launch("mvn1_norm", create_kernel_params(ops[:2], ops[2:], attrs), ops, stream)
+    return out
+
+
+def mvn6(x, out, axes, normalize_variance, eps, eps_mode=0, scale=None, bias=None, order=None, stream=None):
+    """axes index x in memory order (outermost first), like torch dims; eps_mode 0 = inside the square root,
+    1 = outside.  scale / bias: optional tensors of x's rank, broadcast NUMPY-style."""
+    nd = x.dim()
+    ins = [Operand(x, order)] + [Operand(t, order) for t in (scale, bias) if t is not None]
+    ops = ins + [Operand(out, order)]
+    mask = 1 | (2 if scale is not None else 0) | (4 if bias is not None else 0) | 8
+    mem_axes = [nd - 1 - (a % nd) for a in axes]
+    attrs = (_i64(-(2 ** 63), mask, _bool_attr(normalize_variance), eps_mode) + np.float32(eps).tobytes() +
+             _i64(len(mem_axes), *mem_axes))
+    sw_kernel_launch("mvn6", create_kernel_params(ins, ops[-1:], attrs), ops, stream)
     return out
 
 
