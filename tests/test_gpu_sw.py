@@ -483,6 +483,8 @@ MVN6_CASES = [
     ((3, 5, 16, 24), (2, 3), (1, 1, 16, 24), (1, 5, 1, 1)),  # two innermost axes
     ((5, 7, 30), (2,), (1, 1, 30), (1, 1, 30)),           # row not a multiple of 8: generic
     ((4, 6, 10), (1,), (1, 6, 1), None),                  # middle axis: generic
+    ((3, 64, 200), (1,), (1, 64, 1), (1, 1, 200)),        # innermost dimension kept: lanes along it
+    ((2, 5, 6, 70), (1, 2), (1, 5, 6, 1), None),
     ((2, 3, 4, 5), (1, 3), (1, 3, 1, 5), (1, 1, 1, 5)),   # split axes
     ((2, 20000), (1,), None, None),                       # long row
     ((6, 1, 64), (1, 2), None, None),                     # unit dimension among the axes

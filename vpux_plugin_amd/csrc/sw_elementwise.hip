@@ -284,22 +284,52 @@ struct EltFn {
 // Unary activations with the OpenVINO operator definitions the VPU ops carry over (operator list:
 // src/vpux_compiler/src/dialect/VPUIP/IR/ops/sw_kernel.cpp:650-941,1266-1285,1689-1845): fp32 arithmetic,
 // one rounding to the storage type.
+// Building blocks for fp16 tensors, where the result is rounded to 11 bits: hardware exp2 / log2 /
+// reciprocal (about 1 ulp of fp32 each) instead of the correctly rounded library routines.
+__device__ __forceinline__ float fast_exp(float x) {
+    return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
+}
+__device__ __forceinline__ float fast_rcp(float x) {
+    return __builtin_amdgcn_rcpf(x);
+}
+// log(1 + t) for 0 <= t <= 1: the series where 1 + t would lose the low bits of t
+__device__ __forceinline__ float fast_log1p_unit(float t) {
+    const float series = t * (1.f - t * (0.5f - t * (0.33333333f - t * 0.25f)));
+    const float direct = __builtin_amdgcn_logf(1.f + t) * 0.69314718055994530942f;
+    return t < 0.03125f ? series : direct;
+}
+__device__ __forceinline__ float fast_softplus(float x) {
+    return fmaxf(x, 0.f) + fast_log1p_unit(fast_exp(-fabsf(x)));
+}
+__device__ __forceinline__ float fast_tanh(float x) {
+    const float x2 = x * x;
+    const float small = x * (1.f - x2 * (0.33333333f - x2 * 0.13333333f));
+    const float big = 1.f - 2.f * fast_rcp(1.f + fast_exp(2.f * fabsf(x)));
+    return fabsf(x) < 0.05f ? small : __builtin_copysignf(big, x);
+}
+
 template <typename T, int OP>
 struct ActFn {
     static constexpr bool kF32 = true;
+    static constexpr bool kFast = std::is_same<T, half_t>::value;
     float p0, p1;
     __device__ __forceinline__ float f32(T v) const {
         const float x = (float)v;
+        constexpr float kSixth = 0.16666667163372039794921875f;  // RN(1/6)
         if (OP == ACT_RELU) return x > 0.f ? x : 0.f;
         if (OP == ACT_LEAKY_RELU) return x < 0.f ? x * p0 : x;
         if (OP == ACT_CLAMP) return x < p0 ? p0 : (x > p1 ? p1 : x);
         if (OP == ACT_NEGATIVE) return -x;
         if (OP == ACT_ABS) return fabsf(x);
-        if (OP == ACT_HSWISH) return x * fminf(fmaxf(x + 3.f, 0.f), 6.f) / 6.f;
-        if (OP == ACT_HSIGMOID) return fminf(fmaxf(x + 3.f, 0.f), 6.f) / 6.f;
+        if (OP == ACT_HSWISH) {
+            // x * relu6(x + 3) / 6 with the exact quotient of div_const; an infinite product stays infinite
+            const float a = x * fminf(fmaxf(x + 3.f, 0.f), 6.f);
+            return fabsf(a) == INFINITY ? a : div_const(a, 6.f, kSixth);
+        }
+        if (OP == ACT_HSIGMOID) return div_const(fminf(fmaxf(x + 3.f, 0.f), 6.f), 6.f, kSixth);
         if (OP == ACT_HARDSIGMOID) return fmaxf(0.f, fminf(1.f, p0 * x + p1));
-        if (OP == ACT_SIGMOID) return 1.f / (1.f + expf(-x));
-        if (OP == ACT_TANH) return tanhf(x);
+        if (OP == ACT_SIGMOID) return kFast ? fast_rcp(1.f + fast_exp(-x)) : 1.f / (1.f + expf(-x));
+        if (OP == ACT_TANH) return kFast ? fast_tanh(x) : tanhf(x);
         if (OP == ACT_EXP) return expf(x);
         if (OP == ACT_SQRT) return sqrtf(x);
         if (OP == ACT_LOG) return logf(x);
@@ -308,9 +338,15 @@ struct ActFn {
         if (OP == ACT_SIGN) return x > 0.f ? 1.f : (x < 0.f ? -1.f : x);
         if (OP == ACT_ELU) return x < 0.f ? p0 * (expf(x) - 1.f) : x;
         if (OP == ACT_SELU) return x > 0.f ? p1 * x : p0 * p1 * (expf(x) - 1.f);
-        if (OP == ACT_SWISH) return x / (1.f + expf(-p0 * x));
-        if (OP == ACT_MISH) return x * tanhf(x < 20.f ? log1pf(expf(x)) : x);
-        if (OP == ACT_SOFTPLUS) return x < 20.f ? log1pf(expf(x)) : x;
+        if (OP == ACT_SWISH) return kFast ? x * fast_rcp(1.f + fast_exp(-p0 * x)) : x / (1.f + expf(-p0 * x));
+        if (OP == ACT_MISH) {
+            if (!kFast) return x * tanhf(x < 20.f ? log1pf(expf(x)) : x);
+            // tanh(log(1 + e^x)) = n / (n + 2) with n = e^x (e^x + 2): no cancellation at either end
+            const float e = fast_exp(fminf(x, 20.f));
+            const float n = e * (e + 2.f);
+            return x * (n * fast_rcp(n + 2.f));
+        }
+        if (OP == ACT_SOFTPLUS) return kFast ? fast_softplus(x) : (x < 20.f ? log1pf(expf(x)) : x);
         if (OP == ACT_GELU) return 0.5f * x * (1.f + erff(x * 0.70710678118654752440f));
         return erff(x);
     }

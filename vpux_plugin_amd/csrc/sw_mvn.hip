@@ -240,41 +240,6 @@ __global__ __launch_bounds__(kThreads) void mvn_merge_kernel(const Record* parti
     if (threadIdx.x == 0) merged[group] = Record{total.n, total.mean, total.m2, 0.f};
 }
 
-// Per-channel statistics of a channel-minor layout (NHWC / NWHC): element (n,s,c) at
-// n*S*C + s*C + c.  A workgroup takes 64 channels of one batch element; lane (r, c) walks the
-// spatial positions r, r+4, ... so that every access covers 64 adjacent channels.
-__global__ __launch_bounds__(kThreads) void mvn_channel_minor_kernel(const half_t* __restrict__ in,
-                                                                     half_t* __restrict__ out, int64_t S, int64_t C,
-                                                                     int normalize_variance, float eps) {
-    __shared__ float red[4][64];
-    const int cl = threadIdx.x & 63, r = threadIdx.x >> 6;
-    const int64_t ctiles = (C + 63) / 64;
-    const int64_t n = blockIdx.x / ctiles;
-    const int64_t c = (blockIdx.x % ctiles) * 64 + cl;
-    const bool ok = c < C;
-    const half_t* px = in + n * S * C + c;
-    half_t* py = out + n * S * C + c;
-    float s = 0.f;
-    if (ok)
-        for (int64_t i = r; i < S; i += 4) s += (float)px[i * C];
-    red[r][cl] = s;
-    __syncthreads();
-    const float mean = ((red[0][cl] + red[1][cl]) + (red[2][cl] + red[3][cl])) / (float)S;
-    __syncthreads();
-    float q = 0.f;
-    if (ok)
-        for (int64_t i = r; i < S; i += 4) {
-            const float d = (float)px[i * C] - mean;
-            q += d * d;
-        }
-    red[r][cl] = q;
-    __syncthreads();
-    const float var = ((red[0][cl] + red[1][cl]) + (red[2][cl] + red[3][cl])) / (float)S;
-    const float inv = normalize_variance ? 1.0f / __builtin_sqrtf(var + eps) : 1.0f;
-    if (ok)
-        for (int64_t i = r; i < S; i += 4) py[i * C] = (half_t)(((float)px[i * C] - mean) * inv);
-}
-
 // position (counted from the innermost memory dimension) of logical dimension `logical`
 int mem_pos_of(uint64_t order, int nd, int logical) {
     for (int i = 0; i < nd; i++)
@@ -400,7 +365,10 @@ __global__ __launch_bounds__(kThreads) void mvn_sum_finish_kernel(const float2* 
 }
 
 // Per-channel sums of a channel-minor layout: a workgroup takes 64 channels of one spatial range
-// of one batch element (lane (r, c) walks positions r, r+4, ...).
+// of one batch element (lane (r, c) walks positions r, r+4, ...).  With SHIFT the sums are of
+// x - x[first position of the channel], which keeps the sum of squares free of cancellation when a
+// channel's mean is far from zero (used where the variance is taken from these sums).
+template <bool SHIFT>
 __global__ __launch_bounds__(kThreads) void mvn_sum_cminor_kernel(const half_t* __restrict__ in, int64_t S, int64_t C,
                                                                   int subparts, int64_t cpad, float2* __restrict__ partial) {
     __shared__ float2 red[4][64];
@@ -414,8 +382,9 @@ __global__ __launch_bounds__(kThreads) void mvn_sum_cminor_kernel(const half_t* 
     float sum = 0.f, sq = 0.f;
     if (c < C) {
         const half_t* px = in + n * S * C + c;
+        const float shift = SHIFT ? (float)px[0] : 0.f;
         for (int64_t i = s0 + r; i < s1; i += 4) {
-            const float x = (float)px[i * C];
+            const float x = (float)px[i * C] - shift;
             sum += x;
             sq += x * x;
         }
@@ -434,8 +403,28 @@ __global__ __launch_bounds__(kThreads) void mvn_sum_cminor_finish_kernel(const f
     const int part = (int)((idx / C) % o.parts);
     const int64_t n = idx / (C * o.parts);
     float2 acc{0.f, 0.f};
+#pragma unroll 8
     for (int j = 0; j < isplit; j++) acc = add2(acc, partial[(n * subparts + part * isplit + j) * cpad + c]);
     o.put(n * C + c, part, acc.x, acc.y);
+}
+
+// mvn1 on a channel-minor layout with per-channel statistics: folds the shifted partial sums of one
+// (n, c) and leaves {mean, 1/std} as fp32 in the layout mvn_norm_cminor_kernel reads.
+__global__ __launch_bounds__(kThreads) void mvn_cminor_stats_kernel(const half_t* __restrict__ in, const float2* __restrict__ partial,
+                                                                    float* __restrict__ stats, int64_t total, int64_t S, int64_t C,
+                                                                    int64_t cpad, int subparts, int normalize_variance, float eps) {
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t c = idx % C, n = idx / C;
+    float2 acc{0.f, 0.f};
+#pragma unroll 8
+    for (int j = 0; j < subparts; j++) acc = add2(acc, partial[(n * subparts + j) * cpad + c]);
+    const float shift = (float)in[n * S * C + c];
+    const float cnt = (float)S;
+    const float m = acc.x / cnt;
+    const float var = fmaxf(acc.y / cnt - m * m, 0.f);
+    stats[(n * 2) * C + c] = shift + m;
+    stats[(n * 2 + 1) * C + c] = normalize_variance ? 1.0f / __builtin_sqrtf(var + eps) : 1.0f;
 }
 
 // One lane per output statistic; the handful of partial sums is folded in double.
@@ -497,7 +486,9 @@ __global__ __launch_bounds__(kThreads) void mvn_norm_runs_kernel(const half_t* _
 }
 
 // Channel-minor layout with per-channel statistics: element e of batch element n has channel e % C.
-template <typename TS>
+// VEC: the channel count is a multiple of 8 and everything is 16-byte aligned, so a lane's 8 elements are 8
+// consecutive channels and their statistics two contiguous runs.
+template <typename TS, bool VEC>
 __global__ __launch_bounds__(kThreads) void mvn_norm_cminor_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
                                                                    const TS* __restrict__ mv, int64_t per_n, int64_t C,
                                                                    int pieces, int out_w) {
@@ -508,6 +499,21 @@ __global__ __launch_bounds__(kThreads) void mvn_norm_cminor_kernel(const half_t*
     const half_t* gi = in + n * per_n;
     half_t* go = out + n * per_n;
     uint32_t c = (uint32_t)(e0 % C);
+    if (VEC) {
+        if (e0 >= per_n) return;
+        const u32x4 q = *reinterpret_cast<const u32x4*>(gi + e0);
+        const half_t* p = reinterpret_cast<const half_t*>(&q);
+        TS m[8], iv[8];
+        typedef uint32_t words_t __attribute__((ext_vector_type(sizeof(TS) * 2)));  // 8 statistics = 16 or 32 bytes
+        *reinterpret_cast<words_t*>(m) = *reinterpret_cast<const words_t*>(mean + c);
+        if (out_w == 2) *reinterpret_cast<words_t*>(iv) = *reinterpret_cast<const words_t*>(inv + c);
+        u32x4 y;
+        half_t* py = reinterpret_cast<half_t*>(&y);
+#pragma unroll
+        for (int k = 0; k < 8; k++) py[k] = round_f16(((float)p[k] - (float)m[k]) * (out_w == 2 ? (float)iv[k] : 1.0f));
+        __builtin_nontemporal_store(y, reinterpret_cast<u32x4*>(go + e0));
+        return;
+    }
     for (int k = 0; k < 8; k++) {
         if (e0 + k < per_n) {
             const float i = out_w == 2 ? (float)inv[c] : 1.0f;
@@ -585,28 +591,34 @@ __device__ __forceinline__ float mvn6_inv(float var, int normalize_variance, int
     return eps_mode == 0 ? 1.0f / __builtin_sqrtf(var + eps) : 1.0f / (__builtin_sqrtf(var) + eps);
 }
 
-// Sum over the TEAM = 64 * WPR lanes that share a row (one wavefront, or the whole workgroup).
-template <int WPR>
+// Sum over the TEAM lanes that share a row: half a wavefront, a wavefront, or the whole workgroup.
+template <int TEAM>
 __device__ __forceinline__ float team_sum(float v, float* smem) {
+    if (TEAM == 32) {  // the row operations and the 16-lane swap stay inside each half
+        v += dppf<0xB1>(v);
+        v += dppf<0x4E>(v);
+        v += dppf<0x141>(v);
+        v += dppf<0x140>(v);
+        return v + swz16(v);
+    }
     v = wave_sum(v);
-    if (WPR == 1) return v;
+    if (TEAM == 64) return v;
     __syncthreads();
     if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
     __syncthreads();
     return (smem[0] + smem[1]) + (smem[2] + smem[3]);
 }
 
-// Rows that are contiguous in memory and a multiple of 8 long: the row lives in the registers of one
-// wavefront (WPR = 1, four rows per workgroup) or of the workgroup (WPR = 4).
-template <int WPR, int VPT>
+// Rows that are contiguous in memory and a multiple of 8 long: the row lives in the registers of half a
+// wavefront (TEAM = 32, eight rows per workgroup), of a wavefront (64) or of the workgroup (256).
+template <int TEAM, int VPT>
 __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
                                                              const half_t* __restrict__ sc, const half_t* __restrict__ bi,
                                                              Mvn6Geom g, int normalize_variance, int eps_mode, float eps) {
     __shared__ float red[4];
-    constexpr int TEAM = 64 * WPR;
-    const int t = WPR == 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
-    int64_t row = WPR == 1 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : (int64_t)blockIdx.x;
-    const bool live = row < g.rows;  // uniform per team; dead teams of a WPR == 1 workgroup skip memory only
+    const int t = (int)(threadIdx.x % TEAM);
+    int64_t row = (int64_t)blockIdx.x * (kThreads / TEAM) + threadIdx.x / TEAM;
+    const bool live = row < g.rows;  // uniform per team; dead teams skip memory only
     if (!live) row = 0;
     const RowBase b = row_base(g, row);
     float x[VPT][8];
@@ -628,7 +640,7 @@ __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __res
         }
     }
     const float n = (float)g.row_len;
-    const float mean = team_sum<WPR>(sum, red) / n;
+    const float mean = team_sum<TEAM>(sum, red) / n;
     float q = 0.f;
 #pragma unroll
     for (int j = 0; j < VPT; j++) {
@@ -639,7 +651,7 @@ __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __res
             q += e0 < g.row_len ? d * d : 0.f;
         }
     }
-    const float var = team_sum<WPR>(q, red) / n;
+    const float var = team_sum<TEAM>(q, red) / n;
     const float inv = mvn6_inv(var, normalize_variance, eps_mode, eps);
     const float sc_row = sc && !g.sc_along_row ? (float)sc[b.sc] : 1.0f;
     const float bi_row = bi && !g.bi_along_row ? (float)bi[b.bi] : 0.0f;
@@ -696,6 +708,67 @@ __device__ __forceinline__ ElemOff elem_off(const Mvn6Geom& g, uint32_t e) {
     return o;
 }
 
+// The innermost dimension is kept and contiguous (normalising over channels of a channel-major tensor,
+// say): a workgroup takes P adjacent positions of it, so that every access covers a contiguous run, and
+// splits the reduced elements over its 256 / P lane groups (group r walks elements r, r + G, ...; three
+// passes, the later ones from cache).  Smaller P gives more workgroups when the tensor has few positions.
+template <int P>
+__global__ __launch_bounds__(kThreads) void mvn6_inner_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                              const half_t* __restrict__ sc, const half_t* __restrict__ bi,
+                                                              Mvn6Geom g, int normalize_variance, int eps_mode, float eps) {
+    constexpr int G = kThreads / P;
+    __shared__ float red[G][P];
+    const int cl = threadIdx.x % P;
+    const uint32_t r = P == 64 ? (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / P)) : threadIdx.x / P;
+    const int64_t tiles = (g.kdim[0] + P - 1) / P;
+    int64_t o = blockIdx.x / tiles;
+    const int64_t i0 = (blockIdx.x % tiles) * P + cl;
+    const bool ok = i0 < g.kdim[0];
+    RowBase b{0, 0, 0, 0};
+    for (int d = 1; d < g.nk; d++) {
+        const int64_t c = o % g.kdim[d];
+        o /= g.kdim[d];
+        b.in += c * g.k_in[d];
+        b.out += c * g.k_out[d];
+        b.sc += c * g.k_sc[d];
+        b.bi += c * g.k_bi[d];
+    }
+    const int64_t i = ok ? i0 : 0;
+    b.in += i * g.k_in[0];
+    b.out += i * g.k_out[0];
+    b.sc += i * g.k_sc[0];
+    b.bi += i * g.k_bi[0];
+    const float n = (float)g.row_len;
+    const auto total = [&](float v) {
+        __syncthreads();
+        red[r][cl] = v;
+        __syncthreads();
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < G; k++) t += red[k][cl];
+        return t;
+    };
+    float sum = 0.f;
+    for (uint32_t e = r; e < g.row_len; e += G) sum += (float)in[b.in + elem_off(g, e).in];
+    const float mean = total(sum) / n;
+    float q = 0.f;
+    if (normalize_variance)
+        for (uint32_t e = r; e < g.row_len; e += G) {
+            const float d = (float)in[b.in + elem_off(g, e).in] - mean;
+            q += d * d;
+        }
+    const float var = total(q) / n;
+    const float inv = mvn6_inv(var, normalize_variance, eps_mode, eps);
+    if (!ok) return;
+    for (uint32_t e = r; e < g.row_len; e += G) {
+        const ElemOff off = elem_off(g, e);
+        float y = ((float)in[b.in + off.in] - mean) * inv;
+        if (sc) y *= (float)sc[b.sc + off.sc];
+        if (bi) y += (float)bi[b.bi + off.bi];
+        out[b.out + off.out] = (half_t)y;
+    }
+}
+
 // Any layout, any row length: one workgroup per row, three passes over the row (the second and
 // third come from cache).
 __global__ __launch_bounds__(kThreads) void mvn6_generic_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
@@ -706,14 +779,14 @@ __global__ __launch_bounds__(kThreads) void mvn6_generic_kernel(const half_t* __
     float sum = 0.f;
     for (uint32_t e = threadIdx.x; e < g.row_len; e += kThreads) sum += (float)in[b.in + elem_off(g, e).in];
     const float n = (float)g.row_len;
-    const float mean = team_sum<4>(sum, red) / n;
+    const float mean = team_sum<256>(sum, red) / n;
     float q = 0.f;
     if (normalize_variance)
         for (uint32_t e = threadIdx.x; e < g.row_len; e += kThreads) {
             const float d = (float)in[b.in + elem_off(g, e).in] - mean;
             q += d * d;
         }
-    const float var = team_sum<4>(q, red) / n;
+    const float var = team_sum<256>(q, red) / n;
     const float inv = mvn6_inv(var, normalize_variance, eps_mode, eps);
     for (uint32_t e = threadIdx.x; e < g.row_len; e += kThreads) {
         const ElemOff o = elem_off(g, e);
@@ -722,6 +795,41 @@ __global__ __launch_bounds__(kThreads) void mvn6_generic_kernel(const half_t* __
         if (bi) y += (float)bi[b.bi + o.bi];
         out[b.out + o.out] = (half_t)y;
     }
+}
+
+
+// mvn1 with per-channel statistics on a channel-minor layout: shifted partial sums over spatial ranges,
+// a fold to {mean, 1/std}, then the element-wise pass.
+int launch_channel_minor(const half_t* in, half_t* out, int64_t N, int64_t S, int64_t C, int nv, float eps, hipStream_t s) {
+    const int64_t ctiles = (C + 63) / 64, cpad = ctiles * 64;
+    int64_t subparts = (1024 + N * ctiles - 1) / (N * ctiles);
+    if (subparts > S / 64) subparts = S / 64;
+    if (subparts < 1) subparts = 1;
+    const int64_t per_n = S * C, piece = kThreads * 8, pieces = (per_n + piece - 1) / piece;
+    VPX_REQUIRE(N * subparts * ctiles < (1ll << 31) && N * pieces < (1ll << 31) && C < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "mvn1: tensor exceeds the launch limit");
+    void* ws = nullptr;
+    const size_t partial_bytes = sizeof(float2) * (size_t)(N * subparts * cpad);
+    int rc = get_workspace(s, partial_bytes + sizeof(float) * (size_t)(N * 2 * C), &ws);
+    if (rc) return rc;
+    float2* partial = (float2*)ws;
+    float* stats = (float*)((char*)ws + partial_bytes);
+    hipLaunchKernelGGL(mvn_sum_cminor_kernel<true>, dim3((unsigned)(N * subparts * ctiles)), dim3(kThreads), 0, s, in, S, C,
+                       (int)subparts, cpad, partial);
+    VPX_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(mvn_cminor_stats_kernel, dim3((unsigned)((N * C + kThreads - 1) / kThreads)), dim3(kThreads), 0, s, in,
+                       (const float2*)partial, stats, N * C, S, C, cpad, (int)subparts, nv, eps);
+    VPX_HIP_CHECK(hipGetLastError());
+    const bool vec = C % 8 == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
+                     (reinterpret_cast<uintptr_t>(stats) & 31) == 0;
+    if (vec)
+        hipLaunchKernelGGL((mvn_norm_cminor_kernel<float, true>), dim3((unsigned)(N * pieces)), dim3(kThreads), 0, s, in, out,
+                           (const float*)stats, per_n, C, (int)pieces, 2);
+    else
+        hipLaunchKernelGGL((mvn_norm_cminor_kernel<float, false>), dim3((unsigned)(N * pieces)), dim3(kThreads), 0, s, in, out,
+                           (const float*)stats, per_n, C, (int)pieces, 2);
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
 }
 
 }  // namespace
@@ -758,12 +866,7 @@ int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool n
         groups = N * C;
         group_size = S;
     } else {  // channel-minor layout, per-channel statistics
-        const int64_t ctiles = (C + 63) / 64;
-        VPX_REQUIRE(N * ctiles < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "mvn1: tensor exceeds the launch limit");
-        hipLaunchKernelGGL(mvn_channel_minor_kernel, dim3((unsigned)(N * ctiles)), dim3(kThreads), 0, s, pi, po, S, C, nv,
-                           eps);
-        VPX_HIP_CHECK(hipGetLastError());
-        return VPX_RESULT_SUCCESS;
+        return launch_channel_minor(pi, po, N, S, C, nv, eps, s);
     }
     const bool aligned = group_size % 8 == 0 && (reinterpret_cast<uintptr_t>(pi) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(po) & 15) == 0;
@@ -804,7 +907,7 @@ int launch_mvn_sum(const MemRef& in, const MemRef& out, bool across_channels, bo
         void* ws = nullptr;
         rc = get_workspace(s, sizeof(float2) * (size_t)(sh.N * subparts * cpad), &ws);
         if (rc) return rc;
-        hipLaunchKernelGGL(mvn_sum_cminor_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, s, pi, sh.S, sh.C, (int)subparts,
+        hipLaunchKernelGGL(mvn_sum_cminor_kernel<false>, dim3((unsigned)blocks), dim3(kThreads), 0, s, pi, sh.S, sh.C, (int)subparts,
                            cpad, (float2*)ws);
         VPX_HIP_CHECK(hipGetLastError());
         hipLaunchKernelGGL(mvn_sum_cminor_finish_kernel, dim3((unsigned)((total + kThreads - 1) / kThreads)), dim3(kThreads), 0,
@@ -892,8 +995,14 @@ static int mvn_norm_impl(const MemRef& in, const MemRef& mv, const MemRef& out, 
         const int64_t pieces = (per_n + piece - 1) / piece;
         VPX_REQUIRE(sh.N * pieces < (1ll << 31) && sh.C < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
                     "mvn1_norm: tensor exceeds the launch limit");
-        hipLaunchKernelGGL((mvn_norm_cminor_kernel<TS>), dim3((unsigned)(sh.N * pieces)), dim3(kThreads), 0, s, pi, po, pm, per_n,
-                           sh.C, (int)pieces, out_w);
+        const bool vec = sh.C % 8 == 0 && ((reinterpret_cast<uintptr_t>(pi) | reinterpret_cast<uintptr_t>(po)) & 15) == 0 &&
+                         (reinterpret_cast<uintptr_t>(pm) & 31) == 0;
+        if (vec)
+            hipLaunchKernelGGL((mvn_norm_cminor_kernel<TS, true>), dim3((unsigned)(sh.N * pieces)), dim3(kThreads), 0, s, pi, po, pm,
+                               per_n, sh.C, (int)pieces, out_w);
+        else
+            hipLaunchKernelGGL((mvn_norm_cminor_kernel<TS, false>), dim3((unsigned)(sh.N * pieces)), dim3(kThreads), 0, s, pi, po, pm,
+                               per_n, sh.C, (int)pieces, out_w);
         VPX_HIP_CHECK(hipGetLastError());
         return VPX_RESULT_SUCCESS;
     }
@@ -997,9 +1106,11 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
     Mvn6Geom g{};
     int64_t row_len = 1;
     g.rows = 1;
-    bool innermost = true;  // the reduced dimensions are the innermost ones
+    bool innermost = true;   // the reduced dimensions are the innermost ones
+    bool inner_kept = false;  // the innermost dimension (of more than one element) is kept
     for (int d = 0; d < in.nd; d++) {
         if (in.dims[d] == 1) continue;
+        if (g.nk + g.nr == 0) inner_kept = !reduced[d];
         const int64_t ssc = scale && scale->dims[d] != 1 ? scale->strides[d] : 0;
         const int64_t sbi = bias && bias->dims[d] != 1 ? bias->strides[d] : 0;
         if (reduced[d]) {
@@ -1040,15 +1151,25 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
         if (fast && bias && g.bi_along_row) fast = aligned_rows(pb, g.k_bi, g.nk);
     }
     if (fast) {
-        const dim3 wave_rows((unsigned)((g.rows + 3) / 4)), block_rows((unsigned)g.rows);
-#define VPX_MVN6_ROWS(WPR, VPT, GRID) \
-    hipLaunchKernelGGL((mvn6_rows_kernel<WPR, VPT>), GRID, dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps)
-        if (row_len <= 512) VPX_MVN6_ROWS(1, 1, wave_rows);
-        else if (row_len <= 1024) VPX_MVN6_ROWS(1, 2, wave_rows);
-        else if (row_len <= 2048) VPX_MVN6_ROWS(4, 1, block_rows);
-        else if (row_len <= 4096) VPX_MVN6_ROWS(4, 2, block_rows);
-        else VPX_MVN6_ROWS(4, 4, block_rows);
+#define VPX_MVN6_ROWS(TEAM, VPT) \
+    hipLaunchKernelGGL((mvn6_rows_kernel<TEAM, VPT>), dim3((unsigned)((g.rows + kThreads / TEAM - 1) / (kThreads / TEAM))), \
+                       dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps)
+        if (row_len <= 256) VPX_MVN6_ROWS(32, 1);
+        else if (row_len <= 512) VPX_MVN6_ROWS(64, 1);
+        else if (row_len <= 1024) VPX_MVN6_ROWS(64, 2);
+        else if (row_len <= 2048) VPX_MVN6_ROWS(256, 1);
+        else if (row_len <= 4096) VPX_MVN6_ROWS(256, 2);
+        else VPX_MVN6_ROWS(256, 4);
 #undef VPX_MVN6_ROWS
+    } else if (inner_kept && g.k_in[0] == 1 && g.k_out[0] == 1) {
+        const int64_t outer = g.rows / g.kdim[0];
+        const auto blocks = [&](int p) { return outer * ((g.kdim[0] + p - 1) / p); };
+        if (blocks(64) >= 512)
+            hipLaunchKernelGGL(mvn6_inner_kernel<64>, dim3((unsigned)blocks(64)), dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps);
+        else if (blocks(32) >= 512)
+            hipLaunchKernelGGL(mvn6_inner_kernel<32>, dim3((unsigned)blocks(32)), dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps);
+        else
+            hipLaunchKernelGGL(mvn6_inner_kernel<16>, dim3((unsigned)blocks(16)), dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps);
     } else {
         hipLaunchKernelGGL(mvn6_generic_kernel, dim3((unsigned)g.rows), dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps);
     }
