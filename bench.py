@@ -241,6 +241,61 @@ def make_copy(rt):
                     _prebuilt_sw_launch(rt, "convert", blob, ops), n * 4, 0, "hbm", "f16", "stream_kernel<Copy>")
 
 
+def make_layernorm(rt):
+    """mvn6 over the last axis with the fused scale and bias (a LayerNorm): not a BASELINE config."""
+    import torch
+    rows, width = 16384, 4096
+    g = torch.Generator(device="cuda").manual_seed(7)
+    x = torch.randn((rows, width), device="cuda", generator=g).half()
+    sc = torch.rand((1, width), device="cuda", generator=g).half()
+    bi = torch.rand((1, width), device="cuda", generator=g).half()
+    out = torch.empty_like(x)
+    ops = [rt.Operand(t) for t in (x, sc, bi, out)]
+    attrs = (np.asarray([-(2 ** 63), 15, -1, 0], dtype=np.int64).tobytes() + np.float32(1e-5).tobytes() +
+             np.asarray([1, 0], dtype=np.int64).tobytes())
+    blob = rt.create_kernel_params(ops[:3], ops[3:], attrs)
+    return Workload("x_mvn6_layernorm", "MVN-6 fp16 over the last axis [16384,4096] with scale and bias (not a BASELINE config)",
+                    _prebuilt_sw_launch(rt, "mvn6", blob, ops), x.numel() * 4 + width * 4, 0, "hbm", "f16", "mvn6_rows_kernel")
+
+
+def make_activation(rt):
+    """hswish on the C5-sized tensor: not a BASELINE config."""
+    import torch
+    x = torch.randn((4096, 11008), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8)).half()
+    out = torch.empty_like(x)
+    ops = [rt.Operand(x), rt.Operand(out)]
+    blob = rt.create_kernel_params(ops[:1], ops[1:])
+    return Workload("x_activation_hswish", "activation_hswish fp16 [4096,11008] (not a BASELINE config)",
+                    _prebuilt_sw_launch(rt, "activation_hswish", blob, ops), x.numel() * 4, 0, "hbm", "f16", "stream_kernel<ActFn>")
+
+
+def make_mvn_steps(rt):
+    """The compiler's three-step form of C3: mvn1_sum -> mvn1_mean_var -> mvn1_norm (not a BASELINE config)."""
+    import torch
+    from vpux_plugin_amd import configs
+    c = configs.c3_mvn()
+    x = _dev(c["x"], True)
+    N, Cc, H, W = x.shape
+    out = torch.empty_like(x)
+    sums = torch.empty((N, 1, 2, 1), dtype=torch.float32, device="cuda")
+    mv = torch.empty((N, 1, 2, 1), dtype=torch.float32, device="cuda")
+    flags = np.asarray([-1, -1], dtype=np.int64).tobytes()
+    o1 = [rt.Operand(x, "NCHW"), rt.Operand(sums, "NHWC")]
+    o2 = [rt.Operand(sums, "NHWC"), rt.Operand(mv, "NHWC")]
+    o3 = [rt.Operand(x, "NCHW"), rt.Operand(mv, "NHWC"), rt.Operand(out, "NCHW")]
+    a2 = np.asarray([N, Cc, H, W, -1, -1, 1], dtype=np.int64).tobytes() + np.float32(c["eps"]).tobytes()
+    steps = [_prebuilt_sw_launch(rt, "mvn1_sum", rt.create_kernel_params(o1[:1], o1[1:], flags), o1),
+             _prebuilt_sw_launch(rt, "mvn1_mean_var", rt.create_kernel_params(o2[:1], o2[1:], a2), o2),
+             _prebuilt_sw_launch(rt, "mvn1_norm", rt.create_kernel_params(o3[:2], o3[2:], flags), o3)]
+
+    def step():
+        for f in steps:
+            f()
+    step.keep = steps
+    return Workload("x_mvn1_three_steps", "mvn1_sum -> mvn1_mean_var -> mvn1_norm fp16 [4,256,64,64] (not a BASELINE config)",
+                    step, x.numel() * 4, 0, "hbm", "f16", "mvn_norm_runs_kernel")
+
+
 MAKERS = {
     "calib_copy": make_copy,
     "c1_fake_quantize": make_c1,
@@ -251,6 +306,9 @@ MAKERS = {
     "c5_dequantize": lambda rt: make_c5(rt, "dequant"),
     "c5_eltwise_add": lambda rt: make_c5(rt, "add"),
     "c5_nce_eltwise": lambda rt: make_c5(rt, "nce_eltwise"),
+    "x_mvn6_layernorm": make_layernorm,
+    "x_activation_hswish": make_activation,
+    "x_mvn1_three_steps": make_mvn_steps,
 }
 
 

@@ -109,6 +109,23 @@ typedef enum vpx_softmax_mode_t {
  *       uint64 w[2 + 2*ndims]: w0 = axis | padSize << 32, w1 = mode | ndims << 32, then per dimension
  *       (innermost first) dim | dim << 32 and inStride | outStride << 32 in elements
  *       (update_sw_kernel_params.cpp:36-147)
+ *   mvn1_sum       in, sums                          | int64 acrossChannels; int64 normalizeVariance
+ *       sums: f32 [N, C or 1, parts, 2 or 1] in NHWC order = {sum, sum of squares} (sw_kernel.cpp:964-968;
+ *       src/vpux_compiler/tblgen/vpux/compiler/dialect/VPU/ops.td:3659-3715)
+ *   mvn1_mean_var  sums, meanVar                     | int64 origShape[4]; int64 acrossChannels; int64 normalizeVariance;
+ *       int64 groupC; float eps (sw_kernel.cpp:969-981); meanVar: f16/f32 [N, C or 1, 1, 2 or 1] in NHWC order
+ *       = {mean, 1/sqrt(var + eps)}
+ *   mvn1_norm      in, meanVar, out                  | int64 acrossChannels; int64 normalizeVariance (sw_kernel.cpp:982-986)
+ *   mvn6           in, [scale], [bias], out, marker  | the memref list ends at an INT64_MIN word, which opens the
+ *       attributes: int64 marker; int64 mask (bit 0 input, 1 scale, 2 bias, 3 output); int64 normalizeVariance;
+ *       int64 epsMode (0 inside, 1 outside the square root); float eps; int64 numAxes; int64 memAxes[numAxes]
+ *       (axes counted from the innermost memory dimension; sw_kernel.cpp:164-185, 987-1004)
+ *   activation_<name>, leaky_relu_fp16  in, out      | the op's float attributes as 32-bit floats, in order:
+ *       leaky_relu_fp16 {negative_slope}; activation_clamp {min, max}; activation_hardsigmoid {alpha, beta};
+ *       activation_elu {alpha}; activation_selu {alpha, lambda}; activation_swish {beta}; none for relu, negative,
+ *       abs, hswish, hsigmoid, sigmoid, tanh, exp, sqrt, log, floor, ceil, sign, mish, softplus, gelu, erf
+ *       (sw_kernel.cpp:650-941, 1266-1285, 1689-1845)
+ *   prelu_fp16     in, slope, out                    | (none); slope broadcasts NUMPY-style (sw_kernel.cpp:1102-1104)
  */
 
 #ifdef __cplusplus
