@@ -239,6 +239,17 @@ def mvn_f16(x, across_channels, normalize_variance, eps, layout="NCHW"):
     return y
 
 
+def dynamic_dequantize(q, scale, zero_point=None, to_f16=True):
+    """VPU.DynamicDequantize (ops.td:7780-7819): (q - zp) * scale with NUMPY-broadcast scale / zero-point tensors, in
+    fp32, then the float16 class's rounding for fp16 output.  scale: float32 array or uint16 fp16 bits.
+    "parity unpinned" against the SHAVE kernel; pinned by the static dequantize golden (content_tests.cpp:754-788)."""
+    q = np.asarray(q)
+    sc = f16_to_f32(scale) if np.asarray(scale).dtype == np.uint16 else np.asarray(scale, dtype=np.float32)
+    z = np.zeros((1,) * q.ndim, np.int32) if zero_point is None else np.asarray(zero_point).astype(np.int32)
+    r = ((q.astype(np.int32) - z).astype(np.float32) * sc).astype(np.float32)
+    return f32_to_f16(r) if to_f16 else r
+
+
 # The three-step decomposition of MVN-1 (decompose_mvn.cpp:82-129; ops.td:3659-3845), in numpy.  Tensors are
 # logical [N,C,H,W] arrays; statistics tensors are in their memory order [N, parts, 2 or 1, C or 1].
 # "parity unpinned" like mvn_f16: the reference holds no vectors for these kernels.  Pinned by the tests through

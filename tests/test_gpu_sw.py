@@ -347,6 +347,58 @@ def test_quantize_per_axis_ambiguous_axis_is_refused(rt, dev):
         rt.quantize(x, torch.empty((4, 2, 4), dtype=torch.int8, device=dev), [0.1] * 3, [0] * 3)  # no dimension of size 3
 
 
+# ---------------------------------------------------------------------------------- dynamic_dequantize
+
+DYN_DQ_CASES = [
+    # q shape, q dtype, scale shape, scale dtype, zp shape / dtype, out dtype
+    ((512, 1024), np.int8, (512, 1), np.float16, None, np.float16),                       # per-row scale, vector path
+    ((512, 1024), np.int8, (512, 1), np.float16, ((512, 1), np.int8), np.float16),
+    ((64, 8, 128), np.int8, (64, 8, 1), np.float16, ((64, 8, 1), np.int8), np.float16),   # group-wise weights
+    ((33, 1000), np.uint8, (1, 1000), np.float32, ((1, 1000), np.uint8), np.float16),     # per-column: one value per lane
+    ((7, 5, 3), np.int8, (1, 1, 1), np.float16, None, np.float32),
+    ((128, 256), np.uint8, (128, 1), np.float32, ((1, 1), np.uint8), np.float32),
+]
+
+
+@pytest.mark.parametrize("case", DYN_DQ_CASES, ids=[str(c[0]) + c[1].__name__ for c in DYN_DQ_CASES])
+def test_dynamic_dequantize(rt, orc, dev, case):
+    import torch
+    shape, qdt, sc_shape, sc_dt, zp_spec, out_dt = case
+    rng = np.random.default_rng(61)
+    info = np.iinfo(qdt)
+    q = rng.integers(info.min, info.max + 1, shape).astype(qdt)
+    sc32 = rng.uniform(1e-3, 0.1, sc_shape).astype(np.float32)
+    sc32.flat[0] = 2.0 ** -22  # results below 2^-15 take the float16 class's own rounding
+    sc = sc32.astype(sc_dt)
+    zp = None if zp_spec is None else rng.integers(np.iinfo(zp_spec[1]).min // 2, np.iinfo(zp_spec[1]).max // 2 + 1, zp_spec[0]).astype(zp_spec[1])
+    out = torch.empty(shape, dtype=getattr(torch, out_dt.__name__), device=dev)
+    rt.dynamic_dequantize(to_dev(q, dev), to_dev(sc, dev), out, None if zp is None else to_dev(zp, dev))
+    sc_arg = sc.view(np.uint16) if sc_dt is np.float16 else sc
+    if out_dt is np.float16:
+        assert_f16_exact(f16_bits(out), orc.dynamic_dequantize(q, sc_arg, zp), str(shape))
+    else:
+        assert np.array_equal(out.cpu().numpy(), orc.dynamic_dequantize(q, sc_arg, zp, to_f16=False))
+
+
+def test_dynamic_dequantize_views_and_errors(rt, orc, dev):
+    import torch
+    rng = np.random.default_rng(62)
+    q = rng.integers(-128, 128, (16, 64, 256)).astype(np.int8)
+    sc = rng.uniform(1e-3, 0.1, (16, 64, 1)).astype(np.float16)
+    qd, sd = to_dev(q, dev), to_dev(sc, dev)
+    out = torch.zeros((16, 64, 256), dtype=torch.float16, device=dev)
+    rt.dynamic_dequantize(qd[:, 8:24, 64:192], sd[:, 8:24], out[:, 4:20, 128:256])
+    want = np.zeros((16, 64, 256), np.uint16)
+    want[:, 4:20, 128:256] = orc.dynamic_dequantize(q[:, 8:24, 64:192], sc[:, 8:24].view(np.uint16))
+    assert_f16_exact(f16_bits(out), want, "sub-views")
+    with pytest.raises(rt.VpxError) as e:
+        rt.dynamic_dequantize(qd, to_dev(np.ones((16, 3, 1), np.float16), dev), out)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    with pytest.raises(rt.VpxError) as e:
+        rt.dynamic_dequantize(qd.to(torch.int32), sd, out)
+    assert e.value.code == rt.ERROR_UNSUPPORTED_FEATURE
+
+
 # ---------------------------------------------------------------------------------- MVN decomposition
 
 def _mvn_input(orc, rng, shape):

@@ -530,3 +530,18 @@ def test_mvn6_against_mvn1_and_hand_cases(orc):
     bi = orc.f32_to_f16(np.array([[1]], np.float32))
     assert orc.f16_to_f32(orc.mvn6_f16(row, (1,), False, 0.0, 0, sc, bi))[0].tolist() == [-2.0, 0.0, 1.0, -0.5]
 
+
+def test_dynamic_dequantize_matches_static_golden_and_broadcasts(orc):
+    q = np.array([[-127, 0, 127]], np.int8)
+    y = orc.f16_to_f32(orc.dynamic_dequantize(q, np.array([[2.0 / 254.0]], np.float32)))
+    assert y.tolist() == [[-1.0, 0.0, 1.0]]                       # content_tests.cpp:754-788 through the tensor-scale form
+    q = np.arange(-6, 6, dtype=np.int8).reshape(3, 4)
+    sc = np.array([[0.5], [2.0], [0.25]], np.float32)
+    zp = np.array([[1], [0], [-2]], np.int8)
+    want = (q.astype(np.float64) - zp) * sc
+    assert np.array_equal(orc.f16_to_f32(orc.dynamic_dequantize(q, sc, zp)), want.astype(np.float32))
+    assert np.array_equal(orc.dynamic_dequantize(q, sc, zp, to_f16=False), want.astype(np.float32))
+    # the same numbers as the static per-axis dequantize when scale and zero point are per row
+    stat = orc.dequantize(q, sc.ravel().astype(np.float64), zp.ravel().astype(np.int64), to_f16=True, axis=0)
+    assert np.array_equal(orc.dynamic_dequantize(q, sc, zp), stat)
+

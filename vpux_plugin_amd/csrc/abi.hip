@@ -304,7 +304,7 @@ struct Entry {
     int n_float_attrs;  // K_ACT: 32-bit float attributes that follow the memrefs
 };
 
-enum { K_CONVERT, K_ELTWISE, K_FQ, K_QUANT, K_DEQUANT, K_MVN, K_SOFTMAX, K_ACT, K_MVN_SUM, K_MVN_MEAN_VAR, K_MVN_NORM, K_MVN6 };
+enum { K_CONVERT, K_ELTWISE, K_FQ, K_QUANT, K_DEQUANT, K_MVN, K_SOFTMAX, K_ACT, K_MVN_SUM, K_MVN_MEAN_VAR, K_MVN_NORM, K_MVN6, K_DYN_DEQUANT };
 
 const Entry kEntries[] = {
         {"convert", 1, 1, K_CONVERT, 0},
@@ -321,6 +321,7 @@ const Entry kEntries[] = {
         {"mvn1_sum", 1, 1, K_MVN_SUM, 0},
         {"mvn1_mean_var", 1, 1, K_MVN_MEAN_VAR, 0},
         {"mvn1_norm", 2, 1, K_MVN_NORM, 0},
+        {"dynamic_dequantize", -1, 1, K_DYN_DEQUANT, 0},  // input, scale, optional zero point; list ends at an INT64_MAX word
         {"mvn6", -1, 1, K_MVN6, 0},  // input, optional scale, optional bias; the memref list ends at an INT64_MIN word
         {"softmax", 1, 1, K_SOFTMAX, 0},
         {"softmaxFp32", 1, 1, K_SOFTMAX, 0},
@@ -398,15 +399,16 @@ int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_si
     Args a;
     int n_in = e->n_in;
     if (n_in < 0) {
-        // optional operands: count MemRefData records up to the marker word (sw_kernel.cpp:164-185)
+        // optional operands: count MemRefData records up to the marker word (INT64_MIN, sw_kernel.cpp:164-185) or
+        // the delimiter (INT64_MAX, sw_runtime_kernels/kernels/inc/common_types.h:141-151)
         int n_mem = 0;
         int64_t head = 0;
         while ((size_t)(n_mem + 1) * sizeof(vpx_memref_data_t) <= params_size && n_mem <= 4) {
             memcpy(&head, (const uint8_t*)params + (size_t)n_mem * sizeof(vpx_memref_data_t), 8);
-            if (head == INT64_MIN) break;
+            if (head == INT64_MIN || head == INT64_MAX) break;
             n_mem++;
         }
-        VPX_REQUIRE(head == INT64_MIN && n_mem >= 2 && n_mem <= 4, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+        VPX_REQUIRE((head == INT64_MIN || head == INT64_MAX) && n_mem >= 2 && n_mem <= 4, VPX_RESULT_ERROR_INVALID_ARGUMENT,
                     "%s: the memref list must hold 2..4 records and end at the marker word", entry);
         n_in = n_mem - e->n_out;
     }
@@ -464,6 +466,12 @@ int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_si
         VPX_REQUIRE(ok, VPX_RESULT_ERROR_INVALID_ARGUMENT,
                     "mvn1_mean_var: params blob is too short for {origShape[4], acrossChannels, normalizeVariance, groupC, eps}");
         return launch_mvn_mean_var(a.mem[0], a.mem[1], shape, across != 0, normvar != 0, group_c, eps, s);
+    }
+    case K_DYN_DEQUANT: {
+        VPX_REQUIRE(a.mem.size() == 3 || a.mem.size() == 4, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "dynamic_dequantize: expects input, scale, an optional zero point and the output, got %zu memrefs", a.mem.size());
+        const bool has_zp = a.mem.size() == 4;
+        return launch_dynamic_dequantize(a.mem[0], a.mem[1], has_zp ? &a.mem[2] : nullptr, a.mem[has_zp ? 3 : 2], s);
     }
     case K_MVN6: {
         // {marker, io mask}, normalizeVariance, epsMode, eps, numAxes, memAxes[numAxes] (sw_kernel.cpp:987-1004)

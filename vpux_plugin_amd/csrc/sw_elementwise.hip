@@ -21,6 +21,14 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 template <int BYTES>
 struct Words;
 template <>
+struct Words<1> {
+    typedef uint8_t type;
+};
+template <>
+struct Words<2> {
+    typedef uint16_t type;
+};
+template <>
 struct Words<4> {
     typedef uint32_t type;
 };
@@ -33,7 +41,7 @@ struct Words<16> {
     typedef u32x4 type;
 };
 
-// N elements of T moved by one 32/64/128-bit access per lane.  Adjacent lanes touch adjacent
+// N elements of T moved by one 8...128-bit access per lane.  Adjacent lanes touch adjacent
 // words, so a wavefront's access is one contiguous run; the wider operand of a kernel gets the
 // 128-bit form.  Stores are non-temporal (results are not re-read); loads are ordinary, which
 // measures faster than non-temporal loads on this memory system.
@@ -463,6 +471,39 @@ __global__ __launch_bounds__(kBlock) void nd_unary_kernel(const TI* in, TO* out,
     out[off[1]] = fn(in[off[0]]);
 }
 
+// dynamic_dequantize: y = (q - zp) * scale with scale and zero point read from tensors that broadcast onto
+// the input (VPU.DynamicDequantize, src/vpux_compiler/tblgen/vpux/compiler/dialect/VPU/ops.td:7780-7819).
+// A lane takes VEC values along the innermost dimension; with VEC > 1 scale and zero point are constant along it
+// (per-row or per-group scales of a weight matrix) and `ix` counts the innermost dimension in vectors.
+template <typename TQ, typename TS, typename TO, int VEC>
+__global__ __launch_bounds__(kBlock) void dyn_dequant_kernel(const TQ* __restrict__ in, const TS* __restrict__ scale,
+                                                             const uint8_t* __restrict__ zp, int zp_signed, TO* __restrict__ out,
+                                                             NdIndex ix, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    int64_t off[4];
+    nd_offsets<4>(ix, i, off);
+    const float sc = (float)scale[off[1]];
+    int z = 0;
+    if (zp) z = zp_signed ? (int)(int8_t)zp[off[2]] : (int)zp[off[2]];
+    Pack<TQ, VEC> x;
+    x.load(in + off[0], 0);
+    float r[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++) r[k] = (float)((int)x.get(k) - z) * sc;
+    Pack<TO, VEC> y;
+    if constexpr (std::is_same<TO, half_t>::value) {
+        half_t h[VEC];
+        narrow_vec(r, h);
+#pragma unroll
+        for (int k = 0; k < VEC; k++) y.set(k, h[k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC; k++) y.set(k, r[k]);
+    }
+    y.store(out + off[3], 0);
+}
+
 template <typename T, class Fn>
 __global__ __launch_bounds__(kBlock) void nd_binary_kernel(const T* a, const T* b, T* out, Fn fn, NdIndex ix,
                                                            int64_t n) {
@@ -872,6 +913,72 @@ int launch_dequantize(const MemRef& in, const MemRef& out, double scale, int64_t
         return convert_impl<int8_t, float>(in, out, DequantFn<int8_t, float, true>{scale, z}, s);
     return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "dequantize: %s -> %s is not implemented", dtype_name(in.dtype),
                 dtype_name(out.dtype));
+}
+
+
+// ---------------------------------------------------------------- dynamic_dequantize
+template <typename TQ, typename TS, typename TO>
+static int dyn_dequant_impl(const MemRef& in, const MemRef& scale, const MemRef* zp, const MemRef& out, hipStream_t s) {
+    NdIndex ix{};
+    int rc = fill_index(ix, 0, in, out, "dynamic_dequantize input");
+    if (rc) return rc;
+    rc = fill_index(ix, 1, scale, out, "dynamic_dequantize scale");
+    if (rc) return rc;
+    if (zp) {
+        rc = fill_index(ix, 2, *zp, out, "dynamic_dequantize zero point");
+        if (rc) return rc;
+    }
+    rc = fill_index(ix, 3, out, out, "dynamic_dequantize output");
+    if (rc) return rc;
+    int64_t n = out.numel();
+    if (n == 0) return VPX_RESULT_SUCCESS;
+    const uint8_t* pz = zp ? (const uint8_t*)zp->data : nullptr;
+    const int zp_signed = zp && zp->dtype == VPX_NN_I8 ? 1 : 0;
+    constexpr int VEC = 16 / (int)sizeof(TO);
+    bool vec = ix.dims[0] % VEC == 0 && ix.stride[0][0] == 1 && ix.stride[3][0] == 1 && ix.stride[1][0] == 0 &&
+               ix.stride[2][0] == 0 && (reinterpret_cast<uintptr_t>(in.data) % (VEC * sizeof(TQ))) == 0 && aligned16(out.data);
+    for (int d = 1; d < ix.nd && vec; d++) vec = ix.stride[0][d] % VEC == 0 && ix.stride[3][d] % VEC == 0;
+    unsigned blocks;
+    if (vec) {
+        ix.dims[0] /= VEC;
+        ix.stride[0][0] = VEC;
+        ix.stride[3][0] = VEC;
+        n /= VEC;
+        rc = grid_1d(n, &blocks);
+        if (rc) return rc;
+        hipLaunchKernelGGL((dyn_dequant_kernel<TQ, TS, TO, VEC>), dim3(blocks), dim3(kBlock), 0, s, (const TQ*)in.data,
+                           (const TS*)scale.data, pz, zp_signed, (TO*)out.data, ix, n);
+    } else {
+        rc = grid_1d(n, &blocks);
+        if (rc) return rc;
+        hipLaunchKernelGGL((dyn_dequant_kernel<TQ, TS, TO, 1>), dim3(blocks), dim3(kBlock), 0, s, (const TQ*)in.data,
+                           (const TS*)scale.data, pz, zp_signed, (TO*)out.data, ix, n);
+    }
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
+template <typename TQ, typename TS>
+static int dyn_dequant_out(const MemRef& in, const MemRef& scale, const MemRef* zp, const MemRef& out, hipStream_t s) {
+    if (out.dtype == VPX_NN_FP16) return dyn_dequant_impl<TQ, TS, half_t>(in, scale, zp, out, s);
+    return dyn_dequant_impl<TQ, TS, float>(in, scale, zp, out, s);
+}
+
+int launch_dynamic_dequantize(const MemRef& in, const MemRef& scale, const MemRef* zp, const MemRef& out, hipStream_t s) {
+    VPX_REQUIRE(in.dtype == VPX_NN_I8 || in.dtype == VPX_NN_U8, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "dynamic_dequantize: only I8 / U8 input is implemented, got %s", dtype_name(in.dtype));
+    VPX_REQUIRE(scale.dtype == VPX_NN_FP16 || scale.dtype == VPX_NN_FP32, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "dynamic_dequantize: scale must be FP16 or FP32, got %s", dtype_name(scale.dtype));
+    VPX_REQUIRE(out.dtype == VPX_NN_FP16 || out.dtype == VPX_NN_FP32, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "dynamic_dequantize: output must be FP16 or FP32, got %s", dtype_name(out.dtype));
+    if (zp)
+        VPX_REQUIRE(zp->dtype == VPX_NN_I8 || zp->dtype == VPX_NN_U8, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                    "dynamic_dequantize: only I8 / U8 zero points are implemented, got %s", dtype_name(zp->dtype));
+    VPX_REQUIRE(same_shape(in, out), VPX_RESULT_ERROR_INVALID_ARGUMENT, "dynamic_dequantize: input and output shapes differ");
+    const bool s16 = scale.dtype == VPX_NN_FP16;
+    if (in.dtype == VPX_NN_I8)
+        return s16 ? dyn_dequant_out<int8_t, half_t>(in, scale, zp, out, s) : dyn_dequant_out<int8_t, float>(in, scale, zp, out, s);
+    return s16 ? dyn_dequant_out<uint8_t, half_t>(in, scale, zp, out, s) : dyn_dequant_out<uint8_t, float>(in, scale, zp, out, s);
 }
 
 // ---------------------------------------------------------------- per-axis quantize / dequantize

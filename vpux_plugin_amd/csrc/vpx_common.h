@@ -106,6 +106,9 @@ int launch_softmax(const SoftmaxPlan& p, uint32_t dtype, const void* in, void* o
 int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool normalize_variance, float eps,
                hipStream_t s);
 
+// y = (q - zp) * scale with tensor scale / zero point that broadcast onto the input; zp may be null
+int launch_dynamic_dequantize(const MemRef& in, const MemRef& scale, const MemRef* zp, const MemRef& out, hipStream_t s);
+
 // MVN-1 decomposition (mvn1_sum -> mvn1_mean_var -> mvn1_norm)
 int launch_mvn_sum(const MemRef& in, const MemRef& out, bool across_channels, bool normalize_variance, hipStream_t s);
 int launch_mvn_mean_var(const MemRef& sum, const MemRef& out, const int64_t orig_shape[4], bool across_channels,

@@ -372,6 +372,14 @@ def mvn1_norm(x, mean_var, out, across_channels, normalize_variance, order="NCHW
     return out
 
 
+def dynamic_dequantize(q, scale, out, zero_point=None, order=None, stream=None):
+    """scale (fp16 / fp32) and the optional zero point (int8 / uint8) are tensors of q's rank that broadcast onto it."""
+    ins = [Operand(q, order), Operand(scale, order)] + ([Operand(zero_point, order)] if zero_point is not None else [])
+    ops = ins + [Operand(out, order)]
+    sw_kernel_launch("dynamic_dequantize", create_kernel_params(ins, ops[-1:], _i64(2 ** 63 - 1)), ops, stream)
+    return out
+
+
 def mvn6(x, out, axes, normalize_variance, eps, eps_mode=0, scale=None, bias=None, order=None, stream=None):
     """axes index x in memory order (outermost first), like torch dims; eps_mode 0 = inside the square root,
     1 = outside.  scale / bias: optional tensors of x's rank, broadcast NUMPY-style."""
