@@ -118,6 +118,30 @@ def test_naive_path_covers_odd_shapes_and_weight_zero_points(rt, orc, dev):
     assert name == "nce_conv_naive" and np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("geom,kernel", [
+    (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_tile"),
+    (dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_stream"),
+    (dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)), "nce_conv_mfma"),
+    (dict(N=1, H=12, W=12, IC=16, OC=32, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_mfma16"),
+    (dict(N=1, H=300, W=1, IC=128, OC=520, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_gemm_mfma"),
+])
+def test_unsigned_weights_around_128_take_the_mfma_kernels(rt, orc, dev, geom, kernel):
+    """u8 weights with zero point 128 are signed weights in unsigned storage: re-biased copy, same kernels."""
+    rng = np.random.default_rng(63)
+    g = dict(geom)
+    strides, pads = g.pop("strides"), g.pop("pads")
+    for in_u8, zp_in in ((True, 128), (True, 7), (False, -5)):
+        inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, w_u8=True, **g)
+        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, U8, zp_in=zp_in, zp_w=128, zp_out=3,
+                                   strides=strides, pads=pads)
+        assert name == kernel
+        assert np.array_equal(got, want), "%s zp_in=%d: %d mismatches" % (kernel, zp_in, int((got != want).sum()))
+    # any other zero point still takes the general kernel
+    inp, w, mults, shifts, bias = rand_case(rng, in_u8=True, w_u8=True, **g)
+    got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, U8, zp_in=128, zp_w=127, strides=strides, pads=pads)
+    assert name == "nce_conv_naive" and np.array_equal(got, want)
+
+
 @pytest.fixture(params=["8", "4"])
 def gemm_waves(request):
     """Both shapes of the matmul kernel: two waves per SIMD (64 x 128 each) and one (128 x 128)."""

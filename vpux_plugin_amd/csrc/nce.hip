@@ -1334,6 +1334,13 @@ int launch_nce_eltwise(const vpx_nce_task_t& t, const Ppe& ppe, hipStream_t s, c
     return VPX_RESULT_SUCCESS;
 }
 
+// u8 weights whose zero point is 128 (symmetric weights kept in unsigned storage) are the signed weights
+// w - 128: one pass flips the top bit of every byte into a scratch copy and the signed kernels run on that.
+__global__ __launch_bounds__(256) void nce_weights_to_s8_kernel(const i32x4* __restrict__ in, i32x4* __restrict__ out, int64_t n_vec) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_vec; i += (int64_t)gridDim.x * 256) out[i] = in[i] ^ (int32_t)0x80808080;
+}
+
+
 }  // namespace
 
 int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name) {
@@ -1370,7 +1377,9 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const bool zp_in_ok = in_u8 ? (t.zp_in >= 0 && t.zp_in <= 255) : (t.zp_in >= -128 && t.zp_in <= 127);
     // the fast epilogue adds the output zero point after limiting the scaled value to +-2^30
     const bool zp_out_ok = t.zp_out >= -(1 << 20) && t.zp_out <= (1 << 20);
-    const bool mfma_ok = !w_u8 && t.zp_w == 0 && zp_in_ok && zp_out_ok && Mtot < (1ll << 31) && g.OC < (1ll << 31);
+    // signed weights without a zero point, or unsigned ones around 128 (re-biased into a scratch copy below)
+    const bool w_rebias = w_u8 && t.zp_w == 128 && Ktot % 16 == 0;
+    const bool mfma_ok = ((!w_u8 && t.zp_w == 0) || w_rebias) && zp_in_ok && zp_out_ok && Mtot < (1ll << 31) && g.OC < (1ll << 31);
     const bool is_gemm = g.KY == 1 && g.KX == 1 && g.SY == 1 && g.SX == 1 && t.kernel_padding[0] == 0 &&
                          t.kernel_padding[1] == 0 && t.kernel_padding[2] == 0 && t.kernel_padding[3] == 0;
     const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights)) & 15) == 0;
@@ -1384,8 +1393,33 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     // A 256-column matmul tile wastes three quarters of its MFMAs on 64 output channels: such 1x1 layers go
     // to the convolution kernels, whose tiles are 64 channels wide (measured 7 us against 18 us at [100352 x 64 x 64]).
     const bool use_gemm = allow_gemm && is_gemm && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || Mtot < 1024);
+    const void* wptr = t.weights;  // the signed weights the MFMA kernels read
+    size_t wofs = 0;               // scratch bytes taken by their re-biased copy
+    const auto scratch = [&](size_t bytes, void** out) {
+        void* base = nullptr;
+        const int r = get_workspace(s, wofs + bytes, &base);
+        *out = (char*)base + wofs;
+        return r;
+    };
+    const auto rebias_weights = [&]() -> int {
+        if (!w_rebias) return VPX_RESULT_SUCCESS;
+        const size_t wbytes = (size_t)g.OC * (size_t)Ktot;
+        void* copy = nullptr;
+        const int r = get_workspace(s, (wbytes + 255) / 256 * 256, &copy);
+        if (r) return r;
+        const int64_t n_vec = (int64_t)(wbytes / 16);
+        const int64_t blocks = (n_vec + 255) / 256;
+        hipLaunchKernelGGL(nce_weights_to_s8_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, s,
+                           (const i32x4*)t.weights, (i32x4*)copy, n_vec);
+        VPX_HIP_CHECK(hipGetLastError());
+        wptr = copy;
+        wofs = (wbytes + 255) / 256 * 256;
+        return VPX_RESULT_SUCCESS;
+    };
     if (allow_mfma && mfma_ok && aligned && (use_gemm || g.IC % 32 == 0)) {
         int rc = VPX_RESULT_SUCCESS;
+        rc = rebias_weights();
+        if (rc) return rc;
         const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
         PpeFast pf;
         pf.zp_out = t.zp_out;
@@ -1410,11 +1444,11 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             int32_t* colsum = nullptr;
             if (corr != 0) {
                 void* ws = nullptr;
-                rc = get_workspace(s, sizeof(int32_t) * (size_t)g.OC, &ws);
+                rc = scratch(sizeof(int32_t) * (size_t)g.OC, &ws);
                 if (rc) return rc;
                 colsum = (int32_t*)ws;
                 hipLaunchKernelGGL(nce_colsum_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s,
-                                   (const int8_t*)t.weights, colsum, g.OC, Ktot);
+                                   (const int8_t*)wptr, colsum, g.OC, Ktot);
                 VPX_HIP_CHECK(hipGetLastError());
             }
 #define VPX_GEMM_W(U8, SGN, NW)                                                                                      \
@@ -1422,7 +1456,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         auto kern = nce_gemm_mfma<U8, SGN, NW>;                                                                      \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
-        hipLaunchKernelGGL(kern, grid, block, lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,              \
+        hipLaunchKernelGGL(kern, grid, block, lds, s, (const int8_t*)t.input, (const int8_t*)wptr,              \
                            t.weight_table, colsum, (uint8_t*)t.output, Mtot, g.OC, g.IC, tiles_m, tiles_n, gp);      \
     } while (0)
 #define VPX_GEMM(U8, SGN)                                                                                            \
@@ -1494,7 +1528,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         auto kern = nce_conv_tile<U8, TMW, SAME, ICS, NW>;                                                            \
         rc = set_dyn_lds(kern, lds);                                                                                  \
         if (rc) return rc;                                                                                            \
-        hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,       \
+        hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,       \
                            t.weight_table, (uint8_t*)t.output, g, pg, pad_byte, gp);                                  \
     } while (0)
 #define VPX_TILE(U8, TMW, SAME, ICS)                                                                                  \
@@ -1569,11 +1603,11 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     int32_t* colsum = nullptr;
                     if (corr != 0) {
                         void* ws = nullptr;
-                        rc = get_workspace(s, sizeof(int32_t) * (size_t)g.OC, &ws);
+                        rc = scratch(sizeof(int32_t) * (size_t)g.OC, &ws);
                         if (rc) return rc;
                         colsum = (int32_t*)ws;
                         hipLaunchKernelGGL(nce_colsum_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s,
-                                           (const int8_t*)t.weights, colsum, g.OC, Ktot);
+                                           (const int8_t*)wptr, colsum, g.OC, Ktot);
                         VPX_HIP_CHECK(hipGetLastError());
                     }
                     const int per_wave = (pg.MT + 8 / pg.nt - 1) / (8 / pg.nt);  // eight waves: at most 4 row blocks each
@@ -1582,7 +1616,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         auto kern = nce_conv_stream<U8, TMW, SAME, NW>;                                                               \
         rc = set_dyn_lds(kern, lds);                                                                                  \
         if (rc) return rc;                                                                                            \
-        hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,       \
+        hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,       \
                            t.weight_table, colsum, (uint8_t*)t.output, g, pg, sg, pad_byte, gp);                      \
     } while (0)
 #define VPX_STREAM(TMW, NW)                                                                                           \
@@ -1605,10 +1639,10 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         // Fallback: activation fragments gathered from global memory; per-channel parameters come
         // from a small preparation kernel.
         void* ws = nullptr;
-        rc = get_workspace(s, sizeof(ChanPrep) * (size_t)g.OC, &ws);
+        rc = scratch(sizeof(ChanPrep) * (size_t)g.OC, &ws);
         if (rc) return rc;
         ChanPrep* prep = (ChanPrep*)ws;
-        hipLaunchKernelGGL(nce_fold_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s, (const int8_t*)t.weights,
+        hipLaunchKernelGGL(nce_fold_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s, (const int8_t*)wptr,
                            t.weight_table, prep, g.OC, Ktot, corr, ppe);
         VPX_HIP_CHECK(hipGetLastError());
 
@@ -1626,7 +1660,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         auto kern = nce_conv_mfma<BM, BN, U8, SGN>;                                                                  \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights, prep,    \
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)wptr, prep,    \
                            (uint8_t*)t.output, g, pad_byte, swz, tc, icc, pf);                                       \
     } while (0)
         if (in_u8 && out_signed) VPX_CONV(true, true);
@@ -1649,19 +1683,21 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         if (pf.lo > tmax) pf.lo = tmax;
         if (pf.hi < tmin) pf.hi = tmin;
         if (pf.lo > pf.hi) pf.lo = pf.hi;
+        int rc = rebias_weights();
+        if (rc) return rc;
         void* ws = nullptr;
-        int rc = get_workspace(s, sizeof(ChanPrep) * (size_t)g.OC, &ws);
+        rc = scratch(sizeof(ChanPrep) * (size_t)g.OC, &ws);
         if (rc) return rc;
         ChanPrep* prep = (ChanPrep*)ws;
-        hipLaunchKernelGGL(nce_fold_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s, (const int8_t*)t.weights,
+        hipLaunchKernelGGL(nce_fold_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s, (const int8_t*)wptr,
                            t.weight_table, prep, g.OC, Ktot, corr, ppe);
         VPX_HIP_CHECK(hipGetLastError());
         const size_t lds = (size_t)64 * ((Ktot + 31) / 32 * 32 + 16);
         const dim3 grid((unsigned)((Mtot + 255) / 256), (unsigned)((g.OC + 63) / 64));
         const int pad_byte = t.zp_in & 0xff;
-        if (in_u8) hipLaunchKernelGGL(nce_conv_mfma16<true>, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,
+        if (in_u8) hipLaunchKernelGGL(nce_conv_mfma16<true>, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,
                                       prep, (uint8_t*)t.output, g, pad_byte, pf);
-        else hipLaunchKernelGGL(nce_conv_mfma16<false>, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)t.weights,
+        else hipLaunchKernelGGL(nce_conv_mfma16<false>, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,
                                 prep, (uint8_t*)t.output, g, pad_byte, pf);
         VPX_HIP_CHECK(hipGetLastError());
         *kernel_name = "nce_conv_mfma16";
