@@ -25,8 +25,9 @@ METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
 # Bytes moved through L2 per step, from rocprofv3 FETCH_SIZE / WRITE_SIZE counters scaled by a plain
 # copy of known size (profiles/<workload>__*.md hold the runs these come from).
 MEASURED_TRAFFIC = {
-    "c1_fake_quantize": 871101, "c2_softmax": 134269999, "c3_mvn": 25451430, "c4_conv": 16264736,
-    "c5_matmul": 384962929, "c5_dequantize": 135336726, "c5_eltwise_add": 270546244,
+    "c1_fake_quantize": 873999, "c2_softmax": 134297740, "c3_mvn": 25428126, "c4_conv": 16267937,
+    "c5_matmul": 384891258, "c5_dequantize": 135345881, "c5_eltwise_add": 270527001, "c5_nce_eltwise": 135250494,
+    "x_mvn6_layernorm": 268482311, "x_activation_hswish": 180552223, "x_mvn1_three_steps": 25333612,
 }
 
 
