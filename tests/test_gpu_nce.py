@@ -142,6 +142,32 @@ def test_unsigned_weights_around_128_take_the_mfma_kernels(rt, orc, dev, geom, k
     assert name == "nce_conv_naive" and np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("seed", [1234, 99])
+def test_conv_random_geometries(rt, orc, dev, seed):
+    """Thirty seeded draws of shape, kernel, stride, padding, types, zero points and PPE mode, whichever kernel they select."""
+    rng = np.random.default_rng(seed)
+    for i in range(30):
+        IC = int(rng.choice([16, 32, 48, 64, 64, 96, 128, 128, 192, 256, 320, 512]))
+        OC = int(rng.integers(1, 200))
+        KY, KX = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        SY, SX = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        pl, pr, pt, pb = [int(v) for v in rng.integers(0, 3, 4)]
+        pl, pr, pt, pb = min(pl, KX - 1), min(pr, KX - 1), min(pt, KY - 1), min(pb, KY - 1)
+        H, W, N = int(rng.integers(KY, 40)), int(rng.integers(KX, 70)), int(rng.integers(1, 4))
+        in_u8, out_signed = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        zp_in = int(rng.integers(0, 256)) if in_u8 else int(rng.integers(-128, 128))
+        mode = [rt.PPE_NOOP, rt.PPE_LPRELU, rt.PPE_LRELU][int(rng.integers(0, 3))]
+        kw = dict(I8 if out_signed else U8, lrelu_mult=int(rng.integers(0, 2048)), lrelu_shift=int(rng.integers(0, 20)))
+        what = "seed %d case %d: N=%d H=%d W=%d IC=%d OC=%d K=%dx%d S=%dx%d pads=%s in_u8=%s out_signed=%s zp_in=%d mode=%d" % (
+            seed, i, N, H, W, IC, OC, KY, KX, SY, SX, (pl, pr, pt, pb), in_u8, out_signed, zp_in, mode)
+        print(what, flush=True)
+        inp, w, mults, shifts, bias = rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=in_u8, shift_lo=14, shift_hi=26)
+        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_out=int(rng.integers(-5, 6)),
+                                   strides=(SY, SX), pads=(pl, pr, pt, pb), out_signed=out_signed, mode=mode)
+        assert name != "nce_conv_naive", what
+        assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))
+
+
 @pytest.fixture(params=["8", "4"])
 def gemm_waves(request):
     """Both shapes of the matmul kernel: two waves per SIMD (64 x 128 each) and one (128 x 128)."""
