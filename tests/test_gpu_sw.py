@@ -744,3 +744,77 @@ def test_mvn_rejects_bad_arguments(rt, dev):
     with pytest.raises(rt.VpxError) as e:
         rt.mvn(x4, torch.empty_like(x4), True, True, 1e-9)
     assert e.value.code == rt.ERROR_UNSUPPORTED_FEATURE
+
+
+# ---------------------------------------------------------------------------------- seeded random shapes
+
+def _random_shape(rng, nd, sizes, budget):
+    shape = []
+    for _ in range(nd):
+        m = max(1, min(int(rng.choice(sizes)), budget))
+        shape.append(m)
+        budget //= m
+    return tuple(shape)
+
+
+@pytest.mark.parametrize("seed", [7, 8])
+def test_random_shapes_softmax(rt, orc, dev, seed):
+    rng = np.random.default_rng(seed)
+    for i in range(40):
+        nd = int(rng.integers(1, 5))
+        shape = _random_shape(rng, nd, [1, 2, 3, 5, 8, 17, 64, 100, 257, 512, 1000, 4097], 300000)
+        axis = int(rng.integers(0, nd))
+        pad = int(rng.integers(0, min(4, shape[axis])))
+        print("seed %d case %d: shape %s axis %d pad %d" % (seed, i, shape, axis, pad), flush=True)
+        xb = orc.f32_to_f16(rng.normal(0, 3, shape).astype(np.float32))
+        want = orc.softmax_f16(xb, axis, pad=pad)
+        for packed in (True, False):
+            got = f16_bits(_softmax(rt, dev, xb, axis, pad=pad, packed=packed))
+            assert_close_f16(got.reshape(want.shape), want, orc, "softmax %s axis %d pad %d" % (shape, axis, pad))
+
+
+@pytest.mark.parametrize("seed", [7, 8])
+def test_random_shapes_eltwise_broadcast(rt, orc, dev, seed):
+    import torch
+    rng = np.random.default_rng(seed)
+    for i in range(40):
+        nd = int(rng.integers(1, 5))
+        shape = _random_shape(rng, nd, [1, 2, 3, 7, 8, 16, 24, 56, 64, 100, 256], 400000)
+        bshape = tuple(s if rng.random() < 0.5 else 1 for s in shape)
+        ashape = shape if rng.random() < 0.7 else tuple(s if rng.random() < 0.5 else 1 for s in shape)
+        oshape = tuple(max(a, b) for a, b in zip(ashape, bshape))
+        op = str(rng.choice(["add", "sub", "mul", "prelu"]))
+        print("seed %d case %d: %s %s %s" % (seed, i, op, ashape, bshape), flush=True)
+        a = orc.f32_to_f16(rng.normal(0, 2, ashape).astype(np.float32))
+        b = orc.f32_to_f16(rng.normal(0, 2, bshape).astype(np.float32))
+        out = torch.empty(oshape, dtype=torch.float16, device=dev)
+        if op == "prelu":
+            rt.prelu(to_dev(a, dev, True), to_dev(b, dev, True), out)
+        else:
+            rt.eltwise(op, to_dev(a, dev, True), to_dev(b, dev, True), out)
+        assert_f16_exact(f16_bits(out), orc.eltwise_f16(op, a, b), "%s %s %s" % (op, ashape, bshape))
+
+
+@pytest.mark.parametrize("seed", [7, 8])
+def test_random_shapes_mvn6(rt, orc, dev, seed):
+    import torch
+    rng = np.random.default_rng(seed)
+    for i in range(25):
+        nd = int(rng.integers(2, 5))
+        shape = tuple(int(rng.choice([1, 2, 3, 8, 16, 40, 64, 128])) for _ in range(nd))
+        axes = tuple(sorted(rng.choice(nd, size=int(rng.integers(1, nd + 1)), replace=False).tolist()))
+        sc_shape = tuple(s if rng.random() < 0.5 else 1 for s in shape) if rng.random() < 0.6 else None
+        bi_shape = tuple(s if rng.random() < 0.5 else 1 for s in shape) if rng.random() < 0.6 else None
+        mode = int(rng.integers(0, 2))
+        print("seed %d case %d: %s axes %s scale %s bias %s mode %d" % (seed, i, shape, axes, sc_shape, bi_shape, mode), flush=True)
+        x = orc.f32_to_f16(rng.normal(0.5, 2, shape).astype(np.float32))
+        sc = orc.f32_to_f16(rng.uniform(0.5, 2, sc_shape).astype(np.float32)) if sc_shape else None
+        bi = orc.f32_to_f16(rng.normal(0, 1, bi_shape).astype(np.float32)) if bi_shape else None
+        out = torch.empty(shape, dtype=torch.float16, device=dev)
+        rt.mvn6(to_dev(x, dev, True), out, axes, True, 1e-3, mode, scale=None if sc is None else to_dev(sc, dev, True),
+                bias=None if bi is None else to_dev(bi, dev, True))
+        g = orc.f16_to_f32(f16_bits(out)).astype(np.float64)
+        w = orc.f16_to_f32(orc.mvn6_f16(x, axes, True, 1e-3, mode, sc, bi)).astype(np.float64)
+        # rows of a few elements have statistics of a few values: absolute floor for results next to zero
+        assert np.all(np.abs(g - w) <= REL_TOL * np.abs(w) + 2e-4), (shape, axes, float(np.abs(g - w).max()))
+
