@@ -125,6 +125,8 @@ typedef enum vpx_softmax_mode_t {
  *       activation_elu {alpha}; activation_selu {alpha, lambda}; activation_swish {beta}; none for relu, negative,
  *       abs, hswish, hsigmoid, sigmoid, tanh, exp, sqrt, log, floor, ceil, sign, mish, softplus, gelu, erf
  *       (sw_kernel.cpp:650-941, 1266-1285, 1689-1845)
+ *   dynamic_quantize    in, out, scale, zeroPoint    | (none); f32 in, u8 out, one f32 scale and one u8 zero point, all three
+ *       written by the kernel (sw_kernel.cpp:1177-1179; arithmetic of ONNX DynamicQuantizeLinear)
  *   dynamic_dequantize  in, scale, [zeroPoint], out  | int64 INT64_MAX (ends the memref list; sw_kernel.cpp:1180-1183,
  *       sw_runtime_kernels/kernels/inc/common_types.h:141-151); out = (in - zeroPoint) * scale, scale and
  *       zero point broadcast onto the input

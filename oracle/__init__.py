@@ -239,6 +239,21 @@ def mvn_f16(x, across_channels, normalize_variance, eps, layout="NCHW"):
     return y
 
 
+def dynamic_quantize(x):
+    """VPU.DynamicQuantize (ops.td:6646-6660) with the arithmetic of ONNX DynamicQuantizeLinear, in float32: the range
+    [min(0, min x), max(0, max x)] maps onto 0..255; returns (uint8 values, float32 scale, uint8 zero point).
+    "parity unpinned": the reference holds the signature only; pinned by the ONNX specification's examples."""
+    x = np.asarray(x, dtype=np.float32)
+    with np.errstate(all="ignore"):
+        lo = np.float32(min(0.0, np.nanmin(x, initial=0.0)))
+        hi = np.float32(max(0.0, np.nanmax(x, initial=0.0)))
+        scale = np.float32(1.0) if hi == lo else np.float32((hi - lo) / np.float32(255.0))
+        zp = np.uint8(np.rint(np.clip(np.float32(0.0) - lo / scale, 0.0, 255.0)))
+        v = np.rint(x / scale) + np.float32(zp)
+        y = np.where(np.isnan(v), 0.0, np.clip(v, 0.0, 255.0)).astype(np.uint8)
+    return y, scale, zp
+
+
 def dynamic_dequantize(q, scale, zero_point=None, to_f16=True):
     """VPU.DynamicDequantize (ops.td:7780-7819): (q - zp) * scale with NUMPY-broadcast scale / zero-point tensors, in
     fp32, then the float16 class's rounding for fp16 output.  scale: float32 array or uint16 fp16 bits.

@@ -347,6 +347,25 @@ def test_quantize_per_axis_ambiguous_axis_is_refused(rt, dev):
         rt.quantize(x, torch.empty((4, 2, 4), dtype=torch.int8, device=dev), [0.1] * 3, [0] * 3)  # no dimension of size 3
 
 
+# ---------------------------------------------------------------------------------- dynamic_quantize
+
+@pytest.mark.parametrize("shape", [(6,), (3, 4), (1000, 1003), (4096, 1024), (2, 3, 5, 7), (1, 1), (0, 4)])
+def test_dynamic_quantize(rt, orc, dev, shape):
+    import torch
+    rng = np.random.default_rng(64)
+    for lo, hi in ((-3.0, 5.0), (1.0, 4.0), (-9.0, -2.0), (0.0, 0.0)):
+        x = rng.uniform(lo, hi, shape).astype(np.float32)
+        if x.size > 10:
+            x.flat[3] = np.nan  # takes no part in the range, quantizes to 0
+        out = torch.full(shape, 99, dtype=torch.uint8, device=dev)
+        scale = torch.zeros(1, dtype=torch.float32, device=dev)
+        zp = torch.zeros(1, dtype=torch.uint8, device=dev)
+        rt.dynamic_quantize(to_dev(x, dev), out, scale, zp)
+        wy, wsc, wzp = orc.dynamic_quantize(x)
+        assert scale.item() == wsc and zp.item() == wzp, (shape, lo, hi, scale.item(), wsc, zp.item(), wzp)
+        assert np.array_equal(out.cpu().numpy(), wy), (shape, lo, hi)
+
+
 # ---------------------------------------------------------------------------------- dynamic_dequantize
 
 DYN_DQ_CASES = [

@@ -545,3 +545,22 @@ def test_dynamic_dequantize_matches_static_golden_and_broadcasts(orc):
     stat = orc.dequantize(q, sc.ravel().astype(np.float64), zp.ravel().astype(np.int64), to_f16=True, axis=0)
     assert np.array_equal(orc.dynamic_dequantize(q, sc, zp), stat)
 
+
+def test_dynamic_quantize_onnx_examples(orc):
+    """The three worked examples of the ONNX DynamicQuantizeLinear specification."""
+    y, sc, zp = orc.dynamic_quantize(np.array([0, 2, -3, -2.5, 1.34, 0.5], np.float32))
+    assert np.isclose(sc, 0.0196078438) and zp == 153 and y.tolist() == [153, 255, 0, 26, 221, 179]
+    y, sc, zp = orc.dynamic_quantize(np.array([-1.0, -2.1, -1.3, -2.5, -3.34, -4.0], np.float32))
+    assert np.isclose(sc, 0.0156862754) and zp == 255 and y.tolist() == [191, 121, 172, 96, 42, 0]
+    y, sc, zp = orc.dynamic_quantize(np.array([1, 2.1, 1.3, 2.5, 3.34, 4.0, 1.5, 2.6, 3.9, 4.0, 3.0, 2.345], np.float32).reshape(3, 4))
+    assert np.isclose(sc, 0.0156862754) and zp == 0
+    assert y.ravel().tolist() == [64, 134, 83, 159, 213, 255, 96, 166, 249, 255, 191, 149]
+    y, sc, zp = orc.dynamic_quantize(np.zeros(5, np.float32))
+    assert sc == 1.0 and zp == 0 and not y.any()
+    # round trip: dequantized values are within half a step of the input
+    rng = np.random.default_rng(71)
+    x = rng.normal(0.3, 2, 10000).astype(np.float32)
+    y, sc, zp = orc.dynamic_quantize(x)
+    back = orc.dynamic_dequantize(y, np.full((1,), sc, np.float32), np.full((1,), zp, np.uint8), to_f16=False)
+    assert np.all(np.abs(back - x) <= 0.5 * sc * (1 + 1e-5))
+

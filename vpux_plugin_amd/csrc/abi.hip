@@ -304,7 +304,7 @@ struct Entry {
     int n_float_attrs;  // K_ACT: 32-bit float attributes that follow the memrefs
 };
 
-enum { K_CONVERT, K_ELTWISE, K_FQ, K_QUANT, K_DEQUANT, K_MVN, K_SOFTMAX, K_ACT, K_MVN_SUM, K_MVN_MEAN_VAR, K_MVN_NORM, K_MVN6, K_DYN_DEQUANT };
+enum { K_CONVERT, K_ELTWISE, K_FQ, K_QUANT, K_DEQUANT, K_MVN, K_SOFTMAX, K_ACT, K_MVN_SUM, K_MVN_MEAN_VAR, K_MVN_NORM, K_MVN6, K_DYN_DEQUANT, K_DYN_QUANT };
 
 const Entry kEntries[] = {
         {"convert", 1, 1, K_CONVERT, 0},
@@ -321,6 +321,7 @@ const Entry kEntries[] = {
         {"mvn1_sum", 1, 1, K_MVN_SUM, 0},
         {"mvn1_mean_var", 1, 1, K_MVN_MEAN_VAR, 0},
         {"mvn1_norm", 2, 1, K_MVN_NORM, 0},
+        {"dynamic_quantize", 1, 3, K_DYN_QUANT, 0},  // outputs: values, scale, zero point (sw_kernel.cpp:1177-1179)
         {"dynamic_dequantize", -1, 1, K_DYN_DEQUANT, 0},  // input, scale, optional zero point; list ends at an INT64_MAX word
         {"mvn6", -1, 1, K_MVN6, 0},  // input, optional scale, optional bias; the memref list ends at an INT64_MIN word
         {"softmax", 1, 1, K_SOFTMAX, 0},
@@ -467,6 +468,7 @@ int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_si
                     "mvn1_mean_var: params blob is too short for {origShape[4], acrossChannels, normalizeVariance, groupC, eps}");
         return launch_mvn_mean_var(a.mem[0], a.mem[1], shape, across != 0, normvar != 0, group_c, eps, s);
     }
+    case K_DYN_QUANT: return launch_dynamic_quantize(a.mem[0], a.mem[1], a.mem[2], a.mem[3], s);
     case K_DYN_DEQUANT: {
         VPX_REQUIRE(a.mem.size() == 3 || a.mem.size() == 4, VPX_RESULT_ERROR_INVALID_ARGUMENT,
                     "dynamic_dequantize: expects input, scale, an optional zero point and the output, got %zu memrefs", a.mem.size());

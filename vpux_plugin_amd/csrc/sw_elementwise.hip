@@ -471,6 +471,84 @@ __global__ __launch_bounds__(kBlock) void nd_unary_kernel(const TI* in, TO* out,
     out[off[1]] = fn(in[off[0]]);
 }
 
+// dynamic_quantize (VPU.DynamicQuantize, src/vpux_compiler/tblgen/vpux/compiler/dialect/VPU/ops.td:6646-6660: f32 in,
+// u8 out, one f32 scale, one u8 zero point).  The reference holds only the signature; the arithmetic is that of the
+// ONNX operator the op is imported from (DynamicQuantizeLinear): the range [min(0, min x), max(0, max x)] maps onto
+// 0..255, scale = range / 255 (1 for an all-zero tensor), zero point = rne(clamp(-min / scale)),
+// y = clamp(rne(x / scale) + zero point); NaNs do not take part in the range.
+struct MinMax {
+    float lo, hi;
+};
+__device__ __forceinline__ MinMax mm_merge(MinMax a, MinMax b) {
+    return MinMax{fminf(a.lo, b.lo), fmaxf(a.hi, b.hi)};
+}
+__device__ __forceinline__ MinMax mm_block(MinMax m, MinMax* smem) {
+    smem[threadIdx.x] = m;
+    __syncthreads();
+    for (int step = kBlock / 2; step > 0; step >>= 1) {
+        if ((int)threadIdx.x < step) smem[threadIdx.x] = mm_merge(smem[threadIdx.x], smem[threadIdx.x + step]);
+        __syncthreads();
+    }
+    return smem[0];
+}
+__global__ __launch_bounds__(kBlock) void dynq_range_kernel(const float* __restrict__ x, int64_t n, MinMax* __restrict__ partial) {
+    __shared__ MinMax smem[kBlock];
+    MinMax m{0.f, 0.f};
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+        const float v = x[i];
+        m.lo = fminf(m.lo, v);  // fminf / fmaxf return the other operand for a NaN
+        m.hi = fmaxf(m.hi, v);
+    }
+    m = mm_block(m, smem);
+    if (threadIdx.x == 0) partial[blockIdx.x] = m;
+}
+__global__ __launch_bounds__(kBlock) void dynq_params_kernel(const MinMax* __restrict__ partial, int count, float* __restrict__ scale,
+                                                             uint8_t* __restrict__ zp) {
+    __shared__ MinMax smem[kBlock];
+    MinMax m{0.f, 0.f};
+    for (int i = threadIdx.x; i < count; i += kBlock) m = mm_merge(m, partial[i]);
+    m = mm_block(m, smem);
+    if (threadIdx.x == 0) {
+        const float sc = m.hi == m.lo ? 1.0f : (m.hi - m.lo) / 255.0f;
+        const float z = fminf(fmaxf(0.0f - m.lo / sc, 0.0f), 255.0f);
+        *scale = sc;
+        *zp = (uint8_t)rintf(z);
+    }
+}
+struct DynQuantMap {
+    static constexpr int VEC = 4;
+    const float* __restrict__ in;
+    uint8_t* __restrict__ out;
+    const float* __restrict__ scale;
+    const uint8_t* __restrict__ zp;
+    __device__ __forceinline__ uint8_t q(float x, float sc, float z) const {
+        const float v = rintf(x / sc) + z;
+        return (uint8_t)fminf(fmaxf(v, 0.f), 255.f);  // NaN -> 0
+    }
+    template <int U>
+    __device__ __forceinline__ void vecs(int64_t v0, int64_t step) const {
+        const float sc = *scale, z = (float)*zp;
+        Pack<float, VEC> x[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) x[u].load(in, v0 + u * step);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            Pack<uint8_t, VEC> y;
+#pragma unroll
+            for (int k = 0; k < VEC; k++) y.set(k, q(x[u].get(k), sc, z));
+            y.store(out, v0 + u * step);
+        }
+    }
+    __device__ __forceinline__ void one(int64_t i) const {
+        out[i] = q(in[i], *scale, (float)*zp);
+    }
+};
+
+__global__ __launch_bounds__(kBlock) void dynq_scalar_kernel(DynQuantMap f, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) f.one(i);
+}
+
 // dynamic_dequantize: y = (q - zp) * scale with scale and zero point read from tensors that broadcast onto
 // the input (VPU.DynamicDequantize, src/vpux_compiler/tblgen/vpux/compiler/dialect/VPU/ops.td:7780-7819).
 // A lane takes VEC values along the innermost dimension; with VEC > 1 scale and zero point are constant along it
@@ -915,6 +993,39 @@ int launch_dequantize(const MemRef& in, const MemRef& out, double scale, int64_t
                 dtype_name(out.dtype));
 }
 
+
+// ---------------------------------------------------------------- dynamic_quantize
+int launch_dynamic_quantize(const MemRef& in, const MemRef& out, const MemRef& scale, const MemRef& zp, hipStream_t s) {
+    VPX_REQUIRE(in.dtype == VPX_NN_FP32 && out.dtype == VPX_NN_U8 && scale.dtype == VPX_NN_FP32 && zp.dtype == VPX_NN_U8,
+                VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "dynamic_quantize: expects FP32 -> U8 with an FP32 scale and a U8 zero point, got %s -> %s, %s, %s",
+                dtype_name(in.dtype), dtype_name(out.dtype), dtype_name(scale.dtype), dtype_name(zp.dtype));
+    VPX_REQUIRE(same_shape(in, out), VPX_RESULT_ERROR_INVALID_ARGUMENT, "dynamic_quantize: input and output shapes differ");
+    VPX_REQUIRE(scale.numel() == 1 && zp.numel() == 1, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "dynamic_quantize: scale and zero point are single values");
+    const int64_t n = in.numel();
+    VPX_REQUIRE(n == 0 || (in.compact && out.compact), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "dynamic_quantize: only compact tensors are supported");
+    int64_t blocks = (n + kBlock * 16 - 1) / (kBlock * 16);
+    if (blocks > 2048) blocks = 2048;
+    if (blocks < 1) blocks = 1;
+    void* ws = nullptr;
+    int rc = get_workspace(s, sizeof(MinMax) * (size_t)blocks, &ws);
+    if (rc) return rc;
+    hipLaunchKernelGGL(dynq_range_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, (const float*)in.data, n, (MinMax*)ws);
+    VPX_HIP_CHECK(hipGetLastError());
+    hipLaunchKernelGGL(dynq_params_kernel, dim3(1), dim3(kBlock), 0, s, (const MinMax*)ws, (int)blocks, (float*)scale.data,
+                       (uint8_t*)zp.data);
+    VPX_HIP_CHECK(hipGetLastError());
+    if (n == 0) return VPX_RESULT_SUCCESS;
+    DynQuantMap f{(const float*)in.data, (uint8_t*)out.data, (const float*)scale.data, (const uint8_t*)zp.data};
+    if (aligned16(in.data) && (reinterpret_cast<uintptr_t>(out.data) & 3) == 0) return launch_stream(f, n, s);
+    unsigned g;
+    rc = grid_1d(n, &g);
+    if (rc) return rc;
+    hipLaunchKernelGGL(dynq_scalar_kernel, dim3(g), dim3(kBlock), 0, s, f, n);
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
 
 // ---------------------------------------------------------------- dynamic_dequantize
 template <typename TQ, typename TS, typename TO>

@@ -106,6 +106,9 @@ int launch_softmax(const SoftmaxPlan& p, uint32_t dtype, const void* in, void* o
 int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool normalize_variance, float eps,
                hipStream_t s);
 
+// whole-tensor range -> one scale and zero point -> u8 values (ONNX DynamicQuantizeLinear arithmetic)
+int launch_dynamic_quantize(const MemRef& in, const MemRef& out, const MemRef& scale, const MemRef& zp, hipStream_t s);
+
 // y = (q - zp) * scale with tensor scale / zero point that broadcast onto the input; zp may be null
 int launch_dynamic_dequantize(const MemRef& in, const MemRef& scale, const MemRef* zp, const MemRef& out, hipStream_t s);
 

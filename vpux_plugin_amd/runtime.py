@@ -372,6 +372,13 @@ def mvn1_norm(x, mean_var, out, across_channels, normalize_variance, order="NCHW
     return out
 
 
+def dynamic_quantize(x, out, scale, zero_point, order=None, stream=None):
+    """x: float32; out: uint8 of x's shape; scale: float32[1]; zero_point: uint8[1] (all written by the kernel)."""
+    ops = [Operand(x, order), Operand(out, order), Operand(scale), Operand(zero_point)]
+    sw_kernel_launch("dynamic_quantize", create_kernel_params(ops[:1], ops[1:]), ops, stream)
+    return out, scale, zero_point
+
+
 def dynamic_dequantize(q, scale, out, zero_point=None, order=None, stream=None):
     """scale (fp16 / fp32) and the optional zero point (int8 / uint8) are tensors of q's rank that broadcast onto it."""
     ins = [Operand(q, order), Operand(scale, order)] + ([Operand(zero_point, order)] if zero_point is not None else [])
