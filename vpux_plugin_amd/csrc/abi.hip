@@ -301,7 +301,7 @@ struct Entry {
     int n_in, n_out;
     int kind;  // dispatch tag
     int op;
-    int n_float_attrs;  // K_ACT: 32-bit float attributes that follow the memrefs
+    int n_float_attrs = 0;  // K_ACT: 32-bit float attributes that follow the memrefs
 };
 
 enum { K_CONVERT, K_ELTWISE, K_FQ, K_QUANT, K_DEQUANT, K_MVN, K_SOFTMAX, K_ACT, K_MVN_SUM, K_MVN_MEAN_VAR, K_MVN_NORM, K_MVN6, K_DYN_DEQUANT, K_DYN_QUANT };

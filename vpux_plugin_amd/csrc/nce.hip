@@ -325,10 +325,7 @@ __device__ __forceinline__ int lds_offset(int row, int chunk) {
 // starts at the wave-uniform LDS byte address `lds_addr`, lane l at +16*l.  Issued as assembly so
 // that the compiler keeps managing only the counter of the LDS reads; completion of these loads is
 // awaited explicitly with dma_wait_all_and_barrier().
-__device__ __forceinline__ void dma16(const void* gptr, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
-}
-// same, the source given as a wave-uniform base plus a 32-bit per-lane byte offset
+// The source is a wave-uniform base plus a 32-bit per-lane byte offset.
 __device__ __forceinline__ void dma16(const void* gbase, unsigned goff, unsigned lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(goff), "s"(gbase) : "memory");
 }
