@@ -297,8 +297,28 @@ def make_mvn_steps(rt):
                     step, x.numel() * 4, 0, "hbm", "f16", "mvn_norm_runs_kernel")
 
 
+def make_int_mm(rt):
+    """The vendor library's int8 GEMM (torch._int_mm, hipBLASLt) on the C5 operands, int32 output and no PPE: the yardstick
+    for what this part sustains on uniform random int8 data, beside which nce_gemm_mfma is read."""
+    import torch
+    from vpux_plugin_amd import configs
+    c = configs.c5_matmul()
+    a, b_nk = _dev(c["a"]), _dev(c["b_nk"])
+    M, K = a.shape
+    N = b_nk.shape[0]
+    b = b_nk.t()
+    out = torch.empty((M, N), dtype=torch.int32, device="cuda")
+
+    def step():
+        torch._int_mm(a, b, out=out)
+    step.keep = (a, b_nk, out)
+    return Workload("calib_int_mm", "torch._int_mm (hipBLASLt) i8 [4096,4096] x [4096,11008] -> i32, no PPE (vendor yardstick)",
+                    step, 0, 2 * M * K * N, "mfma", "int8", "hipBLASLt")
+
+
 MAKERS = {
     "calib_copy": make_copy,
+    "calib_int_mm": make_int_mm,
     "c1_fake_quantize": make_c1,
     "c2_softmax": make_c2,
     "c3_mvn": make_c3,
@@ -463,7 +483,7 @@ def main():
     if args.all:
         others = {}
         for name in sorted(MAKERS):
-            if name == args.workload or name == "calib_copy":
+            if name == args.workload or name.startswith("calib_"):
                 continue
             del w
             torch.cuda.empty_cache()
