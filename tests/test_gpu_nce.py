@@ -168,12 +168,13 @@ def test_conv_random_geometries(rt, orc, dev, seed):
         assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))
 
 
-@pytest.fixture(params=["8", "4"])
+@pytest.fixture(params=[("8", "256"), ("4", "256"), ("4", "128")], ids=["8w256", "4w256", "4w128"])
 def gemm_waves(request):
-    """Both shapes of the matmul kernel: two waves per SIMD (64 x 128 each) and one (128 x 128)."""
-    os.environ["VPX_GEMM_WAVES"] = request.param
+    """The shapes of the matmul kernel: 256 x 256 tiles with two waves per SIMD (128 x 64 each) or one (128 x 128), and
+    128 x 128 tiles (four waves of 64 x 64), which small problems select by themselves."""
+    os.environ["VPX_GEMM_WAVES"], os.environ["VPX_GEMM_TILE"] = request.param
     yield request.param
-    del os.environ["VPX_GEMM_WAVES"]
+    del os.environ["VPX_GEMM_WAVES"], os.environ["VPX_GEMM_TILE"]
 
 
 @pytest.mark.parametrize("M,K,N", [(256, 64, 256), (300, 128, 520), (1, 64, 1), (513, 256, 77), (1024, 512, 768)])

@@ -376,7 +376,7 @@ struct GemmPpe {
 // so that the MFMAs of the second sub-step cover the first fragment reads of panel kt+1.  The column sums of B that the zero-point
 // term needs come from nce_colsum_kernel (only when that term is not zero), and the per-column PPE
 // parameters are unpacked from the weight table in the epilogue.
-template <bool IN_U8, bool OUT_SIGNED, int NW>
+template <bool IN_U8, bool OUT_SIGNED, int NW, int TILE = 256>
 __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restrict__ A, const int8_t* __restrict__ B,
                                                      const int32_t* __restrict__ wt, const int32_t* __restrict__ colsum,
                                                      uint8_t* __restrict__ out,
@@ -384,7 +384,10 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                                                      GemmPpe ppe) {
     // NW = 4: waves 2 x 2, 128 x 128 each, one per SIMD.  NW = 8: waves 2 x 4, 128 x 64 each, two per SIMD,
     // so that one wave's loads and address arithmetic issue while the other's MFMAs run.
-    constexpr int BM = 256, BN = 256, BK = 64, WM = 128, WN = NW == 4 ? 128 : 64, TM = 4, TN = WN / 32;
+    // TILE = 128 (four waves of 64 x 64, 64 KiB of LDS, two workgroups per CU) serves problems with too few 256 x 256 tiles.
+    constexpr int BM = TILE, BN = TILE, BK = 64, WM = BM / 2, WN = BN / (NW / 2), TM = WM / 32, TN = WN / 32;
+    constexpr int MFMA_PER_DMA = TM * TN / (BM * BK / 1024 / NW);  // MFMAs between two DMA instructions of a sub-step
+    static_assert(TM * TN >= TM + TN && MFMA_PER_DMA >= 1, "fragment reads and DMA instructions are interleaved with the MFMAs");
     constexpr int NT = 64 * NW;
     constexpr int NS = 4;                             // LDS panel buffers
     constexpr int CPR = BK / 16;                      // 16-byte chunks per tile row
@@ -457,9 +460,9 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
         else if (n <= TN) fb[slot][n - 1] = *reinterpret_cast<const i32x4*>(pa + BM * BK + lds_offset<BK>(wn0 + (n - 1) * 32 + (lane & 31), chunk));
         else fa[slot][n - TN] = *reinterpret_cast<const i32x4*>(pa + lds_offset<BK>(wm0 + (n - TN) * 32 + (lane & 31), chunk));
     };
-    // One sub-step: 16 MFMAs on fragment slot `cur`; between them, the 8 fragment reads of the next
-    // sub-step (panel at pnext, sub-step knext) into the other slot, DMA instructions dma0..dma0+3 of
-    // panel dma_p, and the column-sum update.
+    // One sub-step: the TM x TN MFMAs on fragment slot `cur`; between them, the TM + TN fragment reads of the
+    // next sub-step (panel at pnext, sub-step knext) into the other slot and this wave's DMA instructions
+    // dma0.. of panel dma_p.
     auto substep = [&](int cur, const uint8_t* pnext, int knext, int dma_p, int dma0) {
 #pragma unroll
         for (int i = 0; i < TM; i++) {
@@ -470,7 +473,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                 const int idx = i * TN + j;
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, fb[cur][j], acc[i][j], 0, 0, 0);
                 if (idx < TM + TN) load_frag(pnext, knext, cur ^ 1, idx);  // early: all back before the barrier
-                if ((idx & 3) == 3) dma_one(dma_p, dma0 + (idx >> 2));
+                if (idx % MFMA_PER_DMA == MFMA_PER_DMA - 1) dma_one(dma_p, dma0 + idx / MFMA_PER_DMA);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -544,7 +547,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     const bool vec_ok = (N & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
     for (int it = 0; it < BM * (BN / 16) / NT; it++) {
         const int cid = tid + NT * it;
-        const int row = cid >> 4, c16 = cid & 15;
+        const int row = cid / (BN / 16), c16 = cid % (BN / 16);
         const int64_t m = m0 + row, n = n0 + c16 * 16;
         if (m >= M || n >= N) continue;
         const i32x4 v = *reinterpret_cast<const i32x4*>(smem + row * kOutStride + c16 * 16);
@@ -1389,6 +1392,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
 
     // A 256-column matmul tile wastes three quarters of its MFMAs on 64 output channels: such 1x1 layers go
     // to the convolution kernels, whose tiles are 64 channels wide (measured 7 us against 18 us at [100352 x 64 x 64]).
+    const int64_t gemm_tiles = ((Mtot + 255) / 256) * ((g.OC + 255) / 256);
     const bool use_gemm = allow_gemm && is_gemm && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || Mtot < 1024);
     const void* wptr = t.weights;  // the signed weights the MFMA kernels read
     size_t wofs = 0;               // scratch bytes taken by their re-biased copy
@@ -1428,15 +1432,19 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         if (pf.lo > pf.hi) pf.lo = pf.hi;  // inverted window: max-then-min always ends at the upper bound
 
         if (use_gemm) {
-            constexpr int BM = 256, BN = 256;
-            const int tiles_m = (int)((Mtot + BM - 1) / BM), tiles_n = (int)((g.OC + BN - 1) / BN);
+            // 256 x 256 tiles when they fill the chip and K is long enough to amortise their prologue and epilogue;
+            // else 128 x 128 (four times as many, two workgroups per CU): [25088 x 512 x 128] 14.1 -> 7.8 us,
+            // [100352 x 256 x 128] 23.8 -> 14.4 us, [512 x 4096 x 4096] 43 -> 24 us.  VPX_GEMM_TILE=128|256 overrides.
+            const char* tenv = std::getenv("VPX_GEMM_TILE");
+            const int tile = tenv && *tenv ? (std::atoi(tenv) == 128 ? 128 : 256) : (gemm_tiles < 200 || g.IC <= 256 ? 128 : 256);
+            const int tiles_m = (int)((Mtot + tile - 1) / tile), tiles_n = (int)((g.OC + tile - 1) / tile);
             const int per_xcd = (tiles_m * tiles_n + 7) / 8;
             // Eight waves (two per SIMD) overlap the PPE epilogue better and win up to K = 4096; beyond
             // that the lower LDS traffic of four 128x128 waves wins.  VPX_GEMM_WAVES=4|8 overrides.
             const char* wenv = std::getenv("VPX_GEMM_WAVES");
-            const int nw = wenv && *wenv ? (std::atoi(wenv) == 4 ? 4 : 8) : (g.IC > 4096 ? 4 : 8);
+            const int nw = tile == 128 ? 4 : (wenv && *wenv ? (std::atoi(wenv) == 4 ? 4 : 8) : (g.IC > 4096 ? 4 : 8));
             const dim3 grid((unsigned)(per_xcd * 8)), block(64 * nw);
-            const size_t lds = 4 * (BM + BN) * 64;  // four K panels; the output staging tile reuses them
+            const size_t lds = 4 * (size_t)(tile + tile) * 64;  // four K panels; the output staging tile reuses them
             GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
             int32_t* colsum = nullptr;
             if (corr != 0) {
@@ -1448,9 +1456,9 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                                    (const int8_t*)wptr, colsum, g.OC, Ktot);
                 VPX_HIP_CHECK(hipGetLastError());
             }
-#define VPX_GEMM_W(U8, SGN, NW)                                                                                      \
+#define VPX_GEMM_W(U8, SGN, NW, TILE)                                                                                \
     do {                                                                                                             \
-        auto kern = nce_gemm_mfma<U8, SGN, NW>;                                                                      \
+        auto kern = nce_gemm_mfma<U8, SGN, NW, TILE>;                                                                \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
         hipLaunchKernelGGL(kern, grid, block, lds, s, (const int8_t*)t.input, (const int8_t*)wptr,              \
@@ -1458,8 +1466,9 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     } while (0)
 #define VPX_GEMM(U8, SGN)                                                                                            \
     do {                                                                                                             \
-        if (nw == 4) VPX_GEMM_W(U8, SGN, 4);                                                                         \
-        else VPX_GEMM_W(U8, SGN, 8);                                                                                 \
+        if (tile == 128) VPX_GEMM_W(U8, SGN, 4, 128);                                                                \
+        else if (nw == 4) VPX_GEMM_W(U8, SGN, 4, 256);                                                               \
+        else VPX_GEMM_W(U8, SGN, 8, 256);                                                                            \
     } while (0)
             if (in_u8 && out_signed) VPX_GEMM(true, true);
             else if (in_u8) VPX_GEMM(true, false);
