@@ -436,13 +436,15 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     const int8_t* bbase = B + n0 * K;
     const unsigned lds0 = lds_address(smem);
     const int nk = (int)(K / BK);
-    // d-th DMA instruction (0..3 A, 4..7 B) of panel p; panels past the end re-fetch the last one into a
-    // buffer nobody reads, which keeps the number of loads in flight the same in every iteration
+    // d-th DMA instruction (first half A, second half B) of panel p.  Panels past the end keep the number of loads
+    // in flight the same in every iteration: every lane re-fetches the tile's first 16 bytes (one cache line for
+    // the whole instruction) into a buffer nobody reads.
     auto dma_one = [&](int p, int d) {
         const unsigned base = lds0 + (unsigned)((p & (NS - 1)) * STAGE);
-        const int64_t k0 = (int64_t)(p < nk ? p : nk - 1) * BK;
-        if (d < DMA_PER_WAVE) dma16(abase + k0, oa[d], base + (unsigned)((wave + NW * d) * 1024));
-        else dma16(bbase + k0, ob[d - DMA_PER_WAVE], base + (unsigned)(BM * BK + (wave + NW * (d - DMA_PER_WAVE)) * 1024));
+        const bool real = p < nk;
+        const int64_t k0 = real ? (int64_t)p * BK : 0;
+        if (d < DMA_PER_WAVE) dma16(abase + k0, real ? oa[d] : 0u, base + (unsigned)((wave + NW * d) * 1024));
+        else dma16(bbase + k0, real ? ob[d - DMA_PER_WAVE] : 0u, base + (unsigned)(BM * BK + (wave + NW * (d - DMA_PER_WAVE)) * 1024));
     };
 
     i32x16 acc[TM][TN];
