@@ -376,7 +376,7 @@ struct GemmPpe {
 // so that the MFMAs of the second sub-step cover the first fragment reads of panel kt+1.  The column sums of B that the zero-point
 // term needs come from nce_colsum_kernel (only when that term is not zero), and the per-column PPE
 // parameters are unpacked from the weight table in the epilogue.
-template <bool IN_U8, bool OUT_SIGNED, int NW, int TILE = 256>
+template <bool IN_U8, bool OUT_SIGNED, int NW, int TILE = 256, bool SHORTK = false>
 __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restrict__ A, const int8_t* __restrict__ B,
                                                      const int32_t* __restrict__ wt, const int32_t* __restrict__ colsum,
                                                      uint8_t* __restrict__ out,
@@ -385,6 +385,9 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     // NW = 4: waves 2 x 2, 128 x 128 each, one per SIMD.  NW = 8: waves 2 x 4, 128 x 64 each, two per SIMD,
     // so that one wave's loads and address arithmetic issue while the other's MFMAs run.
     // TILE = 128 (four waves of 64 x 64, 64 KiB of LDS, two workgroups per CU) serves problems with too few 256 x 256 tiles.
+    // SHORTK (K <= 192, three panels at most): all panels are fetched up front, nothing is pipelined and no panel buffer
+    // is reused, so the workgroup asks only for the LDS it touches and more of them fit a CU (a matmul this short is
+    // bound by its epilogue and stores, not by the MFMAs).
     constexpr int BM = TILE, BN = TILE, BK = 64, WM = BM / 2, WN = BN / (NW / 2), TM = WM / 32, TN = WN / 32;
     constexpr int MFMA_PER_DMA = TM * TN / (BM * BK / 1024 / NW);  // MFMAs between two DMA instructions of a sub-step
     static_assert(TM * TN >= TM + TN && MFMA_PER_DMA >= 1, "fragment reads and DMA instructions are interleaved with the MFMAs");
@@ -475,7 +478,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                 const int idx = i * TN + j;
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, fb[cur][j], acc[i][j], 0, 0, 0);
                 if (idx < TM + TN) load_frag(pnext, knext, cur ^ 1, idx);  // early: all back before the barrier
-                if (idx % MFMA_PER_DMA == MFMA_PER_DMA - 1) dma_one(dma_p, dma0 + idx / MFMA_PER_DMA);
+                if (!SHORTK && idx % MFMA_PER_DMA == MFMA_PER_DMA - 1) dma_one(dma_p, dma0 + idx / MFMA_PER_DMA);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -493,22 +496,40 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // keeps the count of loads in flight below exact
 
+    if (SHORTK) {
 #pragma unroll
-    for (int p = 0; p < NS - 1; p++)
+        for (int p = 0; p < NS - 1; p++)
+            if (p < nk) {
 #pragma unroll
-        for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * DMA_PER_WAVE) : "memory");  // panel 0 is in
+                for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
+            }
+        dma_wait_all_and_barrier();
 #pragma unroll
-    for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
-    for (int kt = 0; kt < nk; kt++) {
-        const uint8_t* pcur = smem + (kt & (NS - 1)) * STAGE;
-        const uint8_t* pnxt = smem + ((kt + 1) & (NS - 1)) * STAGE;
-        substep(0, pcur, 1, kt + NS - 1, 0);
-        // Loads in flight here, oldest first: panel kt+1, panel kt+2 (2 * DMA_PER_WAVE each), half of panel kt+3.
-        // Behind the barrier panel kt+1 is complete for every wave and nobody reads panel kt-1 any
-        // more, whose buffer panel kt+3 is being written to.
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * DMA_PER_WAVE) : "memory");
-        substep(1, pnxt, 0, kt + NS - 1, DMA_PER_WAVE);
+        for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
+        for (int kt = 0; kt < nk; kt++) {
+            const uint8_t* pcur = smem + kt * STAGE;
+            const uint8_t* pnxt = kt + 1 < nk ? pcur + STAGE : pcur;  // the last step prefetches fragments nobody uses
+            substep(0, pcur, 1, 0, 0);
+            substep(1, pnxt, 0, 0, 0);
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < NS - 1; p++)
+#pragma unroll
+            for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * DMA_PER_WAVE) : "memory");  // panel 0 is in
+#pragma unroll
+        for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
+        for (int kt = 0; kt < nk; kt++) {
+            const uint8_t* pcur = smem + (kt & (NS - 1)) * STAGE;
+            const uint8_t* pnxt = smem + ((kt + 1) & (NS - 1)) * STAGE;
+            substep(0, pcur, 1, kt + NS - 1, 0);
+            // Loads in flight here, oldest first: panel kt+1, panel kt+2 (2 * DMA_PER_WAVE each), half of panel kt+3.
+            // Behind the barrier panel kt+1 is complete for every wave and nobody reads panel kt-1 any
+            // more, whose buffer panel kt+3 is being written to.
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * DMA_PER_WAVE) : "memory");
+            substep(1, pnxt, 0, kt + NS - 1, DMA_PER_WAVE);
+        }
     }
     dma_wait_all_and_barrier();  // every wave is done with the panels: LDS becomes the output staging tile
 
@@ -1446,7 +1467,13 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             const char* wenv = std::getenv("VPX_GEMM_WAVES");
             const int nw = tile == 128 ? 4 : (wenv && *wenv ? (std::atoi(wenv) == 4 ? 4 : 8) : (g.IC > 4096 ? 4 : 8));
             const dim3 grid((unsigned)(per_xcd * 8)), block(64 * nw);
-            const size_t lds = 4 * (size_t)(tile + tile) * 64;  // four K panels; the output staging tile reuses them
+            const int64_t nk = g.IC / 64;
+            const bool shortk = tile == 128 && nk <= 3;
+            size_t lds = 4 * (size_t)(tile + tile) * 64;  // four K panels; the output staging tile reuses them
+            if (shortk) {
+                lds = (size_t)nk * (tile + tile) * 64;  // only the panels there are ...
+                if (lds < (size_t)tile * kOutStride) lds = (size_t)tile * kOutStride;  // ... or the staging tile
+            }
             GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
             int32_t* colsum = nullptr;
             if (corr != 0) {
@@ -1458,9 +1485,9 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                                    (const int8_t*)wptr, colsum, g.OC, Ktot);
                 VPX_HIP_CHECK(hipGetLastError());
             }
-#define VPX_GEMM_W(U8, SGN, NW, TILE)                                                                                \
+#define VPX_GEMM_W(U8, SGN, NW, TILE, SHORTK)                                                                        \
     do {                                                                                                             \
-        auto kern = nce_gemm_mfma<U8, SGN, NW, TILE>;                                                                \
+        auto kern = nce_gemm_mfma<U8, SGN, NW, TILE, SHORTK>;                                                        \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
         hipLaunchKernelGGL(kern, grid, block, lds, s, (const int8_t*)t.input, (const int8_t*)wptr,              \
@@ -1468,9 +1495,10 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     } while (0)
 #define VPX_GEMM(U8, SGN)                                                                                            \
     do {                                                                                                             \
-        if (tile == 128) VPX_GEMM_W(U8, SGN, 4, 128);                                                                \
-        else if (nw == 4) VPX_GEMM_W(U8, SGN, 4, 256);                                                               \
-        else VPX_GEMM_W(U8, SGN, 8, 256);                                                                            \
+        if (shortk) VPX_GEMM_W(U8, SGN, 4, 128, true);                                                               \
+        else if (tile == 128) VPX_GEMM_W(U8, SGN, 4, 128, false);                                                    \
+        else if (nw == 4) VPX_GEMM_W(U8, SGN, 4, 256, false);                                                        \
+        else VPX_GEMM_W(U8, SGN, 8, 256, false);                                                                     \
     } while (0)
             if (in_u8 && out_signed) VPX_GEMM(true, true);
             else if (in_u8) VPX_GEMM(true, false);
