@@ -449,7 +449,7 @@ def main():
                          "Infinity Cache left there by the previous one (default 1: same buffers every step)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.exit("bench.py: this path runs on one GPU only (every kernel shards without exchange; see DESIGN.md); "
+        sys.exit("bench.py: this path runs on one GPU only (every kernel shards without exchange, so N GPUs would run N independent copies); "
                  "run it with --gpus 1")
     import torch
     if not torch.cuda.is_available():
