@@ -400,3 +400,66 @@ def test_chain_replayed_from_a_hip_graph(rt, orc, dev):
         chain(*scratch)  # eager work between replays, on the default stream
         torch.cuda.synchronize()
         assert torch.equal(scratch[2], eager[2])
+
+
+def test_two_host_threads_on_their_own_streams(rt, orc, dev):
+    """The launch functions keep no shared state but a per-(device, stream) workspace: two host threads, each on its own
+    stream, run the matmul (column-sum pre-pass in the workspace), MVN (chunk moments in the workspace) and softmax
+    many times over different data; every result must equal the one computed alone."""
+    import threading
+    import torch
+
+    def make(seed):
+        rng = np.random.default_rng(seed)
+        M, K, N = 384, 256, 320
+        d = {
+            "a": dev_t(rng.integers(-128, 128, (M, K)).astype(np.int8), dev),
+            "b": dev_t(rng.integers(-127, 128, (N, K)).astype(np.int8), dev),
+            "wt": dev_t(rt.make_weights_table(rng.integers(2 ** 14, 2 ** 15, N), rng.integers(20, 23, N),
+                                              rng.integers(-500, 500, N).astype(np.int32), K), dev),
+            "x": torch.from_numpy(rng.normal(0, 2, (2, 8, 64, 64)).astype(np.float16)).to(dev),
+            "s": torch.from_numpy(rng.normal(0, 3, (512, 512)).astype(np.float16)).to(dev),
+            "zp": int(seed % 5) + 1,
+        }
+        return d
+
+    ppe = rt.PpeInt(rt.PPE_LPRELU, -128, 127, 1638, 14)
+
+    def run(d, stream):
+        q = torch.empty((384, 320), dtype=torch.int8, device=dev)
+        y = torch.empty_like(d["x"])
+        p = torch.empty_like(d["s"])
+        rt.nce_matmul(d["a"], d["b"], d["wt"], q, ppe, zp_a=d["zp"], stream=stream)
+        rt.mvn(d["x"], y, True, True, 1e-6, stream=stream)
+        rt.softmax(d["s"], p, 1, stream=stream)
+        return q, y, p
+
+    data = [make(11), make(12)]
+    alone = []
+    for d in data:
+        out = run(d, torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        alone.append([t.clone() for t in out])
+    errors = []
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for it in range(40):
+                    out = run(data[i], stream)
+                    stream.synchronize()
+                    for got, want, what in zip(out, alone[i], ("matmul", "mvn", "softmax")):
+                        if not torch.equal(got, want):
+                            errors.append("thread %d iteration %d: %s differs" % (i, it, what))
+                            return
+        except Exception as e:  # surfaced by the assertion below
+            errors.append("thread %d: %r" % (i, e))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
