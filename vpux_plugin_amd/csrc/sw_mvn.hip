@@ -1141,6 +1141,12 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
     const half_t* pb = bias ? (const half_t*)bias->data : nullptr;
     const int nv = normalize_variance ? 1 : 0;
 
+    // Long contiguous rows of a compact tensor, eps inside the root, no scale or bias: the chunked two-launch
+    // scheme of mvn1 (a row is a group there).
+    if (innermost && row_len > 8192 && !scale && !bias && eps_mode == 0 && in.compact && out.compact) {
+        const bool aligned = row_len % 8 == 0 && ((reinterpret_cast<uintptr_t>(pi) | reinterpret_cast<uintptr_t>(po)) & 15) == 0;
+        return aligned ? launch_groups<true>(pi, po, g.rows, row_len, nv, eps, s) : launch_groups<false>(pi, po, g.rows, row_len, nv, eps, s);
+    }
     bool fast = innermost && row_len % 8 == 0 && row_len <= 8192;
     if (fast) {
         fast = along_row(true, g.rdim, g.r_in, g.nr) == 1 && along_row(true, g.rdim, g.r_out, g.nr) == 1;
