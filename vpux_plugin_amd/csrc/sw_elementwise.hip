@@ -425,12 +425,13 @@ struct FqVecFn {
     }
 };
 
-// createQuantizeFn, src/vpux_compiler/src/dialect/const/attributes/quantize.cpp:91-106
+// createQuantizeFn, src/vpux_compiler/src/dialect/const/attributes/quantize.cpp:91-106: the FakeQuantize onto
+// [qmin, qmax] with the limits of a launch prepared on the host (both divisions by constants, see div_const)
 template <typename TI, typename TQ>
 struct QuantFn {
-    float in_min, in_max, qmin, qmax, lm1;
+    FqConst c;
     __device__ __forceinline__ TQ operator()(TI x) const {
-        return (TQ)(int)fq_f32((float)x, in_min, in_max, qmin, qmax, lm1);
+        return (TQ)(int)fq_f32_const((float)x, c);
     }
 };
 
@@ -954,13 +955,19 @@ int launch_fake_quantize(const MemRef& in, const MemRef lims[4], const MemRef& o
 template <typename TI, typename TQ>
 static int quantize_impl(const MemRef& in, const MemRef& out, double scale, int64_t zp, int64_t qmin, int64_t qmax,
                          hipStream_t s) {
-    // Limits of the FakeQuantize the reference quantizer is built from (quantize.cpp:91-96).
+    // Limits of the FakeQuantize the reference quantizer is built from (quantize.cpp:91-96); the same float
+    // operations as the device's own preparation of a FakeQuantize (FqMap::prep).
     QuantFn<TI, TQ> fn;
-    fn.in_min = (float)((double)(qmin - zp) * scale);
-    fn.in_max = (float)((double)(qmax - zp) * scale);
-    fn.qmin = (float)qmin;
-    fn.qmax = (float)qmax;
-    fn.lm1 = (float)(qmax - qmin + 1) - 1.0f;
+    FqConst& c = fn.c;
+    c.ilo = (float)((double)(qmin - zp) * scale);
+    c.ihi = (float)((double)(qmax - zp) * scale);
+    c.olo = (float)qmin;
+    c.ohi = (float)qmax;
+    c.lm1 = (float)(qmax - qmin + 1) - 1.0f;
+    c.irange = c.ihi - c.ilo;
+    c.r_irange = 1.0f / c.irange;
+    c.r_lm1 = 1.0f / c.lm1;
+    c.orange = c.ohi - c.olo;
     return convert_impl<TI, TQ>(in, out, fn, s);
 }
 
