@@ -313,7 +313,10 @@ def test_quantize_dequantize(rt, orc, dev, signed, scale, zp):
 
 
 @pytest.mark.parametrize("shape,axis,order", [((2, 6, 5, 7), 1, "NCHW"), ((3, 300, 4, 4), 1, "NCHW"), ((2, 5, 7, 6), 3, "NHWC"),
-                                              ((8, 8, 3, 3), 1, "NCHW"), ((16, 64), 1, None), ((700, 3), 0, None)])
+                                              ((8, 8, 3, 3), 1, "NCHW"), ((16, 64), 1, None), ((700, 3), 0, None),
+                                              # one vector per lane: channels shared by a vector, or consecutive channels
+                                              ((4, 24, 8, 16), 1, "NCHW"), ((33, 7, 128), 0, None), ((50, 72), 1, None),
+                                              ((2, 9, 11, 40), 3, "NHWC"), ((300, 1024), 0, None)])
 def test_quantize_dequantize_per_axis(rt, orc, dev, shape, axis, order):
     """One scale / zero point per slice of `axis`.  The blob does not name the axis: it is the dimension
     whose size equals the parameter count, and the channel dimension when several have it ((8, 8, 3, 3))."""
@@ -335,6 +338,17 @@ def test_quantize_dequantize_per_axis(rt, orc, dev, shape, axis, order):
     rt.dequantize(q, y32, scales, zps, order=order)
     f32scales = scales.astype(np.float32).astype(np.float64)
     assert np.array_equal(y32.cpu().numpy(), orc.dequantize(want, f32scales, zps, to_f16=False, axis=axis))
+    # same call again (the parameter table is already on the device), then other parameters of the same count
+    rt.quantize(to_dev(x, dev, True), q, scales, zps, order=order)
+    assert np.array_equal(q.cpu().numpy(), want)
+    scales2 = scales[::-1].copy()
+    shipped2 = orc.f16_to_f32(orc.f32_to_f16(scales2.astype(np.float32))).astype(np.float64)
+    rt.quantize(to_dev(x, dev, True), q, scales2, zps, order=order)
+    assert np.array_equal(q.cpu().numpy(), orc.quantize(x, shipped2, zps, True, axis=axis))
+    x32 = rng.normal(0, 3, shape).astype(np.float32)
+    q32 = torch.empty(shape, dtype=torch.uint8, device=dev)
+    rt.quantize(to_dev(x32, dev), q32, scales, zps + 100, order=order)
+    assert np.array_equal(q32.cpu().numpy(), orc.quantize(x32, f32scales, zps + 100, False, axis=axis))
 
 
 def test_quantize_per_axis_ambiguous_axis_is_refused(rt, dev):

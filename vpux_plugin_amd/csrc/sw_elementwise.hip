@@ -8,6 +8,10 @@
 
 #include "vpx_common.h"
 
+#include <cstring>
+#include <mutex>
+#include <vector>
+
 namespace vpx {
 
 namespace {
@@ -1113,8 +1117,10 @@ struct AxisChunk {
 
 // Kernel arguments are the one path from host to device memory that a caller's graph capture can
 // record: the per-channel table goes to the workspace 256 entries per launch.
-__global__ __launch_bounds__(256) void fill_axis_table(float2* table, AxisChunk c, int count) {
-    if ((int)threadIdx.x < count) table[threadIdx.x] = float2{c.a[threadIdx.x], c.b[threadIdx.x]};
+__global__ __launch_bounds__(256) void fill_axis_table(float4* table, AxisChunk c, int count) {
+    // {a, b, b - a, 1 / (b - a)}: the last two are the constants of a channel's FakeQuantize (unused by dequantize)
+    const float lo = c.a[threadIdx.x], hi = c.b[threadIdx.x];
+    if ((int)threadIdx.x < count) table[threadIdx.x] = float4{lo, hi, hi - lo, 1.0f / (hi - lo)};
 }
 
 struct AxisGeom {
@@ -1129,26 +1135,130 @@ __device__ __forceinline__ uint32_t axis_channel(uint32_t i, const AxisGeom& g) 
 // table entry: {in_min, in_max} of the channel's quantizer (quantize.cpp:91-96)
 template <typename TI, typename TQ>
 __global__ __launch_bounds__(kBlock) void quantize_axis_kernel(const TI* __restrict__ in, TQ* __restrict__ out,
-                                                               const float2* __restrict__ table, AxisGeom g, uint32_t n,
+                                                               const float4* __restrict__ table, AxisGeom g, uint32_t n,
                                                                float qmin, float qmax, float lm1) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
-    const float2 p = table[axis_channel(i, g)];
+    const float4 p = table[axis_channel(i, g)];
     out[i] = (TQ)(int)fq_f32((float)in[i], p.x, p.y, qmin, qmax, lm1);
 }
 
 // table entry: {scale, zero point as a float (an integer of at most 9 bits)}
 template <typename TQ, typename TO>
 __global__ __launch_bounds__(kBlock) void dequantize_axis_kernel(const TQ* __restrict__ in, TO* __restrict__ out,
-                                                                 const float2* __restrict__ table, AxisGeom g, uint32_t n) {
+                                                                 const float4* __restrict__ table, AxisGeom g, uint32_t n) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
-    const float2 p = table[axis_channel(i, g)];
+    const float4 p = table[axis_channel(i, g)];
     out[i] = narrow<TO>((float)((double)((int)in[i] - (int)p.y) * (double)p.x));
 }
 
+// One 128-bit access of the wider operand per lane: the axis is not the innermost dimension and the run below it is
+// a multiple of the vector, so a lane's values share a channel, whose FakeQuantize constants come from its table entry.
+template <typename TI, typename TQ>
+__global__ __launch_bounds__(kBlock) void quantize_axis_vec_kernel(const TI* __restrict__ in, TQ* __restrict__ out,
+                                                                   const float4* __restrict__ table, AxisGeom g, uint32_t n_vec,
+                                                                   float qmin, float qmax, float lm1) {
+    constexpr int V = 16 / (int)sizeof(TI);
+    const uint32_t v = blockIdx.x * kBlock + threadIdx.x;
+    if (v >= n_vec) return;
+    Pack<TI, V> x;
+    x.load(in, v);
+    Pack<TQ, V> y;
+    const float4 p = table[axis_channel(v * V, g)];
+    const FqConst c{p.x, p.y, qmin, qmax, lm1, p.z, p.w, 1.0f / lm1, qmax - qmin};
+#pragma unroll
+    for (int k = 0; k < V; k++) y.set(k, (TQ)(int)fq_f32_const((float)x.get(k), c));
+    y.store(out, v);
+}
+
+template <typename TQ, typename TO>
+__global__ __launch_bounds__(kBlock) void dequantize_axis_vec_kernel(const TQ* __restrict__ in, TO* __restrict__ out,
+                                                                     const float4* __restrict__ table, AxisGeom g, uint32_t n_vec) {
+    constexpr int V = 16 / (int)sizeof(TO);
+    const uint32_t v = blockIdx.x * kBlock + threadIdx.x;
+    if (v >= n_vec) return;
+    Pack<TQ, V> x;
+    x.load(in, v);
+    const float4 p = table[axis_channel(v * V, g)];
+    float r[V];
+#pragma unroll
+    for (int k = 0; k < V; k++) r[k] = (float)((double)((int)x.get(k) - (int)p.y) * (double)p.x);
+    Pack<TO, V> y;
+    if constexpr (std::is_same<TO, half_t>::value) {
+        half_t h[V];
+        narrow_vec(r, h);
+#pragma unroll
+        for (int k = 0; k < V; k++) y.set(k, h[k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < V; k++) y.set(k, r[k]);
+    }
+    y.store(out, v);
+}
+
+// The axis is the innermost dimension: a lane takes one channel (its table entry is read, and its FakeQuantize
+// constants prepared, once) and walks kAxisRows rows; the 64 lanes of a wavefront touch 64 adjacent values of a row.
+constexpr int kAxisRows = 16;
+template <typename TI, typename TQ>
+__global__ __launch_bounds__(kBlock) void quantize_axis_inner_kernel(const TI* __restrict__ in, TQ* __restrict__ out,
+                                                                     const float4* __restrict__ table, uint32_t count, uint32_t rows,
+                                                                     float qmin, float qmax, float lm1) {
+    const uint32_t ctiles = (count + kBlock - 1) / kBlock;
+    const uint32_t c = (blockIdx.x % ctiles) * kBlock + threadIdx.x;
+    const uint32_t r0 = (blockIdx.x / ctiles) * kAxisRows;
+    if (c >= count) return;
+    const float4 p = table[c];
+    const FqConst cst{p.x, p.y, qmin, qmax, lm1, p.z, p.w, 1.0f / lm1, qmax - qmin};
+    TI x[kAxisRows];
+#pragma unroll
+    for (int r = 0; r < kAxisRows; r++) x[r] = r0 + r < rows ? in[(r0 + r) * count + c] : (TI)0;
+#pragma unroll
+    for (int r = 0; r < kAxisRows; r++)
+        if (r0 + r < rows) out[(r0 + r) * count + c] = (TQ)(int)fq_f32_const((float)x[r], cst);
+}
+
+template <typename TQ, typename TO>
+__global__ __launch_bounds__(kBlock) void dequantize_axis_inner_kernel(const TQ* __restrict__ in, TO* __restrict__ out,
+                                                                       const float4* __restrict__ table, uint32_t count, uint32_t rows) {
+    const uint32_t ctiles = (count + kBlock - 1) / kBlock;
+    const uint32_t c = (blockIdx.x % ctiles) * kBlock + threadIdx.x;
+    const uint32_t r0 = (blockIdx.x / ctiles) * kAxisRows;
+    const bool live = c < count;
+    const float4 p = live ? table[c] : float4{0.f, 0.f, 0.f, 0.f};
+    float v[kAxisRows];
+#pragma unroll
+    for (int r = 0; r < kAxisRows; r++) {
+        const int q = live && r0 + r < rows ? (int)in[(r0 + r) * count + c] : 0;
+        v[r] = (float)((double)(q - (int)p.y) * (double)p.x);
+    }
+    if constexpr (std::is_same<TO, half_t>::value) {
+        half_t h[kAxisRows];
+        narrow_vec(v, h);  // every lane of the wavefront takes part in the vote
+#pragma unroll
+        for (int r = 0; r < kAxisRows; r++)
+            if (live && r0 + r < rows) out[(r0 + r) * count + c] = h[r];
+    } else {
+#pragma unroll
+        for (int r = 0; r < kAxisRows; r++)
+            if (live && r0 + r < rows) out[(r0 + r) * count + c] = v[r];
+    }
+}
+
+// Tables already on the device, by content: the parameters of a layer are constants, so after the first call a
+// per-axis launch is one kernel.  Entries are per (device, stream) like the workspace, and live until the process ends.
+struct AxisTableEntry {
+    int dev;
+    hipStream_t stream;
+    std::vector<float> a, b;
+    float4* table;
+};
+std::mutex g_axis_mutex;
+std::vector<AxisTableEntry> g_axis_tables;
+constexpr size_t kMaxAxisTables = 64;
+
 int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t n, const float* a, const float* b, hipStream_t s,
-               AxisGeom& g, float2** table) {
+               AxisGeom& g, float4** table) {
     VPX_REQUIRE(ref.compact && other.compact, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: per-axis form needs compact operands", what);
     VPX_REQUIRE(ref.numel() < (1ll << 32), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: tensor of %lld elements is too large", what,
                 (long long)ref.numel());
@@ -1177,10 +1287,27 @@ int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t
     g.count = (uint32_t)n;
     g.m_inner = magic((uint64_t)inner);
     g.m_count = magic((uint64_t)n);
-    void* ws = nullptr;
-    int rc = get_workspace(s, sizeof(float2) * (size_t)n, &ws);
-    if (rc) return rc;
-    *table = (float2*)ws;
+    int dev = 0;
+    VPX_HIP_CHECK(hipGetDevice(&dev));
+    bool keep = false;
+    {
+        std::lock_guard<std::mutex> lock(g_axis_mutex);
+        for (const AxisTableEntry& e : g_axis_tables)
+            if (e.dev == dev && e.stream == s && (int64_t)e.a.size() == n && memcmp(e.a.data(), a, sizeof(float) * (size_t)n) == 0 &&
+                memcmp(e.b.data(), b, sizeof(float) * (size_t)n) == 0) {
+                *table = e.table;
+                return VPX_RESULT_SUCCESS;
+            }
+        keep = g_axis_tables.size() < kMaxAxisTables;
+    }
+    void* mem = nullptr;
+    if (keep) {
+        VPX_HIP_CHECK(hipMalloc(&mem, sizeof(float4) * (size_t)n));
+    } else {
+        const int rc = get_workspace(s, sizeof(float4) * (size_t)n, &mem);
+        if (rc) return rc;
+    }
+    *table = (float4*)mem;
     for (int64_t c0 = 0; c0 < n; c0 += 256) {
         AxisChunk ch;
         const int cnt = (int)(n - c0 < 256 ? n - c0 : 256);
@@ -1191,6 +1318,10 @@ int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t
         for (int k = cnt; k < 256; k++) ch.a[k] = ch.b[k] = 0.f;
         hipLaunchKernelGGL(fill_axis_table, dim3(1), dim3(256), 0, s, *table + c0, ch, cnt);
         VPX_HIP_CHECK(hipGetLastError());
+    }
+    if (keep) {
+        std::lock_guard<std::mutex> lock(g_axis_mutex);
+        g_axis_tables.push_back(AxisTableEntry{dev, s, std::vector<float>(a, a + n), std::vector<float>(b, b + n), *table});
     }
     return VPX_RESULT_SUCCESS;
 }
@@ -1206,13 +1337,27 @@ int quantize_axis_impl(const MemRef& in, const MemRef& out, const double* scales
         hi[(size_t)c] = (float)((double)(qmax - zps[c]) * scales[c]);
     }
     AxisGeom g;
-    float2* table = nullptr;
+    float4* table = nullptr;
     int rc = axis_setup("quantize", in, out, n, lo.data(), hi.data(), s, g, &table);
     if (rc) return rc;
     const uint32_t total = (uint32_t)in.numel();
     if (total == 0) return VPX_RESULT_SUCCESS;
-    hipLaunchKernelGGL((quantize_axis_kernel<TI, TQ>), dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (const TI*)in.data,
-                       (TQ*)out.data, table, g, total, (float)qmin, (float)qmax, (float)(qmax - qmin + 1) - 1.0f);
+    const float fmin_ = (float)qmin, fmax_ = (float)qmax, lm1 = (float)(qmax - qmin + 1) - 1.0f;
+    constexpr uint32_t V = 16 / sizeof(TI);
+    const bool al = (reinterpret_cast<uintptr_t>(in.data) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.data) % V) == 0;
+    const dim3 vgrid((total / V + kBlock - 1) / kBlock);
+    if (al && g.inner % V == 0)
+        hipLaunchKernelGGL((quantize_axis_vec_kernel<TI, TQ>), vgrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data, table,
+                           g, total / V, fmin_, fmax_, lm1);
+    else if (g.inner == 1) {
+        const uint32_t rows = total / g.count;
+        const dim3 igrid(((g.count + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
+        hipLaunchKernelGGL((quantize_axis_inner_kernel<TI, TQ>), igrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data, table, g.count,
+                           rows, fmin_, fmax_, lm1);
+    }
+    else
+        hipLaunchKernelGGL((quantize_axis_kernel<TI, TQ>), dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (const TI*)in.data,
+                           (TQ*)out.data, table, g, total, fmin_, fmax_, lm1);
     VPX_HIP_CHECK(hipGetLastError());
     return VPX_RESULT_SUCCESS;
 }
@@ -1225,13 +1370,26 @@ int dequantize_axis_impl(const MemRef& in, const MemRef& out, const double* scal
         zp[(size_t)c] = (float)zps[c];
     }
     AxisGeom g;
-    float2* table = nullptr;
+    float4* table = nullptr;
     int rc = axis_setup("dequantize", out, in, n, sc.data(), zp.data(), s, g, &table);
     if (rc) return rc;
     const uint32_t total = (uint32_t)in.numel();
     if (total == 0) return VPX_RESULT_SUCCESS;
-    hipLaunchKernelGGL((dequantize_axis_kernel<TQ, TO>), dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (const TQ*)in.data,
-                       (TO*)out.data, table, g, total);
+    constexpr uint32_t V = 16 / sizeof(TO);
+    const bool al = (reinterpret_cast<uintptr_t>(in.data) % V) == 0 && (reinterpret_cast<uintptr_t>(out.data) & 15) == 0;
+    const dim3 vgrid((total / V + kBlock - 1) / kBlock);
+    if (al && g.inner % V == 0)
+        hipLaunchKernelGGL((dequantize_axis_vec_kernel<TQ, TO>), vgrid, dim3(kBlock), 0, s, (const TQ*)in.data, (TO*)out.data,
+                           table, g, total / V);
+    else if (g.inner == 1) {
+        const uint32_t rows = total / g.count;
+        const dim3 igrid(((g.count + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
+        hipLaunchKernelGGL((dequantize_axis_inner_kernel<TQ, TO>), igrid, dim3(kBlock), 0, s, (const TQ*)in.data, (TO*)out.data, table,
+                           g.count, rows);
+    }
+    else
+        hipLaunchKernelGGL((dequantize_axis_kernel<TQ, TO>), dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (const TQ*)in.data,
+                           (TO*)out.data, table, g, total);
     VPX_HIP_CHECK(hipGetLastError());
     return VPX_RESULT_SUCCESS;
 }
