@@ -44,6 +44,11 @@ template <>
 struct Words<16> {
     typedef u32x4 type;
 };
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+template <>
+struct Words<32> {
+    typedef u32x8 type;  // two 128-bit accesses
+};
 
 // N elements of T moved by one 8...128-bit access per lane.  Adjacent lanes touch adjacent
 // words, so a wavefront's access is one contiguous run; the wider operand of a kernel gets the
@@ -558,22 +563,47 @@ __global__ __launch_bounds__(kBlock) void dynq_scalar_kernel(DynQuantMap f, int6
 // the input (VPU.DynamicDequantize, src/vpux_compiler/tblgen/vpux/compiler/dialect/VPU/ops.td:7780-7819).
 // A lane takes VEC values along the innermost dimension; with VEC > 1 scale and zero point are constant along it
 // (per-row or per-group scales of a weight matrix) and `ix` counts the innermost dimension in vectors.
-template <typename TQ, typename TS, typename TO, int VEC>
+// PER_VALUE: scale and zero point run along the innermost dimension with the values (per-column parameters): a lane
+// reads VEC of each, contiguous like its values.
+template <typename TQ, typename TS, typename TO, int VEC, bool PER_VALUE = false>
 __global__ __launch_bounds__(kBlock) void dyn_dequant_kernel(const TQ* __restrict__ in, const TS* __restrict__ scale,
                                                              const uint8_t* __restrict__ zp, int zp_signed, TO* __restrict__ out,
                                                              NdIndex ix, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
-    int64_t off[4];
-    nd_offsets<4>(ix, i, off);
-    const float sc = (float)scale[off[1]];
-    int z = 0;
-    if (zp) z = zp_signed ? (int)(int8_t)zp[off[2]] : (int)zp[off[2]];
+    int64_t off[4] = {0, 0, 0, 0};
+    if (n < (1ll << 32)) {  // 32-bit divisions: a quarter of the instructions of the 64-bit ones
+        uint32_t lin = (uint32_t)i;
+        for (int d = 0; d < ix.nd; d++) {
+            const uint32_t q = lin / (uint32_t)ix.dims[d];
+            const uint32_t r = lin - q * (uint32_t)ix.dims[d];
+            lin = q;
+#pragma unroll
+            for (int o = 0; o < 4; o++) off[o] += (int64_t)r * ix.stride[o][d];
+        }
+    } else {
+        nd_offsets<4>(ix, i, off);
+    }
     Pack<TQ, VEC> x;
     x.load(in + off[0], 0);
     float r[VEC];
+    if (PER_VALUE) {
+        Pack<TS, VEC> sc;
+        sc.load(scale + off[1], 0);
+        Pack<uint8_t, VEC> z;
+        if (zp) z.load(zp + off[2], 0);
 #pragma unroll
-    for (int k = 0; k < VEC; k++) r[k] = (float)((int)x.get(k) - z) * sc;
+        for (int k = 0; k < VEC; k++) {
+            const int zk = zp ? (zp_signed ? (int)(int8_t)z.get(k) : (int)z.get(k)) : 0;
+            r[k] = (float)((int)x.get(k) - zk) * (float)sc.get(k);
+        }
+    } else {
+        const float sc = (float)scale[off[1]];
+        int z = 0;
+        if (zp) z = zp_signed ? (int)(int8_t)zp[off[2]] : (int)zp[off[2]];
+#pragma unroll
+        for (int k = 0; k < VEC; k++) r[k] = (float)((int)x.get(k) - z) * sc;
+    }
     Pack<TO, VEC> y;
     if constexpr (std::is_same<TO, half_t>::value) {
         half_t h[VEC];
@@ -1057,19 +1087,33 @@ static int dyn_dequant_impl(const MemRef& in, const MemRef& scale, const MemRef*
     const uint8_t* pz = zp ? (const uint8_t*)zp->data : nullptr;
     const int zp_signed = zp && zp->dtype == VPX_NN_I8 ? 1 : 0;
     constexpr int VEC = 16 / (int)sizeof(TO);
-    bool vec = ix.dims[0] % VEC == 0 && ix.stride[0][0] == 1 && ix.stride[3][0] == 1 && ix.stride[1][0] == 0 &&
-               ix.stride[2][0] == 0 && (reinterpret_cast<uintptr_t>(in.data) % (VEC * sizeof(TQ))) == 0 && aligned16(out.data);
+    bool vec = ix.dims[0] % VEC == 0 && ix.stride[0][0] == 1 && ix.stride[3][0] == 1 &&
+               (reinterpret_cast<uintptr_t>(in.data) % (VEC * sizeof(TQ))) == 0 && aligned16(out.data);
     for (int d = 1; d < ix.nd && vec; d++) vec = ix.stride[0][d] % VEC == 0 && ix.stride[3][d] % VEC == 0;
+    // parameters constant along the innermost dimension (per row / per group), or running along it with the values
+    const bool per_row = ix.stride[1][0] == 0 && ix.stride[2][0] == 0;
+    bool per_value = ix.stride[1][0] == 1 && (!zp || ix.stride[2][0] == 1) &&
+                     (reinterpret_cast<uintptr_t>(scale.data) % (VEC * sizeof(TS))) == 0 && (!zp || reinterpret_cast<uintptr_t>(pz) % VEC == 0);
+    for (int d = 1; d < ix.nd && per_value; d++) per_value = ix.stride[1][d] % VEC == 0 && ix.stride[2][d] % VEC == 0;
+    vec = vec && (per_row || per_value);
     unsigned blocks;
     if (vec) {
         ix.dims[0] /= VEC;
         ix.stride[0][0] = VEC;
         ix.stride[3][0] = VEC;
+        if (!per_row) {
+            ix.stride[1][0] = VEC;
+            if (zp) ix.stride[2][0] = VEC;
+        }
         n /= VEC;
         rc = grid_1d(n, &blocks);
         if (rc) return rc;
-        hipLaunchKernelGGL((dyn_dequant_kernel<TQ, TS, TO, VEC>), dim3(blocks), dim3(kBlock), 0, s, (const TQ*)in.data,
-                           (const TS*)scale.data, pz, zp_signed, (TO*)out.data, ix, n);
+        if (per_row)
+            hipLaunchKernelGGL((dyn_dequant_kernel<TQ, TS, TO, VEC, false>), dim3(blocks), dim3(kBlock), 0, s, (const TQ*)in.data,
+                               (const TS*)scale.data, pz, zp_signed, (TO*)out.data, ix, n);
+        else
+            hipLaunchKernelGGL((dyn_dequant_kernel<TQ, TS, TO, VEC, true>), dim3(blocks), dim3(kBlock), 0, s, (const TQ*)in.data,
+                               (const TS*)scale.data, pz, zp_signed, (TO*)out.data, ix, n);
     } else {
         rc = grid_1d(n, &blocks);
         if (rc) return rc;
