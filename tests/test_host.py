@@ -28,8 +28,14 @@ def test_library_exports_every_declared_symbol(rt):
         assert getattr(L, name) is not None, name
     assert L.vpx_get_version() == 1
     names = [L.vpx_sw_kernel_name(i).decode() for i in range(L.vpx_sw_kernel_count())]
-    for must in ("softmax", "mvn1", "fake_quantize", "quantize", "dequantize", "convert", "eltwise_add"):
+    for must in ("softmax", "mvn1", "fake_quantize", "quantize", "dequantize", "convert", "eltwise_add", "mvn1_sum", "mvn1_mean_var",
+                 "mvn1_norm", "mvn6", "dynamic_quantize", "dynamic_dequantize", "prelu_fp16", "leaky_relu_fp16", "activation_relu",
+                 "activation_clamp"):
         assert must in names and L.vpx_sw_kernel_supported(must.encode()) == 1
+    # every entry the Python binding can name exists in the library
+    for entry, _ in rt.ACTIVATIONS.values():
+        assert entry in names, entry
+    assert len(names) == len(set(names))
     assert L.vpx_sw_kernel_supported(b"no_such_kernel") == 0
     assert L.vpx_sw_kernel_name(10 ** 6) is None
 
