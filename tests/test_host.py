@@ -66,6 +66,15 @@ def test_error_codes_without_gpu(rt):
     assert L.vpx_sw_kernel_launch(b"convert", blob, len(blob), addrs, 3, None) == rt.ERROR_INVALID_ARGUMENT
     assert L.vpx_sw_kernel_launch(b"convert", blob, 10, addrs, 2, None) == rt.ERROR_INVALID_ARGUMENT
     assert L.vpx_sw_kernel_launch(b"convert", blob, len(blob), addrs, 2, None) == rt.ERROR_INVALID_ARGUMENT
+    # kernels with optional operands find the end of their memref list by a marker word
+    assert L.vpx_sw_kernel_launch(b"mvn6", blob, len(blob), addrs, 2, None) == rt.ERROR_INVALID_ARGUMENT
+    assert b"marker" in L.vpx_get_last_error()
+    assert L.vpx_sw_kernel_launch(b"dynamic_dequantize", blob, len(blob), addrs, 2, None) == rt.ERROR_INVALID_ARGUMENT
+    marked = b"\0" * 36 + struct.pack("<q", 2 ** 63 - 1) + b"\0" * 28  # one memref, then the delimiter: too few operands
+    assert L.vpx_sw_kernel_launch(b"dynamic_dequantize", marked, len(marked), addrs, 1, None) == rt.ERROR_INVALID_ARGUMENT
+    # activation attributes must be present
+    short = b"\0" * 72
+    assert L.vpx_sw_kernel_launch(b"activation_clamp", short, len(short), addrs, 2, None) == rt.ERROR_INVALID_ARGUMENT
     assert L.vpx_nce_task(None, None) == rt.ERROR_INVALID_NULL_HANDLE
     t = rt.NceTask()
     assert L.vpx_nce_task(C.byref(t), None) == rt.ERROR_INVALID_NULL_HANDLE  # null buffers
