@@ -142,6 +142,29 @@ def test_unsigned_weights_around_128_take_the_mfma_kernels(rt, orc, dev, geom, k
     assert name == "nce_conv_naive" and np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("geom,kernel", [
+    (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_tile"),
+    (dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_stream"),
+    (dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)), "nce_conv_mfma"),
+    (dict(N=1, H=300, W=1, IC=128, OC=520, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_gemm_mfma"),
+    (dict(N=1, H=700, W=1, IC=512, OC=300, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_gemm_mfma"),
+])
+@pytest.mark.parametrize("mode", ["NOOP", "LPRELU", "LRELU"])
+def test_negative_multipliers(rt, orc, dev, geom, kernel, mode):
+    """Channels whose multiplier is negative (a negative weight scale): the scaled value changes sign, and with it the
+    branch of the PReLU stage a given accumulator takes."""
+    rng = np.random.default_rng(66)
+    g = dict(geom)
+    strides, pads = g.pop("strides"), g.pop("pads")
+    inp, w, mults, shifts, bias = rand_case(rng, in_u8=True, **g)
+    mults = np.where(rng.random(mults.shape) < 0.5, -mults, mults)
+    kw = dict(I8, lrelu_mult=1638, lrelu_shift=14)
+    got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=120, zp_out=-3, strides=strides, pads=pads,
+                               out_signed=True, mode=getattr(rt, "PPE_" + mode))
+    assert name == kernel
+    assert np.array_equal(got, want), "%s %s: %d mismatches" % (kernel, mode, int((got != want).sum()))
+
+
 @pytest.mark.parametrize("seed", [1234, 99])
 def test_conv_random_geometries(rt, orc, dev, seed):
     """Thirty seeded draws of shape, kernel, stride, padding, types, zero points and PPE mode, whichever kernel they select."""
@@ -296,6 +319,13 @@ def test_nce_eltwise(rt, orc, dev, subtract, mode):
                                in2_mult, out_mult, out_shift, subtract=subtract, out_signed=out_signed)
         got = out.cpu().numpy()
         assert np.array_equal(got, want), "%s: %d mismatches" % (shape, int((got != want).sum()))
+        # a negative output multiplier (negative output scale) flips which sums take the PReLU branch
+        ppe = rt.PpeInt(md, clamp[0], clamp[1], pm, ps, -out_mult, out_shift, in1_mult, in2_mult)
+        rt.nce_eltwise(dev_t(a, dev), dev_t(b, dev), out, ppe, zp1, zp2, zpo, subtract=subtract)
+        want = orc.nce_eltwise(a, b, orc.ppe(pm if mode == "LPRELU" else 1, ps, zpo, clamp[0], clamp[1]), zp1, zp2, in1_mult,
+                               in2_mult, -out_mult, out_shift, subtract=subtract, out_signed=out_signed)
+        got = out.cpu().numpy()
+        assert np.array_equal(got, want), "%s, negative multiplier: %d mismatches" % (shape, int((got != want).sum()))
 
 
 def test_nce_eltwise_full_size_residual(rt, orc, dev):

@@ -168,8 +168,9 @@ __device__ __forceinline__ int med3_i32(int v, int lo, int hi) {
     return r;
 }
 
-// `c.bias` must already carry the +2^31 that turns the int -> double bit trick's sign flip into part
-// of the bias addition (see ppe_prepare_packed).
+// `c` must come from ppe_prepare_packed: its bias carries the +2^31 that turns the int -> double bit trick's sign
+// flip into part of the bias addition, and for a negative multiplier its two factors (and bounds) are swapped, so
+// that "the scaled value is negative" is simply "acc + bias is negative", whatever the multiplier's sign.
 template <bool SAME_F, bool GENERAL>
 __device__ __forceinline__ unsigned ppe_pack4(int a0, int a1, int a2, int a3, const ChanPrep& c, const PpePack& p) {
     const int a[4] = {a0, a1, a2, a3};
@@ -180,7 +181,7 @@ __device__ __forceinline__ unsigned ppe_pack4(int a0, int a1, int a2, int a3, co
         double f = c.f_pos;
         int bm = c.bmax_pos;
         if (!SAME_F) {
-            const bool neg = (int)(bu ^ (unsigned)c.sgn) >= 0;  // flipped domain: top bit clear means negative
+            const bool neg = (int)bu >= 0;  // flipped domain: top bit clear means acc + bias < 0
             f = neg ? c.f_neg : c.f_pos;
             if (GENERAL) bm = neg ? c.bmax_neg : c.bmax_pos;
         }
@@ -202,6 +203,14 @@ __device__ __forceinline__ unsigned ppe_pack4(int a0, int a1, int a2, int a3, co
 __device__ __forceinline__ ChanPrep ppe_prepare_packed(int mult, int shift, int bias, int prelu_mult, int prelu_shift) {
     ChanPrep c = ppe_prepare(mult, shift, bias, prelu_mult, prelu_shift);
     c.bias = (int)((unsigned)c.bias + 0x80000000u);
+    if (c.sgn) {  // mult < 0: b < 0 scales to a non-negative value and takes f_pos, b > 0 takes f_neg (b = 0 gives 0 either way)
+        const double f = c.f_pos;
+        c.f_pos = c.f_neg;
+        c.f_neg = f;
+        const int bm = c.bmax_pos;
+        c.bmax_pos = c.bmax_neg;
+        c.bmax_neg = bm;
+    }
     return c;
 }
 
@@ -1322,12 +1331,13 @@ int launch_nce_eltwise(const vpx_nce_task_t& t, const Ppe& ppe, hipStream_t s, c
         const float a = std::fabs((float)f);
         return a <= 0.5f ? 0x7fffffff : (int)(1.0e9f / a);
     };
-    e.cp.f_pos = f_pos;
-    e.cp.f_neg = f_neg;
+    const bool swap = t.ppe.quant_mult < 0;  // as ppe_prepare_packed does
+    e.cp.f_pos = swap ? f_neg : f_pos;
+    e.cp.f_neg = swap ? f_pos : f_neg;
     e.cp.bias = (int)((unsigned)(int)bias + 0x80000000u);
-    e.cp.sgn = t.ppe.quant_mult < 0 ? -1 : 0;
-    e.cp.bmax_pos = bmax(f_pos);
-    e.cp.bmax_neg = bmax(f_neg);
+    e.cp.sgn = swap ? -1 : 0;
+    e.cp.bmax_pos = bmax(e.cp.f_pos);
+    e.cp.bmax_neg = bmax(e.cp.f_neg);
     const int off = out_signed ? 128 : 0, z = t.zp_out + off;
     e.pk = PpePack{6755399441055744.0 + (double)(z & ~1), z & 1, lo + off, hi + off, out_signed ? 0x80808080u : 0u};
     e.general = (e.cp.bmax_pos != 0x7fffffff || e.cp.bmax_neg != 0x7fffffff || (z & 1)) ? 1 : 0;
