@@ -853,3 +853,82 @@ def test_random_shapes_mvn6(rt, orc, dev, seed):
         # rows of a few elements have statistics of a few values: absolute floor for results next to zero
         assert np.all(np.abs(g - w) <= REL_TOL * np.abs(w) + 2e-4), (shape, axes, float(np.abs(g - w).max()))
 
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_random_shapes_quantization_family(rt, orc, dev, seed):
+    """Per-axis quantize / dequantize on random ranks and axes, dynamic_dequantize with random broadcast patterns."""
+    import torch
+    rng = np.random.default_rng(seed)
+    sizes = [1, 2, 3, 4, 7, 8, 16, 24, 40, 64, 100, 128]
+    for i in range(30):
+        nd = int(rng.integers(1, 5))
+        shape = tuple(int(rng.choice(sizes)) for _ in range(nd))
+        cands = [a for a in range(nd) if shape[a] > 1 and shape.count(shape[a]) == 1]
+        if not cands:
+            continue
+        axis = int(rng.choice(cands))
+        n = shape[axis]
+        print("seed %d per-axis case %d: %s axis %d" % (seed, i, shape, axis), flush=True)
+        scales, zps = rng.uniform(0.004, 0.08, n), rng.integers(-20, 21, n)
+        shipped = orc.f16_to_f32(orc.f32_to_f16(scales.astype(np.float32))).astype(np.float64)
+        x = orc.f32_to_f16(rng.normal(0, 3, shape).astype(np.float32))
+        q = torch.empty(shape, dtype=torch.int8, device=dev)
+        rt.quantize(to_dev(x, dev, True), q, scales, zps)
+        want = orc.quantize(x, shipped, zps, True, axis=axis)
+        assert np.array_equal(q.cpu().numpy(), want), (shape, axis)
+        y = torch.empty(shape, dtype=torch.float16, device=dev)
+        rt.dequantize(q, y, scales, zps)
+        assert_f16_exact(f16_bits(y).reshape(-1), orc.dequantize(want, shipped, zps, axis=axis).reshape(-1), "%s axis %d" % (shape, axis))
+    for i in range(30):
+        nd = int(rng.integers(1, 4))
+        shape = tuple(int(rng.choice(sizes)) for _ in range(nd))
+        sshape = tuple(s if rng.random() < 0.5 else 1 for s in shape)
+        zshape = tuple(s if rng.random() < 0.5 else 1 for s in shape) if rng.random() < 0.6 else None
+        print("seed %d dynamic_dequantize case %d: %s scale %s zp %s" % (seed, i, shape, sshape, zshape), flush=True)
+        q = rng.integers(-128, 128, shape).astype(np.int8)
+        sc = rng.uniform(1e-3, 0.1, sshape).astype(np.float16)
+        zp = None if zshape is None else rng.integers(-10, 11, zshape).astype(np.int8)
+        out = torch.empty(shape, dtype=torch.float16, device=dev)
+        rt.dynamic_dequantize(to_dev(q, dev), to_dev(sc, dev), out, None if zp is None else to_dev(zp, dev))
+        assert_f16_exact(f16_bits(out), orc.dynamic_dequantize(q, sc.view(np.uint16), zp), "%s %s %s" % (shape, sshape, zshape))
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_random_shapes_mvn1_and_fake_quantize(rt, orc, dev, seed):
+    """mvn1 and its three-step form on random 4-D shapes in both layouts; FakeQuantize with per-tensor / per-channel limits."""
+    import torch
+    rng = np.random.default_rng(seed)
+    for i in range(30):
+        N, Cc, H, W = int(rng.integers(1, 4)), int(rng.choice([1, 3, 8, 16, 64, 100])), int(rng.integers(1, 40)), int(rng.integers(1, 40))
+        layout, across, nv = str(rng.choice(["NCHW", "NHWC"])), bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        print("seed %d mvn case %d: %s %s across=%s nv=%s" % (seed, i, (N, Cc, H, W), layout, across, nv), flush=True)
+        x = orc.f32_to_f16((rng.uniform(-4, 4, (N, Cc, H, W)) + rng.normal(0, 2, (1, Cc, 1, 1))).astype(np.float32))
+        xm = _to_layout(x, layout)
+        xd = to_dev(xm, dev, True)
+        out = torch.empty_like(xd)
+        rt.mvn(xd, out, across, nv, 1e-4, order=layout)
+        w = orc.f16_to_f32(orc.mvn_f16(xm, across, nv, 1e-4, layout=layout)).astype(np.float64)
+        g = orc.f16_to_f32(f16_bits(out)).astype(np.float64)
+        # groups of a handful of elements: the tolerance is relative to the normalised scale (1), not to each value
+        assert np.all(np.abs(g - w) <= REL_TOL * np.abs(w) + 2e-3), float(np.abs(g - w).max())
+        c = 1 if across else Cc
+        sums = torch.empty((N, 1, 2 if nv else 1, c), dtype=torch.float32, device=dev)
+        mv = torch.empty((N, 1, 2 if nv else 1, c), dtype=torch.float32, device=dev)
+        o2 = torch.empty_like(xd)
+        rt.mvn1_sum(xd, sums, across, nv, order=layout)
+        rt.mvn1_mean_var(sums, mv, (N, Cc, H, W), across, nv, 1e-4)
+        rt.mvn1_norm(xd, mv, o2, across, nv, order=layout)
+        g2 = orc.f16_to_f32(f16_bits(o2)).astype(np.float64)
+        assert np.all(np.abs(g2 - w) <= REL_TOL * np.abs(w) + 2e-3), float(np.abs(g2 - w).max())
+    for i in range(20):
+        N, Cc, H, W = int(rng.integers(1, 3)), int(rng.choice([1, 3, 8, 16, 64])), int(rng.integers(1, 30)), int(rng.integers(1, 30))
+        per_ch, levels = bool(rng.integers(0, 2)), int(rng.choice([2, 16, 255, 256]))
+        print("seed %d fake_quantize case %d: %s per_channel=%s levels=%d" % (seed, i, (N, Cc, H, W), per_ch, levels), flush=True)
+        lshape = (1, Cc, 1, 1) if per_ch else (1, 1, 1, 1)
+        lo, hi = -rng.uniform(0.5, 4, lshape), rng.uniform(0.5, 4, lshape)
+        c = {"x": orc.f32_to_f16(rng.normal(0, 2, (N, Cc, H, W)).astype(np.float32)), "levels": levels,
+             "in_lo": orc.f32_to_f16(lo.astype(np.float32)), "in_hi": orc.f32_to_f16(hi.astype(np.float32)),
+             "out_lo": orc.f32_to_f16(lo.astype(np.float32)), "out_hi": orc.f32_to_f16(hi.astype(np.float32))}
+        assert_f16_exact(_run_fq(rt, dev, c), orc.fake_quantize_f16(c["x"], c["in_lo"], c["in_hi"], c["out_lo"], c["out_hi"], levels),
+                         "%s per_channel=%s levels=%d" % ((N, Cc, H, W), per_ch, levels))
+
