@@ -384,6 +384,8 @@ def test_dynamic_quantize(rt, orc, dev, shape):
 
 DYN_DQ_CASES = [
     # q shape, q dtype, scale shape, scale dtype, zp shape / dtype, out dtype
+    # the operand shapes of the reference's lit test (bufferize_sw_ops_to_VPUIP_sw_kernel.mlir:906-929), int8 for its int4
+    ((16, 7, 3, 51), np.int8, (16, 1, 3, 1), np.float16, ((16, 7, 1, 51), np.int8), np.float16),
     ((512, 1024), np.int8, (512, 1), np.float16, None, np.float16),                       # per-row scale, vector path
     ((512, 1024), np.int8, (512, 1), np.float16, ((512, 1), np.int8), np.float16),
     ((64, 8, 128), np.int8, (64, 8, 1), np.float16, ((64, 8, 1), np.int8), np.float16),   # group-wise weights

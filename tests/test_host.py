@@ -253,3 +253,32 @@ def test_kernel_params_blob_layout(rt):
     assert rt.lib().vpx_create_kernel_params(ins, 5, outs, 1, attrs, len(attrs), small, C.byref(sz)) == \
         rt.ERROR_INVALID_ARGUMENT
     assert sz.value == size.value
+
+
+def test_dynamic_dequantize_blob_matches_the_lit_golden(rt):
+    """bufferize_sw_ops_to_VPUIP_sw_kernel.mlir:906-929: operands (input, scale, zero point, output), attrs = [INT64_MAX]."""
+    def desc(dims, dtype, elem_bits):
+        d = (C.c_int32 * len(dims))(*dims)
+        st, acc = [], elem_bits
+        for v in dims:
+            st.append(acc)
+            acc *= v
+        s = (C.c_int64 * len(dims))(*st)
+        return rt.TensorDesc(len(dims), d, s, dtype, 0x4321, rt.LOC_DDR), d, s
+
+    q, *_k1 = desc([51, 3, 7, 16], rt.NN_I8, 8)
+    sc, *_k2 = desc([1, 3, 1, 16], rt.NN_FP16, 16)
+    zp, *_k3 = desc([51, 1, 7, 16], rt.NN_I8, 8)
+    out, *_k4 = desc([51, 3, 7, 16], rt.NN_FP16, 16)
+    ins = (rt.TensorDesc * 3)(q, sc, zp)
+    outs = (rt.TensorDesc * 1)(out)
+    attrs = struct.pack("<q", 9223372036854775807)
+    size = C.c_size_t(0)
+    rt.check(rt.lib().vpx_create_kernel_params(ins, 3, outs, 1, attrs, len(attrs), None, C.byref(size)))
+    buf = C.create_string_buffer(size.value)
+    rt.check(rt.lib().vpx_create_kernel_params(ins, 3, outs, 1, attrs, len(attrs), buf, C.byref(size)))
+    # the delimiter is the first word after the four MemRefData records: that is how the kernel counts its operands
+    assert struct.unpack_from("<q", buf.raw, 4 * 36)[0] == 2 ** 63 - 1
+    for i in range(4):
+        assert struct.unpack_from("<q", buf.raw, i * 36)[0] != 2 ** 63 - 1
+
