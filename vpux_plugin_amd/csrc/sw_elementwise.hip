@@ -132,13 +132,20 @@ __device__ __forceinline__ float narrow<float>(float r) {
 // takes the plain conversion instruction, the others the exact emulation.
 template <int N>
 __device__ __forceinline__ void narrow_vec(const float (&r)[N], half_t (&h)[N]) {
-    bool zone = false;
+    // (bits << 1) - 2 drops the sign and sends zero to the top of the range: the nonzero magnitudes below 2^-15
+    // are the values under 0x6ffffffe, so one running minimum finds them.  NaNs (payload rule) are found two
+    // values per comparison; the votes are combined as wave masks.
+    uint32_t lo = 0xffffffffu;
 #pragma unroll
     for (int k = 0; k < N; k++) {
-        const uint32_t mag = __builtin_bit_cast(uint32_t, r[k]) & 0x7fffffffu;
-        zone = zone || (mag - 1u) < 0x37ffffffu || mag > 0x7f800000u;  // 0 < |r| < 2^-15, or NaN (payload rule)
+        const uint32_t w = (__builtin_bit_cast(uint32_t, r[k]) << 1) - 2u;
+        lo = w < lo ? w : lo;
     }
-    if (__builtin_amdgcn_ballot_w64(zone) != 0) {
+    uint64_t zone = __builtin_amdgcn_ballot_w64(lo < 0x6ffffffeu);
+#pragma unroll
+    for (int k = 0; k + 1 < N; k += 2) zone |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(r[k], r[k + 1]));
+    if (N & 1) zone |= __builtin_amdgcn_ballot_w64(__builtin_isnan(r[N - 1]));
+    if (zone != 0) {
 #pragma unroll
         for (int k = 0; k < N; k++) h[k] = f32_to_f16(r[k]);
     } else {
@@ -309,20 +316,54 @@ __device__ __forceinline__ float fast_exp(float x) {
 __device__ __forceinline__ float fast_rcp(float x) {
     return __builtin_amdgcn_rcpf(x);
 }
-// log(1 + t) for 0 <= t <= 1: the series where 1 + t would lose the low bits of t
+// log(1 + t) for 0 <= t <= 1: two terms of the series where 1 + t would lose the low bits of t
 __device__ __forceinline__ float fast_log1p_unit(float t) {
-    const float series = t * (1.f - t * (0.5f - t * (0.33333333f - t * 0.25f)));
+    const float series = t * __builtin_fmaf(t, -0.5f, 1.f);
     const float direct = __builtin_amdgcn_logf(1.f + t) * 0.69314718055994530942f;
-    return t < 0.03125f ? series : direct;
+    return t < 0.0009765625f ? series : direct;
 }
 __device__ __forceinline__ float fast_softplus(float x) {
     return fmaxf(x, 0.f) + fast_log1p_unit(fast_exp(-fabsf(x)));
 }
+// tanh(x) = 1 - 2 / (1 + e^2x) holds for both signs and saturates by itself; below 2^-6 the
+// subtraction would cancel and x (1 - x^2 / 3) is exact to fp32.
 __device__ __forceinline__ float fast_tanh(float x) {
-    const float x2 = x * x;
-    const float small = x * (1.f - x2 * (0.33333333f - x2 * 0.13333333f));
-    const float big = 1.f - 2.f * fast_rcp(1.f + fast_exp(2.f * fabsf(x)));
-    return fabsf(x) < 0.05f ? small : __builtin_copysignf(big, x);
+    const float small = x * __builtin_fmaf(x * x, -0.33333334f, 1.f);
+    const float big = __builtin_fmaf(-2.f, fast_rcp(1.f + __builtin_amdgcn_exp2f(x * 2.88539008177792681472f)), 1.f);
+    return fabsf(x) < 0.015625f ? small : big;
+}
+// e^x - 1 for x <= 0: four terms of the series above -1/16, where the subtraction would cancel
+__device__ __forceinline__ float fast_expm1_neg(float x) {
+    float p = __builtin_fmaf(x, 0.041666668f, 0.16666667f);
+    p = __builtin_fmaf(p, x, 0.5f);
+    p = __builtin_fmaf(p, x, 1.f);
+    return x > -0.0625f ? p * x : fast_exp(x) - 1.f;
+}
+// erf(v) = sign(v) (1 - t P(t) e^(-v^2)), t = 1 / (1 + 0.4 |v|): the form of Abramowitz & Stegun 7.1.26 with
+// six coefficients fitted here for the RELATIVE error of erfc (1.2e-6 up to |v| = 3.2, where fp16 results have
+// long saturated), because GELU multiplies x by 1 + erf, which is erfc for negative x.  Below 2^-6: the series.
+__device__ __forceinline__ float fast_erf(float v) {
+    const float a = fabsf(v);
+    const float t = fast_rcp(__builtin_fmaf(0.4f, a, 1.f));
+    float p = __builtin_fmaf(t, -0.199453136f, 0.708108477f);
+    p = __builtin_fmaf(p, t, -0.372836827f);
+    p = __builtin_fmaf(p, t, 0.47267826f);
+    p = __builtin_fmaf(p, t, 0.158959478f);
+    p = __builtin_fmaf(p, t, 0.232544093f);
+    const float m = a * a;
+    const float c = p * t * __builtin_amdgcn_exp2f(m * -1.44269504088896340736f);
+    const float big = __builtin_copysignf(1.f - c, v);
+    const float small = v * __builtin_fmaf(m, -0.37612638903183754f, 1.1283791670955126f);
+    return a < 0.015625f ? small : big;
+}
+// sqrt of a value that came from fp16 (so never an fp32 subnormal), correctly rounded: the hardware root and
+// reciprocal root are good to an ulp, the residual x - y^2 is exact in one fma, and y + residual / (2 y)
+// rounds to the nearest fp32.  Zero and infinity keep the hardware result (their residual is not a number).
+__device__ __forceinline__ float fast_sqrt(float x) {
+    const float y = __builtin_amdgcn_sqrtf(x);
+    const float h = 0.5f * __builtin_amdgcn_rsqf(x);
+    const float fixed = __builtin_fmaf(__builtin_fmaf(-y, y, x), h, y);
+    return __builtin_amdgcn_classf(x, 0x260) ? y : fixed;  // +-0, +inf
 }
 
 template <typename T, int OP>
@@ -347,14 +388,14 @@ struct ActFn {
         if (OP == ACT_HARDSIGMOID) return fmaxf(0.f, fminf(1.f, p0 * x + p1));
         if (OP == ACT_SIGMOID) return kFast ? fast_rcp(1.f + fast_exp(-x)) : 1.f / (1.f + expf(-x));
         if (OP == ACT_TANH) return kFast ? fast_tanh(x) : tanhf(x);
-        if (OP == ACT_EXP) return expf(x);
-        if (OP == ACT_SQRT) return sqrtf(x);
+        if (OP == ACT_EXP) return kFast ? fast_exp(x) : expf(x);
+        if (OP == ACT_SQRT) return kFast ? fast_sqrt(x) : sqrtf(x);
         if (OP == ACT_LOG) return logf(x);
         if (OP == ACT_FLOOR) return floorf(x);
         if (OP == ACT_CEIL) return ceilf(x);
         if (OP == ACT_SIGN) return x > 0.f ? 1.f : (x < 0.f ? -1.f : x);
-        if (OP == ACT_ELU) return x < 0.f ? p0 * (expf(x) - 1.f) : x;
-        if (OP == ACT_SELU) return x > 0.f ? p1 * x : p0 * p1 * (expf(x) - 1.f);
+        if (OP == ACT_ELU) return x < 0.f ? p0 * (kFast ? fast_expm1_neg(x) : expf(x) - 1.f) : x;
+        if (OP == ACT_SELU) return x > 0.f ? p1 * x : p0 * p1 * (kFast ? fast_expm1_neg(x) : expf(x) - 1.f);
         if (OP == ACT_SWISH) return kFast ? x * fast_rcp(1.f + fast_exp(-p0 * x)) : x / (1.f + expf(-p0 * x));
         if (OP == ACT_MISH) {
             if (!kFast) return x * tanhf(x < 20.f ? log1pf(expf(x)) : x);
@@ -364,8 +405,8 @@ struct ActFn {
             return x * (n * fast_rcp(n + 2.f));
         }
         if (OP == ACT_SOFTPLUS) return kFast ? fast_softplus(x) : (x < 20.f ? log1pf(expf(x)) : x);
-        if (OP == ACT_GELU) return 0.5f * x * (1.f + erff(x * 0.70710678118654752440f));
-        return erff(x);
+        if (OP == ACT_GELU) return 0.5f * x * (1.f + (kFast ? fast_erf(x * 0.70710678118654752440f) : erff(x * 0.70710678118654752440f)));
+        return kFast ? fast_erf(x) : erff(x);
     }
     __device__ __forceinline__ T operator()(T v) const { return narrow<T>(f32(v)); }
 };
