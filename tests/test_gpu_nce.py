@@ -136,10 +136,45 @@ def test_unsigned_weights_around_128_take_the_mfma_kernels(rt, orc, dev, geom, k
                                    strides=strides, pads=pads)
         assert name == kernel
         assert np.array_equal(got, want), "%s zp_in=%d: %d mismatches" % (kernel, zp_in, int((got != want).sum()))
-    # any other zero point still takes the general kernel
-    inp, w, mults, shifts, bias = rand_case(rng, in_u8=True, w_u8=True, **g)
-    got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, U8, zp_in=128, zp_w=127, strides=strides, pads=pads)
-    assert name == "nce_conv_naive" and np.array_equal(got, want)
+
+
+WEIGHT_ZP_GEOMS = [
+    (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_tile"),
+    (dict(N=2, H=15, W=10, IC=128, OC=40, KY=3, KX=3, strides=(1, 1), pads=(1, 0, 0, 1)), "nce_conv_tile"),
+    (dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_stream"),
+    (dict(N=2, H=17, W=13, IC=64, OC=64, KY=3, KX=3, strides=(2, 2), pads=(1, 1, 1, 1)), "nce_conv_tile"),
+    (dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)), "nce_conv_mfma"),
+    (dict(N=1, H=12, W=12, IC=16, OC=32, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_mfma16"),
+    (dict(N=3, H=40, W=10, IC=64, OC=64, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_conv_tile"),
+    (dict(N=1, H=300, W=1, IC=128, OC=520, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_gemm_mfma"),
+    (dict(N=1, H=777, W=1, IC=1024, OC=300, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_gemm_mfma"),
+    (dict(N=1, H=515, W=1, IC=4160, OC=260, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_gemm_mfma"),
+]
+
+
+@pytest.mark.parametrize("geom,kernel", WEIGHT_ZP_GEOMS, ids=["%s-%dx%d-ic%d" % (k, g["KY"], g["KX"], g["IC"]) for g, k in WEIGHT_ZP_GEOMS])
+def test_weight_zero_points_take_the_mfma_kernels(rt, orc, dev, geom, kernel):
+    """Asymmetric weights (mpe_wtbias): the part of the zero point that the signed re-biased copy does not absorb
+    enters as one term per output position -- the sum of (activation - zero point) under its window."""
+    rng = np.random.default_rng(64)
+    g = dict(geom)
+    strides, pads = g.pop("strides"), g.pop("pads")
+    for in_u8, w_u8, zp_in, zp_w, signed_out in ((True, True, 128, 127, False), (True, True, 3, 255, True), (False, True, -7, 0, False),
+                                                 (True, False, 200, -9, True), (False, False, 11, 127, False), (True, True, 128, 77, False)):
+        inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, w_u8=w_u8, **g)
+        # both zero points shift the accumulators by a large common value: the bias takes it out again and the
+        # shifts follow what is left, so that the outputs use the whole range and both PReLU branches
+        K = w[0].size
+        centre = K * (inp.mean() - zp_in) * (w.mean() - zp_w)
+        spread = 3 * np.sqrt(K) * (inp.std() + abs(inp.mean() - zp_in)) * (w.std() + abs(w.mean() - zp_w)) / 2
+        bias = (bias - np.int64(round(centre))).astype(np.int32)
+        shifts = rng.integers(0, 3, len(shifts)) + max(1, int(np.ceil(np.log2(spread * 2 ** 15 / 128))))
+        kw = dict(I8 if signed_out else U8, lrelu_mult=1638, lrelu_shift=14)
+        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, zp_out=-3 if signed_out else 9,
+                                   strides=strides, pads=pads, out_signed=signed_out, mode=rt.PPE_LPRELU)
+        assert name == kernel
+        assert np.array_equal(got, want), "%s zp_in=%d zp_w=%d: %d mismatches" % (kernel, zp_in, zp_w, int((got != want).sum()))
+        assert len(np.unique(got)) > 20  # the outputs are spread, not saturated
 
 
 @pytest.mark.parametrize("geom,kernel", [
@@ -165,9 +200,10 @@ def test_negative_multipliers(rt, orc, dev, geom, kernel, mode):
     assert np.array_equal(got, want), "%s %s: %d mismatches" % (kernel, mode, int((got != want).sum()))
 
 
-@pytest.mark.parametrize("seed", [1234, 99])
-def test_conv_random_geometries(rt, orc, dev, seed):
-    """Thirty seeded draws of shape, kernel, stride, padding, types, zero points and PPE mode, whichever kernel they select."""
+@pytest.mark.parametrize("seed,weight_zp", [(1234, False), (99, False), (7, True), (8, True)])
+def test_conv_random_geometries(rt, orc, dev, seed, weight_zp):
+    """Thirty seeded draws of shape, kernel, stride, padding, types, zero points and PPE mode, whichever kernel they select;
+    the last two seeds also draw the weight storage type and a weight zero point."""
     rng = np.random.default_rng(seed)
     for i in range(30):
         IC = int(rng.choice([16, 32, 48, 64, 64, 96, 128, 128, 192, 256, 320, 512]))
@@ -184,10 +220,18 @@ def test_conv_random_geometries(rt, orc, dev, seed):
         what = "seed %d case %d: N=%d H=%d W=%d IC=%d OC=%d K=%dx%d S=%dx%d pads=%s in_u8=%s out_signed=%s zp_in=%d mode=%d" % (
             seed, i, N, H, W, IC, OC, KY, KX, SY, SX, (pl, pr, pt, pb), in_u8, out_signed, zp_in, mode)
         print(what, flush=True)
-        inp, w, mults, shifts, bias = rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=in_u8, shift_lo=14, shift_hi=26)
-        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_out=int(rng.integers(-5, 6)),
+        w_u8, zp_w = False, 0
+        if weight_zp:
+            w_u8 = bool(rng.integers(0, 2))
+            zp_w = int(rng.integers(0, 256)) if w_u8 else int(rng.integers(-128, 128))
+            what += " w_u8=%s zp_w=%d" % (w_u8, zp_w)
+        inp, w, mults, shifts, bias = rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=in_u8, w_u8=w_u8, shift_lo=14, shift_hi=26)
+        if weight_zp:  # take the common offset of the accumulators out again, so that the outputs are not saturated
+            bias = (bias - np.int64(round(KY * KX * IC * (inp.mean() - zp_in) * (w.mean() - zp_w)))).astype(np.int32)
+        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, zp_out=int(rng.integers(-5, 6)),
                                    strides=(SY, SX), pads=(pl, pr, pt, pb), out_signed=out_signed, mode=mode)
-        assert name != "nce_conv_naive", what
+        # (16-channel granularity is served up to K = 1008, the weights of 64 channels in 64 KiB of LDS)
+        assert name != "nce_conv_naive" or (IC % 32 != 0 and KY * KX * IC > 1008), what
         assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))
 
 

@@ -20,6 +20,8 @@
 // the top bit) and add the missing term to the bias: acc_true = acc_raw + k * sum_k w[oc][k] with
 // k = 128 - zp_in (u8) or -zp_in (i8); padded taps are filled with the byte that stands for the
 // zero point so they contribute exactly 0, as the MPE does (runtime_dpu_parser_imports.cpp.inc:872-879).
+// A weight zero point (mpe_wtbias, :940-945) adds one term per output position, prepared by two small
+// kernels and added to the accumulators before the PPE (see nce_pixel_sum_kernel).
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -101,6 +103,10 @@ static_assert(sizeof(ChanPrep) == 32, "ChanPrep layout");
 
 struct PpeFast {
     int zp_out, lo, hi;  // clamp bounds already intersected with the storage range
+    // Weights with a zero point: rowterm[m] = (what is left of the weight zero point) x the sum of
+    // (activation - zero point) under the window of output position m, added to every channel of that
+    // position; null when the weights the kernel reads have none (see nce_pixel_sum_kernel).
+    const int32_t* rowterm;
 };
 
 // Any bound between the largest |b| whose result can still lie inside a clamp window and 2^30 / |f|
@@ -373,6 +379,7 @@ struct GemmPpe {
     int corr;                     // zero-point term: acc_true = acc_raw + corr * sum_k B[n][k]
     int zp_out, lo, hi;           // clamp bounds already intersected with the storage range
     int out_signed;               // output storage is i8
+    const int32_t* rowterm;       // as in PpeFast; padded past the last position, so edge tiles may read ahead
 };
 
 // A[M][K] x B[N][K]^T with the PPE fused; see the file header.  K must be a multiple of 64.
@@ -555,6 +562,18 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
         asm volatile("" : "+v"(cp[j].f_pos), "+v"(cp[j].f_neg));
     }
     const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, OUT_SIGNED);
+    if (ppe.rowterm) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const i32x4 v = *reinterpret_cast<const i32x4*>(ppe.rowterm + m0 + wm0 + i * 32 + 8 * g + 4 * (lane >> 5));
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) acc[i][j][g * 4 + q] += v[q];
+            }
+    }
     auto requant_tile = [&](auto clip_c) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
@@ -703,7 +722,7 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t m = m0 + wave * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                if (m < Mtot) out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(acc[i][j][r], cp, ppe);
+                if (m < Mtot) out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(acc[i][j][r] + (ppe.rowterm ? ppe.rowterm[m] : 0), cp, ppe);
             }
         }
     }
@@ -917,6 +936,15 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
         const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
         const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 || pk.odd != 0;
         const int col4 = nj * 32 + ((lane & 31) & ~3);
+        if (ppe.rowterm) {
+            const int32_t* rt = ppe.rowterm + ((int64_t)img * g.OH + oy0) * g.OW;
+#pragma unroll
+            for (int i = 0; i < TMW; i++) {
+                if (mi0 + i * mstep >= pg.MT) continue;
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][r] += rt[(mi0 + i * mstep) * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4)];
+            }
+        }
         auto requant = [&](auto general_c) {
 #pragma unroll
             for (int i = 0; i < TMW; i++) {
@@ -1123,6 +1151,15 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
         const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
         const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 || pk.odd != 0;
         const int col4 = nj * 32 + ((lane & 31) & ~3);
+        if (ppe.rowterm) {
+            const int32_t* rt = ppe.rowterm + ((int64_t)img * g.OH + oy0) * g.OW;
+#pragma unroll
+            for (int i = 0; i < TMW; i++) {
+                if (mi0 + i * mstep >= pg.MT) continue;
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][r] += rt[(mi0 + i * mstep) * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4)];
+            }
+        }
         auto requant = [&](auto general_c) {
 #pragma unroll
             for (int i = 0; i < TMW; i++) {
@@ -1291,7 +1328,7 @@ __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict_
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t m = m0 + wave * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                if (m < Mtot) out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(acc[i][j][r], cp, ppe);
+                if (m < Mtot) out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(acc[i][j][r] + (ppe.rowterm ? ppe.rowterm[m] : 0), cp, ppe);
             }
         }
     }
@@ -1367,6 +1404,48 @@ int launch_nce_eltwise(const vpx_nce_task_t& t, const Ppe& ppe, hipStream_t s, c
     return VPX_RESULT_SUCCESS;
 }
 
+// Weights with a zero point zw.  The MFMA kernels multiply signed bytes W = w - cw (cw = 128 for unsigned storage,
+// re-biased into a scratch copy, else 0), so sum (a - za)(w - zw) lacks (cw - zw) * sum (a - za) over the taps
+// inside the image: one value per output position, the same for all its channels.  Two small kernels prepare
+// it: the channel sum of every input pixel, then the sum of those under each window times (cw - zw); the
+// convolution kernels add the result to their accumulators before the PPE.  A 1x1, stride-1, unpadded layer
+// (a matmul) needs only the first, which then applies the factor itself.
+__global__ __launch_bounds__(256) void nce_pixel_sum_kernel(const uint8_t* __restrict__ in, int32_t* __restrict__ cs, int64_t pixels,
+                                                            int IC, int lpp, int flip, int offset, int factor) {
+    // lpp lanes (a power of two, at most 64) share a pixel; each sums 16-byte chunks
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t pixel = t / lpp;
+    const int sub = (int)(t % lpp);
+    unsigned sum = 0;
+    if (pixel < pixels) {
+        const i32x4* row = reinterpret_cast<const i32x4*>(in + pixel * IC);
+        for (int c = sub; c < IC / 16; c += lpp) {
+            const i32x4 q = row[c];
+#pragma unroll
+            for (int k = 0; k < 4; k++) sum = __builtin_amdgcn_sad_u8((unsigned)(q[k] ^ flip), 0u, sum);  // four bytes at once
+        }
+    }
+    for (int o = lpp >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    if (pixel < pixels && sub == 0) cs[pixel] = ((int)sum - offset) * factor;
+}
+
+__global__ __launch_bounds__(256) void nce_window_sum_kernel(const int32_t* __restrict__ cs, int32_t* __restrict__ rowterm, ConvGeom g,
+                                                             int factor, int64_t total) {
+    const int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (m >= total) return;
+    const int64_t ox = m % g.OW, oy = (m / g.OW) % g.OH, n = m / (g.OW * g.OH);
+    int sum = 0;
+    for (int ky = 0; ky < g.KY; ky++) {
+        const int64_t iy = oy * g.SY + ky - g.PT;
+        if (iy < 0 || iy >= g.H) continue;
+        for (int kx = 0; kx < g.KX; kx++) {
+            const int64_t ix = ox * g.SX + kx - g.PL;
+            if (ix >= 0 && ix < g.W) sum += cs[(n * g.H + iy) * g.W + ix];
+        }
+    }
+    rowterm[m] = sum * factor;
+}
+
 // u8 weights whose zero point is 128 (symmetric weights kept in unsigned storage) are the signed weights
 // w - 128: one pass flips the top bit of every byte into a scratch copy and the signed kernels run on that.
 __global__ __launch_bounds__(256) void nce_weights_to_s8_kernel(const i32x4* __restrict__ in, i32x4* __restrict__ out, int64_t n_vec) {
@@ -1410,9 +1489,13 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const bool zp_in_ok = in_u8 ? (t.zp_in >= 0 && t.zp_in <= 255) : (t.zp_in >= -128 && t.zp_in <= 127);
     // the fast epilogue adds the output zero point after limiting the scaled value to +-2^30
     const bool zp_out_ok = t.zp_out >= -(1 << 20) && t.zp_out <= (1 << 20);
-    // signed weights without a zero point, or unsigned ones around 128 (re-biased into a scratch copy below)
-    const bool w_rebias = w_u8 && t.zp_w == 128 && Ktot % 16 == 0;
-    const bool mfma_ok = ((!w_u8 && t.zp_w == 0) || w_rebias) && zp_in_ok && zp_out_ok && Mtot < (1ll << 31) && g.OC < (1ll << 31);
+    // Unsigned weights are re-biased by 128 into a signed scratch copy; what is left of the weight zero point
+    // (wz_rest = 128 - zp_w, or -zp_w for signed storage) enters through one term per output position.
+    const bool w_rebias = w_u8 && Ktot % 16 == 0;
+    const bool zp_w_ok = w_u8 ? (t.zp_w >= 0 && t.zp_w <= 255) : (t.zp_w >= -128 && t.zp_w <= 127);
+    const int wz_rest = (w_u8 ? 128 : 0) - t.zp_w;
+    const bool mfma_ok = (!w_u8 || w_rebias) && zp_w_ok && zp_in_ok && zp_out_ok && Mtot < (1ll << 31) && g.OC < (1ll << 31) &&
+                         (wz_rest == 0 || (g.IC % 16 == 0 && g.N * g.H * g.W < (1ll << 31) && g.IC < (1 << 23)));
     const bool is_gemm = g.KY == 1 && g.KX == 1 && g.SY == 1 && g.SX == 1 && t.kernel_padding[0] == 0 &&
                          t.kernel_padding[1] == 0 && t.kernel_padding[2] == 0 && t.kernel_padding[3] == 0;
     const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights)) & 15) == 0;
@@ -1435,19 +1518,44 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         *out = (char*)base + wofs;
         return r;
     };
+    const int32_t* rowterm = nullptr;  // the per-position term of the weight zero point, when there is one
     const auto rebias_weights = [&]() -> int {
-        if (!w_rebias) return VPX_RESULT_SUCCESS;
-        const size_t wbytes = (size_t)g.OC * (size_t)Ktot;
-        void* copy = nullptr;
-        const int r = get_workspace(s, (wbytes + 255) / 256 * 256, &copy);
+        const size_t wbytes = w_rebias ? ((size_t)g.OC * (size_t)Ktot + 255) / 256 * 256 : 0;
+        const int64_t pixels = g.N * g.H * g.W;
+        const bool direct = is_gemm;  // every output position is one input pixel
+        constexpr int64_t kRowPad = 32 * kPatchMaxMT + 256;  // edge tiles read past the last position
+        const size_t rbytes = wz_rest != 0 ? (size_t)(Mtot + kRowPad + (direct ? 0 : pixels)) * sizeof(int32_t) : 0;
+        if (wbytes + rbytes == 0) return VPX_RESULT_SUCCESS;
+        void* base = nullptr;
+        const int r = get_workspace(s, wbytes + (rbytes + 255) / 256 * 256, &base);
         if (r) return r;
-        const int64_t n_vec = (int64_t)(wbytes / 16);
-        const int64_t blocks = (n_vec + 255) / 256;
-        hipLaunchKernelGGL(nce_weights_to_s8_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, s,
-                           (const i32x4*)t.weights, (i32x4*)copy, n_vec);
-        VPX_HIP_CHECK(hipGetLastError());
-        wptr = copy;
-        wofs = (wbytes + 255) / 256 * 256;
+        if (w_rebias) {
+            const int64_t n_vec = (int64_t)g.OC * Ktot / 16;
+            const int64_t blocks = (n_vec + 255) / 256;
+            hipLaunchKernelGGL(nce_weights_to_s8_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, s,
+                               (const i32x4*)t.weights, (i32x4*)base, n_vec);
+            VPX_HIP_CHECK(hipGetLastError());
+            wptr = base;
+        }
+        if (wz_rest != 0) {
+            int32_t* rt = (int32_t*)((char*)base + wbytes);
+            int32_t* cs = direct ? rt : rt + Mtot + kRowPad;
+            int lpp = 1;
+            while (lpp < g.IC / 16 && lpp < 64) lpp *= 2;
+            const int64_t blocks = (pixels * lpp + 255) / 256;
+            VPX_REQUIRE(blocks < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "NCE task: input of %lld pixels exceeds the launch limit",
+                        (long long)pixels);
+            hipLaunchKernelGGL(nce_pixel_sum_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const uint8_t*)t.input, cs, pixels,
+                               (int)g.IC, lpp, in_u8 ? 0 : (int)0x80808080, (int)((in_u8 ? 0 : 128) * g.IC + t.zp_in * g.IC),
+                               direct ? wz_rest : 1);
+            VPX_HIP_CHECK(hipGetLastError());
+            if (!direct) {
+                hipLaunchKernelGGL(nce_window_sum_kernel, dim3((unsigned)((Mtot + 255) / 256)), dim3(256), 0, s, cs, rt, g, wz_rest, Mtot);
+                VPX_HIP_CHECK(hipGetLastError());
+            }
+            rowterm = rt;
+        }
+        wofs = wbytes + (rbytes + 255) / 256 * 256;
         return VPX_RESULT_SUCCESS;
     };
     if (allow_mfma && mfma_ok && aligned && (use_gemm || g.IC % 32 == 0)) {
@@ -1455,8 +1563,9 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         rc = rebias_weights();
         if (rc) return rc;
         const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
-        PpeFast pf;
+        PpeFast pf{};
         pf.zp_out = t.zp_out;
+        pf.rowterm = rowterm;
         const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
         pf.lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin;
         pf.hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
@@ -1484,7 +1593,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 lds = (size_t)nk * (tile + tile) * 64;  // only the panels there are ...
                 if (lds < (size_t)tile * kOutStride) lds = (size_t)tile * kOutStride;  // ... or the staging tile
             }
-            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
+            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
             int32_t* colsum = nullptr;
             if (corr != 0) {
                 void* ws = nullptr;
@@ -1564,7 +1673,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     pg.ow = fd(g.OW);
                     const size_t lds = need(pg.R);
                     const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
-                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
+                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
                     const int pad_byte = t.zp_in & 0xff;
                     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
                     const char* cw = std::getenv("VPX_CONV_WAVES");
@@ -1645,7 +1754,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     pg.ow = fd(g.OW);
                     const size_t lds = need(pg.R);
                     const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
-                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0};
+                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
                     const int pad_byte = t.zp_in & 0xff;
                     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
                     int32_t* colsum = nullptr;
@@ -1723,7 +1832,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
 
     if (allow_mfma && mfma_ok && aligned && g.IC % 16 == 0 && g.IC % 32 != 0 && ((Ktot + 31) / 32 * 32 + 16) * 64 <= 64 * 1024) {
         const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
-        PpeFast pf;
+        PpeFast pf{};
         pf.zp_out = t.zp_out;
         const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
         pf.lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin;
@@ -1733,6 +1842,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         if (pf.lo > pf.hi) pf.lo = pf.hi;
         int rc = rebias_weights();
         if (rc) return rc;
+        pf.rowterm = rowterm;
         void* ws = nullptr;
         rc = scratch(sizeof(ChanPrep) * (size_t)g.OC, &ws);
         if (rc) return rc;
