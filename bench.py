@@ -25,10 +25,10 @@ METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
 # Bytes moved through L2 per step, from rocprofv3 FETCH_SIZE / WRITE_SIZE counters scaled by a plain
 # copy of known size (profiles/<workload>__*.md hold the runs these come from).
 MEASURED_TRAFFIC = {
-    "c1_fake_quantize": 887334, "c2_softmax": 134303481, "c3_mvn": 25428959, "c4_conv": 16265514,
-    "c5_matmul": 384905636, "c5_dequantize": 135355997, "c5_eltwise_add": 270525739, "c5_nce_eltwise": 135282585,
-    "calib_int_mm": 531759958, "x_mvn6_layernorm": 268497737, "x_activation_hswish": 180604482,
-    "x_mvn1_three_steps": 25334452,
+    "c1_fake_quantize": 885035, "c2_softmax": 134300997, "c3_mvn": 25428500, "c4_conv": 16275405,
+    "c5_matmul": 384934428, "c5_dequantize": 135348685, "c5_eltwise_add": 270539857, "c5_nce_eltwise": 135252959,
+    "calib_int_mm": 531680254, "x_mvn6_layernorm": 268486231, "x_activation_hswish": 180515042,
+    "x_mvn1_three_steps": 25333958,
 }
 
 
