@@ -141,10 +141,18 @@ __device__ __forceinline__ void narrow_vec(const float (&r)[N], half_t (&h)[N]) 
         const uint32_t w = (__builtin_bit_cast(uint32_t, r[k]) << 1) - 2u;
         lo = w < lo ? w : lo;
     }
-    uint64_t zone = __builtin_amdgcn_ballot_w64(lo < 0x6ffffffeu);
+    uint64_t zone = 0;  // lanes that need the exact emulation
 #pragma unroll
     for (int k = 0; k + 1 < N; k += 2) zone |= __builtin_amdgcn_ballot_w64(__builtin_isunordered(r[k], r[k + 1]));
     if (N & 1) zone |= __builtin_amdgcn_ballot_w64(__builtin_isnan(r[N - 1]));
+    if (__builtin_amdgcn_ballot_w64(lo < 0x6ffffffeu) != 0) {
+        // Some value lies below 2^-15 (the negative tail of GELU or Swish does in every wave): only those whose top
+        // eleven mantissa bits are all set round differently, one in 2048.  Look again before leaving the fast path.
+#pragma unroll
+        for (int k = 0; k < N; k++)
+            zone |= __builtin_amdgcn_ballot_w64(__builtin_fabsf(r[k]) < 0x1p-15f &&
+                                                (__builtin_bit_cast(uint32_t, r[k]) & 0x7ff000u) == 0x7ff000u);
+    }
     if (zone != 0) {
 #pragma unroll
         for (int k = 0; k < N; k++) h[k] = f32_to_f16(r[k]);
@@ -339,22 +347,41 @@ __device__ __forceinline__ float fast_expm1_neg(float x) {
     p = __builtin_fmaf(p, x, 1.f);
     return x > -0.0625f ? p * x : fast_exp(x) - 1.f;
 }
-// erf(v) = sign(v) (1 - t P(t) e^(-v^2)), t = 1 / (1 + 0.4 |v|): the form of Abramowitz & Stegun 7.1.26 with
-// six coefficients fitted here for the RELATIVE error of erfc (1.2e-6 up to |v| = 3.2, where fp16 results have
-// long saturated), because GELU multiplies x by 1 + erf, which is erfc for negative x.  Below 2^-6: the series.
+// erfc(a) = 2^P(a) for a >= 0, P a polynomial of degree 8 fitted here to log2 erfc: one exp2 and eight fmas, with
+// a relative error of erfc below 3e-6 up to a = 3.15 (beyond, fp16 results have long saturated; at the clamp 1 - erfc
+// is 1 in fp32).  The relative error is what counts: GELU multiplies x by 1 + erf, which is erfc on the negative side.
+// erf(v) = sign(v) (1 - erfc|v|); below 1/16 the subtraction cancels and three terms of the series are exact to fp32.
 __device__ __forceinline__ float fast_erf(float v) {
-    const float a = fabsf(v);
-    const float t = fast_rcp(__builtin_fmaf(0.4f, a, 1.f));
-    float p = __builtin_fmaf(t, -0.199453136f, 0.708108477f);
-    p = __builtin_fmaf(p, t, -0.372836827f);
-    p = __builtin_fmaf(p, t, 0.47267826f);
-    p = __builtin_fmaf(p, t, 0.158959478f);
-    p = __builtin_fmaf(p, t, 0.232544093f);
-    const float m = a * a;
-    const float c = p * t * __builtin_amdgcn_exp2f(m * -1.44269504088896340736f);
-    const float big = __builtin_copysignf(1.f - c, v);
-    const float small = v * __builtin_fmaf(m, -0.37612638903183754f, 1.1283791670955126f);
-    return a < 0.015625f ? small : big;
+    const float a = fminf(fabsf(v), 4.1f);
+    float p = __builtin_fmaf(a, -3.72667832e-06f, 3.3506035e-05f);
+    p = __builtin_fmaf(p, a, 0.000174893775f);
+    p = __builtin_fmaf(p, a, -0.00430425219f);
+    p = __builtin_fmaf(p, a, 0.0324461259f);
+    p = __builtin_fmaf(p, a, -0.151220308f);
+    p = __builtin_fmaf(p, a, -0.917526312f);
+    p = __builtin_fmaf(p, a, -1.62802012f);
+    p = __builtin_fmaf(p, a, 2.31981246e-06f);
+    const float big = __builtin_copysignf(1.f - __builtin_amdgcn_exp2f(p), v);
+    const float m = v * v;
+    const float small = v * __builtin_fmaf(m, __builtin_fmaf(m, 0.11283791670955126f, -0.37612638903183754f), 1.1283791670955126f);
+    return fabsf(v) >= 0.0625f ? big : small;  // a NaN takes the series, which keeps it
+}
+// GELU 0.5 x (1 + erf(x / sqrt 2)) with the same form in |x| directly: c = erfc(|x| / sqrt 2) = 2^P(|x|).  1 - c
+// is rounded to fp32 before it is added to 1, as erf is in the defining formula: on the negative side that decides
+// the last bits of 1 + erf.  0.5 + 0.5 s in one fma equals 0.5 (1 + s) rounded; no series is needed near 0, where
+// 1 + erf is 1.
+__device__ __forceinline__ float fast_gelu(float x) {
+    const float a = fminf(fabsf(x), 5.8f);
+    float p = __builtin_fmaf(a, -2.34842093e-07f, 2.9970647e-06f);
+    p = __builtin_fmaf(p, a, 2.16017165e-05f);
+    p = __builtin_fmaf(p, a, -0.000759922737f);
+    p = __builtin_fmaf(p, a, 0.00810957688f);
+    p = __builtin_fmaf(p, a, -0.0534623619f);
+    p = __builtin_fmaf(p, a, -0.458764225f);
+    p = __builtin_fmaf(p, a, -1.15118387f);
+    p = __builtin_fmaf(p, a, 2.31379299e-06f);
+    const float s = __builtin_copysignf(1.f - __builtin_amdgcn_exp2f(p), x);
+    return x * __builtin_fmaf(s, 0.5f, 0.5f);
 }
 // sqrt of a value that came from fp16 (so never an fp32 subnormal), correctly rounded: the hardware root and
 // reciprocal root are good to an ulp, the residual x - y^2 is exact in one fma, and y + residual / (2 y)
@@ -405,7 +432,7 @@ struct ActFn {
             return x * (n * fast_rcp(n + 2.f));
         }
         if (OP == ACT_SOFTPLUS) return kFast ? fast_softplus(x) : (x < 20.f ? log1pf(expf(x)) : x);
-        if (OP == ACT_GELU) return 0.5f * x * (1.f + (kFast ? fast_erf(x * 0.70710678118654752440f) : erff(x * 0.70710678118654752440f)));
+        if (OP == ACT_GELU) return kFast ? fast_gelu(x) : 0.5f * x * (1.f + erff(x * 0.70710678118654752440f));
         return kFast ? fast_erf(x) : erff(x);
     }
     __device__ __forceinline__ T operator()(T v) const { return narrow<T>(f32(v)); }
