@@ -90,6 +90,40 @@ VPX_API int vpx_create_kernel_params(const vpx_tensor_desc_t* inputs, uint32_t n
                                      const vpx_tensor_desc_t* outputs, uint32_t n_outputs, const void* attrs,
                                      size_t attrs_size, void* blob, size_t* blob_size);
 
+/* SwKernelOp::getKernelInfo (src/vpux_compiler/src/dialect/VPUIP/IR/ops/sw_kernel.cpp:640-1850) for the operators this
+ * library serves: from the name of a VPU operator ("SoftMax", "MVN", "MVN1Sum", "MVN1MeanVar", "MVN1Normalize", "MVN6",
+ * "FakeQuantize", "Quantize", "Dequantize", "DynamicQuantize", "DynamicDequantize", "Convert", "Add", "Subtract",
+ * "Multiply", "Divide", "Minimum", "Maximum", "PRelu", "ReLU", "LeakyRelu", "Clamp", "Negative", "Abs", "HSwish",
+ * "HSigmoid", "HardSigmoid", "Sigmoid", "Tanh", "Exp", "Sqrt", "Log", "Floor", "Ceiling", "Sign", "Elu", "Selu", "Swish",
+ * "Mish", "SoftPlus", "Gelu", "Erf") and its attributes to the firmware entry name and the serialised attribute
+ * bytes that vpx_create_kernel_params appends to the MemRefData records: int64 per integer or boolean attribute (a
+ * true i1 sign-extends to -1), float32 per float attribute, arrays flattened (kernel_params_utils.cpp:104-125).
+ * `input` is the first operand: its element type selects softmaxFp32 and the packing of quantization parameters
+ * (for Dequantize pass the OUTPUT tensor, whose float type packs them), its order maps logical axes to the
+ * innermost-first memory positions the kernels take (computeReverseMemDim, sw_kernel.cpp:29-40).
+ * Only the fields the operator reads are looked at.  attr_bytes may be NULL to query *attr_size. */
+typedef struct vpx_op_attrs_t {
+    int64_t axis_ind;            /* SoftMax: logical axis, negative counts from the end */
+    int64_t pad_size;            /* SoftMax: trailing elements of the axis to ignore */
+    int32_t across_channels;     /* MVN, MVN1Sum, MVN1MeanVar, MVN1Normalize */
+    int32_t normalize_variance;  /* the MVN family and MVN6 */
+    float eps;                   /* MVN, MVN1MeanVar, MVN6 */
+    int32_t eps_mode;            /* MVN6: 0 inside the square root, 1 outside */
+    const int64_t* axes;         /* MVN6: logical axes */
+    uint32_t num_axes;
+    int32_t has_scale, has_bias; /* MVN6: optional operands present */
+    const int64_t* orig_shape;   /* MVN1MeanVar: the four dimensions of the tensor being normalised */
+    int64_t group_c;             /* MVN1MeanVar: channels per group after the internal reshape (1 without one) */
+    int64_t levels;              /* FakeQuantize */
+    const double* scales;        /* Quantize / Dequantize: parameters of the quantized element type */
+    const int64_t* zero_points;
+    uint32_t num_quant_params;
+    float param0, param1;        /* LeakyRelu slope; Clamp min, max; Elu x; Selu alpha, lambda; Swish beta;
+                                    HardSigmoid alpha, beta */
+} vpx_op_attrs_t;
+VPX_API int vpx_get_kernel_info(const char* op, const vpx_op_attrs_t* attrs, const vpx_tensor_desc_t* input, char* entry,
+                                size_t entry_capacity, void* attr_bytes, size_t* attr_size);
+
 /* RNE fp32 -> fp16 bit pattern and back, the rule of vpux::type::float16
  * (src/vpux_utils/src/core/type/float16.cpp:30-144). */
 VPX_API uint16_t vpx_float_to_half_bits(float v);

@@ -934,3 +934,43 @@ def test_random_shapes_mvn1_and_fake_quantize(rt, orc, dev, seed):
         assert_f16_exact(_run_fq(rt, dev, c), orc.fake_quantize_f16(c["x"], c["in_lo"], c["in_hi"], c["out_lo"], c["out_hi"], levels),
                          "%s per_channel=%s levels=%d" % ((N, Cc, H, W), per_ch, levels))
 
+
+
+# ---------------------------------------------------------------------------------- operator -> kernel info -> blob -> launch
+
+def test_operator_attributes_to_launch(rt, orc, dev):
+    """The compile-side chain end to end: vpx_get_kernel_info names the entry and serialises the operator's attributes
+    (logical axes mapped through the tensor's order), vpx_create_kernel_params builds the blob, the kernel runs it."""
+    import torch
+    rng = np.random.default_rng(91)
+    a = orc.f32_to_f16(rng.normal(0, 2, (2, 5, 7, 16)).astype(np.float32))   # memory order N, H, W, C
+    x = to_dev(a, dev, True)
+
+    def run(op, ins, out, order, **attrs):
+        ops = [rt.Operand(t, order) for t in ins] + [rt.Operand(out, order)]
+        entry, attr_bytes = rt.get_kernel_info(op, ops[0], **attrs)
+        rt.sw_kernel_launch(entry, rt.create_kernel_params(ops[:-1], ops[-1:], attr_bytes), ops)
+        return f16_bits(out)
+
+    # SoftMax over the logical channel axis of an NHWC tensor: the innermost memory dimension
+    got = run("SoftMax", [x], torch.empty_like(x), "NHWC", axis_ind=1)
+    assert_close_f16(got, orc.softmax_f16(a, 3), orc, "softmax over C, NHWC")
+    # over logical W: memory dimension 2
+    got = run("SoftMax", [x], torch.empty_like(x), "NHWC", axis_ind=3)
+    assert_close_f16(got, orc.softmax_f16(a, 2), orc, "softmax over W, NHWC")
+    # MVN6 over logical H and W (memory dimensions 1 and 2), eps outside the root
+    got = run("MVN6", [x], torch.empty_like(x), "NHWC", axes=[2, 3], normalize_variance=1, eps_mode=1, eps=1e-5)
+    _assert_mvn6_close(got, orc.mvn6_f16(a, [1, 2], True, 1e-5, 1), orc, "mvn6 over H, W, NHWC")
+    # MVN-1 per channel on NCHW, and an activation with two attributes
+    b = orc.f32_to_f16(rng.normal(0, 2, (2, 6, 9, 8)).astype(np.float32))
+    y = to_dev(b, dev, True)
+    got = run("MVN", [y], torch.empty_like(y), "NCHW", across_channels=0, normalize_variance=1, eps=1e-9)
+    assert_close_f16(got, orc.mvn_f16(b, False, True, 1e-9), orc, "mvn1")
+    got = run("Clamp", [y], torch.empty_like(y), "NCHW", param0=-1.5, param1=0.75)
+    assert_f16_exact(got, orc.activation_f16("clamp", b, -1.5, 0.75), "clamp")
+    q = torch.empty(y.shape, dtype=torch.uint8, device=dev)
+    ops = [rt.Operand(y), rt.Operand(q)]
+    entry, attr_bytes = rt.get_kernel_info("Quantize", ops[0], scales=[0.05], zero_points=[128])
+    rt.sw_kernel_launch(entry, rt.create_kernel_params(ops[:1], ops[1:], attr_bytes), ops)
+    shipped = float(orc.f16_to_f32(orc.f32_to_f16(np.array([0.05], np.float32)))[0])
+    assert np.array_equal(q.cpu().numpy(), orc.quantize(b, shipped, 128, False))

@@ -282,3 +282,60 @@ def test_dynamic_dequantize_blob_matches_the_lit_golden(rt):
     for i in range(4):
         assert struct.unpack_from("<q", buf.raw, i * 36)[0] != 2 ** 63 - 1
 
+
+
+def test_get_kernel_info_against_lit_goldens_and_the_operator_wrappers(rt):
+    """Operator attributes -> entry name + attribute bytes, as SwKernelOp::getKernelInfo derives them."""
+    import torch
+    i64 = lambda *v: struct.pack("<%dq" % len(v), *v)
+    f32 = lambda v: struct.pack("<f", v)
+    x = torch.empty((1, 1, 1, 1000), dtype=torch.float16)
+    # bufferize_sw_ops_to_VPUIP_sw_kernel.mlir:203-211 (axisInd = 3, padSize = 3 -> [0, 3]) and :225-242 (-> [0, 0])
+    assert rt.get_kernel_info("SoftMax", x, axis_ind=3, pad_size=3) == ("softmax", i64(0, 3))
+    assert rt.get_kernel_info("SoftMax", x, axis_ind=3) == ("softmax", i64(0, 0))
+    assert rt.get_kernel_info("SoftMax", x.float(), axis_ind=-1)[0] == "softmaxFp32"
+    # the axis is a logical one: channels of an NHWC tensor are the innermost memory dimension
+    nhwc = rt.Operand(torch.empty((2, 5, 7, 16), dtype=torch.float16), "NHWC")
+    assert rt.get_kernel_info("SoftMax", nhwc, axis_ind=1)[1] == i64(0, 0)
+    assert rt.get_kernel_info("SoftMax", nhwc, axis_ind=3)[1] == i64(1, 0)
+    assert rt.get_kernel_info("SoftMax", nhwc, axis_ind=0)[1] == i64(3, 0)
+    # dialect/VPUIP/ops/sw_kernel.mlir:42 (attrs = [false, true, 6.0892105102539063E-4]); a true i1 is -1
+    assert rt.get_kernel_info("MVN", across_channels=0, normalize_variance=1, eps=6.0892105102539063E-4) == (
+        "mvn1", i64(0, -1) + f32(6.0892105102539063E-4))
+    # tile_act_shave_kernel_task.mlir:240 (MVN1Sum, attrs = [true, true])
+    assert rt.get_kernel_info("MVN1Sum", across_channels=1, normalize_variance=1) == ("mvn1_sum", i64(-1, -1))
+    assert rt.get_kernel_info("MVN1Normalize", across_channels=0, normalize_variance=1) == ("mvn1_norm", i64(0, -1))
+    assert rt.get_kernel_info("MVN1MeanVar", orig_shape=[1, 32, 21846, 1], across_channels=1, normalize_variance=1, group_c=1,
+                              eps=1e-9) == ("mvn1_mean_var", i64(1, 32, 21846, 1, -1, -1, 1) + f32(1e-9))
+    # MVN6: marker, operand mask, then the axes as innermost-first memory positions
+    entry, attrs = rt.get_kernel_info("MVN6", nhwc, axes=[2, 3], normalize_variance=1, eps_mode=1, eps=1e-5, has_scale=1)
+    assert entry == "mvn6" and attrs == i64(-2 ** 63, 1 | 2 | 8, -1, 1) + f32(1e-5) + i64(2, 2, 1)
+    # bufferize_sw_ops_to_VPUIP_sw_kernel.mlir:906-929
+    assert rt.get_kernel_info("DynamicDequantize") == ("dynamic_dequantize", i64(2 ** 63 - 1))
+    assert rt.get_kernel_info("FakeQuantize", levels=256) == ("fake_quantize", i64(256))
+    entry, attrs = rt.get_kernel_info("Quantize", x, scales=[0.5, 0.25, 2.0], zero_points=[1, 2, 3])
+    assert entry == "quantize" and attrs == rt.get_quant_params_attr([0.5, 0.25, 2.0], [1, 2, 3], rt.NN_FP16).tobytes()
+    assert rt.get_kernel_info("Dequantize", x.float(), scales=[0.5], zero_points=[7])[1] == rt.get_quant_params_attr(
+        [0.5], [7], rt.NN_FP32).tobytes()
+    assert rt.get_kernel_info("LeakyRelu", param0=0.1) == ("leaky_relu_fp16", f32(0.1))
+    assert rt.get_kernel_info("Clamp", param0=-1.5, param1=6.0) == ("activation_clamp", f32(-1.5) + f32(6.0))
+    # every entry the builder names is one the library launches, with the number of float attributes its wrapper sends
+    ops = {"Convert": "convert", "Add": "eltwise_add", "Subtract": "eltwise_sub", "Multiply": "eltwise_mul", "Divide": "eltwise_div",
+           "Minimum": "eltwise_min", "Maximum": "eltwise_max", "PRelu": "prelu_fp16", "DynamicQuantize": "dynamic_quantize",
+           "ReLU": "relu", "LeakyRelu": "leaky_relu", "Clamp": "clamp", "Negative": "negative", "Abs": "abs", "HSwish": "hswish",
+           "HSigmoid": "hsigmoid", "HardSigmoid": "hardsigmoid", "Sigmoid": "sigmoid", "Tanh": "tanh", "Exp": "exp",
+           "Sqrt": "sqrt", "Log": "log", "Floor": "floor", "Ceiling": "ceil", "Sign": "sign", "Elu": "elu", "Selu": "selu",
+           "Swish": "swish", "Mish": "mish", "SoftPlus": "softplus", "Gelu": "gelu", "Erf": "erf"}
+    for op, short in ops.items():
+        entry, attrs = rt.get_kernel_info(op, param0=0.5, param1=2.0)
+        assert rt.lib().vpx_sw_kernel_supported(entry.encode()) == 1, op
+        if short in rt.ACTIVATIONS:
+            assert (entry, len(attrs)) == (rt.ACTIVATIONS[short][0], 4 * rt.ACTIVATIONS[short][1]), op
+        else:
+            assert entry == short and attrs == b"", op
+    with pytest.raises(rt.VpxError) as e:
+        rt.get_kernel_info("TopK")
+    assert e.value.code == rt.ERROR_UNSUPPORTED_FEATURE
+    with pytest.raises(rt.VpxError) as e:
+        rt.get_kernel_info("SoftMax", x, axis_ind=4)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT

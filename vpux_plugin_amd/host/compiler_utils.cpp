@@ -377,6 +377,139 @@ int vpx_get_quant_params_attr(const double* scales, const int64_t* zero_points, 
     return VPX_RESULT_SUCCESS;
 }
 
+namespace {
+
+// computeReverseMemDim (sw_kernel.cpp:29-40): position of a logical dimension counted from the innermost memory
+// dimension.  The order code holds one hex digit (logical index + 1) per memory dimension, the outermost in the
+// lowest digit (NHWC = 0x2431: N, H, W, C).
+int reverse_mem_dim(const vpx_tensor_desc_t& t, int64_t dim, int64_t* out) {
+    const int64_t nd = t.num_dims;
+    if (dim < 0) dim += nd;
+    if (dim < 0 || dim >= nd) return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "axis %lld is outside a tensor of rank %lld", (long long)dim, (long long)nd);
+    for (int64_t i = 0; i < nd; i++) {
+        if ((int64_t)((t.dims_order >> (4 * i)) & 0xf) == dim + 1) {
+            *out = nd - 1 - i;
+            return VPX_RESULT_SUCCESS;
+        }
+    }
+    return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "order 0x%llx does not name dimension %lld", (unsigned long long)t.dims_order, (long long)dim);
+}
+
+struct AttrWriter {
+    std::vector<uint8_t> bytes;
+    void i64(int64_t v) { const uint8_t* p = (const uint8_t*)&v; bytes.insert(bytes.end(), p, p + 8); }
+    void boolean(int32_t v) { i64(v ? -1 : 0); }  // IntegerAttr of an i1 through getSExtValue()
+    void f32(float v) { const uint8_t* p = (const uint8_t*)&v; bytes.insert(bytes.end(), p, p + 4); }
+};
+
+struct SimpleOp {
+    const char* op;
+    const char* entry;
+    int n_float;  // float attributes taken from param0, param1
+};
+const SimpleOp kSimpleOps[] = {
+    {"Convert", "convert", 0}, {"Add", "eltwise_add", 0}, {"Subtract", "eltwise_sub", 0}, {"Multiply", "eltwise_mul", 0},
+    {"Divide", "eltwise_div", 0}, {"Minimum", "eltwise_min", 0}, {"Maximum", "eltwise_max", 0}, {"PRelu", "prelu_fp16", 0},
+    {"DynamicQuantize", "dynamic_quantize", 0}, {"ReLU", "activation_relu", 0}, {"LeakyRelu", "leaky_relu_fp16", 1},
+    {"Clamp", "activation_clamp", 2}, {"Negative", "activation_negative", 0}, {"Abs", "activation_abs", 0},
+    {"HSwish", "activation_hswish", 0}, {"HSigmoid", "activation_hsigmoid", 0}, {"HardSigmoid", "activation_hardsigmoid", 2},
+    {"Sigmoid", "activation_sigmoid", 0}, {"Tanh", "activation_tanh", 0}, {"Exp", "activation_exp", 0},
+    {"Sqrt", "activation_sqrt", 0}, {"Log", "activation_log", 0}, {"Floor", "activation_floor", 0},
+    {"Ceiling", "activation_ceil", 0}, {"Sign", "activation_sign", 0}, {"Elu", "activation_elu", 1},
+    {"Selu", "activation_selu", 2}, {"Swish", "activation_swish", 1}, {"Mish", "activation_mish", 0},
+    {"SoftPlus", "activation_softplus", 0}, {"Gelu", "activation_gelu", 0}, {"Erf", "activation_erf", 0},
+};
+
+}  // namespace
+
+int vpx_get_kernel_info(const char* op, const vpx_op_attrs_t* a, const vpx_tensor_desc_t* input, char* entry,
+                        size_t entry_capacity, void* attr_bytes, size_t* attr_size) {
+    if (!op || !entry || !attr_size) return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "vpx_get_kernel_info: null argument");
+    const std::string name(op);
+    std::string ent;
+    AttrWriter w;
+    const auto need = [&](bool ok, const char* what) {
+        return ok ? VPX_RESULT_SUCCESS : fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "%s: %s is required", op, what);
+    };
+    int rc = VPX_RESULT_SUCCESS;
+    bool found = false;
+    for (const SimpleOp& s : kSimpleOps) {
+        if (name != s.op) continue;
+        if (s.n_float > 0 && (rc = need(a != nullptr, "attributes"))) return rc;
+        if (s.n_float >= 1) w.f32(a->param0);
+        if (s.n_float >= 2) w.f32(a->param1);
+        ent = s.entry;
+        found = true;
+    }
+    if (found) {
+    } else if (name == "SoftMax") {
+        if ((rc = need(a && input, "attributes and the input tensor"))) return rc;
+        int64_t axis = 0;
+        if ((rc = reverse_mem_dim(*input, a->axis_ind, &axis))) return rc;
+        w.i64(axis);
+        w.i64(a->pad_size);
+        ent = input->data_type == VPX_NN_FP32 ? "softmaxFp32" : "softmax";
+    } else if (name == "MVN") {
+        if ((rc = need(a != nullptr, "attributes"))) return rc;
+        w.boolean(a->across_channels);
+        w.boolean(a->normalize_variance);
+        w.f32(a->eps);
+        ent = "mvn1";
+    } else if (name == "MVN1Sum" || name == "MVN1Normalize") {
+        if ((rc = need(a != nullptr, "attributes"))) return rc;
+        w.boolean(a->across_channels);
+        w.boolean(a->normalize_variance);
+        ent = name == "MVN1Sum" ? "mvn1_sum" : "mvn1_norm";
+    } else if (name == "MVN1MeanVar") {
+        if ((rc = need(a && a->orig_shape, "attributes with orig_shape"))) return rc;
+        for (int i = 0; i < 4; i++) w.i64(a->orig_shape[i]);
+        w.boolean(a->across_channels);
+        w.boolean(a->normalize_variance);
+        w.i64(a->group_c);
+        w.f32(a->eps);
+        ent = "mvn1_mean_var";
+    } else if (name == "MVN6") {
+        if ((rc = need(a && input && (a->axes || a->num_axes == 0), "attributes with axes and the input tensor"))) return rc;
+        // optionalIoAttr (sw_kernel.cpp:165-185): a marker after the MemRefData records, then a mask of present operands
+        w.i64(INT64_MIN);
+        w.i64(1 | (a->has_scale ? 2 : 0) | (a->has_bias ? 4 : 0) | 8);
+        w.boolean(a->normalize_variance);
+        w.i64(a->eps_mode);
+        w.f32(a->eps);
+        w.i64(a->num_axes);
+        for (uint32_t i = 0; i < a->num_axes; i++) {
+            int64_t axis = 0;
+            if ((rc = reverse_mem_dim(*input, a->axes[i], &axis))) return rc;
+            w.i64(axis);
+        }
+        ent = "mvn6";
+    } else if (name == "FakeQuantize") {
+        if ((rc = need(a != nullptr, "attributes"))) return rc;
+        w.i64(a->levels);
+        ent = "fake_quantize";
+    } else if (name == "Quantize" || name == "Dequantize") {
+        if ((rc = need(a && input && a->scales && a->zero_points && a->num_quant_params > 0, "quantization parameters and the float tensor"))) return rc;
+        std::vector<uint64_t> words(1 + 2 * ((size_t)a->num_quant_params + 1));
+        uint32_t n_words = 0;
+        if ((rc = vpx_get_quant_params_attr(a->scales, a->zero_points, a->num_quant_params, input->data_type, words.data(), &n_words))) return rc;
+        for (uint32_t i = 0; i < n_words; i++) w.i64((int64_t)words[i]);
+        ent = name == "Quantize" ? "quantize" : "dequantize";
+    } else if (name == "DynamicDequantize") {
+        w.i64(INT64_MAX);  // delimiter: the zero point operand is optional (sw_kernel.cpp:1180-1183)
+        ent = "dynamic_dequantize";
+    } else {
+        return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "vpx_get_kernel_info: operator '%s' has no kernel here", op);
+    }
+    if (ent.size() + 1 > entry_capacity) return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "vpx_get_kernel_info: entry buffer of %zu bytes is too small", entry_capacity);
+    std::memcpy(entry, ent.c_str(), ent.size() + 1);
+    if (attr_bytes) {
+        if (*attr_size < w.bytes.size()) return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "vpx_get_kernel_info: attribute buffer holds %zu bytes, %zu are needed", *attr_size, w.bytes.size());
+        if (!w.bytes.empty()) std::memcpy(attr_bytes, w.bytes.data(), w.bytes.size());
+    }
+    *attr_size = w.bytes.size();
+    return VPX_RESULT_SUCCESS;
+}
+
 int vpx_create_kernel_params(const vpx_tensor_desc_t* inputs, uint32_t n_inputs, const vpx_tensor_desc_t* outputs,
                              uint32_t n_outputs, const void* attrs, size_t attrs_size, void* blob, size_t* blob_size) {
     if (!blob_size || (n_inputs && !inputs) || (n_outputs && !outputs) || (attrs_size && !attrs))

@@ -50,6 +50,16 @@ class PpeInt(C.Structure):
                 ("in1_quant_mult", C.c_int32), ("in2_quant_mult", C.c_int32)]
 
 
+class OpAttrs(C.Structure):
+    """vpx_op_attrs_t: the operator attributes vpx_get_kernel_info reads."""
+    _fields_ = [("axis_ind", C.c_int64), ("pad_size", C.c_int64), ("across_channels", C.c_int32),
+                ("normalize_variance", C.c_int32), ("eps", C.c_float), ("eps_mode", C.c_int32),
+                ("axes", C.POINTER(C.c_int64)), ("num_axes", C.c_uint32), ("has_scale", C.c_int32), ("has_bias", C.c_int32),
+                ("orig_shape", C.POINTER(C.c_int64)), ("group_c", C.c_int64), ("levels", C.c_int64),
+                ("scales", C.POINTER(C.c_double)), ("zero_points", C.POINTER(C.c_int64)), ("num_quant_params", C.c_uint32),
+                ("param0", C.c_float), ("param1", C.c_float)]
+
+
 class QuantType(C.Structure):
     _fields_ = [("is_quantized", C.c_int32), ("scale", C.c_double), ("zero_point", C.c_int64),
                 ("storage_min", C.c_int64), ("storage_max", C.c_int64)]
@@ -72,7 +82,7 @@ ELTWISE_ADD, ELTWISE_SUBTRACT = 0, 1
 EXPORTS = ["vpx_get_last_error", "vpx_get_version", "vpx_sw_kernel_launch", "vpx_sw_kernel_supported",
            "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_approximate",
            "vpx_eltwise_quantization_approximation", "vpx_wt_get_scale", "vpx_wt_get_bias", "vpx_get_weights_table",
-           "vpx_retrieve_ppe_int", "vpx_generate_softmax_attr", "vpx_get_quant_params_attr", "vpx_create_kernel_params",
+           "vpx_retrieve_ppe_int", "vpx_generate_softmax_attr", "vpx_get_quant_params_attr", "vpx_create_kernel_params", "vpx_get_kernel_info",
            "vpx_float_to_half_bits", "vpx_half_bits_to_float"]
 
 _lib = None
@@ -127,6 +137,8 @@ def lib():
                                                 C.POINTER(C.c_uint32)]
         L.vpx_create_kernel_params.argtypes = [C.POINTER(TensorDesc), C.c_uint32, C.POINTER(TensorDesc), C.c_uint32,
                                                C.c_void_p, C.c_size_t, C.c_void_p, C.POINTER(C.c_size_t)]
+        L.vpx_get_kernel_info.argtypes = [C.c_char_p, C.POINTER(OpAttrs), C.POINTER(TensorDesc), C.c_char_p, C.c_size_t,
+                                          C.c_void_p, C.POINTER(C.c_size_t)]
         L.vpx_float_to_half_bits.restype = C.c_uint16
         L.vpx_float_to_half_bits.argtypes = [C.c_float]
         L.vpx_half_bits_to_float.restype = C.c_float
@@ -204,6 +216,37 @@ def get_quant_params_attr(scales, zero_points, float_type):
     check(lib().vpx_get_quant_params_attr(s.ctypes.data, z.ctypes.data, s.size, float_type, words.ctypes.data,
                                           C.byref(n)))
     return words[:n.value].copy()
+
+
+def get_kernel_info(op, operand=None, axes=None, orig_shape=None, scales=None, zero_points=None, **fields):
+    """(entry name, attribute bytes) of a VPU operator, as SwKernelOp::getKernelInfo derives them.  `operand` is the
+    Operand (or torch tensor) whose order and element type the derivation reads; list-valued attributes are keywords."""
+    a = OpAttrs()
+    keep = []
+    for k, v in fields.items():
+        setattr(a, k, v)
+    if axes is not None:
+        arr = (C.c_int64 * len(axes))(*axes)
+        keep.append(arr)
+        a.axes, a.num_axes = arr, len(axes)
+    if orig_shape is not None:
+        arr = (C.c_int64 * 4)(*orig_shape)
+        keep.append(arr)
+        a.orig_shape = arr
+    if scales is not None:
+        sc, zp = (C.c_double * len(scales))(*scales), (C.c_int64 * len(scales))(*zero_points)
+        keep += [sc, zp]
+        a.scales, a.zero_points, a.num_quant_params = sc, zp, len(scales)
+    desc = None
+    if operand is not None:
+        operand = operand if isinstance(operand, Operand) else Operand(operand)
+        desc = C.byref(operand.desc)
+    entry = C.create_string_buffer(64)
+    size = C.c_size_t(0)
+    check(lib().vpx_get_kernel_info(op.encode(), C.byref(a), desc, entry, len(entry), None, C.byref(size)))
+    buf = C.create_string_buffer(max(size.value, 1))
+    check(lib().vpx_get_kernel_info(op.encode(), C.byref(a), desc, entry, len(entry), buf, C.byref(size)))
+    return entry.value.decode(), buf.raw[:size.value]
 
 
 def half_bits(v):
