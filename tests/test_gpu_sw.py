@@ -573,7 +573,10 @@ MVN6_CASES = [
     ((3, 64, 200), (1,), (1, 64, 1), (1, 1, 200)),        # innermost dimension kept: lanes along it
     ((2, 5, 6, 70), (1, 2), (1, 5, 6, 1), None),
     ((2, 3, 4, 5), (1, 3), (1, 3, 1, 5), (1, 1, 1, 5)),   # split axes
-    ((2, 20000), (1,), None, None),                       # long rows: chunked like mvn1 ...
+    ((3, 2, 11008), (2,), (1, 1, 11008), None),           # rows of up to 16384 stay in the registers of a workgroup
+    ((5, 16384), (1,), None, (1, 16384)),
+    ((3, 12296), (1,), None, None),
+    ((2, 20000), (1,), None, None),                       # longer rows: chunked like mvn1 ...
     ((3, 2, 150, 200), (2, 3), None, None),
     ((2, 20001), (1,), None, (1, 20001)),                 # ... or one workgroup per row when there is a bias
     ((6, 1, 64), (1, 2), None, None),                     # unit dimension among the axes

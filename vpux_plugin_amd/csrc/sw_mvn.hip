@@ -611,6 +611,7 @@ __device__ __forceinline__ float team_sum(float v, float* smem) {
 
 // Rows that are contiguous in memory and a multiple of 8 long: the row lives in the registers of half a
 // wavefront (TEAM = 32, eight rows per workgroup), of a wavefront (64) or of the workgroup (256).
+constexpr int kMvn6MaxRegRow = 16384;  // longest row a workgroup keeps in registers (64 values per lane)
 template <int TEAM, int VPT>
 __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
                                                              const half_t* __restrict__ sc, const half_t* __restrict__ bi,
@@ -1143,11 +1144,11 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
 
     // Long contiguous rows of a compact tensor, eps inside the root, no scale or bias: the chunked two-launch
     // scheme of mvn1 (a row is a group there).
-    if (innermost && row_len > 8192 && !scale && !bias && eps_mode == 0 && in.compact && out.compact) {
+    if (innermost && row_len > kMvn6MaxRegRow && !scale && !bias && eps_mode == 0 && in.compact && out.compact) {
         const bool aligned = row_len % 8 == 0 && ((reinterpret_cast<uintptr_t>(pi) | reinterpret_cast<uintptr_t>(po)) & 15) == 0;
         return aligned ? launch_groups<true>(pi, po, g.rows, row_len, nv, eps, s) : launch_groups<false>(pi, po, g.rows, row_len, nv, eps, s);
     }
-    bool fast = innermost && row_len % 8 == 0 && row_len <= 8192;
+    bool fast = innermost && row_len % 8 == 0 && row_len <= kMvn6MaxRegRow;
     if (fast) {
         fast = along_row(true, g.rdim, g.r_in, g.nr) == 1 && along_row(true, g.rdim, g.r_out, g.nr) == 1;
         g.sc_along_row = along_row(scale != nullptr, g.rdim, g.r_sc, g.nr);
@@ -1165,7 +1166,9 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
         else if (row_len <= 1024) VPX_MVN6_ROWS(64, 2);
         else if (row_len <= 2048) VPX_MVN6_ROWS(256, 1);
         else if (row_len <= 4096) VPX_MVN6_ROWS(256, 2);  // one wavefront per 4096-element row measured 9 % slower
-        else VPX_MVN6_ROWS(256, 4);
+        else if (row_len <= 8192) VPX_MVN6_ROWS(256, 4);
+        else if (row_len <= 12288) VPX_MVN6_ROWS(256, 6);
+        else VPX_MVN6_ROWS(256, 8);
 #undef VPX_MVN6_ROWS
     } else if (inner_kept && g.k_in[0] == 1 && g.k_out[0] == 1) {
         const int64_t outer = g.rows / g.kdim[0];
