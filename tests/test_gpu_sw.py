@@ -284,11 +284,13 @@ def test_fake_quantize_rejects_bad_arguments(rt, dev):
 
 # ---------------------------------------------------------------------------------- quantize / dequantize
 
-@pytest.mark.parametrize("signed,scale,zp", [(False, 0.02, 128), (True, 0.05, 0), (True, 0.003, -21), (False, 1 / 255, 3)])
+@pytest.mark.parametrize("signed,scale,zp", [(False, 0.02, 128), (True, 0.05, 0), (True, 0.003, -21), (False, 1 / 255, 3),
+                                             (True, 0.5, 3), (False, 0.25, 100)])
 def test_quantize_dequantize(rt, orc, dev, signed, scale, zp):
     import torch
     rng = np.random.default_rng(27)
-    x = orc.f32_to_f16(np.concatenate([rng.normal(0, 3, 200001), [0.0, -0.0, 1e-4, 65504, -65504, np.inf, -np.inf]])
+    # multiples of 1/8: with the power-of-two scales every other one is an exact tie between two levels
+    x = orc.f32_to_f16(np.concatenate([rng.normal(0, 3, 200001), np.arange(-70, 70, 0.125), [0.0, -0.0, 1e-4, 65504, -65504, np.inf, -np.inf]])
                        .astype(np.float32))
     qdt = torch.int8 if signed else torch.uint8
     q = torch.empty(x.shape, dtype=qdt, device=dev)

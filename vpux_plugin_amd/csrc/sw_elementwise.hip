@@ -504,13 +504,24 @@ struct FqVecFn {
 
 // createQuantizeFn, src/vpux_compiler/src/dialect/const/attributes/quantize.cpp:91-106: the FakeQuantize onto
 // [qmin, qmax] with the limits of a launch prepared on the host (both divisions by constants, see div_const)
-template <typename TI, typename TQ>
+// SIMPLE: the host has checked that level / lm1 * (ohi - olo) + olo gives back level + olo for every level (it
+// does for the 8-bit ranges), so the second division of the FakeQuantize formula is skipped; the input is
+// limited to [ilo, ihi] first, which stands for the formula's two comparisons (the level is monotone in x).
+template <typename TI, typename TQ, bool SIMPLE>
 struct QuantFn {
     FqConst c;
     __device__ __forceinline__ TQ operator()(TI x) const {
+        if (SIMPLE) {
+            const float xc = __builtin_amdgcn_fmed3f((float)x, c.ilo, c.ihi);
+            const float m = div_const(xc - c.ilo, c.irange, c.r_irange) * c.lm1;  // >= 0
+            // round half away from zero: nearest-even, then a tie that went down to the even neighbour goes up
+            const float r = __builtin_rintf(m);
+            return (TQ)((int)r + (int)c.olo + (m - r == 0.5f ? 1 : 0));
+        }
         return (TQ)(int)fq_f32_const((float)x, c);
     }
 };
+
 
 // vpux::dequantize, include/vpux/compiler/utils/quantization.hpp:208-210: double product -> float
 // PLAIN: every nonzero result is at least 2^-14 in magnitude and finite, where the reference's
@@ -1059,8 +1070,7 @@ static int quantize_impl(const MemRef& in, const MemRef& out, double scale, int6
                          hipStream_t s) {
     // Limits of the FakeQuantize the reference quantizer is built from (quantize.cpp:91-96); the same float
     // operations as the device's own preparation of a FakeQuantize (FqMap::prep).
-    QuantFn<TI, TQ> fn;
-    FqConst& c = fn.c;
+    FqConst c;
     c.ilo = (float)((double)(qmin - zp) * scale);
     c.ihi = (float)((double)(qmax - zp) * scale);
     c.olo = (float)qmin;
@@ -1070,7 +1080,11 @@ static int quantize_impl(const MemRef& in, const MemRef& out, double scale, int6
     c.r_irange = 1.0f / c.irange;
     c.r_lm1 = 1.0f / c.lm1;
     c.orange = c.ohi - c.olo;
-    return convert_impl<TI, TQ>(in, out, fn, s);
+    bool simple = c.lm1 >= 1.0f && c.lm1 <= 65535.0f && c.irange > 0.0f;
+    for (int level = 0; simple && level <= (int)c.lm1; level++)
+        simple = (float)level / c.lm1 * c.orange + c.olo == (float)(level + (int)qmin);
+    if (simple) return convert_impl<TI, TQ>(in, out, QuantFn<TI, TQ, true>{c}, s);
+    return convert_impl<TI, TQ>(in, out, QuantFn<TI, TQ, false>{c}, s);
 }
 
 int launch_quantize(const MemRef& in, const MemRef& out, double scale, int64_t zp, hipStream_t s) {
