@@ -138,6 +138,35 @@ def test_eltwise_add_broadcast_and_strides(rt, orc, dev):
     assert e.value.code == rt.ERROR_INVALID_ARGUMENT
 
 
+@pytest.mark.parametrize("shape_a,shape_b", [((37, 1024), (1, 1024)), ((37, 1024), (37, 1)), ((3, 5, 640), (1, 1, 640)),
+                                             ((70001, 512), (1, 512)), ((1, 2048), (1, 2048)), ((9, 4, 520), (9, 1, 520))])
+def test_eltwise_broadcast_over_rows(rt, orc, dev, shape_a, shape_b):
+    """Operands that merge into rows x one inner run (a value per column, or per row): the kernel whose grid walks
+    the rows, also past 65535 of them; then the same through a sub-view and for PReLU and FakeQuantize limits."""
+    import torch
+    rng = np.random.default_rng(25)
+    a = orc.f32_to_f16(rng.normal(0, 2, shape_a).astype(np.float32))
+    b = orc.f32_to_f16(rng.uniform(0.1, 2, shape_b).astype(np.float32))
+    ad, bd = to_dev(a, dev, True), to_dev(b, dev, True)
+    out = torch.empty(shape_a, dtype=torch.float16, device=dev)
+    for op in ("add", "div"):
+        rt.eltwise(op, ad, bd, out)
+        assert_f16_exact(f16_bits(out), orc.eltwise_f16(op, a, b), "%s %s %s" % (op, shape_a, shape_b))
+        rt.eltwise(op, bd, ad, out)
+        assert_f16_exact(f16_bits(out), orc.eltwise_f16(op, b, a), "%s %s %s" % (op, shape_b, shape_a))
+    rt.prelu(ad, bd, out)
+    assert_f16_exact(f16_bits(out), orc.eltwise_f16("prelu", a, b), "prelu %s %s" % (shape_a, shape_b))
+    if len(shape_a) == 2 and shape_a[0] > 4:
+        o2 = torch.zeros(shape_a, dtype=torch.float16, device=dev)
+        rt.eltwise("add", ad[2:-1], bd if shape_b[0] == 1 else bd[2:-1], o2[2:-1])
+        want = np.zeros_like(a)
+        want[2:-1] = orc.eltwise_f16("add", a[2:-1], b if shape_b[0] == 1 else b[2:-1])
+        assert_f16_exact(f16_bits(o2), want, "rows sub-view")
+    lo = orc.f32_to_f16(-b.view(np.float16).astype(np.float32))
+    rt.fake_quantize(ad, to_dev(lo, dev, True), bd, to_dev(lo, dev, True), bd, 256, out)
+    assert_f16_exact(f16_bits(out), orc.fake_quantize_f16(a, lo, b, lo, b, 256), "fake_quantize limits %s" % (shape_b,))
+
+
 def test_eltwise_add_f32(rt, dev):
     import torch
     rng = np.random.default_rng(25)

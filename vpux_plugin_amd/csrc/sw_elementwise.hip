@@ -739,6 +739,27 @@ __device__ __forceinline__ uint32_t fdiv64(uint32_t a, uint32_t d, uint64_t m) {
     return d == 1 ? a : (uint32_t)__umul64hi((uint64_t)a, m);
 }
 
+// One vector of the output from one vector (or one broadcast value) of every input.
+template <typename T, int NOPS, class Fn>
+__device__ __forceinline__ void vnd_apply(const T* const (&src)[5], T* pout, const Fn& fn, const int64_t (&off)[NOPS],
+                                          const int (&inner_stride)[6]) {
+    constexpr int VEC = 16 / sizeof(T);
+    Pack<T, VEC> x[NOPS - 1];
+#pragma unroll
+    for (int o = 0; o < NOPS - 1; o++) {
+        if (inner_stride[o]) {
+            x[o].load(src[o] + off[o], 0);
+        } else {
+            const T e = src[o][off[o]];
+#pragma unroll
+            for (int k = 0; k < VEC; k++) x[o].set(k, e);
+        }
+    }
+    Pack<T, VEC> y;
+    fn(x, y);
+    y.store(pout + off[NOPS - 1], 0);
+}
+
 template <typename T, int NOPS, class Fn>
 __global__ __launch_bounds__(kBlock) void vnd_kernel(const T* p0, const T* p1, const T* p2, const T* p3, const T* p4, T* pout,
                                                      Fn fn, VndIndex ix, uint32_t total_vec) {
@@ -757,21 +778,25 @@ __global__ __launch_bounds__(kBlock) void vnd_kernel(const T* p0, const T* p1, c
 #pragma unroll
         for (int o = 0; o < NOPS; o++) off[o] += (int64_t)r * ix.stride[o][d];
     }
-    const T* src[5] = {p0, p1, p2, p3, p4};
-    Pack<T, VEC> x[NOPS - 1];
+    const T* const src[5] = {p0, p1, p2, p3, p4};
+    vnd_apply<T, NOPS, Fn>(src, pout, fn, off, ix.inner_stride);
+}
+
+// The same for tensors that merge into rows x one inner run (a bias or slope per column, a scale per row): the
+// row comes from the grid, so its offsets are scalar arithmetic and a lane only scales its position in the row.
+constexpr unsigned kRowsPerGridY = 65535;
+template <typename T, int NOPS, class Fn>
+__global__ __launch_bounds__(kBlock) void vrow_kernel(const T* p0, const T* p1, const T* p2, const T* p3, const T* p4, T* pout,
+                                                      Fn fn, VndIndex ix, uint32_t rows) {
+    constexpr int VEC = 16 / sizeof(T);
+    const uint32_t iv = blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t row = blockIdx.y + blockIdx.z * kRowsPerGridY;
+    if (iv >= ix.vec_per_row || row >= rows) return;
+    int64_t off[NOPS];
 #pragma unroll
-    for (int o = 0; o < NOPS - 1; o++) {
-        if (ix.inner_stride[o]) {
-            x[o].load(src[o] + off[o], 0);
-        } else {
-            const T e = src[o][off[o]];
-#pragma unroll
-            for (int k = 0; k < VEC; k++) x[o].set(k, e);
-        }
-    }
-    Pack<T, VEC> y;
-    fn(x, y);
-    y.store(pout + off[NOPS - 1], 0);
+    for (int o = 0; o < NOPS; o++) off[o] = (int64_t)row * ix.stride[o][0] + (int64_t)iv * VEC * ix.inner_stride[o];
+    const T* const src[5] = {p0, p1, p2, p3, p4};
+    vnd_apply<T, NOPS, Fn>(src, pout, fn, off, ix.inner_stride);
 }
 
 // Host side: merges dimensions that every operand walks contiguously or not at all, then checks
@@ -830,6 +855,25 @@ bool make_vnd(const MemRef* const (&ops)[NOPS], VndIndex& ix, uint32_t& total_ve
     }
     total_vec = (uint32_t)total;
     return total > 0;
+}
+
+template <typename T, int NOPS, class Fn>
+int launch_vnd(const T* p0, const T* p1, const T* p2, const T* p3, const T* p4, T* pout, const Fn& fn, const VndIndex& vx,
+               uint32_t total_vec, hipStream_t s) {
+    if (vx.nd <= 1 && vx.vec_per_row >= 64) {
+        const uint32_t rows = vx.nd == 1 ? vx.dims[0] : 1;
+        const dim3 grid((vx.vec_per_row + kBlock - 1) / kBlock, rows < kRowsPerGridY ? rows : kRowsPerGridY,
+                        (rows + kRowsPerGridY - 1) / kRowsPerGridY);
+        if (grid.z <= 65535) {
+            hipLaunchKernelGGL((vrow_kernel<T, NOPS, Fn>), grid, dim3(kBlock), 0, s, p0, p1, p2, p3, p4, pout, fn, vx, rows);
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
+    }
+    hipLaunchKernelGGL((vnd_kernel<T, NOPS, Fn>), dim3((total_vec + kBlock - 1) / kBlock), dim3(kBlock), 0, s, p0, p1, p2, p3, p4,
+                       pout, fn, vx, total_vec);
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
 }
 
 int grid_1d(int64_t n, unsigned* blocks) {
@@ -961,11 +1005,8 @@ static int eltwise_impl(const MemRef& a, const MemRef& b, const MemRef& out, hip
         VndIndex vx;
         uint32_t total_vec = 0;
         if (make_vnd<T, 3>(ops, vx, total_vec)) {
-            hipLaunchKernelGGL((vnd_kernel<T, 3, VecFn>), dim3((total_vec + kBlock - 1) / kBlock), dim3(kBlock), 0, s,
-                               (const T*)a.data, (const T*)b.data, (const T*)nullptr, (const T*)nullptr, (const T*)nullptr,
-                               (T*)out.data, VecFn{}, vx, total_vec);
-            VPX_HIP_CHECK(hipGetLastError());
-            return VPX_RESULT_SUCCESS;
+            return launch_vnd<T, 3, VecFn>((const T*)a.data, (const T*)b.data, (const T*)nullptr, (const T*)nullptr, (const T*)nullptr,
+                                           (T*)out.data, VecFn{}, vx, total_vec, s);
         }
     }
     NdIndex ix{};
@@ -1036,12 +1077,9 @@ int launch_fake_quantize(const MemRef& in, const MemRef lims[4], const MemRef& o
         VndIndex vx;
         uint32_t total_vec = 0;
         if (make_vnd<half_t, 6>(ops, vx, total_vec)) {
-            hipLaunchKernelGGL((vnd_kernel<half_t, 6, FqVecFn>), dim3((total_vec + kBlock - 1) / kBlock), dim3(kBlock), 0, s,
-                               (const half_t*)in.data, (const half_t*)lims[0].data, (const half_t*)lims[1].data,
-                               (const half_t*)lims[2].data, (const half_t*)lims[3].data, (half_t*)out.data, FqVecFn{lm1}, vx,
-                               total_vec);
-            VPX_HIP_CHECK(hipGetLastError());
-            return VPX_RESULT_SUCCESS;
+            return launch_vnd<half_t, 6, FqVecFn>((const half_t*)in.data, (const half_t*)lims[0].data, (const half_t*)lims[1].data,
+                                                  (const half_t*)lims[2].data, (const half_t*)lims[3].data, (half_t*)out.data,
+                                                  FqVecFn{lm1}, vx, total_vec, s);
         }
     }
     NdIndex io{}, lim{};
