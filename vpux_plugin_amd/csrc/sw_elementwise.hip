@@ -67,6 +67,7 @@ struct Pack {
 };
 
 constexpr int kBlock = 256;
+constexpr unsigned kRowsPerGridY = 65535;  // rows one grid.y covers in the kernels that take the row from the grid
 constexpr int kUnroll = 4;
 
 // fp32 -> fp16 with the exact behaviour of vpux::type::float16
@@ -644,14 +645,20 @@ __global__ __launch_bounds__(kBlock) void dynq_scalar_kernel(DynQuantMap f, int6
 // (per-row or per-group scales of a weight matrix) and `ix` counts the innermost dimension in vectors.
 // PER_VALUE: scale and zero point run along the innermost dimension with the values (per-column parameters): a lane
 // reads VEC of each, contiguous like its values.
-template <typename TQ, typename TS, typename TO, int VEC, bool PER_VALUE = false>
+template <typename TQ, typename TS, typename TO, int VEC, bool PER_VALUE = false, bool GRID2D = false>
 __global__ __launch_bounds__(kBlock) void dyn_dequant_kernel(const TQ* __restrict__ in, const TS* __restrict__ scale,
                                                              const uint8_t* __restrict__ zp, int zp_signed, TO* __restrict__ out,
                                                              NdIndex ix, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n) return;
     int64_t off[4] = {0, 0, 0, 0};
-    if (n < (1ll << 32)) {  // 32-bit divisions: a quarter of the instructions of the 64-bit ones
+    if (GRID2D) {  // at most two dimensions: the position in the row from grid x, the row from grid y and z
+        const uint32_t row = blockIdx.y + blockIdx.z * kRowsPerGridY;
+        if (i >= ix.dims[0] || (ix.nd == 2 && row >= (uint32_t)ix.dims[1])) return;
+#pragma unroll
+        for (int o = 0; o < 4; o++) off[o] = i * ix.stride[o][0] + (ix.nd == 2 ? (int64_t)row * ix.stride[o][1] : 0);
+    } else if (i >= n) {
+        return;
+    } else if (n < (1ll << 32)) {  // 32-bit divisions: a quarter of the instructions of the 64-bit ones
         uint32_t lin = (uint32_t)i;
         for (int d = 0; d < ix.nd; d++) {
             const uint32_t q = lin / (uint32_t)ix.dims[d];
@@ -784,7 +791,6 @@ __global__ __launch_bounds__(kBlock) void vnd_kernel(const T* p0, const T* p1, c
 
 // The same for tensors that merge into rows x one inner run (a bias or slope per column, a scale per row): the
 // row comes from the grid, so its offsets are scalar arithmetic and a lane only scales its position in the row.
-constexpr unsigned kRowsPerGridY = 65535;
 template <typename T, int NOPS, class Fn>
 __global__ __launch_bounds__(kBlock) void vrow_kernel(const T* p0, const T* p1, const T* p2, const T* p3, const T* p4, T* pout,
                                                       Fn fn, VndIndex ix, uint32_t rows) {
@@ -1188,6 +1194,29 @@ int launch_dynamic_quantize(const MemRef& in, const MemRef& out, const MemRef& s
     return VPX_RESULT_SUCCESS;
 }
 
+// Drops unit dimensions and merges neighbours that every operand walks as one run (or not at all).
+static void merge_index(NdIndex& ix, int slots) {
+    int nd = 0;
+    for (int d = 0; d < ix.nd; d++) {
+        if (ix.dims[d] == 1) continue;
+        bool merge = nd > 0 && (int64_t)ix.dims[nd - 1] * ix.dims[d] < (1ll << 31);
+        for (int o = 0; o < slots && merge; o++) merge = ix.stride[o][d] == ix.stride[o][nd - 1] * ix.dims[nd - 1];
+        if (merge) {
+            ix.dims[nd - 1] *= ix.dims[d];
+        } else {
+            ix.dims[nd] = ix.dims[d];
+            for (int o = 0; o < slots; o++) ix.stride[o][nd] = ix.stride[o][d];
+            nd++;
+        }
+    }
+    if (nd == 0) {
+        ix.dims[0] = 1;
+        for (int o = 0; o < slots; o++) ix.stride[o][0] = 0;
+        nd = 1;
+    }
+    ix.nd = nd;
+}
+
 // ---------------------------------------------------------------- dynamic_dequantize
 template <typename TQ, typename TS, typename TO>
 static int dyn_dequant_impl(const MemRef& in, const MemRef& scale, const MemRef* zp, const MemRef& out, hipStream_t s) {
@@ -1204,6 +1233,9 @@ static int dyn_dequant_impl(const MemRef& in, const MemRef& scale, const MemRef*
     if (rc) return rc;
     int64_t n = out.numel();
     if (n == 0) return VPX_RESULT_SUCCESS;
+    if (!zp)
+        for (int d = 0; d < ix.nd; d++) ix.stride[2][d] = ix.stride[1][d];  // an absent operand must not block a merge
+    merge_index(ix, 4);
     const uint8_t* pz = zp ? (const uint8_t*)zp->data : nullptr;
     const int zp_signed = zp && zp->dtype == VPX_NN_I8 ? 1 : 0;
     constexpr int VEC = 16 / (int)sizeof(TO);
@@ -1226,6 +1258,19 @@ static int dyn_dequant_impl(const MemRef& in, const MemRef& scale, const MemRef*
             if (zp) ix.stride[2][0] = VEC;
         }
         n /= VEC;
+        const uint32_t rows = ix.nd == 2 ? (uint32_t)ix.dims[1] : 1;
+        if (ix.nd <= 2 && ix.dims[0] >= 64 && (rows + kRowsPerGridY - 1) / kRowsPerGridY <= 65535) {
+            const dim3 grid(((unsigned)ix.dims[0] + kBlock - 1) / kBlock, rows < kRowsPerGridY ? rows : kRowsPerGridY,
+                            (rows + kRowsPerGridY - 1) / kRowsPerGridY);
+            if (per_row)
+                hipLaunchKernelGGL((dyn_dequant_kernel<TQ, TS, TO, VEC, false, true>), grid, dim3(kBlock), 0, s, (const TQ*)in.data,
+                                   (const TS*)scale.data, pz, zp_signed, (TO*)out.data, ix, n);
+            else
+                hipLaunchKernelGGL((dyn_dequant_kernel<TQ, TS, TO, VEC, true, true>), grid, dim3(kBlock), 0, s, (const TQ*)in.data,
+                                   (const TS*)scale.data, pz, zp_signed, (TO*)out.data, ix, n);
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
         rc = grid_1d(n, &blocks);
         if (rc) return rc;
         if (per_row)
