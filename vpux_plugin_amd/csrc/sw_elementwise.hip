@@ -508,17 +508,25 @@ struct FqVecFn {
 // SIMPLE: the host has checked that level / lm1 * (ohi - olo) + olo gives back level + olo for every level (it
 // does for the 8-bit ranges), so the second division of the FakeQuantize formula is skipped; the input is
 // limited to [ilo, ihi] first, which stands for the formula's two comparisons (the level is monotone in x).
+// One value of the SIMPLE form below: `c` needs ilo, ihi, irange, r_irange, lm1 and olo.
+__device__ __forceinline__ int quantize_simple(float x, const FqConst& c) {
+    const float m = div_const(__builtin_amdgcn_fmed3f(x, c.ilo, c.ihi) - c.ilo, c.irange, c.r_irange) * c.lm1;  // >= 0
+    // round half away from zero: nearest-even, then a tie that went down to the even neighbour goes up
+    const float r = __builtin_rintf(m);
+    return (int)r + (int)c.olo + (m - r == 0.5f ? 1 : 0);
+}
+// Whether level / lm1 * (qmax - qmin) + qmin gives back level + qmin for every level, in float arithmetic (host).
+static bool levels_are_identity(float qmin, float qmax, float lm1) {
+    bool same = lm1 >= 1.0f && lm1 <= 65535.0f;
+    for (int level = 0; same && level <= (int)lm1; level++) same = (float)level / lm1 * (qmax - qmin) + qmin == (float)(level + (int)qmin);
+    return same;
+}
+
 template <typename TI, typename TQ, bool SIMPLE>
 struct QuantFn {
     FqConst c;
     __device__ __forceinline__ TQ operator()(TI x) const {
-        if (SIMPLE) {
-            const float xc = __builtin_amdgcn_fmed3f((float)x, c.ilo, c.ihi);
-            const float m = div_const(xc - c.ilo, c.irange, c.r_irange) * c.lm1;  // >= 0
-            // round half away from zero: nearest-even, then a tie that went down to the even neighbour goes up
-            const float r = __builtin_rintf(m);
-            return (TQ)((int)r + (int)c.olo + (m - r == 0.5f ? 1 : 0));
-        }
+        if (SIMPLE) return (TQ)quantize_simple((float)x, c);
         return (TQ)(int)fq_f32_const((float)x, c);
     }
 };
@@ -537,6 +545,13 @@ struct DequantFn {
         return narrow<TO>(r);
     }
 };
+
+// The same product with a scale that is a float (the per-axis tables hold what the blob shipped as fp16 or fp32):
+// an 8-bit difference times 24 bits is exact in double, so the double product rounded to float is the float
+// product rounded once.
+__device__ __forceinline__ float dequant_f32(int diff, float scale) {
+    return (float)diff * scale;
+}
 
 // ---------------------------------------------------------------- strided / broadcast path
 template <int NOPS>
@@ -1124,10 +1139,7 @@ static int quantize_impl(const MemRef& in, const MemRef& out, double scale, int6
     c.r_irange = 1.0f / c.irange;
     c.r_lm1 = 1.0f / c.lm1;
     c.orange = c.ohi - c.olo;
-    bool simple = c.lm1 >= 1.0f && c.lm1 <= 65535.0f && c.irange > 0.0f;
-    for (int level = 0; simple && level <= (int)c.lm1; level++)
-        simple = (float)level / c.lm1 * c.orange + c.olo == (float)(level + (int)qmin);
-    if (simple) return convert_impl<TI, TQ>(in, out, QuantFn<TI, TQ, true>{c}, s);
+    if (c.irange > 0.0f && levels_are_identity(c.olo, c.ohi, c.lm1)) return convert_impl<TI, TQ>(in, out, QuantFn<TI, TQ, true>{c}, s);
     return convert_impl<TI, TQ>(in, out, QuantFn<TI, TQ, false>{c}, s);
 }
 
@@ -1326,10 +1338,19 @@ struct AxisChunk {
 
 // Kernel arguments are the one path from host to device memory that a caller's graph capture can
 // record: the per-channel table goes to the workspace 256 entries per launch.
-__global__ __launch_bounds__(256) void fill_axis_table(float4* table, AxisChunk c, int count) {
-    // {a, b, b - a, 1 / (b - a)}: the last two are the constants of a channel's FakeQuantize (unused by dequantize)
+__global__ __launch_bounds__(256) void fill_axis_table(float4* table, float* planes, int64_t n, AxisChunk c, int count) {
+    // {a, b, b - a, 1 / (b - a)}: the last two are the constants of a channel's FakeQuantize (unused by dequantize).
+    // Behind the table the same four values lie as four planes of n floats, for the kernels in which a lane
+    // takes eight adjacent channels and reads each constant of the eight as two 128-bit words.
     const float lo = c.a[threadIdx.x], hi = c.b[threadIdx.x];
-    if ((int)threadIdx.x < count) table[threadIdx.x] = float4{lo, hi, hi - lo, 1.0f / (hi - lo)};
+    if ((int)threadIdx.x < count) {
+        const float4 e{lo, hi, hi - lo, 1.0f / (hi - lo)};
+        table[threadIdx.x] = e;
+        planes[threadIdx.x] = e.x;
+        planes[n + threadIdx.x] = e.y;
+        planes[2 * n + threadIdx.x] = e.z;
+        planes[3 * n + threadIdx.x] = e.w;
+    }
 }
 
 struct AxisGeom {
@@ -1359,12 +1380,12 @@ __global__ __launch_bounds__(kBlock) void dequantize_axis_kernel(const TQ* __res
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i >= n) return;
     const float4 p = table[axis_channel(i, g)];
-    out[i] = narrow<TO>((float)((double)((int)in[i] - (int)p.y) * (double)p.x));
+    out[i] = narrow<TO>(dequant_f32((int)in[i] - (int)p.y, p.x));
 }
 
 // One 128-bit access of the wider operand per lane: the axis is not the innermost dimension and the run below it is
 // a multiple of the vector, so a lane's values share a channel, whose FakeQuantize constants come from its table entry.
-template <typename TI, typename TQ>
+template <typename TI, typename TQ, bool SIMPLE>
 __global__ __launch_bounds__(kBlock) void quantize_axis_vec_kernel(const TI* __restrict__ in, TQ* __restrict__ out,
                                                                    const float4* __restrict__ table, AxisGeom g, uint32_t n_vec,
                                                                    float qmin, float qmax, float lm1) {
@@ -1377,7 +1398,7 @@ __global__ __launch_bounds__(kBlock) void quantize_axis_vec_kernel(const TI* __r
     const float4 p = table[axis_channel(v * V, g)];
     const FqConst c{p.x, p.y, qmin, qmax, lm1, p.z, p.w, 1.0f / lm1, qmax - qmin};
 #pragma unroll
-    for (int k = 0; k < V; k++) y.set(k, (TQ)(int)fq_f32_const((float)x.get(k), c));
+    for (int k = 0; k < V; k++) y.set(k, SIMPLE ? (TQ)quantize_simple((float)x.get(k), c) : (TQ)(int)fq_f32_const((float)x.get(k), c));
     y.store(out, v);
 }
 
@@ -1392,7 +1413,7 @@ __global__ __launch_bounds__(kBlock) void dequantize_axis_vec_kernel(const TQ* _
     const float4 p = table[axis_channel(v * V, g)];
     float r[V];
 #pragma unroll
-    for (int k = 0; k < V; k++) r[k] = (float)((double)((int)x.get(k) - (int)p.y) * (double)p.x);
+    for (int k = 0; k < V; k++) r[k] = dequant_f32((int)x.get(k) - (int)p.y, p.x);
     Pack<TO, V> y;
     if constexpr (std::is_same<TO, half_t>::value) {
         half_t h[V];
@@ -1439,7 +1460,7 @@ __global__ __launch_bounds__(kBlock) void dequantize_axis_inner_kernel(const TQ*
 #pragma unroll
     for (int r = 0; r < kAxisRows; r++) {
         const int q = live && r0 + r < rows ? (int)in[(r0 + r) * count + c] : 0;
-        v[r] = (float)((double)(q - (int)p.y) * (double)p.x);
+        v[r] = dequant_f32(q - (int)p.y, p.x);
     }
     if constexpr (std::is_same<TO, half_t>::value) {
         half_t h[kAxisRows];
@@ -1511,9 +1532,9 @@ int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t
     }
     void* mem = nullptr;
     if (keep) {
-        VPX_HIP_CHECK(hipMalloc(&mem, sizeof(float4) * (size_t)n));
+        VPX_HIP_CHECK(hipMalloc(&mem, 2 * sizeof(float4) * (size_t)n));
     } else {
-        const int rc = get_workspace(s, sizeof(float4) * (size_t)n, &mem);
+        const int rc = get_workspace(s, 2 * sizeof(float4) * (size_t)n, &mem);
         if (rc) return rc;
     }
     *table = (float4*)mem;
@@ -1525,7 +1546,7 @@ int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t
             ch.b[k] = b[c0 + k];
         }
         for (int k = cnt; k < 256; k++) ch.a[k] = ch.b[k] = 0.f;
-        hipLaunchKernelGGL(fill_axis_table, dim3(1), dim3(256), 0, s, *table + c0, ch, cnt);
+        hipLaunchKernelGGL(fill_axis_table, dim3(1), dim3(256), 0, s, *table + c0, (float*)(*table + n) + c0, n, ch, cnt);
         VPX_HIP_CHECK(hipGetLastError());
     }
     if (keep) {
@@ -1533,6 +1554,106 @@ int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t
         g_axis_tables.push_back(AxisTableEntry{dev, s, std::vector<float>(a, a + n), std::vector<float>(b, b + n), *table});
     }
     return VPX_RESULT_SUCCESS;
+}
+
+// The same with eight adjacent channels per lane, for channel counts that are a multiple of eight: one 128-bit
+// access per lane and row for the 16-bit side, the eight channels' constants kept in registers across the rows.
+template <typename TI, typename TQ, bool SIMPLE>
+__global__ __launch_bounds__(kBlock) void quantize_axis_inner8_kernel(const TI* __restrict__ in, TQ* __restrict__ out,
+                                                                      const float4* __restrict__ table, uint32_t count, uint32_t rows,
+                                                                      float qmin, float qmax, float lm1) {
+    const uint32_t cvecs = count / 8;
+    const uint32_t ctiles = (cvecs + kBlock - 1) / kBlock;
+    const uint32_t cv = (blockIdx.x % ctiles) * kBlock + threadIdx.x;
+    const uint32_t r0 = (blockIdx.x / ctiles) * kAxisRows;
+    if (cv >= cvecs) return;
+    float4 p[8];
+    {
+        const float4* planes = reinterpret_cast<const float4*>(table + count);  // four planes of count floats
+        const uint32_t pv = count / 4;                                         // float4 words per plane
+        float4 q[4][2];
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            q[c][0] = planes[c * pv + cv * 2];
+            q[c][1] = planes[c * pv + cv * 2 + 1];
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int h = k >> 2, e = k & 3;
+            auto pick = [&](const float4& v) { return e == 0 ? v.x : (e == 1 ? v.y : (e == 2 ? v.z : v.w)); };
+            p[k] = float4{pick(q[0][h]), pick(q[1][h]), pick(q[2][h]), pick(q[3][h])};
+        }
+    }
+    const float r_lm1 = 1.0f / lm1, orange = qmax - qmin;
+    constexpr int kBatch = 8;  // rows whose loads are issued together
+#pragma unroll
+    for (int rb = 0; rb < kAxisRows; rb += kBatch) {
+        Pack<TI, 8> xs[kBatch];
+#pragma unroll
+        for (int r = 0; r < kBatch; r++)
+            if (r0 + rb + r < rows) xs[r].load(in, (int64_t)(r0 + rb + r) * cvecs + cv);
+#pragma unroll
+        for (int r = 0; r < kBatch; r++) {
+        if (r0 + rb + r >= rows) break;
+        const int64_t v = (int64_t)(r0 + rb + r) * cvecs + cv;
+        const Pack<TI, 8>& x = xs[r];
+        Pack<TQ, 8> y;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float f = (float)x.get(k);
+            const FqConst cst{p[k].x, p[k].y, qmin, qmax, lm1, p[k].z, p[k].w, r_lm1, orange};
+            y.set(k, SIMPLE ? (TQ)quantize_simple(f, cst) : (TQ)(int)fq_f32_const(f, cst));
+        }
+        y.store(out, v);
+        }
+    }
+}
+template <typename TQ, typename TO>
+__global__ __launch_bounds__(kBlock) void dequantize_axis_inner8_kernel(const TQ* __restrict__ in, TO* __restrict__ out,
+                                                                        const float4* __restrict__ table, uint32_t count, uint32_t rows) {
+    const uint32_t cvecs = count / 8;
+    const uint32_t ctiles = (cvecs + kBlock - 1) / kBlock;
+    const uint32_t cv = (blockIdx.x % ctiles) * kBlock + threadIdx.x;
+    const uint32_t r0 = (blockIdx.x / ctiles) * kAxisRows;
+    const bool live = cv < cvecs;  // dead lanes still take part in the votes of narrow_vec
+    float sc[8];
+    int zp[8];
+    {
+        const float4* planes = reinterpret_cast<const float4*>(table + count);  // plane 0: scales, plane 1: zero points
+        const uint32_t pv = count / 4, at = live ? cv * 2 : 0;
+        const float4 s0 = planes[at], s1 = planes[at + 1], z0 = planes[pv + at], z1 = planes[pv + at + 1];
+        const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        const float zv[8] = {z0.x, z0.y, z0.z, z0.w, z1.x, z1.y, z1.z, z1.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            sc[k] = sv[k];
+            zp[k] = (int)zv[k];
+        }
+    }
+    Pack<TQ, 8> xs[kAxisRows];  // every row's load is issued before the first result is needed
+#pragma unroll
+    for (int r = 0; r < kAxisRows; r++)
+        if (r0 + r < rows) xs[r].load(in, (int64_t)(r0 + r) * cvecs + (live ? cv : 0));
+#pragma unroll
+    for (int r = 0; r < kAxisRows; r++) {
+        if (r0 + r >= rows) break;  // uniform over the workgroup
+        const int64_t v = (int64_t)(r0 + r) * cvecs + (live ? cv : 0);
+        const Pack<TQ, 8>& x = xs[r];
+        float f[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) f[k] = dequant_f32((int)x.get(k) - zp[k], sc[k]);
+        Pack<TO, 8> y;
+        if constexpr (std::is_same<TO, half_t>::value) {
+            half_t h[8];
+            narrow_vec(f, h);
+#pragma unroll
+            for (int k = 0; k < 8; k++) y.set(k, h[k]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) y.set(k, f[k]);
+        }
+        if (live) y.store(out, v);
+    }
 }
 
 template <typename TI, typename TQ>
@@ -1555,14 +1676,30 @@ int quantize_axis_impl(const MemRef& in, const MemRef& out, const double* scales
     constexpr uint32_t V = 16 / sizeof(TI);
     const bool al = (reinterpret_cast<uintptr_t>(in.data) & 15) == 0 && (reinterpret_cast<uintptr_t>(out.data) % V) == 0;
     const dim3 vgrid((total / V + kBlock - 1) / kBlock);
-    if (al && g.inner % V == 0)
-        hipLaunchKernelGGL((quantize_axis_vec_kernel<TI, TQ>), vgrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data, table,
-                           g, total / V, fmin_, fmax_, lm1);
+    const bool simple = levels_are_identity(fmin_, fmax_, lm1);
+    if (al && g.inner % V == 0) {
+        if (simple)
+            hipLaunchKernelGGL((quantize_axis_vec_kernel<TI, TQ, true>), vgrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data, table,
+                               g, total / V, fmin_, fmax_, lm1);
+        else
+            hipLaunchKernelGGL((quantize_axis_vec_kernel<TI, TQ, false>), vgrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data, table,
+                               g, total / V, fmin_, fmax_, lm1);
+    }
     else if (g.inner == 1) {
         const uint32_t rows = total / g.count;
-        const dim3 igrid(((g.count + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
-        hipLaunchKernelGGL((quantize_axis_inner_kernel<TI, TQ>), igrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data, table, g.count,
-                           rows, fmin_, fmax_, lm1);
+        if (g.count % 8 == 0 && (reinterpret_cast<uintptr_t>(in.data) % (8 * sizeof(TI))) == 0 && (reinterpret_cast<uintptr_t>(out.data) & 7) == 0) {
+            const dim3 igrid(((g.count / 8 + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
+            if (simple)
+                hipLaunchKernelGGL((quantize_axis_inner8_kernel<TI, TQ, true>), igrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data,
+                                   table, g.count, rows, fmin_, fmax_, lm1);
+            else
+                hipLaunchKernelGGL((quantize_axis_inner8_kernel<TI, TQ, false>), igrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data,
+                                   table, g.count, rows, fmin_, fmax_, lm1);
+        } else {
+            const dim3 igrid(((g.count + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
+            hipLaunchKernelGGL((quantize_axis_inner_kernel<TI, TQ>), igrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data, table,
+                               g.count, rows, fmin_, fmax_, lm1);
+        }
     }
     else
         hipLaunchKernelGGL((quantize_axis_kernel<TI, TQ>), dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (const TI*)in.data,
@@ -1592,9 +1729,15 @@ int dequantize_axis_impl(const MemRef& in, const MemRef& out, const double* scal
                            table, g, total / V);
     else if (g.inner == 1) {
         const uint32_t rows = total / g.count;
-        const dim3 igrid(((g.count + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
-        hipLaunchKernelGGL((dequantize_axis_inner_kernel<TQ, TO>), igrid, dim3(kBlock), 0, s, (const TQ*)in.data, (TO*)out.data, table,
-                           g.count, rows);
+        if (g.count % 8 == 0 && (reinterpret_cast<uintptr_t>(in.data) & 7) == 0 && (reinterpret_cast<uintptr_t>(out.data) % (8 * sizeof(TO))) == 0) {
+            const dim3 igrid(((g.count / 8 + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
+            hipLaunchKernelGGL((dequantize_axis_inner8_kernel<TQ, TO>), igrid, dim3(kBlock), 0, s, (const TQ*)in.data, (TO*)out.data, table,
+                               g.count, rows);
+        } else {
+            const dim3 igrid(((g.count + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
+            hipLaunchKernelGGL((dequantize_axis_inner_kernel<TQ, TO>), igrid, dim3(kBlock), 0, s, (const TQ*)in.data, (TO*)out.data, table,
+                               g.count, rows);
+        }
     }
     else
         hipLaunchKernelGGL((dequantize_axis_kernel<TQ, TO>), dim3((total + kBlock - 1) / kBlock), dim3(kBlock), 0, s, (const TQ*)in.data,
