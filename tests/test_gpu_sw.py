@@ -611,6 +611,9 @@ MVN6_CASES = [
     ((3, 2, 150, 200), (2, 3), None, None),
     ((2, 20001), (1,), None, (1, 20001)),                 # ... or one workgroup per row when there is a bias
     ((6, 1, 64), (1, 2), None, None),                     # unit dimension among the axes
+    ((300, 50), (1,), None, None),                        # many short rows, not a multiple of 8: runs of rows per workgroup
+    ((64, 3, 7, 7), (2, 3), None, None),
+    ((70, 1001), (-1,), None, None),
 ]
 
 
@@ -751,7 +754,9 @@ def _mvn(rt, dev, xb, across, nv, eps, order="NCHW"):
 
 
 @pytest.mark.parametrize("shape", [(2, 3, 8, 8), (1, 16, 64, 64), (3, 7, 5, 9), (2, 64, 33, 31), (1, 2, 1, 4097),
-                                   (1, 600, 64, 64)])
+                                   (1, 600, 64, 64),
+                                   # many short groups: runs of whole groups per workgroup, odd lengths, a ragged last run
+                                   (4, 64, 7, 7), (3, 50, 14, 14), (2, 333, 1, 5), (1, 70, 31, 33), (67, 1, 1, 1), (5, 13, 1, 1024)])
 @pytest.mark.parametrize("across", [True, False])
 @pytest.mark.parametrize("nv", [True, False])
 def test_mvn_nchw(rt, orc, dev, shape, across, nv):

@@ -240,6 +240,97 @@ __global__ __launch_bounds__(kThreads) void mvn_merge_kernel(const Record* parti
     if (threadIdx.x == 0) merged[group] = Record{total.n, total.mean, total.m2, 0.f};
 }
 
+// Many short groups that follow one another in memory (per-channel statistics of small planes, 14 x 14 or 7 x 7; rows
+// of a few hundred values): a workgroup takes a run of whole groups of about kSmallChunk values, moves it between
+// global memory and LDS in aligned 128-bit words whatever the group length (the values of neighbouring groups that
+// share its first and last word are read too, but never written), and half-wavefronts normalise one group each in LDS:
+// sum, centred sum of squares, scale -- three passes over at most kSmallGroup values.
+constexpr int kSmallGroup = 1024;   // longest group this form takes
+constexpr int kSmallChunk = 4096;   // values per workgroup, at most
+__device__ __forceinline__ float half_wave_sum(float v) {
+    v += dppf<0xB1>(v);
+    v += dppf<0x4E>(v);
+    v += dppf<0x141>(v);
+    v += dppf<0x140>(v);
+    return v + swz16(v);
+}
+template <int K>  // values per lane: a group has at most 32 K
+__global__ __launch_bounds__(kThreads) void mvn_small_groups_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                                    int64_t groups, int len, int per_wg, int normalize_variance,
+                                                                    int eps_mode, float eps) {
+    __shared__ __attribute__((aligned(16))) half_t buf[kSmallChunk + 16];
+    const int64_t g0 = (int64_t)blockIdx.x * per_wg;
+    const int ng = groups - g0 < per_wg ? (int)(groups - g0) : per_wg;
+    const int64_t e0 = g0 * len, e1 = e0 + (int64_t)ng * len, total = groups * len;
+    const int64_t a0 = e0 & ~7ll;                  // first aligned word that holds a value of the run
+    const int words = (int)((e1 - a0 + 7) >> 3);
+    for (int w = threadIdx.x; w < words; w += kThreads) {
+        const int64_t at = a0 + (int64_t)w * 8;
+        if (at + 8 <= total) {
+            *reinterpret_cast<u32x4*>(buf + w * 8) = *reinterpret_cast<const u32x4*>(in + at);
+        } else {
+            for (int k = 0; k < 8; k++) buf[w * 8 + k] = at + k < total ? in[at + k] : (half_t)0.f;
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 31, team = threadIdx.x >> 5;
+    const float n = (float)len;
+    for (int g = team; g < ng; g += kThreads / 32) {   // uniform per half-wavefront
+        half_t* x = buf + (int)(e0 - a0) + g * len;
+        float v[K];  // the lane's values stay in registers between the passes
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int i = lane + 32 * k;
+            v[k] = i < len ? (float)x[i] : 0.f;
+            sum += v[k];
+        }
+        const float mean = half_wave_sum(sum) / n;
+        float q = 0.f;
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const float d = v[k] - mean;
+            q += lane + 32 * k < len ? d * d : 0.f;
+        }
+        const float inv = !normalize_variance ? 1.0f
+                          : (eps_mode == 0 ? 1.0f / __builtin_sqrtf(half_wave_sum(q) / n + eps) : 1.0f / (__builtin_sqrtf(half_wave_sum(q) / n) + eps));
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int i = lane + 32 * k;
+            if (i < len) x[i] = (half_t)((v[k] - mean) * inv);
+        }
+    }
+    __syncthreads();
+    for (int w = threadIdx.x; w < words; w += kThreads) {
+        const int64_t at = a0 + (int64_t)w * 8;
+        if (at >= e0 && at + 8 <= e1) {
+            __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(buf + w * 8), reinterpret_cast<u32x4*>(out + at));
+        } else {
+            for (int k = 0; k < 8; k++)
+                if (at + k >= e0 && at + k < e1) out[at + k] = buf[w * 8 + k];
+        }
+    }
+}
+
+// Whether the short-group form applies, and its launch.
+static bool small_groups_ok(const half_t* in, const half_t* out, int64_t groups, int64_t len) {
+    return len >= 1 && len <= kSmallGroup && groups >= 64 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
+           (groups + (kSmallChunk / len) - 1) / (kSmallChunk / len) < (1ll << 31);
+}
+static int launch_small_groups(const half_t* in, half_t* out, int64_t groups, int64_t len, int nv, int eps_mode, float eps, hipStream_t s) {
+    const int per_wg = (int)(kSmallChunk / len);
+    const unsigned blocks = (unsigned)((groups + per_wg - 1) / per_wg);
+#define VPX_SMALL(K) hipLaunchKernelGGL(mvn_small_groups_kernel<K>, dim3(blocks), dim3(kThreads), 0, s, in, out, groups, (int)len, per_wg, nv, eps_mode, eps)
+    if (len <= 64) VPX_SMALL(2);
+    else if (len <= 128) VPX_SMALL(4);
+    else if (len <= 256) VPX_SMALL(8);
+    else if (len <= 512) VPX_SMALL(16);
+    else VPX_SMALL(32);
+#undef VPX_SMALL
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
 // position (counted from the innermost memory dimension) of logical dimension `logical`
 int mem_pos_of(uint64_t order, int nd, int logical) {
     for (int i = 0; i < nd; i++)
@@ -869,6 +960,7 @@ int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool n
     } else {  // channel-minor layout, per-channel statistics
         return launch_channel_minor(pi, po, N, S, C, nv, eps, s);
     }
+    if (small_groups_ok(pi, po, groups, group_size)) return launch_small_groups(pi, po, groups, group_size, nv, 0, eps, s);
     const bool aligned = group_size % 8 == 0 && (reinterpret_cast<uintptr_t>(pi) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(po) & 15) == 0;
     return aligned ? launch_groups<true>(pi, po, groups, group_size, nv, eps, s)
@@ -1148,6 +1240,10 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
         const bool aligned = row_len % 8 == 0 && ((reinterpret_cast<uintptr_t>(pi) | reinterpret_cast<uintptr_t>(po)) & 15) == 0;
         return aligned ? launch_groups<true>(pi, po, g.rows, row_len, nv, eps, s) : launch_groups<false>(pi, po, g.rows, row_len, nv, eps, s);
     }
+    // Short contiguous rows whose length is not a multiple of eight (7 x 7 planes, rows of 100): runs of whole rows
+    // per workgroup, as for mvn1's short groups.
+    if (innermost && row_len % 8 != 0 && !scale && !bias && in.compact && out.compact && small_groups_ok(pi, po, g.rows, row_len))
+        return launch_small_groups(pi, po, g.rows, row_len, nv, eps_mode, eps, s);
     bool fast = innermost && row_len % 8 == 0 && row_len <= kMvn6MaxRegRow;
     if (fast) {
         fast = along_row(true, g.rdim, g.r_in, g.nr) == 1 && along_row(true, g.rdim, g.r_out, g.nr) == 1;
