@@ -780,10 +780,11 @@ def assert_close_f16_mvn(got_bits, want_bits, orc, what):
         what, len(bad), bad[0], g[tuple(bad[0])], w[tuple(bad[0])])
 
 
+@pytest.mark.parametrize("C", [70, 64, 264, 8, 2048])   # multiples of eight take the eight-channels-per-lane sums
 @pytest.mark.parametrize("across", [True, False])
-def test_mvn_nhwc(rt, orc, dev, across):
+def test_mvn_nhwc(rt, orc, dev, across, C):
     rng = np.random.default_rng(41)
-    x = (rng.uniform(-8, 8, (2, 9, 7, 70)) + rng.normal(0, 2, (1, 1, 1, 70))).astype(np.float32)  # N,H,W,C in memory
+    x = (rng.uniform(-8, 8, (2, 9, 7, C)) + rng.normal(0, 2, (1, 1, 1, C))).astype(np.float32)  # N,H,W,C in memory
     xb = orc.f32_to_f16(x)
     got = _mvn(rt, dev, xb, across, True, 1e-9, order="NHWC")
     assert_close_f16_mvn(got, orc.mvn_f16(xb, across, True, 1e-9, layout="NHWC"), orc, "mvn NHWC across=%s" % across)

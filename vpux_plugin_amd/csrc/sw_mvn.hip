@@ -485,6 +485,68 @@ __global__ __launch_bounds__(kThreads) void mvn_sum_cminor_kernel(const half_t* 
     if (r == 0) partial[(n * subparts + sp) * cpad + c] = add2(add2(red[0][cl], red[1][cl]), add2(red[2][cl], red[3][cl]));
 }
 
+// The same sums with eight adjacent channels per lane (channel counts that are a multiple of eight, up to 2048): a
+// lane's 128-bit loads walk the positions of its channel octet, the workgroup's lanes cover 256 / (C / 8) positions
+// at a time, and the lanes that share an octet meet in LDS.  Same partial layout as the kernel above.
+template <bool SHIFT>
+__global__ __launch_bounds__(kThreads) void mvn_sum_cminor8_kernel(const half_t* __restrict__ in, int64_t S, int64_t C,
+                                                                   int subparts, int64_t cpad, float2* __restrict__ partial) {
+    extern __shared__ float2 red8[];  // [slots][C]
+    const int cv = (int)(C / 8), slots = kThreads / cv;
+    const int sp = (int)(blockIdx.x % subparts);
+    const int64_t n = blockIdx.x / subparts;
+    const int64_t s0 = sp * S / subparts, s1 = (sp + 1) * S / subparts;
+    const int slot = threadIdx.x / cv, oct = threadIdx.x % cv;
+    float sum[8], sq[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) sum[k] = sq[k] = 0.f;
+    if (slot < slots) {
+        const half_t* px = in + n * S * C + oct * 8;
+        float shift[8];
+        {
+            const u32x4 q = *reinterpret_cast<const u32x4*>(px);
+            const half_t* h = reinterpret_cast<const half_t*>(&q);
+#pragma unroll
+            for (int k = 0; k < 8; k++) shift[k] = SHIFT ? (float)h[k] : 0.f;
+        }
+        for (int64_t i = s0 + slot; i < s1; i += slots) {
+            const u32x4 q = *reinterpret_cast<const u32x4*>(px + i * C);
+            const half_t* h = reinterpret_cast<const half_t*>(&q);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float x = (float)h[k] - shift[k];
+                sum[k] += x;
+                sq[k] += x * x;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) red8[(int64_t)slot * C + oct * 8 + k] = float2{sum[k], sq[k]};
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < C; c += kThreads) {
+        float2 t = red8[c];
+        for (int r = 1; r < slots; r++) t = add2(t, red8[(int64_t)r * C + c]);
+        partial[(n * subparts + sp) * cpad + c] = t;
+    }
+}
+
+// Launches whichever sum kernel fits; `subparts` spatial ranges per image, partials [N][subparts][cpad].
+template <bool SHIFT>
+static int launch_sum_cminor(const half_t* in, int64_t N, int64_t S, int64_t C, int64_t subparts, int64_t cpad, float2* partial,
+                             hipStream_t s) {
+    if (C % 8 == 0 && C >= 8 && C <= 2048 && (reinterpret_cast<uintptr_t>(in) & 15) == 0) {
+        const int slots = kThreads / (int)(C / 8);
+        const size_t lds = sizeof(float2) * (size_t)slots * (size_t)C;  // at most 16 KiB
+        hipLaunchKernelGGL(mvn_sum_cminor8_kernel<SHIFT>, dim3((unsigned)(N * subparts)), dim3(kThreads), lds, s, in, S, C, (int)subparts,
+                           cpad, partial);
+    } else {
+        hipLaunchKernelGGL(mvn_sum_cminor_kernel<SHIFT>, dim3((unsigned)(N * subparts * (cpad / 64))), dim3(kThreads), 0, s, in, S, C,
+                           (int)subparts, cpad, partial);
+    }
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
 __global__ __launch_bounds__(kThreads) void mvn_sum_cminor_finish_kernel(const float2* __restrict__ partial, int64_t total,
                                                                          int64_t C, int64_t cpad, int subparts, int isplit,
                                                                          SumOut o) {
@@ -894,7 +956,10 @@ __global__ __launch_bounds__(kThreads) void mvn6_generic_kernel(const half_t* __
 // a fold to {mean, 1/std}, then the element-wise pass.
 int launch_channel_minor(const half_t* in, half_t* out, int64_t N, int64_t S, int64_t C, int nv, float eps, hipStream_t s) {
     const int64_t ctiles = (C + 63) / 64, cpad = ctiles * 64;
-    int64_t subparts = (1024 + N * ctiles - 1) / (N * ctiles);
+    // spatial ranges per image: enough workgroups to fill the chip (the eight-channel kernel has no channel tiles)
+    const bool octets = C % 8 == 0 && C >= 8 && C <= 2048 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
+    const int64_t per_range = octets ? N : N * ctiles;
+    int64_t subparts = ((octets ? 2048 : 1024) + per_range - 1) / per_range;
     if (subparts > S / 64) subparts = S / 64;
     if (subparts < 1) subparts = 1;
     const int64_t per_n = S * C, piece = kThreads * 8, pieces = (per_n + piece - 1) / piece;
@@ -906,9 +971,8 @@ int launch_channel_minor(const half_t* in, half_t* out, int64_t N, int64_t S, in
     if (rc) return rc;
     float2* partial = (float2*)ws;
     float* stats = (float*)((char*)ws + partial_bytes);
-    hipLaunchKernelGGL(mvn_sum_cminor_kernel<true>, dim3((unsigned)(N * subparts * ctiles)), dim3(kThreads), 0, s, in, S, C,
-                       (int)subparts, cpad, partial);
-    VPX_HIP_CHECK(hipGetLastError());
+    rc = launch_sum_cminor<true>(in, N, S, C, subparts, cpad, partial, s);
+    if (rc) return rc;
     hipLaunchKernelGGL(mvn_cminor_stats_kernel, dim3((unsigned)((N * C + kThreads - 1) / kThreads)), dim3(kThreads), 0, s, in,
                        (const float2*)partial, stats, N * C, S, C, cpad, (int)subparts, nv, eps);
     VPX_HIP_CHECK(hipGetLastError());
@@ -1000,9 +1064,8 @@ int launch_mvn_sum(const MemRef& in, const MemRef& out, bool across_channels, bo
         void* ws = nullptr;
         rc = get_workspace(s, sizeof(float2) * (size_t)(sh.N * subparts * cpad), &ws);
         if (rc) return rc;
-        hipLaunchKernelGGL(mvn_sum_cminor_kernel<false>, dim3((unsigned)blocks), dim3(kThreads), 0, s, pi, sh.S, sh.C, (int)subparts,
-                           cpad, (float2*)ws);
-        VPX_HIP_CHECK(hipGetLastError());
+        rc = launch_sum_cminor<false>(pi, sh.N, sh.S, sh.C, subparts, cpad, (float2*)ws, s);
+        if (rc) return rc;
         hipLaunchKernelGGL(mvn_sum_cminor_finish_kernel, dim3((unsigned)((total + kThreads - 1) / kThreads)), dim3(kThreads), 0,
                            s, (const float2*)ws, total, sh.C, cpad, (int)subparts, (int)isplit, o);
         VPX_HIP_CHECK(hipGetLastError());
