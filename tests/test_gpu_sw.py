@@ -675,6 +675,11 @@ def _softmax(rt, dev, x_bits, axis, pad=0, packed=True, f32=False):
                                         ((65, 500), 1), ((7, 511), 1), ((130, 197), 1), ((3, 1023), 1), ((9, 4099), 1),
                                         ((3, 32768), 1), ((5, 20000), 1), ((6, 8191), 1), ((2, 33000), 1), ((2, 40001), 1),
                                         ((20000, 8), 1), ((17000, 509), 1),
+                                        # many short rows: runs of rows through LDS (any length), a ragged last run
+                                        ((70, 32), 1), ((3001, 64), 1), ((129, 128), 1), ((2, 50, 197), 2), ((100, 37), 1),
+                                        ((77, 3, 5), 2), ((333, 383), 1), ((64, 24), 1),
+                                        # rows past the registers of a workgroup: one 1024-lane workgroup per row, two passes
+                                        ((3, 40000), 1), ((2, 131072), 1), ((2, 33333), 1),
                                         # outer axis with contiguous inner dimensions: every slab shape (steps x columns x waves)
                                         ((3, 12, 64), 1), ((2, 50, 8, 24), 1), ((2, 200, 520), 1), ((3, 21, 36), 1),
                                         ((2, 100, 4, 5), 1), ((1, 400, 132), 1), ((2, 40, 6), 1), ((1, 200, 30), 1),
@@ -703,6 +708,14 @@ def test_softmax_padding_fp32_and_subviews(rt, orc, dev):
     assert_close_f16(got, orc.softmax_f16(orc.f32_to_f16(x[:, :512]), 1, pad=8), orc, "padSize 8, wave path")
     y32 = _softmax(rt, dev, x, 1, f32=True).cpu().numpy()
     np.testing.assert_allclose(y32, orc.softmax_f32(x, 1), rtol=REL_TOL, atol=1e-30)
+    # long rows: fp32, and fp16 with a padded tail
+    xl = rng.normal(0, 2, (3, 9000)).astype(np.float32)
+    np.testing.assert_allclose(_softmax(rt, dev, xl, 1, f32=True).cpu().numpy(), orc.softmax_f32(xl, 1), rtol=REL_TOL, atol=1e-30)
+    np.testing.assert_allclose(_softmax(rt, dev, xl[:, :8999], 1, f32=True).cpu().numpy(), orc.softmax_f32(xl[:, :8999], 1), rtol=REL_TOL, atol=1e-30)
+    xlb = orc.f32_to_f16(rng.normal(0, 2, (2, 50000)).astype(np.float32))
+    got = f16_bits(_softmax(rt, dev, xlb, 1, pad=5))
+    assert_close_f16(got, orc.softmax_f16(xlb, 1, pad=5), orc, "long rows, padSize 5")
+    assert np.all(got[:, -5:] == 0)
     # rows taken from a wider buffer: strides differ from the compact ones
     wide = to_dev(orc.f32_to_f16(rng.normal(0, 2, (8, 4, 768)).astype(np.float32)), dev, True)
     out = torch.zeros_like(wide)

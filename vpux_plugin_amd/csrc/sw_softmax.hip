@@ -441,6 +441,153 @@ __global__ __launch_bounds__(KW == 1 ? 256 : 64 * KW) void softmax_slab_f16(cons
     }
 }
 
+// Many short fp16 rows that follow one another in memory (rows of 32 ... 1024 values, any length: 197 as well as
+// 64): a workgroup takes a run of whole rows of about 4096 values, moves it between global memory and LDS in aligned
+// 128-bit words whatever the row length (values of neighbouring rows that share its first and last word are read
+// too, never written), and every half-wavefront handles one row at a time with the row's values in registers.
+constexpr int kShortRow = 1024;
+constexpr int kShortChunk = 4096;
+__device__ __forceinline__ float half_wave_max(float v) {
+    v = fmaxf(v, __shfl_xor(v, 1, 64));
+    v = fmaxf(v, __shfl_xor(v, 2, 64));
+    v = fmaxf(v, __shfl_xor(v, 4, 64));
+    v = fmaxf(v, __shfl_xor(v, 8, 64));
+    return fmaxf(v, __shfl_xor(v, 16, 64));
+}
+__device__ __forceinline__ float half_wave_sum(float v) {
+    v += __shfl_xor(v, 1, 64);
+    v += __shfl_xor(v, 2, 64);
+    v += __shfl_xor(v, 4, 64);
+    v += __shfl_xor(v, 8, 64);
+    return v + __shfl_xor(v, 16, 64);
+}
+template <int K>  // values per lane: a row has at most 32 K
+__global__ __launch_bounds__(256) void softmax_short_rows_f16(const half_t* __restrict__ in, half_t* __restrict__ out, int64_t rows,
+                                                              int len, int per_wg) {
+    __shared__ __attribute__((aligned(16))) half_t buf[kShortChunk + 16];
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const int64_t r0 = (int64_t)blockIdx.x * per_wg;
+    const int nr = rows - r0 < per_wg ? (int)(rows - r0) : per_wg;
+    const int64_t e0 = r0 * len, e1 = e0 + (int64_t)nr * len, total = rows * len;
+    const int64_t a0 = e0 & ~7ll;
+    const int words = (int)((e1 - a0 + 7) >> 3);
+    for (int w = threadIdx.x; w < words; w += 256) {
+        const int64_t at = a0 + (int64_t)w * 8;
+        if (at + 8 <= total) {
+            *reinterpret_cast<u32x4*>(buf + w * 8) = *reinterpret_cast<const u32x4*>(in + at);
+        } else {
+            for (int k = 0; k < 8; k++) buf[w * 8 + k] = at + k < total ? in[at + k] : (half_t)0.f;
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 31, team = threadIdx.x >> 5;
+    for (int r = team; r < nr; r += 8) {  // uniform per half-wavefront
+        half_t* x = buf + (int)(e0 - a0) + r * len;
+        float v[K];
+        float m = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int i = lane + 32 * k;
+            v[k] = i < len ? (float)x[i] : -INFINITY;
+            m = fmaxf(m, v[k]);
+        }
+        m = half_wave_max(m);
+        const float nmb = -m * kLog2e;
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            v[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(v[k], kLog2e, nmb));  // exp2(-inf) = 0 for the slots past the row
+            sum += v[k];
+        }
+        const float inv = 1.0f / half_wave_sum(sum);
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int i = lane + 32 * k;
+            if (i < len) x[i] = (half_t)(v[k] * inv);
+        }
+    }
+    __syncthreads();
+    for (int w = threadIdx.x; w < words; w += 256) {
+        const int64_t at = a0 + (int64_t)w * 8;
+        if (at >= e0 && at + 8 <= e1) {
+            __builtin_nontemporal_store(*reinterpret_cast<const u32x4*>(buf + w * 8), reinterpret_cast<u32x4*>(out + at));
+        } else {
+            for (int k = 0; k < 8; k++)
+                if (at + k >= e0 && at + k < e1) out[at + k] = buf[w * 8 + k];
+        }
+    }
+}
+
+// Rows longer than the registers of a workgroup hold (a vocabulary of 128 K entries): one workgroup of 1024 lanes per
+// row, a first pass that keeps a running maximum and a sum rescaled to it per lane (128-bit loads where the row is
+// aligned), and a second pass over the row -- by then in L2 -- that writes the quotients.
+template <typename T>
+__global__ __launch_bounds__(1024) void softmax_long_rows(const T* __restrict__ in, T* __restrict__ out, RowMap map, int64_t len,
+                                                          int64_t valid) {
+    __shared__ float red_m[16], red_s[16];
+    int64_t ioff, ooff;
+    row_offsets(map, blockIdx.x, ioff, ooff);
+    const T* px = in + ioff;
+    T* py = out + ooff;
+    constexpr int N = VecTraits<T>::N;
+    typedef uint32_t Vec __attribute__((ext_vector_type(4)));  // 16 bytes: eight fp16 or four fp32 values
+    const bool vec = valid % N == 0 && (reinterpret_cast<uintptr_t>(px) & 15) == 0 && (reinterpret_cast<uintptr_t>(py) & 15) == 0;
+    float m = -INFINITY, s = 0.f;
+    auto push = [&](float x) {
+        if (x > m) {
+            s *= fast_exp(m - x);  // exp(-inf) = 0 on the first value
+            m = x;
+        }
+        s += fast_exp(x - m);
+    };
+    if (vec) {
+        for (int64_t i = (int64_t)threadIdx.x * N; i < valid; i += 1024 * N) {
+            const Vec q = *reinterpret_cast<const Vec*>(px + i);
+            const T* e = reinterpret_cast<const T*>(&q);
+            float lm = (float)e[0];
+#pragma unroll
+            for (int k = 1; k < N; k++) lm = fmaxf(lm, (float)e[k]);
+            if (lm > m) {
+                s *= fast_exp(m - lm);
+                m = lm;
+            }
+#pragma unroll
+            for (int k = 0; k < N; k++) s += fast_exp((float)e[k] - m);
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < valid; i += 1024) push((float)px[i]);
+    }
+    // combine the lanes: maximum first, then the sums rescaled to it
+    float wm = m;
+    for (int o = 32; o > 0; o >>= 1) wm = fmaxf(wm, __shfl_xor(wm, o, 64));
+    float ws = m == -INFINITY ? 0.f : s * fast_exp(m - wm);
+    for (int o = 32; o > 0; o >>= 1) ws += __shfl_xor(ws, o, 64);
+    if ((threadIdx.x & 63) == 0) {
+        red_m[threadIdx.x >> 6] = wm;
+        red_s[threadIdx.x >> 6] = ws;
+    }
+    __syncthreads();
+    float M = red_m[0];
+    for (int w = 1; w < 16; w++) M = fmaxf(M, red_m[w]);
+    float S = 0.f;
+    for (int w = 0; w < 16; w++) S += red_m[w] == -INFINITY ? 0.f : red_s[w] * fast_exp(red_m[w] - M);
+    const float inv = 1.0f / S;
+    if (vec) {
+        for (int64_t i = (int64_t)threadIdx.x * N; i < valid; i += 1024 * N) {
+            const Vec q = *reinterpret_cast<const Vec*>(px + i);
+            const T* e = reinterpret_cast<const T*>(&q);
+            Vec y;
+            T* ye = reinterpret_cast<T*>(&y);
+#pragma unroll
+            for (int k = 0; k < N; k++) ye[k] = (T)(fast_exp((float)e[k] - M) * inv);
+            *reinterpret_cast<Vec*>(py + i) = y;
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < valid; i += 1024) py[i] = (T)(fast_exp((float)px[i] - M) * inv);
+    }
+    for (int64_t i = valid + threadIdx.x; i < len; i += 1024) py[i] = (T)0.f;  // padded tail, as the other kernels write it
+}
+
 template <typename T, int NV, int ROWS>
 void launch_rows_wave(const T* in, T* out, const RowMap& map, int64_t rows, int len, int valid, hipStream_t s) {
     const int64_t waves = (rows + ROWS - 1) / ROWS;
@@ -490,6 +637,22 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
             aligned = aligned && map.in_stride[d] % 8 == 0 && map.out_stride[d] % 8 == 0;
             same_mis = same_mis && (map.in_stride[d] - map.out_stride[d]) % 8 == 0;
         }
+        // short rows, one after another in memory: runs of rows through LDS, half a wavefront per row
+        const bool packed = map.nd == 0 || (map.nd == 1 && map.in_stride[0] == len && map.out_stride[0] == len);
+        if (packed && rows >= 64 && (len <= 128 || (len % 8 != 0 && len <= 384)) &&
+            ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+            const int per_wg = (int)(kShortChunk / len);
+            const dim3 grid((unsigned)((rows + per_wg - 1) / per_wg));
+#define VPX_SHORT(K) hipLaunchKernelGGL(softmax_short_rows_f16<K>, grid, dim3(256), 0, s, hin, hout, rows, (int)len, per_wg)
+            if (len <= 32) VPX_SHORT(1);
+            else if (len <= 64) VPX_SHORT(2);
+            else if (len <= 128) VPX_SHORT(4);
+            else if (len <= 256) VPX_SHORT(8);
+            else VPX_SHORT(12);
+#undef VPX_SHORT
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
         if (aligned || same_mis) {
             const int l = (int)len;
             const int span = aligned ? l : l + 7;  // aligned vectors a misaligned row can touch
@@ -531,6 +694,11 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
             VPX_HIP_CHECK(hipGetLastError());
             return VPX_RESULT_SUCCESS;
         }
+    }
+    if (ax == 0 && p.in_stride[0] == 1 && p.out_stride[0] == 1 && len >= 2048) {
+        hipLaunchKernelGGL(softmax_long_rows<T>, dim3((unsigned)rows), dim3(1024), 0, s, in, out, map, len, valid);
+        VPX_HIP_CHECK(hipGetLastError());
+        return VPX_RESULT_SUCCESS;
     }
     if (ax == 0) {
         hipLaunchKernelGGL(softmax_rows_block<T>, dim3((unsigned)rows), dim3(256), 0, s, in, out, map, len, valid,
