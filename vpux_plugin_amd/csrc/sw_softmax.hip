@@ -447,19 +447,20 @@ __global__ __launch_bounds__(KW == 1 ? 256 : 64 * KW) void softmax_slab_f16(cons
 // too, never written), and every half-wavefront handles one row at a time with the row's values in registers.
 constexpr int kShortRow = 1024;
 constexpr int kShortChunk = 4096;
+// All-reduce over the 32 lanes of half a wavefront: four DPP steps and one 16-lane swap, which all stay inside the half.
+template <class Op>
+__device__ __forceinline__ float half_wave_allreduce(float v, Op op) {
+    v = op(v, dpp<0xB1>(v));
+    v = op(v, dpp<0x4E>(v));
+    v = op(v, dpp<0x141>(v));
+    v = op(v, dpp<0x140>(v));
+    return op(v, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F)));
+}
 __device__ __forceinline__ float half_wave_max(float v) {
-    v = fmaxf(v, __shfl_xor(v, 1, 64));
-    v = fmaxf(v, __shfl_xor(v, 2, 64));
-    v = fmaxf(v, __shfl_xor(v, 4, 64));
-    v = fmaxf(v, __shfl_xor(v, 8, 64));
-    return fmaxf(v, __shfl_xor(v, 16, 64));
+    return half_wave_allreduce(v, [](float a, float b) { return fmaxf(a, b); });
 }
 __device__ __forceinline__ float half_wave_sum(float v) {
-    v += __shfl_xor(v, 1, 64);
-    v += __shfl_xor(v, 2, 64);
-    v += __shfl_xor(v, 4, 64);
-    v += __shfl_xor(v, 8, 64);
-    return v + __shfl_xor(v, 16, 64);
+    return half_wave_allreduce(v, [](float a, float b) { return a + b; });
 }
 template <int K>  // values per lane: a row has at most 32 K
 __global__ __launch_bounds__(256) void softmax_short_rows_f16(const half_t* __restrict__ in, half_t* __restrict__ out, int64_t rows,
