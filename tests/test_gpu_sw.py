@@ -683,7 +683,10 @@ def _softmax(rt, dev, x_bits, axis, pad=0, packed=True, f32=False):
                                         # outer axis with contiguous inner dimensions: every slab shape (steps x columns x waves)
                                         ((3, 12, 64), 1), ((2, 50, 8, 24), 1), ((2, 200, 520), 1), ((3, 21, 36), 1),
                                         ((2, 100, 4, 5), 1), ((1, 400, 132), 1), ((2, 40, 6), 1), ((1, 200, 30), 1),
-                                        ((1, 1000, 66), 1), ((1, 1024, 2, 64), 1), ((1, 1100, 64), 1), ((2, 2, 512, 512), 2)])
+                                        ((1, 1000, 66), 1), ((1, 1024, 2, 64), 1), ((1, 1100, 64), 1), ((2, 2, 512, 512), 2),
+                                        # outer axis past the slabs: wavefronts along the axis, lanes along the columns
+                                        ((4, 2048, 128), 1), ((2, 1500, 70), 1), ((3, 1200, 5, 13), 1), ((2, 4000, 520), 1),
+                                        ((5000, 64), 0), ((1, 1030, 1024), 1)])
 def test_softmax_shapes_and_axes(rt, orc, dev, shape, axis):
     rng = np.random.default_rng(hash((shape, axis)) % 2 ** 32)
     x = rng.normal(0, 3, shape).astype(np.float32)
@@ -712,6 +715,13 @@ def test_softmax_padding_fp32_and_subviews(rt, orc, dev):
     xl = rng.normal(0, 2, (3, 9000)).astype(np.float32)
     np.testing.assert_allclose(_softmax(rt, dev, xl, 1, f32=True).cpu().numpy(), orc.softmax_f32(xl, 1), rtol=REL_TOL, atol=1e-30)
     np.testing.assert_allclose(_softmax(rt, dev, xl[:, :8999], 1, f32=True).cpu().numpy(), orc.softmax_f32(xl[:, :8999], 1), rtol=REL_TOL, atol=1e-30)
+    xo = rng.normal(0, 2, (3, 70, 200)).astype(np.float32)   # fp32 over an outer axis, with and without a padded tail
+    np.testing.assert_allclose(_softmax(rt, dev, xo, 1, f32=True).cpu().numpy(), orc.softmax_f32(xo, 1), rtol=REL_TOL, atol=1e-30)
+    np.testing.assert_allclose(_softmax(rt, dev, xo, 1, pad=6, f32=True).cpu().numpy(), orc.softmax_f32(xo, 1, pad=6), rtol=REL_TOL, atol=1e-30)
+    xob = orc.f32_to_f16(rng.normal(0, 2, (2, 1300, 96)).astype(np.float32))
+    got = f16_bits(_softmax(rt, dev, xob, 1, pad=4))
+    assert_close_f16(got, orc.softmax_f16(xob, 1, pad=4), orc, "outer axis, padSize 4")
+    assert np.all(got[:, -4:, :] == 0)
     xlb = orc.f32_to_f16(rng.normal(0, 2, (2, 50000)).astype(np.float32))
     got = f16_bits(_softmax(rt, dev, xlb, 1, pad=5))
     assert_close_f16(got, orc.softmax_f16(xlb, 1, pad=5), orc, "long rows, padSize 5")

@@ -589,6 +589,94 @@ __global__ __launch_bounds__(1024) void softmax_long_rows(const T* __restrict__ 
     for (int64_t i = valid + threadIdx.x; i < len; i += 1024) py[i] = (T)0.f;  // padded tail, as the other kernels write it
 }
 
+// Softmax over an outer axis that is too long for the register slabs: a workgroup of 16 wavefronts takes VEC x 64
+// adjacent columns of the contiguous inner run, its wavefronts split the steps of the axis and keep, per column, a
+// running maximum and a sum rescaled to it; they meet in LDS, and a second pass over the same steps -- by then in
+// cache -- writes the quotients.  `om` maps the dimensions above the axis.
+template <typename T, int VEC>
+__global__ __launch_bounds__(1024) void softmax_cols(const T* __restrict__ in, T* __restrict__ out, RowMap om, int tiles_per_outer,
+                                                     int64_t len, int64_t valid, int64_t inner, int64_t in_as, int64_t out_as) {
+    constexpr int KW = 16;
+    __shared__ float sm[KW][64 * VEC], ss[KW][64 * VEC];
+    typedef T Vec __attribute__((ext_vector_type(VEC)));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t outer = blockIdx.x / tiles_per_outer;
+    const int64_t c0 = (int64_t)(blockIdx.x % tiles_per_outer) * (64 * VEC) + lane * VEC;
+    const bool live = c0 < inner;  // inner is a multiple of VEC
+    int64_t ioff = 0, ooff = 0;
+    if (om.nd > 0) row_offsets(om, outer, ioff, ooff);
+    const T* px = in + ioff + (live ? c0 : 0);
+    T* py = out + ooff + (live ? c0 : 0);
+    float m[VEC], s[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++) {
+        m[k] = -INFINITY;
+        s[k] = 0.f;
+    }
+    // eight steps at a time: their loads are in flight together, and the running sum is rescaled once per eight
+    constexpr int B = 8;
+    for (int64_t a0 = wave; a0 < valid; a0 += KW * B) {
+        Vec q[B];
+#pragma unroll
+        for (int j = 0; j < B; j++) {
+            const int64_t a = a0 + (int64_t)j * KW;
+            if (a < valid) q[j] = *reinterpret_cast<const Vec*>(px + a * in_as);
+        }
+#pragma unroll
+        for (int k = 0; k < VEC; k++) {
+            float nm = m[k];
+#pragma unroll
+            for (int j = 0; j < B; j++)
+                if (a0 + (int64_t)j * KW < valid) nm = fmaxf(nm, (float)q[j][k]);
+            if (nm > -INFINITY) {
+                float acc = s[k] * fast_exp(m[k] - nm);
+#pragma unroll
+                for (int j = 0; j < B; j++)
+                    if (a0 + (int64_t)j * KW < valid) acc += fast_exp((float)q[j][k] - nm);
+                s[k] = acc;
+            }
+            m[k] = nm;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; k++) {
+        sm[wave][lane * VEC + k] = m[k];
+        ss[wave][lane * VEC + k] = s[k];
+    }
+    __syncthreads();
+    float inv[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++) {
+        float M = sm[0][lane * VEC + k];
+        for (int w = 1; w < KW; w++) M = fmaxf(M, sm[w][lane * VEC + k]);
+        float S = 0.f;
+        for (int w = 0; w < KW; w++) {
+            const float mw = sm[w][lane * VEC + k];
+            S += mw == -INFINITY ? 0.f : ss[w][lane * VEC + k] * fast_exp(mw - M);
+        }
+        m[k] = M;
+        inv[k] = 1.0f / S;
+    }
+    if (!live) return;
+    for (int64_t a0 = wave; a0 < len; a0 += KW * B) {
+        Vec q[B];
+#pragma unroll
+        for (int j = 0; j < B; j++) {
+            const int64_t a = a0 + (int64_t)j * KW;
+            if (a < valid) q[j] = *reinterpret_cast<const Vec*>(px + a * in_as);
+        }
+#pragma unroll
+        for (int j = 0; j < B; j++) {
+            const int64_t a = a0 + (int64_t)j * KW;
+            if (a >= len) break;
+            Vec y;
+#pragma unroll
+            for (int k = 0; k < VEC; k++) y[k] = a < valid ? (T)(fast_exp((float)q[j][k] - m[k]) * inv[k]) : (T)0.f;
+            *reinterpret_cast<Vec*>(py + a * out_as) = y;
+        }
+    }
+}
+
 template <typename T, int NV, int ROWS>
 void launch_rows_wave(const T* in, T* out, const RowMap& map, int64_t rows, int len, int valid, hipStream_t s) {
     const int64_t waves = (rows + ROWS - 1) / ROWS;
@@ -759,6 +847,55 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
             else if (L <= 256) VPX_SLAB(2, 4, 64, tiles, 256);
             else VPX_SLAB(2, 16, 64, tiles, 1024);
 #undef VPX_SLAB
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
+    }
+    // outer axis, contiguous inner run of at least 64 columns: wavefronts along the axis, lanes along the columns
+    if (ax > 0 && p.in_stride[0] == 1 && p.out_stride[0] == 1 && len >= 32) {
+        int64_t inner = 1;
+        bool ok = true;
+        for (int d = 0; d < ax && ok; d++) {
+            ok = p.dims[d] == 1 || (p.in_stride[d] == inner && p.out_stride[d] == inner);
+            inner *= p.dims[d];
+        }
+        RowMap om{};
+        int64_t outer = 1;
+        for (int d = ax + 1; d < p.nd; d++) {
+            outer *= p.dims[d];
+            if (p.dims[d] == 1) continue;
+            om.dims[om.nd] = p.dims[d];
+            om.in_stride[om.nd] = p.in_stride[d];
+            om.out_stride[om.nd] = p.out_stride[d];
+            om.nd++;
+        }
+        const int64_t in_as = p.in_stride[ax], out_as = p.out_stride[ax];
+        auto aligned_to = [&](int vec) {
+            const size_t bytes = sizeof(T) * (size_t)vec;
+            bool a = inner % vec == 0 && in_as % vec == 0 && out_as % vec == 0 && (reinterpret_cast<uintptr_t>(in) % bytes) == 0 &&
+                     (reinterpret_cast<uintptr_t>(out) % bytes) == 0;
+            for (int d = 0; d < om.nd; d++) a = a && om.in_stride[d] % vec == 0 && om.out_stride[d] % vec == 0;
+            return a;
+        };
+        if (ok && inner >= 64) {
+            // the widest vector that still leaves a workgroup for every compute unit
+            int vec = 1;
+            for (int v = 16 / (int)sizeof(T); v > 1; v /= 2)
+                if (aligned_to(v) && outer * ((inner + 64 * v - 1) / (64 * v)) >= 256) {
+                    vec = v;
+                    break;
+                }
+            const int64_t tpo = (inner + 64 * vec - 1) / (64 * vec);
+            VPX_REQUIRE(outer * tpo < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "softmax: %lld tiles exceed the launch limit",
+                        (long long)(outer * tpo));
+            const dim3 grid((unsigned)(outer * tpo));
+#define VPX_COLS(V) hipLaunchKernelGGL((softmax_cols<T, V>), grid, dim3(1024), 0, s, in, out, om, (int)tpo, len, valid, inner, in_as, out_as)
+            if (vec == 8) {
+                if constexpr (sizeof(T) == 2) VPX_COLS(8);
+            } else if (vec == 4) VPX_COLS(4);
+            else if (vec == 2) VPX_COLS(2);
+            else VPX_COLS(1);
+#undef VPX_COLS
             VPX_HIP_CHECK(hipGetLastError());
             return VPX_RESULT_SUCCESS;
         }
