@@ -607,7 +607,8 @@ MVN6_CASES = [
     ((3, 2, 11008), (2,), (1, 1, 11008), None),           # rows of up to 16384 stay in the registers of a workgroup
     ((5, 16384), (1,), None, (1, 16384)),
     ((3, 12296), (1,), None, None),
-    ((2, 20000), (1,), None, None),                       # longer rows: chunked like mvn1 ...
+    ((130, 20000), (1,), None, None),                     # many longer rows: a row in LDS, one pass over memory
+    ((2, 20000), (1,), None, None),                       # few longer rows: chunked like mvn1 ...
     ((3, 2, 150, 200), (2, 3), None, None),
     ((2, 20001), (1,), None, (1, 20001)),                 # ... or one workgroup per row when there is a bias
     ((6, 1, 64), (1, 2), None, None),                     # unit dimension among the axes
@@ -779,7 +780,9 @@ def _mvn(rt, dev, xb, across, nv, eps, order="NCHW"):
 @pytest.mark.parametrize("shape", [(2, 3, 8, 8), (1, 16, 64, 64), (3, 7, 5, 9), (2, 64, 33, 31), (1, 2, 1, 4097),
                                    (1, 600, 64, 64),
                                    # many short groups: runs of whole groups per workgroup, odd lengths, a ragged last run
-                                   (4, 64, 7, 7), (3, 50, 14, 14), (2, 333, 1, 5), (1, 70, 31, 33), (67, 1, 1, 1), (5, 13, 1, 1024)])
+                                   (4, 64, 7, 7), (3, 50, 14, 14), (2, 333, 1, 5), (1, 70, 31, 33), (67, 1, 1, 1), (5, 13, 1, 1024),
+                                   # many groups of a few thousand to 76 800 values: the whole group in LDS, one pass over memory
+                                   (2, 70, 112, 112), (1, 130, 80, 96), (1, 128, 200, 384), (1, 128, 4104, 1)])
 @pytest.mark.parametrize("across", [True, False])
 @pytest.mark.parametrize("nv", [True, False])
 def test_mvn_nchw(rt, orc, dev, shape, across, nv):

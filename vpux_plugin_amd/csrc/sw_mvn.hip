@@ -312,6 +312,73 @@ __global__ __launch_bounds__(kThreads) void mvn_small_groups_kernel(const half_t
     }
 }
 
+// Groups of a few thousand to some 75 000 values (112 x 112 or 224 x 224 planes), many of them: one workgroup of
+// 1024 lanes keeps its whole group in LDS, so the tensor is read once and written once where the chunked form reads
+// it twice.  Sum on the way in, centred sum of squares and the scaled values from LDS.
+constexpr int kLdsGroupMax = 76800;  // values: 150 KiB of the 160 KiB a compute unit has
+__global__ __launch_bounds__(1024) void mvn_lds_group_kernel(const half_t* __restrict__ in, half_t* __restrict__ out, int64_t len,
+                                                             int normalize_variance, int eps_mode, float eps) {
+    extern __shared__ __attribute__((aligned(16))) u32x4 grp[];
+    __shared__ float red[16];
+    const half_t* px = in + (int64_t)blockIdx.x * len;
+    half_t* py = out + (int64_t)blockIdx.x * len;
+    const int nvec = (int)(len / 8), lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    auto block_sum = [&](float v) {
+        v = wave_sum(v);
+        __syncthreads();
+        if (lane == 0) red[wave] = v;
+        __syncthreads();
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < 16; w++) t += red[w];
+        return t;
+    };
+    float sum = 0.f;
+    for (int v = threadIdx.x; v < nvec; v += 1024) {
+        const u32x4 q = reinterpret_cast<const u32x4*>(px)[v];
+        grp[v] = q;
+        const half_t* h = reinterpret_cast<const half_t*>(&q);
+#pragma unroll
+        for (int k = 0; k < 8; k++) sum += (float)h[k];
+    }
+    const float n = (float)len;
+    const float mean = block_sum(sum) / n;
+    float sq = 0.f;
+    for (int v = threadIdx.x; v < nvec; v += 1024) {
+        const u32x4 q = grp[v];
+        const half_t* h = reinterpret_cast<const half_t*>(&q);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float d = (float)h[k] - mean;
+            sq += d * d;
+        }
+    }
+    const float var = block_sum(sq) / n;
+    const float inv = !normalize_variance ? 1.0f : (eps_mode == 0 ? 1.0f / __builtin_sqrtf(var + eps) : 1.0f / (__builtin_sqrtf(var) + eps));
+    for (int v = threadIdx.x; v < nvec; v += 1024) {
+        const u32x4 q = grp[v];
+        const half_t* h = reinterpret_cast<const half_t*>(&q);
+        u32x4 o;
+        half_t* ho = reinterpret_cast<half_t*>(&o);
+#pragma unroll
+        for (int k = 0; k < 8; k++) ho[k] = (half_t)(((float)h[k] - mean) * inv);
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(py) + v);
+    }
+}
+static bool lds_groups_ok(const half_t* in, const half_t* out, int64_t groups, int64_t len) {
+    return len > kChunk && len <= kLdsGroupMax && len % 8 == 0 && groups >= 128 && groups < (1ll << 31) &&
+           ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+}
+static int launch_lds_groups(const half_t* in, half_t* out, int64_t groups, int64_t len, int nv, int eps_mode, float eps, hipStream_t s) {
+    const size_t lds = (size_t)len * sizeof(half_t);
+    // more than 64 KiB of dynamic LDS is an opt-in per device and function; asking again costs little
+    VPX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(mvn_lds_group_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      kLdsGroupMax * (int)sizeof(half_t)));
+    hipLaunchKernelGGL(mvn_lds_group_kernel, dim3((unsigned)groups), dim3(1024), lds, s, in, out, len, nv, eps_mode, eps);
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
 // Whether the short-group form applies, and its launch.
 static bool small_groups_ok(const half_t* in, const half_t* out, int64_t groups, int64_t len) {
     return len >= 1 && len <= kSmallGroup && groups >= 64 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
@@ -1025,6 +1092,7 @@ int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool n
         return launch_channel_minor(pi, po, N, S, C, nv, eps, s);
     }
     if (small_groups_ok(pi, po, groups, group_size)) return launch_small_groups(pi, po, groups, group_size, nv, 0, eps, s);
+    if (lds_groups_ok(pi, po, groups, group_size)) return launch_lds_groups(pi, po, groups, group_size, nv, 0, eps, s);
     const bool aligned = group_size % 8 == 0 && (reinterpret_cast<uintptr_t>(pi) & 15) == 0 &&
                          (reinterpret_cast<uintptr_t>(po) & 15) == 0;
     return aligned ? launch_groups<true>(pi, po, groups, group_size, nv, eps, s)
@@ -1299,6 +1367,8 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
 
     // Long contiguous rows of a compact tensor, eps inside the root, no scale or bias: the chunked two-launch
     // scheme of mvn1 (a row is a group there).
+    if (innermost && row_len > kMvn6MaxRegRow && !scale && !bias && in.compact && out.compact && lds_groups_ok(pi, po, g.rows, row_len))
+        return launch_lds_groups(pi, po, g.rows, row_len, nv, eps_mode, eps, s);
     if (innermost && row_len > kMvn6MaxRegRow && !scale && !bias && eps_mode == 0 && in.compact && out.compact) {
         const bool aligned = row_len % 8 == 0 && ((reinterpret_cast<uintptr_t>(pi) | reinterpret_cast<uintptr_t>(po)) & 15) == 0;
         return aligned ? launch_groups<true>(pi, po, g.rows, row_len, nv, eps, s) : launch_groups<false>(pi, po, g.rows, row_len, nv, eps, s);
