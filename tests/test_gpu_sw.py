@@ -681,6 +681,8 @@ def _softmax(rt, dev, x_bits, axis, pad=0, packed=True, f32=False):
                                         ((77, 3, 5), 2), ((333, 383), 1), ((64, 24), 1),
                                         # rows past the registers of a workgroup: one 1024-lane workgroup per row, two passes
                                         ((3, 40000), 1), ((2, 131072), 1), ((2, 33333), 1),
+                                        # 64 or more aligned rows of up to 76 800 values: the row in LDS, one pass over memory
+                                        ((70, 50264), 1), ((64, 76800), 1), ((66, 33000), 1),
                                         # outer axis with contiguous inner dimensions: every slab shape (steps x columns x waves)
                                         ((3, 12, 64), 1), ((2, 50, 8, 24), 1), ((2, 200, 520), 1), ((3, 21, 36), 1),
                                         ((2, 100, 4, 5), 1), ((1, 400, 132), 1), ((2, 40, 6), 1), ((1, 200, 30), 1),

@@ -519,6 +519,60 @@ __global__ __launch_bounds__(256) void softmax_short_rows_f16(const half_t* __re
     }
 }
 
+// fp16 rows of up to 76 800 values (a 50 257- or 65 536-entry vocabulary), aligned: the row stays in the LDS of one
+// 1024-lane workgroup, so memory is read once: maximum on the way in, the sum of exponentials and the quotients
+// from LDS.
+constexpr int kLdsRowMax = 76800;
+__global__ __launch_bounds__(1024) void softmax_lds_rows_f16(const half_t* __restrict__ in, half_t* __restrict__ out, RowMap map, int len) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) u32x4 row[];
+    __shared__ float red[16];
+    int64_t ioff, ooff;
+    row_offsets(map, blockIdx.x, ioff, ooff);
+    const u32x4* px = reinterpret_cast<const u32x4*>(in + ioff);
+    u32x4* py = reinterpret_cast<u32x4*>(out + ooff);
+    const int nvec = len / 8, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float m = -INFINITY;
+    for (int v = threadIdx.x; v < nvec; v += 1024) {
+        const u32x4 q = px[v];
+        row[v] = q;
+        const half_t* h = reinterpret_cast<const half_t*>(&q);
+#pragma unroll
+        for (int k = 0; k < 8; k++) m = fmaxf(m, (float)h[k]);
+    }
+    m = wave_allreduce(m, [](float a, float b) { return fmaxf(a, b); });
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = red[0];
+#pragma unroll
+    for (int w = 1; w < 16; w++) m = fmaxf(m, red[w]);
+    const float nmb = -m * kLog2e;
+    float s = 0.f;
+    for (int v = threadIdx.x; v < nvec; v += 1024) {
+        const u32x4 q = row[v];
+        const half_t* h = reinterpret_cast<const half_t*>(&q);
+#pragma unroll
+        for (int k = 0; k < 8; k++) s += __builtin_amdgcn_exp2f(__builtin_fmaf((float)h[k], kLog2e, nmb));
+    }
+    s = wave_allreduce(s, [](float a, float b) { return a + b; });
+    __syncthreads();
+    if (lane == 0) red[wave] = s;
+    __syncthreads();
+    s = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; w++) s += red[w];
+    const float inv = 1.0f / s;
+    for (int v = threadIdx.x; v < nvec; v += 1024) {
+        const u32x4 q = row[v];
+        const half_t* h = reinterpret_cast<const half_t*>(&q);
+        u32x4 o;
+        half_t* ho = reinterpret_cast<half_t*>(&o);
+#pragma unroll
+        for (int k = 0; k < 8; k++) ho[k] = (half_t)(__builtin_amdgcn_exp2f(__builtin_fmaf((float)h[k], kLog2e, nmb)) * inv);
+        __builtin_nontemporal_store(o, py + v);
+    }
+}
+
 // Rows longer than the registers of a workgroup hold (a vocabulary of 128 K entries): one workgroup of 1024 lanes per
 // row, a first pass that keeps a running maximum and a sum rescaled to it per lane (128-bit loads where the row is
 // aligned), and a second pass over the row -- by then in L2 -- that writes the quotients.
@@ -780,6 +834,19 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
             else if (len <= 2 * per) launch_rows_wave<T, 2, 1>(in, out, map, rows, l, v, s);
             else if (len <= 4 * per) launch_rows_wave<T, 4, 1>(in, out, map, rows, l, v, s);
             else launch_rows_wave<T, 8, 1>(in, out, map, rows, l, v, s);
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
+    }
+    if (inner && std::is_same<T, half_t>::value && valid == len && len % 8 == 0 && len <= kLdsRowMax && rows >= 64 &&
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+        bool al = true;
+        for (int d = 0; d < map.nd; d++) al = al && (map.dims[d] == 1 || (map.in_stride[d] % 8 == 0 && map.out_stride[d] % 8 == 0));
+        if (al) {
+            VPX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(softmax_lds_rows_f16), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                              kLdsRowMax * 2));
+            hipLaunchKernelGGL(softmax_lds_rows_f16, dim3((unsigned)rows), dim3(1024), (size_t)len * 2, s, reinterpret_cast<const half_t*>(in),
+                               reinterpret_cast<half_t*>(out), map, (int)len);
             VPX_HIP_CHECK(hipGetLastError());
             return VPX_RESULT_SUCCESS;
         }
