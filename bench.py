@@ -25,10 +25,10 @@ METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
 # Bytes moved through L2 per step, from rocprofv3 FETCH_SIZE / WRITE_SIZE counters scaled by a plain
 # copy of known size (profiles/<workload>__*.md hold the runs these come from).
 MEASURED_TRAFFIC = {
-    "c1_fake_quantize": 885035, "c2_softmax": 134300997, "c3_mvn": 25428500, "c4_conv": 16275405,
-    "c5_matmul": 384934428, "c5_dequantize": 135348685, "c5_eltwise_add": 270539857, "c5_nce_eltwise": 135252959,
-    "calib_int_mm": 531680254, "x_mvn6_layernorm": 268486231, "x_activation_hswish": 180515042,
-    "x_mvn1_three_steps": 25333958,
+    "c1_fake_quantize": 880079, "c2_softmax": 134293332, "c3_mvn": 25440485, "c4_conv": 16276094,
+    "c5_matmul": 385007798, "c5_dequantize": 135326848, "c5_eltwise_add": 270538895, "c5_nce_eltwise": 135268239,
+    "calib_int_mm": 531804959, "x_mvn6_layernorm": 268494127, "x_activation_hswish": 180532564,
+    "x_mvn1_three_steps": 25333054,
 }
 
 
