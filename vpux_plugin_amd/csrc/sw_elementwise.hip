@@ -112,8 +112,16 @@ struct FqConst {
     float r_lm1;             // RN(1 / lm1)
     float orange;            // ohi - olo
 };
+// round half away from zero for t >= 0: nearest-even, then a tie that went down to the even neighbour goes up
+// (two instructions fewer than the general roundf; negative arguments only occur where the caller discards the result)
+__device__ __forceinline__ float round_half_up_nonneg(float t) {
+    const float r = __builtin_rintf(t);
+    return t - r == 0.5f ? r + 1.0f : r;
+}
 __device__ __forceinline__ float fq_f32_const(float x, const FqConst& c) {
-    const float q = div_const(roundf(div_const(x - c.ilo, c.irange, c.r_irange) * c.lm1), c.lm1, c.r_lm1) * c.orange + c.olo;
+    // the level is only used for ilo < x <= ihi, where it is not negative
+    const float level = round_half_up_nonneg(div_const(x - c.ilo, c.irange, c.r_irange) * c.lm1);
+    const float q = div_const(level, c.lm1, c.r_lm1) * c.orange + c.olo;
     return x <= c.ilo ? c.olo : (x > c.ihi ? c.ohi : q);
 }
 
