@@ -678,7 +678,7 @@ def _softmax(rt, dev, x_bits, axis, pad=0, packed=True, f32=False):
                                         ((20000, 8), 1), ((17000, 509), 1),
                                         # many short rows: runs of rows through LDS (any length), a ragged last run
                                         ((70, 32), 1), ((3001, 64), 1), ((129, 128), 1), ((2, 50, 197), 2), ((100, 37), 1),
-                                        ((77, 3, 5), 2), ((333, 383), 1), ((64, 24), 1),
+                                        ((77, 3, 5), 2), ((333, 383), 1), ((64, 24), 1), ((50, 16), 1), ((3, 7, 128), 2), ((77, 256), 1),
                                         # rows past the registers of a workgroup: one 1024-lane workgroup per row, two passes
                                         ((3, 40000), 1), ((2, 131072), 1), ((2, 33333), 1),
                                         # 64 or more aligned rows of up to 76 800 values: the row in LDS, one pass over memory

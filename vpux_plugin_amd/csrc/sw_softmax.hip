@@ -443,6 +443,48 @@ __global__ __launch_bounds__(KW == 1 ? 256 : 64 * KW) void softmax_slab_f16(cons
     }
 }
 
+// Packed, aligned fp16 rows of 8, 16, 32, 64, 128 or 256 values: T = len / 8 adjacent lanes hold a row, one 128-bit
+// word each, so a wavefront's accesses are one contiguous run, and the row's maximum and sum cross the T lanes by DPP
+// (and one 16-lane swap for the longest).
+template <int T>
+__global__ __launch_bounds__(256) void softmax_tiny_rows_f16(const half_t* __restrict__ in, half_t* __restrict__ out, int64_t n_vec) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (v >= n_vec) return;  // n_vec is a multiple of T and so is 256: a row's lanes leave together
+    const u32x4 q = reinterpret_cast<const u32x4*>(in)[v];
+    const half_t* h = reinterpret_cast<const half_t*>(&q);
+    float x[8];
+    float m = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        x[k] = (float)h[k];
+        m = fmaxf(m, x[k]);
+    }
+    auto across = [](float a, auto op) {
+        if (T >= 2) a = op(a, dpp<0xB1>(a));
+        if (T >= 4) a = op(a, dpp<0x4E>(a));
+        if (T >= 8) a = op(a, dpp<0x141>(a));
+        if (T >= 16) a = op(a, dpp<0x140>(a));
+        if (T >= 32) a = op(a, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, a), 0x401F)));  // lane ^ 16
+        return a;
+    };
+    m = across(m, [](float a, float b) { return fmaxf(a, b); });
+    const float nmb = -m * kLog2e;
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        x[k] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[k], kLog2e, nmb));
+        s += x[k];
+    }
+    s = across(s, [](float a, float b) { return a + b; });
+    const float inv = 1.0f / s;
+    u32x4 o;
+    half_t* ho = reinterpret_cast<half_t*>(&o);
+#pragma unroll
+    for (int k = 0; k < 8; k++) ho[k] = (half_t)(x[k] * inv);
+    __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out) + v);
+}
+
 // Many short fp16 rows that follow one another in memory (rows of 32 ... 1024 values, any length: 197 as well as
 // 64): a workgroup takes a run of whole rows of about 4096 values, moves it between global memory and LDS in aligned
 // 128-bit words whatever the row length (values of neighbouring rows that share its first and last word are read
@@ -784,8 +826,22 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
         }
         // short rows, one after another in memory: runs of rows through LDS, half a wavefront per row
         const bool packed = map.nd == 0 || (map.nd == 1 && map.in_stride[0] == len && map.out_stride[0] == len);
-        if (packed && rows >= 64 && (len <= 128 || (len % 8 != 0 && len <= 384)) &&
-            ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+        const bool base16 = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+        if (packed && base16 && (len == 8 || len == 16 || len == 32 || len == 64 || len == 128 || len == 256) && rows * (len / 8) < (1ll << 39)) {
+            const int64_t n_vec = rows * (len / 8);
+            const dim3 grid((unsigned)((n_vec + 255) / 256));
+#define VPX_TINY(T) hipLaunchKernelGGL(softmax_tiny_rows_f16<T>, grid, dim3(256), 0, s, hin, hout, n_vec)
+            if (len == 8) VPX_TINY(1);
+            else if (len == 16) VPX_TINY(2);
+            else if (len == 32) VPX_TINY(4);
+            else if (len == 64) VPX_TINY(8);
+            else if (len == 128) VPX_TINY(16);
+            else VPX_TINY(32);
+#undef VPX_TINY
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
+        if (packed && rows >= 64 && (len <= 128 || (len % 8 != 0 && len <= 384)) && base16) {
             const int per_wg = (int)(kShortChunk / len);
             const dim3 grid((unsigned)((rows + per_wg - 1) / per_wg));
 #define VPX_SHORT(K) hipLaunchKernelGGL(softmax_short_rows_f16<K>, grid, dim3(256), 0, s, hin, hout, rows, (int)len, per_wg)
