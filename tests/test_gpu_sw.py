@@ -612,6 +612,11 @@ MVN6_CASES = [
     ((3, 2, 150, 200), (2, 3), None, None),
     ((2, 20001), (1,), None, (1, 20001)),                 # ... or one workgroup per row when there is a bias
     ((6, 1, 64), (1, 2), None, None),                     # unit dimension among the axes
+    ((1000, 8), (1,), None, None),                        # packed power-of-two rows: len / 8 lanes per row
+    ((77, 5, 32), (2,), None, None),
+    ((130, 64), (1,), None, None),
+    ((9, 128), (1,), None, None),
+    ((33, 16, 16), (1, 2), None, None),
     ((300, 50), (1,), None, None),                        # many short rows, not a multiple of 8: runs of rows per workgroup
     ((64, 3, 7, 7), (2, 3), None, None),
     ((70, 1001), (-1,), None, None),
@@ -783,6 +788,7 @@ def _mvn(rt, dev, xb, across, nv, eps, order="NCHW"):
                                    (1, 600, 64, 64),
                                    # many short groups: runs of whole groups per workgroup, odd lengths, a ragged last run
                                    (4, 64, 7, 7), (3, 50, 14, 14), (2, 333, 1, 5), (1, 70, 31, 33), (67, 1, 1, 1), (5, 13, 1, 1024),
+                                   (3, 40, 8, 8), (2, 9, 16, 16), (5, 7, 4, 4), (1, 3, 2, 4),   # planes of 8 ... 256 values
                                    # many groups of a few thousand to 76 800 values: the whole group in LDS, one pass over memory
                                    (2, 70, 112, 112), (1, 130, 80, 96), (1, 128, 200, 384), (1, 128, 4104, 1)])
 @pytest.mark.parametrize("across", [True, False])

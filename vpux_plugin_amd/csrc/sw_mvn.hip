@@ -379,6 +379,65 @@ static int launch_lds_groups(const half_t* in, half_t* out, int64_t groups, int6
     return VPX_RESULT_SUCCESS;
 }
 
+// Packed, aligned groups of 8, 16, ... 256 values (a power of two): T = len / 8 adjacent lanes hold a group, one
+// 128-bit word each, and its sums cross the T lanes by DPP (one 16-lane swap for T = 32).
+template <int T>
+__global__ __launch_bounds__(kThreads) void mvn_tiny_groups_kernel(const half_t* __restrict__ in, half_t* __restrict__ out, int64_t n_vec,
+                                                                   int normalize_variance, int eps_mode, float eps) {
+    const int64_t v = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (v >= n_vec) return;  // n_vec is a multiple of T and so is the workgroup: a group's lanes leave together
+    const u32x4 q = reinterpret_cast<const u32x4*>(in)[v];
+    const half_t* h = reinterpret_cast<const half_t*>(&q);
+    auto across = [](float a) {
+        if (T >= 2) a += dppf<0xB1>(a);
+        if (T >= 4) a += dppf<0x4E>(a);
+        if (T >= 8) a += dppf<0x141>(a);
+        if (T >= 16) a += dppf<0x140>(a);
+        if (T >= 32) a += swz16(a);
+        return a;
+    };
+    float x[8];
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        x[k] = (float)h[k];
+        sum += x[k];
+    }
+    constexpr float n = (float)(8 * T);
+    const float mean = across(sum) / n;
+    float sq = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        x[k] -= mean;
+        sq += x[k] * x[k];
+    }
+    const float var = across(sq) / n;
+    const float inv = !normalize_variance ? 1.0f : (eps_mode == 0 ? 1.0f / __builtin_sqrtf(var + eps) : 1.0f / (__builtin_sqrtf(var) + eps));
+    u32x4 o;
+    half_t* ho = reinterpret_cast<half_t*>(&o);
+#pragma unroll
+    for (int k = 0; k < 8; k++) ho[k] = (half_t)(x[k] * inv);
+    __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out) + v);
+}
+static bool tiny_groups_ok(const half_t* in, const half_t* out, int64_t groups, int64_t len) {
+    return (len == 8 || len == 16 || len == 32 || len == 64 || len == 128 || len == 256) && groups * (len / 8) < (1ll << 39) &&
+           ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+}
+static int launch_tiny_groups(const half_t* in, half_t* out, int64_t groups, int64_t len, int nv, int eps_mode, float eps, hipStream_t s) {
+    const int64_t n_vec = groups * (len / 8);
+    const dim3 grid((unsigned)((n_vec + kThreads - 1) / kThreads));
+#define VPX_TINY(T) hipLaunchKernelGGL(mvn_tiny_groups_kernel<T>, grid, dim3(kThreads), 0, s, in, out, n_vec, nv, eps_mode, eps)
+    if (len == 8) VPX_TINY(1);
+    else if (len == 16) VPX_TINY(2);
+    else if (len == 32) VPX_TINY(4);
+    else if (len == 64) VPX_TINY(8);
+    else if (len == 128) VPX_TINY(16);
+    else VPX_TINY(32);
+#undef VPX_TINY
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
+
 // Whether the short-group form applies, and its launch.
 static bool small_groups_ok(const half_t* in, const half_t* out, int64_t groups, int64_t len) {
     return len >= 1 && len <= kSmallGroup && groups >= 64 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
@@ -1091,6 +1150,7 @@ int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool n
     } else {  // channel-minor layout, per-channel statistics
         return launch_channel_minor(pi, po, N, S, C, nv, eps, s);
     }
+    if (tiny_groups_ok(pi, po, groups, group_size)) return launch_tiny_groups(pi, po, groups, group_size, nv, 0, eps, s);
     if (small_groups_ok(pi, po, groups, group_size)) return launch_small_groups(pi, po, groups, group_size, nv, 0, eps, s);
     if (lds_groups_ok(pi, po, groups, group_size)) return launch_lds_groups(pi, po, groups, group_size, nv, 0, eps, s);
     const bool aligned = group_size % 8 == 0 && (reinterpret_cast<uintptr_t>(pi) & 15) == 0 &&
@@ -1375,6 +1435,8 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
     }
     // Short contiguous rows whose length is not a multiple of eight (7 x 7 planes, rows of 100): runs of whole rows
     // per workgroup, as for mvn1's short groups.
+    if (innermost && !scale && !bias && in.compact && out.compact && tiny_groups_ok(pi, po, g.rows, row_len))
+        return launch_tiny_groups(pi, po, g.rows, row_len, nv, eps_mode, eps, s);
     if (innermost && row_len % 8 != 0 && !scale && !bias && in.compact && out.compact && small_groups_ok(pi, po, g.rows, row_len))
         return launch_small_groups(pi, po, g.rows, row_len, nv, eps_mode, eps, s);
     bool fast = innermost && row_len % 8 == 0 && row_len <= kMvn6MaxRegRow;
