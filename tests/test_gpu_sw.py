@@ -594,6 +594,14 @@ def _assert_mvn6_close(got_bits, want_bits, orc, what):
 MVN6_CASES = [
     # shape, axes, scale shape, bias shape
     ((8, 128, 768), (2,), (1, 1, 768), (1, 1, 768)),      # LayerNorm, one wavefront per row
+    # LayerNorm over many rows: a team walks 2 or 4 rows with scale / bias in registers; the last workgroup is ragged
+    ((70001, 256), (1,), (1, 256), (1, 256)),
+    ((131075, 64), (1,), (1, 64), None),
+    ((33, 1001, 512), (2,), None, (1, 1, 512)),
+    ((65539, 768), (1,), (1, 768), (1, 768)),
+    ((32771, 768), (1,), (1, 768), (1, 768)),
+    ((3, 11000, 1024), (2,), (1, 1, 1024), (1, 1, 1024)),
+    ((40000, 256), (1,), (40000, 256), (1, 256)),         # a scale of full shape is read per row
     ((4, 77, 512), (-1,), None, None),
     ((4, 16, 2048), (2,), (1, 1, 2048), None),            # one workgroup per row
     ((2, 8, 8192), (2,), None, (1, 1, 8192)),

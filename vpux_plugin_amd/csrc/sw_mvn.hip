@@ -854,9 +854,11 @@ struct RowBase {
 
 __device__ __forceinline__ RowBase row_base(const Mvn6Geom& g, int64_t row) {
     RowBase b{0, 0, 0, 0};
+    uint32_t r = (uint32_t)row;  // the host keeps the row count below 2^31
     for (int d = 0; d < g.nk; d++) {
-        const int64_t c = row % g.kdim[d];
-        row /= g.kdim[d];
+        const bool last = d == g.nk - 1;  // what is left indexes the outermost kept dimension: no division
+        const int64_t c = last ? r : r % (uint32_t)g.kdim[d];
+        if (!last) r /= (uint32_t)g.kdim[d];
         b.in += c * g.k_in[d];
         b.out += c * g.k_out[d];
         b.sc += c * g.k_sc[d];
@@ -891,13 +893,28 @@ __device__ __forceinline__ float team_sum(float v, float* smem) {
 // Rows that are contiguous in memory and a multiple of 8 long: the row lives in the registers of half a
 // wavefront (TEAM = 32, eight rows per workgroup), of a wavefront (64) or of the workgroup (256).
 constexpr int kMvn6MaxRegRow = 16384;  // longest row a workgroup keeps in registers (64 values per lane)
-template <int TEAM, int VPT>
+template <int TEAM, int VPT, int RPT = 1>  // RPT: consecutive rows a team walks, keeping a scale / bias that runs along the row in registers
 __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
                                                              const half_t* __restrict__ sc, const half_t* __restrict__ bi,
                                                              Mvn6Geom g, int normalize_variance, int eps_mode, float eps) {
     __shared__ float red[4];
     const int t = (int)(threadIdx.x % TEAM);
-    int64_t row = (int64_t)blockIdx.x * (kThreads / TEAM) + threadIdx.x / TEAM;
+    const int64_t row0 = ((int64_t)blockIdx.x * (kThreads / TEAM) + threadIdx.x / TEAM) * RPT;
+    // scale and bias that run along the row (and do not depend on it): loaded once for the RPT rows
+    u32x4 scv[VPT], biv[VPT];
+    if (RPT > 1) {
+#pragma unroll
+        for (int j = 0; j < VPT; j++) {
+            const uint32_t e0 = (uint32_t)(j * TEAM + t) * 8;
+            if (e0 < g.row_len) {
+                if (sc) scv[j] = *reinterpret_cast<const u32x4*>(sc + e0);
+                if (bi) biv[j] = *reinterpret_cast<const u32x4*>(bi + e0);
+            }
+        }
+    }
+#pragma unroll 1
+    for (int rr = 0; rr < RPT; rr++) {
+    int64_t row = row0 + rr;
     const bool live = row < g.rows;  // uniform per team; dead teams skip memory only
     if (!live) row = 0;
     const RowBase b = row_base(g, row);
@@ -944,7 +961,7 @@ __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __res
         for (int k = 0; k < 8; k++) y[k] = (x[j][k] - mean) * inv;
         if (sc) {
             if (g.sc_along_row) {
-                const u32x4 v = *reinterpret_cast<const u32x4*>(sc + b.sc + e0);
+                const u32x4 v = RPT > 1 ? scv[j] : *reinterpret_cast<const u32x4*>(sc + b.sc + e0);
                 const half_t* p = reinterpret_cast<const half_t*>(&v);
 #pragma unroll
                 for (int k = 0; k < 8; k++) y[k] *= (float)p[k];
@@ -955,7 +972,7 @@ __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __res
         }
         if (bi) {
             if (g.bi_along_row) {
-                const u32x4 v = *reinterpret_cast<const u32x4*>(bi + b.bi + e0);
+                const u32x4 v = RPT > 1 ? biv[j] : *reinterpret_cast<const u32x4*>(bi + b.bi + e0);
                 const half_t* p = reinterpret_cast<const half_t*>(&v);
 #pragma unroll
                 for (int k = 0; k < 8; k++) y[k] += (float)p[k];
@@ -969,6 +986,7 @@ __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __res
 #pragma unroll
         for (int k = 0; k < 8; k++) po[k] = (half_t)y[k];
         __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(out + b.out + e0));
+    }
     }
 }
 
@@ -1416,6 +1434,25 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
             g.rows *= in.dims[d];
         }
     }
+    // Kept dimensions that every operand walks as one (stride of the outer = stride x extent of the inner) fold
+    // into one, so a packed tensor's rows are found without a division.
+    for (int d = 0; d + 1 < g.nk;) {
+        const int64_t e = g.kdim[d];
+        if (g.k_in[d + 1] == g.k_in[d] * e && g.k_out[d + 1] == g.k_out[d] * e && g.k_sc[d + 1] == g.k_sc[d] * e &&
+            g.k_bi[d + 1] == g.k_bi[d] * e && e * g.kdim[d + 1] < (1ll << 31)) {
+            g.kdim[d] = (int32_t)(e * g.kdim[d + 1]);
+            for (int k = d + 1; k + 1 < g.nk; k++) {
+                g.kdim[k] = g.kdim[k + 1];
+                g.k_in[k] = g.k_in[k + 1];
+                g.k_out[k] = g.k_out[k + 1];
+                g.k_sc[k] = g.k_sc[k + 1];
+                g.k_bi[k] = g.k_bi[k + 1];
+            }
+            g.nk--;
+        } else {
+            d++;
+        }
+    }
     VPX_REQUIRE(row_len < (1ll << 31) && g.rows < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
                 "mvn6: %lld rows of %lld elements exceed the launch limit", (long long)g.rows, (long long)row_len);
     g.row_len = (uint32_t)row_len;
@@ -1452,15 +1489,36 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
 #define VPX_MVN6_ROWS(TEAM, VPT) \
     hipLaunchKernelGGL((mvn6_rows_kernel<TEAM, VPT>), dim3((unsigned)((g.rows + kThreads / TEAM - 1) / (kThreads / TEAM))), \
                        dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps)
-        if (row_len <= 256) VPX_MVN6_ROWS(32, 1);
-        else if (row_len <= 512) VPX_MVN6_ROWS(64, 1);
-        else if (row_len <= 1024) VPX_MVN6_ROWS(64, 2);
+        // A scale / bias shared by all rows stays in registers while a team walks 2 or 4 consecutive rows, as long
+        // as that leaves 4096 workgroups (two rounds of the chip) or more.
+        bool shared_rows = (scale && g.sc_along_row) || (bias && g.bi_along_row);
+        for (int d = 0; d < g.nk; d++)
+            if ((scale && g.sc_along_row && g.k_sc[d] != 0) || (bias && g.bi_along_row && g.k_bi[d] != 0)) shared_rows = false;
+        const bool half768 = shared_rows && row_len == 768;  // 32 lanes x 3 words, none idle: pays with scale / bias
+        const int team = row_len <= 256 || half768 ? 32 : 64;
+        const int64_t team_rows = g.rows / (kThreads / team);
+        const int rpt = !shared_rows ? 1 : team_rows >= 4 * 4096 ? 4 : team_rows >= 2 * 4096 ? 2 : 1;
+#define VPX_MVN6_ROWS_R(TEAM, VPT, RPT) \
+    hipLaunchKernelGGL((mvn6_rows_kernel<TEAM, VPT, RPT>), dim3((unsigned)((g.rows + RPT * kThreads / TEAM - 1) / (RPT * kThreads / TEAM))), \
+                       dim3(kThreads), 0, s, pi, po, ps, pb, g, nv, eps_mode, eps)
+#define VPX_MVN6_SHORT(TEAM, VPT)                   \
+    do {                                            \
+        if (rpt == 4) VPX_MVN6_ROWS_R(TEAM, VPT, 4); \
+        else if (rpt == 2) VPX_MVN6_ROWS_R(TEAM, VPT, 2); \
+        else VPX_MVN6_ROWS(TEAM, VPT);              \
+    } while (0)
+        if (row_len <= 256) VPX_MVN6_SHORT(32, 1);
+        else if (row_len <= 512) VPX_MVN6_SHORT(64, 1);
+        else if (half768) VPX_MVN6_SHORT(32, 3);
+        else if (row_len <= 1024) VPX_MVN6_SHORT(64, 2);
         else if (row_len <= 2048) VPX_MVN6_ROWS(256, 1);
         else if (row_len <= 4096) VPX_MVN6_ROWS(256, 2);  // one wavefront per 4096-element row measured 9 % slower
         else if (row_len <= 8192) VPX_MVN6_ROWS(256, 4);
         else if (row_len <= 12288) VPX_MVN6_ROWS(256, 6);
         else VPX_MVN6_ROWS(256, 8);
 #undef VPX_MVN6_ROWS
+#undef VPX_MVN6_ROWS_R
+#undef VPX_MVN6_SHORT
     } else if (inner_kept && g.k_in[0] == 1 && g.k_out[0] == 1) {
         const int64_t outer = g.rows / g.kdim[0];
         const auto blocks = [&](int p) { return outer * ((g.kdim[0] + p - 1) / p); };
