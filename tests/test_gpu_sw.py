@@ -602,6 +602,15 @@ MVN6_CASES = [
     ((32771, 768), (1,), (1, 768), (1, 768)),
     ((3, 11000, 1024), (2,), (1, 1, 1024), (1, 1, 1024)),
     ((40000, 256), (1,), (40000, 256), (1, 256)),         # a scale of full shape is read per row
+    # one wavefront per row of up to 3072 values, 3 ... 6 words per lane
+    ((301, 1280), (1,), (1, 1280), (1, 1280)),
+    ((3, 35, 1536), (2,), (1, 1, 1536), None),
+    ((99, 2560), (1,), None, (1, 2560)),
+    ((77, 3072), (1,), (1, 3072), (1, 3072)),
+    ((45, 1032), (1,), None, None),
+    ((21, 5120), (1,), (1, 5120), (1, 5120)),
+    ((9, 10240), (1,), None, (1, 10240)),
+    ((7, 13824), (1,), (1, 13824), None),
     ((4, 77, 512), (-1,), None, None),
     ((4, 16, 2048), (2,), (1, 1, 2048), None),            # one workgroup per row
     ((2, 8, 8192), (2,), None, (1, 1, 8192)),

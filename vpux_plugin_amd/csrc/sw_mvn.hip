@@ -1511,10 +1511,17 @@ int launch_mvn6(const MemRef& in, const MemRef* scale, const MemRef* bias, const
         else if (row_len <= 512) VPX_MVN6_SHORT(64, 1);
         else if (half768) VPX_MVN6_SHORT(32, 3);
         else if (row_len <= 1024) VPX_MVN6_SHORT(64, 2);
+        else if (row_len <= 1536) VPX_MVN6_SHORT(64, 3);
+        else if (row_len <= 2048) VPX_MVN6_SHORT(64, 4);
+        else if (row_len <= 2560) VPX_MVN6_SHORT(64, 5);
+        else if (row_len > 2560 && row_len <= 3072) VPX_MVN6_SHORT(64, 6);
         else if (row_len <= 2048) VPX_MVN6_ROWS(256, 1);
         else if (row_len <= 4096) VPX_MVN6_ROWS(256, 2);  // one wavefront per 4096-element row measured 9 % slower
+        else if (row_len <= 6144) VPX_MVN6_ROWS(256, 3);
         else if (row_len <= 8192) VPX_MVN6_ROWS(256, 4);
+        else if (row_len <= 10240) VPX_MVN6_ROWS(256, 5);
         else if (row_len <= 12288) VPX_MVN6_ROWS(256, 6);
+        else if (row_len <= 14336) VPX_MVN6_ROWS(256, 7);
         else VPX_MVN6_ROWS(256, 8);
 #undef VPX_MVN6_ROWS
 #undef VPX_MVN6_ROWS_R
