@@ -298,6 +298,26 @@ def test_fake_quantize_per_channel_limits(rt, orc, dev):
     assert_f16_exact(got, orc.fake_quantize_f16(x, lo, hi, lo, one, 256), "per-channel")
 
 
+@pytest.mark.parametrize("shape", [(3, 7, 5, 256), (1000, 8), (2, 31, 264), (1, 1, 9, 64), (70000, 16)])
+def test_fake_quantize_limits_per_innermost_channel(rt, orc, dev, shape):
+    """Channel-minor activations: one limit per innermost channel, some limits a single value; a lane keeps eight
+    channels' constants over a run of rows (row counts that do not fill the last run, channel runs shorter than a
+    workgroup, results below 2^-15 for the narrowing's slow path)."""
+    rng = np.random.default_rng(27)
+    ch = shape[-1]
+    lshape = (1,) * (len(shape) - 1) + (ch,)
+    x = orc.f32_to_f16(rng.normal(0, 2, shape).astype(np.float32))
+    lo = orc.f32_to_f16(-rng.uniform(0.5, 3, lshape).astype(np.float32))
+    hi = orc.f32_to_f16(rng.uniform(0.5, 3, lshape).astype(np.float32))
+    one = orc.f32_to_f16(np.full((1,) * len(shape), 1.0, np.float32))
+    tiny_lo = orc.f32_to_f16(rng.uniform(-3e-5, 0, lshape).astype(np.float32))
+    tiny_hi = orc.f32_to_f16(rng.uniform(1e-5, 6e-5, lshape).astype(np.float32))
+    for levels, ol, oh in ((256, lo, hi), (16, lo, one), (255, tiny_lo, tiny_hi)):
+        c = {"x": x, "in_lo": lo, "in_hi": hi, "out_lo": ol, "out_hi": oh, "levels": levels}
+        got = _run_fq(rt, dev, c)
+        assert_f16_exact(got, orc.fake_quantize_f16(x, lo, hi, ol, oh, levels), "%s levels %d" % (shape, levels))
+
+
 def test_fake_quantize_rejects_bad_arguments(rt, dev):
     import torch
     x = torch.zeros((1, 2, 3, 4), dtype=torch.float32, device=dev)
@@ -347,7 +367,9 @@ def test_quantize_dequantize(rt, orc, dev, signed, scale, zp):
                                               ((8, 8, 3, 3), 1, "NCHW"), ((16, 64), 1, None), ((700, 3), 0, None),
                                               # one vector per lane: channels shared by a vector, or consecutive channels
                                               ((4, 24, 8, 16), 1, "NCHW"), ((33, 7, 128), 0, None), ((50, 72), 1, None),
-                                              ((2, 9, 11, 40), 3, "NHWC"), ((300, 1024), 0, None)])
+                                              ((2, 9, 11, 40), 3, "NHWC"), ((300, 1024), 0, None),
+                                              # innermost axis, eight channels per lane: runs shorter and longer than a workgroup
+                                              ((1000, 8), 1, None), ((4099, 264), 1, None), ((37, 2056), 1, None)])
 def test_quantize_dequantize_per_axis(rt, orc, dev, shape, axis, order):
     """One scale / zero point per slice of `axis`.  The blob does not name the axis: it is the dimension
     whose size equals the parameter count, and the channel dimension when several have it ((8, 8, 3, 3))."""

@@ -1149,6 +1149,59 @@ int launch_eltwise(int op, const MemRef& a, const MemRef& b, const MemRef& out, 
 }
 
 // ---------------------------------------------------------------- fake_quantize
+// FakeQuantize of a packed tensor whose limits hold one value per innermost channel (or one value): a lane owns
+// eight adjacent channels, prepares their constants once (the one IEEE division per channel) and walks kFqInnerRows
+// rows.  Lanes are dealt along the rows' 128-bit words first, so short channel runs leave no lane idle.
+constexpr int kFqInnerRows = 8;
+__global__ __launch_bounds__(kBlock) void fq_inner8_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                           const half_t* __restrict__ l0, const half_t* __restrict__ l1,
+                                                           const half_t* __restrict__ l2, const half_t* __restrict__ l3,
+                                                           uint32_t per_channel,  // bit k: limit k has a value per channel
+                                                           uint32_t cvecs, int64_t rows, float lm1, float r_lm1) {
+    const int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t cv = (uint32_t)(g % cvecs);
+    const int64_t r0 = g / cvecs * kFqInnerRows;  // lanes past the last row group compute on row 0 and store nothing
+    const half_t* lim[4] = {l0, l1, l2, l3};
+    float c[4][8];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        if (per_channel >> k & 1) {
+            Pack<half_t, 8> v;
+            v.load(lim[k], cv);
+#pragma unroll
+            for (int e = 0; e < 8; e++) c[k][e] = (float)v.get(e);
+        } else {
+            const float f = (float)lim[k][0];
+#pragma unroll
+            for (int e = 0; e < 8; e++) c[k][e] = f;
+        }
+    }
+    float r_irange[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) r_irange[e] = 1.0f / (c[1][e] - c[0][e]);
+    Pack<half_t, 8> xs[kFqInnerRows];
+#pragma unroll
+    for (int r = 0; r < kFqInnerRows; r++) {
+        const int64_t row = r0 + r < rows ? r0 + r : 0;
+        xs[r].load(in, row * cvecs + cv);
+    }
+#pragma unroll
+    for (int r = 0; r < kFqInnerRows; r++) {
+        float f[8];
+        half_t h[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const FqConst cst{c[0][e], c[1][e], c[2][e], c[3][e], lm1, c[1][e] - c[0][e], r_irange[e], r_lm1, c[3][e] - c[2][e]};
+            f[e] = fq_f32_const((float)xs[r].get(e), cst);
+        }
+        narrow_vec(f, h);  // every lane of the wavefront votes, also those without a row
+        Pack<half_t, 8> y;
+#pragma unroll
+        for (int e = 0; e < 8; e++) y.set(e, h[e]);
+        if (r0 + r < rows) y.store(out, (r0 + r) * cvecs + cv);
+    }
+}
+
 int launch_fake_quantize(const MemRef& in, const MemRef lims[4], const MemRef& out, int64_t levels, hipStream_t s) {
     // Only FP16 in/out, like the reference kernel (sw_kernel.cpp:1156-1157).
     VPX_REQUIRE(in.dtype == VPX_NN_FP16 && out.dtype == VPX_NN_FP16, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
@@ -1168,6 +1221,25 @@ int launch_fake_quantize(const MemRef& in, const MemRef lims[4], const MemRef& o
         FqMap f{(const half_t*)in.data, (half_t*)out.data, (const half_t*)lims[0].data, (const half_t*)lims[1].data,
                 (const half_t*)lims[2].data, (const half_t*)lims[3].data, lm1};
         return launch_stream(f, n, s);
+    }
+    if (in.compact && out.compact && aligned16(in.data) && aligned16(out.data) && in.nd >= 1 && in.dims[0] % 8 == 0) {
+        // limits per innermost channel (channel-minor activations): constants per lane, kept across rows
+        const int64_t ch = in.dims[0];
+        uint32_t per_channel = 0;
+        const int64_t rows = n / ch, lanes = (rows + kFqInnerRows - 1) / kFqInnerRows * (ch / 8);
+        bool ok = n > 0 && lanes / kBlock < (1ll << 31) - 1;
+        for (int k = 0; k < 4 && ok; k++) {
+            if (lims[k].numel() == 1) continue;
+            ok = lims[k].numel() == ch && lims[k].dims[0] == ch && lims[k].strides[0] == 1 && aligned16(lims[k].data);
+            per_channel |= 1u << k;
+        }
+        if (ok) {
+            hipLaunchKernelGGL(fq_inner8_kernel, dim3((unsigned)((lanes + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, (const half_t*)in.data,
+                               (half_t*)out.data, (const half_t*)lims[0].data, (const half_t*)lims[1].data, (const half_t*)lims[2].data,
+                               (const half_t*)lims[3].data, per_channel, (uint32_t)(ch / 8), rows, lm1, 1.0f / lm1);
+            VPX_HIP_CHECK(hipGetLastError());
+            return VPX_RESULT_SUCCESS;
+        }
     }
     {
         // limits that broadcast (per channel and the like): five inputs, vectors along the innermost run
@@ -1644,11 +1716,12 @@ template <typename TI, typename TQ, bool SIMPLE>
 __global__ __launch_bounds__(kBlock) void quantize_axis_inner8_kernel(const TI* __restrict__ in, TQ* __restrict__ out,
                                                                       const float4* __restrict__ table, uint32_t count, uint32_t rows,
                                                                       float qmin, float qmax, float lm1) {
+    // lanes are dealt along a row's 128-bit words first, then over runs of kAxisRows rows: short channel runs idle no lane
     const uint32_t cvecs = count / 8;
-    const uint32_t ctiles = (cvecs + kBlock - 1) / kBlock;
-    const uint32_t cv = (blockIdx.x % ctiles) * kBlock + threadIdx.x;
-    const uint32_t r0 = (blockIdx.x / ctiles) * kAxisRows;
-    if (cv >= cvecs) return;
+    const int64_t lane = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t cv = (uint32_t)(lane % cvecs);
+    const int64_t r0 = lane / cvecs * kAxisRows;
+    if (r0 >= rows) return;
     float4 p[8];
     {
         const float4* planes = reinterpret_cast<const float4*>(table + count);  // four planes of count floats
@@ -1694,15 +1767,15 @@ template <typename TQ, typename TO>
 __global__ __launch_bounds__(kBlock) void dequantize_axis_inner8_kernel(const TQ* __restrict__ in, TO* __restrict__ out,
                                                                         const float4* __restrict__ table, uint32_t count, uint32_t rows) {
     const uint32_t cvecs = count / 8;
-    const uint32_t ctiles = (cvecs + kBlock - 1) / kBlock;
-    const uint32_t cv = (blockIdx.x % ctiles) * kBlock + threadIdx.x;
-    const uint32_t r0 = (blockIdx.x / ctiles) * kAxisRows;
-    const bool live = cv < cvecs;  // dead lanes still take part in the votes of narrow_vec
+    const int64_t lane = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const uint32_t cv = (uint32_t)(lane % cvecs);
+    const int64_t r0 = lane / cvecs * kAxisRows;  // lanes past the last run of rows read row 0 and store nothing: every
+                                                  // lane takes part in the votes of narrow_vec
     float sc[8];
     int zp[8];
     {
         const float4* planes = reinterpret_cast<const float4*>(table + count);  // plane 0: scales, plane 1: zero points
-        const uint32_t pv = count / 4, at = live ? cv * 2 : 0;
+        const uint32_t pv = count / 4, at = cv * 2;
         const float4 s0 = planes[at], s1 = planes[at + 1], z0 = planes[pv + at], z1 = planes[pv + at + 1];
         const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
         const float zv[8] = {z0.x, z0.y, z0.z, z0.w, z1.x, z1.y, z1.z, z1.w};
@@ -1714,12 +1787,10 @@ __global__ __launch_bounds__(kBlock) void dequantize_axis_inner8_kernel(const TQ
     }
     Pack<TQ, 8> xs[kAxisRows];  // every row's load is issued before the first result is needed
 #pragma unroll
-    for (int r = 0; r < kAxisRows; r++)
-        if (r0 + r < rows) xs[r].load(in, (int64_t)(r0 + r) * cvecs + (live ? cv : 0));
+    for (int r = 0; r < kAxisRows; r++) xs[r].load(in, (r0 + r < rows ? r0 + r : 0) * cvecs + cv);
 #pragma unroll
     for (int r = 0; r < kAxisRows; r++) {
-        if (r0 + r >= rows) break;  // uniform over the workgroup
-        const int64_t v = (int64_t)(r0 + r) * cvecs + (live ? cv : 0);
+        const int64_t v = (r0 + r) * cvecs + cv;
         const Pack<TQ, 8>& x = xs[r];
         float f[8];
 #pragma unroll
@@ -1734,7 +1805,7 @@ __global__ __launch_bounds__(kBlock) void dequantize_axis_inner8_kernel(const TQ
 #pragma unroll
             for (int k = 0; k < 8; k++) y.set(k, f[k]);
         }
-        if (live) y.store(out, v);
+        if (r0 + r < rows) y.store(out, v);
     }
 }
 
@@ -1770,7 +1841,7 @@ int quantize_axis_impl(const MemRef& in, const MemRef& out, const double* scales
     else if (g.inner == 1) {
         const uint32_t rows = total / g.count;
         if (g.count % 8 == 0 && (reinterpret_cast<uintptr_t>(in.data) % (8 * sizeof(TI))) == 0 && (reinterpret_cast<uintptr_t>(out.data) & 7) == 0) {
-            const dim3 igrid(((g.count / 8 + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
+            const dim3 igrid((unsigned)(((int64_t)(g.count / 8) * ((rows + kAxisRows - 1) / kAxisRows) + kBlock - 1) / kBlock));
             if (simple)
                 hipLaunchKernelGGL((quantize_axis_inner8_kernel<TI, TQ, true>), igrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data,
                                    table, g.count, rows, fmin_, fmax_, lm1);
@@ -1812,7 +1883,7 @@ int dequantize_axis_impl(const MemRef& in, const MemRef& out, const double* scal
     else if (g.inner == 1) {
         const uint32_t rows = total / g.count;
         if (g.count % 8 == 0 && (reinterpret_cast<uintptr_t>(in.data) & 7) == 0 && (reinterpret_cast<uintptr_t>(out.data) % (8 * sizeof(TO))) == 0) {
-            const dim3 igrid(((g.count / 8 + kBlock - 1) / kBlock) * ((rows + kAxisRows - 1) / kAxisRows));
+            const dim3 igrid((unsigned)(((int64_t)(g.count / 8) * ((rows + kAxisRows - 1) / kAxisRows) + kBlock - 1) / kBlock));
             hipLaunchKernelGGL((dequantize_axis_inner8_kernel<TQ, TO>), igrid, dim3(kBlock), 0, s, (const TQ*)in.data, (TO*)out.data, table,
                                g.count, rows);
         } else {
