@@ -1153,14 +1153,40 @@ int launch_eltwise(int op, const MemRef& a, const MemRef& b, const MemRef& out, 
 // eight adjacent channels, prepares their constants once (the one IEEE division per channel) and walks kFqInnerRows
 // rows.  Lanes are dealt along the rows' 128-bit words first, so short channel runs leave no lane idle.
 constexpr int kFqInnerRows = 8;
+// How the channel-minor kernels deal the 128-bit words of a [rows x cvecs] tensor: a lane visits words
+// first + k * step (k < R, below end) that all hold the same eight channels `cv`.  When a workgroup's lanes cover
+// whole rows (cvecs divides the workgroup) the R visits of a workgroup are R adjacent runs of kBlock words, else a
+// lane walks R consecutive rows of its column of words.
+struct InnerDeal {
+    uint32_t cv;
+    int64_t first, step, end;
+};
+__device__ __forceinline__ InnerDeal inner_deal(uint32_t cvecs, int64_t rows, int R) {
+    InnerDeal d;
+    d.end = rows * cvecs;
+    if (kBlock % cvecs == 0) {
+        d.cv = threadIdx.x % cvecs;
+        d.first = (int64_t)blockIdx.x * kBlock * R + threadIdx.x;
+        d.step = kBlock;
+    } else {
+        const int64_t lane = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+        d.cv = (uint32_t)(lane % cvecs);
+        d.first = lane / cvecs * R * cvecs + d.cv;
+        d.step = cvecs;
+    }
+    return d;
+}
+static inline unsigned inner_deal_blocks(uint32_t cvecs, int64_t rows, int R) {
+    if (kBlock % cvecs == 0) return (unsigned)((rows * cvecs + (int64_t)kBlock * R - 1) / ((int64_t)kBlock * R));
+    return (unsigned)(((rows + R - 1) / R * cvecs + kBlock - 1) / kBlock);
+}
 __global__ __launch_bounds__(kBlock) void fq_inner8_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
                                                            const half_t* __restrict__ l0, const half_t* __restrict__ l1,
                                                            const half_t* __restrict__ l2, const half_t* __restrict__ l3,
                                                            uint32_t per_channel,  // bit k: limit k has a value per channel
                                                            uint32_t cvecs, int64_t rows, float lm1, float r_lm1) {
-    const int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const uint32_t cv = (uint32_t)(g % cvecs);
-    const int64_t r0 = g / cvecs * kFqInnerRows;  // lanes past the last row group compute on row 0 and store nothing
+    const InnerDeal d = inner_deal(cvecs, rows, kFqInnerRows);  // lanes past the end compute on word cv and store nothing
+    const uint32_t cv = d.cv;
     const half_t* lim[4] = {l0, l1, l2, l3};
     float c[4][8];
 #pragma unroll
@@ -1182,8 +1208,8 @@ __global__ __launch_bounds__(kBlock) void fq_inner8_kernel(const half_t* __restr
     Pack<half_t, 8> xs[kFqInnerRows];
 #pragma unroll
     for (int r = 0; r < kFqInnerRows; r++) {
-        const int64_t row = r0 + r < rows ? r0 + r : 0;
-        xs[r].load(in, row * cvecs + cv);
+        const int64_t v = d.first + r * d.step;
+        xs[r].load(in, v < d.end ? v : cv);
     }
 #pragma unroll
     for (int r = 0; r < kFqInnerRows; r++) {
@@ -1198,7 +1224,7 @@ __global__ __launch_bounds__(kBlock) void fq_inner8_kernel(const half_t* __restr
         Pack<half_t, 8> y;
 #pragma unroll
         for (int e = 0; e < 8; e++) y.set(e, h[e]);
-        if (r0 + r < rows) y.store(out, (r0 + r) * cvecs + cv);
+        if (d.first + r * d.step < d.end) y.store(out, d.first + r * d.step);
     }
 }
 
@@ -1234,7 +1260,7 @@ int launch_fake_quantize(const MemRef& in, const MemRef lims[4], const MemRef& o
             per_channel |= 1u << k;
         }
         if (ok) {
-            hipLaunchKernelGGL(fq_inner8_kernel, dim3((unsigned)((lanes + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, (const half_t*)in.data,
+            hipLaunchKernelGGL(fq_inner8_kernel, dim3(inner_deal_blocks((uint32_t)(ch / 8), rows, kFqInnerRows)), dim3(kBlock), 0, s, (const half_t*)in.data,
                                (half_t*)out.data, (const half_t*)lims[0].data, (const half_t*)lims[1].data, (const half_t*)lims[2].data,
                                (const half_t*)lims[3].data, per_channel, (uint32_t)(ch / 8), rows, lm1, 1.0f / lm1);
             VPX_HIP_CHECK(hipGetLastError());
@@ -1718,10 +1744,9 @@ __global__ __launch_bounds__(kBlock) void quantize_axis_inner8_kernel(const TI* 
                                                                       float qmin, float qmax, float lm1) {
     // lanes are dealt along a row's 128-bit words first, then over runs of kAxisRows rows: short channel runs idle no lane
     const uint32_t cvecs = count / 8;
-    const int64_t lane = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const uint32_t cv = (uint32_t)(lane % cvecs);
-    const int64_t r0 = lane / cvecs * kAxisRows;
-    if (r0 >= rows) return;
+    const InnerDeal d = inner_deal(cvecs, rows, kAxisRows);
+    const uint32_t cv = d.cv;
+    if (d.first >= d.end) return;
     float4 p[8];
     {
         const float4* planes = reinterpret_cast<const float4*>(table + count);  // four planes of count floats
@@ -1746,11 +1771,11 @@ __global__ __launch_bounds__(kBlock) void quantize_axis_inner8_kernel(const TI* 
         Pack<TI, 8> xs[kBatch];
 #pragma unroll
         for (int r = 0; r < kBatch; r++)
-            if (r0 + rb + r < rows) xs[r].load(in, (int64_t)(r0 + rb + r) * cvecs + cv);
+            if (d.first + (rb + r) * d.step < d.end) xs[r].load(in, d.first + (rb + r) * d.step);
 #pragma unroll
         for (int r = 0; r < kBatch; r++) {
-        if (r0 + rb + r >= rows) break;
-        const int64_t v = (int64_t)(r0 + rb + r) * cvecs + cv;
+        const int64_t v = d.first + (rb + r) * d.step;
+        if (v >= d.end) break;
         const Pack<TI, 8>& x = xs[r];
         Pack<TQ, 8> y;
 #pragma unroll
@@ -1767,10 +1792,8 @@ template <typename TQ, typename TO>
 __global__ __launch_bounds__(kBlock) void dequantize_axis_inner8_kernel(const TQ* __restrict__ in, TO* __restrict__ out,
                                                                         const float4* __restrict__ table, uint32_t count, uint32_t rows) {
     const uint32_t cvecs = count / 8;
-    const int64_t lane = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const uint32_t cv = (uint32_t)(lane % cvecs);
-    const int64_t r0 = lane / cvecs * kAxisRows;  // lanes past the last run of rows read row 0 and store nothing: every
-                                                  // lane takes part in the votes of narrow_vec
+    const InnerDeal d = inner_deal(cvecs, rows, kAxisRows);  // lanes past the end read word cv and store nothing: every
+    const uint32_t cv = d.cv;                                // lane takes part in the votes of narrow_vec
     float sc[8];
     int zp[8];
     {
@@ -1787,10 +1810,10 @@ __global__ __launch_bounds__(kBlock) void dequantize_axis_inner8_kernel(const TQ
     }
     Pack<TQ, 8> xs[kAxisRows];  // every row's load is issued before the first result is needed
 #pragma unroll
-    for (int r = 0; r < kAxisRows; r++) xs[r].load(in, (r0 + r < rows ? r0 + r : 0) * cvecs + cv);
+    for (int r = 0; r < kAxisRows; r++) xs[r].load(in, d.first + r * d.step < d.end ? d.first + r * d.step : cv);
 #pragma unroll
     for (int r = 0; r < kAxisRows; r++) {
-        const int64_t v = (r0 + r) * cvecs + cv;
+        const int64_t v = d.first + r * d.step;
         const Pack<TQ, 8>& x = xs[r];
         float f[8];
 #pragma unroll
@@ -1805,7 +1828,7 @@ __global__ __launch_bounds__(kBlock) void dequantize_axis_inner8_kernel(const TQ
 #pragma unroll
             for (int k = 0; k < 8; k++) y.set(k, f[k]);
         }
-        if (r0 + r < rows) y.store(out, v);
+        if (v < d.end) y.store(out, v);
     }
 }
 
@@ -1841,7 +1864,7 @@ int quantize_axis_impl(const MemRef& in, const MemRef& out, const double* scales
     else if (g.inner == 1) {
         const uint32_t rows = total / g.count;
         if (g.count % 8 == 0 && (reinterpret_cast<uintptr_t>(in.data) % (8 * sizeof(TI))) == 0 && (reinterpret_cast<uintptr_t>(out.data) & 7) == 0) {
-            const dim3 igrid((unsigned)(((int64_t)(g.count / 8) * ((rows + kAxisRows - 1) / kAxisRows) + kBlock - 1) / kBlock));
+            const dim3 igrid(inner_deal_blocks(g.count / 8, rows, kAxisRows));
             if (simple)
                 hipLaunchKernelGGL((quantize_axis_inner8_kernel<TI, TQ, true>), igrid, dim3(kBlock), 0, s, (const TI*)in.data, (TQ*)out.data,
                                    table, g.count, rows, fmin_, fmax_, lm1);
@@ -1883,7 +1906,7 @@ int dequantize_axis_impl(const MemRef& in, const MemRef& out, const double* scal
     else if (g.inner == 1) {
         const uint32_t rows = total / g.count;
         if (g.count % 8 == 0 && (reinterpret_cast<uintptr_t>(in.data) & 7) == 0 && (reinterpret_cast<uintptr_t>(out.data) % (8 * sizeof(TO))) == 0) {
-            const dim3 igrid((unsigned)(((int64_t)(g.count / 8) * ((rows + kAxisRows - 1) / kAxisRows) + kBlock - 1) / kBlock));
+            const dim3 igrid(inner_deal_blocks(g.count / 8, rows, kAxisRows));
             hipLaunchKernelGGL((dequantize_axis_inner8_kernel<TQ, TO>), igrid, dim3(kBlock), 0, s, (const TQ*)in.data, (TO*)out.data, table,
                                g.count, rows);
         } else {
