@@ -884,7 +884,7 @@ __device__ __forceinline__ float team_sum(float v, float* smem) {
     }
     v = wave_sum(v);
     if (TEAM == 64) return v;
-    __syncthreads();
+    // one barrier: each sum of a workgroup's lifetime has four slots of its own
     if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
     __syncthreads();
     return (smem[0] + smem[1]) + (smem[2] + smem[3]);
@@ -897,7 +897,8 @@ template <int TEAM, int VPT, int RPT = 1>  // RPT: consecutive rows a team walks
 __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
                                                              const half_t* __restrict__ sc, const half_t* __restrict__ bi,
                                                              Mvn6Geom g, int normalize_variance, int eps_mode, float eps) {
-    __shared__ float red[4];
+    __shared__ float red[8];
+    static_assert(TEAM != 256 || RPT == 1, "the workgroup-wide sums have slots for one row");
     const int t = (int)(threadIdx.x % TEAM);
     const int64_t row0 = ((int64_t)blockIdx.x * (kThreads / TEAM) + threadIdx.x / TEAM) * RPT;
     // scale and bias that run along the row (and do not depend on it): loaded once for the RPT rows
@@ -948,7 +949,7 @@ __global__ __launch_bounds__(kThreads) void mvn6_rows_kernel(const half_t* __res
             q += e0 < g.row_len ? d * d : 0.f;
         }
     }
-    const float var = team_sum<TEAM>(q, red) / n;
+    const float var = team_sum<TEAM>(q, red + 4) / n;
     const float inv = mvn6_inv(var, normalize_variance, eps_mode, eps);
     const float sc_row = sc && !g.sc_along_row ? (float)sc[b.sc] : 1.0f;
     const float bi_row = bi && !g.bi_along_row ? (float)bi[b.bi] : 0.0f;
@@ -1072,7 +1073,7 @@ __global__ __launch_bounds__(kThreads) void mvn6_inner_kernel(const half_t* __re
 __global__ __launch_bounds__(kThreads) void mvn6_generic_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
                                                                 const half_t* __restrict__ sc, const half_t* __restrict__ bi,
                                                                 Mvn6Geom g, int normalize_variance, int eps_mode, float eps) {
-    __shared__ float red[4];
+    __shared__ float red[8];
     const RowBase b = row_base(g, blockIdx.x);
     float sum = 0.f;
     for (uint32_t e = threadIdx.x; e < g.row_len; e += kThreads) sum += (float)in[b.in + elem_off(g, e).in];
@@ -1084,7 +1085,7 @@ __global__ __launch_bounds__(kThreads) void mvn6_generic_kernel(const half_t* __
             const float d = (float)in[b.in + elem_off(g, e).in] - mean;
             q += d * d;
         }
-    const float var = team_sum<256>(q, red) / n;
+    const float var = team_sum<256>(q, red + 4) / n;
     const float inv = mvn6_inv(var, normalize_variance, eps_mode, eps);
     for (uint32_t e = threadIdx.x; e < g.row_len; e += kThreads) {
         const ElemOff o = elem_off(g, e);
