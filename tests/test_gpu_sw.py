@@ -717,7 +717,7 @@ def _softmax(rt, dev, x_bits, axis, pad=0, packed=True, f32=False):
                                         ((9, 1000), 1), ((4, 8200), 1), ((2, 3, 4, 4), 3), ((6, 32, 4, 4), 1),
                                         ((5, 17, 300), 1), ((17, 64), 0), ((2, 3, 50, 7), 2),
                                         # rows that are not 16-byte aligned, long rows (one workgroup per row), and beyond
-                                        ((65, 500), 1), ((7, 511), 1), ((130, 197), 1), ((3, 1023), 1), ((9, 4099), 1),
+                                        ((65, 500), 1), ((7, 511), 1), ((130, 197), 1), ((300, 192), 1), ((77, 160), 1), ((130, 248), 1), ((3, 1023), 1), ((9, 4099), 1),
                                         ((3, 32768), 1), ((5, 20000), 1), ((6, 8191), 1), ((2, 33000), 1), ((2, 40001), 1),
                                         ((20000, 8), 1), ((17000, 509), 1),
                                         # many short rows: runs of rows through LDS (any length), a ragged last run

@@ -841,7 +841,7 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
             VPX_HIP_CHECK(hipGetLastError());
             return VPX_RESULT_SUCCESS;
         }
-        if (packed && rows >= 64 && (len <= 128 || (len % 8 != 0 && len <= 384)) && base16) {
+        if (packed && rows >= 64 && (len < 256 || (len % 8 != 0 && len <= 384)) && base16) {  // one wavefront per row idles lanes below 256 values
             const int per_wg = (int)(kShortChunk / len);
             const dim3 grid((unsigned)((rows + per_wg - 1) / per_wg));
 #define VPX_SHORT(K) hipLaunchKernelGGL(softmax_short_rows_f16<K>, grid, dim3(256), 0, s, hin, hout, rows, (int)len, per_wg)
