@@ -2,14 +2,21 @@
 """Benchmark of the vpux hot path on one MI355X.
 
 A step is one pass of the selected configuration's hot path over one batch of synthetic input that
-is already resident in HBM.  The default workload is BASELINE configuration 2 (softmax fp16
-[8,16,512,512]); `--workload` selects another one and `--all` appends a short measurement of every
-configuration to the same JSON line.
+is already resident in HBM.  The headline workload is BASELINE configuration 5's int8 matmul
+(A[4096,4096] x B[4096,11008] with the integer PPE), the largest configuration and the one the
+metric's first clause (int8 TOP/s) is quoted on; the same run appends `other_configs` with the
+remaining BASELINE configurations (C1 FakeQuantize, C2 softmax, C3 MVN, C4 conv, C5 dequantize and
+C5 add), each with its own roofline and CPU baseline.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2_softmax] [--all] [--no-cpu]
+Every configuration is timed over a rotation of separate buffer sets whose total exceeds the 256 MB
+Infinity Cache, so a step does not find its operands in cache; the same-buffers figure and a HIP-graph
+replay are reported beside it as named extras.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5_matmul] [--only] [--no-cpu] [--extra]
 """
 import argparse
 import ctypes as C
+import itertools
 import json
 import os
 import sys
@@ -22,8 +29,9 @@ I8_PEAK_TOPS = 5000.0     # MI355X dense int8 MFMA, published
 
 METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
 
-# Bytes moved through L2 per step, from rocprofv3 FETCH_SIZE / WRITE_SIZE counters scaled by a plain
-# copy of known size (profiles/<workload>__*.md hold the runs these come from).
+# Bytes moved through L2 per step.  These are NOT measured in this run: they are the rocprofv3 FETCH_SIZE /
+# WRITE_SIZE counters of an earlier run of the same workload, scaled by a plain copy of known size
+# (profiles/<workload>__*.md hold those runs and their commands); the JSON line labels them as such.
 MEASURED_TRAFFIC = {
     "c1_fake_quantize": 880079, "c2_softmax": 134293332, "c3_mvn": 25440485, "c4_conv": 16276094,
     "c5_matmul": 385007798, "c5_dequantize": 135326848, "c5_eltwise_add": 270538895, "c5_nce_eltwise": 135268239,
@@ -44,10 +52,12 @@ class Workload:
     """name, description, a zero-argument `step` that enqueues one pass on the current stream,
     algorithmic bytes and ops per step, roofline bound and the CPU-oracle sample runner."""
 
-    def __init__(self, name, desc, step, bytes_per_step, ops_per_step, bound, dtype, kernel, cpu_sample=None):
+    def __init__(self, name, desc, step, bytes_per_step, ops_per_step, bound, dtype, kernel, cpu_sample=None,
+                 cpu_units=(1, 1, "full tensor")):
         self.name, self.desc, self.step = name, desc, step
         self.bytes, self.ops, self.bound, self.dtype, self.kernel = bytes_per_step, ops_per_step, bound, dtype, kernel
-        self.cpu_sample = cpu_sample
+        # cpu_sample(oracle, units) -> (callable, work in bytes or ops); cpu_units = (first sample, whole workload, what a unit is)
+        self.cpu_sample, self.cpu_units = cpu_sample, cpu_units
 
 
 def _prebuilt_sw_launch(rt, entry, blob, operands):
@@ -82,7 +92,8 @@ def make_c1(rt):
     def cpu(orc, frac):
         return lambda: orc.fake_quantize_f16(c["x"], c["in_lo"], c["in_hi"], c["out_lo"], c["out_hi"], 256), n * 4
     return Workload("c1_fake_quantize", "FakeQuantize fp16 NCHW [1,64,56,56], per-tensor, 256 levels, +-4",
-                    _prebuilt_sw_launch(rt, "fake_quantize", blob, ops), n * 4, 0, "hbm", "f16", "stream_kernel<FqMap>", cpu)
+                    _prebuilt_sw_launch(rt, "fake_quantize", blob, ops), n * 4, 0, "hbm", "f16", "stream_kernel<FqMap>", cpu,
+                    (1, 1, "full tensor"))
 
 
 def make_c2(rt):
@@ -102,7 +113,8 @@ def make_c2(rt):
         xs = np.ascontiguousarray(c["x"].reshape(-1, 512)[:rows])
         return lambda: orc.softmax_f16(xs, 1), xs.size * 4
     return Workload("c2_softmax", "Softmax fp16 last axis [8,16,512,512], 5% of logits masked to -60000",
-                    _prebuilt_sw_launch(rt, "softmax", blob, ops), n * 4, 0, "hbm", "f16", "softmax_rows_f16", cpu)
+                    _prebuilt_sw_launch(rt, "softmax", blob, ops), n * 4, 0, "hbm", "f16", "softmax_rows_f16", cpu,
+                    (2048, 65536, "rows"))
 
 
 def make_c3(rt):
@@ -120,7 +132,8 @@ def make_c3(rt):
         xs = np.ascontiguousarray(c["x"][:groups])
         return lambda: orc.mvn_f16(xs, True, True, c["eps"]), xs.size * 4
     return Workload("c3_mvn", "MVN fp16 across C,H,W [4,256,64,64], eps 1e-9, normalize_variance",
-                    _prebuilt_sw_launch(rt, "mvn1", blob, ops), n * 4, 0, "hbm", "f16", "mvn_chunk_kernel", cpu)
+                    _prebuilt_sw_launch(rt, "mvn1", blob, ops), n * 4, 0, "hbm", "f16", "mvn_chunk_kernel", cpu,
+                    (1, 4, "batch elements"))
 
 
 def _nce_step(rt, task):
@@ -171,7 +184,24 @@ def make_c4(rt):
         return lambda: orc.nce_conv(c["input"], c["weights"], wt_h, p, zp_in=128, pads=(1, 1, 1, 1), rows=(0, rows)), \
             2 * rows * 64 * 9 * 64
     return Workload("c4_conv", "int8 Conv 3x3 s1 p1 NHWC [32,56,56,64] u8 zp128 x [64,3,3,64] i8, PPE ReLU clamp [0,255]",
-                    step, nbytes, ops, "mfma", "int8", "nce_conv_tile", cpu)
+                    step, nbytes, ops, "mfma", "int8", "nce_conv_tile", cpu, (3136, 100352, "output positions"))
+
+
+_C5_CACHE = {}
+
+
+def _c5_quantized(M, N):
+    """Stand-in for the matmul's i8 output (uniform codes), generated once on the host."""
+    if "q" not in _C5_CACHE:
+        _C5_CACHE["q"] = np.random.default_rng(55).integers(-128, 128, (M, N), dtype=np.int8)
+    return _C5_CACHE["q"]
+
+
+def _c5_dequantized(M, N):
+    """The dequantized tensor the residual is added to: code * 0.05, exact in fp16 for |code| <= 128 after rounding."""
+    if "deq" not in _C5_CACHE:
+        _C5_CACHE["deq"] = (_c5_quantized(M, N).astype(np.float32) * np.float32(0.05)).astype(np.float16).view(np.uint16)
+    return _C5_CACHE["deq"]
 
 
 def make_c5(rt, part="matmul"):
@@ -196,8 +226,10 @@ def make_c5(rt, part="matmul"):
             a_s = np.ascontiguousarray(c["a"][:rows])
             return lambda: orc.nce_matmul(a_s, c["b_nk"], wt_h, p, zp_a=c["zp_a"]), 2 * rows * K * N
         return Workload("c5_matmul", "int8 MatMul A[4096,4096] zp3 x B[4096,11008], PPE per-column + LeakyReLU 0.1 -> i8",
-                        step, M * K + N * K + M * N + N * 16, 2 * M * K * N, "mfma", "int8", "nce_gemm_mfma", cpu)
-    q = torch.randint(-128, 128, (M, N), dtype=torch.int8, device="cuda")
+                        step, M * K + N * K + M * N + N * 16, 2 * M * K * N, "mfma", "int8", "nce_gemm_mfma", cpu,
+                        (8, 4096, "rows of A"))
+    q_h = _c5_quantized(M, N)
+    q = _dev(q_h)
     if part == "nce_eltwise":
         # the quantized form of the same residual add: i8 + i8 -> i8 on the NCE eltwise path
         res_q = torch.randint(-128, 128, (M, N), dtype=torch.int8, device="cuda")
@@ -219,15 +251,26 @@ def make_c5(rt, part="matmul"):
     if part == "dequant":
         ops = [rt.Operand(q), rt.Operand(deq)]
         blob = rt.create_kernel_params(ops[:1], ops[1:], rt.get_quant_params_attr(c["deq_scale"], c["deq_zp"], rt.NN_FP16).tobytes())
+
+        def cpu(orc, rows):
+            qs = np.ascontiguousarray(q_h[:rows])
+            return lambda: orc.dequantize(qs, [c["deq_scale"]], [c["deq_zp"]], to_f16=True), qs.size * 3
         return Workload("c5_dequantize", "Dequantize i8 -> fp16 [4096,11008], per-tensor",
-                        _prebuilt_sw_launch(rt, "dequantize", blob, ops), M * N * 3, 0, "hbm", "f16", "stream_kernel<DequantFn>")
+                        _prebuilt_sw_launch(rt, "dequantize", blob, ops), M * N * 3, 0, "hbm", "f16", "stream_kernel<DequantFn>",
+                        cpu, (256, 4096, "rows"))
     res = _dev(c["residual"], True)
     y = torch.empty_like(deq)
-    deq.normal_()
+    deq_h = _c5_dequantized(M, N)
+    deq.copy_(_dev(deq_h, True))
     ops = [rt.Operand(deq), rt.Operand(res), rt.Operand(y)]
     blob = rt.create_kernel_params(ops[:2], ops[2:])
+
+    def cpu(orc, rows):
+        a_s, b_s = np.ascontiguousarray(deq_h[:rows]), np.ascontiguousarray(c["residual"][:rows])
+        return lambda: orc.eltwise_f16("add", a_s, b_s), a_s.size * 6
     return Workload("c5_eltwise_add", "Eltwise Add fp16 [4096,11008] + residual",
-                    _prebuilt_sw_launch(rt, "eltwise_add", blob, ops), M * N * 6, 0, "hbm", "f16", "stream_kernel<EltFn add>")
+                    _prebuilt_sw_launch(rt, "eltwise_add", blob, ops), M * N * 6, 0, "hbm", "f16", "stream_kernel<EltFn add>",
+                    cpu, (256, 4096, "rows"))
 
 
 def make_copy(rt):
@@ -356,9 +399,10 @@ def time_steps(step, steps, warmup, graph=False):
         torch.cuda.synchronize()
         run = g.replay
     else:
-        def run():
-            for _ in range(steps):
-                step()
+        def run(seq=(step,) * steps):
+            for f in seq:
+                f()
+    # events are recorded on the stream the steps are launched on (the current stream)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -371,13 +415,17 @@ def time_steps(step, steps, warmup, graph=False):
 
 
 def roofline(w, dev_ms):
+    traffic = MEASURED_TRAFFIC.get(w.name)
+    src = "profiles/%s__*.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run, not measured in this run)" % w.name
     if w.bound == "hbm":
         achieved = w.bytes / (dev_ms * 1e-3) / 1e9
         return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(w.name), "kernel": w.kernel}
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": src if traffic else None,
+                "kernel": w.kernel, "algorithmic_bytes": w.bytes}
     achieved = w.ops / (dev_ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": round(achieved, 2), "peak": I8_PEAK_TOPS, "unit": "TOP/s",
-            "frac": round(achieved / I8_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC.get(w.name), "kernel": w.kernel}
+            "frac": round(achieved / I8_PEAK_TOPS, 4), "traffic": traffic, "traffic_source": src if traffic else None,
+            "kernel": w.kernel, "algorithmic_ops": w.ops}
 
 
 def value_of(w, ms):
@@ -386,14 +434,13 @@ def value_of(w, ms):
     return w.ops / (ms * 1e-3) / 1e12, "TOP/s"
 
 
-def cpu_baseline(w, budget_s=12.0):
-    """Times the CPU oracle on a bounded sample of the same workload, all host threads."""
+def cpu_baseline(w, budget_s=8.0, one_thread_s=2.5):
+    """Times the CPU oracle on a bounded sample of the same workload: all host threads, then one thread."""
     import oracle
     if w.cpu_sample is None:
         return None
     cores = min(oracle.num_threads(), int(os.environ.get("OMP_NUM_THREADS", "1024")))
-    units = {"c1_fake_quantize": 1, "c2_softmax": 2048, "c3_mvn": 1, "c4_conv": 3136, "c5_matmul": 8}[w.name]
-    full = {"c1_fake_quantize": 1, "c2_softmax": 65536, "c3_mvn": 4, "c4_conv": 100352, "c5_matmul": 4096}[w.name]
+    units, full, what = w.cpu_units
     fn, work = w.cpu_sample(oracle, units)
     t0 = time.perf_counter()
     fn()
@@ -411,29 +458,77 @@ def cpu_baseline(w, budget_s=12.0):
     for _ in range(reps):
         fn()
     dt = (time.perf_counter() - t0) / reps
-    if w.bound == "hbm":
-        val, unit = work / dt / 1e9, "GB/s"
-    else:
-        val, unit = work / dt / 1e12, "TOP/s"
-    what = {"c1_fake_quantize": "full tensor", "c2_softmax": "%d of 65536 rows" % units, "c3_mvn": "%d of 4 batch elements" % units,
-            "c4_conv": "%d of 100352 output positions" % units, "c5_matmul": "%d of 4096 rows of A" % units}[w.name]
-    # a sample sized for about four seconds on one thread
-    units1 = max(1, int(units * min(1.0, 4.0 / max(dt * cores, 1e-6))))
+    div = 1e9 if w.bound == "hbm" else 1e12
+    unit = "GB/s" if w.bound == "hbm" else "TOP/s"
+    val = work / dt / div
+    sample = "full tensor" if units == full else "%d of %d %s" % (units, full, what)
+    # a sample sized for the one-thread budget
+    units1 = max(1, int(units * min(1.0, one_thread_s / max(dt * cores, 1e-6))))
     fn1, work1 = w.cpu_sample(oracle, units1)
     oracle.set_num_threads(1)
     try:
         t0 = time.perf_counter()
         n1 = 0
-        while n1 < reps and (n1 == 0 or time.perf_counter() - t0 < 4.0):
+        while n1 < reps and (n1 == 0 or time.perf_counter() - t0 < one_thread_s):
             fn1()
             n1 += 1
         dt1 = (time.perf_counter() - t0) / n1
     finally:
         oracle.set_num_threads(cores)
-    val1 = work1 / dt1 / (1e9 if w.bound == "hbm" else 1e12)
     return {"value": round(val, 4), "unit": unit, "cores": cores, "kind": "port",
-            "sample": "%s, %d repetition(s), %.3f s per repetition, %.1f s in total" % (what, reps, dt, reps * dt),
-            "value_one_thread": round(val1, 4)}
+            "sample": "%s, %d repetition(s), %.3f s per repetition, %.1f s in total" % (sample, reps, dt, reps * dt),
+            "value_one_thread": round(work1 / dt1 / div, 4)}
+
+
+CACHE_BYTES = 256 << 20   # Infinity Cache of the part
+MAX_SETS = 512
+
+
+def footprint(w):
+    """Bytes one buffer set of a workload occupies (what a step touches)."""
+    return w.bytes if w.bytes else 1 << 30
+
+
+def build_sets(name, rt, rotate):
+    """The workload plus as many further copies on separate buffers as the rotation asks for: by default enough that
+    their total is at least 1.25 times the Infinity Cache, so that a set has left the cache when its turn comes again."""
+    w = MAKERS[name](rt)
+    n = rotate if rotate > 0 else min(MAX_SETS, max(2, -(-(CACHE_BYTES * 5 // 4) // footprint(w))))
+    sets = [w] + [MAKERS[name](rt) for _ in range(n - 1)]
+    ring = itertools.cycle([x.step for x in sets])
+
+    def step():
+        next(ring)()
+    return w, sets, step
+
+
+def measure(name, rt, steps, warmup, rotate, cpu, extras=True):
+    """One configuration: rotated eager timing (the figure of record), then the same-buffers and HIP-graph extras."""
+    import torch
+    w, sets, step = build_sets(name, rt, rotate)
+    wall_ms, dev_ms = time_steps(step, steps, warmup)
+    value, unit = value_of(w, wall_ms)
+    rec = {"value": round(value, 2), "unit": unit, "dtype": w.dtype, "description": w.desc, "steps": steps, "warmup": warmup,
+           "launch": "eager", "buffer_sets": len(sets), "buffer_bytes_total": len(sets) * footprint(w),
+           "ms_per_step": round(wall_ms, 6), "device_ms_per_step": round(dev_ms, 6), "roofline": roofline(w, dev_ms)}
+    if extras:
+        _, same_ms = time_steps(w.step, steps, min(warmup, 5))
+        _, graph_ms = time_steps(step, steps, 2, graph=True)
+        rec["extras"] = {"same_buffers_device_ms_per_step": round(same_ms, 6),
+                         "same_buffers_frac": roofline(w, same_ms)["frac"],
+                         "graph_device_ms_per_step": round(graph_ms, 6),
+                         "graph_frac": roofline(w, graph_ms)["frac"]}
+    if cpu:
+        rec["cpu_baseline"] = cpu_baseline(w)
+    del sets, step
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    return w, rec
+
+
+HEADLINE = "c5_matmul"
+OTHER_CONFIGS = ["c1_fake_quantize", "c2_softmax", "c3_mvn", "c4_conv", "c5_dequantize", "c5_eltwise_add"]
+EXTRA_CONFIGS = ["c5_nce_eltwise", "x_mvn6_layernorm", "x_activation_hswish", "x_mvn1_three_steps"]
 
 
 def main():
@@ -441,13 +536,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2_softmax", choices=sorted(MAKERS))
-    ap.add_argument("--all", action="store_true", help="also measure every other configuration (short runs)")
-    ap.add_argument("--graph", action="store_true", help="replay the timed steps from one HIP graph")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--rotate", type=int, default=1, metavar="N",
-                    help="cycle through N separate buffer sets so that a step does not find its operands in the 256 MB "
-                         "Infinity Cache left there by the previous one (default 1: same buffers every step)")
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(MAKERS))
+    ap.add_argument("--only", action="store_true", help="measure the headline workload only (no other_configs)")
+    ap.add_argument("--extra", action="store_true", help="also measure the workloads beside the BASELINE configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--rotate", type=int, default=0, metavar="N",
+                    help="number of separate buffer sets a workload cycles through (default 0: as many as make their "
+                         "total exceed 1.25 x the 256 MB Infinity Cache; 1: the same buffers every step)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on one GPU only (every kernel shards without exchange, so N GPUs would run N independent copies); "
@@ -459,43 +554,29 @@ def main():
     rt.lib()
     torch.cuda.set_device(0)
 
-    w = MAKERS[args.workload](rt)
-    step = w.step
-    if args.rotate > 1:
-        sets = [w] + [MAKERS[args.workload](rt) for _ in range(args.rotate - 1)]
-        counter = [0]
-
-        def step():
-            sets[counter[0] % len(sets)].step()
-            counter[0] += 1
-    wall_ms, dev_ms = time_steps(step, args.steps, args.warmup, graph=args.graph)
-    value, unit = value_of(w, wall_ms)
+    t_start = time.perf_counter()
+    w, rec = measure(args.workload, rt, args.steps, args.warmup, args.rotate, cpu=not args.no_cpu)
     line = {
-        "metric": METRIC, "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(wall_ms, 6), "higher_is_better": True, "scaling": "weak",
+        "metric": METRIC, "value": rec["value"], "unit": rec["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": rec["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": w.dtype, "data": "synthetic",
-        "config": {"workload": w.name, "description": w.desc, "launch": "hip graph" if args.graph else "eager",
-                   "buffer_sets": args.rotate},
-        "device_ms_per_step": round(dev_ms, 6),
-        "roofline": roofline(w, dev_ms),
+        "config": {"workload": w.name, "description": w.desc, "launch": "eager", "buffer_sets": rec["buffer_sets"],
+                   "buffer_bytes_total": rec["buffer_bytes_total"]},
+        "device_ms_per_step": rec["device_ms_per_step"],
+        "roofline": rec["roofline"],
+        "extras": rec.get("extras"),
     }
-    if not args.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(w)
-    if args.all:
+    if "cpu_baseline" in rec:
+        line["cpu_baseline"] = rec["cpu_baseline"]
+    if not args.only:
         others = {}
-        for name in sorted(MAKERS):
-            if name == args.workload or name.startswith("calib_"):
-                continue
-            del w
-            torch.cuda.empty_cache()
-            w = MAKERS[name](rt)
-            steps = 50 if name == "c5_matmul" else 200
-            wall, dev = time_steps(w.step, steps, 10, graph=False)
-            _, gdev = time_steps(w.step, steps, 2, graph=True)
-            v, u = value_of(w, wall)
-            others[name] = {"value": round(v, 2), "unit": u, "ms_per_step": round(wall, 6),
-                            "device_ms_per_step": round(dev, 6), "graph_device_ms_per_step": round(gdev, 6),
-                            "roofline": roofline(w, min(dev, gdev))}
+        names = [n for n in OTHER_CONFIGS + [HEADLINE] + (EXTRA_CONFIGS if args.extra else []) if n != args.workload]
+        for name in names:
+            steps = min(args.steps, 100) if name == "c5_matmul" else args.steps
+            _, r = measure(name, rt, steps, min(args.warmup, 10), args.rotate, cpu=not args.no_cpu)
+            others[name] = r
+            sys.stderr.write("bench.py: %s done at %.0f s\n" % (name, time.perf_counter() - t_start))
+            sys.stderr.flush()
         line["other_configs"] = others
     print(json.dumps(line), flush=True)
 

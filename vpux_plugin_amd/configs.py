@@ -3,7 +3,10 @@
 Each generator takes a `scale` divisor so that tests can run the same distribution at a smaller
 size; scale=1 is the full configuration.  fp16 tensors are returned as uint16 bit patterns produced
 with numpy's IEEE round-to-nearest-even (inputs never fall in the range where the reference's
-float16 rounding differs from IEEE)."""
+float16 rounding differs from IEEE).  Results are cached per argument set (callers must not
+modify the arrays): a benchmark that uploads several copies of a configuration generates it once."""
+import functools
+
 import numpy as np
 
 
@@ -11,6 +14,7 @@ def _f16_bits(x):
     return np.asarray(x, dtype=np.float32).astype(np.float16).view(np.uint16)
 
 
+@functools.lru_cache(maxsize=2)
 def c1_fake_quantize(seed=1, shape=(1, 64, 56, 56)):
     """FakeQuantize fp16 NCHW, per-tensor, 256 levels, limits +-4; x ~ N(0,1.5) clipped to [-6,6]."""
     rng = np.random.default_rng(seed)
@@ -20,6 +24,7 @@ def c1_fake_quantize(seed=1, shape=(1, 64, 56, 56)):
             "levels": 256}
 
 
+@functools.lru_cache(maxsize=2)
 def c2_softmax(seed=2, shape=(8, 16, 512, 512)):
     """Softmax over the last axis; logits ~ N(0,3), 5% of the entries set to -60000 (masking)."""
     rng = np.random.default_rng(seed)
@@ -29,6 +34,7 @@ def c2_softmax(seed=2, shape=(8, 16, 512, 512)):
     return {"x": _f16_bits(x), "axis": len(shape) - 1}
 
 
+@functools.lru_cache(maxsize=2)
 def c3_mvn(seed=3, shape=(4, 256, 64, 64)):
     """MVN across C,H,W, eps 1e-9 inside sqrt, normalize_variance; U(-8,8) + per-channel N(0,2)."""
     rng = np.random.default_rng(seed)
@@ -37,6 +43,7 @@ def c3_mvn(seed=3, shape=(4, 256, 64, 64)):
     return {"x": _f16_bits(x), "across_channels": True, "normalize_variance": True, "eps": 1e-9}
 
 
+@functools.lru_cache(maxsize=2)
 def c4_conv(seed=4, N=32, H=56, W=56, IC=64, OC=64):
     """3x3 s1 p1 conv, NHWC u8 input zp 128, i8 symmetric weights, i32 bias, per-OC multiplier in
     [2^14, 2^15) with shift 20..24, output zp 0, ReLU clamp [0,255]."""
@@ -51,6 +58,7 @@ def c4_conv(seed=4, N=32, H=56, W=56, IC=64, OC=64):
     }
 
 
+@functools.lru_cache(maxsize=2)
 def c5_matmul(seed=5, M=4096, K=4096, N=11008):
     """A [M,K] i8 zp 3, B [N,K] i8 per-column symmetric; PPE per-column mult in [2^14,2^15), shift 27..28
     (accumulator sigma ~3.5e5 * sqrt(K/4096) maps +-3 sigma onto the i8 range at K=4096), LeakyReLU 0.1
