@@ -197,6 +197,84 @@ def test_softmax_packed_params_golden(rt):
     assert (w[0] & 0xffffffff, w[1] & 0xffffffff) == (1, 3) and w[2] & 0xffffffff == 1
 
 
+def test_softmax_packed_params_describe_the_same_rows(rt):
+    """Whatever the packing drops or fuses, walking the packed levels must visit exactly the (input offset, output offset)
+    pairs of the original tensor, and the packed axis must group them into the original softmax rows."""
+    import itertools
+    rng = np.random.default_rng(77)
+    for case in range(300):
+        rank = int(rng.integers(1, 6))
+        dims = [int(rng.choice([1, 1, 2, 3, 4, 5])) for _ in range(rank)]
+        axis = int(rng.integers(0, rank))
+
+        def strides_for(gap_prob):
+            st, run = [], int(rng.choice([1, 1, 1, 2, 3]))
+            for d in dims:
+                st.append(run)
+                run *= d
+                if rng.random() < gap_prob:
+                    run *= int(rng.integers(2, 4))
+            return st
+        si, so = strides_for(0.3), strides_for(0.3 if case % 2 else 0.0)
+        pad = 0
+        w = [int(v) for v in rt.generate_softmax_attr(dims, si, so, axis, pad)]
+        p_axis, p_pad = w[0] & 0xffffffff, w[0] >> 32
+        mode, nd = w[1] & 0xffffffff, w[1] >> 32
+        assert nd >= 3 and len(w) == 2 + 2 * nd and p_pad == pad
+        pd = [v & 0xffffffff for v in w[2::2]]
+        assert pd == [v >> 32 for v in w[2::2]]
+        psi, pso = [v & 0xffffffff for v in w[3::2]], [v >> 32 for v in w[3::2]]
+
+        def rows(dd, a, s_in, s_out):
+            out = set()
+            others = [range(n) if k != a else [0] for k, n in enumerate(dd)]
+            for idx in itertools.product(*others):
+                base_i = sum(i * s for i, s in zip(idx, s_in))
+                base_o = sum(i * s for i, s in zip(idx, s_out))
+                out.add(tuple((base_i + k * s_in[a], base_o + k * s_out[a]) for k in range(dd[a])))
+            return out
+        assert rows(dims, axis, si, so) == rows(pd, p_axis, psi, pso), (dims, si, so, axis, w)
+        # variant selection: outer axis -> 3; inner axis -> 1, or 2 for packed rows of 2 or 4 values
+        if p_axis != 0:
+            assert mode == 3
+        else:
+            assert psi[0] == 1 and pso[0] == 1
+            tiny = pd[0] in (2, 4) and psi[1] == pd[0] and psi[2] == pso[2]
+            assert mode == (2 if tiny else 1)
+        # nothing left to fuse: above the axis no two real levels are gapless in both operands (unit levels are padding)
+        for k in range(p_axis + 1, nd - 1):
+            if pd[k + 1] != 1:
+                assert not (psi[k + 1] == psi[k] * pd[k] and pso[k + 1] == pso[k] * pd[k]), (dims, si, so, axis, w)
+
+
+def test_eltwise_approximation_properties(rt):
+    """The four integers must reproduce in_scale / out_scale for both inputs, fit their registers, and give both inputs
+    the same shift (that is what lets the datapath add before the output multiplier)."""
+    rng = np.random.default_rng(78)
+    for _ in range(400):
+        s1, s2, so = (float(np.exp(rng.uniform(np.log(2e-3), np.log(0.5)))) for _ in range(3))
+        try:
+            m1, m2, mo, sh = rt.eltwise_quantization_approximation(s1, s2, so)
+        except rt.VpxError:
+            continue
+        assert 0 <= m1 <= 65535 and 0 <= m2 <= 65535 and 0 < mo <= 32767 and 0 <= sh <= 63
+        for m, sc in ((m1, s1), (m2, s2)):
+            got = m * mo / 2.0 ** sh
+            # the smaller input's factor may have been shifted down: its relative error is bounded by one unit of that factor
+            assert abs(got - sc / so) <= (sc / so) * (2.0 ** -13 + 1.0 / max(m, 1)), (s1, s2, so, m1, m2, mo, sh)
+    # both scales negative: an add folds the sign into the output multiplier
+    m1, m2, mo, sh = rt.eltwise_quantization_approximation(-0.02, -0.03, 0.05)
+    p1, p2, po, ps = rt.eltwise_quantization_approximation(0.02, 0.03, 0.05)
+    # (a negative scale's multiplier is floored away from zero, so its magnitude may be one more)
+    assert 0 <= m1 - p1 <= 1 and 0 <= m2 - p2 <= 1 and (mo, sh) == (-po, ps)
+    # a multiply (type 2) folds a single negative sign
+    m1, m2, mo, sh = rt.eltwise_quantization_approximation(-0.02, 0.03, 0.05, 2)
+    assert 0 <= m1 - p1 <= 1 and m2 == p2 and (mo, sh) == (-po, ps)
+    # scales too far apart for either alignment are refused
+    with pytest.raises(rt.VpxError):
+        rt.eltwise_quantization_approximation(1e-12, 1e-12, 1e8)
+
+
 def test_softmax_first_form_axis_convention():
     g = GOLD["softmax_first_form"]
     nd = len(g["shape_nchw"])

@@ -116,43 +116,56 @@ int vpx_approximate(int bits, double target, int64_t* mult, int64_t* shift, int6
     return VPX_RESULT_SUCCESS;
 }
 
+// Two input scales and the inverse output scale as 15-bit multipliers with shifts, brought to the form the eltwise
+// datapath has: both inputs multiplied by 16-bit unsigned factors, one shared shift after the output multiplier
+// (quantization.cpp:455-516).  The two input shifts are equalised by scaling one factor: up to the larger shift when
+// the factor still fits 16 bits and the summed shift fits the 6-bit field, otherwise down to the smaller one.
 int vpx_eltwise_quantization_approximation(double in1_scale, double in2_scale, double out_scale, int eltwise_type,
                                            int64_t* in1_mult, int64_t* in2_mult, int64_t* out_mult, int64_t* out_shift) {
-    Approximation in1 = approximate(15, in1_scale), in2 = approximate(15, in2_scale), out = approximate(15, 1.0 / out_scale);
-    if (in1.postShift || in2.postShift || out.postShift)
-        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "eltwise approximation: postShift is not supported");
-    const int64_t minShift = std::min(in1.shift, in2.shift), maxShift = std::max(in1.shift, in2.shift);
-    const int64_t maxRegisterShift = 63;      // 6-bit shift register
-    const int64_t maxRegisterMult = 65535;    // unsigned 16-bit input multipliers
-    if (in1.mult < 0 || in2.mult < 0) {
-        const bool oneNegative = (in1.mult < 0) != (in2.mult < 0);
-        if (eltwise_type == 0 || eltwise_type == 1) {
-            if (oneNegative)
-                return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Unsupported case for ADD/SUB eltwise, just one negative scale %lld %lld.",
-                            (long long)in1.mult, (long long)in2.mult);
-            out.mult = -out.mult;
-        }
-        if (eltwise_type == 2 && oneNegative) out.mult = -out.mult;
-        in1.mult = (uint16_t)std::llabs(in1.mult);
-        in2.mult = (uint16_t)std::llabs(in2.mult);
+    if (!in1_mult || !in2_mult || !out_mult || !out_shift)
+        return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "eltwise approximation: null output");
+    constexpr int64_t kShiftFieldMax = (1 << 6) - 1;
+    constexpr int64_t kFactorMax = (1 << 16) - 1;
+    enum { kAdd = 0, kSubtract = 1, kMultiply = 2 };
+
+    const Approximation src[2] = {approximate(15, in1_scale), approximate(15, in2_scale)};
+    const Approximation dst = approximate(15, 1.0 / out_scale);
+    if (src[0].postShift || src[1].postShift || dst.postShift)
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "eltwise approximation: a scale needs a post-shift, which the datapath lacks");
+
+    // signs: the input factors are unsigned, so a negative pair is folded into the output multiplier
+    int64_t factor[2] = {src[0].mult, src[1].mult};
+    int64_t result_mult = dst.mult;
+    const int negatives = (factor[0] < 0) + (factor[1] < 0);
+    if (negatives) {
+        const bool sum_like = eltwise_type == kAdd || eltwise_type == kSubtract;
+        if (sum_like && negatives == 1)
+            return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                        "eltwise approximation: input multipliers %lld and %lld differ in sign, which an add / subtract cannot express",
+                        (long long)factor[0], (long long)factor[1]);
+        if (sum_like || (eltwise_type == kMultiply && negatives == 1)) result_mult = -result_mult;
+        for (int64_t& f : factor) f = (int64_t)(uint16_t)(f < 0 ? -f : f);
     }
-    const bool toMax = maxShift + out.shift <= maxRegisterShift && in1.mult <= (maxRegisterMult >> (maxShift - in1.shift)) &&
-                       in2.mult <= (maxRegisterMult >> (maxShift - in2.shift));
-    if (toMax) {
-        in1.mult = (uint16_t)(in1.mult << (maxShift - in1.shift));
-        in2.mult = (uint16_t)(in2.mult << (maxShift - in2.shift));
-        out.shift += maxShift;
-    } else if (minShift + out.shift < maxRegisterShift) {
-        in1.mult = (uint16_t)(in1.mult >> (in1.shift - minShift));
-        in2.mult = (uint16_t)(in2.mult >> (in2.shift - minShift));
-        out.shift += minShift;
+
+    const int64_t hi = std::max(src[0].shift, src[1].shift), lo = std::min(src[0].shift, src[1].shift);
+    bool up = hi + dst.shift <= kShiftFieldMax;
+    for (int k = 0; k < 2 && up; k++) up = factor[k] <= (kFactorMax >> (hi - src[k].shift));
+    int64_t common;
+    if (up) {
+        common = hi;
+        for (int k = 0; k < 2; k++) factor[k] = (int64_t)(uint16_t)(factor[k] << (hi - src[k].shift));
+    } else if (lo + dst.shift < kShiftFieldMax) {
+        common = lo;
+        for (int k = 0; k < 2; k++) factor[k] = (int64_t)(uint16_t)(factor[k] >> (src[k].shift - lo));
     } else {
-        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Elwise add input1_MULT/input2_MULT/output_SHIFT out of register range");
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "eltwise approximation: shifts %lld / %lld with output shift %lld do not fit the 6-bit shift field",
+                    (long long)src[0].shift, (long long)src[1].shift, (long long)dst.shift);
     }
-    *in1_mult = in1.mult;
-    *in2_mult = in2.mult;
-    *out_mult = out.mult;
-    *out_shift = out.shift;
+    *in1_mult = factor[0];
+    *in2_mult = factor[1];
+    *out_mult = result_mult;
+    *out_shift = dst.shift + common;
     return VPX_RESULT_SUCCESS;
 }
 
@@ -267,79 +280,56 @@ int vpx_retrieve_ppe_int(int post_op, double param0, double param1, const vpx_qu
     }
 }
 
-int vpx_generate_softmax_attr(uint32_t ndims_in, const int64_t* dims, const int64_t* in_strides_, const int64_t* out_strides_,
+// Packed softmax parameters (update_sw_kernel_params.cpp:36-147): the tensor is reduced to the fewest (size, input
+// stride, output stride) levels that still describe it, innermost first, and the kernel variant is chosen from them.
+int vpx_generate_softmax_attr(uint32_t rank, const int64_t* dims, const int64_t* in_strides, const int64_t* out_strides,
                               int64_t axis, int64_t pad_size, uint64_t* words, uint32_t* n_words) {
-    if (!dims || !in_strides_ || !out_strides_ || !words || !n_words)
-        return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "generateVpuipSoftmaxAttr: null argument");
-    if (ndims_in < 1 || ndims_in > VPX_MAX_ND_DIMS || axis < 0 || axis >= (int64_t)ndims_in)
-        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "generateVpuipSoftmaxAttr: axis %lld outside rank %u", (long long)axis, ndims_in);
-    constexpr int MAXD = VPX_MAX_ND_DIMS + 1;
-    int64_t inDims[MAXD] = {}, inStrides[MAXD] = {}, outStrides[MAXD] = {};
-    int ndims = (int)ndims_in;
-    for (int i = 0; i < ndims; i++) {
-        inDims[i] = dims[i];
-        inStrides[i] = in_strides_[i];
-        outStrides[i] = out_strides_[i];
+    if (!dims || !in_strides || !out_strides || !words || !n_words)
+        return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "softmax parameters: null argument");
+    if (rank < 1 || rank > VPX_MAX_ND_DIMS || axis < 0 || axis >= (int64_t)rank)
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "softmax parameters: axis %lld outside rank %u", (long long)axis, rank);
+    struct Level {
+        int64_t size, in_step, out_step;
+        bool reduced;  // the softmax axis
+    };
+    // 1. levels of size one say nothing, except the axis itself
+    std::vector<Level> kept;
+    for (uint32_t d = 0; d < rank; d++)
+        if (dims[d] != 1 || (int64_t)d == axis) kept.push_back(Level{dims[d], in_strides[d], out_strides[d], (int64_t)d == axis});
+    // 2. above the axis, neighbours that both operands walk without a gap become one level
+    size_t axis_at = 0;
+    while (!kept[axis_at].reduced) axis_at++;
+    std::vector<Level> levels(kept.begin(), kept.begin() + (std::ptrdiff_t)axis_at + 1);
+    for (size_t d = axis_at + 1; d < kept.size(); d++) {
+        const Level& below = kept[d - 1];
+        const bool gapless = kept[d].in_step == below.in_step * below.size && kept[d].out_step == below.out_step * below.size;
+        if (d >= axis_at + 2 && gapless)
+            levels.back().size *= kept[d].size;
+        else
+            levels.push_back(kept[d]);
     }
-    // unit dimensions other than the axis carry no information
-    for (int i = ndims - 1; i >= 0; i--) {
-        if (ndims <= 1) break;
-        if (inDims[i] == 1 && axis != i) {
-            for (int j = i; j < ndims - 1; j++) {
-                inDims[j] = inDims[j + 1];
-                inStrides[j] = inStrides[j + 1];
-                outStrides[j] = outStrides[j + 1];
-            }
-            if (axis > i) axis--;
-            ndims--;
-        }
+    // 3. an innermost axis that is not unit-stride is served as an outer axis over an inner level of one element
+    if (axis_at == 0 && (levels[0].in_step > 1 || levels[0].out_step > 1)) {
+        levels.insert(levels.begin(), Level{1, levels[0].in_step, levels[0].out_step, false});
+        axis_at = 1;
     }
-    // dimensions outer to the axis merge when both stride sets are contiguous across them
-    for (int i = ndims - 2; i > axis; i--) {
-        if (inStrides[i + 1] == inStrides[i] * inDims[i] && outStrides[i + 1] == outStrides[i] * inDims[i]) {
-            inDims[i] = inDims[i + 1] * inDims[i];
-            for (int j = i + 1; j < ndims - 1; j++) {
-                inDims[j] = inDims[j + 1];
-                inStrides[j] = inStrides[j + 1];
-                outStrides[j] = outStrides[j + 1];
-            }
-            ndims--;
-        }
+    // 4. the kernel wants at least three levels: unit levels stacked on the outermost one
+    const Level top = levels.back();
+    while (levels.size() < 3) levels.push_back(Level{1, top.in_step * top.size, top.out_step * top.size, false});
+
+    int64_t mode = VPX_SOFTMAX_OUTER;
+    if (axis_at == 0) {
+        const bool tiny_rows = (levels[0].size == 2 || levels[0].size == 4) && pad_size == 0 && levels[1].in_step == levels[0].size &&
+                               levels[2].in_step == levels[2].out_step;
+        mode = tiny_rows ? VPX_SOFTMAX_INNER_HARDCODED : VPX_SOFTMAX_INNER;
     }
-    // a strided innermost axis is handled as an outer axis over a unit inner dimension
-    if (axis == 0 && (inStrides[0] > 1 || outStrides[0] > 1)) {
-        for (int i = ndims; i >= 1; i--) {
-            inDims[i] = inDims[i - 1];
-            inStrides[i] = inStrides[i - 1];
-            outStrides[i] = outStrides[i - 1];
-        }
-        inDims[0] = 1;
-        ndims++;
-        axis = 1;
-    }
-    if (ndims < 3) {
-        for (int i = ndims; i < 3; i++) {
-            inStrides[i] = inStrides[ndims - 1] * inDims[ndims - 1];
-            outStrides[i] = outStrides[ndims - 1] * inDims[ndims - 1];
-            inDims[i] = 1;
-        }
-        ndims = 3;
-    }
-    int64_t mode;
-    if (axis == 0) {
-        const bool hardcoded = (inDims[0] == 2 || inDims[0] == 4) && pad_size == 0 && inStrides[2] == outStrides[2] &&
-                               inDims[0] == inStrides[1];
-        mode = hardcoded ? VPX_SOFTMAX_INNER_HARDCODED : VPX_SOFTMAX_INNER;
-    } else {
-        mode = VPX_SOFTMAX_OUTER;
-    }
-    auto pack = [](int64_t lo, int64_t hi) { return ((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo; };
+    const auto two_i32 = [](int64_t lo, int64_t hi) { return ((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo; };
     uint32_t n = 0;
-    words[n++] = pack(axis, pad_size);
-    words[n++] = pack(mode, ndims);
-    for (int i = 0; i < ndims; i++) {
-        words[n++] = pack(inDims[i], inDims[i]);
-        words[n++] = pack(inStrides[i], outStrides[i]);
+    words[n++] = two_i32((int64_t)axis_at, pad_size);
+    words[n++] = two_i32(mode, (int64_t)levels.size());
+    for (const Level& l : levels) {
+        words[n++] = two_i32(l.size, l.size);
+        words[n++] = two_i32(l.in_step, l.out_step);
     }
     *n_words = n;
     return VPX_RESULT_SUCCESS;
