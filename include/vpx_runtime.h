@@ -27,7 +27,11 @@ extern "C" {
 #define VPX_API
 #endif
 
-/* Same numeric values as vcl_result_t (npu_driver_compiler.h:94-103). */
+/* SUCCESS, OUT_OF_MEMORY, INVALID_ARGUMENT, INVALID_NULL_HANDLE and UNKNOWN carry the numeric values of the
+ * vcl_result_t members of the same name (npu_driver_compiler.h:94-103).  UNSUPPORTED_FEATURE is this library's
+ * own (vcl_result_t has no such member; the value is the one Level Zero gives ZE_RESULT_ERROR_UNSUPPORTED_FEATURE,
+ * the family vcl_result_t's numbering follows).  VCL_RESULT_ERROR_IO and VCL_RESULT_ERROR_INVALID_IR have no use
+ * here (no file or IR handling) and are not mirrored. */
 typedef enum vpx_result_t {
     VPX_RESULT_SUCCESS = 0,
     VPX_RESULT_ERROR_OUT_OF_MEMORY = 0x70000002,
@@ -99,6 +103,15 @@ VPX_API const char* vpx_sw_kernel_name(uint32_t i);
  * expand_dpu_config_invariant_ppe.cpp:322-380): t = (acc + bias) * mult; if t < 0 then
  * t *= prelu_mult and shift += prelu_shift; r = round_half_even(t / 2^shift) + zp_out;
  * clamp to [clamp_low, clamp_high]; saturate to the output type.
+ *
+ * output_type VPX_NN_FP16 (CONV tasks; "INT32 s17.15 fixed-point convert to FP16",
+ * src/vpux_compiler/src/dialect/VPUMI37XX/ops/external/runtime_dpu_parser_imports.cpp.inc:546-574): the same
+ * pipeline with the round stage keeping 15 fractional bits, fx = round_half_even(t / 2^(shift - 15)) saturated to
+ * 32 bits; the output is fx * 2^-15 narrowed to fp16 with one round-to-nearest-even (infinity from 65520 up).
+ * The weight table then holds mult / shift of w_scale * in_scale (no output scale, nce_sparsity.cpp:112-126),
+ * zp_out must be 0, clamp_low is not used and clamp_high packs two fp16 bounds as 0xllllhhhh
+ * (include/vpux/compiler/dialect/VPU/utils/ppe_utils.hpp:36-87; INT32_MAX = no clamp), as
+ * vpx_retrieve_ppe_int produces them for a float output.
  * ------------------------------------------------------------------------------------------ */
 
 /* VPUIP::NCETaskType (tblgen/.../VPUIP/attributes.td:56-70) */
@@ -139,7 +152,7 @@ typedef struct vpx_nce_task_t {
     void* output;
     int32_t input_type;   /* VPX_NN_U8 or VPX_NN_I8 */
     int32_t weights_type; /* VPX_NN_U8 or VPX_NN_I8 */
-    int32_t output_type;  /* VPX_NN_U8 or VPX_NN_I8 */
+    int32_t output_type;  /* VPX_NN_U8, VPX_NN_I8, or VPX_NN_FP16 (CONV tasks) */
     int64_t N, H, W, IC;  /* input shape */
     int64_t OC;
     int32_t kernel_size[2];    /* KY, KX */
@@ -151,6 +164,13 @@ typedef struct vpx_nce_task_t {
 } vpx_nce_task_t;
 
 VPX_API int vpx_nce_task(const vpx_nce_task_t* task, void* stream);
+
+/* Testing and tuning hook (no counterpart in the reference): overrides how vpx_nce_task picks its device kernel.
+ * `knob` is one of "VPX_NCE_KERNEL" (naive | gather | conv), "VPX_GEMM_TILE" (128 | 256), "VPX_GEMM_WAVES" (4 | 8),
+ * "VPX_CONV_KERNEL" (stream), "VPX_CONV_ROWS" (n), "VPX_CONV_WAVES" (4 | 8); `value` NULL or "" restores the default.
+ * Environment variables of the same names give the initial values; they are read once, at the first NCE task or the
+ * first call of this function, never during a launch.  Process-wide; results do not depend on any of them. */
+VPX_API int vpx_set_tuning(const char* knob, const char* value);
 
 /* Name of the device kernel the last successful vpx_nce_task on this thread dispatched to
  * ("" before the first); for tests and profiles. */

@@ -364,8 +364,23 @@ def ppe_requant(acc, bias, mult, shift, p):
     return lib().orc_ppe_requant(C.c_int32(acc), C.c_int32(bias), C.c_int32(mult), C.c_int32(shift), C.byref(p))
 
 
+def ppe_requant_f16(acc, bias, mult, shift, p):
+    """fp16 bit pattern of the s17.15 fixed-point output path."""
+    fn = lib().orc_ppe_requant_f16
+    fn.restype = C.c_uint16
+    return fn(C.c_int32(acc), C.c_int32(bias), C.c_int32(mult), C.c_int32(shift), C.byref(p))
+
+
+def pack_clamp_f16(lo, hi):
+    """Two fp16 bounds in one int32 as the compiler packs them for a float output: 0xllllhhhh built by adding the
+    sign-extended 16-bit patterns (ppe_utils.hpp:57-73)."""
+    lo_b, hi_b = (int(np.array([v], dtype=np.float32).astype(np.float16).view(np.int16)[0]) for v in (lo, hi))
+    v = ((lo_b << 16) + hi_b) & 0xffffffff
+    return v - (1 << 32) if v & 0x80000000 else v
+
+
 def nce_conv(inp, w, wt, p, zp_in=0, zp_w=0, strides=(1, 1), pads=(0, 0, 0, 0), out_signed=False, rows=None,
-             want_acc=False):
+             want_acc=False, out_f16=False):
     """inp NHWC int8/uint8, w [OC,KY,KX,IC] int8/uint8, wt [OC,4] int32; pads = (top,left,bottom,right).
 
     rows=(row0,nrows) computes only those flattened output rows (the rest of the result is zero)."""
@@ -376,10 +391,10 @@ def nce_conv(inp, w, wt, p, zp_in=0, zp_w=0, strides=(1, 1), pads=(0, 0, 0, 0), 
     OC, KY, KX, IC2 = w.shape
     assert IC == IC2
     d = _Conv(N, H, W, IC, OC, KY, KX, strides[0], strides[1], pads[0], pads[1], pads[2], pads[3],
-              int(inp.dtype == np.int8), int(w.dtype == np.int8), int(out_signed), zp_in, zp_w, p)
+              int(inp.dtype == np.int8), int(w.dtype == np.int8), 2 if out_f16 else int(out_signed), zp_in, zp_w, p)
     OH = (H + pads[0] + pads[2] - KY) // strides[0] + 1
     OW = (W + pads[1] + pads[3] - KX) // strides[1] + 1
-    out = np.zeros((N, OH, OW, OC), dtype=np.int8 if out_signed else np.uint8)
+    out = np.zeros((N, OH, OW, OC), dtype=np.uint16 if out_f16 else (np.int8 if out_signed else np.uint8))
     acc = np.zeros((N, OH, OW, OC), dtype=np.int32) if want_acc else None
     row0, nrows = rows if rows is not None else (0, N * OH * OW)
     lib().orc_nce_conv_rows(C.byref(d), _p(inp), _p(w), _p(wt), _p(out), _p(acc) if want_acc else None,
@@ -400,13 +415,13 @@ def nce_eltwise(a, b, p, zp_a, zp_b, mult_a, mult_b, out_mult, out_shift, subtra
     return out
 
 
-def nce_matmul(a, b_nk, wt, p, zp_a=0, zp_b=0, out_signed=True, rows=None, want_acc=False):
+def nce_matmul(a, b_nk, wt, p, zp_a=0, zp_b=0, out_signed=True, rows=None, want_acc=False, out_f16=False):
     """A [M,K] x B stored [N,K] -> [M,N]: the 1x1-convolution form NCE.MatMul lowers to (ops.td:228-357)."""
     M, K = a.shape
     Nn, K2 = b_nk.shape
     assert K == K2
     r = nce_conv(a.reshape(1, M, 1, K), b_nk.reshape(Nn, 1, 1, K), wt, p, zp_in=zp_a, zp_w=zp_b,
-                 out_signed=out_signed, rows=rows, want_acc=want_acc)
+                 out_signed=out_signed, rows=rows, want_acc=want_acc, out_f16=out_f16)
     if want_acc:
         return r[0].reshape(M, Nn), r[1].reshape(M, Nn)
     return r.reshape(M, Nn)

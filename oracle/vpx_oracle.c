@@ -427,6 +427,74 @@ int32_t orc_ppe_requant(int32_t acc, int32_t bias, int32_t mult, int32_t shift, 
     return (int32_t)r;
 }
 
+/* fp16 output of an integer convolution: "INT32 s17.15 fixed-point convert to FP16"
+ * (runtime_dpu_parser_imports.cpp.inc:546-552, ppe_i32_convert = 1).  The pipeline is the same up to
+ * the round stage, which here keeps 15 fractional bits: fx = round_half_even(t / 2^(s - 15)) saturated
+ * to 32 bits is the s17.15 number, fx * 2^-15 is narrowed to fp16 with one round-to-nearest-even
+ * (65520 and above become infinity), and the clamp is the pair of fp16 bounds the compiler packs into
+ * clamp_high as 0xllllhhhh (dialect/VPU/utils/ppe_utils.hpp:36-87; clamp_low is ignored by that
+ * convention and 0x7fffffff, whose halves are not numbers, means no clamp).  No zero point is added
+ * (setupQuantInFloatOut programs none).  "parity unpinned" against silicon like orc_ppe_requant. */
+static uint16_t s1715_to_f16(int64_t fx) {
+    const uint16_t sign = fx < 0 ? 0x8000u : 0u;
+    uint64_t a = (uint64_t)(fx < 0 ? -fx : fx); /* value = a * 2^-15 */
+    if (a == 0) return sign;
+    int top = 63;
+    while (!((a >> top) & 1u)) top--; /* a in [2^top, 2^(top+1)) : value in [2^(top-15), ...) */
+    int e = top - 15;                 /* unbiased exponent of the value */
+    int drop;                         /* low bits of a that do not fit the significand */
+    if (e < -14) {                    /* subnormal half: quantum 2^-24 = a-units of 2^-9; nothing is dropped */
+        return (uint16_t)(sign | (uint16_t)(a << 9));
+    }
+    drop = top - 10;
+    uint64_t q = a, rem = 0, half = 0;
+    if (drop > 0) {
+        q = a >> drop;
+        rem = a & ((1ull << drop) - 1ull);
+        half = 1ull << (drop - 1);
+        if (rem > half || (rem == half && (q & 1ull))) q++;
+        if (q == (1ull << 11)) { /* carried into the next binade */
+            q >>= 1;
+            e++;
+        }
+    } else {
+        q = a << (-drop);
+    }
+    if (e > 15) return (uint16_t)(sign | 0x7c00u);
+    return (uint16_t)(sign | (uint16_t)((e + 15) << 10) | (uint16_t)(q & 0x3ffu));
+}
+
+uint16_t orc_ppe_requant_f16(int32_t acc, int32_t bias, int32_t mult, int32_t shift, const orc_ppe_t* ppe) {
+    const int32_t biased = (int32_t)((uint32_t)acc + (uint32_t)bias);
+    int64_t t = (int64_t)biased * (int64_t)mult;
+    int s = shift;
+    if (t < 0) {
+        t *= (int64_t)ppe->prelu_mult;
+        s += ppe->prelu_shift;
+    }
+    s -= 15;
+    int64_t fx;
+    if (s >= 0) {
+        fx = shift_round_half_even(t, s);
+    } else {
+        const int up = -s; /* at most 15: |t| < 2^58 may overflow 64 bits only when it saturates anyway */
+        if (t > (INT64_MAX >> up)) fx = INT64_MAX;
+        else if (t < -(INT64_MAX >> up)) fx = -INT64_MAX;
+        else fx = t * ((int64_t)1 << up);
+    }
+    if (fx > INT32_MAX) fx = INT32_MAX;
+    if (fx < INT32_MIN) fx = INT32_MIN;
+    uint16_t h = s1715_to_f16(fx);
+    if (ppe->clamp_high != INT32_MAX) {
+        const uint16_t hi = (uint16_t)((uint32_t)ppe->clamp_high & 0xffffu);
+        const uint16_t lo = (uint16_t)(((uint32_t)ppe->clamp_high >> 16) & 0xffffu);
+        const float v = orc_f16_to_f32(h);
+        if ((lo & 0x7fffu) <= 0x7c00u && v < orc_f16_to_f32(lo)) h = lo;
+        if ((hi & 0x7fffu) <= 0x7c00u && v > orc_f16_to_f32(hi)) h = hi;
+    }
+    return h;
+}
+
 /* ------------------------------------------------------------------ NCE conv / matmul */
 
 static inline int32_t load8(const void* p, int64_t i, int is_signed) {
@@ -477,8 +545,12 @@ void orc_nce_conv_rows(const orc_conv_t* d, const void* in, const void* w, const
             }
             int32_t mult, shift;
             orc_wt_unpack_scale(wt[oc * 4 + 2], &mult, &shift);
-            const int32_t r = orc_ppe_requant(acc, wt[oc * 4 + 3], mult, shift, &d->ppe);
             if (acc_out) acc_out[row * OC + oc] = acc;
+            if (d->out_signed == 2) { /* fp16 output */
+                ((uint16_t*)out)[row * OC + oc] = orc_ppe_requant_f16(acc, wt[oc * 4 + 3], mult, shift, &d->ppe);
+                continue;
+            }
+            const int32_t r = orc_ppe_requant(acc, wt[oc * 4 + 3], mult, shift, &d->ppe);
             /* convert: saturate to the storage type */
             if (d->out_signed)
                 ((int8_t*)out)[row * OC + oc] = (int8_t)(r < -128 ? -128 : (r > 127 ? 127 : r));

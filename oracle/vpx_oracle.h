@@ -110,6 +110,10 @@ typedef struct {
     int32_t clamp_high;
 } orc_ppe_t;
 int32_t orc_ppe_requant(int32_t acc, int32_t bias, int32_t mult, int32_t shift, const orc_ppe_t* ppe);
+/* fp16 output (s17.15 fixed point converted to fp16, runtime_dpu_parser_imports.cpp.inc:546-574): returns the bit
+ * pattern; zp_out is not used, clamp_low is ignored and clamp_high holds two fp16 bounds as 0xllllhhhh
+ * (ppe_utils.hpp:36-87), INT32_MAX meaning none */
+uint16_t orc_ppe_requant_f16(int32_t acc, int32_t bias, int32_t mult, int32_t shift, const orc_ppe_t* ppe);
 
 /* ---- NCE convolution / matmul (VPU.NCE.Convolution ops.td:138-226, NCE.MatMul :228-357) ----
  * in  : NHWC [N][H][W][IC] 8-bit (signed flag), zero point zp_in
@@ -119,7 +123,7 @@ int32_t orc_ppe_requant(int32_t acc, int32_t bias, int32_t mult, int32_t shift, 
 typedef struct {
     int64_t N, H, W, IC, OC, KY, KX;
     int64_t stride_y, stride_x, pad_top, pad_left, pad_bottom, pad_right;
-    int32_t in_signed, w_signed, out_signed;
+    int32_t in_signed, w_signed, out_signed; /* out_signed: 0 = u8, 1 = i8, 2 = fp16 (16-bit output elements) */
     int32_t zp_in, zp_w;
     orc_ppe_t ppe;
 } orc_conv_t;

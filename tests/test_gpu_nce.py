@@ -14,7 +14,7 @@ def dev_t(a, dev):
 
 
 def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0, zp_out=0, strides=(1, 1),
-             pads=(0, 0, 0, 0), out_signed=False, mode=None, force=None, rows=None):
+             pads=(0, 0, 0, 0), out_signed=False, mode=None, force=None, rows=None, out_f16=False):
     """pads = (left, right, top, bottom).  Returns (gpu_out, oracle_out, kernel_name)."""
     import torch
     OC, KY, KX, IC = w.shape
@@ -28,24 +28,22 @@ def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0,
     N, H, W, _ = inp.shape
     OH = (H + pads[2] + pads[3] - KY) // strides[0] + 1
     OW = (W + pads[0] + pads[1] - KX) // strides[1] + 1
-    out = torch.full((N, OH, OW, OC), 77, dtype=torch.int8 if out_signed else torch.uint8, device=dev)
-    old = os.environ.pop("VPX_NCE_KERNEL", None)
+    out = torch.full((N, OH, OW, OC), 77, dtype=torch.float16 if out_f16 else (torch.int8 if out_signed else torch.uint8), device=dev)
     if force == "stream":  # start the choice of LDS-patch kernel below the fastest one
-        os.environ["VPX_CONV_KERNEL"] = force
+        rt.set_tuning("VPX_CONV_KERNEL", force)
     elif force:
-        os.environ["VPX_NCE_KERNEL"] = force
+        rt.set_tuning("VPX_NCE_KERNEL", force)
     try:
         rt.nce_task(dev_t(inp, dev), dev_t(w, dev), dev_t(wt, dev), out, p, zp_in=zp_in, zp_w=zp_w, zp_out=zp_out,
                     strides=strides, pads=pads)
         torch.cuda.synchronize()
     finally:
-        os.environ.pop("VPX_NCE_KERNEL", None)
-        os.environ.pop("VPX_CONV_KERNEL", None)
-        if old is not None:
-            os.environ["VPX_NCE_KERNEL"] = old
+        rt.set_tuning("VPX_NCE_KERNEL", None)
+        rt.set_tuning("VPX_CONV_KERNEL", None)
     want = orc.nce_conv(inp, w, wt, op, zp_in=zp_in, zp_w=zp_w, strides=strides,
-                        pads=(pads[2], pads[0], pads[3], pads[1]), out_signed=out_signed, rows=rows)
-    return out.cpu().numpy(), want, rt.nce_last_kernel()
+                        pads=(pads[2], pads[0], pads[3], pads[1]), out_signed=out_signed, rows=rows, out_f16=out_f16)
+    got = out.cpu().numpy()
+    return (got.view(np.uint16) if out_f16 else got), want, rt.nce_last_kernel()
 
 
 def rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=True, w_u8=False, shift_lo=12, shift_hi=20):
@@ -100,12 +98,12 @@ def test_conv_patch_tile_heights(rt, orc, dev, rows, force, kernel):
     """Both LDS-patch kernels with the tile height forced: tiles that end past the last output row, one-row tiles."""
     rng = np.random.default_rng(55 + rows)
     inp, w, mults, shifts, bias = rand_case(rng, 2, 13, 24, 64, 80, 3, 3)
-    os.environ["VPX_CONV_ROWS"] = str(rows)
+    rt.set_tuning("VPX_CONV_ROWS", rows)
     try:
         got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, U8, zp_in=121, zp_out=3,
                                    strides=(1, 1), pads=(1, 1, 1, 1), force=force)
     finally:
-        del os.environ["VPX_CONV_ROWS"]
+        rt.set_tuning("VPX_CONV_ROWS", None)
     assert name == kernel
     assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
 
@@ -236,12 +234,14 @@ def test_conv_random_geometries(rt, orc, dev, seed, weight_zp):
 
 
 @pytest.fixture(params=[("8", "256"), ("4", "256"), ("4", "128")], ids=["8w256", "4w256", "4w128"])
-def gemm_waves(request):
+def gemm_waves(request, rt):
     """The shapes of the matmul kernel: 256 x 256 tiles with two waves per SIMD (128 x 64 each) or one (128 x 128), and
     128 x 128 tiles (four waves of 64 x 64), which small problems select by themselves."""
-    os.environ["VPX_GEMM_WAVES"], os.environ["VPX_GEMM_TILE"] = request.param
+    rt.set_tuning("VPX_GEMM_WAVES", request.param[0])
+    rt.set_tuning("VPX_GEMM_TILE", request.param[1])
     yield request.param
-    del os.environ["VPX_GEMM_WAVES"], os.environ["VPX_GEMM_TILE"]
+    rt.set_tuning("VPX_GEMM_WAVES", None)
+    rt.set_tuning("VPX_GEMM_TILE", None)
 
 
 @pytest.mark.parametrize("M,K,N", [(256, 64, 256), (300, 128, 520), (1, 64, 1), (513, 256, 77), (1024, 512, 768)])
@@ -278,6 +278,69 @@ def test_ppe_modes_and_rounding_edges(rt, orc, dev, mode):
     assert got.min() >= -100 and got.max() <= 90
 
 
+F16_NONE = {"clamp_low": -(2 ** 31), "clamp_high": 2 ** 31 - 1}
+
+
+@pytest.mark.parametrize("mode", ["NOOP", "LPRELU", "LRELU", "LRELUX"])
+@pytest.mark.parametrize("geom,kernel,force", [
+    (dict(N=1, H=700, W=1, IC=128, OC=520, KY=1, KX=1), "nce_gemm_mfma", "tile256"),     # 256 x 256 tiles, ragged edges
+    (dict(N=1, H=130, W=1, IC=64, OC=200, KY=1, KX=1), "nce_gemm_mfma", None),           # 128 x 128 tiles
+    (dict(N=2, H=9, W=11, IC=64, OC=70, KY=3, KX=3), "nce_conv_mfma", None),             # convolution: gather kernel
+    (dict(N=1, H=10, W=12, IC=48, OC=40, KY=3, KX=3), "nce_conv_mfma16", None),
+    (dict(N=2, H=6, W=7, IC=5, OC=9, KY=3, KX=2), "nce_conv_naive", None),
+    (dict(N=1, H=40, W=1, IC=64, OC=96, KY=1, KX=1), "nce_conv_naive", "naive"),
+])
+def test_f16_output_s1715_path(rt, orc, dev, geom, kernel, force, mode):
+    """fp16 output of an integer convolution / matmul ("INT32 s17.15 fixed-point convert to FP16"): bit-exact against the
+    oracle on every kernel that serves it.  Parity unpinned against silicon, like the integer PPE."""
+    rng = np.random.default_rng(300 + geom["H"])
+    conv = geom["KY"] > 1
+    pads, strides = ((1, 1, 1, 1) if conv else (0, 0, 0, 0)), (1, 1)
+    md = getattr(rt, "PPE_" + mode)
+    for in_u8, zp_in, zp_w, shift_lo, shift_hi in ((True, 128, 0, 14, 24), (False, -4, 0, 8, 30), (True, 9, 3, 16, 22)):
+        if zp_w and geom["IC"] % 16:
+            zp_w = 0
+        inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, shift_lo=shift_lo, shift_hi=shift_hi, **geom)
+        kw = dict(F16_NONE, lrelu_mult=1638, lrelu_shift=14)
+        if mode == "LRELUX":
+            kw["clamp_high"] = orc.pack_clamp_f16(0.0, 6.0)
+        if force == "tile256":
+            rt.set_tuning("VPX_GEMM_TILE", 256)
+        try:
+            got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, strides=strides,
+                                       pads=pads, mode=md, force=None if force == "tile256" else force, out_f16=True)
+        finally:
+            rt.set_tuning("VPX_GEMM_TILE", None)
+        assert name == kernel
+        assert np.array_equal(got, want), "%s %s zp_in=%d: %d mismatches" % (name, mode, zp_in, int((got != want).sum()))
+        vals = got.view(np.float16).astype(np.float32)
+        if mode in ("LRELU", "LRELUX"):
+            assert vals.min() >= 0.0
+        if mode == "LRELUX":
+            assert vals.max() <= 6.0 and (vals == 6.0).any()
+
+
+def test_f16_output_scale_is_weight_scale_times_input_scale(rt, orc, dev):
+    """With the weight table built for a float output (no output scale) the result is the real-valued convolution:
+    sum (q_in - zp) * s_in * q_w * s_w, within the 15-bit multiplier's and fp16's precision."""
+    import torch
+    rng = np.random.default_rng(311)
+    M, K, N = 64, 128, 192
+    a = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    b = rng.integers(-127, 128, (N, K)).astype(np.int8)
+    s_in, zp = 0.02, 128
+    s_w = np.exp(rng.uniform(np.log(1e-3), np.log(2e-2), N))
+    wt = rt.get_weights_table(s_in, 1.0, s_w, None, N, weights_ptr_step=K)
+    out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    rt.nce_matmul(dev_t(a, dev), dev_t(b, dev), dev_t(wt, dev), out, rt.retrieve_ppe_int(rt.POSTOP_NONE, None), zp_a=zp)
+    torch.cuda.synchronize()
+    real = ((a.astype(np.float64) - zp) * s_in) @ (b.astype(np.float64) * s_w[:, None]).T
+    got = out.cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(got - real) <= np.abs(real) * (2.0 ** -10 + 2.0 ** -13) + 2.0 ** -14)
+    want = orc.nce_matmul(a, b, wt, orc.ppe(1, 0, 0, -(2 ** 31), 2 ** 31 - 1), zp_a=zp, out_f16=True)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want)
+
+
 def test_conv_config_c4_full_size(rt, orc, dev):
     from vpux_plugin_amd import configs
     c = configs.c4_conv()
@@ -290,10 +353,18 @@ def test_conv_config_c4_full_size(rt, orc, dev):
 
 
 def test_matmul_config_c5_full_size_and_chain(rt, orc, dev):
-    """Full [4096x4096]x[4096x11008]: the MFMA result is compared bit for bit with the naive device path
-    over the whole tensor and with the CPU oracle on sampled rows; then Dequantize and the fp16 Add."""
+    """Full [4096x4096]x[4096x11008]: the MFMA result is compared bit for bit with the CPU oracle over the whole
+    tensor (run here, all host threads), with the committed checksums of the oracle's result
+    (tests/golden/c5_matmul_checksum.json, written by tests/golden/make_c5_checksum.py) and with the naive device
+    path; then Dequantize and the fp16 Add, likewise over the whole tensors."""
+    import hashlib
+    import json
     import torch
     from vpux_plugin_amd import configs
+    here = os.path.dirname(os.path.abspath(__file__))
+    with open(os.path.join(here, "golden", "c5_matmul_checksum.json")) as f:
+        gold = json.load(f)
+    sha = lambda arr: hashlib.sha256(np.ascontiguousarray(arr).tobytes()).hexdigest()
     c = configs.c5_matmul()
     M, K = c["a"].shape
     N = c["b_nk"].shape[0]
@@ -304,19 +375,25 @@ def test_matmul_config_c5_full_size_and_chain(rt, orc, dev):
     rt.nce_matmul(a, b, wtd, out, p, zp_a=c["zp_a"], zp_out=c["zp_out"])
     assert rt.nce_last_kernel() == "nce_gemm_mfma"
     out2 = torch.empty_like(out)
-    os.environ["VPX_NCE_KERNEL"] = "naive"
+    rt.set_tuning("VPX_NCE_KERNEL", "naive")
     try:
         rt.nce_matmul(a, b, wtd, out2, p, zp_a=c["zp_a"], zp_out=c["zp_out"])
         assert rt.nce_last_kernel() == "nce_conv_naive"
     finally:
-        del os.environ["VPX_NCE_KERNEL"]
+        rt.set_tuning("VPX_NCE_KERNEL", None)
     torch.cuda.synchronize()
     assert bool((out == out2).all())
-    rows = np.sort(np.random.default_rng(90).choice(M, 24, replace=False))
-    op = orc.ppe(c["lrelu_mult"], c["lrelu_shift"], c["zp_out"], *c["clamp"])
-    want = orc.nce_matmul(np.ascontiguousarray(c["a"][rows]), c["b_nk"], wt, op, zp_a=c["zp_a"])
     got = out.cpu().numpy()
-    assert np.array_equal(got[rows], want)
+    # committed checksums of the oracle's full result: the bytes, and row / column sums that localise a difference
+    g = gold["matmul_i8"]
+    assert int(got.astype(np.int64).sum()) == g["sum"]
+    assert sha(got.astype(np.int64).sum(axis=1)) == g["row_sums_sha256"]
+    assert sha(got.astype(np.int64).sum(axis=0)) == g["col_sums_sha256"]
+    assert sha(got) == g["sha256"]
+    # the oracle itself, whole tensor
+    op = orc.ppe(c["lrelu_mult"], c["lrelu_shift"], c["zp_out"], *c["clamp"])
+    want = orc.nce_matmul(c["a"], c["b_nk"], wt, op, zp_a=c["zp_a"])
+    assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
     hist = np.bincount(got.astype(np.int64).ravel() + 128, minlength=256)
     assert hist[0] / got.size < 0.05 and hist[255] / got.size < 0.05 and (hist > 0).sum() > 100  # spans i8
     # C5 chain: Dequantize to fp16, then fp16 Add of the residual
@@ -327,14 +404,12 @@ def test_matmul_config_c5_full_size_and_chain(rt, orc, dev):
     rt.eltwise("add", deq, res, y)
     torch.cuda.synchronize()
     shipped = float(orc.f16_to_f32(orc.f32_to_f16(np.array([c["deq_scale"]], np.float32)))[0])
-    wd = orc.dequantize(got[rows], shipped, c["deq_zp"])
-    assert np.array_equal(deq.cpu().numpy().view(np.uint16)[rows], wd)
-    wy = orc.eltwise_f16("add", wd, c["residual"][rows])
-    assert np.array_equal(y.cpu().numpy().view(np.uint16)[rows], wy)
-    # all 256 codes dequantize exactly as the oracle says, so the full tensor is pinned by the table
-    codes = np.arange(-128, 128, dtype=np.int8)
-    table = torch.from_numpy(orc.dequantize(codes, shipped, c["deq_zp"]).view(np.float16)).to(dev)
-    assert bool((deq == table[(out.long() + 128)]).all())
+    deq_bits = deq.cpu().numpy().view(np.uint16)
+    assert np.array_equal(deq_bits, orc.dequantize(got, shipped, c["deq_zp"]))
+    assert sha(deq_bits) == gold["dequantize_f16_bits"]["sha256"]
+    y_bits = y.cpu().numpy().view(np.uint16)
+    assert np.array_equal(y_bits, orc.eltwise_f16("add", deq_bits, c["residual"]))
+    assert sha(y_bits) == gold["add_f16_bits"]["sha256"]
 
 
 @pytest.mark.parametrize("subtract", [False, True])
@@ -408,6 +483,9 @@ def test_nce_rejects_bad_descriptors(rt, dev):
     assert e.value.code == rt.ERROR_INVALID_ARGUMENT
     with pytest.raises(rt.VpxError) as e:
         rt.nce_task(inp.float(), w, wt, out, ok)
+    with pytest.raises(rt.VpxError) as e:  # a float output has no zero point
+        rt.nce_task(inp, w, wt, out.half(), ok, zp_out=3)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT and "zero point" in e.value.text
     big_k = torch.zeros((8, 7, 7, 16), dtype=torch.int8, device=dev)
     with pytest.raises(rt.VpxError) as e:
         rt.nce_task(inp, big_k, wt, out, ok)

@@ -163,6 +163,11 @@ def test_ppe_int_attr_goldens(rt):
     for c in g["cases"]:
         p = rt.retrieve_ppe_int(ops[c["post_op"]], u8t if c["out"] == "u8" else None, c.get("param0", 0.0),
                                 c.get("param1", 0.0))
+        if "clamp_high_unpacked_f16" in c:
+            # two fp16 bit patterns in one word, low bound in the upper half (the reference's test unpacks it the same way)
+            halves = np.array([(p.clamp_high >> 16) & 0xffff, p.clamp_high & 0xffff], dtype=np.uint16).view(np.float16)
+            assert [float(v) for v in halves] == c["clamp_high_unpacked_f16"], c
+            c = dict(c, clamp_high=p.clamp_high)
         assert (p.mode, p.clamp_low, p.clamp_high, p.lrelu_mult, p.lrelu_shift) == \
                (modes[c["mode"]], c["clamp_low"], c["clamp_high"], c["lrelu_mult"], c["lrelu_shift"]), c
     # ReLU on a float output selects LRELU; slope 0 LeakyReLU has multiplier 0; clamp [0, 6] on u8 zp 0 is LRELUX

@@ -4,6 +4,7 @@ closed forms and fp64 brute force.  No GPU."""
 import json
 import math
 import os
+from fractions import Fraction
 
 import numpy as np
 import pytest
@@ -316,6 +317,92 @@ def test_ppe_requant_properties(orc):
     pos = orc.ppe_requant(10 ** 6, 0, 16384, 14, wide) - 3
     neg = orc.ppe_requant(-10 ** 6, 0, 16384, 14, wide) - 3
     assert abs(neg / pos + 1638 / 16384) < 1e-5
+
+
+def _f16_bits_of_fixed(fx):
+    """fx * 2^-15 narrowed to fp16 by numpy: the value is exact in a double, so this is one round-to-nearest-even."""
+    with np.errstate(over="ignore"):
+        return int(np.array([fx / 32768.0], dtype=np.float64).astype(np.float16).view(np.uint16)[0])
+
+
+def test_ppe_requant_f16_fixed_point_conversion(orc):
+    """acc with multiplier 1 and shift 15 is the s17.15 number itself: the conversion alone, against numpy."""
+    none = orc.ppe(1, 0, 0, -(2 ** 31), 2 ** 31 - 1)
+    rng = np.random.default_rng(17)
+    cases = list(range(-70000, 70001, 1))
+    # every 11-bit significand boundary: ties and their neighbours at each magnitude, both signs
+    for top in range(11, 31):
+        step = 1 << (top - 10)
+        for q in (1 << 10, (1 << 10) + 1, (1 << 11) - 2, (1 << 11) - 1):
+            base = q * step
+            for d in (-1, 0, 1, step // 2 - 1, step // 2, step // 2 + 1, step - 1):
+                cases += [base + d, -(base + d)]
+    cases += [2 ** 31 - 1, -(2 ** 31), 65519 * 32768 + 16384, 65520 * 32768, 65504 * 32768, 1, -1, 2, 3, 0]
+    cases += [int(v) for v in rng.integers(-2 ** 31, 2 ** 31, 20000)]
+    for fx in cases:
+        if not -(2 ** 31) <= fx < 2 ** 31:
+            continue
+        assert orc.ppe_requant_f16(fx, 0, 1, 15, none) == _f16_bits_of_fixed(fx), fx
+    assert orc.ppe_requant_f16(1, 0, 1, 15, none) == 0x0200          # 2^-15 is a subnormal half
+    assert orc.ppe_requant_f16(65520 * 32768, 0, 1, 15, none) == 0x7c00  # rounds to infinity
+    assert orc.ppe_requant_f16(-32768, 0, 1, 15, none) == 0xbc00      # -1.0
+
+
+def test_ppe_requant_f16_against_exact_arithmetic(orc):
+    """Whole pipeline against exact rationals: scale, PReLU on negatives, one rounding to 15 fractional bits,
+    saturation to 32 bits, narrowing, packed fp16 clamp."""
+    rng = np.random.default_rng(18)
+    none = orc.ppe(1, 0, 0, -(2 ** 31), 2 ** 31 - 1)
+    lrelu = orc.ppe(1638, 14, 0, -(2 ** 31), 2 ** 31 - 1)
+    relu = orc.ppe(0, 0, 0, -(2 ** 31), 2 ** 31 - 1)
+    clamp = orc.ppe(0, 0, 0, -(2 ** 31), orc.pack_clamp_f16(20.0, 300.0))
+    # the packed word of the reference's own test (ppe_factory_tests.cpp:781-791 unpacks it to 20.0 and 300.0)
+    packed = orc.pack_clamp_f16(20.0, 300.0) & 0xffffffff
+    assert (packed >> 16, packed & 0xffff) == (0x4d00, 0x5cb0)
+    for it in range(6000):
+        acc = int(rng.integers(-2 ** 31, 2 ** 31)) if it % 3 else int(rng.integers(-2 ** 16, 2 ** 16))
+        bias = int(rng.integers(-2 ** 15, 2 ** 15))
+        mult = int(rng.integers(2 ** 14, 2 ** 15)) * (1 if it % 7 else -1)
+        shift = int(rng.integers(0, 50))
+        for p, pm, ps in ((none, 1, 0), (lrelu, 1638, 14), (relu, 0, 0), (clamp, 0, 0)):
+            biased = (acc + bias + 2 ** 31) % 2 ** 32 - 2 ** 31
+            t = biased * mult
+            s = shift
+            if t < 0:
+                t *= pm
+                s += ps
+            fx = Fraction(t * 2 ** 15, 2 ** s)
+            fl = math.floor(fx)
+            rem = fx - fl
+            if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+                fl += 1
+            fl = min(max(fl, -(2 ** 31)), 2 ** 31 - 1)
+            want = _f16_bits_of_fixed(fl)
+            if p is clamp:
+                v = float(np.array([want], dtype=np.uint16).view(np.float16)[0])
+                want = 0x4d00 if v < 20.0 else (0x5cb0 if v > 300.0 else want)
+            assert orc.ppe_requant_f16(acc, bias, mult, shift, p) == want, (acc, bias, mult, shift, pm, ps)
+    # the value is (acc + bias) * mult * 2^-shift: scale 0.5 (16384 / 2^15) of 6 is 3.0
+    assert orc.ppe_requant_f16(6, 0, 16384, 15, none) == 0x4200
+    # LeakyReLU 0.1 = 1638 / 2^14 on a negative value: -1000 * 0.5 * 0.0999755859375 = -49.98779296875 -> fp16
+    assert orc.ppe_requant_f16(-1000, 0, 16384, 15, lrelu) == int(np.array([-49.98779296875]).astype(np.float16).view(np.uint16)[0])
+
+
+def test_nce_matmul_f16_output_uses_the_fixed_point_path(orc):
+    rng = np.random.default_rng(19)
+    A = rng.integers(0, 256, (5, 48), dtype=np.uint8)
+    B = rng.integers(-127, 128, (7, 48)).astype(np.int8)
+    mults, shifts = rng.integers(2 ** 14, 2 ** 15, 7), rng.integers(14, 26, 7)
+    bias = rng.integers(-2 ** 12, 2 ** 12, 7).astype(np.int32)
+    wt = orc.make_weights_table(mults, shifts, bias, 48)
+    p = orc.ppe(1638, 14, 0, -(2 ** 31), 2 ** 31 - 1)
+    out, acc = orc.nce_matmul(A, B, wt, p, zp_a=128, want_acc=True, out_f16=True)
+    assert out.dtype == np.uint16 and out.shape == (5, 7)
+    ref_acc = (A.astype(np.int64) - 128) @ B.astype(np.int64).T
+    assert np.array_equal(acc, ref_acc)
+    for m in range(5):
+        for n in range(7):
+            assert out[m, n] == orc.ppe_requant_f16(int(acc[m, n]), int(bias[n]), int(mults[n]), int(shifts[n]), p)
 
 
 def test_nce_conv_against_brute_force(orc):

@@ -22,10 +22,14 @@
 // zero point so they contribute exactly 0, as the MPE does (runtime_dpu_parser_imports.cpp.inc:872-879).
 // A weight zero point (mpe_wtbias, :940-945) adds one term per output position, prepared by two small
 // kernels and added to the accumulators before the PPE (see nce_pixel_sum_kernel).
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
+#include <set>
 #include <type_traits>
+#include <utility>
 
 #include "vpx_common.h"
 
@@ -40,7 +44,10 @@ typedef int32_t i32x16 __attribute__((ext_vector_type(16)));
 
 struct Ppe {
     int prelu_mult, prelu_shift, zp_out, clamp_lo, clamp_hi;
+    float f16_lo, f16_hi;  // fp16 output only: the clamp bounds unpacked from clamp_high (infinite when absent)
 };
+
+enum OutKind { OUT_U8 = 0, OUT_I8 = 1, OUT_F16 = 2 };
 
 // Raw per-channel PPE parameters, unpacked from weight-table words 2 and 3.
 struct ChanParams {
@@ -75,6 +82,51 @@ __device__ __forceinline__ int ppe_requant(int acc, ChanParams c, Ppe p) {
     return (int)r;
 }
 
+// fp16 output ("INT32 s17.15 fixed-point convert to FP16", runtime_dpu_parser_imports.cpp.inc:546-552): the
+// round stage keeps 15 fractional bits, the 32-bit result fx stands for fx * 2^-15, and that value is narrowed to
+// fp16 with one round-to-nearest-even.  A float holds 24 bits: the 31-bit magnitude is first cut to 24 bits with
+// the lost bits OR-ed into the last one (round to odd), which makes the hardware's second rounding to 11 bits exact.
+__device__ __forceinline__ uint16_t f16_from_s1715(int fx, float lo, float hi) {
+    unsigned a = fx < 0 ? 0u - (unsigned)fx : (unsigned)fx;
+    const int lz = __builtin_clz(a | 1u);
+    const int drop = lz < 8 ? 8 - lz : 0;
+    const unsigned sticky = (a & ((1u << drop) - 1u)) != 0u ? 1u : 0u;
+    a = (a >> drop) | sticky;
+    float v = __builtin_ldexpf((float)a, drop - 15);  // exact
+    v = fx < 0 ? -v : v;
+    _Float16 h = (_Float16)v;
+    const float r = (float)h;
+    h = r < lo ? (_Float16)lo : h;
+    h = r > hi ? (_Float16)hi : h;
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+// The same pipeline as ppe_requant up to the round stage, in 64-bit integers (general, slow form).
+__device__ __forceinline__ uint16_t ppe_requant_f16(int acc, ChanParams c, Ppe p) {
+    const int biased = (int)((unsigned)acc + (unsigned)c.bias);
+    long long t = (long long)biased * (long long)c.mult;
+    int s = c.shift - 15;
+    if (t < 0) {
+        t *= (long long)p.prelu_mult;
+        s += p.prelu_shift;
+    }
+    long long r;
+    if (s <= 0) {
+        // |t| < 2^58 and s >= -15: saturate before the shift could overflow
+        const long long lim = 0x7fffffffffffffffll >> (-s);
+        r = t > lim ? 0x7fffffffffffffffll : (t < -lim ? -0x7fffffffffffffffll : t * (1ll << (-s)));
+    } else if (s >= 64) {
+        r = 0;
+    } else {
+        const long long q = t >> s;
+        const unsigned long long rem = (unsigned long long)t & ((1ull << s) - 1ull);
+        const unsigned long long half = 1ull << (s - 1);
+        r = q + ((rem > half || (rem == half && (q & 1))) ? 1 : 0);
+    }
+    r = r > 2147483647ll ? 2147483647ll : (r < -2147483648ll ? -2147483648ll : r);
+    return f16_from_s1715((int)r, p.f16_lo, p.f16_hi);
+}
+
 template <bool OUT_SIGNED>
 __device__ __forceinline__ int saturate8i(int r) {
     if (OUT_SIGNED) return r < -128 ? -128 : (r > 127 ? 127 : r);
@@ -107,6 +159,7 @@ struct PpeFast {
     // (activation - zero point) under the window of output position m, added to every channel of that
     // position; null when the weights the kernel reads have none (see nce_pixel_sum_kernel).
     const int32_t* rowterm;
+    float f16_lo, f16_hi;  // fp16 output: clamp bounds
 };
 
 // Any bound between the largest |b| whose result can still lie inside a clamp window and 2^30 / |f|
@@ -145,6 +198,19 @@ __device__ __forceinline__ int ppe_fast(int acc, const ChanPrep& c, const PpeFas
     const int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, y) + p.zp_out;
     const int t = q > p.lo ? q : p.lo;
     return t < p.hi ? t : p.hi;
+}
+
+// fp16 output, fast form.  `c` comes from ppe_prepare with shift - 15, so b * f is the value in units of 2^-15;
+// the fused multiply-add rounds the exact product once to an integer (ties to even), the subtraction that
+// follows is exact, and the saturation to 32 bits absorbs products too large for that trick.
+__device__ __forceinline__ uint16_t ppe_fast_f16(int acc, const ChanPrep& c, float lo, float hi) {
+    const int b = (int)((unsigned)acc + (unsigned)c.bias);
+    const bool neg = (b ^ c.sgn) < 0;
+    const double f = neg ? c.f_neg : c.f_pos;
+    constexpr double kMagic = 6755399441055744.0;  // 1.5 * 2^52
+    double v = __builtin_fma((double)b, f, kMagic) - kMagic;
+    v = v > 2147483647.0 ? 2147483647.0 : (v < -2147483648.0 ? -2147483648.0 : v);
+    return f16_from_s1715((int)v, lo, hi);
 }
 
 // Four results of one output channel as four bytes.  Same arithmetic as ppe_fast with the tail
@@ -225,7 +291,7 @@ __device__ __forceinline__ ChanPrep ppe_prepare_packed(int mult, int shift, int 
 // prepared epilogue parameters.
 __global__ __launch_bounds__(256) void nce_fold_kernel(const int8_t* __restrict__ w, const int32_t* __restrict__ wt,
                                                        ChanPrep* __restrict__ prep, int64_t OC, int64_t K, int corr,
-                                                       Ppe ppe) {
+                                                       Ppe ppe, int shift_sub) {
     const int lane = threadIdx.x & 63;
     const int64_t oc = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (oc >= OC) return;
@@ -245,7 +311,8 @@ __global__ __launch_bounds__(256) void nce_fold_kernel(const int8_t* __restrict_
     }
     if (lane == 0) {
         const uint32_t w2 = (uint32_t)wt[oc * 4 + 2];
-        const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+        // shift_sub = 15 for an fp16 output (the scaled value keeps 15 fractional bits), else 0
+        const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu) - shift_sub,
                                        (int)((unsigned)wt[oc * 4 + 3] + (unsigned)(corr * sum)), ppe.prelu_mult, ppe.prelu_shift);
         prep[oc] = c;
     }
@@ -290,7 +357,7 @@ struct ConvGeom {
     int KY, KX, SY, SX, PT, PL;
 };
 
-template <bool IN_SIGNED, bool W_SIGNED, bool OUT_SIGNED>
+template <bool IN_SIGNED, bool W_SIGNED, int OUT>
 __global__ __launch_bounds__(256) void nce_conv_naive(const uint8_t* __restrict__ in, const uint8_t* __restrict__ w,
                                                       const int32_t* __restrict__ wt, uint8_t* __restrict__ out,
                                                       ConvGeom g, int zp_in, int zp_w, Ppe ppe, int64_t total) {
@@ -319,7 +386,8 @@ __global__ __launch_bounds__(256) void nce_conv_naive(const uint8_t* __restrict_
     }
     const uint32_t w2 = (uint32_t)wt[oc * 4 + 2];
     ChanParams c{wt[oc * 4 + 3], (int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu)};
-    out[idx] = saturate8<OUT_SIGNED>(ppe_requant(acc, c, ppe));
+    if (OUT == OUT_F16) reinterpret_cast<uint16_t*>(out)[idx] = ppe_requant_f16(acc, c, ppe);
+    else out[idx] = saturate8<OUT == OUT_I8>(ppe_requant(acc, c, ppe));
 }
 
 // ---------------------------------------------------------------- GEMM path
@@ -380,6 +448,7 @@ struct GemmPpe {
     int zp_out, lo, hi;           // clamp bounds already intersected with the storage range
     int out_signed;               // output storage is i8
     const int32_t* rowterm;       // as in PpeFast; padded past the last position, so edge tiles may read ahead
+    float f16_lo, f16_hi;         // fp16 output: clamp bounds
 };
 
 // A[M][K] x B[N][K]^T with the PPE fused; see the file header.  K must be a multiple of 64.
@@ -392,7 +461,7 @@ struct GemmPpe {
 // so that the MFMAs of the second sub-step cover the first fragment reads of panel kt+1.  The column sums of B that the zero-point
 // term needs come from nce_colsum_kernel (only when that term is not zero), and the per-column PPE
 // parameters are unpacked from the weight table in the epilogue.
-template <bool IN_U8, bool OUT_SIGNED, int NW, int TILE = 256, bool SHORTK = false>
+template <bool IN_U8, int OUT, int NW, int TILE = 256, bool SHORTK = false>
 __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restrict__ A, const int8_t* __restrict__ B,
                                                      const int32_t* __restrict__ wt, const int32_t* __restrict__ colsum,
                                                      uint8_t* __restrict__ out,
@@ -550,6 +619,27 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     dma_wait_all_and_barrier();  // every wave is done with the panels: LDS becomes the output staging tile
 
     // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
+    if constexpr (OUT == OUT_F16) {
+        // fp16 output: 16-bit values straight from the registers, 32 adjacent columns (64 bytes) per half-wavefront
+        uint16_t* out16 = reinterpret_cast<uint16_t*>(out);
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const uint32_t w2 = (uint32_t)w2r[j];
+            const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu) - 15,
+                                           (int)((unsigned)w3r[j] + (unsigned)(ppe.corr * csr[j])), ppe.prelu_mult, ppe.prelu_shift);
+            const int64_t n = n0 + wn0 + j * 32 + (lane & 31);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int64_t m = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                    const int extra = ppe.rowterm ? ppe.rowterm[m] : 0;
+                    if (m < M && n < N) out16[m * N + n] = ppe_fast_f16(acc[i][j][r] + extra, c, ppe.f16_lo, ppe.f16_hi);
+                }
+        }
+        return;
+    }
+    constexpr bool OUT_SIGNED = OUT == OUT_I8;
     ChanPrep cp[TN];
     bool clip = false;
 #pragma unroll
@@ -615,7 +705,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
 // The weights of the BN channels, all taps, sit in LDS as [BN][KY*KX*IC] rows (swizzle as above
 // on 64-byte granules, applied when a row is a whole number of them); activation fragments come
 // straight from global memory, 16 bytes per lane.
-template <int BM, int BN, bool IN_U8, bool OUT_SIGNED>
+template <int BM, int BN, bool IN_U8, int OUT>
 __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                      const ChanPrep* __restrict__ prep, uint8_t* __restrict__ out,
                                                      ConvGeom g, int pad_byte, int swz, int tc, int icc, PpeFast ppe) {
@@ -722,7 +812,10 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t m = m0 + wave * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                if (m < Mtot) out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(acc[i][j][r] + (ppe.rowterm ? ppe.rowterm[m] : 0), cp, ppe);
+                if (m >= Mtot) continue;
+                const int a = acc[i][j][r] + (ppe.rowterm ? ppe.rowterm[m] : 0);
+                if (OUT == OUT_F16) reinterpret_cast<uint16_t*>(out)[m * g.OC + oc] = ppe_fast_f16(a, cp, ppe.f16_lo, ppe.f16_hi);
+                else out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(a, cp, ppe);
             }
         }
     }
@@ -1248,7 +1341,7 @@ __global__ __launch_bounds__(256) void nce_eltwise_kernel(const uint8_t* __restr
 // 16 but not of 32.  K = KY*KX*IC is walked as a flat run of 16-byte chunks, two per MFMA step:
 // lanes 0-31 feed chunk 2j, lanes 32-63 chunk 2j+1, which may belong to different taps.  All
 // weights of the 64 output channels (K rounded up to 32, zero-filled) sit in LDS.
-template <bool IN_U8>
+template <bool IN_U8, int OUT>
 __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                        const ChanPrep* __restrict__ prep, uint8_t* __restrict__ out,
                                                        ConvGeom g, int pad_byte, PpeFast ppe) {
@@ -1328,18 +1421,33 @@ __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict_
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int64_t m = m0 + wave * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                if (m < Mtot) out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(acc[i][j][r] + (ppe.rowterm ? ppe.rowterm[m] : 0), cp, ppe);
+                if (m >= Mtot) continue;
+                const int a = acc[i][j][r] + (ppe.rowterm ? ppe.rowterm[m] : 0);
+                if (OUT == OUT_F16) reinterpret_cast<uint16_t*>(out)[m * g.OC + oc] = ppe_fast_f16(a, cp, ppe.f16_lo, ppe.f16_hi);
+                else out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(a, cp, ppe);
             }
         }
     }
 }
 
+// Kernels that may ask for more than 64 KiB of dynamic LDS are given the largest size any launch of them uses,
+// once per (device, kernel): the attribute is then never changed again, so concurrent launches that want
+// different sizes cannot undo each other's setting.
+constexpr size_t kMaxDynLds = 160 * 1024 - 512;
+std::mutex g_lds_mutex;
+std::set<std::pair<int, const void*>> g_lds_done;
+
 template <class KernelT>
 int set_dyn_lds(KernelT kernel, size_t bytes) {
-    if (bytes > 64 * 1024) {
-        VPX_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
-    }
+    if (bytes <= 64 * 1024) return VPX_RESULT_SUCCESS;
+    VPX_REQUIRE(bytes <= kMaxDynLds, VPX_RESULT_ERROR_UNKNOWN, "a launch asks for %zu bytes of LDS", bytes);
+    int dev = 0;
+    VPX_HIP_CHECK(hipGetDevice(&dev));
+    const void* fn = reinterpret_cast<const void*>(kernel);
+    std::lock_guard<std::mutex> lock(g_lds_mutex);
+    if (g_lds_done.count({dev, fn})) return VPX_RESULT_SUCCESS;
+    VPX_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxDynLds));
+    g_lds_done.insert({dev, fn});
     return VPX_RESULT_SUCCESS;
 }
 
@@ -1453,11 +1561,60 @@ __global__ __launch_bounds__(256) void nce_weights_to_s8_kernel(const i32x4* __r
 }
 
 
+// Dispatch overrides for tests and tuning.  The VPX_* environment variables of the same names are read once, at
+// the first use; afterwards only vpx_set_tuning changes a value, so a launch never reads the environment.
+enum { NCE_AUTO = 0, NCE_NAIVE, NCE_GATHER, NCE_CONV };
+struct Tuning {
+    std::atomic<int> nce_kernel{NCE_AUTO};  // VPX_NCE_KERNEL = naive | gather | conv: restrict the choice to slower, more general paths
+    std::atomic<int> gemm_tile{0};          // VPX_GEMM_TILE = 128 | 256 (0: chosen from the shape)
+    std::atomic<int> gemm_waves{0};         // VPX_GEMM_WAVES = 4 | 8
+    std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = stream: skip the resident-weights tile kernel
+    std::atomic<int> conv_rows{0};          // VPX_CONV_ROWS = n: cap on the output rows per workgroup of the LDS-patch kernels
+    std::atomic<int> conv_waves{0};         // VPX_CONV_WAVES = 4 | 8
+};
+Tuning g_tuning;
+std::once_flag g_tuning_once;
+
+bool set_knob(const char* knob, const char* value) {
+    const char* v = value ? value : "";
+    if (!std::strcmp(knob, "VPX_NCE_KERNEL")) {
+        g_tuning.nce_kernel = !std::strcmp(v, "naive") ? NCE_NAIVE : (!std::strcmp(v, "gather") ? NCE_GATHER : (!std::strcmp(v, "conv") ? NCE_CONV : NCE_AUTO));
+    } else if (!std::strcmp(knob, "VPX_GEMM_TILE")) {
+        g_tuning.gemm_tile = *v ? (std::atoi(v) == 128 ? 128 : 256) : 0;
+    } else if (!std::strcmp(knob, "VPX_GEMM_WAVES")) {
+        g_tuning.gemm_waves = *v ? (std::atoi(v) == 4 ? 4 : 8) : 0;
+    } else if (!std::strcmp(knob, "VPX_CONV_KERNEL")) {
+        g_tuning.conv_stream = !std::strcmp(v, "stream") ? 1 : 0;
+    } else if (!std::strcmp(knob, "VPX_CONV_ROWS")) {
+        g_tuning.conv_rows = std::atoi(v) > 0 ? std::atoi(v) : 0;
+    } else if (!std::strcmp(knob, "VPX_CONV_WAVES")) {
+        g_tuning.conv_waves = std::atoi(v) == 4 ? 4 : 0;
+    } else {
+        return false;
+    }
+    return true;
+}
+
+const Tuning& tuning() {
+    std::call_once(g_tuning_once, [] {
+        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES"})
+            if (const char* v = std::getenv(k)) set_knob(k, v);
+    });
+    return g_tuning;
+}
+
 }  // namespace
+
+int set_tuning(const char* knob, const char* value) {
+    (void)tuning();  // the environment is consulted before the first explicit setting, never after it
+    VPX_REQUIRE(knob != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "tuning knob name is null");
+    VPX_REQUIRE(set_knob(knob, value), VPX_RESULT_ERROR_INVALID_ARGUMENT, "unknown tuning knob '%s'", knob);
+    return VPX_RESULT_SUCCESS;
+}
 
 int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name) {
     const bool in_u8 = t.input_type == VPX_NN_U8, w_u8 = t.weights_type == VPX_NN_U8,
-               out_signed = t.output_type == VPX_NN_I8;
+               out_signed = t.output_type == VPX_NN_I8, out_f16 = t.output_type == VPX_NN_FP16;
     ConvGeom g{};
     g.N = t.N; g.H = t.H; g.W = t.W; g.IC = t.IC; g.OC = t.OC;
     g.KY = t.kernel_size[0]; g.KX = t.kernel_size[1];
@@ -1472,6 +1629,19 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     ppe.zp_out = t.zp_out;
     ppe.clamp_lo = t.ppe.clamp_low;
     ppe.clamp_hi = t.ppe.clamp_high;
+    ppe.f16_lo = -INFINITY;
+    ppe.f16_hi = INFINITY;
+    if (out_f16 && t.ppe.clamp_high != INT32_MAX) {
+        // two fp16 bounds in one word, 0xllllhhhh (dialect/VPU/utils/ppe_utils.hpp:36-87); clamp_low is not used
+        const auto half = [](uint32_t h) {
+            const uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+            const float mag = e == 0 ? std::ldexp((float)m, -24) : (e == 31 ? (m ? NAN : INFINITY) : std::ldexp((float)(m | 0x400u), (int)e - 25));
+            return (h & 0x8000u) ? -mag : mag;
+        };
+        const float lo = half(((uint32_t)t.ppe.clamp_high >> 16) & 0xffffu), hi = half((uint32_t)t.ppe.clamp_high & 0xffffu);
+        if (!std::isnan(lo)) ppe.f16_lo = lo;
+        if (!std::isnan(hi)) ppe.f16_hi = hi;
+    }
     switch (t.ppe.mode) {
     case VPX_PPE_NOOP: ppe.prelu_mult = 1; ppe.prelu_shift = 0; break;
     case VPX_PPE_LRELU:
@@ -1501,10 +1671,11 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights)) & 15) == 0;
     // VPX_NCE_KERNEL=naive|gather|conv restricts the choice to the slower, more general paths (used by tests
     // to check the device paths against each other).
-    const char* force = std::getenv("VPX_NCE_KERNEL");
-    const bool allow_gemm = !force || !*force;
-    const bool allow_lds = allow_gemm || std::strcmp(force, "conv") == 0;
-    const bool allow_mfma = allow_lds || std::strcmp(force, "gather") == 0;
+    const Tuning& knobs = tuning();
+    const int force = knobs.nce_kernel.load();
+    const bool allow_gemm = force == NCE_AUTO;
+    const bool allow_lds = allow_gemm || force == NCE_CONV;
+    const bool allow_mfma = allow_lds || force == NCE_GATHER;
 
     // A 256-column matmul tile wastes three quarters of its MFMAs on 64 output channels: such 1x1 layers go
     // to the convolution kernels, whose tiles are 64 channels wide (measured 7 us against 18 us at [100352 x 64 x 64]).
@@ -1566,6 +1737,8 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         PpeFast pf{};
         pf.zp_out = t.zp_out;
         pf.rowterm = rowterm;
+        pf.f16_lo = ppe.f16_lo;
+        pf.f16_hi = ppe.f16_hi;
         const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
         pf.lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin;
         pf.hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
@@ -1577,23 +1750,23 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             // 256 x 256 tiles when they fill the chip and K is long enough to amortise their prologue and epilogue;
             // else 128 x 128 (four times as many, two workgroups per CU): [25088 x 512 x 128] 14.1 -> 7.8 us,
             // [100352 x 256 x 128] 23.8 -> 14.4 us, [512 x 4096 x 4096] 43 -> 24 us.  VPX_GEMM_TILE=128|256 overrides.
-            const char* tenv = std::getenv("VPX_GEMM_TILE");
-            const int tile = tenv && *tenv ? (std::atoi(tenv) == 128 ? 128 : 256) : (gemm_tiles < 200 || g.IC <= 256 ? 128 : 256);
+            const int tile_knob = knobs.gemm_tile.load();
+            const int tile = tile_knob ? tile_knob : (gemm_tiles < 200 || g.IC <= 256 ? 128 : 256);
             const int tiles_m = (int)((Mtot + tile - 1) / tile), tiles_n = (int)((g.OC + tile - 1) / tile);
             const int per_xcd = (tiles_m * tiles_n + 7) / 8;
             // Eight waves (two per SIMD) overlap the PPE epilogue better and win up to K = 4096; beyond
             // that the lower LDS traffic of four 128x128 waves wins.  VPX_GEMM_WAVES=4|8 overrides.
-            const char* wenv = std::getenv("VPX_GEMM_WAVES");
-            const int nw = tile == 128 ? 4 : (wenv && *wenv ? (std::atoi(wenv) == 4 ? 4 : 8) : (g.IC > 4096 ? 4 : 8));
+            const int waves_knob = knobs.gemm_waves.load();
+            const int nw = tile == 128 ? 4 : (waves_knob ? waves_knob : (g.IC > 4096 ? 4 : 8));
             const dim3 grid((unsigned)(per_xcd * 8)), block(64 * nw);
             const int64_t nk = g.IC / 64;
-            const bool shortk = tile == 128 && nk <= 3;
+            const bool shortk = tile == 128 && nk <= 3 && !out_f16;
             size_t lds = 4 * (size_t)(tile + tile) * 64;  // four K panels; the output staging tile reuses them
             if (shortk) {
                 lds = (size_t)nk * (tile + tile) * 64;  // only the panels there are ...
                 if (lds < (size_t)tile * kOutStride) lds = (size_t)tile * kOutStride;  // ... or the staging tile
             }
-            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
+            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi};
             int32_t* colsum = nullptr;
             if (corr != 0) {
                 void* ws = nullptr;
@@ -1619,10 +1792,15 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         else if (nw == 4) VPX_GEMM_W(U8, SGN, 4, 256, false);                                                        \
         else VPX_GEMM_W(U8, SGN, 8, 256, false);                                                                     \
     } while (0)
-            if (in_u8 && out_signed) VPX_GEMM(true, true);
-            else if (in_u8) VPX_GEMM(true, false);
-            else if (out_signed) VPX_GEMM(false, true);
-            else VPX_GEMM(false, false);
+            if (out_f16) {
+                // fp16 output: the eight-wave 256-tile and the four-wave 128-tile forms only
+                if (in_u8) { if (tile == 128) VPX_GEMM_W(true, OUT_F16, 4, 128, false); else VPX_GEMM_W(true, OUT_F16, 8, 256, false); }
+                else { if (tile == 128) VPX_GEMM_W(false, OUT_F16, 4, 128, false); else VPX_GEMM_W(false, OUT_F16, 8, 256, false); }
+            }
+            else if (in_u8 && out_signed) VPX_GEMM(true, OUT_I8);
+            else if (in_u8) VPX_GEMM(true, OUT_U8);
+            else if (out_signed) VPX_GEMM(false, OUT_I8);
+            else VPX_GEMM(false, OUT_U8);
 #undef VPX_GEMM
 #undef VPX_GEMM_W
             VPX_HIP_CHECK(hipGetLastError());
@@ -1631,13 +1809,13 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         }
 
         // Preferred: input patch in LDS, one launch.  R = output rows per workgroup.
-        if (allow_lds && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20) &&
-            g.IC < (1 << 14) && g.W * g.SX < (1 << 14) && g.N * g.OH * g.OH < (1ll << 32)) {
+        // (an fp16 output takes the gather kernel below: the tile kernels' epilogues stage bytes)
+        if (allow_lds && !out_f16 && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20) &&
+            g.IC < (1 << 14) && g.W * g.SX < (1 << 14) && g.N * g.OH * g.OW < (1ll << 31)) {
             // IC of 64 or 128: the one-tile-per-workgroup kernel with padded LDS rows (a tap's fragments of more
             // channels do not fit the registers twice)
             // VPX_CONV_KERNEL=stream starts the choice below the tile kernel (tests compare them)
-            const char* ck = std::getenv("VPX_CONV_KERNEL");
-            const int first = ck && std::strcmp(ck, "stream") == 0 ? 1 : 0;
+            const int first = knobs.conv_stream.load() ? 1 : 0;
             // (with 128 channels and a stride the haloed patch crowds the resident weights out of LDS: the
             // streamed-weights kernel below measures 15.7 us against 20.2 at [32,56,56,128] -> 128, 3x3, stride 2)
             if ((g.IC == 64 || (g.IC == 128 && g.SY * g.SX == 1)) && first <= 0) {
@@ -1654,8 +1832,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 if (need(R) <= 160 * 1024 - 512) {
                     const int64_t ocb = (g.OC + 63) / 64;
                     while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 512 && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
-                    if (const char* e = std::getenv("VPX_CONV_ROWS")) {
-                        const int v = std::atoi(e);
+                    if (const int v = knobs.conv_rows.load()) {
                         if (v >= 1 && v <= R) R = v;
                     }
                     const int tiles_y = (int)((g.OH + R - 1) / R);
@@ -1676,8 +1853,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
                     const int pad_byte = t.zp_in & 0xff;
                     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
-                    const char* cw = std::getenv("VPX_CONV_WAVES");
-                    const int nw = cw && std::atoi(cw) == 4 ? 4 : 8;
+                    const int nw = knobs.conv_waves.load() == 4 ? 4 : 8;
                     const int per_wave = (pg.MT + nw / pg.nt - 1) / (nw / pg.nt);
                     const int ics = (int)(g.IC / 64);
 #define VPX_TILE_W(U8, TMW, SAME, ICS, NW)                                                                            \
@@ -1735,8 +1911,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 if (need(R) <= 160 * 1024 - 512) {
                     const int64_t ocb = (g.OC + 63) / 64;
                     while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 512 && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
-                    if (const char* e = std::getenv("VPX_CONV_ROWS")) {
-                        const int v = std::atoi(e);
+                    if (const int v = knobs.conv_rows.load()) {
                         if (v >= 1 && v <= R) R = v;
                     }
                     const int tiles_y = (int)((g.OH + R - 1) / R);
@@ -1800,7 +1975,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         if (rc) return rc;
         ChanPrep* prep = (ChanPrep*)ws;
         hipLaunchKernelGGL(nce_fold_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s, (const int8_t*)wptr,
-                           t.weight_table, prep, g.OC, Ktot, corr, ppe);
+                           t.weight_table, prep, g.OC, Ktot, corr, ppe, out_f16 ? 15 : 0);
         VPX_HIP_CHECK(hipGetLastError());
 
         constexpr int BM = 256, BN = 64;
@@ -1820,10 +1995,12 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)wptr, prep,    \
                            (uint8_t*)t.output, g, pad_byte, swz, tc, icc, pf);                                       \
     } while (0)
-        if (in_u8 && out_signed) VPX_CONV(true, true);
-        else if (in_u8) VPX_CONV(true, false);
-        else if (out_signed) VPX_CONV(false, true);
-        else VPX_CONV(false, false);
+        if (out_f16 && in_u8) VPX_CONV(true, OUT_F16);
+        else if (out_f16) VPX_CONV(false, OUT_F16);
+        else if (in_u8 && out_signed) VPX_CONV(true, OUT_I8);
+        else if (in_u8) VPX_CONV(true, OUT_U8);
+        else if (out_signed) VPX_CONV(false, OUT_I8);
+        else VPX_CONV(false, OUT_U8);
 #undef VPX_CONV
         VPX_HIP_CHECK(hipGetLastError());
         *kernel_name = "nce_conv_mfma";
@@ -1834,6 +2011,8 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
         PpeFast pf{};
         pf.zp_out = t.zp_out;
+        pf.f16_lo = ppe.f16_lo;
+        pf.f16_hi = ppe.f16_hi;
         const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
         pf.lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin;
         pf.hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
@@ -1848,15 +2027,19 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         if (rc) return rc;
         ChanPrep* prep = (ChanPrep*)ws;
         hipLaunchKernelGGL(nce_fold_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s, (const int8_t*)wptr,
-                           t.weight_table, prep, g.OC, Ktot, corr, ppe);
+                           t.weight_table, prep, g.OC, Ktot, corr, ppe, out_f16 ? 15 : 0);
         VPX_HIP_CHECK(hipGetLastError());
         const size_t lds = (size_t)64 * ((Ktot + 31) / 32 * 32 + 16);
         const dim3 grid((unsigned)((Mtot + 255) / 256), (unsigned)((g.OC + 63) / 64));
         const int pad_byte = t.zp_in & 0xff;
-        if (in_u8) hipLaunchKernelGGL(nce_conv_mfma16<true>, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,
-                                      prep, (uint8_t*)t.output, g, pad_byte, pf);
-        else hipLaunchKernelGGL(nce_conv_mfma16<false>, grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,
-                                prep, (uint8_t*)t.output, g, pad_byte, pf);
+#define VPX_CONV16(U8, OUT)                                                                                           \
+    hipLaunchKernelGGL((nce_conv_mfma16<U8, OUT>), grid, dim3(256), lds, s, (const int8_t*)t.input, (const int8_t*)wptr, prep, \
+                       (uint8_t*)t.output, g, pad_byte, pf)
+        if (in_u8 && out_f16) VPX_CONV16(true, OUT_F16);
+        else if (in_u8) VPX_CONV16(true, OUT_U8);
+        else if (out_f16) VPX_CONV16(false, OUT_F16);
+        else VPX_CONV16(false, OUT_U8);
+#undef VPX_CONV16
         VPX_HIP_CHECK(hipGetLastError());
         *kernel_name = "nce_conv_mfma16";
         return VPX_RESULT_SUCCESS;
@@ -1870,15 +2053,22 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     hipLaunchKernelGGL((nce_conv_naive<IS, WS, OS>), grid, dim3(256), 0, s, (const uint8_t*)t.input,                 \
                        (const uint8_t*)t.weights, t.weight_table, (uint8_t*)t.output, g, t.zp_in, t.zp_w, ppe, total)
     const int sel = (in_u8 ? 0 : 4) | (w_u8 ? 0 : 2) | (out_signed ? 1 : 0);
-    switch (sel) {
-    case 0: VPX_NAIVE(false, false, false); break;
-    case 1: VPX_NAIVE(false, false, true); break;
-    case 2: VPX_NAIVE(false, true, false); break;
-    case 3: VPX_NAIVE(false, true, true); break;
-    case 4: VPX_NAIVE(true, false, false); break;
-    case 5: VPX_NAIVE(true, false, true); break;
-    case 6: VPX_NAIVE(true, true, false); break;
-    default: VPX_NAIVE(true, true, true); break;
+    if (out_f16) {
+        switch (sel >> 1) {
+        case 0: VPX_NAIVE(false, false, OUT_F16); break;
+        case 1: VPX_NAIVE(false, true, OUT_F16); break;
+        case 2: VPX_NAIVE(true, false, OUT_F16); break;
+        default: VPX_NAIVE(true, true, OUT_F16); break;
+        }
+    } else switch (sel) {
+    case 0: VPX_NAIVE(false, false, OUT_U8); break;
+    case 1: VPX_NAIVE(false, false, OUT_I8); break;
+    case 2: VPX_NAIVE(false, true, OUT_U8); break;
+    case 3: VPX_NAIVE(false, true, OUT_I8); break;
+    case 4: VPX_NAIVE(true, false, OUT_U8); break;
+    case 5: VPX_NAIVE(true, false, OUT_I8); break;
+    case 6: VPX_NAIVE(true, true, OUT_U8); break;
+    default: VPX_NAIVE(true, true, OUT_I8); break;
     }
 #undef VPX_NAIVE
     VPX_HIP_CHECK(hipGetLastError());

@@ -81,6 +81,9 @@ struct NdIndex {
 // so they can share it; calls on different streams get different buffers.
 int get_workspace(hipStream_t stream, size_t bytes, void** out);
 
+// Dispatch override for tests and tuning (knob names are those of the VPX_* environment variables, read once).
+int set_tuning(const char* knob, const char* value);
+
 // ---- kernel launchers (defined in the .hip files) ------------------------------------------
 int launch_convert(const MemRef& in, const MemRef& out, hipStream_t s);
 int launch_eltwise(int op, const MemRef& a, const MemRef& b, const MemRef& out, hipStream_t s);

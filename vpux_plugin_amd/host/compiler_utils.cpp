@@ -246,7 +246,19 @@ int vpx_retrieve_ppe_int(int post_op, double param0, double param1, const vpx_qu
         }
         return VPX_RESULT_SUCCESS;
     case VPX_POSTOP_CLAMP: {
-        if (!q) return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "Clamp on a float output uses the fp PPE clamp, not the integer pipeline");
+        if (!q) {
+            // fp16 output: both bounds as fp16 bit patterns in clamp_high (0xllllhhhh, the sign-extended patterns
+            // added, ppe_utils.hpp:57-73), clamp_low stays at its neutral value; a maximum that fp16 cannot hold
+            // leaves a plain ReLU (ppe_factory.cpp:170-178)
+            if (param1 < 65504.0) {
+                const int32_t lo = (int32_t)(int16_t)floatToHalfBits((float)param0), hi = (int32_t)(int16_t)floatToHalfBits((float)param1);
+                ppe->clamp_high = (int32_t)(((uint32_t)lo << 16) + (uint32_t)hi);
+                ppe->mode = VPX_PPE_LRELUX;
+            } else {
+                ppe->mode = VPX_PPE_LRELU;
+            }
+            return VPX_RESULT_SUCCESS;
+        }
         const int64_t zp = out_type->zero_point;
         const int64_t qMin = (int64_t)std::round(param0 / out_type->scale) + zp;
         const int64_t qMax = (int64_t)std::round(param1 / out_type->scale) + zp;

@@ -80,7 +80,7 @@ ELTWISE_ADD, ELTWISE_SUBTRACT = 0, 1
 
 # every symbol include/vpx_runtime.h and include/vpx_compiler_utils.h declare
 EXPORTS = ["vpx_get_last_error", "vpx_get_version", "vpx_sw_kernel_launch", "vpx_sw_kernel_supported",
-           "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_approximate",
+           "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_set_tuning", "vpx_approximate",
            "vpx_eltwise_quantization_approximation", "vpx_wt_get_scale", "vpx_wt_get_bias", "vpx_get_weights_table",
            "vpx_retrieve_ppe_int", "vpx_generate_softmax_attr", "vpx_get_quant_params_attr", "vpx_create_kernel_params", "vpx_get_kernel_info",
            "vpx_float_to_half_bits", "vpx_half_bits_to_float"]
@@ -123,6 +123,7 @@ def lib():
         L.vpx_sw_kernel_launch.argtypes = [C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(MemRefAddr), C.c_uint32,
                                            C.c_void_p]
         L.vpx_nce_task.argtypes = [C.POINTER(NceTask), C.c_void_p]
+        L.vpx_set_tuning.argtypes = [C.c_char_p, C.c_char_p]
         L.vpx_approximate.argtypes = [C.c_int, C.c_double] + [C.POINTER(C.c_int64)] * 3
         L.vpx_eltwise_quantization_approximation.argtypes = [C.c_double] * 3 + [C.c_int] + [C.POINTER(C.c_int64)] * 4
         L.vpx_wt_get_scale.restype = C.c_int32
@@ -509,6 +510,11 @@ def nce_matmul(a, b_nk, weight_table, out, ppe, zp_a=0, zp_b=0, zp_out=0, stream
     Nn, _ = b_nk.shape
     return nce_task(a.view(1, M, 1, K), b_nk.view(Nn, 1, 1, K), weight_table, out.view(1, M, 1, Nn), ppe, zp_in=zp_a,
                     zp_w=zp_b, zp_out=zp_out, stream=stream)
+
+
+def set_tuning(knob, value=None):
+    """Override the NCE dispatcher (tests, tuning): knob is a VPX_* name, value a string or None for the default."""
+    check(lib().vpx_set_tuning(knob.encode(), None if value is None else str(value).encode()))
 
 
 def nce_last_kernel():
