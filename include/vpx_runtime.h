@@ -69,6 +69,19 @@ typedef struct vpx_memref_addr_t {
 VPX_API int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_size,
                                  const vpx_memref_addr_t* addrs, uint32_t num_addrs, void* stream);
 
+/* The same launch for callers that cannot allocate device memory (code under HIP graph capture on a stream the
+ * library has not seen, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Kernels that need scratch memory (mvn1 / mvn6 chunk moments, the MVN-1 decomposition's partial sums,
+ * dynamic_quantize's range pass, per-axis quantize / dequantize tables) take it from one fixed array of
+ * VPX_NOALLOC_SCRATCH_BYTES in device memory that the library holds on every device it runs on; a launch that
+ * would need more returns VPX_RESULT_ERROR_OUT_OF_MEMORY and enqueues nothing.  The call performs no hipMalloc /
+ * hipFree.  All calls on one device share that array and it keeps the previous call's contents: calls through
+ * this entry point that may overlap on one device (different streams, or different threads) race; order them on
+ * one stream.  Arguments, results and errors are otherwise those of vpx_sw_kernel_launch. */
+#define VPX_NOALLOC_SCRATCH_BYTES (4u << 20)
+VPX_API int vpx_sw_kernel_launch_noalloc(const char* entry, const void* params, size_t params_size,
+                                         const vpx_memref_addr_t* addrs, uint32_t num_addrs, void* stream);
+
 /* 1 when `entry` names a kernel this library implements, else 0. */
 VPX_API int vpx_sw_kernel_supported(const char* entry);
 

@@ -34,30 +34,86 @@ const char* dtype_name(uint32_t t) {
 }
 
 // ---- scratch memory ---------------------------------------------------------------------------
+// Two providers behind get_workspace():
+//  * a grown-on-demand block per (device, stream handle), allocated with hipMalloc (vpx_workspace_reserve sizes it
+//    ahead of time; vpx_workspace_release frees it).  Growing is refused while the stream is capturing.
+//  * a fixed array in device memory for the entry point that may not allocate (vpx_sw_kernel_launch_noalloc).
 namespace {
 struct Scratch {
     void* ptr = nullptr;
     size_t size = 0;
+    std::vector<void*> retired;  // outgrown blocks: work already queued may still use them, freed on release
 };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, Scratch> g_ws;
+
+// The fixed scratch array.  Its name is a host-side handle, not a device address: host code uses the per-device
+// address that hipGetSymbolAddress returns (each device holds its own copy of the array).
+static __device__ __align__(256) unsigned char scratch[VPX_NOALLOC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+void* g_static_scratch[kMaxDevices] = {};  // guarded by g_ws_mutex
+thread_local bool t_noalloc = false;
+
+bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return st != hipStreamCaptureStatusNone;
+}
+
+int grow_workspace(Scratch& sc, hipStream_t stream, size_t bytes) {
+    if (sc.size >= bytes) return VPX_RESULT_SUCCESS;
+    VPX_REQUIRE(!stream_is_capturing(stream), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                "the stream is capturing and its scratch block (%zu bytes) is smaller than the %zu bytes this launch needs: "
+                "call vpx_workspace_reserve before the capture, or use vpx_sw_kernel_launch_noalloc",
+                sc.size, bytes);
+    size_t want = 64 * 1024;
+    while (want < bytes) want *= 2;
+    void* p = nullptr;
+    VPX_HIP_CHECK(hipMalloc(&p, want));
+    if (sc.ptr) sc.retired.push_back(sc.ptr);
+    sc.ptr = p;
+    sc.size = want;
+    return VPX_RESULT_SUCCESS;
+}
+
+// Device address of the fixed scratch array on the current device (looked up once per device).
+int static_scratch_address(void** out) {
+    int dev = 0;
+    VPX_HIP_CHECK(hipGetDevice(&dev));
+    VPX_REQUIRE(dev >= 0 && dev < kMaxDevices, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "device ordinal %d is beyond the %d this library tracks",
+                dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    if (!g_static_scratch[dev]) {
+        void* p = nullptr;
+        VPX_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        VPX_REQUIRE(p != nullptr, VPX_RESULT_ERROR_UNKNOWN, "hipGetSymbolAddress returned a null address for the scratch array");
+        g_static_scratch[dev] = p;
+    }
+    *out = g_static_scratch[dev];
+    return VPX_RESULT_SUCCESS;
+}
 }  // namespace
 
+bool noalloc_call() {
+    return t_noalloc;
+}
+
 int get_workspace(hipStream_t stream, size_t bytes, void** out) {
+    if (t_noalloc) {
+        VPX_REQUIRE(bytes <= (size_t)VPX_NOALLOC_SCRATCH_BYTES, VPX_RESULT_ERROR_OUT_OF_MEMORY,
+                    "this launch needs %zu bytes of scratch memory; the allocation-free entry point holds %zu", bytes,
+                    (size_t)VPX_NOALLOC_SCRATCH_BYTES);
+        return static_scratch_address(out);
+    }
     int dev = 0;
     VPX_HIP_CHECK(hipGetDevice(&dev));
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     Scratch& sc = g_ws[std::make_pair(dev, stream)];
-    if (sc.size < bytes) {
-        size_t want = 64 * 1024;
-        while (want < bytes) want *= 2;
-        void* p = nullptr;
-        VPX_HIP_CHECK(hipMalloc(&p, want));
-        // Work already queued on this stream may still use the old block, so it is kept until the
-        // process ends; sizes double, which bounds the total at twice the largest request.
-        sc.ptr = p;
-        sc.size = want;
-    }
+    const int rc = grow_workspace(sc, stream, bytes);
+    if (rc) return rc;
     *out = sc.ptr;
     return VPX_RESULT_SUCCESS;
 }
@@ -389,9 +445,8 @@ const char* vpx_sw_kernel_name(uint32_t i) {
     return i < kNumEntries ? kEntries[i].name : nullptr;
 }
 
-int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_size, const vpx_memref_addr_t* addrs,
-                         uint32_t num_addrs, void* stream) {
-    last_error().clear();
+static int sw_kernel_launch(const char* entry, const void* params, size_t params_size, const vpx_memref_addr_t* addrs,
+                            uint32_t num_addrs, void* stream) {
     VPX_REQUIRE(entry != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "kernel entry name is null");
     VPX_REQUIRE(params != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "%s: params blob is null", entry);
     VPX_REQUIRE(addrs != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "%s: memref address table is null", entry);
@@ -505,6 +560,26 @@ int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_si
     }
     default: return fail(VPX_RESULT_ERROR_UNKNOWN, "%s: no dispatcher", entry);
     }
+}
+
+int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_size, const vpx_memref_addr_t* addrs,
+                         uint32_t num_addrs, void* stream) {
+    last_error().clear();
+    return sw_kernel_launch(entry, params, size_t(params_size), addrs, num_addrs, stream);
+}
+
+int vpx_sw_kernel_launch_noalloc(const char* entry, const void* params, size_t params_size, const vpx_memref_addr_t* addrs,
+                                 uint32_t num_addrs, void* stream) {
+    last_error().clear();
+    // set-up, once per device: the device address of the fixed scratch array
+    void* fixed = nullptr;
+    const int rc = static_scratch_address(&fixed);
+    if (rc) return rc;
+    struct Mode {
+        Mode() { t_noalloc = true; }
+        ~Mode() { t_noalloc = false; }
+    } mode;  // get_workspace() hands out `fixed` instead of allocating while this call runs on this thread
+    return sw_kernel_launch(entry, params, params_size, addrs, num_addrs, stream);
 }
 
 int vpx_nce_task(const vpx_nce_task_t* t, void* stream) {

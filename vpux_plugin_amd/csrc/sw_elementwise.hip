@@ -1708,7 +1708,7 @@ int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t
                 *table = e.table;
                 return VPX_RESULT_SUCCESS;
             }
-        keep = g_axis_tables.size() < kMaxAxisTables;
+        keep = g_axis_tables.size() < kMaxAxisTables && !noalloc_call();
     }
     void* mem = nullptr;
     if (keep) {

@@ -80,6 +80,9 @@ struct NdIndex {
 // Library-owned scratch memory, one buffer per (device, stream): calls on one stream are ordered,
 // so they can share it; calls on different streams get different buffers.
 int get_workspace(hipStream_t stream, size_t bytes, void** out);
+// True while the calling thread is inside the entry point that may not allocate: get_workspace() then hands out the
+// fixed scratch array (at most VPX_NOALLOC_SCRATCH_BYTES), and launchers must not call hipMalloc for caches of their own.
+bool noalloc_call();
 
 // Dispatch override for tests and tuning (knob names are those of the VPX_* environment variables, read once).
 int set_tuning(const char* knob, const char* value);

@@ -79,7 +79,7 @@ ELTWISE_ADD, ELTWISE_SUBTRACT = 0, 1
 
 
 # every symbol include/vpx_runtime.h and include/vpx_compiler_utils.h declare
-EXPORTS = ["vpx_get_last_error", "vpx_get_version", "vpx_sw_kernel_launch", "vpx_sw_kernel_supported",
+EXPORTS = ["vpx_get_last_error", "vpx_get_version", "vpx_sw_kernel_launch", "vpx_sw_kernel_launch_noalloc", "vpx_sw_kernel_supported",
            "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_set_tuning", "vpx_approximate",
            "vpx_eltwise_quantization_approximation", "vpx_wt_get_scale", "vpx_wt_get_bias", "vpx_get_weights_table",
            "vpx_retrieve_ppe_int", "vpx_generate_softmax_attr", "vpx_get_quant_params_attr", "vpx_create_kernel_params", "vpx_get_kernel_info",
@@ -122,6 +122,7 @@ def lib():
         L.vpx_nce_last_kernel.restype = C.c_char_p
         L.vpx_sw_kernel_launch.argtypes = [C.c_char_p, C.c_void_p, C.c_size_t, C.POINTER(MemRefAddr), C.c_uint32,
                                            C.c_void_p]
+        L.vpx_sw_kernel_launch_noalloc.argtypes = L.vpx_sw_kernel_launch.argtypes
         L.vpx_nce_task.argtypes = [C.POINTER(NceTask), C.c_void_p]
         L.vpx_set_tuning.argtypes = [C.c_char_p, C.c_char_p]
         L.vpx_approximate.argtypes = [C.c_int, C.c_double] + [C.POINTER(C.c_int64)] * 3
@@ -302,16 +303,21 @@ def _stream_handle(stream):
     return C.c_void_p(stream.cuda_stream)
 
 
-def sw_kernel_launch(entry, blob, operands, stream=None, side_dims=False):
+NOALLOC_SCRATCH_BYTES = 4 << 20  # VPX_NOALLOC_SCRATCH_BYTES
+
+
+def sw_kernel_launch(entry, blob, operands, stream=None, side_dims=False, noalloc=False):
     """Launch `entry` with the serialized blob; operands supply the device addresses.  With
-    side_dims=True dims/strides travel in the address table instead of the blob tail."""
+    side_dims=True dims/strides travel in the address table instead of the blob tail; with noalloc=True
+    the call goes through vpx_sw_kernel_launch_noalloc (fixed scratch array, no device allocation)."""
     addrs = (MemRefAddr * len(operands))()
     for i, o in enumerate(operands):
         addrs[i].data = o.t.data_ptr()
         if side_dims:
             addrs[i].dims = C.cast(o.dims, C.POINTER(C.c_int32))
             addrs[i].strides = C.cast(o.strides, C.POINTER(C.c_int64))
-    check(lib().vpx_sw_kernel_launch(entry.encode(), blob, len(blob), addrs, len(operands), _stream_handle(stream)))
+    fn = lib().vpx_sw_kernel_launch_noalloc if noalloc else lib().vpx_sw_kernel_launch
+    check(fn(entry.encode(), blob, len(blob), addrs, len(operands), _stream_handle(stream)))
 
 
 def _i64(*vals):
@@ -367,10 +373,10 @@ def fake_quantize(x, in_lo, in_hi, out_lo, out_hi, levels, out, order=None, stre
     return out
 
 
-def quantize(x, out, scale, zero_point, order=None, stream=None):
+def quantize(x, out, scale, zero_point, order=None, stream=None, noalloc=False):
     ops = [Operand(x, order), Operand(out, order)]
     attrs = get_quant_params_attr(scale, zero_point, _torch_dtype_code(x)).tobytes()
-    sw_kernel_launch("quantize", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    sw_kernel_launch("quantize", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream, noalloc=noalloc)
     return out
 
 
@@ -381,11 +387,11 @@ def dequantize(q, out, scale, zero_point, order=None, stream=None):
     return out
 
 
-def mvn(x, out, across_channels, normalize_variance, eps, order="NCHW", stream=None):
+def mvn(x, out, across_channels, normalize_variance, eps, order="NCHW", stream=None, noalloc=False):
     ops = [Operand(x, order), Operand(out, order)]
     # a true boolean attribute serialises as int64 -1 (sign-extended i1)
     attrs = _i64(-1 if across_channels else 0, -1 if normalize_variance else 0) + np.float32(eps).tobytes()
-    sw_kernel_launch("mvn1", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    sw_kernel_launch("mvn1", create_kernel_params(ops[:1], ops[1:], attrs), ops, stream, noalloc=noalloc)
     return out
 
 
@@ -416,10 +422,10 @@ def mvn1_norm(x, mean_var, out, across_channels, normalize_variance, order="NCHW
     return out
 
 
-def dynamic_quantize(x, out, scale, zero_point, order=None, stream=None):
+def dynamic_quantize(x, out, scale, zero_point, order=None, stream=None, noalloc=False):
     """x: float32; out: uint8 of x's shape; scale: float32[1]; zero_point: uint8[1] (all written by the kernel)."""
     ops = [Operand(x, order), Operand(out, order), Operand(scale), Operand(zero_point)]
-    sw_kernel_launch("dynamic_quantize", create_kernel_params(ops[:1], ops[1:]), ops, stream)
+    sw_kernel_launch("dynamic_quantize", create_kernel_params(ops[:1], ops[1:]), ops, stream, noalloc=noalloc)
     return out, scale, zero_point
 
 
