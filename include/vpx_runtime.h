@@ -82,6 +82,21 @@ VPX_API int vpx_sw_kernel_launch(const char* entry, const void* params, size_t p
 VPX_API int vpx_sw_kernel_launch_noalloc(const char* entry, const void* params, size_t params_size,
                                          const vpx_memref_addr_t* addrs, uint32_t num_addrs, void* stream);
 
+/* Scratch memory of vpx_sw_kernel_launch and vpx_nce_task (no counterpart in the reference, whose kernels get
+ * their buffers from the compiler's memory scheduler).  The library keeps one block per (device, stream handle) and
+ * grows it with hipMalloc when a launch needs more: mvn1 / mvn6 / mvn1_sum with several chunks per group (12 bytes
+ * per 4096 values), dynamic_quantize, per-axis quantize / dequantize tables, and an NCE task with a non-zero
+ * activation zero point, unsigned weights or a weight zero point (4 bytes per output channel and per output
+ * position, plus a signed copy of unsigned weights).  A launch on a capturing stream that would have to grow the
+ * block returns VPX_RESULT_ERROR_UNSUPPORTED_FEATURE instead.
+ * vpx_workspace_reserve grows the block of `stream` on the current device to at least `bytes` ahead of time (before
+ * a capture, or to keep hipMalloc out of a serving loop).  vpx_workspace_release waits for the stream, then frees
+ * its block, the blocks it outgrew and the per-axis tables cached for it; the next launch allocates afresh.
+ * Blocks are keyed by the stream HANDLE: release before destroying a stream (a new stream may get the same
+ * handle), and do not run one handle's work concurrently from several threads' per-thread streams. */
+VPX_API int vpx_workspace_reserve(void* stream, size_t bytes);
+VPX_API int vpx_workspace_release(void* stream);
+
 /* 1 when `entry` names a kernel this library implements, else 0. */
 VPX_API int vpx_sw_kernel_supported(const char* entry);
 
@@ -174,6 +189,12 @@ typedef struct vpx_nce_task_t {
     int32_t zp_in, zp_w, zp_out;
     vpx_ppe_int_t ppe;
     int32_t eltwise_type; /* vpx_eltwise_type_t, ELTWISE tasks only */
+    /* VPU.NCE.MatMul's group dimension (tblgen/vpux/compiler/dialect/VPU/ops.td:228-357: input [G,1,K,M,1],
+     * weights [G,N,K,1,1], weight table [G,N,1,1,4], all GNHWC in memory): `groups` independent CONV tasks of the
+     * shape above whose inputs, weights, weight tables and outputs lie one after the other, densely, behind the four
+     * pointers.  0 and 1 both mean a single task.  A matmul the MFMA matmul kernel serves is one launch for all
+     * groups (the group on the grid's second dimension, one column-sum pass over all groups' weights). */
+    int32_t groups;
 } vpx_nce_task_t;
 
 VPX_API int vpx_nce_task(const vpx_nce_task_t* task, void* stream);

@@ -225,13 +225,29 @@ void orc_dequantize_f16(const void* q, int in_is_signed, uint16_t* y, int64_t ou
 
 /* ------------------------------------------------------------------ Eltwise */
 
+/* Minimum / Maximum (OpenVINO operator semantics; the kernel sources are absent, so parity unpinned): IEEE 754-2008
+ * minNum / maxNum -- a NaN operand yields the other operand, NaN only when both are -- with -0 ordered below +0, so
+ * that the result is one definite bit pattern for every pair of inputs. */
+static float elt_min(float a, float b) {
+    if (isnan(a)) return b;
+    if (isnan(b)) return a;
+    if (a == b) return signbit(a) ? a : b;
+    return a < b ? a : b;
+}
+static float elt_max(float a, float b) {
+    if (isnan(a)) return b;
+    if (isnan(b)) return a;
+    if (a == b) return signbit(a) ? b : a;
+    return a > b ? a : b;
+}
+
 static float elt_apply(int op, float a, float b) {
     switch (op) {
     case ORC_ELT_ADD: return a + b;
     case ORC_ELT_SUB: return a - b;
     case ORC_ELT_MUL: return a * b;
-    case ORC_ELT_MIN: return fminf(a, b);
-    case ORC_ELT_MAX: return fmaxf(a, b);
+    case ORC_ELT_MIN: return elt_min(a, b);
+    case ORC_ELT_MAX: return elt_max(a, b);
     case ORC_ELT_DIV: return a / b;
     case ORC_ELT_PRELU: return a < 0.0f ? a * b : a;
     default: return 0.0f;

@@ -278,6 +278,38 @@ def test_ppe_modes_and_rounding_edges(rt, orc, dev, mode):
     assert got.min() >= -100 and got.max() <= 90
 
 
+@pytest.mark.parametrize("G,M,K,N,in_u8,zp_a,w_u8,zp_b,out_f16,kernel", [
+    (3, 300, 128, 520, False, 3, False, 0, False, "nce_gemm_mfma"),    # one launch, column sums of all groups in one pass
+    (5, 64, 64, 48, True, 121, False, 0, False, "nce_gemm_mfma"),      # 128 x 128 tiles, short K
+    (2, 256, 192, 320, True, 7, True, 131, False, "nce_gemm_mfma"),    # weight zero point: per-position term, M % 4 == 0
+    (2, 130, 128, 96, False, -2, False, 0, True, "nce_gemm_mfma"),     # fp16 output
+    (3, 33, 128, 80, True, 9, True, 120, False, "nce_gemm_mfma"),      # weight zero point with M % 4 != 0: group after group
+    (2, 40, 48, 72, False, 1, False, 0, False, "nce_conv_mfma16"),     # K not a multiple of 64: group after group
+])
+def test_grouped_matmul_one_task(rt, orc, dev, G, M, K, N, in_u8, zp_a, w_u8, zp_b, out_f16, kernel):
+    """VPU.NCE.MatMul with G groups ([G,1,K,M,1] x [G,N,K,1,1], weight table [G,N,1,1,4]) as one task: bit-exact against
+    G separate runs of the oracle."""
+    import torch
+    rng = np.random.default_rng(400 + G * M)
+    a = rng.integers(0, 256, (G, M, K), dtype=np.uint8) if in_u8 else rng.integers(-128, 128, (G, M, K)).astype(np.int8)
+    b = rng.integers(0, 256, (G, N, K), dtype=np.uint8) if w_u8 else rng.integers(-127, 128, (G, N, K)).astype(np.int8)
+    wt = np.stack([rt.make_weights_table(rng.integers(2 ** 14, 2 ** 15, N), rng.integers(16, 22, N),
+                                         rng.integers(-2 ** 15, 2 ** 15, N).astype(np.int32), K) for _ in range(G)])
+    if out_f16:
+        ppe, op = rt.PpeInt(rt.PPE_LPRELU, -(2 ** 31), 2 ** 31 - 1, 1638, 14), orc.ppe(1638, 14, 0, -(2 ** 31), 2 ** 31 - 1)
+    else:
+        ppe, op = rt.PpeInt(rt.PPE_LPRELU, -128, 127, 1638, 14), orc.ppe(1638, 14, 5, -128, 127)
+    out = torch.full((G, M, N), 77, dtype=torch.float16 if out_f16 else torch.int8, device=dev)
+    rt.nce_matmul(dev_t(a, dev), dev_t(b, dev), dev_t(wt, dev), out, ppe, zp_a=zp_a, zp_b=zp_b, zp_out=0 if out_f16 else 5)
+    torch.cuda.synchronize()
+    assert rt.nce_last_kernel() == kernel
+    got = out.cpu().numpy()
+    for g in range(G):
+        want = orc.nce_matmul(a[g], b[g], wt[g], op, zp_a=zp_a, zp_b=zp_b, out_f16=out_f16)
+        gg = got[g].view(np.uint16) if out_f16 else got[g]
+        assert np.array_equal(gg, want), "group %d: %d mismatches" % (g, int((gg != want).sum()))
+
+
 F16_NONE = {"clamp_low": -(2 ** 31), "clamp_high": 2 ** 31 - 1}
 
 
@@ -552,6 +584,65 @@ def test_chain_replayed_from_a_hip_graph(rt, orc, dev):
         chain(*scratch)  # eager work between replays, on the default stream
         torch.cuda.synchronize()
         assert torch.equal(scratch[2], eager[2])
+
+
+def test_workspace_reserve_release_and_cold_capture(rt, orc, dev):
+    """A launch that needs scratch memory on a capturing stream the library has not seen is refused (it would have to
+    call hipMalloc inside the capture); after vpx_workspace_reserve the same capture goes through and replays to the
+    eager result; vpx_workspace_release frees the block and the next launch allocates afresh."""
+    import torch
+    rng = np.random.default_rng(98)
+    x = torch.from_numpy(rng.normal(0, 2, (2, 64, 64, 64)).astype(np.float16)).to(dev)  # 64 chunks per group: chunk moments in scratch
+    eager = torch.empty_like(x)
+    rt.mvn(x, eager, True, True, 1e-9)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    y = torch.zeros_like(x)
+    graph = torch.cuda.CUDAGraph()
+    refused = []
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            try:
+                rt.mvn(x, y, True, True, 1e-9)
+            except rt.VpxError as err:
+                refused.append(err)
+            y.fill_(1)  # the capture itself stays valid and is ended normally
+    assert len(refused) == 1 and refused[0].code == rt.ERROR_UNSUPPORTED_FEATURE and "vpx_workspace_reserve" in refused[0].text
+    del graph
+    torch.cuda.synchronize()
+    rt.workspace_reserve(1 << 16, stream=stream)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            rt.mvn(x, y, True, True, 1e-9)
+    for _ in range(3):
+        y.fill_(3)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), eager.view(torch.int16))
+    del graph
+    rt.workspace_release(stream=stream)
+    rt.workspace_release(stream=stream)  # nothing left: still succeeds
+    with torch.cuda.stream(stream):
+        y.fill_(5)
+        rt.mvn(x, y, True, True, 1e-9)  # allocates a fresh block
+        # per-axis quantize tables are cached per stream and released with it
+        q = torch.empty((64, 24), dtype=torch.uint8, device=dev)
+        h = torch.from_numpy(rng.normal(0, 1, (64, 24)).astype(np.float16)).to(dev)
+        sc, zp = rng.uniform(0.01, 0.1, 24), rng.integers(100, 150, 24)
+        rt.quantize(h, q, sc, zp)
+        q2 = torch.empty_like(q)
+        rt.quantize(h, q2, sc, zp)  # cache hit
+    stream.synchronize()
+    assert torch.equal(y.view(torch.int16), eager.view(torch.int16)) and torch.equal(q, q2)
+    rt.workspace_release(stream=stream)
+    with torch.cuda.stream(stream):
+        q3 = torch.empty_like(q)
+        rt.quantize(h, q3, sc, zp)  # table rebuilt after the release
+    stream.synchronize()
+    assert torch.equal(q, q3)
+    rt.workspace_release(stream=stream)
 
 
 def test_two_host_threads_on_their_own_streams(rt, orc, dev):

@@ -101,17 +101,22 @@ def test_eltwise_random_bit_patterns(rt, orc, dev, op):
     n = 1_000_003
     a = rng.integers(0, 65536, n).astype(np.uint16)
     b = rng.integers(0, 65536, n).astype(np.uint16)
-    if op in ("min", "max"):  # NaN handling of fmin/fmax differs between libm and the GPU; keep NaNs out
-        a[is_nan16(a)] = 0x3c00
-        b[is_nan16(b)] = 0xbc00
+    if op in ("min", "max"):
+        # every pairing of special values: NaN with a number (the number wins), NaN with NaN, zeros of both signs
+        # (-0 is below +0), infinities
+        sp = np.array([0x7e00, 0xfe00, 0x7c01, 0x0000, 0x8000, 0x7c00, 0xfc00, 0x3c00, 0xbc00, 0x0001, 0x8001], np.uint16)
+        a[:sp.size ** 2] = np.repeat(sp, sp.size)
+        b[:sp.size ** 2] = np.tile(sp, sp.size)
     out = torch.empty(n, dtype=torch.float16, device=dev)
     rt.eltwise(op, to_dev(a, dev, True), to_dev(b, dev, True), out)
     got, want = f16_bits(out), orc.eltwise_f16(op, a, b)
-    if op in ("min", "max"):  # +0 / -0 order is unspecified for fmin/fmax
-        zero = ((got | want) & 0x7fff) == 0
-        got, want = got.copy(), want.copy()
-        got[zero] = 0
-        want[zero] = 0
+    if op in ("min", "max"):
+        k = 11 * 11
+        one_nan = is_nan16(a[:k]) ^ is_nan16(b[:k])
+        other = np.where(is_nan16(a[:k]), b[:k], a[:k])
+        assert np.array_equal(got[:k][one_nan], other[one_nan])  # a NaN operand yields the other operand
+        assert is_nan16(got[:k][is_nan16(a[:k]) & is_nan16(b[:k])]).all()
+        assert got[3 * 11 + 4] == (0x8000 if op == "min" else 0x0000) and got[4 * 11 + 3] == got[3 * 11 + 4]  # (+0, -0)
     assert_f16_exact(got, want, op)
 
 

@@ -651,3 +651,18 @@ def test_dynamic_quantize_onnx_examples(orc):
     back = orc.dynamic_dequantize(y, np.full((1,), sc, np.float32), np.full((1,), zp, np.uint8), to_f16=False)
     assert np.all(np.abs(back - x) <= 0.5 * sc * (1 + 1e-5))
 
+
+
+def test_eltwise_min_max_special_values(orc):
+    """Minimum / Maximum are IEEE minNum / maxNum with -0 below +0 (written out here case by case, not through the
+    C library): a NaN operand yields the other operand, two NaNs a NaN, and equal-comparing zeros keep the sign the
+    ordering asks for."""
+    nan, pz, nz, inf, ninf, one, mone = 0x7e00, 0x0000, 0x8000, 0x7c00, 0xfc00, 0x3c00, 0xbc00
+    a = np.array([nan, one, nan, pz, nz, inf, ninf, one, nz, pz], np.uint16)
+    b = np.array([one, nan, nan, nz, pz, one, one, mone, nz, pz], np.uint16)
+    mn = orc.eltwise_f16("min", a, b)
+    mx = orc.eltwise_f16("max", a, b)
+    assert mn[:2].tolist() == [one, one] and mx[:2].tolist() == [one, one]
+    assert (mn[2] & 0x7fff) > 0x7c00 and (mx[2] & 0x7fff) > 0x7c00
+    assert mn[3:].tolist() == [nz, nz, one, ninf, mone, nz, pz]
+    assert mx[3:].tolist() == [pz, pz, inf, one, one, nz, pz]

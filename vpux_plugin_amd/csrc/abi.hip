@@ -118,6 +118,32 @@ int get_workspace(hipStream_t stream, size_t bytes, void** out) {
     return VPX_RESULT_SUCCESS;
 }
 
+int workspace_reserve(hipStream_t stream, size_t bytes) {
+    int dev = 0;
+    VPX_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    return grow_workspace(g_ws[std::make_pair(dev, stream)], stream, bytes);
+}
+
+int workspace_release(hipStream_t stream) {
+    VPX_REQUIRE(!stream_is_capturing(stream), VPX_RESULT_ERROR_INVALID_ARGUMENT, "the stream is capturing: its scratch memory cannot be released");
+    // work already queued may still read or write the blocks
+    VPX_HIP_CHECK(hipStreamSynchronize(stream));
+    int dev = 0;
+    VPX_HIP_CHECK(hipGetDevice(&dev));
+    {
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        const auto it = g_ws.find(std::make_pair(dev, stream));
+        if (it != g_ws.end()) {
+            Scratch sc = it->second;
+            g_ws.erase(it);
+            for (void* p : sc.retired) VPX_HIP_CHECK(hipFree(p));
+            if (sc.ptr) VPX_HIP_CHECK(hipFree(sc.ptr));
+        }
+    }
+    return release_axis_tables(dev, stream);
+}
+
 // ---- blob parsing -----------------------------------------------------------------------------
 namespace {
 
@@ -606,6 +632,8 @@ int vpx_nce_task(const vpx_nce_task_t* t, void* stream) {
                             t->zp_out <= (1 << 20),
                     VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE eltwise: zero point out of range");
     }
+    VPX_REQUIRE(t->groups >= 0 && (t->groups <= 1 || !eltwise), VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                "NCE task: groups = %d (CONV tasks take 0, 1 or more; ELTWISE tasks 0 or 1)", t->groups);
     const auto is8 = [](int32_t ty) { return ty == VPX_NN_U8 || ty == VPX_NN_I8; };
     const bool f16_out = t->output_type == VPX_NN_FP16 && !eltwise;
     VPX_REQUIRE(is8(t->input_type) && is8(t->weights_type) && (is8(t->output_type) || f16_out), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
@@ -633,6 +661,16 @@ int vpx_nce_task(const vpx_nce_task_t* t, void* stream) {
     const int rc = launch_nce(*t, (hipStream_t)stream, &name);
     if (rc == VPX_RESULT_SUCCESS) g_last_nce_kernel = name;
     return rc;
+}
+
+int vpx_workspace_reserve(void* stream, size_t bytes) {
+    last_error().clear();
+    return workspace_reserve(static_cast<hipStream_t>(stream), bytes);
+}
+
+int vpx_workspace_release(void* stream) {
+    last_error().clear();
+    return workspace_release(static_cast<hipStream_t>(stream));
 }
 
 int vpx_set_tuning(const char* knob, const char* value) {

@@ -485,6 +485,16 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
 
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
+    // Grouped matmul: blockIdx.y is the group; every operand holds the groups one after the other.
+    if (const int64_t grp = blockIdx.y) {
+        A += grp * M * K;
+        B += grp * N * K;
+        wt += grp * N * 4;
+        if (colsum) colsum += grp * N;
+        out += grp * M * N * (OUT == OUT_F16 ? 2 : 1);
+        if (ppe.rowterm) ppe.rowterm += grp * M;
+    }
+
     // Workgroup ids are dealt round-robin to the 8 XCDs.  Give each XCD a contiguous run of tile
     // ids and walk tiles in groups of 4 tile-rows, so that workgroups resident on one XCD at the
     // same time share A and B panels in that XCD's L2.
@@ -1681,6 +1691,25 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     // to the convolution kernels, whose tiles are 64 channels wide (measured 7 us against 18 us at [100352 x 64 x 64]).
     const int64_t gemm_tiles = ((Mtot + 255) / 256) * ((g.OC + 255) / 256);
     const bool use_gemm = allow_gemm && is_gemm && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || Mtot < 1024);
+    // VPU.NCE.MatMul's groups: one launch of the matmul kernel when it serves the shape (the preparation passes then
+    // walk all groups' weights / activations as one tensor), else one task after the other on the stream.
+    const int64_t G = t.groups > 1 ? t.groups : 1;
+    const bool one_launch = G > 1 && allow_mfma && mfma_ok && aligned && use_gemm && (wz_rest == 0 || Mtot % 4 == 0) && G <= 65535 &&
+                            G * g.OC < (1ll << 31) && G * Mtot < (1ll << 31);
+    if (G > 1 && !one_launch) {
+        const int64_t out_bytes = out_f16 ? 2 : 1;
+        for (int64_t grp = 0; grp < G; grp++) {
+            vpx_nce_task_t sub = t;
+            sub.groups = 1;
+            sub.input = (const char*)t.input + grp * g.N * g.H * g.W * g.IC;
+            sub.weights = (const char*)t.weights + grp * g.OC * Ktot;
+            sub.weight_table = t.weight_table + grp * g.OC * 4;
+            sub.output = (char*)t.output + grp * Mtot * g.OC * out_bytes;
+            const int rc = launch_nce(sub, s, kernel_name);
+            if (rc) return rc;
+        }
+        return VPX_RESULT_SUCCESS;
+    }
     const void* wptr = t.weights;  // the signed weights the MFMA kernels read
     size_t wofs = 0;               // scratch bytes taken by their re-biased copy
     const auto scratch = [&](size_t bytes, void** out) {
@@ -1691,17 +1720,18 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     };
     const int32_t* rowterm = nullptr;  // the per-position term of the weight zero point, when there is one
     const auto rebias_weights = [&]() -> int {
-        const size_t wbytes = w_rebias ? ((size_t)g.OC * (size_t)Ktot + 255) / 256 * 256 : 0;
-        const int64_t pixels = g.N * g.H * g.W;
+        // (G > 1 here only on the matmul path: all groups' weights and pixels are walked as one tensor)
+        const size_t wbytes = w_rebias ? ((size_t)(G * g.OC) * (size_t)Ktot + 255) / 256 * 256 : 0;
+        const int64_t pixels = G * g.N * g.H * g.W;
         const bool direct = is_gemm;  // every output position is one input pixel
         constexpr int64_t kRowPad = 32 * kPatchMaxMT + 256;  // edge tiles read past the last position
-        const size_t rbytes = wz_rest != 0 ? (size_t)(Mtot + kRowPad + (direct ? 0 : pixels)) * sizeof(int32_t) : 0;
+        const size_t rbytes = wz_rest != 0 ? (size_t)(G * Mtot + kRowPad + (direct ? 0 : pixels)) * sizeof(int32_t) : 0;
         if (wbytes + rbytes == 0) return VPX_RESULT_SUCCESS;
         void* base = nullptr;
         const int r = get_workspace(s, wbytes + (rbytes + 255) / 256 * 256, &base);
         if (r) return r;
         if (w_rebias) {
-            const int64_t n_vec = (int64_t)g.OC * Ktot / 16;
+            const int64_t n_vec = G * g.OC * Ktot / 16;
             const int64_t blocks = (n_vec + 255) / 256;
             hipLaunchKernelGGL(nce_weights_to_s8_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, s,
                                (const i32x4*)t.weights, (i32x4*)base, n_vec);
@@ -1710,7 +1740,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         }
         if (wz_rest != 0) {
             int32_t* rt = (int32_t*)((char*)base + wbytes);
-            int32_t* cs = direct ? rt : rt + Mtot + kRowPad;
+            int32_t* cs = direct ? rt : rt + G * Mtot + kRowPad;
             int lpp = 1;
             while (lpp < g.IC / 16 && lpp < 64) lpp *= 2;
             const int64_t blocks = (pixels * lpp + 255) / 256;
@@ -1758,7 +1788,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             // that the lower LDS traffic of four 128x128 waves wins.  VPX_GEMM_WAVES=4|8 overrides.
             const int waves_knob = knobs.gemm_waves.load();
             const int nw = tile == 128 ? 4 : (waves_knob ? waves_knob : (g.IC > 4096 ? 4 : 8));
-            const dim3 grid((unsigned)(per_xcd * 8)), block(64 * nw);
+            const dim3 grid((unsigned)(per_xcd * 8), (unsigned)G), block(64 * nw);
             const int64_t nk = g.IC / 64;
             const bool shortk = tile == 128 && nk <= 3 && !out_f16;
             size_t lds = 4 * (size_t)(tile + tile) * 64;  // four K panels; the output staging tile reuses them
@@ -1770,11 +1800,11 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             int32_t* colsum = nullptr;
             if (corr != 0) {
                 void* ws = nullptr;
-                rc = scratch(sizeof(int32_t) * (size_t)g.OC, &ws);
+                rc = scratch(sizeof(int32_t) * (size_t)(G * g.OC), &ws);
                 if (rc) return rc;
                 colsum = (int32_t*)ws;
-                hipLaunchKernelGGL(nce_colsum_kernel, dim3((unsigned)((g.OC + 3) / 4)), dim3(256), 0, s,
-                                   (const int8_t*)wptr, colsum, g.OC, Ktot);
+                hipLaunchKernelGGL(nce_colsum_kernel, dim3((unsigned)((G * g.OC + 3) / 4)), dim3(256), 0, s,
+                                   (const int8_t*)wptr, colsum, G * g.OC, Ktot);
                 VPX_HIP_CHECK(hipGetLastError());
             }
 #define VPX_GEMM_W(U8, SGN, NW, TILE, SHORTK)                                                                        \

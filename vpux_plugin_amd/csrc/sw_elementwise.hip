@@ -10,6 +10,7 @@
 
 #include <cstring>
 #include <mutex>
+#include <unordered_map>
 #include <vector>
 
 namespace vpx {
@@ -1656,7 +1657,8 @@ __global__ __launch_bounds__(kBlock) void dequantize_axis_inner_kernel(const TQ*
 }
 
 // Tables already on the device, by content: the parameters of a layer are constants, so after the first call a
-// per-axis launch is one kernel.  Entries are per (device, stream) like the workspace, and live until the process ends.
+// per-axis launch is one kernel.  Entries belong to a (device, stream) like the workspace and are found through a
+// 64-bit hash of the parameter bytes (a hit is confirmed by comparing them); vpx_workspace_release frees them.
 struct AxisTableEntry {
     int dev;
     hipStream_t stream;
@@ -1664,8 +1666,23 @@ struct AxisTableEntry {
     float4* table;
 };
 std::mutex g_axis_mutex;
-std::vector<AxisTableEntry> g_axis_tables;
+std::unordered_multimap<uint64_t, AxisTableEntry> g_axis_tables;
 constexpr size_t kMaxAxisTables = 64;
+
+uint64_t axis_key(int dev, hipStream_t s, const float* a, const float* b, int64_t n) {
+    uint64_t h = 0xcbf29ce484222325ull ^ (uint64_t)(uint32_t)dev ^ ((uint64_t)(uintptr_t)s << 7);
+    auto mix = [&h](const float* v, int64_t cnt) {
+        for (int64_t i = 0; i < cnt; i++) {
+            uint32_t w;
+            memcpy(&w, v + i, 4);
+            h = (h ^ w) * 0x100000001b3ull;
+            h ^= h >> 29;
+        }
+    };
+    mix(a, n);
+    mix(b, n);
+    return h;
+}
 
 int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t n, const float* a, const float* b, hipStream_t s,
                AxisGeom& g, float4** table) {
@@ -1700,15 +1717,25 @@ int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t
     int dev = 0;
     VPX_HIP_CHECK(hipGetDevice(&dev));
     bool keep = false;
+    const uint64_t key = axis_key(dev, s, a, b, n);
     {
         std::lock_guard<std::mutex> lock(g_axis_mutex);
-        for (const AxisTableEntry& e : g_axis_tables)
+        const auto range = g_axis_tables.equal_range(key);
+        for (auto it = range.first; it != range.second; ++it) {
+            const AxisTableEntry& e = it->second;
             if (e.dev == dev && e.stream == s && (int64_t)e.a.size() == n && memcmp(e.a.data(), a, sizeof(float) * (size_t)n) == 0 &&
                 memcmp(e.b.data(), b, sizeof(float) * (size_t)n) == 0) {
                 *table = e.table;
                 return VPX_RESULT_SUCCESS;
             }
+        }
         keep = g_axis_tables.size() < kMaxAxisTables && !noalloc_call();
+    }
+    // a table built under stream capture would need a hipMalloc inside the capture: take the workspace instead
+    if (keep) {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &st) != hipSuccess) (void)hipGetLastError();
+        else if (st != hipStreamCaptureStatusNone) keep = false;
     }
     void* mem = nullptr;
     if (keep) {
@@ -1731,7 +1758,7 @@ int axis_setup(const char* what, const MemRef& ref, const MemRef& other, int64_t
     }
     if (keep) {
         std::lock_guard<std::mutex> lock(g_axis_mutex);
-        g_axis_tables.push_back(AxisTableEntry{dev, s, std::vector<float>(a, a + n), std::vector<float>(b, b + n), *table});
+        g_axis_tables.emplace(key, AxisTableEntry{dev, s, std::vector<float>(a, a + n), std::vector<float>(b, b + n), *table});
     }
     return VPX_RESULT_SUCCESS;
 }
@@ -1923,6 +1950,19 @@ int dequantize_axis_impl(const MemRef& in, const MemRef& out, const double* scal
 }
 
 }  // namespace
+
+int release_axis_tables(int dev, hipStream_t s) {
+    std::lock_guard<std::mutex> lock(g_axis_mutex);
+    for (auto it = g_axis_tables.begin(); it != g_axis_tables.end();) {
+        if (it->second.dev == dev && it->second.stream == s) {
+            VPX_HIP_CHECK(hipFree(it->second.table));
+            it = g_axis_tables.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    return VPX_RESULT_SUCCESS;
+}
 
 int launch_quantize_per_axis(const MemRef& in, const MemRef& out, const double* scales, const int64_t* zps, int64_t n,
                              hipStream_t s) {

@@ -83,6 +83,8 @@ int get_workspace(hipStream_t stream, size_t bytes, void** out);
 // True while the calling thread is inside the entry point that may not allocate: get_workspace() then hands out the
 // fixed scratch array (at most VPX_NOALLOC_SCRATCH_BYTES), and launchers must not call hipMalloc for caches of their own.
 bool noalloc_call();
+// Frees the per-axis quantization tables cached for (device, stream); the caller has drained the stream.
+int release_axis_tables(int dev, hipStream_t stream);
 
 // Dispatch override for tests and tuning (knob names are those of the VPX_* environment variables, read once).
 int set_tuning(const char* knob, const char* value);

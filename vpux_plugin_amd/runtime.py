@@ -71,7 +71,7 @@ class NceTask(C.Structure):
                 ("output_type", C.c_int32), ("N", C.c_int64), ("H", C.c_int64), ("W", C.c_int64), ("IC", C.c_int64),
                 ("OC", C.c_int64), ("kernel_size", C.c_int32 * 2), ("kernel_strides", C.c_int32 * 2),
                 ("kernel_padding", C.c_int32 * 4), ("zp_in", C.c_int32), ("zp_w", C.c_int32), ("zp_out", C.c_int32),
-                ("ppe", PpeInt), ("eltwise_type", C.c_int32)]
+                ("ppe", PpeInt), ("eltwise_type", C.c_int32), ("groups", C.c_int32)]
 
 
 NCE_CONV, NCE_ELTWISE = 0, 4
@@ -80,7 +80,7 @@ ELTWISE_ADD, ELTWISE_SUBTRACT = 0, 1
 
 # every symbol include/vpx_runtime.h and include/vpx_compiler_utils.h declare
 EXPORTS = ["vpx_get_last_error", "vpx_get_version", "vpx_sw_kernel_launch", "vpx_sw_kernel_launch_noalloc", "vpx_sw_kernel_supported",
-           "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_set_tuning", "vpx_approximate",
+           "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_set_tuning", "vpx_workspace_reserve", "vpx_workspace_release", "vpx_approximate",
            "vpx_eltwise_quantization_approximation", "vpx_wt_get_scale", "vpx_wt_get_bias", "vpx_get_weights_table",
            "vpx_retrieve_ppe_int", "vpx_generate_softmax_attr", "vpx_get_quant_params_attr", "vpx_create_kernel_params", "vpx_get_kernel_info",
            "vpx_float_to_half_bits", "vpx_half_bits_to_float"]
@@ -125,6 +125,8 @@ def lib():
         L.vpx_sw_kernel_launch_noalloc.argtypes = L.vpx_sw_kernel_launch.argtypes
         L.vpx_nce_task.argtypes = [C.POINTER(NceTask), C.c_void_p]
         L.vpx_set_tuning.argtypes = [C.c_char_p, C.c_char_p]
+        L.vpx_workspace_reserve.argtypes = [C.c_void_p, C.c_size_t]
+        L.vpx_workspace_release.argtypes = [C.c_void_p]
         L.vpx_approximate.argtypes = [C.c_int, C.c_double] + [C.POINTER(C.c_int64)] * 3
         L.vpx_eltwise_quantization_approximation.argtypes = [C.c_double] * 3 + [C.c_int] + [C.POINTER(C.c_int64)] * 4
         L.vpx_wt_get_scale.restype = C.c_int32
@@ -471,14 +473,19 @@ def softmax(x, out, axis, pad_size=0, order=None, packed=True, stream=None):
 
 
 def nce_task(inp, weights, weight_table, out, ppe, zp_in=0, zp_w=0, zp_out=0, strides=(1, 1),
-             pads=(0, 0, 0, 0), stream=None):
+             pads=(0, 0, 0, 0), stream=None, groups=None):
     """inp NHWC, weights [OC,KY,KX,IC], weight_table [OC,4] int32 (device), out NHWC.
-    pads = (left, right, top, bottom)."""
-    N, H, W, IC = inp.shape
-    OC, KY, KX, IC2 = weights.shape
+    pads = (left, right, top, bottom).  With groups=G every tensor carries a leading dimension of G
+    (dense), and the G tasks go down in one call."""
+    if groups is not None:
+        assert inp.shape[0] == weights.shape[0] == weight_table.shape[0] == out.shape[0] == groups
+        assert all(x.is_contiguous() for x in (inp, weights, weight_table, out))
+    N, H, W, IC = inp.shape[-4:]
+    OC, KY, KX, IC2 = weights.shape[-4:]
     assert IC == IC2
     t = NceTask()
     t.task_type = 0
+    t.groups = groups or 0
     t.input, t.weights, t.weight_table, t.output = inp.data_ptr(), weights.data_ptr(), weight_table.data_ptr(), out.data_ptr()
     t.input_type, t.weights_type, t.output_type = (_torch_dtype_code(x) for x in (inp, weights, out))
     t.N, t.H, t.W, t.IC, t.OC = N, H, W, IC, OC
@@ -511,7 +518,13 @@ def nce_eltwise(in1, in2, out, ppe, zp_in1=0, zp_in2=0, zp_out=0, subtract=False
 
 
 def nce_matmul(a, b_nk, weight_table, out, ppe, zp_a=0, zp_b=0, zp_out=0, stream=None):
-    """A [M,K] x B stored [N,K] -> out [M,N]: NCE.MatMul as the 1x1 convolution task."""
+    """A [M,K] x B stored [N,K] -> out [M,N]: NCE.MatMul as the 1x1 convolution task.  Three-dimensional operands
+    (A [G,M,K], B [G,N,K], weight table [G,N,4], out [G,M,N]) are the operator's grouped form, one call."""
+    if a.dim() == 3:
+        G, M, K = a.shape
+        Nn = b_nk.shape[1]
+        return nce_task(a.view(G, 1, M, 1, K), b_nk.view(G, Nn, 1, 1, K), weight_table, out.view(G, 1, M, 1, Nn), ppe,
+                        zp_in=zp_a, zp_w=zp_b, zp_out=zp_out, stream=stream, groups=G)
     M, K = a.shape
     Nn, _ = b_nk.shape
     return nce_task(a.view(1, M, 1, K), b_nk.view(Nn, 1, 1, K), weight_table, out.view(1, M, 1, Nn), ppe, zp_in=zp_a,
@@ -521,6 +534,16 @@ def nce_matmul(a, b_nk, weight_table, out, ppe, zp_a=0, zp_b=0, zp_out=0, stream
 def set_tuning(knob, value=None):
     """Override the NCE dispatcher (tests, tuning): knob is a VPX_* name, value a string or None for the default."""
     check(lib().vpx_set_tuning(knob.encode(), None if value is None else str(value).encode()))
+
+
+def workspace_reserve(nbytes, stream=None):
+    """Grow the library's scratch block of `stream` on the current device to at least nbytes."""
+    check(lib().vpx_workspace_reserve(_stream_handle(stream), nbytes))
+
+
+def workspace_release(stream=None):
+    """Wait for `stream`, then free its scratch block and cached per-axis tables."""
+    check(lib().vpx_workspace_release(_stream_handle(stream)))
 
 
 def nce_last_kernel():
