@@ -132,7 +132,7 @@ def make_c3(rt):
         xs = np.ascontiguousarray(c["x"][:groups])
         return lambda: orc.mvn_f16(xs, True, True, c["eps"]), xs.size * 4
     return Workload("c3_mvn", "MVN fp16 across C,H,W [4,256,64,64], eps 1e-9, normalize_variance",
-                    _prebuilt_sw_launch(rt, "mvn1", blob, ops), n * 4, 0, "hbm", "f16", "mvn_chunk_kernel", cpu,
+                    _prebuilt_sw_launch(rt, "mvn1", blob, ops), n * 4, 0, "hbm", "f16", "mvn_fused_kernel", cpu,
                     (1, 4, "batch elements"))
 
 

@@ -880,6 +880,33 @@ def test_mvn_config_c3_full_size(rt, orc, dev):
     assert np.array_equal(got, _mvn(rt, dev, c["x"], True, True, c["eps"]))
 
 
+@pytest.mark.parametrize("shape", [(4, 64, 64, 64), (1, 3, 72, 200), (3, 5, 40, 104), (7, 2, 64, 40), (2, 33, 97, 8), (1, 128, 128, 128)])
+def test_mvn_one_launch_kernel_and_its_fallback(rt, orc, dev, shape):
+    """Long groups in one launch (workgroups of a group meet at the group's counter): against the oracle, bit for bit
+    against the same kernel when no workgroup waits for the others (each recomputes its group's moments, as a
+    workgroup does whose wait runs out), repeated launches (the counters are left at zero), and within tolerance
+    against the two-launch kernels."""
+    import torch
+    rng = np.random.default_rng(sum(shape))
+    x = (rng.uniform(-8, 8, shape) + rng.normal(0, 2, (1, shape[1], 1, 1))).astype(np.float32)
+    xb = orc.f32_to_f16(x)
+    want = orc.mvn_f16(xb, True, True, 1e-9)
+    runs = [_mvn(rt, dev, xb, True, True, 1e-9) for _ in range(3)]
+    assert_close_f16_mvn(runs[0], want, orc, "one launch %s" % (shape,))
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+    rt.set_tuning("VPX_MVN_FUSED", "nowait")
+    try:
+        alone = _mvn(rt, dev, xb, True, True, 1e-9)
+        rt.set_tuning("VPX_MVN_FUSED", None)
+        after = _mvn(rt, dev, xb, True, True, 1e-9)  # the counters were left clean by the launch that did not wait
+        rt.set_tuning("VPX_MVN_FUSED", "off")
+        two = _mvn(rt, dev, xb, True, True, 1e-9)
+    finally:
+        rt.set_tuning("VPX_MVN_FUSED", None)
+    assert np.array_equal(alone, runs[0]) and np.array_equal(after, runs[0])
+    assert_close_f16_mvn(two, want, orc, "two launches %s" % (shape,))
+
+
 def test_mvn_large_offset_and_constant(rt, orc, dev):
     rng = np.random.default_rng(42)
     x = (1000.0 + rng.normal(0, 1, (2, 4, 64, 64))).astype(np.float32)  # mean >> spread

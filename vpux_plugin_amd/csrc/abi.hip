@@ -43,13 +43,16 @@ struct Scratch {
     void* ptr = nullptr;
     size_t size = 0;
     std::vector<void*> retired;  // outgrown blocks: work already queued may still use them, freed on release
+    void* sync = nullptr;        // kSyncBytes of counters for kernels whose workgroups meet inside one launch
 };
 std::mutex g_ws_mutex;
 std::map<std::pair<int, hipStream_t>, Scratch> g_ws;
 
 // The fixed scratch array.  Its name is a host-side handle, not a device address: host code uses the per-device
 // address that hipGetSymbolAddress returns (each device holds its own copy of the array).
-static __device__ __align__(256) unsigned char scratch[VPX_NOALLOC_SCRATCH_BYTES];
+// (the counters of the allocation-free entry point sit behind the bytes get_workspace() hands out; device arrays
+// start as zeros)
+static __device__ __align__(256) unsigned char scratch[VPX_NOALLOC_SCRATCH_BYTES + kSyncBytes];
 constexpr int kMaxDevices = 64;
 void* g_static_scratch[kMaxDevices] = {};  // guarded by g_ws_mutex
 thread_local bool t_noalloc = false;
@@ -118,7 +121,42 @@ int get_workspace(hipStream_t stream, size_t bytes, void** out) {
     return VPX_RESULT_SUCCESS;
 }
 
+// Counters that start as zeros and that every kernel using them leaves as zeros (the last workgroup through resets
+// them), so launches on one stream can share them without a clearing pass.  One area per (device, stream handle),
+// allocated and cleared on first need; nothing else is ever written there.
+int get_sync_area(hipStream_t stream, void** out) {
+    if (t_noalloc) {
+        void* base = nullptr;
+        const int rc = static_scratch_address(&base);
+        if (rc) return rc;
+        *out = (char*)base + VPX_NOALLOC_SCRATCH_BYTES;
+        return VPX_RESULT_SUCCESS;
+    }
+    int dev = 0;
+    VPX_HIP_CHECK(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    Scratch& sc = g_ws[std::make_pair(dev, stream)];
+    if (!sc.sync) {
+        VPX_REQUIRE(!stream_is_capturing(stream), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                    "the stream is capturing and has no counter area yet: call vpx_workspace_reserve before the capture, "
+                    "or use vpx_sw_kernel_launch_noalloc");
+        void* p = nullptr;
+        VPX_HIP_CHECK(hipMalloc(&p, kSyncBytes));
+        const hipError_t e = hipMemsetAsync(p, 0, kSyncBytes, stream);
+        if (e != hipSuccess) {
+            (void)hipFree(p);
+            VPX_HIP_CHECK(e);
+        }
+        sc.sync = p;
+    }
+    *out = sc.sync;
+    return VPX_RESULT_SUCCESS;
+}
+
 int workspace_reserve(hipStream_t stream, size_t bytes) {
+    void* sync = nullptr;
+    const int rc = get_sync_area(stream, &sync);
+    if (rc) return rc;
     int dev = 0;
     VPX_HIP_CHECK(hipGetDevice(&dev));
     std::lock_guard<std::mutex> lock(g_ws_mutex);
@@ -139,6 +177,7 @@ int workspace_release(hipStream_t stream) {
             g_ws.erase(it);
             for (void* p : sc.retired) VPX_HIP_CHECK(hipFree(p));
             if (sc.ptr) VPX_HIP_CHECK(hipFree(sc.ptr));
+            if (sc.sync) VPX_HIP_CHECK(hipFree(sc.sync));
         }
     }
     return release_axis_tables(dev, stream);

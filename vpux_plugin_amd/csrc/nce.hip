@@ -1581,6 +1581,7 @@ struct Tuning {
     std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = stream: skip the resident-weights tile kernel
     std::atomic<int> conv_rows{0};          // VPX_CONV_ROWS = n: cap on the output rows per workgroup of the LDS-patch kernels
     std::atomic<int> conv_waves{0};         // VPX_CONV_WAVES = 4 | 8
+    std::atomic<int> mvn_fused{1};          // VPX_MVN_FUSED = off | nowait (see tuning_mvn_fused)
 };
 Tuning g_tuning;
 std::once_flag g_tuning_once;
@@ -1599,6 +1600,8 @@ bool set_knob(const char* knob, const char* value) {
         g_tuning.conv_rows = std::atoi(v) > 0 ? std::atoi(v) : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_WAVES")) {
         g_tuning.conv_waves = std::atoi(v) == 4 ? 4 : 0;
+    } else if (!std::strcmp(knob, "VPX_MVN_FUSED")) {
+        g_tuning.mvn_fused = !std::strcmp(v, "off") ? 0 : (!std::strcmp(v, "nowait") ? 2 : 1);
     } else {
         return false;
     }
@@ -1607,13 +1610,17 @@ bool set_knob(const char* knob, const char* value) {
 
 const Tuning& tuning() {
     std::call_once(g_tuning_once, [] {
-        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES"})
+        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES", "VPX_MVN_FUSED"})
             if (const char* v = std::getenv(k)) set_knob(k, v);
     });
     return g_tuning;
 }
 
 }  // namespace
+
+int tuning_mvn_fused() {
+    return tuning().mvn_fused.load();
+}
 
 int set_tuning(const char* knob, const char* value) {
     (void)tuning();  // the environment is consulted before the first explicit setting, never after it

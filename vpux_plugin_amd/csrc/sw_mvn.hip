@@ -16,6 +16,8 @@
 // part the barrier alone costs about 30 us (device-scope atomics from 1024 workgroups on 8 dies
 // meet in memory, not in a cache), against about 3 us for a launch boundary, and the second read
 // of the input comes from L2 / Infinity Cache anyway.
+#include <atomic>
+
 #include "vpx_common.h"
 
 namespace vpx {
@@ -464,6 +466,246 @@ int mem_pos_of(uint64_t order, int nd, int logical) {
     return -1;
 }
 
+// ------------------------------------------------------------------------------------------------
+// A few long groups in ONE launch, the tensor read once: as many workgroups as the device has compute units, each
+// keeps a slice of one group in registers and publishes the slice's {mean, M2}, each word tagged, with write-through
+// stores; the first wavefront then polls the records of ITS group (not of the whole grid) with loads that bypass the
+// caches until every tag names this launch, merges them in a fixed order and hands the result to the other wavefronts,
+// which normalise the slice from the registers.  No read-modify-write is involved: arrivals do not queue at a counter.
+// The tag is the group's launch count + 1; the count lives in the zero-initialised sync area.  The wait is bounded: a
+// workgroup that does not see its group complete in time (the others are not resident, e.g. the device is shared)
+// computes the group's moments itself, slice by slice with the same arithmetic, so the result is the same bits and
+// every wave exits.
+constexpr int kFusedMaxVec = 16;           // 128-bit words per lane: slices of up to 32768 values
+constexpr int kSyncStride = 64;            // words per group in the sync area: the launch count at +0, alone in its cache lines
+constexpr int kFusedMaxGroups = 16;        // groups this form takes: each owns a fixed run of kMergeInKernel record slots, so a
+                                           // slot only ever carries tags of its own group's launch count
+constexpr size_t kSyncRecords = 4 * 1024;  // byte offset of the records in the sync area (the groups' counters before it)
+static_assert(kFusedMaxGroups * kSyncStride * sizeof(unsigned) <= kSyncRecords &&
+              kSyncRecords + sizeof(Record) * kFusedMaxGroups * kMergeInKernel <= kSyncBytes, "sync area layout");
+
+// A published slice: two 64-bit words, {mean, tag} and {M2, tag}, each written and read as one access that goes
+// through to memory (agent scope), so neither needs the other to be valid; the count of a slice follows from its index.
+struct __attribute__((aligned(16))) Tagged {
+    unsigned long long mean, m2;
+};
+__device__ __forceinline__ unsigned long long tagged(float v, unsigned tag) {
+    return (unsigned long long)__builtin_bit_cast(unsigned, v) | ((unsigned long long)tag << 32);
+}
+
+template <int V>
+struct Slice {
+    u32x4 q[V];
+    unsigned valid;  // bit j: word j lies inside the slice
+};
+
+template <int V>
+__device__ __forceinline__ void load_slice(const half_t* __restrict__ g, int64_t base, int64_t end, Slice<V>& sl) {
+    sl.valid = 0;
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        const int64_t e0 = base + (int64_t)(j * kThreads + threadIdx.x) * 8;
+        const bool ok = e0 < end;  // slices and groups are whole words
+        sl.q[j] = ok ? *reinterpret_cast<const u32x4*>(g + e0) : u32x4{0, 0, 0, 0};
+        sl.valid |= ok ? (1u << j) : 0u;
+    }
+}
+
+// Moments of the slice held by the workgroup: per wavefront by lane shuffles (mean first, then centred squares),
+// the four wavefronts' results merged in a fixed order by every lane.
+template <int V>
+__device__ __forceinline__ Moments slice_moments(const Slice<V>& sl, Moments* red) {
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        const half_t* p = reinterpret_cast<const half_t*>(&sl.q[j]);
+#pragma unroll
+        for (int k = 0; k < 8; k++) sum += (float)p[k];
+    }
+    const float n = wave_sum((float)(8 * __builtin_popcount(sl.valid)));
+    const float mean = n > 0.f ? wave_sum(sum) / n : 0.f;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        const half_t* p = reinterpret_cast<const half_t*>(&sl.q[j]);
+        float qj = 0.f;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float d = (float)p[k] - mean;
+            qj += d * d;
+        }
+        q += (sl.valid >> j) & 1u ? qj : 0.f;
+    }
+    q = wave_sum(q);
+    __syncthreads();  // the previous use of `red` is over
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = Moments{n, mean, q};
+    __syncthreads();
+    return merge(merge(red[0], red[1]), merge(red[2], red[3]));
+}
+
+template <int V>
+__global__ __launch_bounds__(kThreads) void mvn_fused_kernel(const half_t* __restrict__ in, half_t* __restrict__ out,
+                                                             int64_t group_size, int wpg, int64_t slice, unsigned* sync,
+                                                             int normalize_variance, float eps, unsigned long long spin_ticks) {
+    __shared__ Moments red[4];
+    __shared__ Moments others[kMergeInKernel];
+    __shared__ Moments shared_total;
+    __shared__ int complete;
+    const int64_t group = blockIdx.x / wpg;
+    const int part = blockIdx.x % wpg;
+    const int lane = threadIdx.x & 63;
+    unsigned* count = sync + group * kSyncStride;
+    Tagged* mine = reinterpret_cast<Tagged*>(reinterpret_cast<char*>(sync) + kSyncRecords) + group * kMergeInKernel;
+    unsigned tag = 0;
+    if (wpg > 1 && threadIdx.x < 64) {
+        tag = __hip_atomic_load(count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+        tag = tag == 0u ? 1u : tag;
+    }
+    const half_t* gin = in + group * group_size;
+    const int64_t base = (int64_t)part * slice;
+    const int64_t end = base + slice < group_size ? base + slice : group_size;
+    Slice<V> sl;
+    load_slice<V>(gin, base, end, sl);
+    Moments total = slice_moments<V>(sl, red);
+    if (wpg > 1) {
+        if (threadIdx.x < 64) {  // the first wavefront
+            if (lane == 0) {
+                __hip_atomic_store(&mine[part].mean, tagged(total.mean, tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&mine[part].m2, tagged(total.m2, tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            const unsigned long long t0 = wall_clock64();
+            unsigned long long rm[kMergeInKernel / 64], rq[kMergeInKernel / 64];
+            bool ok;
+            for (;;) {
+                bool ready = true;
+#pragma unroll
+                for (int k = 0; k < kMergeInKernel / 64; k++) {
+                    const int i = k * 64 + lane;
+                    rm[k] = rq[k] = 0;
+                    if (i < wpg) {
+                        rm[k] = __hip_atomic_load(&mine[i].mean, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        rq[k] = __hip_atomic_load(&mine[i].m2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        ready = ready && (unsigned)(rm[k] >> 32) == tag && (unsigned)(rq[k] >> 32) == tag;
+                    }
+                }
+                ok = __builtin_amdgcn_ballot_w64(!ready) == 0;
+                if (ok || wall_clock64() - t0 >= spin_ticks) break;  // (pausing between polls measured slower)
+            }
+            if (ok) {
+                Moments acc{0.f, 0.f, 0.f};
+#pragma unroll
+                for (int k = 0; k < kMergeInKernel / 64; k++) {
+                    const int i = k * 64 + lane;
+                    if (i < wpg) {
+                        const int64_t b = (int64_t)i * slice;
+                        const int64_t cnt = (b + slice < group_size ? b + slice : group_size) - b;
+                        acc = merge(acc, Moments{(float)cnt, __builtin_bit_cast(float, (unsigned)rm[k]), __builtin_bit_cast(float, (unsigned)rq[k])});
+                    }
+                }
+                const Moments t = wave_merge(acc);
+                if (lane == 0) shared_total = t;
+            }
+            if (lane == 0) complete = ok ? 1 : 0;
+        }
+        __syncthreads();
+        if (complete) {
+            total = shared_total;
+        } else {
+            for (int p = 0; p < wpg; p++) {
+                const int64_t b = (int64_t)p * slice;
+                const int64_t e = b + slice < group_size ? b + slice : group_size;
+                Slice<V> t;
+                load_slice<V>(gin, b, e, t);
+                const Moments mp = slice_moments<V>(t, red);
+                if (threadIdx.x == 0) others[p] = mp;
+            }
+            __syncthreads();
+            total = merge_partials([&](int i) { return others[i]; }, wpg);  // the order the first wavefront uses above
+        }
+        // The group's first workgroup advances the launch count, and it alone: stores of many workgroups to one word
+        // queue up (64 of them cost 1.5 us here).  When its wait was met, every workgroup of the group has read the
+        // count already (a record carries the tag only after its writer has); when its wait ran out, a workgroup that
+        // starts even later reads the advanced count, publishes under the next tag, meets nobody and recomputes, like
+        // everyone else in a launch that far apart.  A workgroup whose wait ran out withdraws its record (tag 0 is
+        // never used), so that whichever tag the next launch uses, the slot is not taken for published until its
+        // owner writes it again.
+        if (threadIdx.x == 0) {
+            if (part == 0) __hip_atomic_store(count, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (!complete) {
+                __hip_atomic_store(&mine[part].mean, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&mine[part].m2, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    const float mean = total.mean, inv = inv_std(total, normalize_variance, eps);
+    half_t* gout = out + group * group_size;
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+        if (!((sl.valid >> j) & 1u)) continue;
+        const half_t* p = reinterpret_cast<const half_t*>(&sl.q[j]);
+        u32x4 r;
+        half_t* o = reinterpret_cast<half_t*>(&r);
+#pragma unroll
+        for (int k = 0; k < 8; k++) o[k] = (half_t)(((float)p[k] - mean) * inv);
+        __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(gout + base + (int64_t)(j * kThreads + threadIdx.x) * 8));
+    }
+}
+
+int device_compute_units(int* out) {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    VPX_HIP_CHECK(hipGetDevice(&dev));
+    int v = dev >= 0 && dev < 64 ? cached[dev].load() : 0;
+    if (v == 0) {
+        VPX_HIP_CHECK(hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev));
+        if (dev >= 0 && dev < 64) cached[dev].store(v);
+    }
+    *out = v;
+    return VPX_RESULT_SUCCESS;
+}
+
+// Takes the launch when the groups are few and the tensor fits the registers of one workgroup per compute unit.
+// *done is set when the kernel was launched.
+int launch_fused_groups(const half_t* in, half_t* out, int64_t groups, int64_t group_size, int nv, float eps, hipStream_t s,
+                        bool* done) {
+    *done = false;
+    const int mode = tuning_mvn_fused();  // 0: never, 1: default, 2: spin limit 0 (every workgroup recomputes)
+    if (mode == 0) return VPX_RESULT_SUCCESS;
+    int cus = 0;
+    int rc = device_compute_units(&cus);
+    if (rc) return rc;
+    if (groups > cus || groups > kFusedMaxGroups) return VPX_RESULT_SUCCESS;
+    int64_t wpg = cus / groups;  // (two workgroups per compute unit measured 1.2 us slower at [4,256,64,64])
+    if (wpg > kMergeInKernel) wpg = kMergeInKernel;
+    const int64_t words = group_size / 8;
+    const int64_t most = (words + kThreads - 1) / kThreads;  // at least one word per lane
+    if (wpg > most) wpg = most;
+    const int64_t slice = (words + wpg - 1) / wpg * 8;
+    wpg = (group_size + slice - 1) / slice;  // no empty slices
+    int v = 1;
+    while (v < kFusedMaxVec && (int64_t)v * kThreads * 8 < slice) v *= 2;
+    if ((int64_t)v * kThreads * 8 < slice) return VPX_RESULT_SUCCESS;
+    void* sync = nullptr;
+    rc = get_sync_area(s, &sync);
+    if (rc) return rc;
+    const unsigned long long spin = mode == 2 ? 0ull : 500000ull;  // 5 ms of the 100 MHz counter
+    const dim3 grid((unsigned)(groups * wpg)), block(kThreads);
+#define VPX_FUSED(V)                                                                                                  \
+    hipLaunchKernelGGL((mvn_fused_kernel<V>), grid, block, 0, s, in, out, group_size, (int)wpg, slice, (unsigned*)sync, \
+                       nv, eps, spin)
+    switch (v) {
+    case 1: VPX_FUSED(1); break;
+    case 2: VPX_FUSED(2); break;
+    case 4: VPX_FUSED(4); break;
+    case 8: VPX_FUSED(8); break;
+    default: VPX_FUSED(16); break;
+    }
+#undef VPX_FUSED
+    VPX_HIP_CHECK(hipGetLastError());
+    *done = true;
+    return VPX_RESULT_SUCCESS;
+}
+
 template <bool ALIGNED>
 int launch_groups(const half_t* in, half_t* out, int64_t groups, int64_t group_size, int nv, float eps, hipStream_t s) {
     const int64_t chunks64 = (group_size + kChunk - 1) / kChunk;
@@ -471,6 +713,11 @@ int launch_groups(const half_t* in, half_t* out, int64_t groups, int64_t group_s
                 "mvn1: %lld groups of %lld elements exceed the launch limit", (long long)groups, (long long)group_size);
     const int chunks = (int)chunks64;
     const unsigned blocks = (unsigned)(groups * chunks);
+    if (ALIGNED && chunks > 1) {
+        bool done = false;
+        const int rc = launch_fused_groups(in, out, groups, group_size, nv, eps, s, &done);
+        if (rc || done) return rc;
+    }
     if (chunks == 1) {
         hipLaunchKernelGGL((mvn_chunk_kernel<0, ALIGNED>), dim3(blocks), dim3(kThreads), 0, s, in, out, group_size, 1,
                            (Record*)nullptr, (const Record*)nullptr, nv, eps);

@@ -80,6 +80,10 @@ struct NdIndex {
 // Library-owned scratch memory, one buffer per (device, stream): calls on one stream are ordered,
 // so they can share it; calls on different streams get different buffers.
 int get_workspace(hipStream_t stream, size_t bytes, void** out);
+// A small area of zero-initialised counters per (device, stream handle) for kernels whose workgroups meet inside a
+// launch; a kernel that uses it leaves every word zero again.
+constexpr size_t kSyncBytes = 128 * 1024;
+int get_sync_area(hipStream_t stream, void** out);
 // True while the calling thread is inside the entry point that may not allocate: get_workspace() then hands out the
 // fixed scratch array (at most VPX_NOALLOC_SCRATCH_BYTES), and launchers must not call hipMalloc for caches of their own.
 bool noalloc_call();
@@ -88,6 +92,9 @@ int release_axis_tables(int dev, hipStream_t stream);
 
 // Dispatch override for tests and tuning (knob names are those of the VPX_* environment variables, read once).
 int set_tuning(const char* knob, const char* value);
+// VPX_MVN_FUSED: 0 = never take the one-launch MVN kernel, 1 = default, 2 = its workgroups do not wait for each other
+// (every one recomputes the group's moments: the path a workgroup takes when the others are not resident)
+int tuning_mvn_fused();
 
 // ---- kernel launchers (defined in the .hip files) ------------------------------------------
 int launch_convert(const MemRef& in, const MemRef& out, hipStream_t s);
