@@ -1,4 +1,5 @@
 // C ABI of the execution library: blob parsing, validation, dispatch, error text, scratch memory.
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <map>
@@ -150,6 +151,19 @@ int get_sync_area(hipStream_t stream, void** out) {
         sc.sync = p;
     }
     *out = sc.sync;
+    return VPX_RESULT_SUCCESS;
+}
+
+int device_compute_units(int* out) {
+    static std::atomic<int> cached[kMaxDevices];
+    int dev = 0;
+    VPX_HIP_CHECK(hipGetDevice(&dev));
+    int v = dev >= 0 && dev < kMaxDevices ? cached[dev].load() : 0;
+    if (v == 0) {
+        VPX_HIP_CHECK(hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev));
+        if (dev >= 0 && dev < kMaxDevices) cached[dev].store(v);
+    }
+    *out = v;
     return VPX_RESULT_SUCCESS;
 }
 

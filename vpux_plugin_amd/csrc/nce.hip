@@ -572,7 +572,16 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
             for (int j = 0; j < TN; j++) {
                 const int idx = i * TN + j;
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, fb[cur][j], acc[i][j], 0, 0, 0);
-                if (idx < TM + TN) load_frag(pnext, knext, cur ^ 1, idx);  // early: all back before the barrier
+                // all fragment reads of the next sub-step behind the first two MFMAs: the reads of the eight waves
+                // queue at the LDS, and the last one issued must be back before this sub-step's MFMAs are through
+                constexpr int FH = (TM + TN + 1) / 2;
+                if (idx == 0) {
+#pragma unroll
+                    for (int n = 0; n < FH; n++) load_frag(pnext, knext, cur ^ 1, n);
+                } else if (idx == 1) {
+#pragma unroll
+                    for (int n = FH; n < TM + TN; n++) load_frag(pnext, knext, cur ^ 1, n);
+                }
                 if (!SHORTK && idx % MFMA_PER_DMA == MFMA_PER_DMA - 1) dma_one(dma_p, dma0 + idx / MFMA_PER_DMA);
                 __builtin_amdgcn_sched_barrier(0);
             }

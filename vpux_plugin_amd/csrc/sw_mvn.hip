@@ -651,19 +651,6 @@ __global__ __launch_bounds__(kThreads) void mvn_fused_kernel(const half_t* __res
     }
 }
 
-int device_compute_units(int* out) {
-    static std::atomic<int> cached[64];
-    int dev = 0;
-    VPX_HIP_CHECK(hipGetDevice(&dev));
-    int v = dev >= 0 && dev < 64 ? cached[dev].load() : 0;
-    if (v == 0) {
-        VPX_HIP_CHECK(hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev));
-        if (dev >= 0 && dev < 64) cached[dev].store(v);
-    }
-    *out = v;
-    return VPX_RESULT_SUCCESS;
-}
-
 // Takes the launch when the groups are few and the tensor fits the registers of one workgroup per compute unit.
 // *done is set when the kernel was launched.
 int launch_fused_groups(const half_t* in, half_t* out, int64_t groups, int64_t group_size, int nv, float eps, hipStream_t s,

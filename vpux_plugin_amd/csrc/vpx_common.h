@@ -84,6 +84,8 @@ int get_workspace(hipStream_t stream, size_t bytes, void** out);
 // launch; a kernel that uses it leaves every word zero again.
 constexpr size_t kSyncBytes = 128 * 1024;
 int get_sync_area(hipStream_t stream, void** out);
+// Compute units of the current device (cached per device).
+int device_compute_units(int* out);
 // True while the calling thread is inside the entry point that may not allocate: get_workspace() then hands out the
 // fixed scratch array (at most VPX_NOALLOC_SCRATCH_BYTES), and launchers must not call hipMalloc for caches of their own.
 bool noalloc_call();
