@@ -33,10 +33,10 @@ METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
 # WRITE_SIZE counters of an earlier run of the same workload, scaled by a plain copy of known size
 # (profiles/<workload>__*.md hold those runs and their commands); the JSON line labels them as such.
 MEASURED_TRAFFIC = {
-    "c1_fake_quantize": 880079, "c2_softmax": 134293332, "c3_mvn": 25440485, "c4_conv": 16276094,
-    "c5_matmul": 385007798, "c5_dequantize": 135326848, "c5_eltwise_add": 270538895, "c5_nce_eltwise": 135268239,
-    "calib_int_mm": 531804959, "x_mvn6_layernorm": 268476854, "x_activation_hswish": 180532564,
-    "x_mvn1_three_steps": 25333054,
+    "c1_fake_quantize": 888359, "c2_softmax": 134285956, "c3_mvn": 17028413, "c4_conv": 16276480,
+    "c5_matmul": 384936464, "c5_dequantize": 135341729, "c5_eltwise_add": 270522802, "c5_nce_eltwise": 135260398,
+    "calib_int_mm": 532970109, "x_mvn6_layernorm": 268490358, "x_activation_hswish": 180562131,
+    "x_mvn1_three_steps": 25324896,
 }
 
 
