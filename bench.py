@@ -511,6 +511,8 @@ def measure(name, rt, steps, warmup, rotate, cpu, extras=True):
     rec = {"value": round(value, 2), "unit": unit, "dtype": w.dtype, "description": w.desc, "steps": steps, "warmup": warmup,
            "launch": "eager", "buffer_sets": len(sets), "buffer_bytes_total": len(sets) * footprint(w),
            "ms_per_step": round(wall_ms, 6), "device_ms_per_step": round(dev_ms, 6), "roofline": roofline(w, dev_ms)}
+    if name in NOTES:
+        rec["note"] = NOTES[name]
     if extras:
         _, same_ms = time_steps(w.step, steps, min(warmup, 5))
         _, graph_ms = time_steps(step, steps, 2, graph=True)
@@ -525,6 +527,18 @@ def measure(name, rt, steps, warmup, rotate, cpu, extras=True):
     torch.cuda.empty_cache()
     return w, rec
 
+
+# What bounds a configuration besides its roofline, said in the line itself.
+NOTES = {
+    "c1_fake_quantize": "0.8 MB per launch: launch-bound, not bandwidth-bound. An empty kernel of the same grid takes 2.6 us, the "
+                        "kernel 2.5-3 us (graph_device_ms_per_step); the eager figure of record is the host's launch rate over "
+                        "418 separate parameter blobs. A single launch of this size cannot reach 0.70 of the HBM peak (that would be 0.14 us).",
+    "c3_mvn": "16 MB in one launch of 8.2 us, of which about 2.6 us are the launch floor; 0.70 of the HBM peak would be 3.0 us end to end.",
+    "c4_conv": "7.4 GOP: about 2 us of MFMA or HBM time behind a launch floor of about 3 us; the kernel's four phases "
+               "(load, MFMA, requantise, store) overlap only across the two workgroups a compute unit holds.",
+    "c5_matmul": "power-limited: the part runs this kernel at 1.84-1.86 GHz on random int8 operands (2.4 GHz on zeros), where the "
+                 "dense int8 peak is 3.9 POP/s; frac is against the 5.0 POP/s of 2.4 GHz. The value includes the column-sum pre-pass.",
+}
 
 HEADLINE = "c5_matmul"
 OTHER_CONFIGS = ["c1_fake_quantize", "c2_softmax", "c3_mvn", "c4_conv", "c5_dequantize", "c5_eltwise_add"]
@@ -566,6 +580,8 @@ def main():
         "roofline": rec["roofline"],
         "extras": rec.get("extras"),
     }
+    if "note" in rec:
+        line["config"]["note"] = rec["note"]
     if "cpu_baseline" in rec:
         line["cpu_baseline"] = rec["cpu_baseline"]
     if not args.only:
