@@ -74,7 +74,8 @@ VPX_API int vpx_sw_kernel_launch(const char* entry, const void* params, size_t p
  * reference.  Kernels that need scratch memory (mvn1 / mvn6 chunk moments, the MVN-1 decomposition's partial sums,
  * dynamic_quantize's range pass, per-axis quantize / dequantize tables) take it from one fixed array of
  * VPX_NOALLOC_SCRATCH_BYTES in device memory that the library holds on every device it runs on; a launch that
- * would need more returns VPX_RESULT_ERROR_OUT_OF_MEMORY and enqueues nothing.  The call performs no hipMalloc /
+ * would need more returns VPX_RESULT_ERROR_OUT_OF_MEMORY and enqueues nothing (the library keeps a further 128 KiB of
+ * counters behind it for kernels whose workgroups meet inside one launch).  The call performs no hipMalloc /
  * hipFree.  All calls on one device share that array and it keeps the previous call's contents: calls through
  * this entry point that may overlap on one device (different streams, or different threads) race; order them on
  * one stream.  Arguments, results and errors are otherwise those of vpx_sw_kernel_launch. */
