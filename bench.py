@@ -537,7 +537,7 @@ NOTES = {
     "c4_conv": "7.4 GOP: about 2 us of MFMA or HBM time behind a launch floor of about 3 us; the kernel's four phases "
                "(load, MFMA, requantise, store) overlap only across the two workgroups a compute unit holds.",
     "c5_matmul": "power-limited: the part runs this kernel at 1.84-1.86 GHz on random int8 operands (2.4 GHz on zeros), where the "
-                 "dense int8 peak is 3.9 POP/s; frac is against the 5.0 POP/s of 2.4 GHz. The value includes the column-sum pre-pass.",
+                 "dense int8 peak is 3.9 POP/s; frac is against the 5.0 POP/s of 2.4 GHz.",
 }
 
 HEADLINE = "c5_matmul"

@@ -194,7 +194,7 @@ typedef struct vpx_nce_task_t {
      * weights [G,N,K,1,1], weight table [G,N,1,1,4], all GNHWC in memory): `groups` independent CONV tasks of the
      * shape above whose inputs, weights, weight tables and outputs lie one after the other, densely, behind the four
      * pointers.  0 and 1 both mean a single task.  A matmul the MFMA matmul kernel serves is one launch for all
-     * groups (the group on the grid's second dimension, one column-sum pass over all groups' weights). */
+     * groups (the group on the grid's second dimension). */
     int32_t groups;
 } vpx_nce_task_t;
 

@@ -536,8 +536,8 @@ def test_c_abi_host_example(rt):
 
 
 def test_chain_replayed_from_a_hip_graph(rt, orc, dev):
-    """MatMul + PPE -> Dequantize -> fp16 Add (with a non-zero activation zero point, so the column-sum
-    pre-pass and the library workspace are in play) captured once into a HIP graph and replayed several
+    """MatMul + PPE -> Dequantize -> fp16 Add (with a non-zero activation zero point, so the zero-point
+    term is in play) captured once into a HIP graph and replayed several
     times with eager launches and synchronisations in between: every replay must reproduce the eager result."""
     import torch
     rng = np.random.default_rng(97)
@@ -647,7 +647,7 @@ def test_workspace_reserve_release_and_cold_capture(rt, orc, dev):
 
 def test_two_host_threads_on_their_own_streams(rt, orc, dev):
     """The launch functions keep no shared state but a per-(device, stream) workspace: two host threads, each on its own
-    stream, run the matmul (column-sum pre-pass in the workspace), MVN (chunk moments in the workspace) and softmax
+    stream, run the matmul, MVN (chunk moments in the workspace or the sync area) and softmax
     many times over different data; every result must equal the one computed alone."""
     import threading
     import torch

@@ -563,6 +563,12 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     // One sub-step: the TM x TN MFMAs on fragment slot `cur`; between them, the TM + TN fragment reads of the
     // next sub-step (panel at pnext, sub-step knext) into the other slot and this wave's DMA instructions
     // dma0.. of panel dma_p.
+    // Column sums of B for the zero-point term, from the fragments as they pass: lane l sums the 16-byte chunks it
+    // holds of column l % 32 (lanes l and l ^ 32 hold alternate chunks); four dot instructions per fragment on the
+    // vector ALU, which the MFMAs leave idle.
+    int cs[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) cs[j] = 0;
     auto substep = [&](int cur, const uint8_t* pnext, int knext, int dma_p, int dma0) {
 #pragma unroll
         for (int i = 0; i < TM; i++) {
@@ -572,6 +578,10 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
             for (int j = 0; j < TN; j++) {
                 const int idx = i * TN + j;
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, fb[cur][j], acc[i][j], 0, 0, 0);
+                if (i == TM - 1) {  // behind the last MFMA that reads the fragment (always: a branch here costs more than the four dots)
+#pragma unroll
+                    for (int d = 0; d < 4; d++) cs[j] = __builtin_amdgcn_sdot4(fb[cur][j][d], 0x01010101, cs[j], false);
+                }
                 // all fragment reads of the next sub-step behind the first two MFMAs: the reads of the eight waves
                 // queue at the LDS, and the last one issued must be back before this sub-step's MFMAs are through
                 constexpr int FH = (TM + TN + 1) / 2;
@@ -594,7 +604,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     for (int j = 0; j < TN; j++) {
         int64_t n = n0 + wn0 + j * 32 + (lane & 31);
         n = n < N ? n : N - 1;
-        csr[j] = colsum ? colsum[n] : 0;  // sum_k B[n][k], present when the zero-point term is not 0
+        csr[j] = 0;
         w2r[j] = wt[n * 4 + 2];
         w3r[j] = wt[n * 4 + 3];
     }
@@ -636,6 +646,8 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
         }
     }
     dma_wait_all_and_barrier();  // every wave is done with the panels: LDS becomes the output staging tile
+#pragma unroll
+    for (int j = 0; j < TN; j++) csr[j] = cs[j] + __shfl_xor(cs[j], 32, 64);  // sum_k B[n][k] of column n = lane % 32 of block j
 
     // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
     if constexpr (OUT == OUT_F16) {
@@ -1813,16 +1825,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 if (lds < (size_t)tile * kOutStride) lds = (size_t)tile * kOutStride;  // ... or the staging tile
             }
             GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi};
-            int32_t* colsum = nullptr;
-            if (corr != 0) {
-                void* ws = nullptr;
-                rc = scratch(sizeof(int32_t) * (size_t)(G * g.OC), &ws);
-                if (rc) return rc;
-                colsum = (int32_t*)ws;
-                hipLaunchKernelGGL(nce_colsum_kernel, dim3((unsigned)((G * g.OC + 3) / 4)), dim3(256), 0, s,
-                                   (const int8_t*)wptr, colsum, G * g.OC, Ktot);
-                VPX_HIP_CHECK(hipGetLastError());
-            }
+            const int32_t* colsum = nullptr;  // the kernel sums the columns of B itself, from the fragments it reads
 #define VPX_GEMM_W(U8, SGN, NW, TILE, SHORTK)                                                                        \
     do {                                                                                                             \
         auto kern = nce_gemm_mfma<U8, SGN, NW, TILE, SHORTK>;                                                        \
