@@ -441,6 +441,7 @@ __device__ __forceinline__ unsigned quad_transpose_bytes(unsigned w, int lane) {
 }
 
 constexpr int kOutStride = 288;  // bytes per row of the 256-column output staging tile in LDS
+constexpr int kGemmLdsHead = 1024;  // bytes in front of the matmul kernel's panel buffers (column sums of B)
 
 struct GemmPpe {
     int prelu_mult, prelu_shift;  // applied to negative scaled values (1,0 = none; 0,0 = ReLU)
@@ -483,7 +484,9 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     constexpr int DMA_PER_WAVE = BM * BK / 1024 / NW;  // per operand, per panel
     constexpr int STAGE = (BM + BN) * BK;
 
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem_raw[];
+    int* const colsums = reinterpret_cast<int*>(smem_raw);  // TILE column sums of B, handed from the upper waves to the lower
+    uint8_t* const smem = smem_raw + kGemmLdsHead;          // the panel buffers, later the output staging tile
 
     // Grouped matmul: blockIdx.y is the group; every operand holds the groups one after the other.
     if (const int64_t grp = blockIdx.y) {
@@ -564,12 +567,14 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     // next sub-step (panel at pnext, sub-step knext) into the other slot and this wave's DMA instructions
     // dma0.. of panel dma_p.
     // Column sums of B for the zero-point term, from the fragments as they pass: lane l sums the 16-byte chunks it
-    // holds of column l % 32 (lanes l and l ^ 32 hold alternate chunks); four dot instructions per fragment on the
-    // vector ALU, which the MFMAs leave idle.
+    // holds of column l % 32 (lanes l and l ^ 32 hold alternate chunks), four dot instructions per fragment.  Vector
+    // ALU instructions between the MFMAs are not free (they take issue slots of the SIMD), so only the waves of the
+    // tile's upper half (SUM) do this -- the lower half reads the same columns -- and hand the sums over through LDS.
     int cs[TN];
 #pragma unroll
     for (int j = 0; j < TN; j++) cs[j] = 0;
-    auto substep = [&](int cur, const uint8_t* pnext, int knext, int dma_p, int dma0) {
+    auto substep = [&](auto sum_c, int cur, const uint8_t* pnext, int knext, int dma_p, int dma0) {
+        constexpr bool SUM = decltype(sum_c)::value;
 #pragma unroll
         for (int i = 0; i < TM; i++) {
             i32x4 a = fa[cur][i];
@@ -578,7 +583,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
             for (int j = 0; j < TN; j++) {
                 const int idx = i * TN + j;
                 acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, fb[cur][j], acc[i][j], 0, 0, 0);
-                if (i == TM - 1) {  // behind the last MFMA that reads the fragment (always: a branch here costs more than the four dots)
+                if (SUM && i == TM - 1) {  // behind the last MFMA that reads the fragment
 #pragma unroll
                     for (int d = 0; d < 4; d++) cs[j] = __builtin_amdgcn_sdot4(fb[cur][j][d], 0x01010101, cs[j], false);
                 }
@@ -610,44 +615,56 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // keeps the count of loads in flight below exact
 
-    if (SHORTK) {
+    auto main_loop = [&](auto sum_c) {
+        if (SHORTK) {
 #pragma unroll
-        for (int p = 0; p < NS - 1; p++)
-            if (p < nk) {
+            for (int p = 0; p < NS - 1; p++)
+                if (p < nk) {
+#pragma unroll
+                    for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
+                }
+            dma_wait_all_and_barrier();
+#pragma unroll
+            for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
+            for (int kt = 0; kt < nk; kt++) {
+                const uint8_t* pcur = smem + kt * STAGE;
+                const uint8_t* pnxt = kt + 1 < nk ? pcur + STAGE : pcur;  // the last step prefetches fragments nobody uses
+                substep(sum_c, 0, pcur, 1, 0, 0);
+                substep(sum_c, 1, pnxt, 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < NS - 1; p++)
 #pragma unroll
                 for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
+            asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * DMA_PER_WAVE) : "memory");  // panel 0 is in
+#pragma unroll
+            for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
+            for (int kt = 0; kt < nk; kt++) {
+                const uint8_t* pcur = smem + (kt & (NS - 1)) * STAGE;
+                const uint8_t* pnxt = smem + ((kt + 1) & (NS - 1)) * STAGE;
+                substep(sum_c, 0, pcur, 1, kt + NS - 1, 0);
+                // Loads in flight here, oldest first: panel kt+1, panel kt+2 (2 * DMA_PER_WAVE each), half of panel kt+3.
+                // Behind the barrier panel kt+1 is complete for every wave and nobody reads panel kt-1 any
+                // more, whose buffer panel kt+3 is being written to.
+                asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * DMA_PER_WAVE) : "memory");
+                substep(sum_c, 1, pnxt, 0, kt + NS - 1, DMA_PER_WAVE);
             }
-        dma_wait_all_and_barrier();
-#pragma unroll
-        for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
-        for (int kt = 0; kt < nk; kt++) {
-            const uint8_t* pcur = smem + kt * STAGE;
-            const uint8_t* pnxt = kt + 1 < nk ? pcur + STAGE : pcur;  // the last step prefetches fragments nobody uses
-            substep(0, pcur, 1, 0, 0);
-            substep(1, pnxt, 0, 0, 0);
         }
-    } else {
+    };
+    // (a matmul of at most three panels is all epilogue: there every wave sums its own columns and nothing is handed over)
+    if (SHORTK || wm0 == 0) main_loop(std::true_type{});
+    else main_loop(std::false_type{});
 #pragma unroll
-        for (int p = 0; p < NS - 1; p++)
-#pragma unroll
-            for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * DMA_PER_WAVE) : "memory");  // panel 0 is in
-#pragma unroll
-        for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
-        for (int kt = 0; kt < nk; kt++) {
-            const uint8_t* pcur = smem + (kt & (NS - 1)) * STAGE;
-            const uint8_t* pnxt = smem + ((kt + 1) & (NS - 1)) * STAGE;
-            substep(0, pcur, 1, kt + NS - 1, 0);
-            // Loads in flight here, oldest first: panel kt+1, panel kt+2 (2 * DMA_PER_WAVE each), half of panel kt+3.
-            // Behind the barrier panel kt+1 is complete for every wave and nobody reads panel kt-1 any
-            // more, whose buffer panel kt+3 is being written to.
-            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * DMA_PER_WAVE) : "memory");
-            substep(1, pnxt, 0, kt + NS - 1, DMA_PER_WAVE);
-        }
+    for (int j = 0; j < TN; j++) {
+        csr[j] = cs[j] + __shfl_xor(cs[j], 32, 64);  // every lane takes part
+        if (!SHORTK && wm0 == 0 && lane < 32) colsums[wn0 + j * 32 + lane] = csr[j];
     }
     dma_wait_all_and_barrier();  // every wave is done with the panels: LDS becomes the output staging tile
+    if (!SHORTK) {
 #pragma unroll
-    for (int j = 0; j < TN; j++) csr[j] = cs[j] + __shfl_xor(cs[j], 32, 64);  // sum_k B[n][k] of column n = lane % 32 of block j
+        for (int j = 0; j < TN; j++) csr[j] = colsums[wn0 + j * 32 + (lane & 31)];  // sum_k B[n][k] of column n of block j
+    }
 
     // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
     if constexpr (OUT == OUT_F16) {
@@ -1824,6 +1841,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 lds = (size_t)nk * (tile + tile) * 64;  // only the panels there are ...
                 if (lds < (size_t)tile * kOutStride) lds = (size_t)tile * kOutStride;  // ... or the staging tile
             }
+            lds += kGemmLdsHead;
             GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi};
             const int32_t* colsum = nullptr;  // the kernel sums the columns of B itself, from the fragments it reads
 #define VPX_GEMM_W(U8, SGN, NW, TILE, SHORTK)                                                                        \
