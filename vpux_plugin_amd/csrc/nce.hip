@@ -540,9 +540,9 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     // d-th DMA instruction (first half A, second half B) of panel p.  Panels past the end keep the number of loads
     // in flight the same in every iteration: every lane re-fetches the tile's first 16 bytes (one cache line for
     // the whole instruction) into a buffer nobody reads.
-    auto dma_one = [&](int p, int d) {
+    auto dma_one = [&](auto known_real, int p, int d) {
         const unsigned base = lds0 + (unsigned)((p & (NS - 1)) * STAGE);
-        const bool real = p < nk;
+        const bool real = decltype(known_real)::value || p < nk;  // (known: no select instructions in the loop body)
         const int64_t k0 = real ? (int64_t)p * BK : 0;
         if (d < DMA_PER_WAVE) dma16(abase + k0, real ? oa[d] : 0u, base + (unsigned)((wave + NW * d) * 1024));
         else dma16(bbase + k0, real ? ob[d - DMA_PER_WAVE] : 0u, base + (unsigned)(BM * BK + (wave + NW * (d - DMA_PER_WAVE)) * 1024));
@@ -563,6 +563,29 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
         else if (n <= TN) fb[slot][n - 1] = *reinterpret_cast<const i32x4*>(pa + BM * BK + lds_offset<BK>(wn0 + (n - 1) * 32 + (lane & 31), chunk));
         else fa[slot][n - TN] = *reinterpret_cast<const i32x4*>(pa + lds_offset<BK>(wm0 + (n - TN) * 32 + (lane & 31), chunk));
     };
+    // The same reads for a panel buffer known at compile time: the lane's part of the address is one of eight registers
+    // that do not change over the K loop (operand, sub-step, lower or upper pair of buffers) and everything else is the
+    // instruction's immediate offset, so the unrolled loop below computes no LDS address.
+    typedef const __attribute__((address_space(3))) uint8_t* lds_bytes_t;  // 32-bit LDS addresses: one register each
+    typedef const __attribute__((address_space(3))) i32x4* lds_v4_t;
+    lds_bytes_t frag_base[2][2][2];  // [buffer pair][operand: 0 = A, 1 = B][sub-step]
+#pragma unroll
+    for (int hi = 0; hi < 2; hi++)
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+            const int chunk = kk * 2 + (lane >> 5);
+            frag_base[hi][0][kk] = (lds_bytes_t)(smem + hi * 2 * STAGE + lds_offset<BK>(wm0 + (lane & 31), chunk));
+            frag_base[hi][1][kk] = (lds_bytes_t)(smem + hi * 2 * STAGE + BM * BK + lds_offset<BK>(wn0 + (lane & 31), chunk));
+            asm volatile("" : "+v"(frag_base[hi][0][kk]), "+v"(frag_base[hi][1][kk]));  // keep them: re-deriving costs vector ALU slots per read
+        }
+    auto load_frag_static = [&](auto stage_c, int kk, int slot, int n) {
+        constexpr int stage = decltype(stage_c)::value;
+        constexpr int imm = (stage & 1) * STAGE;
+        // rows 32 apart are 32 * BK bytes apart and share their swizzle
+        if (n == 0) fa[slot][0] = *(lds_v4_t)(frag_base[stage >> 1][0][kk] + imm);
+        else if (n <= TN) fb[slot][n - 1] = *(lds_v4_t)(frag_base[stage >> 1][1][kk] + imm + (n - 1) * 32 * BK);
+        else fa[slot][n - TN] = *(lds_v4_t)(frag_base[stage >> 1][0][kk] + imm + (n - TN) * 32 * BK);
+    };
     // One sub-step: the TM x TN MFMAs on fragment slot `cur`; between them, the TM + TN fragment reads of the
     // next sub-step (panel at pnext, sub-step knext) into the other slot and this wave's DMA instructions
     // dma0.. of panel dma_p.
@@ -573,8 +596,13 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     int cs[TN];
 #pragma unroll
     for (int j = 0; j < TN; j++) cs[j] = 0;
-    auto substep = [&](auto sum_c, int cur, const uint8_t* pnext, int knext, int dma_p, int dma0) {
+    auto substep = [&](auto sum_c, auto next_stage_c, int cur, const uint8_t* pnext, int knext, int dma_p, int dma0) {
         constexpr bool SUM = decltype(sum_c)::value;
+        constexpr int NEXT_STAGE = decltype(next_stage_c)::value;  // buffer the next sub-step's panel sits in, -1: see pnext
+        auto load_next = [&](int n) {
+            if constexpr (NEXT_STAGE >= 0) load_frag_static(next_stage_c, knext, cur ^ 1, n);
+            else load_frag(pnext, knext, cur ^ 1, n);
+        };
 #pragma unroll
         for (int i = 0; i < TM; i++) {
             i32x4 a = fa[cur][i];
@@ -592,12 +620,13 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                 constexpr int FH = (TM + TN + 1) / 2;
                 if (idx == 0) {
 #pragma unroll
-                    for (int n = 0; n < FH; n++) load_frag(pnext, knext, cur ^ 1, n);
+                    for (int n = 0; n < FH; n++) load_next(n);
                 } else if (idx == 1) {
 #pragma unroll
-                    for (int n = FH; n < TM + TN; n++) load_frag(pnext, knext, cur ^ 1, n);
+                    for (int n = FH; n < TM + TN; n++) load_next(n);
                 }
-                if (!SHORTK && idx % MFMA_PER_DMA == MFMA_PER_DMA - 1) dma_one(dma_p, dma0 + idx / MFMA_PER_DMA);
+                if (!SHORTK && idx % MFMA_PER_DMA == MFMA_PER_DMA - 1)
+                    dma_one(std::integral_constant<bool, (NEXT_STAGE >= 0)>{}, dma_p, dma0 + idx / MFMA_PER_DMA);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -615,13 +644,14 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // keeps the count of loads in flight below exact
 
+    constexpr std::integral_constant<int, -1> kDynamicStage{};
     auto main_loop = [&](auto sum_c) {
         if (SHORTK) {
 #pragma unroll
             for (int p = 0; p < NS - 1; p++)
                 if (p < nk) {
 #pragma unroll
-                    for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
+                    for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(std::false_type{}, p, d);
                 }
             dma_wait_all_and_barrier();
 #pragma unroll
@@ -629,26 +659,43 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
             for (int kt = 0; kt < nk; kt++) {
                 const uint8_t* pcur = smem + kt * STAGE;
                 const uint8_t* pnxt = kt + 1 < nk ? pcur + STAGE : pcur;  // the last step prefetches fragments nobody uses
-                substep(sum_c, 0, pcur, 1, 0, 0);
-                substep(sum_c, 1, pnxt, 0, 0, 0);
+                substep(sum_c, kDynamicStage, 0, pcur, 1, 0, 0);
+                substep(sum_c, kDynamicStage, 1, pnxt, 0, 0, 0);
             }
         } else {
 #pragma unroll
             for (int p = 0; p < NS - 1; p++)
 #pragma unroll
-                for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(p, d);
+                for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(std::false_type{}, p, d);
             asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * DMA_PER_WAVE) : "memory");  // panel 0 is in
 #pragma unroll
             for (int n = 0; n < TM + TN; n++) load_frag(smem, 0, 0, n);
-            for (int kt = 0; kt < nk; kt++) {
+            int kt = 0;
+            // Four panels per trip while all loads are real ones: the panel buffers are then known by number, the
+            // fragment reads take immediate offsets and the loads need no selects.
+            if ((nk & (NS - 1)) == 0) {
+                auto one_panel = [&](auto u_c, int k) {
+                    constexpr int u = decltype(u_c)::value;
+                    substep(sum_c, std::integral_constant<int, u>{}, 0, nullptr, 1, k + NS - 1, 0);
+                    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * DMA_PER_WAVE) : "memory");
+                    substep(sum_c, std::integral_constant<int, (u + 1) & (NS - 1)>{}, 1, nullptr, 0, k + NS - 1, DMA_PER_WAVE);
+                };
+                for (; kt + 2 * NS <= nk; kt += NS) {
+                    one_panel(std::integral_constant<int, 0>{}, kt);
+                    one_panel(std::integral_constant<int, 1>{}, kt + 1);
+                    one_panel(std::integral_constant<int, 2>{}, kt + 2);
+                    one_panel(std::integral_constant<int, 3>{}, kt + 3);
+                }
+            }
+            for (; kt < nk; kt++) {
                 const uint8_t* pcur = smem + (kt & (NS - 1)) * STAGE;
                 const uint8_t* pnxt = smem + ((kt + 1) & (NS - 1)) * STAGE;
-                substep(sum_c, 0, pcur, 1, kt + NS - 1, 0);
+                substep(sum_c, kDynamicStage, 0, pcur, 1, kt + NS - 1, 0);
                 // Loads in flight here, oldest first: panel kt+1, panel kt+2 (2 * DMA_PER_WAVE each), half of panel kt+3.
                 // Behind the barrier panel kt+1 is complete for every wave and nobody reads panel kt-1 any
                 // more, whose buffer panel kt+3 is being written to.
                 asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * DMA_PER_WAVE) : "memory");
-                substep(sum_c, 1, pnxt, 0, kt + NS - 1, DMA_PER_WAVE);
+                substep(sum_c, kDynamicStage, 1, pnxt, 0, kt + NS - 1, DMA_PER_WAVE);
             }
         }
     };
