@@ -360,9 +360,37 @@ def make_int_mm(rt):
                     step, 0, 2 * M * K * N, "mfma", "int8", "hipBLASLt")
 
 
+def make_mfma_loop(rt, operands, fragment_reads):
+    """`v_mfma_i32_32x32x32_i8` alone (or with the matmul kernel's LDS fragment reads) on every compute unit: the rate the
+    part sustains on these operand bytes before anything comes from global memory."""
+    import torch
+    if operands == "random":
+        g = torch.Generator(device="cuda").manual_seed(5)
+        src = torch.randint(-128, 128, (65536,), device="cuda", generator=g, dtype=torch.int8)
+    else:
+        src = torch.zeros((65536,), device="cuda", dtype=torch.int8)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty((cus * 8192,), device="cuda", dtype=torch.uint8)
+    iters = 2000
+    ops = rt.calib_mfma_i8(src, sink, iters, fragment_reads)
+    torch.cuda.synchronize()
+
+    def step():
+        rt.calib_mfma_i8(src, sink, iters, fragment_reads)
+    step.keep = (src, sink)
+    name = "calib_mfma_%s%s" % (operands, "_lds" if fragment_reads else "")
+    desc = "loop of v_mfma_i32_32x32x32_i8 on %s int8 operands, two waves per SIMD, %s" % (
+        operands, "with the matmul kernel's twelve LDS fragment reads per sixteen MFMAs" if fragment_reads else "registers only")
+    return Workload(name, desc, step, 0, ops, "mfma", "int8", "calib_mfma_i8_kernel")
+
+
 MAKERS = {
     "calib_copy": make_copy,
     "calib_int_mm": make_int_mm,
+    "calib_mfma_random": lambda rt: make_mfma_loop(rt, "random", False),
+    "calib_mfma_random_lds": lambda rt: make_mfma_loop(rt, "random", True),
+    "calib_mfma_zero": lambda rt: make_mfma_loop(rt, "zero", False),
+    "calib_mfma_zero_lds": lambda rt: make_mfma_loop(rt, "zero", True),
     "c1_fake_quantize": make_c1,
     "c2_softmax": make_c2,
     "c3_mvn": make_c3,
@@ -536,8 +564,10 @@ NOTES = {
     "c3_mvn": "16 MB in one launch of 8.2 us, of which about 2.6 us are the launch floor; 0.70 of the HBM peak would be 3.0 us end to end.",
     "c4_conv": "7.4 GOP: about 2 us of MFMA or HBM time behind a launch floor of about 3 us; the kernel's four phases "
                "(load, MFMA, requantise, store) overlap only across the two workgroups a compute unit holds.",
-    "c5_matmul": "power-limited: the part runs this kernel at 1.84-1.86 GHz on random int8 operands (2.4 GHz on zeros), where the "
-                 "dense int8 peak is 3.9 POP/s; frac is against the 5.0 POP/s of 2.4 GHz.",
+    "c5_matmul": "power-limited: the part runs this kernel at 1.83-1.86 GHz on random int8 operands (2.4 GHz on zeros), where the "
+                 "dense int8 peak is 3.9 POP/s; frac is against the 5.0 POP/s of 2.4 GHz. mfma_calibration in this line is what "
+                 "a bare loop of the same MFMA sustains on this part: about 0.98 of the peak on zeros, 0.68 on random int8 operands, "
+                 "0.62 with this kernel's LDS fragment reads added.",
 }
 
 HEADLINE = "c5_matmul"
@@ -594,6 +624,14 @@ def main():
             sys.stderr.write("bench.py: %s done at %.0f s\n" % (name, time.perf_counter() - t_start))
             sys.stderr.flush()
         line["other_configs"] = others
+        # what the MFMA pipe sustains on this part today, beside the matmul it bounds (register-only loops, no global memory)
+        calib = {}
+        for name in ("calib_mfma_zero", "calib_mfma_random", "calib_mfma_random_lds"):
+            cw = MAKERS[name](rt)
+            _, ms = time_steps(cw.step, 50, 5)
+            calib[name] = {"description": cw.desc, "device_ms_per_step": round(ms, 6), "achieved": round(cw.ops / (ms * 1e-3) / 1e12, 1),
+                           "unit": "TOP/s", "frac_of_peak": round(cw.ops / (ms * 1e-3) / 1e12 / I8_PEAK_TOPS, 4)}
+        line["mfma_calibration"] = calib
     print(json.dumps(line), flush=True)
 
 

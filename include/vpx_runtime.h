@@ -209,6 +209,15 @@ VPX_API int vpx_nce_task(const vpx_nce_task_t* task, void* stream);
  * first call of this function, never during a launch.  Process-wide; results do not depend on any of them. */
 VPX_API int vpx_set_tuning(const char* knob, const char* value);
 
+/* Measurement aid (no counterpart in the reference): a loop of `v_mfma_i32_32x32x32_i8` alone on every compute unit,
+ * eight waves of 128 x 64 register tiles as in the matmul kernel, sixteen MFMAs per wave and iteration; with
+ * `fragment_reads` non-zero each wave also reads the twelve 16-byte LDS fragments those MFMAs consume.  It shows what the
+ * part sustains on the given operand bytes before anything comes from global memory (the shader clock depends on the
+ * data), which is what the matmul's fraction of the nominal peak has to be read against.
+ * `operands`: 64 KiB of device memory, copied to LDS by every workgroup; `sink`: 8 KiB per compute unit of device memory
+ * that receives the accumulators; `*ops` (may be NULL) is set to the integer operations the launch performs. */
+VPX_API int vpx_calib_mfma_i8(const void* operands, void* sink, int iters, int fragment_reads, int64_t* ops, void* stream);
+
 /* Name of the device kernel the last successful vpx_nce_task on this thread dispatched to
  * ("" before the first); for tests and profiles. */
 VPX_API const char* vpx_nce_last_kernel(void);

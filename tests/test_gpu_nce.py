@@ -706,3 +706,46 @@ def test_two_host_threads_on_their_own_streams(rt, orc, dev):
         t.join()
     assert not errors, errors
 
+
+
+def test_mfma_calibration_loop(rt, dev):
+    """The register-only MFMA loop the bench calibrates the int8 roofline with: its operation count is what it says
+    (the accumulators hold exactly `iters` times the products of the fragments it loaded)."""
+    import torch
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    rng = np.random.default_rng(11)
+    src = rng.integers(-128, 128, 65536, dtype=np.int8)
+    sink = torch.zeros((cus, 8, 64, 4), dtype=torch.int32, device=dev)
+    iters = 37
+    ops = rt.calib_mfma_i8(dev_t(src, dev), sink, iters, False)
+    torch.cuda.synchronize()
+    assert ops == iters * 16 * 2 * 32 * 32 * 32 * 8 * cus
+    got = sink.cpu().numpy().astype(np.int64)
+    assert np.array_equal(got[0], got[-1])          # every compute unit ran the same loop
+    s = src.astype(np.int64)
+    m = np.arange(32)
+    for wave in range(8):
+        def colsum(base):
+            # sum over the 32 rows of a fragment, per lane half c and byte t
+            off = base + (wave & 3) * 2048 + m[:, None, None] * 64 + ((np.arange(2)[None, :, None] ^ ((m[:, None, None] >> 2) & 3)) << 4) \
+                + np.arange(16)[None, None, :]
+            return s[off].sum(axis=0)
+        want = 0
+        for h in range(2):
+            sa = sum(colsum(i * 8192 + h * 32) for i in range(4))
+            sb = sum(colsum(32768 + j * 8192 + h * 32) for j in range(2))
+            want += int((sa * sb).sum())
+        want *= iters
+        assert (int(got[0, wave].sum()) - want) % (1 << 32) == 0, wave
+    # with the fragment reads: zeros stay zeros, and a launch is deterministic
+    z = torch.zeros(65536, dtype=torch.int8, device=dev)
+    rt.calib_mfma_i8(z, sink, 5, True)
+    torch.cuda.synchronize()
+    assert int(sink.abs().max()) == 0
+    a = torch.empty_like(sink)
+    rt.calib_mfma_i8(dev_t(src, dev), sink, 9, True)
+    rt.calib_mfma_i8(dev_t(src, dev), a, 9, True)
+    torch.cuda.synchronize()
+    assert torch.equal(a, sink) and int(sink.abs().max()) > 0
+    with pytest.raises(RuntimeError):
+        rt.calib_mfma_i8(dev_t(src, dev), sink, 0, False)

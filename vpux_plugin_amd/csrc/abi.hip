@@ -731,6 +731,11 @@ int vpx_set_tuning(const char* knob, const char* value) {
     return set_tuning(knob, value);
 }
 
+int vpx_calib_mfma_i8(const void* operands, void* sink, int iters, int fragment_reads, int64_t* ops, void* stream) {
+    last_error().clear();
+    return calib_mfma_i8(operands, sink, iters, fragment_reads, ops, static_cast<hipStream_t>(stream));
+}
+
 const char* vpx_nce_last_kernel(void) {
     return g_last_nce_kernel;
 }

@@ -92,6 +92,9 @@ bool noalloc_call();
 // Frees the per-axis quantization tables cached for (device, stream); the caller has drained the stream.
 int release_axis_tables(int dev, hipStream_t stream);
 
+// Register-only int8 MFMA loop over every compute unit (calibration of the MFMA roofline); *ops = operations enqueued.
+int calib_mfma_i8(const void* operands, void* sink, int iters, int fragment_reads, int64_t* ops, hipStream_t s);
+
 // Dispatch override for tests and tuning (knob names are those of the VPX_* environment variables, read once).
 int set_tuning(const char* knob, const char* value);
 // VPX_MVN_FUSED: 0 = never take the one-launch MVN kernel, 1 = default, 2 = its workgroups do not wait for each other

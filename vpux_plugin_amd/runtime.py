@@ -80,7 +80,7 @@ ELTWISE_ADD, ELTWISE_SUBTRACT = 0, 1
 
 # every symbol include/vpx_runtime.h and include/vpx_compiler_utils.h declare
 EXPORTS = ["vpx_get_last_error", "vpx_get_version", "vpx_sw_kernel_launch", "vpx_sw_kernel_launch_noalloc", "vpx_sw_kernel_supported",
-           "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_set_tuning", "vpx_workspace_reserve", "vpx_workspace_release", "vpx_approximate",
+           "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_set_tuning", "vpx_workspace_reserve", "vpx_workspace_release", "vpx_calib_mfma_i8", "vpx_approximate",
            "vpx_eltwise_quantization_approximation", "vpx_wt_get_scale", "vpx_wt_get_bias", "vpx_get_weights_table",
            "vpx_retrieve_ppe_int", "vpx_generate_softmax_attr", "vpx_get_quant_params_attr", "vpx_create_kernel_params", "vpx_get_kernel_info",
            "vpx_float_to_half_bits", "vpx_half_bits_to_float"]
@@ -127,6 +127,7 @@ def lib():
         L.vpx_set_tuning.argtypes = [C.c_char_p, C.c_char_p]
         L.vpx_workspace_reserve.argtypes = [C.c_void_p, C.c_size_t]
         L.vpx_workspace_release.argtypes = [C.c_void_p]
+        L.vpx_calib_mfma_i8.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_int64), C.c_void_p]
         L.vpx_approximate.argtypes = [C.c_int, C.c_double] + [C.POINTER(C.c_int64)] * 3
         L.vpx_eltwise_quantization_approximation.argtypes = [C.c_double] * 3 + [C.c_int] + [C.POINTER(C.c_int64)] * 4
         L.vpx_wt_get_scale.restype = C.c_int32
@@ -534,6 +535,15 @@ def nce_matmul(a, b_nk, weight_table, out, ppe, zp_a=0, zp_b=0, zp_out=0, stream
 def set_tuning(knob, value=None):
     """Override the NCE dispatcher (tests, tuning): knob is a VPX_* name, value a string or None for the default."""
     check(lib().vpx_set_tuning(knob.encode(), None if value is None else str(value).encode()))
+
+
+def calib_mfma_i8(operands, sink, iters, fragment_reads=False, stream=None):
+    """Enqueue the int8 MFMA calibration loop (operands: 64 KiB on the device, sink: 8 KiB per compute unit);
+    returns the integer operations the launch performs."""
+    ops = C.c_int64(0)
+    check(lib().vpx_calib_mfma_i8(operands.data_ptr(), sink.data_ptr(), int(iters), int(bool(fragment_reads)), C.byref(ops),
+                                  _stream_handle(stream)))
+    return ops.value
 
 
 def workspace_reserve(nbytes, stream=None):
