@@ -286,6 +286,28 @@ __device__ __forceinline__ ChanPrep ppe_prepare_packed(int mult, int shift, int 
     return c;
 }
 
+// The same four bytes from accumulators that already contain the bias (the MFMA chain started from it), for layers
+// that need neither the clipping nor the odd zero-point unit of GENERAL: one conversion, one fused multiply-add,
+// one median per value.  LEAKY: the negative branch scales by a slope in [0, 1] of the same sign (ReLU, LeakyReLU,
+// PReLU up to 1): then b * f_neg >= b * f_pos exactly when b < 0, so the larger of the two rounded products is the
+// result and no sign test is needed (rounding is monotone).  `c` comes from ppe_prepare (not _packed).
+template <bool LEAKY>
+__device__ __forceinline__ unsigned ppe_pack4_biased(int a0, int a1, int a2, int a3, double f_pos, double f_neg, const PpePack& p) {
+    const int a[4] = {a0, a1, a2, a3};
+    unsigned w = 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const double bd = (double)a[r];
+        int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, __builtin_fma(bd, f_pos, p.magic));
+        if (LEAKY) {
+            const int qn = (int)(unsigned)__builtin_bit_cast(unsigned long long, __builtin_fma(bd, f_neg, p.magic));
+            q = q > qn ? q : qn;
+        }
+        w |= (unsigned)med3_i32(q, p.lo, p.hi) << (8 * r);
+    }
+    return w ^ p.flip;
+}
+
 // ---------------------------------------------------------------- per-channel parameter fold
 // One wavefront per output channel: sum of the channel's weights (for the zero-point term) and the
 // prepared epilogue parameters.
@@ -428,16 +450,27 @@ __device__ __forceinline__ unsigned dpp_u32(unsigned v) {
 
 // Each lane of a quad holds one dword = 4 bytes of ONE column (rows R..R+3).  Afterwards lane t of
 // the quad holds row R+t of the quad's FOUR columns, i.e. 4 bytes that are adjacent in memory.
+// The two byte selectors depend on the lane only; QuadTranspose keeps them in registers so that a run of transposes
+// does not rebuild them every time.
+struct QuadTranspose {
+    unsigned sel1, sel2;
+    __device__ __forceinline__ explicit QuadTranspose(int lane) {
+        // (v_perm_b32 selector bytes: 0-3 pick from the second source, 4-7 from the first)
+        sel1 = (lane & 1) ? 0x03070105u : 0x06020400u;
+        sel2 = (lane & 2) ? 0x03020706u : 0x05040100u;
+        asm volatile("" : "+v"(sel1), "+v"(sel2));
+    }
+    __device__ __forceinline__ unsigned operator()(unsigned w) const {
+        const unsigned p = dpp_u32<0xB1>(w);  // lane ^ 1
+        // even lane: [w.b0, p.b0, w.b2, p.b2]   odd lane: [p.b1, w.b1, p.b3, w.b3]
+        const unsigned a = __builtin_amdgcn_perm(p, w, sel1);
+        const unsigned q = dpp_u32<0x4E>(a);  // lane ^ 2
+        // lanes 0,1: [a.b0, a.b1, q.b0, q.b1]   lanes 2,3: [q.b2, q.b3, a.b2, a.b3]
+        return __builtin_amdgcn_perm(q, a, sel2);
+    }
+};
 __device__ __forceinline__ unsigned quad_transpose_bytes(unsigned w, int lane) {
-    const unsigned p = dpp_u32<0xB1>(w);  // lane ^ 1
-    // even lane: [w.b0, p.b0, w.b2, p.b2]   odd lane: [p.b1, w.b1, p.b3, w.b3]
-    // (v_perm_b32 selector bytes: 0-3 pick from the second source, 4-7 from the first)
-    const unsigned sel1 = (lane & 1) ? 0x03070105u : 0x06020400u;
-    const unsigned a = __builtin_amdgcn_perm(p, w, sel1);
-    const unsigned q = dpp_u32<0x4E>(a);  // lane ^ 2
-    // lanes 0,1: [a.b0, a.b1, q.b0, q.b1]   lanes 2,3: [q.b2, q.b3, a.b2, a.b3]
-    const unsigned sel2 = (lane & 2) ? 0x03020706u : 0x05040100u;
-    return __builtin_amdgcn_perm(q, a, sel2);
+    return QuadTranspose(lane)(w);
 }
 
 constexpr int kOutStride = 288;  // bytes per row of the 256-column output staging tile in LDS
@@ -1169,6 +1202,227 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
     }
 }
 
+// ---------------------------------------------------------------- patch convolution, weights in registers
+// KY x KX taps of 64 input channels: the weights of a 64-channel block are 16 x KY x KX vector registers per lane in
+// the B layout of `v_mfma_i32_16x16x64_i8`, so every wave keeps all of them and the main loop reads only activations
+// from LDS (one 16-byte fragment per four MFMAs, where nce_conv_tile reads six per four).  A wave walks blocks of 16
+// output positions x 64 channels: KY*KX fragment reads and 4*KY*KX MFMAs, then the PPE of the block's 16 values per
+// lane and one 16-byte store per lane -- no workgroup barrier after the staging, no output staging in LDS.  The two
+// waves of a SIMD are started half a block apart (`lag`), so that one requantises while the other multiplies.
+//
+// Channel order inside a block: column n of MFMA tile j is output channel 16*(n/4) + 4*j + n%4.  After the 4x4 byte
+// transpose a lane then holds channels 16*q .. 16*q+15 of one position in its four result dwords (tile j -> dword j),
+// which is the 16 bytes it stores.  The weight rows sit in LDS in tile order (row 16*j + n), which the fragment reads
+// of sixteen lanes walk conflict-free.
+template <bool IN_U8, bool SAME_F, int KY, int KX>
+__global__ __launch_bounds__(512) void nce_conv_regw(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
+                                                     const int32_t* __restrict__ wt, uint8_t* __restrict__ out, ConvGeom g,
+                                                     PatchGeom pg, int pad_byte, GemmPpe ppe, int lag) {
+    constexpr int BN = 64, IC = 64, PS = IC + 16, NW = 8, NT = 64 * NW, TAPS = KY * KX, Ktot = TAPS * IC, WS = Ktot + 16;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t* const wlds = smem;             // [64][Ktot + 16], rows in tile order
+    uint8_t* const patch = smem + BN * WS;  // [PH*PW][IC + 16]
+    __shared__ int csum[BN];                // weight sums, by LDS row
+
+    // A launch of a few microseconds is bound by instructions as much as by anything else: all index arithmetic below
+    // is 32-bit, on offsets from a few 64-bit bases that are the same for the whole wave.
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int H = (int)g.H, W = (int)g.W, OC = (int)g.OC, OW = (int)g.OW, OH = (int)g.OH;
+    const int img = fdiv(blockIdx.x, pg.tiles_y);
+    const int oy0 = (blockIdx.x - img * (int)pg.tiles_y.d) * pg.R;
+    const int oc0 = blockIdx.y * BN;
+
+    // ---- weights and patch -> LDS.  All loads are issued up front, weights first: they come from L2 and are back
+    // before the patch rows are, so the waves copy their weight fragments to registers while the patch is on its way.
+    const int n16 = lane & 15, c4 = lane >> 4;
+    i32x4 wb[TAPS][4];
+    {
+        constexpr int cpr = Ktot / 16;                 // 16-byte chunks per weight row
+        constexpr int wchunks = BN * cpr;
+        constexpr int UW = (wchunks + NT - 1) / NT, UP = 5;
+        constexpr int cpp = IC / 16;
+        const int row_chunks = pg.PW * cpp;
+        const int upr = (int)pg.upr.d, units = pg.PH * upr;
+        const int pad32 = (pad_byte & 0xff) * 0x01010101;
+        const int iy0 = oy0 * g.SY - g.PT;
+        // patch pixel (py, px) is input pixel (iy0 + py, px - PL): byte offset py * W*IC + px * IC from `corner`, which
+        // may lie outside the tensor; lanes whose pixel is padding read the first pixel of the tile's first real row
+        const int8_t* corner = in + (((int64_t)img * H + iy0) * W - g.PL) * IC;
+        const int safe_off = ((iy0 < 0 ? -iy0 : 0) * W + g.PL) * IC;
+        const int8_t* wsrc = w + (int64_t)oc0 * Ktot;
+        const bool full_rows = oc0 + BN <= OC;         // the 64 weight rows are one contiguous run
+        i32x4 qw[UW], qp[UP];
+        int dw[UW], dp[UP];
+        bool pin[UP];
+        // (nothing here may use a loaded value: the first use is where the wave waits for the load)
+        auto load_patch = [&](int u0) {
+#pragma unroll
+            for (int u = 0; u < UP; u++) {
+                const int unit = u0 + wave + NW * u;   // wave-uniform, as are py and sub
+                const int py = fdiv(unit, pg.upr), sub = unit - py * upr;
+                const int qi = sub * 64 + lane;
+                const bool ok = unit < units && qi < row_chunks;
+                const int px = qi / cpp;
+                const int iy = iy0 + py;
+                const bool inside = ok && (unsigned)iy < (unsigned)H && (unsigned)(px - g.PL) < (unsigned)W;
+                const int off = inside ? py * (W * IC) + qi * 16 : safe_off;
+                qp[u] = *reinterpret_cast<const i32x4*>(corner + off);
+                pin[u] = inside;
+                dp[u] = ok ? py * (pg.PW * PS) + px * PS + (qi % cpp) * 16 : -1;
+            }
+        };
+        auto store_patch = [&]() {
+#pragma unroll
+            for (int u = 0; u < UP; u++)
+                if (dp[u] >= 0) {
+                    i32x4 v = pin[u] ? qp[u] : i32x4{pad32, pad32, pad32, pad32};
+                    if (IN_U8) v ^= (int32_t)0x80808080;
+                    *reinterpret_cast<i32x4*>(patch + dp[u]) = v;
+                }
+        };
+#pragma unroll
+        for (int u = 0; u < UW; u++) {
+            const int q = u * NT + tid;
+            const bool ok = q < wchunks;
+            const int qq = ok ? q : 0;
+            const int row = qq / cpr, c = qq - row * cpr;
+            int src = qq * 16;
+            if (!full_rows) src = (oc0 + row < OC ? row : OC - 1 - oc0) * Ktot + c * 16;  // channels past the end repeat the last one
+            qw[u] = *reinterpret_cast<const i32x4*>(wsrc + src);
+            const int lrow = ((row >> 2) & 3) * 16 + (row >> 4) * 4 + (row & 3);
+            dw[u] = ok ? lrow * WS + c * 16 : -1;
+        }
+        load_patch(0);
+#pragma unroll
+        for (int u = 0; u < UW; u++)
+            if (dw[u] >= 0) *reinterpret_cast<i32x4*>(wlds + dw[u]) = qw[u];
+        __syncthreads();
+        // this wave's copy of the weights
+#pragma unroll
+        for (int t = 0; t < TAPS; t++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) wb[t][j] = *reinterpret_cast<const i32x4*>(wlds + (j * 16 + n16) * WS + t * IC + c4 * 16);
+        // the sums of the weight rows where the zero-point term needs them
+        if (ppe.corr != 0 && tid < 256) {
+            const int row = tid >> 2, part = tid & 3;
+            int sum = 0;
+            for (int c = part; c < Ktot / 16; c += 4) {
+                const i32x4 q = *reinterpret_cast<const i32x4*>(wlds + row * WS + c * 16);
+#pragma unroll
+                for (int j = 0; j < 4; j++) sum = __builtin_amdgcn_sdot4(q[j], 0x01010101, sum, false);
+            }
+            sum += (int)dpp_u32<0xB1>((unsigned)sum);
+            sum += (int)dpp_u32<0x4E>((unsigned)sum);
+            if (part == 0) csum[row] = sum;
+        }
+        store_patch();
+        for (int u0 = NW * UP; u0 < units; u0 += NW * UP) {  // tall patches: the rest, a round trip each
+            load_patch(u0);
+            store_patch();
+        }
+    }
+    __syncthreads();
+
+    // ---- per-channel PPE parameters of the lane's four channels
+    ChanPrep cp[4];
+    bool clip = false;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        int n = oc0 + (n16 >> 2) * 16 + j * 4 + (n16 & 3);
+        n = n < OC ? n : OC - 1;
+        const int cs = ppe.corr != 0 ? csum[j * 16 + n16] : 0;
+        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        cp[j] = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+                            (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
+        clip = clip || cp[j].bmax_pos != 0x7fffffff || cp[j].bmax_neg != 0x7fffffff;
+        asm volatile("" : "+v"(cp[j].f_pos), "+v"(cp[j].f_neg));
+    }
+    const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
+    // the short PPE serves slopes in [0, 1] (ReLU, LeakyReLU), an even zero-point offset and scales up to 1/2
+    const bool slope_ok = SAME_F || (ppe.prelu_mult >= 0 && (ppe.prelu_shift >= 31 || ppe.prelu_mult <= (1 << ppe.prelu_shift)));
+    const bool general = __builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0 || !slope_ok;
+    const QuadTranspose transpose(lane);
+
+    const int rows_here = OH - oy0 < pg.R ? OH - oy0 : pg.R;
+    const int valid = rows_here * OW;
+    const int nblk = (valid + 15) >> 4;
+    const int64_t pos0 = ((int64_t)img * OH + oy0) * OW;
+    const int32_t* rt = ppe.rowterm ? ppe.rowterm + pos0 : nullptr;
+    uint8_t* const out0 = out + pos0 * OC;  // the tile's first output position
+    const bool vec_ok = (OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    const int q16 = oc0 + (n16 >> 2) * 16;  // first of the 16 channels this lane stores
+    int soff[TAPS];
+#pragma unroll
+    for (int t = 0; t < TAPS; t++) soff[t] = ((t / KX) * pg.PW + (t % KX)) * PS;
+
+    // the second wave of every SIMD starts late, so that its MFMAs meet the first one's PPE
+    if (wave >= NW / 2)
+        for (int i = 0; i < lag; i++) __builtin_amdgcn_s_sleep(1);
+
+    auto one_block = [&](int b, auto general_c) {
+        int p = b * 16 + n16;
+        p = p < valid ? p : 0;
+        const int r = fdiv(p, pg.ow), ox = p - r * OW;
+        const uint8_t* pa = patch + (r * g.SY * pg.PW + ox * g.SX) * PS + c4 * 16;
+        constexpr bool GENERAL = decltype(general_c)::value;
+        i32x4 acc[4];  // the short PPE's accumulators start from the bias
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int b0 = GENERAL ? 0 : cp[j].bias;
+            acc[j] = i32x4{b0, b0, b0, b0};
+        }
+        i32x4 fa[TAPS];  // all of the block's fragments are asked for before the first MFMA waits for one
+#pragma unroll
+        for (int t = 0; t < TAPS; t++) fa[t] = *reinterpret_cast<const i32x4*>(pa + soff[t]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < TAPS; t++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[t], wb[t][j], acc[j], 0, 0, 0);
+        if (rt) {  // (padded past the last position: an edge block may read ahead)
+            i32x4 v;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) v[r4] = rt[b * 16 + 4 * c4 + r4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[j] += v;
+        }
+        i32x4 o;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            unsigned v;
+            if constexpr (GENERAL) {
+                ChanPrep c = cp[j];  // the form ppe_pack4 takes: sign flip in the bias, factors swapped for a negative multiplier
+                c.bias = (int)((unsigned)c.bias + 0x80000000u);
+                if (c.sgn) {
+                    c.f_pos = cp[j].f_neg;
+                    c.f_neg = cp[j].f_pos;
+                    c.bmax_pos = cp[j].bmax_neg;
+                    c.bmax_neg = cp[j].bmax_pos;
+                }
+                v = ppe_pack4<SAME_F, true>(acc[j][0], acc[j][1], acc[j][2], acc[j][3], c, pk);
+            } else {
+                v = ppe_pack4_biased<!SAME_F>(acc[j][0], acc[j][1], acc[j][2], acc[j][3], cp[j].f_pos, cp[j].f_neg, pk);
+            }
+            o[j] = (int)transpose(v);
+        }
+        const int pi = b * 16 + 4 * c4 + (lane & 3);
+        if (pi < valid && q16 < OC) {
+            uint8_t* dst = out0 + (pi * OC + q16);
+            if (vec_ok && q16 + 16 <= OC) {
+                __builtin_nontemporal_store(o, reinterpret_cast<i32x4*>(dst));
+            } else {
+                for (int e = 0; e < 16 && q16 + e < OC; e++) dst[e] = (uint8_t)(o[e >> 2] >> (8 * (e & 3)));
+            }
+        }
+    };
+    if (general) {
+        for (int b = wave; b < nblk; b += NW) one_block(b, std::true_type{});
+    } else {
+        for (int b = wave; b < nblk; b += NW) one_block(b, std::false_type{});
+    }
+}
+
 // ---------------------------------------------------------------- patch convolution with streamed weights
 // For layers whose weights do not fit LDS next to the input patch (many input channels): the patch
 // stays resident, the weights pass through two small LDS buffers a slice at a time -- one tap x KSL
@@ -1663,7 +1917,8 @@ struct Tuning {
     std::atomic<int> nce_kernel{NCE_AUTO};  // VPX_NCE_KERNEL = naive | gather | conv: restrict the choice to slower, more general paths
     std::atomic<int> gemm_tile{0};          // VPX_GEMM_TILE = 128 | 256 (0: chosen from the shape)
     std::atomic<int> gemm_waves{0};         // VPX_GEMM_WAVES = 4 | 8
-    std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = stream: skip the resident-weights tile kernel
+    std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = tile | stream: start the choice of LDS-patch kernel below the fastest one (1: tile, 2: stream)
+    std::atomic<int> conv_lag{-1};          // VPX_CONV_LAG = n: start-up lag of the second wave per SIMD in nce_conv_regw, units of 64 cycles
     std::atomic<int> conv_rows{0};          // VPX_CONV_ROWS = n: cap on the output rows per workgroup of the LDS-patch kernels
     std::atomic<int> conv_waves{0};         // VPX_CONV_WAVES = 4 | 8
     std::atomic<int> mvn_fused{1};          // VPX_MVN_FUSED = off | nowait (see tuning_mvn_fused)
@@ -1680,7 +1935,9 @@ bool set_knob(const char* knob, const char* value) {
     } else if (!std::strcmp(knob, "VPX_GEMM_WAVES")) {
         g_tuning.gemm_waves = *v ? (std::atoi(v) == 4 ? 4 : 8) : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_KERNEL")) {
-        g_tuning.conv_stream = !std::strcmp(v, "stream") ? 1 : 0;
+        g_tuning.conv_stream = !std::strcmp(v, "stream") ? 2 : (!std::strcmp(v, "tile") ? 1 : 0);
+    } else if (!std::strcmp(knob, "VPX_CONV_LAG")) {
+        g_tuning.conv_lag = *v ? std::atoi(v) : -1;
     } else if (!std::strcmp(knob, "VPX_CONV_ROWS")) {
         g_tuning.conv_rows = std::atoi(v) > 0 ? std::atoi(v) : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_WAVES")) {
@@ -1695,7 +1952,7 @@ bool set_knob(const char* knob, const char* value) {
 
 const Tuning& tuning() {
     std::call_once(g_tuning_once, [] {
-        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES", "VPX_MVN_FUSED"})
+        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES", "VPX_CONV_LAG", "VPX_MVN_FUSED"})
             if (const char* v = std::getenv(k)) set_knob(k, v);
     });
     return g_tuning;
@@ -1929,10 +2186,68 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             // IC of 64 or 128: the one-tile-per-workgroup kernel with padded LDS rows (a tap's fragments of more
             // channels do not fit the registers twice)
             // VPX_CONV_KERNEL=stream starts the choice below the tile kernel (tests compare them)
-            const int first = knobs.conv_stream.load() ? 1 : 0;
+            const int first = knobs.conv_stream.load();
             // (with 128 channels and a stride the haloed patch crowds the resident weights out of LDS: the
             // streamed-weights kernel below measures 15.7 us against 20.2 at [32,56,56,128] -> 128, 3x3, stride 2)
-            if ((g.IC == 64 || (g.IC == 128 && g.SY * g.SX == 1)) && first <= 0) {
+            // 3x3 taps of 64 channels: the weights fit the registers of every wave
+            if (g.IC == 64 && g.KY == 3 && g.KX == 3 && first <= 0) {
+                PatchGeom pg{};
+                const int64_t PS = g.IC + 16, WS = Ktot + 16;
+                auto need = [&](int R) {
+                    return 64 * (size_t)WS + (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)PS;
+                };
+                int cus = 0;
+                rc = device_compute_units(&cus);
+                if (rc) return rc;
+                const int64_t ocb = (g.OC + 63) / 64;
+                // one workgroup per compute unit where the layer allows: rows per tile from the rows there are
+                int R = (int)((g.N * g.OH * ocb + cus - 1) / cus);
+                const int rmin = (int)((128 + g.OW - 1) / g.OW);  // eight waves want eight blocks of 16 positions
+                if (R < rmin) R = rmin;
+                if (R > g.OH) R = (int)g.OH;
+                while (R > 1 && need(R) > kMaxDynLds) R--;
+                if (const int v = knobs.conv_rows.load()) {
+                    if (v >= 1 && v <= R) R = v;
+                }
+                if (need(R) <= kMaxDynLds) {
+                    const int tiles_y = (int)((g.OH + R - 1) / R);
+                    auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
+                    pg.R = (int)((g.OH + tiles_y - 1) / tiles_y);
+                    pg.PH = (pg.R - 1) * g.SY + g.KY;
+                    pg.PW = (int)(g.OW - 1) * g.SX + g.KX;
+                    pg.MT = (int)((pg.R * g.OW + 31) / 32);
+                    pg.nt = 2;
+                    pg.ntiles = (int)(g.N * tiles_y);
+                    pg.tiles_y = fd(tiles_y);
+                    pg.cpr = fd(Ktot / 16);
+                    pg.cpp = fd(g.IC / 16);
+                    pg.upr = fd((pg.PW * (g.IC / 16) + 63) / 64);
+                    pg.ow = fd(g.OW);
+                    const size_t lds = need(pg.R);
+                    const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
+                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
+                    const int pad_byte = t.zp_in & 0xff;
+                    const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
+                    const int lag = knobs.conv_lag.load() >= 0 ? knobs.conv_lag.load() : 0;
+#define VPX_REGW(U8, SAME)                                                                                            \
+    do {                                                                                                              \
+        auto kern = nce_conv_regw<U8, SAME, 3, 3>;                                                                    \
+        rc = set_dyn_lds(kern, lds);                                                                                  \
+        if (rc) return rc;                                                                                            \
+        hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, \
+                           (uint8_t*)t.output, g, pg, pad_byte, gp, lag);                                             \
+    } while (0)
+                    if (in_u8 && same_f) VPX_REGW(true, true);
+                    else if (in_u8) VPX_REGW(true, false);
+                    else if (same_f) VPX_REGW(false, true);
+                    else VPX_REGW(false, false);
+#undef VPX_REGW
+                    VPX_HIP_CHECK(hipGetLastError());
+                    *kernel_name = "nce_conv_regw";
+                    return VPX_RESULT_SUCCESS;
+                }
+            }
+            if ((g.IC == 64 || (g.IC == 128 && g.SY * g.SX == 1)) && first <= 1) {
                 PatchGeom pg{};
                 const int64_t PS = g.IC + 16, WS = Ktot + 16;
                 auto need = [&](int R) {
@@ -2008,7 +2323,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 }
             }
             // any IC that is a multiple of 64: resident patch, weights streamed a slice at a time
-            if (first <= 1) {
+            if (first <= 2) {
                 PatchGeom pg{};
                 StreamGeom sg{};
                 sg.ksl = g.IC % 256 == 0 ? 256 : (g.IC % 128 == 0 ? 128 : 64);
