@@ -6,6 +6,8 @@
 //                     NCE.MatMul arrives): a plain A[M][K] x B[N][K]^T GEMM.  256x256 output tile per
 //                     workgroup, v_mfma_i32_32x32x32_i8, K panels from global memory straight into
 //                     XOR-swizzled LDS (global_load_lds, no register staging), four buffers.
+//   nce_conv_regw   : 3x3 taps of 64 input channels: the input rows of a tile sit in LDS, the weights of 64 output
+//                     channels in the registers of every wave.
 //   nce_conv_tile   : KYxKX / stride / padding with 64 or 128 input channels: the input rows of a tile
 //                     and the weights of 64 output channels sit in LDS, every tap is an LDS read.
 //   nce_conv_stream : the same with any multiple of 64 input channels: the weights pass through LDS a
@@ -792,16 +794,24 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                     for (int q = 0; q < 4; q++) acc[i][j][g * 4 + q] += v[q];
             }
     }
-    auto requant_tile = [&](auto clip_c) {
+    // kind 0: every PPE setting; 1: no clipping, even zero-point offset, slope in [0, 1] (ReLU, LeakyReLU): no sign
+    // test, see ppe_pack4_biased; 2: the same with slope 1 (no PReLU stage)
+    auto requant_tile = [&](auto kind_c) {
+        constexpr int KIND = decltype(kind_c)::value;
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col4 = wn0 + j * 32 + ((lane & 31) & ~3);
+            const int pb = (int)((unsigned)cp[j].bias - 0x80000000u);  // the bias without the sign flip of the packed form
 #pragma unroll
             for (int i = 0; i < TM; i++) {
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    unsigned w = ppe_pack4<false, decltype(clip_c)::value>(acc[i][j][g * 4], acc[i][j][g * 4 + 1],
-                                                                           acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3], cp[j], pk);
+                    unsigned w;
+                    if constexpr (KIND == 0)
+                        w = ppe_pack4<false, true>(acc[i][j][g * 4], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3], cp[j], pk);
+                    else  // (the larger of the two products is the same whichever way a negative multiplier swapped the factors)
+                        w = ppe_pack4_biased<KIND == 1>(acc[i][j][g * 4] + pb, acc[i][j][g * 4 + 1] + pb, acc[i][j][g * 4 + 2] + pb,
+                                                        acc[i][j][g * 4 + 3] + pb, cp[j].f_pos, cp[j].f_neg, pk);
                     w = quad_transpose_bytes(w, lane);
                     const int row = wm0 + i * 32 + 8 * g + 4 * (lane >> 5) + (lane & 3);
                     *reinterpret_cast<unsigned*>(smem + row * kOutStride + col4) = w;
@@ -809,9 +819,11 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
             }
         }
     };
-    // scale factors above 1/2 are rare (shift < 15): only then is the clipping variant needed
-    if (__builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0) requant_tile(std::true_type{});
-    else requant_tile(std::false_type{});
+    // scale factors above 1/2 are rare (shift < 15), as are odd zero-point offsets and slopes outside [0, 1]
+    const bool slope_ok = ppe.prelu_mult >= 0 && (ppe.prelu_shift >= 31 || ppe.prelu_mult <= (1 << ppe.prelu_shift));
+    if (__builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0 || !slope_ok) requant_tile(std::integral_constant<int, 0>{});
+    else if (ppe.prelu_mult == 1 && ppe.prelu_shift == 0) requant_tile(std::integral_constant<int, 2>{});
+    else requant_tile(std::integral_constant<int, 1>{});
     __syncthreads();
     const bool vec_ok = (N & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
     for (int it = 0; it < BM * (BN / 16) / NT; it++) {
@@ -1207,8 +1219,11 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
 // the B layout of `v_mfma_i32_16x16x64_i8`, so every wave keeps all of them and the main loop reads only activations
 // from LDS (one 16-byte fragment per four MFMAs, where nce_conv_tile reads six per four).  A wave walks blocks of 16
 // output positions x 64 channels: KY*KX fragment reads and 4*KY*KX MFMAs, then the PPE of the block's 16 values per
-// lane and one 16-byte store per lane -- no workgroup barrier after the staging, no output staging in LDS.  The two
-// waves of a SIMD are started half a block apart (`lag`), so that one requantises while the other multiplies.
+// lane and one 16-byte store per lane -- no workgroup barrier after the staging, no output staging in LDS.
+// (On this part the vector ALU work of one wave does not run under the MFMAs of the other wave of its SIMD, and
+// interleaving the PPE of block b-1 with the MFMAs of block b inside a wave needs a second set of accumulators,
+// which at two waves per SIMD spills: measured, a pipelined four-wave form with 32x32x32 MFMAs took 10.7 us where
+// this one takes 9.6 us at [32,56,56,64] -> 64.)
 //
 // Channel order inside a block: column n of MFMA tile j is output channel 16*(n/4) + 4*j + n%4.  After the 4x4 byte
 // transpose a lane then holds channels 16*q .. 16*q+15 of one position in its four result dwords (tile j -> dword j),
@@ -1217,7 +1232,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
 template <bool IN_U8, bool SAME_F, int KY, int KX>
 __global__ __launch_bounds__(512) void nce_conv_regw(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                      const int32_t* __restrict__ wt, uint8_t* __restrict__ out, ConvGeom g,
-                                                     PatchGeom pg, int pad_byte, GemmPpe ppe, int lag) {
+                                                     PatchGeom pg, int pad_byte, GemmPpe ppe) {
     constexpr int BN = 64, IC = 64, PS = IC + 16, NW = 8, NT = 64 * NW, TAPS = KY * KX, Ktot = TAPS * IC, WS = Ktot + 16;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* const wlds = smem;             // [64][Ktot + 16], rows in tile order
@@ -1355,10 +1370,6 @@ __global__ __launch_bounds__(512) void nce_conv_regw(const int8_t* __restrict__ 
     int soff[TAPS];
 #pragma unroll
     for (int t = 0; t < TAPS; t++) soff[t] = ((t / KX) * pg.PW + (t % KX)) * PS;
-
-    // the second wave of every SIMD starts late, so that its MFMAs meet the first one's PPE
-    if (wave >= NW / 2)
-        for (int i = 0; i < lag; i++) __builtin_amdgcn_s_sleep(1);
 
     auto one_block = [&](int b, auto general_c) {
         int p = b * 16 + n16;
@@ -1918,7 +1929,6 @@ struct Tuning {
     std::atomic<int> gemm_tile{0};          // VPX_GEMM_TILE = 128 | 256 (0: chosen from the shape)
     std::atomic<int> gemm_waves{0};         // VPX_GEMM_WAVES = 4 | 8
     std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = tile | stream: start the choice of LDS-patch kernel below the fastest one (1: tile, 2: stream)
-    std::atomic<int> conv_lag{-1};          // VPX_CONV_LAG = n: start-up lag of the second wave per SIMD in nce_conv_regw, units of 64 cycles
     std::atomic<int> conv_rows{0};          // VPX_CONV_ROWS = n: cap on the output rows per workgroup of the LDS-patch kernels
     std::atomic<int> conv_waves{0};         // VPX_CONV_WAVES = 4 | 8
     std::atomic<int> mvn_fused{1};          // VPX_MVN_FUSED = off | nowait (see tuning_mvn_fused)
@@ -1936,8 +1946,6 @@ bool set_knob(const char* knob, const char* value) {
         g_tuning.gemm_waves = *v ? (std::atoi(v) == 4 ? 4 : 8) : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_KERNEL")) {
         g_tuning.conv_stream = !std::strcmp(v, "stream") ? 2 : (!std::strcmp(v, "tile") ? 1 : 0);
-    } else if (!std::strcmp(knob, "VPX_CONV_LAG")) {
-        g_tuning.conv_lag = *v ? std::atoi(v) : -1;
     } else if (!std::strcmp(knob, "VPX_CONV_ROWS")) {
         g_tuning.conv_rows = std::atoi(v) > 0 ? std::atoi(v) : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_WAVES")) {
@@ -1952,7 +1960,7 @@ bool set_knob(const char* knob, const char* value) {
 
 const Tuning& tuning() {
     std::call_once(g_tuning_once, [] {
-        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES", "VPX_CONV_LAG", "VPX_MVN_FUSED"})
+        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES", "VPX_MVN_FUSED"})
             if (const char* v = std::getenv(k)) set_knob(k, v);
     });
     return g_tuning;
@@ -2228,14 +2236,13 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
                     const int pad_byte = t.zp_in & 0xff;
                     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
-                    const int lag = knobs.conv_lag.load() >= 0 ? knobs.conv_lag.load() : 0;
 #define VPX_REGW(U8, SAME)                                                                                            \
     do {                                                                                                              \
         auto kern = nce_conv_regw<U8, SAME, 3, 3>;                                                                    \
         rc = set_dyn_lds(kern, lds);                                                                                  \
         if (rc) return rc;                                                                                            \
         hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, \
-                           (uint8_t*)t.output, g, pg, pad_byte, gp, lag);                                             \
+                           (uint8_t*)t.output, g, pg, pad_byte, gp);                                                  \
     } while (0)
                     if (in_u8 && same_f) VPX_REGW(true, true);
                     else if (in_u8) VPX_REGW(true, false);
