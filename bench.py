@@ -33,7 +33,7 @@ METRIC = "int8 conv/matmul TOPS (% MFMA peak); SW-kernel GB/s (% HBM peak)"
 # WRITE_SIZE counters of an earlier run of the same workload, scaled by a plain copy of known size
 # (profiles/<workload>__*.md hold those runs and their commands); the JSON line labels them as such.
 MEASURED_TRAFFIC = {
-    "c1_fake_quantize": 888359, "c2_softmax": 134285956, "c3_mvn": 17028413, "c4_conv": 16276480,
+    "c1_fake_quantize": 888359, "c2_softmax": 134285956, "c3_mvn": 17028413, "c4_conv": 14908721,
     "c5_matmul": 339645868, "c5_dequantize": 135341729, "c5_eltwise_add": 270522802, "c5_nce_eltwise": 135260398,
     "calib_int_mm": 532970109, "x_mvn6_layernorm": 268490358, "x_activation_hswish": 180562131,
     "x_mvn1_three_steps": 25324896,
@@ -184,7 +184,7 @@ def make_c4(rt):
         return lambda: orc.nce_conv(c["input"], c["weights"], wt_h, p, zp_in=128, pads=(1, 1, 1, 1), rows=(0, rows)), \
             2 * rows * 64 * 9 * 64
     return Workload("c4_conv", "int8 Conv 3x3 s1 p1 NHWC [32,56,56,64] u8 zp128 x [64,3,3,64] i8, PPE ReLU clamp [0,255]",
-                    step, nbytes, ops, "mfma", "int8", "nce_conv_tile", cpu, (3136, 100352, "output positions"))
+                    step, nbytes, ops, "mfma", "int8", "nce_conv_regw", cpu, (3136, 100352, "output positions"))
 
 
 _C5_CACHE = {}
@@ -562,8 +562,9 @@ NOTES = {
                         "kernel 2.5-3 us (graph_device_ms_per_step); the eager figure of record is the host's launch rate over "
                         "418 separate parameter blobs. A single launch of this size cannot reach 0.70 of the HBM peak (that would be 0.14 us).",
     "c3_mvn": "16 MB in one launch of 8.2 us, of which about 2.6 us are the launch floor; 0.70 of the HBM peak would be 3.0 us end to end.",
-    "c4_conv": "7.4 GOP: about 2 us of MFMA or HBM time behind a launch floor of about 3 us; the kernel's four phases "
-               "(load, MFMA, requantise, store) overlap only across the two workgroups a compute unit holds.",
+    "c4_conv": "7.4 GOP: about 1.5 us of MFMA time and 1.5 us of HBM time. Measured by early returns: an empty kernel of this grid "
+               "1.6 us, the tile's loads back after 4.0 us, operands staged after 6.1 us, MFMAs + requantisation + stores 3.5 us "
+               "(on this part vector-ALU work does not run under MFMAs of the same SIMD, so the PPE's 5.5 instructions per value add to the MFMA time).",
     "c5_matmul": "power-limited: the part runs this kernel at 1.83-1.86 GHz on random int8 operands (2.4 GHz on zeros), where the "
                  "dense int8 peak is 3.9 POP/s; frac is against the 5.0 POP/s of 2.4 GHz. mfma_calibration in this line is what "
                  "a bare loop of the same MFMA sustains on this part: about 0.98 of the peak on zeros, 0.68 on random int8 operands, "
