@@ -29,7 +29,7 @@ def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0,
     OH = (H + pads[2] + pads[3] - KY) // strides[0] + 1
     OW = (W + pads[0] + pads[1] - KX) // strides[1] + 1
     out = torch.full((N, OH, OW, OC), 77, dtype=torch.float16 if out_f16 else (torch.int8 if out_signed else torch.uint8), device=dev)
-    if force in ("tile", "stream"):  # start the choice of LDS-patch kernel below the fastest one
+    if force in ("regw", "tile", "stream"):  # start the choice of LDS-patch kernel at this one
         rt.set_tuning("VPX_CONV_KERNEL", force)
     elif force:
         rt.set_tuning("VPX_NCE_KERNEL", force)
@@ -56,7 +56,8 @@ def rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=True, w_u8=False, shift_lo=12,
 
 
 def patch_kernel(g):
-    """The LDS-patch kernel a layer of 64 or 128 input channels takes: 3x3 taps of 64 channels keep the weights in registers."""
+    """The LDS-patch kernel a layer of 64 or 128 input channels takes when asked for the weights-in-registers kernel:
+    that one serves 3x3 taps of 64 channels (by itself the dispatcher picks it from about 50 000 input pixels on)."""
     return "nce_conv_regw" if (g["IC"], g["KY"], g["KX"]) == (64, 3, 3) else "nce_conv_tile"
 
 
@@ -64,7 +65,7 @@ U8 = {"clamp_low": 0, "clamp_high": 255}
 I8 = {"clamp_low": -128, "clamp_high": 127}
 
 
-@pytest.mark.parametrize("force", [None, "tile", "stream", "gather", "naive"])
+@pytest.mark.parametrize("force", [None, "regw", "stream", "gather", "naive"])
 @pytest.mark.parametrize("geom", [
     dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
     dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)),
@@ -85,8 +86,8 @@ def test_conv_paths(rt, orc, dev, geom, force):
     tile = g["IC"] in (64, 128)
     lds = g["IC"] % 64 == 0
     gather = "nce_conv_mfma" if g["IC"] % 32 == 0 else "nce_conv_mfma16"
-    expect = {None: patch_kernel(g) if tile else ("nce_conv_stream" if lds else gather),
-              "tile": "nce_conv_tile" if tile else ("nce_conv_stream" if lds else gather),
+    expect = {None: "nce_conv_tile" if tile else ("nce_conv_stream" if lds else gather),
+              "regw": patch_kernel(g) if tile else ("nce_conv_stream" if lds else gather),
               "stream": "nce_conv_stream" if lds else gather,
               "gather": gather, "naive": "nce_conv_naive"}[force]
     rng = np.random.default_rng(50 + g["H"])
@@ -99,7 +100,7 @@ def test_conv_paths(rt, orc, dev, geom, force):
 
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 5])
-@pytest.mark.parametrize("force,kernel", [(None, "nce_conv_regw"), ("tile", "nce_conv_tile"), ("stream", "nce_conv_stream")])
+@pytest.mark.parametrize("force,kernel", [("regw", "nce_conv_regw"), (None, "nce_conv_tile"), ("stream", "nce_conv_stream")])
 def test_conv_patch_tile_heights(rt, orc, dev, rows, force, kernel):
     """The LDS-patch kernels with the tile height forced: tiles that end past the last output row, one-row tiles."""
     rng = np.random.default_rng(55 + rows)
@@ -124,6 +125,7 @@ def test_naive_path_covers_odd_shapes_and_weight_zero_points(rt, orc, dev):
 
 @pytest.mark.parametrize("geom,kernel", [
     (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_regw"),
+    (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_tile"),
     (dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_stream"),
     (dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)), "nce_conv_mfma"),
     (dict(N=1, H=12, W=12, IC=16, OC=32, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_mfma16"),
@@ -137,16 +139,18 @@ def test_unsigned_weights_around_128_take_the_mfma_kernels(rt, orc, dev, geom, k
     for in_u8, zp_in in ((True, 128), (True, 7), (False, -5)):
         inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, w_u8=True, **g)
         got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, U8, zp_in=zp_in, zp_w=128, zp_out=3,
-                                   strides=strides, pads=pads)
+                                   strides=strides, pads=pads, force="regw" if kernel == "nce_conv_regw" else None)
         assert name == kernel
         assert np.array_equal(got, want), "%s zp_in=%d: %d mismatches" % (kernel, zp_in, int((got != want).sum()))
 
 
 WEIGHT_ZP_GEOMS = [
     (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_regw"),
+    (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_tile"),
     (dict(N=2, H=15, W=10, IC=128, OC=40, KY=3, KX=3, strides=(1, 1), pads=(1, 0, 0, 1)), "nce_conv_tile"),
     (dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_stream"),
     (dict(N=2, H=17, W=13, IC=64, OC=64, KY=3, KX=3, strides=(2, 2), pads=(1, 1, 1, 1)), "nce_conv_regw"),
+    (dict(N=2, H=17, W=13, IC=64, OC=64, KY=3, KX=3, strides=(2, 2), pads=(1, 1, 1, 1)), "nce_conv_tile"),
     (dict(N=2, H=12, W=13, IC=64, OC=64, KY=3, KX=2, strides=(2, 1), pads=(1, 1, 1, 1)), "nce_conv_tile"),
     (dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)), "nce_conv_mfma"),
     (dict(N=1, H=12, W=12, IC=16, OC=32, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_mfma16"),
@@ -176,7 +180,8 @@ def test_weight_zero_points_take_the_mfma_kernels(rt, orc, dev, geom, kernel):
         shifts = rng.integers(0, 3, len(shifts)) + max(1, int(np.ceil(np.log2(spread * 2 ** 15 / 128))))
         kw = dict(I8 if signed_out else U8, lrelu_mult=1638, lrelu_shift=14)
         got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, zp_out=-3 if signed_out else 9,
-                                   strides=strides, pads=pads, out_signed=signed_out, mode=rt.PPE_LPRELU)
+                                   strides=strides, pads=pads, out_signed=signed_out, mode=rt.PPE_LPRELU,
+                                   force="regw" if kernel == "nce_conv_regw" else None)
         assert name == kernel
         assert np.array_equal(got, want), "%s zp_in=%d zp_w=%d: %d mismatches" % (kernel, zp_in, zp_w, int((got != want).sum()))
         assert len(np.unique(got)) > 20  # the outputs are spread, not saturated
@@ -184,6 +189,7 @@ def test_weight_zero_points_take_the_mfma_kernels(rt, orc, dev, geom, kernel):
 
 @pytest.mark.parametrize("geom,kernel", [
     (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_regw"),
+    (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_tile"),
     (dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_stream"),
     (dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)), "nce_conv_mfma"),
     (dict(N=1, H=300, W=1, IC=128, OC=520, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_gemm_mfma"),
@@ -200,7 +206,7 @@ def test_negative_multipliers(rt, orc, dev, geom, kernel, mode):
     mults = np.where(rng.random(mults.shape) < 0.5, -mults, mults)
     kw = dict(I8, lrelu_mult=1638, lrelu_shift=14)
     got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=120, zp_out=-3, strides=strides, pads=pads,
-                               out_signed=True, mode=getattr(rt, "PPE_" + mode))
+                               out_signed=True, mode=getattr(rt, "PPE_" + mode), force="regw" if kernel == "nce_conv_regw" else None)
     assert name == kernel
     assert np.array_equal(got, want), "%s %s: %d mismatches" % (kernel, mode, int((got != want).sum()))
 

@@ -1928,7 +1928,7 @@ struct Tuning {
     std::atomic<int> nce_kernel{NCE_AUTO};  // VPX_NCE_KERNEL = naive | gather | conv: restrict the choice to slower, more general paths
     std::atomic<int> gemm_tile{0};          // VPX_GEMM_TILE = 128 | 256 (0: chosen from the shape)
     std::atomic<int> gemm_waves{0};         // VPX_GEMM_WAVES = 4 | 8
-    std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = tile | stream: start the choice of LDS-patch kernel below the fastest one (1: tile, 2: stream)
+    std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = regw | tile | stream: start the choice of LDS-patch kernel at this one (-1, 1, 2; 0: by size)
     std::atomic<int> conv_rows{0};          // VPX_CONV_ROWS = n: cap on the output rows per workgroup of the LDS-patch kernels
     std::atomic<int> conv_waves{0};         // VPX_CONV_WAVES = 4 | 8
     std::atomic<int> mvn_fused{1};          // VPX_MVN_FUSED = off | nowait (see tuning_mvn_fused)
@@ -1945,7 +1945,7 @@ bool set_knob(const char* knob, const char* value) {
     } else if (!std::strcmp(knob, "VPX_GEMM_WAVES")) {
         g_tuning.gemm_waves = *v ? (std::atoi(v) == 4 ? 4 : 8) : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_KERNEL")) {
-        g_tuning.conv_stream = !std::strcmp(v, "stream") ? 2 : (!std::strcmp(v, "tile") ? 1 : 0);
+        g_tuning.conv_stream = !std::strcmp(v, "stream") ? 2 : (!std::strcmp(v, "tile") ? 1 : (!std::strcmp(v, "regw") ? -1 : 0));
     } else if (!std::strcmp(knob, "VPX_CONV_ROWS")) {
         g_tuning.conv_rows = std::atoi(v) > 0 ? std::atoi(v) : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_WAVES")) {
@@ -2197,8 +2197,10 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             const int first = knobs.conv_stream.load();
             // (with 128 channels and a stride the haloed patch crowds the resident weights out of LDS: the
             // streamed-weights kernel below measures 15.7 us against 20.2 at [32,56,56,128] -> 128, 3x3, stride 2)
-            // 3x3 taps of 64 channels: the weights fit the registers of every wave
-            if (g.IC == 64 && g.KY == 3 && g.KX == 3 && first <= 0) {
+            // 3x3 taps of 64 channels: the weights fit the registers of every wave.  Copying them there costs about a
+            // microsecond per workgroup, which pays from about 50 000 input pixels on ([32,56,56,64] -> 64: 9.0 us against
+            // 9.5 us; [4,224,224,64] -> 64: 13.8 against 28.8; [32,28,28,64] -> 64: 7.0 against 6.4).
+            if (g.IC == 64 && g.KY == 3 && g.KX == 3 && (first < 0 || (first == 0 && g.N * g.H * g.W >= 50000))) {
                 PatchGeom pg{};
                 const int64_t PS = g.IC + 16, WS = Ktot + 16;
                 auto need = [&](int R) {
