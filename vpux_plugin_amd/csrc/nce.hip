@@ -1167,7 +1167,10 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
                                          (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
         asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));
         const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
-        const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 || pk.odd != 0;
+        // (the short PPE serves slopes in [0, 1], an even zero-point offset and scales up to 1/2: see ppe_pack4_biased)
+        const bool slope_ok = SAME_F || (ppe.prelu_mult >= 0 && (ppe.prelu_shift >= 31 || ppe.prelu_mult <= (1 << ppe.prelu_shift)));
+        const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 || pk.odd != 0 || !slope_ok;
+        const int pb = (int)((unsigned)cp.bias - 0x80000000u);  // the bias without the sign flip of the packed form
         const int col4 = nj * 32 + ((lane & 31) & ~3);
         if (ppe.rowterm) {
             const int32_t* rt = ppe.rowterm + ((int64_t)img * g.OH + oy0) * g.OW;
@@ -1184,8 +1187,12 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
                 if (mi0 + i * mstep >= pg.MT) continue;
 #pragma unroll
                 for (int gq = 0; gq < 4; gq++) {
-                    unsigned v = ppe_pack4<SAME_F, decltype(general_c)::value>(acc[i][gq * 4], acc[i][gq * 4 + 1],
-                                                                               acc[i][gq * 4 + 2], acc[i][gq * 4 + 3], cp, pk);
+                    unsigned v;
+                    if constexpr (decltype(general_c)::value)
+                        v = ppe_pack4<SAME_F, true>(acc[i][gq * 4], acc[i][gq * 4 + 1], acc[i][gq * 4 + 2], acc[i][gq * 4 + 3], cp, pk);
+                    else
+                        v = ppe_pack4_biased<!SAME_F>(acc[i][gq * 4] + pb, acc[i][gq * 4 + 1] + pb, acc[i][gq * 4 + 2] + pb,
+                                                      acc[i][gq * 4 + 3] + pb, cp.f_pos, cp.f_neg, pk);
                     v = quad_transpose_bytes(v, lane);
                     const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
                     *reinterpret_cast<unsigned*>(patch + row * kPatchOutStride + col4) = v;
@@ -1602,7 +1609,10 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
                                          (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * cs)), ppe.prelu_mult, ppe.prelu_shift);
         asm volatile("" : "+v"(cp.f_pos), "+v"(cp.f_neg));
         const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
-        const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 || pk.odd != 0;
+        // (the short PPE serves slopes in [0, 1], an even zero-point offset and scales up to 1/2: see ppe_pack4_biased)
+        const bool slope_ok = SAME_F || (ppe.prelu_mult >= 0 && (ppe.prelu_shift >= 31 || ppe.prelu_mult <= (1 << ppe.prelu_shift)));
+        const bool general = __builtin_amdgcn_ballot_w64(cp.bmax_pos != 0x7fffffff || cp.bmax_neg != 0x7fffffff) != 0 || pk.odd != 0 || !slope_ok;
+        const int pb = (int)((unsigned)cp.bias - 0x80000000u);  // the bias without the sign flip of the packed form
         const int col4 = nj * 32 + ((lane & 31) & ~3);
         if (ppe.rowterm) {
             const int32_t* rt = ppe.rowterm + ((int64_t)img * g.OH + oy0) * g.OW;
@@ -1619,8 +1629,12 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
                 if (mi0 + i * mstep >= pg.MT) continue;
 #pragma unroll
                 for (int gq = 0; gq < 4; gq++) {
-                    unsigned v = ppe_pack4<SAME_F, decltype(general_c)::value>(acc[i][gq * 4], acc[i][gq * 4 + 1],
-                                                                               acc[i][gq * 4 + 2], acc[i][gq * 4 + 3], cp, pk);
+                    unsigned v;
+                    if constexpr (decltype(general_c)::value)
+                        v = ppe_pack4<SAME_F, true>(acc[i][gq * 4], acc[i][gq * 4 + 1], acc[i][gq * 4 + 2], acc[i][gq * 4 + 3], cp, pk);
+                    else
+                        v = ppe_pack4_biased<!SAME_F>(acc[i][gq * 4] + pb, acc[i][gq * 4 + 1] + pb, acc[i][gq * 4 + 2] + pb,
+                                                      acc[i][gq * 4 + 3] + pb, cp.f_pos, cp.f_neg, pk);
                     v = quad_transpose_bytes(v, lane);
                     const int row = (mi0 + i * mstep) * 32 + 8 * gq + 4 * (lane >> 5) + (lane & 3);
                     *reinterpret_cast<unsigned*>(patch + row * kPatchOutStride + col4) = v;
