@@ -246,6 +246,50 @@ def test_conv_random_geometries(rt, orc, dev, seed, weight_zp):
         assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("seed", [3, 4, 5])
+def test_weights_in_registers_conv_random_geometries(rt, orc, dev, seed):
+    """The 3x3 x 64-channel kernel that keeps the weights in registers, asked for whatever the layer's size: seeded draws
+    of batch, size, stride, padding, channel count (tails of the 64- and 16-channel blocks), tile height, storage types,
+    zero points (weights too: the per-position term) and PPE settings on both sides of the short requantisation's
+    conditions (slope above 1, odd output zero point, scales above 1/2)."""
+    rng = np.random.default_rng(seed)
+    for i in range(24):
+        OC = int(rng.choice([1, 15, 16, 40, 64, 64, 72, 100, 128, 130]))
+        SY, SX = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        pl, pr, pt, pb = [int(v) for v in rng.integers(0, 3, 4)]
+        H, W, N = int(rng.integers(3, 45)), int(rng.integers(3, 75)), int(rng.integers(1, 4))
+        in_u8, out_signed = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        zp_in = int(rng.integers(0, 256)) if in_u8 else int(rng.integers(-128, 128))
+        mode = [rt.PPE_NOOP, rt.PPE_LPRELU, rt.PPE_LRELU][int(rng.integers(0, 3))]
+        # slopes: 0, inside (0, 1), exactly 1, above 1 (the multiplier field is unsigned)
+        lm, ls = [(0, 0), (1638, 14), (int(rng.integers(1, 2048)), 11), (4, 2), (5, 1), (2047, 3)][int(rng.integers(0, 6))]
+        kw = dict(I8 if out_signed else U8, lrelu_mult=lm, lrelu_shift=ls)
+        shift_lo, shift_hi = [(14, 26), (10, 16)][int(rng.integers(0, 2))]  # the second range holds scales above 1/2
+        w_u8, zp_w = False, 0
+        if rng.integers(0, 3) == 0:
+            w_u8 = bool(rng.integers(0, 2))
+            zp_w = int(rng.integers(0, 256)) if w_u8 else int(rng.integers(-128, 128))
+        rows = int(rng.integers(0, 6))  # 0: the dispatcher's choice
+        what = "seed %d case %d: N=%d H=%d W=%d OC=%d S=%dx%d pads=%s in_u8=%s out_signed=%s zp_in=%d mode=%d slope=%d/2^%d shifts=%d..%d w_u8=%s zp_w=%d rows=%d" % (
+            seed, i, N, H, W, OC, SY, SX, (pl, pr, pt, pb), in_u8, out_signed, zp_in, mode, lm, ls, shift_lo, shift_hi, w_u8, zp_w, rows)
+        print(what, flush=True)
+        inp, w, mults, shifts, bias = rand_case(rng, N, H, W, 64, OC, 3, 3, in_u8=in_u8, w_u8=w_u8, shift_lo=shift_lo, shift_hi=shift_hi)
+        if rng.integers(0, 2):
+            mults = np.where(rng.random(mults.shape) < 0.5, -mults, mults)
+        bias = (bias - np.int64(round(576 * (inp.mean() - zp_in) * (w.mean() - zp_w)))).astype(np.int32)
+        if rows:
+            rt.set_tuning("VPX_CONV_ROWS", rows)
+        try:
+            got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, zp_out=int(rng.integers(-5, 6)),
+                                       strides=(SY, SX), pads=(pl, pr, pt, pb), out_signed=out_signed, mode=mode, force="regw")
+        finally:
+            rt.set_tuning("VPX_CONV_ROWS", None)
+        # (weights whose zero point a signed copy cannot absorb with M % 4 != 0 positions, and the like, may take other kernels)
+        if zp_w == 0:
+            assert name == "nce_conv_regw", what
+        assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))
+
+
 @pytest.fixture(params=[("8", "256"), ("4", "256"), ("4", "128")], ids=["8w256", "4w256", "4w128"])
 def gemm_waves(request, rt):
     """The shapes of the matmul kernel: 256 x 256 tiles with two waves per SIMD (128 x 64 each) or one (128 x 128), and
