@@ -513,28 +513,42 @@ __device__ __forceinline__ void load_slice(const half_t* __restrict__ g, int64_t
 
 // Moments of the slice held by the workgroup: per wavefront by lane shuffles (mean first, then centred squares),
 // the four wavefronts' results merged in a fixed order by every lane.
+// The slice as single-precision values (the conversion is exact): both passes of the moments and the normalisation
+// read these, so every value is converted once.
 template <int V>
-__device__ __forceinline__ Moments slice_moments(const Slice<V>& sl, Moments* red) {
-    float sum = 0.f;
+struct SliceF {
+    float f[V][8];
+};
+template <int V>
+__device__ __forceinline__ void widen_slice(const Slice<V>& sl, SliceF<V>& w) {
 #pragma unroll
     for (int j = 0; j < V; j++) {
         const half_t* p = reinterpret_cast<const half_t*>(&sl.q[j]);
 #pragma unroll
-        for (int k = 0; k < 8; k++) sum += (float)p[k];
+        for (int k = 0; k < 8; k++) w.f[j][k] = (float)p[k];
     }
-    const float n = wave_sum((float)(8 * __builtin_popcount(sl.valid)));
+}
+
+template <int V>
+__device__ __forceinline__ Moments slice_moments(const SliceF<V>& w, unsigned valid, Moments* red) {
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < V; j++) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) sum += w.f[j][k];
+    }
+    const float n = wave_sum((float)(8 * __builtin_popcount(valid)));
     const float mean = n > 0.f ? wave_sum(sum) / n : 0.f;
     float q = 0.f;
 #pragma unroll
     for (int j = 0; j < V; j++) {
-        const half_t* p = reinterpret_cast<const half_t*>(&sl.q[j]);
         float qj = 0.f;
 #pragma unroll
         for (int k = 0; k < 8; k++) {
-            const float d = (float)p[k] - mean;
+            const float d = w.f[j][k] - mean;
             qj += d * d;
         }
-        q += (sl.valid >> j) & 1u ? qj : 0.f;
+        q += (valid >> j) & 1u ? qj : 0.f;
     }
     q = wave_sum(q);
     __syncthreads();  // the previous use of `red` is over
@@ -566,7 +580,9 @@ __global__ __launch_bounds__(kThreads) void mvn_fused_kernel(const half_t* __res
     const int64_t end = base + slice < group_size ? base + slice : group_size;
     Slice<V> sl;
     load_slice<V>(gin, base, end, sl);
-    Moments total = slice_moments<V>(sl, red);
+    SliceF<V> wide;
+    widen_slice<V>(sl, wide);
+    Moments total = slice_moments<V>(wide, sl.valid, red);
     if (wpg > 1) {
         if (threadIdx.x < 64) {  // the first wavefront
             if (lane == 0) {
@@ -616,7 +632,9 @@ __global__ __launch_bounds__(kThreads) void mvn_fused_kernel(const half_t* __res
                 const int64_t e = b + slice < group_size ? b + slice : group_size;
                 Slice<V> t;
                 load_slice<V>(gin, b, e, t);
-                const Moments mp = slice_moments<V>(t, red);
+                SliceF<V> tw;
+                widen_slice<V>(t, tw);
+                const Moments mp = slice_moments<V>(tw, t.valid, red);
                 if (threadIdx.x == 0) others[p] = mp;
             }
             __syncthreads();
@@ -642,11 +660,10 @@ __global__ __launch_bounds__(kThreads) void mvn_fused_kernel(const half_t* __res
 #pragma unroll
     for (int j = 0; j < V; j++) {
         if (!((sl.valid >> j) & 1u)) continue;
-        const half_t* p = reinterpret_cast<const half_t*>(&sl.q[j]);
         u32x4 r;
         half_t* o = reinterpret_cast<half_t*>(&r);
 #pragma unroll
-        for (int k = 0; k < 8; k++) o[k] = (half_t)(((float)p[k] - mean) * inv);
+        for (int k = 0; k < 8; k++) o[k] = (half_t)((wide.f[j][k] - mean) * inv);
         __builtin_nontemporal_store(r, reinterpret_cast<u32x4*>(gout + base + (int64_t)(j * kThreads + threadIdx.x) * 8));
     }
 }
