@@ -1501,9 +1501,10 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
         }
     };
 
-    // ---- patch and the first weight slice -> LDS
-    i32x4 wq[UWS];
-    slice_issue(0, wq);
+    // ---- patch and the first weight slice -> LDS.  Weight slices are asked for two slices ahead: the MFMAs of a
+    // slice can be much shorter than a trip to L2.
+    i32x4 wq[2][UWS];
+    slice_issue(0, wq[0]);
     {
         constexpr int UP = NW == 8 ? 4 : 6;
         const int cpp = IC / 16;
@@ -1537,7 +1538,9 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
                 }
         }
     }
-    slice_commit(0, wq);
+    const int slices = g.KY * g.KX * sg.spt;
+    slice_commit(0, wq[0]);
+    if (slices > 1) slice_issue(1, wq[1]);
     __syncthreads();
 
     // ---- main loop
@@ -1562,13 +1565,14 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[i][r] = 0;
 
-    const int slices = g.KY * g.KX * sg.spt;
     const int ksteps = KSL / 32;
     int ky = 0, kx = 0, sub = 0;  // position of the current slice
-    for (int sl = 0; sl < slices; sl++) {
-        const int buf = sl & 1;
+    // slice sl: its registers (set sl & 1) were stored to LDS an iteration ago and take slice sl + 2 now
+    auto one_slice = [&](int sl, auto parity_c) {
+        constexpr int par = decltype(parity_c)::value;
+        const int buf = par;
         const bool more = sl + 1 < slices;
-        if (more) slice_issue(sl + 1, wq);
+        if (sl + 2 < slices) slice_issue(sl + 2, wq[par]);
         const uint8_t* pa0 = patch + (ky * pg.PW + kx) * PS + sub * KSL;
         const uint8_t* pb = wbuf + buf * BN * WS + bbase;
         i32x4 fa[2][TMW], fb[2];
@@ -1586,7 +1590,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
 #pragma unroll
             for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[1][i], fb[1], acc[i], 0, 0, 0);
         }
-        if (more) slice_commit(buf ^ 1, wq);
+        if (more) slice_commit(buf ^ 1, wq[par ^ 1]);
         __syncthreads();  // slice sl+1 is visible; nobody reads buffer `buf` any more
         sub++;
         if (sub == sg.spt) {
@@ -1597,6 +1601,10 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
                 ky++;
             }
         }
+    };
+    for (int sl = 0; sl < slices; sl += 2) {
+        one_slice(sl, std::integral_constant<int, 0>{});
+        if (sl + 1 < slices) one_slice(sl + 1, std::integral_constant<int, 1>{});
     }
 
     // ---- epilogue (the last barrier of the loop has freed the patch)
@@ -2410,7 +2418,11 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         else if (same_f) VPX_STREAM_W(false, TMW, true, NW);                                                          \
         else VPX_STREAM_W(false, TMW, false, NW);                                                                     \
     } while (0)
-                    if (per_wave <= 2) VPX_STREAM(2, 8);
+                    // (a tile of one or two row blocks -- 7 x 7 planes -- would leave six of eight waves multiplying
+                    // padding: four waves, one block each, a third of the LDS reads per weight slice)
+                    if (pg.MT <= 4 / pg.nt) VPX_STREAM(1, 4);
+                    else if (per_wave <= 1) VPX_STREAM(1, 8);
+                    else if (per_wave <= 2) VPX_STREAM(2, 8);
                     else VPX_STREAM(4, 8);
 #undef VPX_STREAM
 #undef VPX_STREAM_W
