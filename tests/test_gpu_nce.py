@@ -57,7 +57,7 @@ def rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=True, w_u8=False, shift_lo=12,
 
 def patch_kernel(g):
     """The LDS-patch kernel a layer of 64 or 128 input channels takes when asked for the weights-in-registers kernel:
-    that one serves 3x3 taps of 64 channels (by itself the dispatcher picks it from about 50 000 input pixels on)."""
+    that one serves 3x3 taps of 64 channels (by itself the dispatcher picks it from about 50 000 output positions on)."""
     return "nce_conv_regw" if (g["IC"], g["KY"], g["KX"]) == (64, 3, 3) else "nce_conv_tile"
 
 

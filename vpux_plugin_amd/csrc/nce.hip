@@ -2217,12 +2217,16 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             // channels do not fit the registers twice)
             // VPX_CONV_KERNEL=stream starts the choice below the tile kernel (tests compare them)
             const int first = knobs.conv_stream.load();
+            int cus_here = 0;
+            rc = device_compute_units(&cus_here);
+            if (rc) return rc;
             // (with 128 channels and a stride the haloed patch crowds the resident weights out of LDS: the
             // streamed-weights kernel below measures 15.7 us against 20.2 at [32,56,56,128] -> 128, 3x3, stride 2)
             // 3x3 taps of 64 channels: the weights fit the registers of every wave.  Copying them there costs about a
-            // microsecond per workgroup, which pays from about 50 000 input pixels on ([32,56,56,64] -> 64: 9.0 us against
-            // 9.5 us; [4,224,224,64] -> 64: 13.8 against 28.8; [32,28,28,64] -> 64: 7.0 against 6.4).
-            if (g.IC == 64 && g.KY == 3 && g.KX == 3 && (first < 0 || (first == 0 && g.N * g.H * g.W >= 50000))) {
+            // microsecond per workgroup, which pays from about 50 000 output positions on ([32,56,56,64] -> 64: 9.1 us
+            // against 9.5 us; [4,224,224,64] -> 64: 13.9 against 29.2; [32,28,28,64] -> 64: 7.0 against 6.0; the same input
+            // at stride 2: 7.5 against 7.1).
+            if (g.IC == 64 && g.KY == 3 && g.KX == 3 && (first < 0 || (first == 0 && g.N * g.OH * g.OW >= 50000))) {
                 PatchGeom pg{};
                 const int64_t PS = g.IC + 16, WS = Ktot + 16;
                 auto need = [&](int R) {
@@ -2291,7 +2295,13 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 while (R > 1 && need(R) > 160 * 1024 - 512) R--;
                 if (need(R) <= 160 * 1024 - 512) {
                     const int64_t ocb = (g.OC + 63) / 64;
-                    while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 512 && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
+                    // shorter tiles while they are few: down to 128 positions, or to 64 while there are fewer tiles
+                    // than compute units ([32,14,14,256] -> 256, 3x3: 12.1 us with 256 tiles of 7 rows, 15.4 us with 128 of 14)
+                    while (R > 1) {
+                        const int64_t tiles = g.N * ((g.OH + R - 1) / R) * ocb;
+                        if (tiles >= 512 || ((R + 1) / 2) * g.OW < (tiles < cus_here ? 64 : 128)) break;
+                        R = (R + 1) / 2;
+                    }
                     if (const int v = knobs.conv_rows.load()) {
                         if (v >= 1 && v <= R) R = v;
                     }
@@ -2370,7 +2380,13 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 while (R > 1 && need(R) > 160 * 1024 - 512) R--;
                 if (need(R) <= 160 * 1024 - 512) {
                     const int64_t ocb = (g.OC + 63) / 64;
-                    while (R > 1 && g.N * ((g.OH + R - 1) / R) * ocb < 512 && ((R + 1) / 2) * g.OW >= 128) R = (R + 1) / 2;
+                    // shorter tiles while they are few: down to 128 positions, or to 64 while there are fewer tiles
+                    // than compute units ([32,14,14,256] -> 256, 3x3: 12.1 us with 256 tiles of 7 rows, 15.4 us with 128 of 14)
+                    while (R > 1) {
+                        const int64_t tiles = g.N * ((g.OH + R - 1) / R) * ocb;
+                        if (tiles >= 512 || ((R + 1) / 2) * g.OW < (tiles < cus_here ? 64 : 128)) break;
+                        R = (R + 1) / 2;
+                    }
                     if (const int v = knobs.conv_rows.load()) {
                         if (v >= 1 && v <= R) R = v;
                     }
