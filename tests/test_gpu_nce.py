@@ -29,8 +29,9 @@ def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0,
     OH = (H + pads[2] + pads[3] - KY) // strides[0] + 1
     OW = (W + pads[0] + pads[1] - KX) // strides[1] + 1
     out = torch.full((N, OH, OW, OC), 77, dtype=torch.float16 if out_f16 else (torch.int8 if out_signed else torch.uint8), device=dev)
-    if force in ("regw", "tile", "stream"):  # start the choice of LDS-patch kernel at this one
+    if force in ("regw", "tile", "stream"):  # the LDS-patch kernels only, starting the choice at this one
         rt.set_tuning("VPX_CONV_KERNEL", force)
+        rt.set_tuning("VPX_NCE_KERNEL", "conv")
     elif force:
         rt.set_tuning("VPX_NCE_KERNEL", force)
     try:
@@ -86,7 +87,10 @@ def test_conv_paths(rt, orc, dev, geom, force):
     tile = g["IC"] in (64, 128)
     lds = g["IC"] % 64 == 0
     gather = "nce_conv_mfma" if g["IC"] % 32 == 0 else "nce_conv_mfma16"
-    expect = {None: "nce_conv_tile" if tile else ("nce_conv_stream" if lds else gather),
+    # (a 1x1 layer without padding is a matmul, with or without a stride, unless its few channels suit the 64-wide tiles better)
+    M = g["N"] * ((g["H"] - 1) // strides[0] + 1) * ((g["W"] - 1) // strides[1] + 1)
+    matmul = (g["KY"], g["KX"]) == (1, 1) and pads == (0, 0, 0, 0) and g["IC"] % 64 == 0 and (g["OC"] > 64 or M < 1024)
+    expect = {None: "nce_gemm_mfma" if matmul else ("nce_conv_tile" if tile else ("nce_conv_stream" if lds else gather)),
               "regw": patch_kernel(g) if tile else ("nce_conv_stream" if lds else gather),
               "stream": "nce_conv_stream" if lds else gather,
               "gather": gather, "naive": "nce_conv_naive"}[force]
@@ -97,6 +101,26 @@ def test_conv_paths(rt, orc, dev, geom, force):
                                    strides=strides, pads=pads, out_signed=out_signed, force=force)
         assert name == expect
         assert np.array_equal(got, want), "%s zp_in=%d: %d mismatches" % (name, zp_in, int((got != want).sum()))
+
+
+@pytest.mark.parametrize("geom", [
+    dict(N=2, H=17, W=13, IC=128, OC=200, strides=(2, 2)),
+    dict(N=3, H=9, W=30, IC=64, OC=70, strides=(1, 2)),
+    dict(N=1, H=41, W=7, IC=320, OC=513, strides=(3, 1)),
+    dict(N=2, H=56, W=56, IC=256, OC=512, strides=(2, 2)),
+])
+def test_strided_1x1_layers_take_the_matmul_kernel(rt, orc, dev, geom):
+    """A 1x1 convolution with a stride (the shortcut branches of a ResNet) is a matmul over rows picked from the input."""
+    g = dict(geom)
+    strides = g.pop("strides")
+    rng = np.random.default_rng(77 + g["H"])
+    for in_u8, zp_in, zp_w, out_signed in ((True, 128, 0, False), (True, 9, 0, True), (False, -5, 0, False), (True, 128, 31, False)):
+        inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, KY=1, KX=1, **g)
+        kw = dict(I8 if out_signed else U8, lrelu_mult=1638, lrelu_shift=14)
+        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, zp_out=4, strides=strides,
+                                   out_signed=out_signed, mode=rt.PPE_LPRELU)
+        assert name == "nce_gemm_mfma"
+        assert np.array_equal(got, want), "zp_in=%d zp_w=%d: %d mismatches" % (zp_in, zp_w, int((got != want).sum()))
 
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 5])

@@ -487,6 +487,15 @@ struct GemmPpe {
     float f16_lo, f16_hi;         // fp16 output: clamp bounds
 };
 
+// Where the rows of A sit: row m at byte m * K (a matrix, or a 1x1 stride-1 layer), or, for a 1x1 layer with a stride,
+// output position m = (n, oy, ox) at pixel (n, oy * sy, ox * sx) of the input tensor -- the matmul kernel's loads
+// take a byte offset per lane, so a strided 1x1 convolution is a matmul whose rows are picked from the input.
+struct GemmRows {
+    int strided;              // 0: dense rows
+    int ow, ohow, sx, sy;     // output width, positions per image, strides
+    int w, hw;                // input width, pixels per image
+};
+
 // A[M][K] x B[N][K]^T with the PPE fused; see the file header.  K must be a multiple of 64.
 //
 // Pipeline.  K is walked in panels of 64 bytes; a panel of A and B (32 KiB) goes from global memory
@@ -502,7 +511,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                                                      const int32_t* __restrict__ wt, const int32_t* __restrict__ colsum,
                                                      uint8_t* __restrict__ out,
                                                      int64_t M, int64_t N, int64_t K, int tiles_m, int tiles_n,
-                                                     GemmPpe ppe) {
+                                                     GemmPpe ppe, GemmRows rows) {
     // NW = 4: waves 2 x 2, 128 x 128 each, one per SIMD.  NW = 8: waves 2 x 4, 128 x 64 each, two per SIMD,
     // so that one wave's loads and address arithmetic issue while the other's MFMAs run.
     // TILE = 128 (four waves of 64 x 64, 64 KiB of LDS, two workgroups per CU) serves problems with too few 256 x 256 tiles.
@@ -566,9 +575,13 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
         m = m < M ? m : M - 1;  // rows past the edge repeat the last one; their outputs are not stored
         n = n < N ? n : N - 1;
         oa[i] = (unsigned)((m - m0) * K + c * 16);
+        if (rows.strided) {  // (offsets from the tensor's first byte; the host has checked that they fit 32 bits)
+            const int mm = (int)m, img = mm / rows.ohow, rem = mm - img * rows.ohow, oy = rem / rows.ow, ox = rem - oy * rows.ow;
+            oa[i] = (unsigned)(img * rows.hw + oy * rows.sy * rows.w + ox * rows.sx) * (unsigned)K + (unsigned)(c * 16);
+        }
         ob[i] = (unsigned)((n - n0) * K + c * 16);
     }
-    const int8_t* abase = A + m0 * K;
+    const int8_t* abase = rows.strided ? A : A + m0 * K;
     const int8_t* bbase = B + n0 * K;
     const unsigned lds0 = lds_address(smem);
     const int nk = (int)(K / BK);
@@ -2055,8 +2068,11 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const int wz_rest = (w_u8 ? 128 : 0) - t.zp_w;
     const bool mfma_ok = (!w_u8 || w_rebias) && zp_w_ok && zp_in_ok && zp_out_ok && Mtot < (1ll << 31) && g.OC < (1ll << 31) &&
                          (wz_rest == 0 || (g.IC % 16 == 0 && g.N * g.H * g.W < (1ll << 31) && g.IC < (1 << 23)));
-    const bool is_gemm = g.KY == 1 && g.KX == 1 && g.SY == 1 && g.SX == 1 && t.kernel_padding[0] == 0 &&
-                         t.kernel_padding[1] == 0 && t.kernel_padding[2] == 0 && t.kernel_padding[3] == 0;
+    const bool is_1x1 = g.KY == 1 && g.KX == 1 && t.kernel_padding[0] == 0 && t.kernel_padding[1] == 0 &&
+                        t.kernel_padding[2] == 0 && t.kernel_padding[3] == 0;
+    const bool is_gemm = is_1x1 && g.SY == 1 && g.SX == 1;
+    // a 1x1 layer with a stride is a matmul over rows picked from the input (one group, tensor below 4 GiB)
+    const bool is_strided_gemm = is_1x1 && !is_gemm && t.groups <= 1 && g.N * g.H * g.W * g.IC < (1ll << 32);
     const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights)) & 15) == 0;
     // VPX_NCE_KERNEL=naive|gather|conv restricts the choice to the slower, more general paths (used by tests
     // to check the device paths against each other).
@@ -2069,7 +2085,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     // A 256-column matmul tile wastes three quarters of its MFMAs on 64 output channels: such 1x1 layers go
     // to the convolution kernels, whose tiles are 64 channels wide (measured 7 us against 18 us at [100352 x 64 x 64]).
     const int64_t gemm_tiles = ((Mtot + 255) / 256) * ((g.OC + 255) / 256);
-    const bool use_gemm = allow_gemm && is_gemm && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || Mtot < 1024);
+    const bool use_gemm = allow_gemm && (is_gemm || is_strided_gemm) && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || Mtot < 1024);
     // VPU.NCE.MatMul's groups: one launch of the matmul kernel when it serves the shape (the preparation passes then
     // walk all groups' weights / activations as one tensor), else one task after the other on the stream.
     const int64_t G = t.groups > 1 ? t.groups : 1;
@@ -2178,13 +2194,14 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             lds += kGemmLdsHead;
             GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi};
             const int32_t* colsum = nullptr;  // the kernel sums the columns of B itself, from the fragments it reads
+            const GemmRows rows{is_gemm ? 0 : 1, (int)g.OW, (int)(g.OH * g.OW), g.SX, g.SY, (int)g.W, (int)(g.H * g.W)};
 #define VPX_GEMM_W(U8, SGN, NW, TILE, SHORTK)                                                                        \
     do {                                                                                                             \
         auto kern = nce_gemm_mfma<U8, SGN, NW, TILE, SHORTK>;                                                        \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
         hipLaunchKernelGGL(kern, grid, block, lds, s, (const int8_t*)t.input, (const int8_t*)wptr,              \
-                           t.weight_table, colsum, (uint8_t*)t.output, Mtot, g.OC, g.IC, tiles_m, tiles_n, gp);      \
+                           t.weight_table, colsum, (uint8_t*)t.output, Mtot, g.OC, g.IC, tiles_m, tiles_n, gp, rows); \
     } while (0)
 #define VPX_GEMM(U8, SGN)                                                                                            \
     do {                                                                                                             \
