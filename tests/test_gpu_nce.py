@@ -62,6 +62,9 @@ def patch_kernel(g):
     return "nce_conv_regw" if (g["IC"], g["KY"], g["KX"]) == (64, 3, 3) else "nce_conv_tile"
 
 
+# kernels the dispatcher picks only when asked to (or, the first, from a size on): the knob that asks
+FORCE_FOR = {"nce_conv_regw": "regw", "nce_conv_mfma16": "gather"}
+
 U8 = {"clamp_low": 0, "clamp_high": 255}
 I8 = {"clamp_low": -128, "clamp_high": 127}
 
@@ -87,12 +90,14 @@ def test_conv_paths(rt, orc, dev, geom, force):
     tile = g["IC"] in (64, 128)
     lds = g["IC"] % 64 == 0
     gather = "nce_conv_mfma" if g["IC"] % 32 == 0 else "nce_conv_mfma16"
+    # (channel counts that are a multiple of 16 only: the row-patch kernel wherever an LDS kernel may run)
+    other = gather if g["IC"] % 32 == 0 else "nce_conv_rows16"
     # (a 1x1 layer without padding is a matmul, with or without a stride, unless its few channels suit the 64-wide tiles better)
     M = g["N"] * ((g["H"] - 1) // strides[0] + 1) * ((g["W"] - 1) // strides[1] + 1)
     matmul = (g["KY"], g["KX"]) == (1, 1) and pads == (0, 0, 0, 0) and g["IC"] % 64 == 0 and (g["OC"] > 64 or M < 1024)
-    expect = {None: "nce_gemm_mfma" if matmul else ("nce_conv_tile" if tile else ("nce_conv_stream" if lds else gather)),
-              "regw": patch_kernel(g) if tile else ("nce_conv_stream" if lds else gather),
-              "stream": "nce_conv_stream" if lds else gather,
+    expect = {None: "nce_gemm_mfma" if matmul else ("nce_conv_tile" if tile else ("nce_conv_stream" if lds else other)),
+              "regw": patch_kernel(g) if tile else ("nce_conv_stream" if lds else other),
+              "stream": "nce_conv_stream" if lds else other,
               "gather": gather, "naive": "nce_conv_naive"}[force]
     rng = np.random.default_rng(50 + g["H"])
     for in_u8, zp_in, out_signed in ((True, 128, False), (True, 7, True), (False, -5, False), (False, 0, True)):
@@ -152,6 +157,7 @@ def test_naive_path_covers_odd_shapes_and_weight_zero_points(rt, orc, dev):
     (dict(N=2, H=9, W=11, IC=64, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_tile"),
     (dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_stream"),
     (dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)), "nce_conv_mfma"),
+    (dict(N=1, H=12, W=12, IC=16, OC=32, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_rows16"),
     (dict(N=1, H=12, W=12, IC=16, OC=32, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_mfma16"),
     (dict(N=1, H=300, W=1, IC=128, OC=520, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_gemm_mfma"),
 ])
@@ -163,7 +169,7 @@ def test_unsigned_weights_around_128_take_the_mfma_kernels(rt, orc, dev, geom, k
     for in_u8, zp_in in ((True, 128), (True, 7), (False, -5)):
         inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, w_u8=True, **g)
         got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, U8, zp_in=zp_in, zp_w=128, zp_out=3,
-                                   strides=strides, pads=pads, force="regw" if kernel == "nce_conv_regw" else None)
+                                   strides=strides, pads=pads, force=FORCE_FOR.get(kernel))
         assert name == kernel
         assert np.array_equal(got, want), "%s zp_in=%d: %d mismatches" % (kernel, zp_in, int((got != want).sum()))
 
@@ -177,6 +183,7 @@ WEIGHT_ZP_GEOMS = [
     (dict(N=2, H=17, W=13, IC=64, OC=64, KY=3, KX=3, strides=(2, 2), pads=(1, 1, 1, 1)), "nce_conv_tile"),
     (dict(N=2, H=12, W=13, IC=64, OC=64, KY=3, KX=2, strides=(2, 1), pads=(1, 1, 1, 1)), "nce_conv_tile"),
     (dict(N=1, H=14, W=14, IC=32, OC=48, KY=3, KX=3, strides=(2, 2), pads=(0, 1, 0, 1)), "nce_conv_mfma"),
+    (dict(N=1, H=12, W=12, IC=16, OC=32, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_rows16"),
     (dict(N=1, H=12, W=12, IC=16, OC=32, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)), "nce_conv_mfma16"),
     (dict(N=3, H=40, W=10, IC=64, OC=64, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_conv_tile"),
     (dict(N=1, H=300, W=1, IC=128, OC=520, KY=1, KX=1, strides=(1, 1), pads=(0, 0, 0, 0)), "nce_gemm_mfma"),
@@ -205,7 +212,7 @@ def test_weight_zero_points_take_the_mfma_kernels(rt, orc, dev, geom, kernel):
         kw = dict(I8 if signed_out else U8, lrelu_mult=1638, lrelu_shift=14)
         got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, zp_out=-3 if signed_out else 9,
                                    strides=strides, pads=pads, out_signed=signed_out, mode=rt.PPE_LPRELU,
-                                   force="regw" if kernel == "nce_conv_regw" else None)
+                                   force=FORCE_FOR.get(kernel))
         assert name == kernel
         assert np.array_equal(got, want), "%s zp_in=%d zp_w=%d: %d mismatches" % (kernel, zp_in, zp_w, int((got != want).sum()))
         assert len(np.unique(got)) > 20  # the outputs are spread, not saturated
@@ -230,7 +237,7 @@ def test_negative_multipliers(rt, orc, dev, geom, kernel, mode):
     mults = np.where(rng.random(mults.shape) < 0.5, -mults, mults)
     kw = dict(I8, lrelu_mult=1638, lrelu_shift=14)
     got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=120, zp_out=-3, strides=strides, pads=pads,
-                               out_signed=True, mode=getattr(rt, "PPE_" + mode), force="regw" if kernel == "nce_conv_regw" else None)
+                               out_signed=True, mode=getattr(rt, "PPE_" + mode), force=FORCE_FOR.get(kernel))
     assert name == kernel
     assert np.array_equal(got, want), "%s %s: %d mismatches" % (kernel, mode, int((got != want).sum()))
 
@@ -314,6 +321,74 @@ def test_weights_in_registers_conv_random_geometries(rt, orc, dev, seed):
         assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_row_patch_conv_random_geometries(rt, orc, dev, seed):
+    """The stem-layer kernel (channel counts that are a multiple of 16 only; input rows resident in LDS, K walked kernel row
+    by kernel row): seeded draws of channel count (one, three, five and seven chunks a pixel), kernel size up to 7x7
+    (odd chunk counts per kernel row meet the spare zero chunk), stride, padding, output channels (tails of the 64- and
+    16-channel blocks), tile height, storage types, zero points (weights too) and PPE settings on both sides of the
+    short requantisation's conditions."""
+    rng = np.random.default_rng(seed)
+    for i in range(24):
+        IC = int(rng.choice([16, 16, 16, 48, 80, 112]))
+        OC = int(rng.choice([1, 15, 16, 32, 40, 64, 64, 72, 100, 128, 130]))
+        KY, KX = int(rng.integers(1, 8)), int(rng.integers(1, 8))
+        SY, SX = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        pl, pr, pt, pb = [int(v) for v in rng.integers(0, 4, 4)]
+        pl, pr, pt, pb = min(pl, KX - 1), min(pr, KX - 1), min(pt, KY - 1), min(pb, KY - 1)
+        H, W, N = int(rng.integers(KY, 45)), int(rng.integers(KX, 75)), int(rng.integers(1, 4))
+        in_u8, out_signed = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        zp_in = int(rng.integers(0, 256)) if in_u8 else int(rng.integers(-128, 128))
+        mode = [rt.PPE_NOOP, rt.PPE_LPRELU, rt.PPE_LRELU][int(rng.integers(0, 3))]
+        lm, ls = [(0, 0), (1638, 14), (int(rng.integers(1, 2048)), 11), (4, 2), (5, 1), (2047, 3)][int(rng.integers(0, 6))]
+        kw = dict(I8 if out_signed else U8, lrelu_mult=lm, lrelu_shift=ls)
+        shift_lo, shift_hi = [(14, 26), (10, 16)][int(rng.integers(0, 2))]  # the second range holds scales above 1/2
+        w_u8, zp_w = False, 0
+        if rng.integers(0, 3) == 0:
+            w_u8 = bool(rng.integers(0, 2))
+            zp_w = int(rng.integers(0, 256)) if w_u8 else int(rng.integers(-128, 128))
+        rows = int(rng.integers(0, 6))  # 0: the dispatcher's choice
+        what = "seed %d case %d: N=%d H=%d W=%d IC=%d OC=%d K=%dx%d S=%dx%d pads=%s in_u8=%s out_signed=%s zp_in=%d mode=%d slope=%d/2^%d shifts=%d..%d w_u8=%s zp_w=%d rows=%d" % (
+            seed, i, N, H, W, IC, OC, KY, KX, SY, SX, (pl, pr, pt, pb), in_u8, out_signed, zp_in, mode, lm, ls, shift_lo, shift_hi, w_u8, zp_w, rows)
+        print(what, flush=True)
+        inp, w, mults, shifts, bias = rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=in_u8, w_u8=w_u8, shift_lo=shift_lo, shift_hi=shift_hi)
+        if rng.integers(0, 2):
+            mults = np.where(rng.random(mults.shape) < 0.5, -mults, mults)
+        bias = (bias - np.int64(round(KY * KX * IC * (inp.mean() - zp_in) * (w.mean() - zp_w)))).astype(np.int32)
+        if rows:
+            rt.set_tuning("VPX_CONV_ROWS", rows)
+        try:
+            got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, zp_out=int(rng.integers(-5, 6)),
+                                       strides=(SY, SX), pads=(pl, pr, pt, pb), out_signed=out_signed, mode=mode)
+        finally:
+            rt.set_tuning("VPX_CONV_ROWS", None)
+        # (the kernel wants the weights of 64 channels -- kernel rows padded to an even chunk count -- and the input rows
+        # under one output row in LDS together; layers beyond that take the gather or the plain kernel)
+        OW = (W + pl + pr - KX) // SX + 1
+        lds = 64 * (KY * ((KX * IC // 16 + 1) // 2 * 2) * 16 + 16) + 64 * 32 + 2 * 64 * 4 + 16 + KY * (((OW - 1) * SX + KX) * IC + 16)
+        if lds <= 160 * 1024 - 512:
+            assert name == "nce_conv_rows16", what
+        assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))
+
+
+def test_row_patch_conv_stem_layer(rt, orc, dev):
+    """A ResNet stem at a size the oracle still finishes quickly ([2,224,224,16] -> 64, 7x7, stride 2, padding 3): full-width
+    rows of 229 pixels in LDS, tiles of several output rows, workgroups that take more than one tile."""
+    rng = np.random.default_rng(21)
+    inp, w, mults, shifts, bias = rand_case(rng, 2, 224, 224, 16, 64, 7, 7, shift_lo=16, shift_hi=20)
+    kw = dict(U8, lrelu_mult=0, lrelu_shift=0)
+    for rows in (0, 1, 3):
+        if rows:
+            rt.set_tuning("VPX_CONV_ROWS", rows)
+        try:
+            got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=128, zp_out=0, strides=(2, 2),
+                                       pads=(3, 3, 3, 3), mode=rt.PPE_LRELU)
+        finally:
+            rt.set_tuning("VPX_CONV_ROWS", None)
+        assert name == "nce_conv_rows16"
+        assert np.array_equal(got, want), "rows=%d: %d mismatches" % (rows, int((got != want).sum()))
+
+
 @pytest.fixture(params=[("8", "256"), ("4", "256"), ("4", "128")], ids=["8w256", "4w256", "4w128"])
 def gemm_waves(request, rt):
     """The shapes of the matmul kernel: 256 x 256 tiles with two waves per SIMD (128 x 64 each) or one (128 x 128), and
@@ -365,7 +440,7 @@ def test_ppe_modes_and_rounding_edges(rt, orc, dev, mode):
     (2, 256, 192, 320, True, 7, True, 131, False, "nce_gemm_mfma"),    # weight zero point: per-position term, M % 4 == 0
     (2, 130, 128, 96, False, -2, False, 0, True, "nce_gemm_mfma"),     # fp16 output
     (3, 33, 128, 80, True, 9, True, 120, False, "nce_gemm_mfma"),      # weight zero point with M % 4 != 0: group after group
-    (2, 40, 48, 72, False, 1, False, 0, False, "nce_conv_mfma16"),     # K not a multiple of 64: group after group
+    (2, 40, 48, 72, False, 1, False, 0, False, "nce_conv_rows16"),     # K not a multiple of 64: group after group
 ])
 def test_grouped_matmul_one_task(rt, orc, dev, G, M, K, N, in_u8, zp_a, w_u8, zp_b, out_f16, kernel):
     """VPU.NCE.MatMul with G groups ([G,1,K,M,1] x [G,N,K,1,1], weight table [G,N,1,1,4]) as one task: bit-exact against

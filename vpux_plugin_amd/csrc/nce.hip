@@ -245,31 +245,35 @@ __device__ __forceinline__ int med3_i32(int v, int lo, int hi) {
 // `c` must come from ppe_prepare_packed: its bias carries the +2^31 that turns the int -> double bit trick's sign
 // flip into part of the bias addition, and for a negative multiplier its two factors (and bounds) are swapped, so
 // that "the scaled value is negative" is simply "acc + bias is negative", whatever the multiplier's sign.
+// (one value: the clamped integer in [0, 255] before the byte is placed and the sign bits flipped)
+template <bool SAME_F, bool GENERAL>
+__device__ __forceinline__ unsigned ppe_one(int a, const ChanPrep& c, const PpePack& p) {
+    unsigned bu = (unsigned)a + (unsigned)c.bias;  // (acc + bias) ^ 0x80000000
+    double f = c.f_pos;
+    int bm = c.bmax_pos;
+    if (!SAME_F) {
+        const bool neg = (int)bu >= 0;  // flipped domain: top bit clear means acc + bias < 0
+        f = neg ? c.f_neg : c.f_pos;
+        if (GENERAL) bm = neg ? c.bmax_neg : c.bmax_pos;
+    }
+    if (GENERAL) {
+        int b = (int)(bu ^ 0x80000000u);
+        b = b > bm ? bm : (b < -bm ? -bm : b);
+        bu = (unsigned)b ^ 0x80000000u;
+    }
+    const double bd = __builtin_bit_cast(double, 0x4330000000000000ull | (unsigned long long)bu) - 4503601774854144.0;
+    const double y = __builtin_fma(bd, f, p.magic);
+    int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, y);
+    if (GENERAL) q += p.odd;
+    return (unsigned)med3_i32(q, p.lo, p.hi);
+}
+
 template <bool SAME_F, bool GENERAL>
 __device__ __forceinline__ unsigned ppe_pack4(int a0, int a1, int a2, int a3, const ChanPrep& c, const PpePack& p) {
     const int a[4] = {a0, a1, a2, a3};
     unsigned w = 0;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        unsigned bu = (unsigned)a[r] + (unsigned)c.bias;  // (acc + bias) ^ 0x80000000
-        double f = c.f_pos;
-        int bm = c.bmax_pos;
-        if (!SAME_F) {
-            const bool neg = (int)bu >= 0;  // flipped domain: top bit clear means acc + bias < 0
-            f = neg ? c.f_neg : c.f_pos;
-            if (GENERAL) bm = neg ? c.bmax_neg : c.bmax_pos;
-        }
-        if (GENERAL) {
-            int b = (int)(bu ^ 0x80000000u);
-            b = b > bm ? bm : (b < -bm ? -bm : b);
-            bu = (unsigned)b ^ 0x80000000u;
-        }
-        const double bd = __builtin_bit_cast(double, 0x4330000000000000ull | (unsigned long long)bu) - 4503601774854144.0;
-        const double y = __builtin_fma(bd, f, p.magic);
-        int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, y);
-        if (GENERAL) q += p.odd;
-        w |= (unsigned)med3_i32(q, p.lo, p.hi) << (8 * r);
-    }
+    for (int r = 0; r < 4; r++) w |= ppe_one<SAME_F, GENERAL>(a[r], c, p) << (8 * r);
     return w ^ p.flip;
 }
 
@@ -294,19 +298,22 @@ __device__ __forceinline__ ChanPrep ppe_prepare_packed(int mult, int shift, int 
 // PReLU up to 1): then b * f_neg >= b * f_pos exactly when b < 0, so the larger of the two rounded products is the
 // result and no sign test is needed (rounding is monotone).  `c` comes from ppe_prepare (not _packed).
 template <bool LEAKY>
+__device__ __forceinline__ unsigned ppe_one_biased(int a, double f_pos, double f_neg, const PpePack& p) {
+    const double bd = (double)a;
+    int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, __builtin_fma(bd, f_pos, p.magic));
+    if (LEAKY) {
+        const int qn = (int)(unsigned)__builtin_bit_cast(unsigned long long, __builtin_fma(bd, f_neg, p.magic));
+        q = q > qn ? q : qn;
+    }
+    return (unsigned)med3_i32(q, p.lo, p.hi);
+}
+
+template <bool LEAKY>
 __device__ __forceinline__ unsigned ppe_pack4_biased(int a0, int a1, int a2, int a3, double f_pos, double f_neg, const PpePack& p) {
     const int a[4] = {a0, a1, a2, a3};
     unsigned w = 0;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const double bd = (double)a[r];
-        int q = (int)(unsigned)__builtin_bit_cast(unsigned long long, __builtin_fma(bd, f_pos, p.magic));
-        if (LEAKY) {
-            const int qn = (int)(unsigned)__builtin_bit_cast(unsigned long long, __builtin_fma(bd, f_neg, p.magic));
-            q = q > qn ? q : qn;
-        }
-        w |= (unsigned)med3_i32(q, p.lo, p.hi) << (8 * r);
-    }
+    for (int r = 0; r < 4; r++) w |= ppe_one_biased<LEAKY>(a[r], f_pos, f_neg, p) << (8 * r);
     return w ^ p.flip;
 }
 
@@ -1825,6 +1832,267 @@ __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict_
     }
 }
 
+// ---------------------------------------------------------------- row-patch convolution, IC a multiple of 16
+// Stem layers again (few input channels, many taps), with the input rows under a band of output rows resident in
+// LDS.  A pixel's channels are contiguous and so are the pixels of a row, hence the KX * IC bytes under one kernel
+// row of one output position are one contiguous run of the patch row: the convolution is KY matmuls over runs that
+// start SX * IC bytes apart.  K is walked kernel row by kernel row in 16-byte chunks, two per MFMA step (lanes 0-31
+// the even chunk, lanes 32-63 the odd one); a row's chunk count is rounded up to even, the spare chunk meets zero
+// weights.  Fragment addresses are a per-lane base plus a wave-uniform offset: no bounds test, padding value or
+// sign flip inside the loop (the staging applies them once per input byte).
+//
+// The weights are the A operand and the activations the B operand, so a lane ends up with one position and
+// sixteen channels: LDS row 8q + 4h + r of a 32-row tile holds channel 16h + 4q + r, and the sixteen accumulator
+// registers of lane half h are channels 16h .. 16h + 15 of its position, stored as one 16-byte word.
+// Workgroups are persistent: the weights of their 64 channels are staged once, then tiles of R output rows follow.
+struct RowsGeom {
+    int R;           // output rows per tile
+    int PH;          // patch rows: (R - 1) * SY + KY
+    int RB;          // bytes per patch row in LDS: the input pixels under one output row and one spare chunk
+    int row_chunks;  // 16-byte chunks per patch row that come from the input
+    int EPR;         // chunks per kernel row in K order, even
+    int WS;          // bytes per weight row in LDS: KY * EPR * 16 + 16
+    int ntiles;      // N * tiles per image
+    FastDiv tiles_y, ow, rc, cpp, kc, epr;  // tiles per image, OW, row_chunks, chunks per pixel, KY * EPR, EPR
+};
+
+template <bool IN_U8, bool SAME_F, int TM>
+__global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
+                                                       const int32_t* __restrict__ wt, uint8_t* __restrict__ out, ConvGeom g,
+                                                       RowsGeom rg, int pad_byte, GemmPpe ppe) {
+    constexpr int BN = 64, NW = 8, NT = 64 * NW, TN = 2, BP = 32 * TM;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint8_t* const wlds = smem;                                          // [64][WS], rows in tile order
+    ChanPrep* const sprep = reinterpret_cast<ChanPrep*>(smem + BN * rg.WS);  // [64], by channel
+    int* const sbias = reinterpret_cast<int*>(sprep + BN);               // [64] biases, [64] row sums, one flag
+    int* const csum = sbias + BN;
+    int* const sflag = csum + BN;
+    uint8_t* const patch = reinterpret_cast<uint8_t*>(sflag + 4);        // [PH][RB]
+
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int H = (int)g.H, W = (int)g.W, IC = (int)g.IC, OC = (int)g.OC, OW = (int)g.OW, OH = (int)g.OH;
+    const int oc0 = blockIdx.y * BN;
+    const int Ktot = g.KY * g.KX * IC, kc = g.KY * rg.EPR, row_in = g.KX * (IC / 16);
+    const int S = kc / 2;  // MFMA steps
+
+    // ---- weights -> LDS, once
+    for (int q = tid; q < BN * kc; q += NT) {
+        const int n = fdiv(q, rg.kc), c = q - n * kc;
+        const int ky = fdiv(c, rg.epr), e = c - ky * rg.EPR;
+        const int oc = oc0 + n < OC ? oc0 + n : OC - 1;  // channels past the end repeat the last one
+        i32x4 v = i32x4{0, 0, 0, 0};
+        if (e < row_in) v = *reinterpret_cast<const i32x4*>(w + (int64_t)oc * Ktot + (ky * row_in + e) * 16);
+        const int lrow = (n & 32) + 8 * ((n >> 2) & 3) + 4 * ((n >> 4) & 1) + (n & 3);
+        *reinterpret_cast<i32x4*>(wlds + lrow * rg.WS + c * 16) = v;
+    }
+    __syncthreads();
+    if (tid < 256) {  // the sums of the weight rows, for the zero-point term
+        const int n = tid >> 2, part = tid & 3;
+        const int lrow = (n & 32) + 8 * ((n >> 2) & 3) + 4 * ((n >> 4) & 1) + (n & 3);
+        int sum = 0;
+        if (ppe.corr != 0)
+            for (int c = part; c < kc; c += 4) {
+                const i32x4 q = *reinterpret_cast<const i32x4*>(wlds + lrow * rg.WS + c * 16);
+#pragma unroll
+                for (int j = 0; j < 4; j++) sum = __builtin_amdgcn_sdot4(q[j], 0x01010101, sum, false);
+            }
+        sum += (int)dpp_u32<0xB1>((unsigned)sum);
+        sum += (int)dpp_u32<0x4E>((unsigned)sum);
+        if (part == 0) csum[n] = sum;
+    }
+    __syncthreads();
+    const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
+    if (tid < BN) {
+        const int n = oc0 + tid < OC ? oc0 + tid : OC - 1;
+        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+                                       (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * csum[tid])), ppe.prelu_mult, ppe.prelu_shift);
+        sprep[tid] = c;
+        sbias[tid] = c.bias;
+        // the short PPE serves slopes in [0, 1] (ReLU, LeakyReLU), an even zero-point offset and scales up to 1/2
+        const bool slope_ok = SAME_F || (ppe.prelu_mult >= 0 && (ppe.prelu_shift >= 31 || ppe.prelu_mult <= (1 << ppe.prelu_shift)));
+        const bool clip = c.bmax_pos != 0x7fffffff || c.bmax_neg != 0x7fffffff;
+        const bool general = __builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0 || !slope_ok;
+        if (tid == 0) sflag[0] = general ? 1 : 0;
+    }
+    // (the barrier after the first patch makes these visible)
+
+    const int pad32 = (pad_byte & 0xff) * 0x01010101;
+    const int total_chunks = rg.PH * rg.row_chunks;
+    const bool vec_ok = (OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    const uint8_t* const wl = wlds + (lane & 31) * rg.WS + half * 16;
+    const int q16 = oc0 + half * 16;  // first of the 16 channels this lane stores in channel tile 0
+
+    for (int tile = blockIdx.x; tile < rg.ntiles; tile += gridDim.x) {
+        const int img = fdiv(tile, rg.tiles_y);
+        const int oy0 = (tile - img * (int)rg.tiles_y.d) * rg.R;
+        // ---- input rows -> LDS: patch row py is input row iy0 + py from pixel -PL on; padding and the sign flip here
+        {
+            constexpr int UP = 4;
+            const int iy0 = oy0 * g.SY - g.PT;
+            const int8_t* corner = in + (((int64_t)img * H + iy0) * W - g.PL) * IC;  // (may lie outside the tensor)
+            const int safe_row = iy0 < 0 ? 0 : (iy0 < H ? iy0 : H - 1);
+            const int safe_off = ((safe_row - iy0) * W + g.PL) * IC;
+            for (int q0 = 0; q0 < total_chunks; q0 += NT * UP) {
+                i32x4 qv[UP];
+                int dst[UP];
+                bool pin[UP];
+#pragma unroll
+                for (int u = 0; u < UP; u++) {
+                    const int q = q0 + u * NT + tid;
+                    const bool ok = q < total_chunks;
+                    const int qq = ok ? q : 0;
+                    const int py = fdiv(qq, rg.rc), qi = qq - py * rg.row_chunks;
+                    const int px = fdiv(qi, rg.cpp);
+                    const int iy = iy0 + py;
+                    const bool inside = ok && (unsigned)iy < (unsigned)H && (unsigned)(px - g.PL) < (unsigned)W;
+                    qv[u] = *reinterpret_cast<const i32x4*>(corner + (inside ? py * (W * IC) + qi * 16 : safe_off));
+                    pin[u] = inside;
+                    dst[u] = ok ? py * rg.RB + qi * 16 : -1;
+                }
+#pragma unroll
+                for (int u = 0; u < UP; u++)
+                    if (dst[u] >= 0) {
+                        i32x4 v = pin[u] ? qv[u] : i32x4{pad32, pad32, pad32, pad32};
+                        if (IN_U8) v ^= (int32_t)0x80808080;
+                        *reinterpret_cast<i32x4*>(patch + dst[u]) = v;
+                    }
+            }
+        }
+        __syncthreads();
+        const bool general = sflag[0] != 0;
+
+        const int rows_here = OH - oy0 < rg.R ? OH - oy0 : rg.R;
+        const int valid = rows_here * OW;
+        const int nblk = (valid + BP - 1) / BP;
+        const int64_t pos0 = ((int64_t)img * OH + oy0) * OW;
+        const int32_t* rt = ppe.rowterm ? ppe.rowterm + pos0 : nullptr;
+        uint8_t* const out0 = out + pos0 * OC;
+
+        auto one_block = [&](int b, auto general_c) {
+            constexpr bool GENERAL = decltype(general_c)::value;
+            const uint8_t* pl[TM];
+            int pc[TM];
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                const int p = b * BP + i * 32 + (lane & 31);
+                pc[i] = p < valid ? p : 0;
+                const int r = fdiv(pc[i], rg.ow), c = pc[i] - r * OW;
+                pl[i] = patch + r * g.SY * rg.RB + c * g.SX * IC + half * 16;
+            }
+            i32x16 acc[TM][TN];  // the short PPE's accumulators start from the bias
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    i32x4 b4 = i32x4{0, 0, 0, 0};
+                    if (!GENERAL) b4 = *reinterpret_cast<const i32x4*>(sbias + 32 * j + 16 * half + 4 * q);
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) acc[i][j][4 * q + r] = b4[r];
+                }
+
+            // fragments of step s + 1 are read before the MFMAs of step s
+            int ls = 0, lt = 0, lrow = 0;  // the next step to read, as (step, step within the kernel row, row offset)
+            i32x4 fa[2][TN], fb[2][TM];
+            auto read = [&](auto buf_c) {
+                constexpr int buf = decltype(buf_c)::value;
+                const int woff = ls * 32, poff = lrow + lt * 32;
+#pragma unroll
+                for (int j = 0; j < TN; j++) fa[buf][j] = *reinterpret_cast<const i32x4*>(wl + j * 32 * rg.WS + woff);
+#pragma unroll
+                for (int i = 0; i < TM; i++) fb[buf][i] = *reinterpret_cast<const i32x4*>(pl[i] + poff);
+                if (ls + 1 < S) {  // (past the end the last step is read again)
+                    ls++;
+                    lt++;
+                    if (lt * 2 == rg.EPR) {
+                        lt = 0;
+                        lrow += rg.RB;
+                    }
+                }
+            };
+            auto multiply = [&](auto buf_c) {
+                constexpr int buf = decltype(buf_c)::value;
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][j], fb[buf][i], acc[i][j], 0, 0, 0);
+            };
+            read(std::integral_constant<int, 0>{});
+            for (int s = 0; s < S; s += 2) {
+                read(std::integral_constant<int, 1>{});
+                multiply(std::integral_constant<int, 0>{});
+                if (s + 1 < S) {
+                    read(std::integral_constant<int, 0>{});
+                    multiply(std::integral_constant<int, 1>{});
+                }
+            }
+
+            if (rt) {
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    const int v = rt[pc[i]];
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) acc[i][j][r] += v;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                i32x4 o[TM];
+#pragma unroll
+                for (int i = 0; i < TM; i++) o[i] = i32x4{0, 0, 0, 0};
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const ChanPrep* cpp = sprep + 32 * j + 16 * half + r;
+                    if constexpr (GENERAL) {
+                        ChanPrep c = *cpp;  // the form ppe_one takes: sign flip in the bias, factors swapped for a negative multiplier
+                        c.bias = (int)((unsigned)c.bias + 0x80000000u);
+                        if (c.sgn) {
+                            const double f = c.f_pos;
+                            c.f_pos = c.f_neg;
+                            c.f_neg = f;
+                            const int bm = c.bmax_pos;
+                            c.bmax_pos = c.bmax_neg;
+                            c.bmax_neg = bm;
+                        }
+#pragma unroll
+                        for (int i = 0; i < TM; i++) o[i][r >> 2] |= (int)(ppe_one<SAME_F, true>(acc[i][j][r], c, pk) << (8 * (r & 3)));
+                    } else {
+                        const double f_pos = cpp->f_pos, f_neg = SAME_F ? 0.0 : cpp->f_neg;
+#pragma unroll
+                        for (int i = 0; i < TM; i++)
+                            o[i][r >> 2] |= (int)(ppe_one_biased<!SAME_F>(acc[i][j][r], f_pos, f_neg, pk) << (8 * (r & 3)));
+                    }
+                }
+                const int qc = q16 + 32 * j;
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    const int pi = b * BP + i * 32 + (lane & 31);
+                    if (pi >= valid || qc >= OC) continue;
+                    o[i] ^= (int)pk.flip;
+                    uint8_t* dst = out0 + ((int64_t)pi * OC + qc);
+                    if (vec_ok && qc + 16 <= OC) {
+                        __builtin_nontemporal_store(o[i], reinterpret_cast<i32x4*>(dst));
+                    } else {
+                        for (int e = 0; e < 16 && qc + e < OC; e++) dst[e] = (uint8_t)(o[i][e >> 2] >> (8 * (e & 3)));
+                    }
+                }
+            }
+        };
+        if (general) {
+            for (int b = wave; b < nblk; b += NW) one_block(b, std::true_type{});
+        } else {
+            for (int b = wave; b < nblk; b += NW) one_block(b, std::false_type{});
+        }
+        __syncthreads();  // the next tile's rows replace this patch
+    }
+}
+
 // Kernels that may ask for more than 64 KiB of dynamic LDS are given the largest size any launch of them uses,
 // once per (device, kernel): the attribute is then never changed again, so concurrent launches that want
 // different sizes cannot undo each other's setting.
@@ -2502,6 +2770,98 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         VPX_HIP_CHECK(hipGetLastError());
         *kernel_name = "nce_conv_mfma";
         return VPX_RESULT_SUCCESS;
+    }
+
+    // Channel counts that are a multiple of 16 but not of 32 (stem layers): the row-patch kernel where a band of input
+    // rows and the weights fit LDS together, else the gather kernel below.
+    if (allow_lds && mfma_ok && aligned && !out_f16 && g.IC % 16 == 0 && g.IC % 32 != 0 && g.H * g.W * g.IC < (1ll << 31) &&
+        g.N * g.OH < (1ll << 30) && g.OC < (1 << 24) && g.KY * g.KX * g.IC < (1 << 16)) {
+        RowsGeom rg{};
+        const int cpt = (int)g.IC / 16;
+        rg.EPR = (g.KX * cpt + 1) / 2 * 2;
+        rg.WS = g.KY * rg.EPR * 16 + 16;
+        const int64_t PW = (g.OW - 1) * g.SX + g.KX;
+        const int64_t RB = PW * g.IC + 16;
+        const size_t fixed = 64 * (size_t)rg.WS + 64 * sizeof(ChanPrep) + 2 * 64 * sizeof(int) + 16;
+        auto need = [&](int64_t R) { return fixed + (size_t)((R - 1) * g.SY + g.KY) * (size_t)RB; };
+        int cus = 0;
+        int rc = device_compute_units(&cus);
+        if (rc) return rc;
+        const int64_t ocb = (g.OC + 63) / 64;
+        const int64_t slots = cus / ocb > 0 ? cus / ocb : 1;  // workgroups per 64-channel block
+        // Tile height and positions per wave block: the cheapest of all that fit, counted in MFMA time (32 clocks
+        // each) plus the staging of the rows at about 64 bytes per clock; a workgroup's eight waves take a block each.
+        const int S = g.KY * rg.EPR / 2;
+        int best_r = 0, best_tm = 0;
+        double best = 0;
+        for (int64_t R = 1; R <= g.OH && need(R) <= kMaxDynLds; R++) {
+            const int64_t ntiles = g.N * ((g.OH + R - 1) / R);
+            const int64_t per_wg = (ntiles + slots - 1) / slots;
+            for (int tm = 2; tm <= 4; tm += 2) {
+                const int64_t blocks = (R * g.OW + 32 * tm - 1) / (32 * tm);
+                const double cost = (double)per_wg * ((double)((blocks + 7) / 8) * tm * (2.0 * S * 32 + 800) * 2 +
+                                                      (double)((R - 1) * g.SY + g.KY) * (double)RB / 64 + 1500);
+                if (best_tm == 0 || cost < best) {
+                    best = cost;
+                    best_r = (int)R;
+                    best_tm = tm;
+                }
+            }
+        }
+        if (const int v = knobs.conv_rows.load()) {
+            if (v >= 1 && v <= g.OH && need(v) <= kMaxDynLds) best_r = v;
+        }
+        if (best_tm != 0 && RB < (1 << 20)) {
+            const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
+            rc = rebias_weights();
+            if (rc) return rc;
+            const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
+            int lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin, hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
+            if (lo > tmax) lo = tmax;
+            if (hi < tmin) hi = tmin;
+            if (lo > hi) lo = hi;
+            auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
+            const int tiles_y = (int)((g.OH + best_r - 1) / best_r);
+            rg.R = best_r;
+            rg.PH = (best_r - 1) * g.SY + g.KY;
+            rg.RB = (int)RB;
+            rg.row_chunks = (int)(PW * cpt);
+            rg.ntiles = (int)(g.N * tiles_y);
+            rg.tiles_y = fd(tiles_y);
+            rg.ow = fd(g.OW);
+            rg.rc = fd(rg.row_chunks);
+            rg.cpp = fd(cpt);
+            rg.kc = fd(g.KY * rg.EPR);
+            rg.epr = fd(rg.EPR);
+            const size_t lds = need(best_r);
+            const int64_t per_wg = (rg.ntiles + slots - 1) / slots;
+            const dim3 grid((unsigned)((rg.ntiles + per_wg - 1) / per_wg), (unsigned)ocb);
+            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, t.zp_out, lo, hi, out_signed ? 1 : 0, rowterm};
+            const int pad_byte = t.zp_in & 0xff;
+            const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
+#define VPX_ROWS_T(U8, SAME, TMV)                                                                                     \
+    do {                                                                                                              \
+        auto kern = nce_conv_rows16<U8, SAME, TMV>;                                                                   \
+        rc = set_dyn_lds(kern, lds);                                                                                  \
+        if (rc) return rc;                                                                                            \
+        hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, \
+                           (uint8_t*)t.output, g, rg, pad_byte, gp);                                                  \
+    } while (0)
+#define VPX_ROWS(U8, SAME)                                                                                            \
+    do {                                                                                                              \
+        if (best_tm == 4) VPX_ROWS_T(U8, SAME, 4);                                                                    \
+        else VPX_ROWS_T(U8, SAME, 2);                                                                                 \
+    } while (0)
+            if (in_u8 && same_f) VPX_ROWS(true, true);
+            else if (in_u8) VPX_ROWS(true, false);
+            else if (same_f) VPX_ROWS(false, true);
+            else VPX_ROWS(false, false);
+#undef VPX_ROWS
+#undef VPX_ROWS_T
+            VPX_HIP_CHECK(hipGetLastError());
+            *kernel_name = "nce_conv_rows16";
+            return VPX_RESULT_SUCCESS;
+        }
     }
 
     if (allow_mfma && mfma_ok && aligned && g.IC % 16 == 0 && g.IC % 32 != 0 && ((Ktot + 31) / 32 * 32 + 16) * 64 <= 64 * 1024) {
