@@ -324,8 +324,8 @@ def test_weights_in_registers_conv_random_geometries(rt, orc, dev, seed):
 @pytest.mark.parametrize("seed", [11, 12, 13])
 def test_row_patch_conv_random_geometries(rt, orc, dev, seed):
     """The stem-layer kernel (channel counts that are a multiple of 16 only; input rows resident in LDS, K walked kernel row
-    by kernel row): seeded draws of channel count (one, three, five and seven chunks a pixel), kernel size up to 7x7
-    (odd chunk counts per kernel row meet the spare zero chunk), stride, padding, output channels (tails of the 64- and
+    in its natural order, two 16-byte chunks a step): seeded draws of channel count (one, three, five and seven chunks a
+    pixel), kernel size up to 7x7 (steps that straddle two kernel rows, odd chunk counts), stride, padding, output channels (tails of the 64- and
     16-channel blocks), tile height, storage types, zero points (weights too) and PPE settings on both sides of the
     short requantisation's conditions."""
     rng = np.random.default_rng(seed)
@@ -362,10 +362,12 @@ def test_row_patch_conv_random_geometries(rt, orc, dev, seed):
                                        strides=(SY, SX), pads=(pl, pr, pt, pb), out_signed=out_signed, mode=mode)
         finally:
             rt.set_tuning("VPX_CONV_ROWS", None)
-        # (the kernel wants the weights of 64 channels -- kernel rows padded to an even chunk count -- and the input rows
-        # under one output row in LDS together; layers beyond that take the gather or the plain kernel)
+        # (the kernel wants the weights of 64 channels and the input rows under one output row in LDS together; layers
+        # beyond that take the gather or the plain kernel)
         OW = (W + pl + pr - KX) // SX + 1
-        lds = 64 * (KY * ((KX * IC // 16 + 1) // 2 * 2) * 16 + 16) + 64 * 32 + 2 * 64 * 4 + 16 + KY * (((OW - 1) * SX + KX) * IC + 16)
+        steps, m = (KY * KX * IC // 16 + 1) // 2, SX * IC // 16
+        row = -(-(((OW - 1) * SX + KX) * IC // 16) // m) * m * 16
+        lds = 64 * (steps * 32 + 16) + 64 * 32 + 2 * 64 * 4 + 16 + (2 * steps + 3) // 4 * 16 + KY * row
         if lds <= 160 * 1024 - 512:
             assert name == "nce_conv_rows16", what
         assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))

@@ -1836,10 +1836,16 @@ __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict_
 // Stem layers again (few input channels, many taps), with the input rows under a band of output rows resident in
 // LDS.  A pixel's channels are contiguous and so are the pixels of a row, hence the KX * IC bytes under one kernel
 // row of one output position are one contiguous run of the patch row: the convolution is KY matmuls over runs that
-// start SX * IC bytes apart.  K is walked kernel row by kernel row in 16-byte chunks, two per MFMA step (lanes 0-31
-// the even chunk, lanes 32-63 the odd one); a row's chunk count is rounded up to even, the spare chunk meets zero
-// weights.  Fragment addresses are a per-lane base plus a wave-uniform offset: no bounds test, padding value or
-// sign flip inside the loop (the staging applies them once per input byte).
+// start SX * IC bytes apart.  K is walked in its natural order in 16-byte chunks, two per MFMA step (lanes 0-31 the
+// even chunk, lanes 32-63 the odd one, which may lie in the next kernel row; an odd chunk count ends on a chunk of
+// zero weights).  A fragment address is a per-lane base plus one of two wave-uniform offsets, by lane half, which a
+// small table in LDS holds per step: no bounds test, padding value or sign flip inside the loop (the staging applies
+// them once per input byte).
+//
+// Patch rows are stored de-interleaved.  Neighbouring output positions start m = SX * IC / 16 chunks apart, so chunk u
+// of a row sits at (u % m) * plane + u / m: the 32 lanes of a fragment read then fall on 32 consecutive chunks
+// whatever the stride (with the plain layout a stride of two puts them on every other chunk, and two lanes of each
+// LDS pass on the same banks: measured 23 against 19.5 us in the loop of a 7x7 stem).
 //
 // The weights are the A operand and the activations the B operand, so a lane ends up with one position and
 // sixteen channels: LDS row 8q + 4h + r of a 32-row tile holds channel 16h + 4q + r, and the sixteen accumulator
@@ -1848,15 +1854,17 @@ __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict_
 struct RowsGeom {
     int R;           // output rows per tile
     int PH;          // patch rows: (R - 1) * SY + KY
-    int RB;          // bytes per patch row in LDS: the input pixels under one output row and one spare chunk
-    int row_chunks;  // 16-byte chunks per patch row that come from the input
-    int EPR;         // chunks per kernel row in K order, even
-    int WS;          // bytes per weight row in LDS: KY * EPR * 16 + 16
+    int RB;          // bytes per patch row in LDS: m planes of `plane` chunks
+    int row_chunks;  // 16-byte chunks per patch row
+    int m, plane;    // chunks between neighbouring output positions; chunks per plane
+    int S;           // MFMA steps: K / 16 chunks, two a step
+    int WS;          // bytes per weight row in LDS: S * 32 + 16
     int ntiles;      // N * tiles per image
-    FastDiv tiles_y, ow, rc, cpp, kc, epr;  // tiles per image, OW, row_chunks, chunks per pixel, KY * EPR, EPR
+    FastDiv tiles_y, ow, rc, cpp, kc, fm, rin;  // tiles per image, OW, row_chunks, chunks per pixel, 2 * S, m, chunks per kernel row
 };
 
-template <bool IN_U8, bool SAME_F, int TM>
+// MULTI: some workgroup takes more than one tile.
+template <bool IN_U8, bool SAME_F, int TM, bool MULTI>
 __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                        const int32_t* __restrict__ wt, uint8_t* __restrict__ out, ConvGeom g,
                                                        RowsGeom rg, int pad_byte, GemmPpe ppe) {
@@ -1867,22 +1875,96 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
     int* const sbias = reinterpret_cast<int*>(sprep + BN);               // [64] biases, [64] row sums, one flag
     int* const csum = sbias + BN;
     int* const sflag = csum + BN;
-    uint8_t* const patch = reinterpret_cast<uint8_t*>(sflag + 4);        // [PH][RB]
+    int* const stab = sflag + 4;                                         // [S][2] fragment offsets, by step and lane half
+    uint8_t* const patch = reinterpret_cast<uint8_t*>(stab + (2 * rg.S + 3) / 4 * 4);  // [PH][RB]
 
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int H = (int)g.H, W = (int)g.W, IC = (int)g.IC, OC = (int)g.OC, OW = (int)g.OW, OH = (int)g.OH;
     const int oc0 = blockIdx.y * BN;
-    const int Ktot = g.KY * g.KX * IC, kc = g.KY * rg.EPR, row_in = g.KX * (IC / 16);
-    const int S = kc / 2;  // MFMA steps
+    const int Ktot = g.KY * g.KX * IC, row_in = g.KX * (IC / 16), nchunks = g.KY * row_in;
+    const int S = rg.S, kc = 2 * S;
 
-    // ---- weights -> LDS, once
+    // ---- input rows -> LDS: patch row py is input row iy0 + py from pixel -PL on; padding and the sign flip applied here.
+    // The first UPF chunks of every thread stay in registers from the load (issued a tile ahead) to the store.
+    constexpr int UPF = TM == 4 ? 6 : 9;  // (what the registers beside the accumulators allow)
+    const int pad32 = (pad_byte & 0xff) * 0x01010101;
+    const int total_chunks = rg.PH * rg.row_chunks;
+    i32x4 qv[UPF];
+    struct Chunk {
+        bool ok, inside;
+        int src, dst;
+    };
+    struct Origin {
+        const int8_t* corner;  // of the patch in the input; may lie outside the tensor
+        int iy0, safe_off;     // first input row; offset from the corner to a pixel that exists
+    };
+    auto origin = [&](int tile_) {
+        const int img = fdiv(tile_, rg.tiles_y);
+        const int iy0 = (tile_ - img * (int)rg.tiles_y.d) * rg.R * g.SY - g.PT;
+        const int safe_row = iy0 < 0 ? 0 : (iy0 < H ? iy0 : H - 1);
+        return Origin{in + (((int64_t)img * H + iy0) * W - g.PL) * IC, iy0, ((safe_row - iy0) * W + g.PL) * IC};
+    };
+    auto chunk = [&](const Origin& o, int q) {
+        Chunk c;
+        c.ok = q < total_chunks;
+        const int qq = c.ok ? q : 0;
+        const int py = fdiv(qq, rg.rc), qi = qq - py * rg.row_chunks;
+        const int px = fdiv(qi, rg.cpp);
+        c.inside = c.ok && (unsigned)(o.iy0 + py) < (unsigned)H && (unsigned)(px - g.PL) < (unsigned)W;
+        c.src = c.inside ? py * (W * IC) + qi * 16 : o.safe_off;
+        const int qd = fdiv(qi, rg.fm);
+        c.dst = py * rg.RB + ((qi - qd * rg.m) * rg.plane + qd) * 16;
+        return c;
+    };
+    auto put = [&](const Chunk& c, i32x4 v) {
+        if (!c.ok) return;
+        if (!c.inside) v = i32x4{pad32, pad32, pad32, pad32};
+        if (IN_U8) v ^= (int32_t)0x80808080;
+        *reinterpret_cast<i32x4*>(patch + c.dst) = v;
+    };
+    // (the chunks' places do not depend on the tile, but worked out once they would sit in registers for the whole
+    // kernel: the thread index goes through an opaque move so that they are worked out where they are used)
+    auto load_patch = [&](int tile_) {
+        const Origin o = origin(tile_);
+        int t0 = tid;
+        asm volatile("" : "+v"(t0));
+#pragma unroll
+        for (int u = 0; u < UPF; u++) qv[u] = *reinterpret_cast<const i32x4*>(o.corner + chunk(o, u * NT + t0).src);
+    };
+    auto store_patch = [&](int tile_) {
+        const Origin o = origin(tile_);
+        int t0 = tid;
+        asm volatile("" : "+v"(t0));
+#pragma unroll
+        for (int u = 0; u < UPF; u++) put(chunk(o, u * NT + t0), qv[u]);
+        for (int q0 = UPF * NT; q0 < total_chunks; q0 += 4 * NT) {  // tall patches: the rest, a round trip each
+            i32x4 rest[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) rest[u] = *reinterpret_cast<const i32x4*>(o.corner + chunk(o, q0 + u * NT + tid).src);
+#pragma unroll
+            for (int u = 0; u < 4; u++) put(chunk(o, q0 + u * NT + tid), rest[u]);
+        }
+    };
+    int wt2 = 0, wt3 = 0;  // this thread's channel of the weight table, asked for before anything else
+    if (tid < BN) {
+        const int n = oc0 + tid < OC ? oc0 + tid : OC - 1;
+        wt2 = wt[n * 4 + 2];
+        wt3 = wt[n * 4 + 3];
+    }
+    load_patch(blockIdx.x);  // (under the staging of the weights)
+
+    // ---- weights -> LDS, once; the table of fragment offsets
+    for (int c = tid; c < 2 * rg.S; c += NT) {
+        const int ky = fdiv(c, rg.rin), e = c - ky * row_in;
+        const int ed = fdiv(e, rg.fm);
+        stab[c] = c < nchunks ? ky * rg.RB + ((e - ed * rg.m) * rg.plane + ed) * 16 : 0;  // (the chunk past the end: zero weights, any bytes)
+    }
     for (int q = tid; q < BN * kc; q += NT) {
         const int n = fdiv(q, rg.kc), c = q - n * kc;
-        const int ky = fdiv(c, rg.epr), e = c - ky * rg.EPR;
         const int oc = oc0 + n < OC ? oc0 + n : OC - 1;  // channels past the end repeat the last one
         i32x4 v = i32x4{0, 0, 0, 0};
-        if (e < row_in) v = *reinterpret_cast<const i32x4*>(w + (int64_t)oc * Ktot + (ky * row_in + e) * 16);
+        if (c < nchunks) v = *reinterpret_cast<const i32x4*>(w + (int64_t)oc * Ktot + c * 16);
         const int lrow = (n & 32) + 8 * ((n >> 2) & 3) + 4 * ((n >> 4) & 1) + (n & 3);
         *reinterpret_cast<i32x4*>(wlds + lrow * rg.WS + c * 16) = v;
     }
@@ -1904,10 +1986,9 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
     __syncthreads();
     const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
     if (tid < BN) {
-        const int n = oc0 + tid < OC ? oc0 + tid : OC - 1;
-        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        const uint32_t w2 = (uint32_t)wt2;
         const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
-                                       (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * csum[tid])), ppe.prelu_mult, ppe.prelu_shift);
+                                       (int)((unsigned)wt3 + (unsigned)(ppe.corr * csum[tid])), ppe.prelu_mult, ppe.prelu_shift);
         sprep[tid] = c;
         sbias[tid] = c.bias;
         // the short PPE serves slopes in [0, 1] (ReLU, LeakyReLU), an even zero-point offset and scales up to 1/2
@@ -1918,8 +1999,15 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
     }
     // (the barrier after the first patch makes these visible)
 
-    const int pad32 = (pad_byte & 0xff) * 0x01010101;
-    const int total_chunks = rg.PH * rg.row_chunks;
+    // A slope of zero (ReLU) in the short form: the negative branch rounds to the zero point whatever the accumulator, so
+    // the larger of the two branches is the positive one held above that value -- one factor and a raised lower bound.
+    const bool relu = !SAME_F && ppe.prelu_mult == 0;
+    PpePack pk1 = pk;
+    if (relu) {
+        const int floor_q = (int)(unsigned)__builtin_bit_cast(unsigned long long, pk.magic);
+        pk1.lo = pk.lo > floor_q ? pk.lo : floor_q;
+        pk1.lo = pk1.lo < pk.hi ? pk1.lo : pk.hi;
+    }
     const bool vec_ok = (OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
     const uint8_t* const wl = wlds + (lane & 31) * rg.WS + half * 16;
     const int q16 = oc0 + half * 16;  // first of the 16 channels this lane stores in channel tile 0
@@ -1927,40 +2015,11 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
     for (int tile = blockIdx.x; tile < rg.ntiles; tile += gridDim.x) {
         const int img = fdiv(tile, rg.tiles_y);
         const int oy0 = (tile - img * (int)rg.tiles_y.d) * rg.R;
-        // ---- input rows -> LDS: patch row py is input row iy0 + py from pixel -PL on; padding and the sign flip here
-        {
-            constexpr int UP = 4;
-            const int iy0 = oy0 * g.SY - g.PT;
-            const int8_t* corner = in + (((int64_t)img * H + iy0) * W - g.PL) * IC;  // (may lie outside the tensor)
-            const int safe_row = iy0 < 0 ? 0 : (iy0 < H ? iy0 : H - 1);
-            const int safe_off = ((safe_row - iy0) * W + g.PL) * IC;
-            for (int q0 = 0; q0 < total_chunks; q0 += NT * UP) {
-                i32x4 qv[UP];
-                int dst[UP];
-                bool pin[UP];
-#pragma unroll
-                for (int u = 0; u < UP; u++) {
-                    const int q = q0 + u * NT + tid;
-                    const bool ok = q < total_chunks;
-                    const int qq = ok ? q : 0;
-                    const int py = fdiv(qq, rg.rc), qi = qq - py * rg.row_chunks;
-                    const int px = fdiv(qi, rg.cpp);
-                    const int iy = iy0 + py;
-                    const bool inside = ok && (unsigned)iy < (unsigned)H && (unsigned)(px - g.PL) < (unsigned)W;
-                    qv[u] = *reinterpret_cast<const i32x4*>(corner + (inside ? py * (W * IC) + qi * 16 : safe_off));
-                    pin[u] = inside;
-                    dst[u] = ok ? py * rg.RB + qi * 16 : -1;
-                }
-#pragma unroll
-                for (int u = 0; u < UP; u++)
-                    if (dst[u] >= 0) {
-                        i32x4 v = pin[u] ? qv[u] : i32x4{pad32, pad32, pad32, pad32};
-                        if (IN_U8) v ^= (int32_t)0x80808080;
-                        *reinterpret_cast<i32x4*>(patch + dst[u]) = v;
-                    }
-            }
-        }
+        store_patch(tile);
         __syncthreads();
+        // the next tile's rows travel while this one is computed (after the last tile: the same rows once more, so that
+        // no branch stands between these loads and their use; a launch of one tile per workgroup has none of this)
+        if (MULTI) load_patch(tile + (int)gridDim.x < rg.ntiles ? tile + (int)gridDim.x : tile);
         const bool general = sflag[0] != 0;
 
         const int rows_here = OH - oy0 < rg.R ? OH - oy0 : rg.R;
@@ -1970,8 +2029,10 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         const int32_t* rt = ppe.rowterm ? ppe.rowterm + pos0 : nullptr;
         uint8_t* const out0 = out + pos0 * OC;
 
-        auto one_block = [&](int b, auto general_c) {
-            constexpr bool GENERAL = decltype(general_c)::value;
+        auto one_block = [&](int b, auto kind_c) {
+            // PPE kinds.  0: the general form; 1: two factors, the short form (see ppe_pack4_biased); 2: one factor
+            constexpr int KIND = decltype(kind_c)::value;
+            constexpr bool GENERAL = KIND == 0;
             const uint8_t* pl[TM];
             int pc[TM];
 #pragma unroll
@@ -1979,7 +2040,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                 const int p = b * BP + i * 32 + (lane & 31);
                 pc[i] = p < valid ? p : 0;
                 const int r = fdiv(pc[i], rg.ow), c = pc[i] - r * OW;
-                pl[i] = patch + r * g.SY * rg.RB + c * g.SX * IC + half * 16;
+                pl[i] = patch + r * g.SY * rg.RB + c * 16;
             }
             i32x16 acc[TM][TN];  // the short PPE's accumulators start from the bias
 #pragma unroll
@@ -1994,24 +2055,20 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                         for (int r = 0; r < 4; r++) acc[i][j][4 * q + r] = b4[r];
                 }
 
-            // fragments of step s + 1 are read before the MFMAs of step s
-            int ls = 0, lt = 0, lrow = 0;  // the next step to read, as (step, step within the kernel row, row offset)
+            // fragments of step s + 1 are read before the MFMAs of step s, their offset in the patch a step before that
+            int ls = 0;  // the next step to read
+            const int* const tab = stab + half;
+            int poff = tab[0];
             i32x4 fa[2][TN], fb[2][TM];
             auto read = [&](auto buf_c) {
                 constexpr int buf = decltype(buf_c)::value;
-                const int woff = ls * 32, poff = lrow + lt * 32;
+                const int woff = ls * 32;
 #pragma unroll
                 for (int j = 0; j < TN; j++) fa[buf][j] = *reinterpret_cast<const i32x4*>(wl + j * 32 * rg.WS + woff);
 #pragma unroll
                 for (int i = 0; i < TM; i++) fb[buf][i] = *reinterpret_cast<const i32x4*>(pl[i] + poff);
-                if (ls + 1 < S) {  // (past the end the last step is read again)
-                    ls++;
-                    lt++;
-                    if (lt * 2 == rg.EPR) {
-                        lt = 0;
-                        lrow += rg.RB;
-                    }
-                }
+                if (ls + 1 < S) ls++;  // (past the end the last step is read again)
+                poff = tab[2 * ls];
             };
             auto multiply = [&](auto buf_c) {
                 constexpr int buf = decltype(buf_c)::value;
@@ -2063,10 +2120,10 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
 #pragma unroll
                         for (int i = 0; i < TM; i++) o[i][r >> 2] |= (int)(ppe_one<SAME_F, true>(acc[i][j][r], c, pk) << (8 * (r & 3)));
                     } else {
-                        const double f_pos = cpp->f_pos, f_neg = SAME_F ? 0.0 : cpp->f_neg;
+                        const double f_pos = cpp->f_pos, f_neg = KIND == 2 ? 0.0 : cpp->f_neg;
 #pragma unroll
                         for (int i = 0; i < TM; i++)
-                            o[i][r >> 2] |= (int)(ppe_one_biased<!SAME_F>(acc[i][j][r], f_pos, f_neg, pk) << (8 * (r & 3)));
+                            o[i][r >> 2] |= (int)(ppe_one_biased<KIND == 1>(acc[i][j][r], f_pos, f_neg, pk1) << (8 * (r & 3)));
                     }
                 }
                 const int qc = q16 + 32 * j;
@@ -2085,9 +2142,11 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
             }
         };
         if (general) {
-            for (int b = wave; b < nblk; b += NW) one_block(b, std::true_type{});
+            for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 0>{});
+        } else if (SAME_F || relu) {
+            for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 2>{});
         } else {
-            for (int b = wave; b < nblk; b += NW) one_block(b, std::false_type{});
+            for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 1>{});
         }
         __syncthreads();  // the next tile's rows replace this patch
     }
@@ -2778,11 +2837,13 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         g.N * g.OH < (1ll << 30) && g.OC < (1 << 24) && g.KY * g.KX * g.IC < (1 << 16)) {
         RowsGeom rg{};
         const int cpt = (int)g.IC / 16;
-        rg.EPR = (g.KX * cpt + 1) / 2 * 2;
-        rg.WS = g.KY * rg.EPR * 16 + 16;
+        rg.S = (g.KY * g.KX * cpt + 1) / 2;
+        rg.WS = rg.S * 32 + 16;
         const int64_t PW = (g.OW - 1) * g.SX + g.KX;
-        const int64_t RB = PW * g.IC + 16;
-        const size_t fixed = 64 * (size_t)rg.WS + 64 * sizeof(ChanPrep) + 2 * 64 * sizeof(int) + 16;
+        rg.m = g.SX * cpt;
+        rg.plane = (int)((PW * cpt + rg.m - 1) / rg.m);
+        const int64_t RB = (int64_t)rg.m * rg.plane * 16;
+        const size_t fixed = 64 * (size_t)rg.WS + 64 * sizeof(ChanPrep) + 2 * 64 * sizeof(int) + 16 + (size_t)(2 * rg.S + 3) / 4 * 16;
         auto need = [&](int64_t R) { return fixed + (size_t)((R - 1) * g.SY + g.KY) * (size_t)RB; };
         int cus = 0;
         int rc = device_compute_units(&cus);
@@ -2791,7 +2852,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         const int64_t slots = cus / ocb > 0 ? cus / ocb : 1;  // workgroups per 64-channel block
         // Tile height and positions per wave block: the cheapest of all that fit, counted in MFMA time (32 clocks
         // each) plus the staging of the rows at about 64 bytes per clock; a workgroup's eight waves take a block each.
-        const int S = g.KY * rg.EPR / 2;
+        const int S = rg.S;
         int best_r = 0, best_tm = 0;
         double best = 0;
         for (int64_t R = 1; R <= g.OH && need(R) <= kMaxDynLds; R++) {
@@ -2831,17 +2892,18 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             rg.ow = fd(g.OW);
             rg.rc = fd(rg.row_chunks);
             rg.cpp = fd(cpt);
-            rg.kc = fd(g.KY * rg.EPR);
-            rg.epr = fd(rg.EPR);
+            rg.kc = fd(2 * rg.S);
+            rg.fm = fd(rg.m);
+            rg.rin = fd(g.KX * cpt);
             const size_t lds = need(best_r);
             const int64_t per_wg = (rg.ntiles + slots - 1) / slots;
             const dim3 grid((unsigned)((rg.ntiles + per_wg - 1) / per_wg), (unsigned)ocb);
             GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, t.zp_out, lo, hi, out_signed ? 1 : 0, rowterm};
             const int pad_byte = t.zp_in & 0xff;
             const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
-#define VPX_ROWS_T(U8, SAME, TMV)                                                                                     \
+#define VPX_ROWS_T(U8, SAME, TMV, MULTIV)                                                                             \
     do {                                                                                                              \
-        auto kern = nce_conv_rows16<U8, SAME, TMV>;                                                                   \
+        auto kern = nce_conv_rows16<U8, SAME, TMV, MULTIV>;                                                           \
         rc = set_dyn_lds(kern, lds);                                                                                  \
         if (rc) return rc;                                                                                            \
         hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, \
@@ -2849,8 +2911,10 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     } while (0)
 #define VPX_ROWS(U8, SAME)                                                                                            \
     do {                                                                                                              \
-        if (best_tm == 4) VPX_ROWS_T(U8, SAME, 4);                                                                    \
-        else VPX_ROWS_T(U8, SAME, 2);                                                                                 \
+        if (best_tm == 4 && per_wg > 1) VPX_ROWS_T(U8, SAME, 4, true);                                                \
+        else if (best_tm == 4) VPX_ROWS_T(U8, SAME, 4, false);                                                        \
+        else if (per_wg > 1) VPX_ROWS_T(U8, SAME, 2, true);                                                           \
+        else VPX_ROWS_T(U8, SAME, 2, false);                                                                          \
     } while (0)
             if (in_u8 && same_f) VPX_ROWS(true, true);
             else if (in_u8) VPX_ROWS(true, false);
