@@ -367,7 +367,8 @@ def test_row_patch_conv_random_geometries(rt, orc, dev, seed):
         OW = (W + pl + pr - KX) // SX + 1
         steps, m = (KY * KX * IC // 16 + 1) // 2, SX * IC // 16
         row = -(-(((OW - 1) * SX + KX) * IC // 16) // m) * m * 16
-        lds = 64 * (steps * 32 + 16) + 64 * 32 + 2 * 64 * 4 + 16 + (2 * steps + 3) // 4 * 16 + KY * row
+        bn = 32 if OC <= 32 else 64  # channels per workgroup
+        lds = bn * (steps * 32 + 16) + bn * 32 + 2 * bn * 4 + 16 + (2 * steps + 3) // 4 * 16 + KY * row
         if lds <= 160 * 1024 - 512:
             assert name == "nce_conv_rows16", what
         assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))

@@ -1863,12 +1863,13 @@ struct RowsGeom {
     FastDiv tiles_y, ow, rc, cpp, kc, fm, rin;  // tiles per image, OW, row_chunks, chunks per pixel, 2 * S, m, chunks per kernel row
 };
 
-// MULTI: some workgroup takes more than one tile.
-template <bool IN_U8, bool SAME_F, int TM, bool MULTI>
+// TN: channel tiles of 32 per workgroup (1 for layers of up to 32 output channels).  MULTI: some workgroup takes more
+// than one tile.
+template <bool IN_U8, int TM, int TN, bool MULTI>
 __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                        const int32_t* __restrict__ wt, uint8_t* __restrict__ out, ConvGeom g,
                                                        RowsGeom rg, int pad_byte, GemmPpe ppe) {
-    constexpr int BN = 64, NW = 8, NT = 64 * NW, TN = 2, BP = 32 * TM;
+    constexpr int BN = 32 * TN, NW = 8, NT = 64 * NW, BP = 32 * TM;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* const wlds = smem;                                          // [64][WS], rows in tile order
     ChanPrep* const sprep = reinterpret_cast<ChanPrep*>(smem + BN * rg.WS);  // [64], by channel
@@ -1969,7 +1970,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         *reinterpret_cast<i32x4*>(wlds + lrow * rg.WS + c * 16) = v;
     }
     __syncthreads();
-    if (tid < 256) {  // the sums of the weight rows, for the zero-point term
+    if (tid < 4 * BN) {  // the sums of the weight rows, for the zero-point term
         const int n = tid >> 2, part = tid & 3;
         const int lrow = (n & 32) + 8 * ((n >> 2) & 3) + 4 * ((n >> 4) & 1) + (n & 3);
         int sum = 0;
@@ -1992,7 +1993,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         sprep[tid] = c;
         sbias[tid] = c.bias;
         // the short PPE serves slopes in [0, 1] (ReLU, LeakyReLU), an even zero-point offset and scales up to 1/2
-        const bool slope_ok = SAME_F || (ppe.prelu_mult >= 0 && (ppe.prelu_shift >= 31 || ppe.prelu_mult <= (1 << ppe.prelu_shift)));
+        const bool slope_ok = (ppe.prelu_mult >= 0 && (ppe.prelu_shift >= 31 || ppe.prelu_mult <= (1 << ppe.prelu_shift)));
         const bool clip = c.bmax_pos != 0x7fffffff || c.bmax_neg != 0x7fffffff;
         const bool general = __builtin_amdgcn_ballot_w64(clip) != 0 || pk.odd != 0 || !slope_ok;
         if (tid == 0) sflag[0] = general ? 1 : 0;
@@ -2001,7 +2002,8 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
 
     // A slope of zero (ReLU) in the short form: the negative branch rounds to the zero point whatever the accumulator, so
     // the larger of the two branches is the positive one held above that value -- one factor and a raised lower bound.
-    const bool relu = !SAME_F && ppe.prelu_mult == 0;
+    const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;  // no PReLU stage
+    const bool relu = ppe.prelu_mult == 0;
     PpePack pk1 = pk;
     if (relu) {
         const int floor_q = (int)(unsigned)__builtin_bit_cast(unsigned long long, pk.magic);
@@ -2118,7 +2120,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                             c.bmax_neg = bm;
                         }
 #pragma unroll
-                        for (int i = 0; i < TM; i++) o[i][r >> 2] |= (int)(ppe_one<SAME_F, true>(acc[i][j][r], c, pk) << (8 * (r & 3)));
+                        for (int i = 0; i < TM; i++) o[i][r >> 2] |= (int)(ppe_one<false, true>(acc[i][j][r], c, pk) << (8 * (r & 3)));
                     } else {
                         const double f_pos = cpp->f_pos, f_neg = KIND == 2 ? 0.0 : cpp->f_neg;
 #pragma unroll
@@ -2143,7 +2145,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         };
         if (general) {
             for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 0>{});
-        } else if (SAME_F || relu) {
+        } else if (same_f || relu) {
             for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 2>{});
         } else {
             for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 1>{});
@@ -2843,13 +2845,14 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         rg.m = g.SX * cpt;
         rg.plane = (int)((PW * cpt + rg.m - 1) / rg.m);
         const int64_t RB = (int64_t)rg.m * rg.plane * 16;
-        const size_t fixed = 64 * (size_t)rg.WS + 64 * sizeof(ChanPrep) + 2 * 64 * sizeof(int) + 16 + (size_t)(2 * rg.S + 3) / 4 * 16;
+        const int bn = g.OC <= 32 ? 32 : 64;  // channels per workgroup
+        const size_t fixed = bn * (size_t)rg.WS + bn * sizeof(ChanPrep) + 2 * bn * sizeof(int) + 16 + (size_t)(2 * rg.S + 3) / 4 * 16;
         auto need = [&](int64_t R) { return fixed + (size_t)((R - 1) * g.SY + g.KY) * (size_t)RB; };
         int cus = 0;
         int rc = device_compute_units(&cus);
         if (rc) return rc;
-        const int64_t ocb = (g.OC + 63) / 64;
-        const int64_t slots = cus / ocb > 0 ? cus / ocb : 1;  // workgroups per 64-channel block
+        const int64_t ocb = (g.OC + bn - 1) / bn;
+        const int64_t slots = cus / ocb > 0 ? cus / ocb : 1;  // workgroups per block of channels
         // Tile height and positions per wave block: the cheapest of all that fit, counted in MFMA time (32 clocks
         // each) plus the staging of the rows at about 64 bytes per clock; a workgroup's eight waves take a block each.
         const int S = rg.S;
@@ -2860,7 +2863,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             const int64_t per_wg = (ntiles + slots - 1) / slots;
             for (int tm = 2; tm <= 4; tm += 2) {
                 const int64_t blocks = (R * g.OW + 32 * tm - 1) / (32 * tm);
-                const double cost = (double)per_wg * ((double)((blocks + 7) / 8) * tm * (2.0 * S * 32 + 800) * 2 +
+                const double cost = (double)per_wg * ((double)((blocks + 7) / 8) * tm * (bn / 32) * (S * 32.0 + 400) * 2 +
                                                       (double)((R - 1) * g.SY + g.KY) * (double)RB / 64 + 1500);
                 if (best_tm == 0 || cost < best) {
                     best = cost;
@@ -2900,26 +2903,25 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             const dim3 grid((unsigned)((rg.ntiles + per_wg - 1) / per_wg), (unsigned)ocb);
             GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, t.zp_out, lo, hi, out_signed ? 1 : 0, rowterm};
             const int pad_byte = t.zp_in & 0xff;
-            const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
-#define VPX_ROWS_T(U8, SAME, TMV, MULTIV)                                                                             \
+#define VPX_ROWS_T(U8, TNV, TMV, MULTIV)                                                                              \
     do {                                                                                                              \
-        auto kern = nce_conv_rows16<U8, SAME, TMV, MULTIV>;                                                           \
+        auto kern = nce_conv_rows16<U8, TMV, TNV, MULTIV>;                                                            \
         rc = set_dyn_lds(kern, lds);                                                                                  \
         if (rc) return rc;                                                                                            \
         hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, \
                            (uint8_t*)t.output, g, rg, pad_byte, gp);                                                  \
     } while (0)
-#define VPX_ROWS(U8, SAME)                                                                                            \
+#define VPX_ROWS(U8, TNV)                                                                                             \
     do {                                                                                                              \
-        if (best_tm == 4 && per_wg > 1) VPX_ROWS_T(U8, SAME, 4, true);                                                \
-        else if (best_tm == 4) VPX_ROWS_T(U8, SAME, 4, false);                                                        \
-        else if (per_wg > 1) VPX_ROWS_T(U8, SAME, 2, true);                                                           \
-        else VPX_ROWS_T(U8, SAME, 2, false);                                                                          \
+        if (best_tm == 4 && per_wg > 1) VPX_ROWS_T(U8, TNV, 4, true);                                                \
+        else if (best_tm == 4) VPX_ROWS_T(U8, TNV, 4, false);                                                        \
+        else if (per_wg > 1) VPX_ROWS_T(U8, TNV, 2, true);                                                           \
+        else VPX_ROWS_T(U8, TNV, 2, false);                                                                          \
     } while (0)
-            if (in_u8 && same_f) VPX_ROWS(true, true);
-            else if (in_u8) VPX_ROWS(true, false);
-            else if (same_f) VPX_ROWS(false, true);
-            else VPX_ROWS(false, false);
+            if (in_u8 && bn == 32) VPX_ROWS(true, 1);
+            else if (in_u8) VPX_ROWS(true, 2);
+            else if (bn == 32) VPX_ROWS(false, 1);
+            else VPX_ROWS(false, 2);
 #undef VPX_ROWS
 #undef VPX_ROWS_T
             VPX_HIP_CHECK(hipGetLastError());
