@@ -2000,16 +2000,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
     }
     // (the barrier after the first patch makes these visible)
 
-    // A slope of zero (ReLU) in the short form: the negative branch rounds to the zero point whatever the accumulator, so
-    // the larger of the two branches is the positive one held above that value -- one factor and a raised lower bound.
-    const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;  // no PReLU stage
-    const bool relu = ppe.prelu_mult == 0;
-    PpePack pk1 = pk;
-    if (relu) {
-        const int floor_q = (int)(unsigned)__builtin_bit_cast(unsigned long long, pk.magic);
-        pk1.lo = pk.lo > floor_q ? pk.lo : floor_q;
-        pk1.lo = pk1.lo < pk.hi ? pk1.lo : pk.hi;
-    }
+    const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;  // no PReLU stage (or a slope of zero, which the host turns into a clamp)
     const bool vec_ok = (OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
     const uint8_t* const wl = wlds + (lane & 31) * rg.WS + half * 16;
     const int q16 = oc0 + half * 16;  // first of the 16 channels this lane stores in channel tile 0
@@ -2125,7 +2116,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                         const double f_pos = cpp->f_pos, f_neg = KIND == 2 ? 0.0 : cpp->f_neg;
 #pragma unroll
                         for (int i = 0; i < TM; i++)
-                            o[i][r >> 2] |= (int)(ppe_one_biased<KIND == 1>(acc[i][j][r], f_pos, f_neg, pk1) << (8 * (r & 3)));
+                            o[i][r >> 2] |= (int)(ppe_one_biased<KIND == 1>(acc[i][j][r], f_pos, f_neg, pk) << (8 * (r & 3)));
                     }
                 }
                 const int qc = q16 + 32 * j;
@@ -2145,7 +2136,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         };
         if (general) {
             for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 0>{});
-        } else if (same_f || relu) {
+        } else if (same_f) {
             for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 2>{});
         } else {
             for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 1>{});
@@ -2382,6 +2373,16 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     }
 
     if (t.task_type == VPX_NCE_ELTWISE) return launch_nce_eltwise(t, ppe, s, kernel_name);
+
+    // A slope of zero (ReLU) is a clamp: the negative branch ends at the zero point whatever the accumulator, and rounding
+    // is monotone, so the result is that of a layer without a PReLU stage held at or above the zero point before the
+    // clamp (max, then min) -- the same layer with the lower bound raised to the zero point.  Every kernel's epilogue then
+    // runs its one-factor form: no sign test, no second product.  (Integer outputs only: an fp16 zero keeps its sign.)
+    if (!out_f16 && ppe.prelu_mult == 0) {
+        ppe.prelu_mult = 1;
+        ppe.prelu_shift = 0;
+        if (ppe.clamp_lo < t.zp_out) ppe.clamp_lo = t.zp_out;
+    }
 
     const int64_t Mtot = g.N * g.OH * g.OW;
     const int64_t Ktot = (int64_t)g.KY * g.KX * g.IC;
