@@ -36,7 +36,7 @@ MEASURED_TRAFFIC = {
     "c1_fake_quantize": 888359, "c2_softmax": 134285956, "c3_mvn": 17028413, "c4_conv": 14908721,
     "c5_matmul": 339645868, "c5_dequantize": 135341729, "c5_eltwise_add": 270522802, "c5_nce_eltwise": 135260398,
     "calib_int_mm": 532970109, "x_mvn6_layernorm": 268490358, "x_activation_hswish": 180562131,
-    "x_mvn1_three_steps": 25324896,
+    "x_mvn1_three_steps": 25324896, "x_stem_conv": 67487813,
 }
 
 
@@ -185,6 +185,24 @@ def make_c4(rt):
             2 * rows * 64 * 9 * 64
     return Workload("c4_conv", "int8 Conv 3x3 s1 p1 NHWC [32,56,56,64] u8 zp128 x [64,3,3,64] i8, PPE ReLU clamp [0,255]",
                     step, nbytes, ops, "mfma", "int8", "nce_conv_regw", cpu, (3136, 100352, "output positions"))
+
+
+def make_stem(rt):
+    """The first layer of a ResNet-50 with the image channels padded to 16: not a BASELINE config."""
+    import torch
+    N, H, IC, OC, K = 32, 224, 16, 64, 7
+    g = torch.Generator(device="cuda").manual_seed(9)
+    inp = torch.randint(0, 256, (N, H, H, IC), dtype=torch.uint8, device="cuda", generator=g)
+    w = torch.randint(-127, 128, (OC, K, K, IC), dtype=torch.int8, device="cuda", generator=g)
+    wt = _dev(rt.make_weights_table(np.full(OC, 20000), np.full(OC, 22), np.zeros(OC, np.int32), K * K * IC))
+    out = torch.empty((N, H // 2, H // 2, OC), dtype=torch.uint8, device="cuda")
+    ppe = rt.PpeInt(rt.PPE_LRELU, 0, 255, 1, 0)
+    task = _nce_task(rt, inp, w, wt, out, ppe, 128, 0, (2, 2), (3, 3, 3, 3))
+    step = _nce_step(rt, task)
+    step.keep = (inp, w, wt, out, task)
+    ops = 2 * N * (H // 2) * (H // 2) * OC * K * K * IC
+    return Workload("x_stem_conv", "int8 Conv 7x7 s2 p3 NHWC [32,224,224,16] u8 zp128 x [64,7,7,16] i8, ReLU (not a BASELINE config)",
+                    step, inp.numel() + out.numel() + w.numel() + wt.numel() * 4, ops, "mfma", "int8", "nce_conv_rows16")
 
 
 _C5_CACHE = {}
@@ -402,6 +420,7 @@ MAKERS = {
     "x_mvn6_layernorm": make_layernorm,
     "x_activation_hswish": make_activation,
     "x_mvn1_three_steps": make_mvn_steps,
+    "x_stem_conv": make_stem,
 }
 
 
@@ -573,7 +592,7 @@ NOTES = {
 
 HEADLINE = "c5_matmul"
 OTHER_CONFIGS = ["c1_fake_quantize", "c2_softmax", "c3_mvn", "c4_conv", "c5_dequantize", "c5_eltwise_add"]
-EXTRA_CONFIGS = ["c5_nce_eltwise", "x_mvn6_layernorm", "x_activation_hswish", "x_mvn1_three_steps"]
+EXTRA_CONFIGS = ["c5_nce_eltwise", "x_mvn6_layernorm", "x_activation_hswish", "x_mvn1_three_steps", "x_stem_conv"]
 
 
 def main():

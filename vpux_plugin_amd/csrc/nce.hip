@@ -2035,7 +2035,9 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                 const int r = fdiv(pc[i], rg.ow), c = pc[i] - r * OW;
                 pl[i] = patch + r * g.SY * rg.RB + c * 16;
             }
-            i32x16 acc[TM][TN];  // the short PPE's accumulators start from the bias
+            // The short PPE's accumulators start from the bias: the lane's sixteen channels of a channel tile are the C
+            // operand of the first step's MFMAs (no copies into every position block's accumulators).
+            i32x16 acc[TM][TN], start[TN];
 #pragma unroll
             for (int j = 0; j < TN; j++)
 #pragma unroll
@@ -2043,9 +2045,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                     i32x4 b4 = i32x4{0, 0, 0, 0};
                     if (!GENERAL) b4 = *reinterpret_cast<const i32x4*>(sbias + 32 * j + 16 * half + 4 * q);
 #pragma unroll
-                    for (int i = 0; i < TM; i++)
-#pragma unroll
-                        for (int r = 0; r < 4; r++) acc[i][j][4 * q + r] = b4[r];
+                    for (int r = 0; r < 4; r++) start[j][4 * q + r] = b4[r];
                 }
 
             // fragments of step s + 1 are read before the MFMAs of step s, their offset in the patch a step before that
@@ -2072,12 +2072,17 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][j], fb[buf][i], acc[i][j], 0, 0, 0);
             };
             read(std::integral_constant<int, 0>{});
-            for (int s = 0; s < S; s += 2) {
-                read(std::integral_constant<int, 1>{});
-                multiply(std::integral_constant<int, 0>{});
+            read(std::integral_constant<int, 1>{});
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[0][j], fb[0][i], start[j], 0, 0, 0);
+            for (int s = 1; s < S; s += 2) {
+                read(std::integral_constant<int, 0>{});
+                multiply(std::integral_constant<int, 1>{});
                 if (s + 1 < S) {
-                    read(std::integral_constant<int, 0>{});
-                    multiply(std::integral_constant<int, 1>{});
+                    read(std::integral_constant<int, 1>{});
+                    multiply(std::integral_constant<int, 0>{});
                 }
             }
 
@@ -2866,7 +2871,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 const int64_t blocks = (R * g.OW + 32 * tm - 1) / (32 * tm);
                 const double cost = (double)per_wg * ((double)((blocks + 7) / 8) * tm * (bn / 32) * (S * 32.0 + 400) * 2 +
                                                       (double)((R - 1) * g.SY + g.KY) * (double)RB / 64 + 1500);
-                if (best_tm == 0 || cost < best) {
+                if (best_tm == 0 || cost < best || (cost == best && (int)R == best_r)) {  // (a tie between the block sizes of one height: the larger)
                     best = cost;
                     best_r = (int)R;
                     best_tm = tm;
