@@ -144,6 +144,40 @@ def test_conv_patch_tile_heights(rt, orc, dev, rows, force, kernel):
     assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
 
 
+@pytest.mark.parametrize("ksplit", ["on", "off"])
+@pytest.mark.parametrize("geom", [
+    # 7 x 7 planes, slices of eight K steps: eight waves, eight shares of K
+    dict(N=3, H=7, W=7, IC=512, OC=128, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
+    dict(N=2, H=14, W=14, IC=256, OC=96, KY=3, KX=3, strides=(2, 2), pads=(1, 1, 1, 1)),
+    # slices of four K steps: four waves, a quarter each
+    dict(N=2, H=8, W=6, IC=128, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
+    dict(N=1, H=5, W=9, IC=384, OC=200, KY=2, KX=3, strides=(1, 1), pads=(1, 0, 0, 1)),
+    # up to 128 positions a tile: two groups of four waves
+    dict(N=2, H=14, W=14, IC=256, OC=64, KY=3, KX=3, strides=(1, 1), pads=(1, 1, 1, 1)),
+    dict(N=1, H=9, W=11, IC=768, OC=70, KY=1, KX=1, strides=(1, 1), pads=(1, 1, 0, 0)),
+])
+def test_streamed_weights_k_split(rt, orc, dev, geom, ksplit):
+    """Small planes in the streamed-weights kernel: the waves of a group split the K steps of every weight slice over a
+    64 x 64 tile and add their partial sums in LDS (the default), against the same kernel with one 32 x 32 tile per wave."""
+    g = dict(geom)
+    strides, pads = g.pop("strides"), g.pop("pads")
+    rng = np.random.default_rng(90 + g["H"] + g["IC"])
+    rt.set_tuning("VPX_STREAM_KSPLIT", None if ksplit == "on" else "off")
+    try:
+        for in_u8, zp_in, zp_w, w_u8, out_signed, mode, zp_out in ((True, 128, 0, False, False, rt.PPE_LRELU, 0), (True, 9, 131, True, True, rt.PPE_LPRELU, 3),
+                                                                   (False, -5, 0, False, False, rt.PPE_NOOP, 4), (False, 0, -7, False, True, rt.PPE_LPRELU, -2)):
+            inp, w, mults, shifts, bias = rand_case(rng, in_u8=in_u8, w_u8=w_u8, **g)
+            K = w[0].size
+            bias = (bias - np.int64(round(K * (inp.mean() - zp_in) * (w.mean() - zp_w)))).astype(np.int32)
+            kw = dict(I8 if out_signed else U8, lrelu_mult=1638, lrelu_shift=14)
+            got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, zp_out=zp_out, strides=strides,
+                                       pads=pads, out_signed=out_signed, mode=mode, force="stream")
+            assert name == "nce_conv_stream"
+            assert np.array_equal(got, want), "zp_in=%d zp_w=%d: %d mismatches" % (zp_in, zp_w, int((got != want).sum()))
+    finally:
+        rt.set_tuning("VPX_STREAM_KSPLIT", None)
+
+
 def test_naive_path_covers_odd_shapes_and_weight_zero_points(rt, orc, dev):
     rng = np.random.default_rng(60)
     inp, w, mults, shifts, bias = rand_case(rng, 2, 6, 7, 5, 9, 3, 2, in_u8=True, w_u8=True)

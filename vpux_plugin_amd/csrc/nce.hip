@@ -1473,7 +1473,12 @@ struct StreamGeom {
     int spt;       // slices per tap = IC / ksl
 };
 
-template <bool IN_U8, int TMW, bool SAME_F, int NW>
+//
+// KSPLIT (tiles of up to 64 positions per four waves -- 7 x 7 planes, halves of 14 x 14 ones): with a 32 x 32 tile per wave
+// every MFMA reads two fragments from LDS, four times what LDS delivers while the four SIMDs multiply.  Here the four
+// waves of a group each take a quarter of a slice's K steps over the whole 64 x 64 tile (four MFMAs per four fragments),
+// and their partial sums meet in LDS after the last slice; each wave then finishes one 32 x 32 tile as before.
+template <bool IN_U8, int TMW, bool SAME_F, int NW, int KSPLIT = 0>
 __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(const int8_t* __restrict__ in,
                                                                            const int8_t* __restrict__ w,
                                                                            const int32_t* __restrict__ wt,
@@ -1498,17 +1503,22 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
     // weight slice transfer: chunk q of a slice = (row q / cps, chunk q % cps), cps = KSL / 16 (4, 8 or 16)
     const int cps_shift = KSL == 64 ? 2 : (KSL == 128 ? 3 : 4);
     const int slice_chunks = BN << cps_shift;
-    auto slice_issue = [&](int sl, i32x4(&q)[UWS]) {
-        const int tap = sl / sg.spt, ic0 = (sl - tap * sg.spt) * KSL;
+    // (a thread's chunks sit at the same place of every slice: their addresses are worked out once, and a slice adds
+    // its offset tap * IC + ic0 = sl * KSL, since the slices of a weight row follow each other in K order)
+    const int8_t* wsrc[UWS];
 #pragma unroll
-        for (int u = 0; u < UWS; u++) {
-            const int qi = u * NT + tid;
-            const int qq = qi < slice_chunks ? qi : 0;
-            const int row = qq >> cps_shift, c = qq & ((1 << cps_shift) - 1);
-            int64_t oc = oc0 + row;
-            oc = oc < g.OC ? oc : g.OC - 1;
-            q[u] = *reinterpret_cast<const i32x4*>(w + oc * Ktot + (int64_t)tap * IC + ic0 + c * 16);
-        }
+    for (int u = 0; u < UWS; u++) {
+        const int qi = u * NT + tid;
+        const int qq = qi < slice_chunks ? qi : 0;
+        const int row = qq >> cps_shift, c = qq & ((1 << cps_shift) - 1);
+        int64_t oc = oc0 + row;
+        oc = oc < g.OC ? oc : g.OC - 1;
+        wsrc[u] = w + oc * Ktot + c * 16;
+    }
+    auto slice_issue = [&](int sl, i32x4(&q)[UWS]) {
+        const int off = sl * KSL;
+#pragma unroll
+        for (int u = 0; u < UWS; u++) q[u] = *reinterpret_cast<const i32x4*>(wsrc[u] + off);
     };
     auto slice_commit = [&](int buf, const i32x4(&q)[UWS]) {
 #pragma unroll
@@ -1521,10 +1531,15 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
         }
     };
 
-    // ---- patch and the first weight slice -> LDS.  Weight slices are asked for two slices ahead: the MFMAs of a
-    // slice can be much shorter than a trip to L2.
-    i32x4 wq[2][UWS];
-    slice_issue(0, wq[0]);
+    // ---- patch and the first weight slice -> LDS.  Weight slices are asked for DEPTH slices ahead and wait in
+    // registers: the MFMAs of a slice (a few hundred clocks) are much shorter than a trip to L2, and with two slices in
+    // flight a workgroup moved 32 KiB per memory latency ([32,7,7,512] -> 512 3x3: 18 slices, 17.9 us).
+    constexpr int DEPTH = 6;
+    const int slices = g.KY * g.KX * sg.spt;
+    i32x4 wq[DEPTH][UWS];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++)
+        if (d < slices) slice_issue(d, wq[d]);
     {
         constexpr int UP = NW == 8 ? 4 : 6;
         const int cpp = IC / 16;
@@ -1558,14 +1573,17 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
                 }
         }
     }
-    const int slices = g.KY * g.KX * sg.spt;
     slice_commit(0, wq[0]);
-    if (slices > 1) slice_issue(1, wq[1]);
     __syncthreads();
 
     // ---- main loop
-    const int nj = pg.nt == 2 ? wave & 1 : 0;
-    const int mi0 = pg.nt == 2 ? wave >> 1 : wave, mstep = pg.nt == 2 ? NW / 2 : NW;
+    static_assert(!KSPLIT || (TMW == 1 && (KSPLIT == 4 || KSPLIT == 8) && NW % KSPLIT == 0), "a K-split wave finishes one row block");
+    constexpr int KS = KSPLIT ? KSPLIT : 4;
+    const int grp = wave / KS, ks = wave % KS;  // KSPLIT: group of KS waves, this wave's share of K
+    const int nj = KSPLIT ? ks & 1 : (pg.nt == 2 ? wave & 1 : 0);
+    // (of eight waves that split K the first four finish a tile each; the others only contribute: a row block past the end)
+    const int mi0 = KSPLIT ? (ks < 4 ? 2 * grp + (ks >> 1) : kPatchMaxMT) : (pg.nt == 2 ? wave >> 1 : wave);
+    const int mstep = pg.nt == 2 ? NW / 2 : NW;
     const int npos = pg.R * (int)g.OW;
     const int kgroup = lane >> 5;
     int abase[TMW];
@@ -1578,6 +1596,24 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
     }
     const int brow = nj * 32 + (lane & 31);
     const int bbase = brow * WS + kgroup * 16;
+    int abase4[2], bbase4[2];  // KSPLIT: both row blocks of the group, both channel tiles
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        int p = (2 * grp + i) * 32 + (lane & 31);
+        p = p < npos ? p : 0;
+        const int r = fdiv(p, pg.ow), ox = p - r * (int)g.OW;
+        abase4[i] = (r * g.SY * pg.PW + ox * g.SX) * PS + kgroup * 16;
+        bbase4[i] = (i * 32 + (lane & 31)) * WS + kgroup * 16;
+    }
+    i32x16 acc4[2][2];
+    if (KSPLIT != 0) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc4[i][j][r] = 0;
+    }
 
     i32x16 acc[TMW];
 #pragma unroll
@@ -1587,13 +1623,39 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
 
     const int ksteps = KSL / 32;
     int ky = 0, kx = 0, sub = 0;  // position of the current slice
-    // slice sl: its registers (set sl & 1) were stored to LDS an iteration ago and take slice sl + 2 now
-    auto one_slice = [&](int sl, auto parity_c) {
-        constexpr int par = decltype(parity_c)::value;
-        const int buf = par;
+    // slice sl: its registers (set sl % DEPTH) were stored to LDS an iteration ago and take slice sl + DEPTH now
+    auto one_slice = [&](int sl, auto set_c) {
+        constexpr int set = decltype(set_c)::value;
+        const int buf = set & 1;  // (DEPTH is even)
         const bool more = sl + 1 < slices;
-        if (sl + 2 < slices) slice_issue(sl + 2, wq[par]);
+        if (sl + DEPTH < slices) slice_issue(sl + DEPTH, wq[set]);
         const uint8_t* pa0 = patch + (ky * pg.PW + kx) * PS + sub * KSL;
+        if constexpr (KSPLIT != 0) {
+            // this wave's K steps of the slice: ks and, where a slice has twice as many steps as the group has waves, ks + KS
+            // (the host asks for slices of KS or 2 KS steps)
+            const uint8_t* pw = wbuf + buf * BN * WS;
+            i32x4 fa[2][2], fb[2][2];
+            const bool two = ksteps > KS;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                if (h == 1 && !two) break;
+                const int k = ks + KS * h;
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    fa[h][i] = *reinterpret_cast<const i32x4*>(pa0 + abase4[i] + k * 32);
+                    fb[h][i] = *reinterpret_cast<const i32x4*>(pw + bbase4[i] + k * 32);
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                if (h == 1 && !two) break;
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc4[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[h][i], fb[h][j], acc4[i][j], 0, 0, 0);
+            }
+        } else {
         const uint8_t* pb = wbuf + buf * BN * WS + bbase;
         i32x4 fa[2][TMW], fb[2];
         auto read_frags = [&](int slot, int k) {
@@ -1610,7 +1672,8 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
 #pragma unroll
             for (int i = 0; i < TMW; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[1][i], fb[1], acc[i], 0, 0, 0);
         }
-        if (more) slice_commit(buf ^ 1, wq[par ^ 1]);
+        }
+        if (more) slice_commit(buf ^ 1, wq[(set + 1) % DEPTH]);
         __syncthreads();  // slice sl+1 is visible; nobody reads buffer `buf` any more
         sub++;
         if (sub == sg.spt) {
@@ -1622,9 +1685,45 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
             }
         }
     };
-    for (int sl = 0; sl < slices; sl += 2) {
+    static_assert(DEPTH == 6, "the loop below names the register sets one by one");
+    for (int sl = 0; sl < slices; sl += DEPTH) {
         one_slice(sl, std::integral_constant<int, 0>{});
         if (sl + 1 < slices) one_slice(sl + 1, std::integral_constant<int, 1>{});
+        if (sl + 2 < slices) one_slice(sl + 2, std::integral_constant<int, 2>{});
+        if (sl + 3 < slices) one_slice(sl + 3, std::integral_constant<int, 3>{});
+        if (sl + 4 < slices) one_slice(sl + 4, std::integral_constant<int, 4>{});
+        if (sl + 5 < slices) one_slice(sl + 5, std::integral_constant<int, 5>{});
+    }
+
+    // ---- KSPLIT: the partial sums of a group's waves meet in LDS (the last barrier of the loop has freed all of it);
+    // wave ks < 4 keeps tile (ks / 2, ks % 2) and adds what the others hold of it
+    if constexpr (KSPLIT != 0) {
+        uint8_t* const red = smem;  // [wave][tile][quad][lane] x 16 bytes
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            if (t == ks) continue;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const i32x16& a = acc4[t >> 1][t & 1];
+                *reinterpret_cast<i32x4*>(red + ((((wave * 4 + t) * 4 + q) * 64 + lane) << 4)) = i32x4{a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+            if (t == ks) acc[0] = acc4[t >> 1][t & 1];
+#pragma unroll
+        for (int o = 1; o < KS; o++) {
+            const int v = grp * KS + ((ks + o) % KS);
+            if (ks >= 4) break;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const i32x4 part = *reinterpret_cast<const i32x4*>(red + ((((v * 4 + ks) * 4 + q) * 64 + lane) << 4));
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[0][4 * q + r] += part[r];
+            }
+        }
+        __syncthreads();  // the output staging below overwrites the partial sums
     }
 
     // ---- epilogue (the last barrier of the loop has freed the patch)
@@ -2291,6 +2390,7 @@ struct Tuning {
     std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = regw | tile | stream: start the choice of LDS-patch kernel at this one (-1, 1, 2; 0: by size)
     std::atomic<int> conv_rows{0};          // VPX_CONV_ROWS = n: cap on the output rows per workgroup of the LDS-patch kernels
     std::atomic<int> conv_waves{0};         // VPX_CONV_WAVES = 4 | 8
+    std::atomic<int> stream_ksplit{1};      // VPX_STREAM_KSPLIT = off: the streamed-weights kernel never splits K over its waves
     std::atomic<int> mvn_fused{1};          // VPX_MVN_FUSED = off | nowait (see tuning_mvn_fused)
 };
 Tuning g_tuning;
@@ -2310,6 +2410,8 @@ bool set_knob(const char* knob, const char* value) {
         g_tuning.conv_rows = std::atoi(v) > 0 ? std::atoi(v) : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_WAVES")) {
         g_tuning.conv_waves = std::atoi(v) == 4 ? 4 : 0;
+    } else if (!std::strcmp(knob, "VPX_STREAM_KSPLIT")) {
+        g_tuning.stream_ksplit = (!std::strcmp(v, "off") || !std::strcmp(v, "0")) ? 0 : 1;
     } else if (!std::strcmp(knob, "VPX_MVN_FUSED")) {
         g_tuning.mvn_fused = !std::strcmp(v, "off") ? 0 : (!std::strcmp(v, "nowait") ? 2 : 1);
     } else {
@@ -2320,7 +2422,7 @@ bool set_knob(const char* knob, const char* value) {
 
 const Tuning& tuning() {
     std::call_once(g_tuning_once, [] {
-        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES", "VPX_MVN_FUSED"})
+        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES", "VPX_STREAM_KSPLIT", "VPX_MVN_FUSED"})
             if (const char* v = std::getenv(k)) set_knob(k, v);
     });
     return g_tuning;
@@ -2755,7 +2857,12 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     pg.cpp = fd(g.IC / 16);
                     pg.upr = fd((pg.PW * (g.IC / 16) + 63) / 64);
                     pg.ow = fd(g.OW);
-                    const size_t lds = need(pg.R);
+                    // tiles of at most 64 positions per four waves: K split over the waves of a group (slices of four or
+                    // eight K steps, both channel tiles in use)
+                    // (one tile of 64 positions: eight waves, eight shares of K, where a slice has eight K steps)
+                    const int ksplit_waves = knobs.stream_ksplit.load() && pg.nt == 2 && sg.ksl >= 128 ? (pg.MT <= 2 ? (sg.ksl == 256 ? 88 : 4) : (pg.MT <= 4 ? 8 : 0)) : 0;
+                    size_t lds = need(pg.R);
+                    if (lds < (size_t)(ksplit_waves % 80) * 16384) lds = (size_t)(ksplit_waves % 80) * 16384;  // the partial sums
                     const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
                     GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
                     const int pad_byte = t.zp_in & 0xff;
@@ -2771,27 +2878,30 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                         VPX_HIP_CHECK(hipGetLastError());
                     }
                     const int per_wave = (pg.MT + 8 / pg.nt - 1) / (8 / pg.nt);  // eight waves: at most 4 row blocks each
-#define VPX_STREAM_W(U8, TMW, SAME, NW)                                                                               \
+#define VPX_STREAM_W(U8, TMW, SAME, NW, KS)                                                                           \
     do {                                                                                                              \
-        auto kern = nce_conv_stream<U8, TMW, SAME, NW>;                                                               \
+        auto kern = nce_conv_stream<U8, TMW, SAME, NW, KS>;                                                           \
         rc = set_dyn_lds(kern, lds);                                                                                  \
         if (rc) return rc;                                                                                            \
         hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,       \
                            t.weight_table, colsum, (uint8_t*)t.output, g, pg, sg, pad_byte, gp);                      \
     } while (0)
-#define VPX_STREAM(TMW, NW)                                                                                           \
+#define VPX_STREAM(TMW, NW, KS)                                                                                       \
     do {                                                                                                              \
-        if (in_u8 && same_f) VPX_STREAM_W(true, TMW, true, NW);                                                       \
-        else if (in_u8) VPX_STREAM_W(true, TMW, false, NW);                                                           \
-        else if (same_f) VPX_STREAM_W(false, TMW, true, NW);                                                          \
-        else VPX_STREAM_W(false, TMW, false, NW);                                                                     \
+        if (in_u8 && same_f) VPX_STREAM_W(true, TMW, true, NW, KS);                                                   \
+        else if (in_u8) VPX_STREAM_W(true, TMW, false, NW, KS);                                                       \
+        else if (same_f) VPX_STREAM_W(false, TMW, true, NW, KS);                                                      \
+        else VPX_STREAM_W(false, TMW, false, NW, KS);                                                                 \
     } while (0)
                     // (a tile of one or two row blocks -- 7 x 7 planes -- would leave six of eight waves multiplying
                     // padding: four waves, one block each, a third of the LDS reads per weight slice)
-                    if (pg.MT <= 4 / pg.nt) VPX_STREAM(1, 4);
-                    else if (per_wave <= 1) VPX_STREAM(1, 8);
-                    else if (per_wave <= 2) VPX_STREAM(2, 8);
-                    else VPX_STREAM(4, 8);
+                    if (ksplit_waves == 4) VPX_STREAM(1, 4, 4);
+                    else if (ksplit_waves == 8) VPX_STREAM(1, 8, 4);
+                    else if (ksplit_waves == 88) VPX_STREAM(1, 8, 8);
+                    else if (pg.MT <= 4 / pg.nt) VPX_STREAM(1, 4, 0);
+                    else if (per_wave <= 1) VPX_STREAM(1, 8, 0);
+                    else if (per_wave <= 2) VPX_STREAM(2, 8, 0);
+                    else VPX_STREAM(4, 8, 0);
 #undef VPX_STREAM
 #undef VPX_STREAM_W
                     VPX_HIP_CHECK(hipGetLastError());
