@@ -360,7 +360,7 @@ def test_row_patch_conv_random_geometries(rt, orc, dev, seed):
     """The stem-layer kernel (channel counts that are a multiple of 16 only; input rows resident in LDS, K walked kernel row
     in its natural order, two 16-byte chunks a step): seeded draws of channel count (one, three, five and seven chunks a
     pixel), kernel size up to 7x7 (steps that straddle two kernel rows, odd chunk counts), stride, padding, output channels (tails of the 64- and
-    16-channel blocks), tile height, storage types, zero points (weights too) and PPE settings on both sides of the
+    16-channel blocks), tile height and width, storage types, zero points (weights too) and PPE settings on both sides of the
     short requantisation's conditions."""
     rng = np.random.default_rng(seed)
     for i in range(24):
@@ -382,8 +382,9 @@ def test_row_patch_conv_random_geometries(rt, orc, dev, seed):
             w_u8 = bool(rng.integers(0, 2))
             zp_w = int(rng.integers(0, 256)) if w_u8 else int(rng.integers(-128, 128))
         rows = int(rng.integers(0, 6))  # 0: the dispatcher's choice
-        what = "seed %d case %d: N=%d H=%d W=%d IC=%d OC=%d K=%dx%d S=%dx%d pads=%s in_u8=%s out_signed=%s zp_in=%d mode=%d slope=%d/2^%d shifts=%d..%d w_u8=%s zp_w=%d rows=%d" % (
-            seed, i, N, H, W, IC, OC, KY, KX, SY, SX, (pl, pr, pt, pb), in_u8, out_signed, zp_in, mode, lm, ls, shift_lo, shift_hi, w_u8, zp_w, rows)
+        cols = int(rng.choice([0, 0, 7, 20, 33]))  # output columns per tile; 0: the dispatcher's choice (the whole width where it fits)
+        what = "seed %d case %d: N=%d H=%d W=%d IC=%d OC=%d K=%dx%d S=%dx%d pads=%s in_u8=%s out_signed=%s zp_in=%d mode=%d slope=%d/2^%d shifts=%d..%d w_u8=%s zp_w=%d rows=%d cols=%d" % (
+            seed, i, N, H, W, IC, OC, KY, KX, SY, SX, (pl, pr, pt, pb), in_u8, out_signed, zp_in, mode, lm, ls, shift_lo, shift_hi, w_u8, zp_w, rows, cols)
         print(what, flush=True)
         inp, w, mults, shifts, bias = rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=in_u8, w_u8=w_u8, shift_lo=shift_lo, shift_hi=shift_hi)
         if rng.integers(0, 2):
@@ -391,11 +392,14 @@ def test_row_patch_conv_random_geometries(rt, orc, dev, seed):
         bias = (bias - np.int64(round(KY * KX * IC * (inp.mean() - zp_in) * (w.mean() - zp_w)))).astype(np.int32)
         if rows:
             rt.set_tuning("VPX_CONV_ROWS", rows)
+        if cols:
+            rt.set_tuning("VPX_CONV_COLS", cols)
         try:
             got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, zp_out=int(rng.integers(-5, 6)),
                                        strides=(SY, SX), pads=(pl, pr, pt, pb), out_signed=out_signed, mode=mode)
         finally:
             rt.set_tuning("VPX_CONV_ROWS", None)
+            rt.set_tuning("VPX_CONV_COLS", None)
         # (the kernel wants the weights of 64 channels and the input rows under one output row in LDS together; layers
         # beyond that take the gather or the plain kernel)
         OW = (W + pl + pr - KX) // SX + 1
@@ -424,6 +428,18 @@ def test_row_patch_conv_stem_layer(rt, orc, dev):
             rt.set_tuning("VPX_CONV_ROWS", None)
         assert name == "nce_conv_rows16"
         assert np.array_equal(got, want), "rows=%d: %d mismatches" % (rows, int((got != want).sum()))
+
+
+def test_row_patch_conv_wide_image(rt, orc, dev):
+    """A 7x7 stride-2 stem on a 1280-pixel-wide image: the rows under one output row do not fit LDS beside the weights, so
+    the kernel walks column tiles (ragged last tile, halo columns on both sides of every tile)."""
+    rng = np.random.default_rng(23)
+    inp, w, mults, shifts, bias = rand_case(rng, 1, 40, 1280, 16, 64, 7, 7, shift_lo=16, shift_hi=20)
+    kw = dict(U8, lrelu_mult=1638, lrelu_shift=14)
+    got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=117, zp_out=5, strides=(2, 2), pads=(3, 2, 3, 3),
+                               mode=rt.PPE_LPRELU)
+    assert name == "nce_conv_rows16"
+    assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
 
 
 @pytest.fixture(params=[("8", "256"), ("4", "256"), ("4", "128")], ids=["8w256", "4w256", "4w128"])

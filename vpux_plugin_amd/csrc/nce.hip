@@ -1949,9 +1949,10 @@ __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict_
 // The weights are the A operand and the activations the B operand, so a lane ends up with one position and
 // sixteen channels: LDS row 8q + 4h + r of a 32-row tile holds channel 16h + 4q + r, and the sixteen accumulator
 // registers of lane half h are channels 16h .. 16h + 15 of its position, stored as one 16-byte word.
-// Workgroups are persistent: the weights of their 64 channels are staged once, then tiles of R output rows follow.
+// Workgroups are persistent: the weights of their 64 channels are staged once, then tiles of R output rows x CW output
+// columns follow (the whole width where the rows under it fit LDS, else column tiles: wide images).
 struct RowsGeom {
-    int R;           // output rows per tile
+    int R, CW;       // output rows and columns per tile
     int PH;          // patch rows: (R - 1) * SY + KY
     int RB;          // bytes per patch row in LDS: m planes of `plane` chunks
     int row_chunks;  // 16-byte chunks per patch row
@@ -1959,6 +1960,7 @@ struct RowsGeom {
     int S;           // MFMA steps: K / 16 chunks, two a step
     int WS;          // bytes per weight row in LDS: S * 32 + 16
     int ntiles;      // N * tiles per image
+    FastDiv tiles_x, cw;  // column tiles per row of tiles, CW
     FastDiv tiles_y, ow, rc, cpp, kc, fm, rin;  // tiles per image, OW, row_chunks, chunks per pixel, 2 * S, m, chunks per kernel row
 };
 
@@ -1996,14 +1998,22 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         int src, dst;
     };
     struct Origin {
-        const int8_t* corner;  // of the patch in the input; may lie outside the tensor
-        int iy0, safe_off;     // first input row; offset from the corner to a pixel that exists
+        const int8_t* corner;   // of the patch in the input; may lie outside the tensor
+        int iy0, ix0, safe_off;  // first input row and column; offset from the corner to a pixel that exists
+    };
+    struct TilePos {
+        int img, oy0, ox0;
+    };
+    auto tile_pos = [&](int tile_) {  // tiles in the order (image, row of tiles, column tile)
+        const int tr = fdiv(tile_, rg.tiles_x), tx = tile_ - tr * (int)rg.tiles_x.d;
+        const int img = fdiv(tr, rg.tiles_y);
+        return TilePos{img, (tr - img * (int)rg.tiles_y.d) * rg.R, tx * rg.CW};
     };
     auto origin = [&](int tile_) {
-        const int img = fdiv(tile_, rg.tiles_y);
-        const int iy0 = (tile_ - img * (int)rg.tiles_y.d) * rg.R * g.SY - g.PT;
+        const TilePos tp = tile_pos(tile_);
+        const int iy0 = tp.oy0 * g.SY - g.PT, ix0 = tp.ox0 * g.SX - g.PL;
         const int safe_row = iy0 < 0 ? 0 : (iy0 < H ? iy0 : H - 1);
-        return Origin{in + (((int64_t)img * H + iy0) * W - g.PL) * IC, iy0, ((safe_row - iy0) * W + g.PL) * IC};
+        return Origin{in + (((int64_t)tp.img * H + iy0) * W + ix0) * IC, iy0, ix0, ((safe_row - iy0) * W - ix0) * IC};
     };
     auto chunk = [&](const Origin& o, int q) {
         Chunk c;
@@ -2011,7 +2021,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         const int qq = c.ok ? q : 0;
         const int py = fdiv(qq, rg.rc), qi = qq - py * rg.row_chunks;
         const int px = fdiv(qi, rg.cpp);
-        c.inside = c.ok && (unsigned)(o.iy0 + py) < (unsigned)H && (unsigned)(px - g.PL) < (unsigned)W;
+        c.inside = c.ok && (unsigned)(o.iy0 + py) < (unsigned)H && (unsigned)(o.ix0 + px) < (unsigned)W;
         c.src = c.inside ? py * (W * IC) + qi * 16 : o.safe_off;
         const int qd = fdiv(qi, rg.fm);
         c.dst = py * rg.RB + ((qi - qd * rg.m) * rg.plane + qd) * 16;
@@ -2105,8 +2115,8 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
     const int q16 = oc0 + half * 16;  // first of the 16 channels this lane stores in channel tile 0
 
     for (int tile = blockIdx.x; tile < rg.ntiles; tile += gridDim.x) {
-        const int img = fdiv(tile, rg.tiles_y);
-        const int oy0 = (tile - img * (int)rg.tiles_y.d) * rg.R;
+        const TilePos tp = tile_pos(tile);
+        const int img = tp.img, oy0 = tp.oy0, ox0 = tp.ox0;
         store_patch(tile);
         __syncthreads();
         // the next tile's rows travel while this one is computed (after the last tile: the same rows once more, so that
@@ -2114,10 +2124,11 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         if (MULTI) load_patch(tile + (int)gridDim.x < rg.ntiles ? tile + (int)gridDim.x : tile);
         const bool general = sflag[0] != 0;
 
+        // positions of a tile are counted over R x CW; those past the last row or column of the tensor are skipped
         const int rows_here = OH - oy0 < rg.R ? OH - oy0 : rg.R;
-        const int valid = rows_here * OW;
-        const int nblk = (valid + BP - 1) / BP;
-        const int64_t pos0 = ((int64_t)img * OH + oy0) * OW;
+        const int cols_here = OW - ox0 < rg.CW ? OW - ox0 : rg.CW;
+        const int nblk = (rows_here * rg.CW + BP - 1) / BP;
+        const int64_t pos0 = ((int64_t)img * OH + oy0) * OW + ox0;
         const int32_t* rt = ppe.rowterm ? ppe.rowterm + pos0 : nullptr;
         uint8_t* const out0 = out + pos0 * OC;
 
@@ -2126,12 +2137,15 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
             constexpr int KIND = decltype(kind_c)::value;
             constexpr bool GENERAL = KIND == 0;
             const uint8_t* pl[TM];
-            int pc[TM];
+            int pc[TM];  // the position's offset from the tile's first one in the output, -1 for none
 #pragma unroll
             for (int i = 0; i < TM; i++) {
                 const int p = b * BP + i * 32 + (lane & 31);
-                pc[i] = p < valid ? p : 0;
-                const int r = fdiv(pc[i], rg.ow), c = pc[i] - r * OW;
+                int r = fdiv(p, rg.cw), c = p - r * rg.CW;
+                const bool ok = r < rows_here && c < cols_here;
+                r = ok ? r : 0;
+                c = ok ? c : 0;
+                pc[i] = ok ? r * OW + c : -1;
                 pl[i] = patch + r * g.SY * rg.RB + c * 16;
             }
             // The short PPE's accumulators start from the bias: the lane's sixteen channels of a channel tile are the C
@@ -2188,7 +2202,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
             if (rt) {
 #pragma unroll
                 for (int i = 0; i < TM; i++) {
-                    const int v = rt[pc[i]];
+                    const int v = rt[pc[i] < 0 ? 0 : pc[i]];
 #pragma unroll
                     for (int j = 0; j < TN; j++)
 #pragma unroll
@@ -2226,10 +2240,9 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                 const int qc = q16 + 32 * j;
 #pragma unroll
                 for (int i = 0; i < TM; i++) {
-                    const int pi = b * BP + i * 32 + (lane & 31);
-                    if (pi >= valid || qc >= OC) continue;
+                    if (pc[i] < 0 || qc >= OC) continue;
                     o[i] ^= (int)pk.flip;
-                    uint8_t* dst = out0 + ((int64_t)pi * OC + qc);
+                    uint8_t* dst = out0 + ((int64_t)pc[i] * OC + qc);
                     if (vec_ok && qc + 16 <= OC) {
                         __builtin_nontemporal_store(o[i], reinterpret_cast<i32x4*>(dst));
                     } else {
@@ -2389,6 +2402,7 @@ struct Tuning {
     std::atomic<int> gemm_waves{0};         // VPX_GEMM_WAVES = 4 | 8
     std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = regw | tile | stream: start the choice of LDS-patch kernel at this one (-1, 1, 2; 0: by size)
     std::atomic<int> conv_rows{0};          // VPX_CONV_ROWS = n: cap on the output rows per workgroup of the LDS-patch kernels
+    std::atomic<int> conv_cols{0};          // VPX_CONV_COLS = n: output columns per tile of the row-patch kernel
     std::atomic<int> conv_waves{0};         // VPX_CONV_WAVES = 4 | 8
     std::atomic<int> stream_ksplit{1};      // VPX_STREAM_KSPLIT = off: the streamed-weights kernel never splits K over its waves
     std::atomic<int> mvn_fused{1};          // VPX_MVN_FUSED = off | nowait (see tuning_mvn_fused)
@@ -2408,6 +2422,8 @@ bool set_knob(const char* knob, const char* value) {
         g_tuning.conv_stream = !std::strcmp(v, "stream") ? 2 : (!std::strcmp(v, "tile") ? 1 : (!std::strcmp(v, "regw") ? -1 : 0));
     } else if (!std::strcmp(knob, "VPX_CONV_ROWS")) {
         g_tuning.conv_rows = std::atoi(v) > 0 ? std::atoi(v) : 0;
+    } else if (!std::strcmp(knob, "VPX_CONV_COLS")) {
+        g_tuning.conv_cols = std::atoi(v) > 0 ? std::atoi(v) : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_WAVES")) {
         g_tuning.conv_waves = std::atoi(v) == 4 ? 4 : 0;
     } else if (!std::strcmp(knob, "VPX_STREAM_KSPLIT")) {
@@ -2422,7 +2438,7 @@ bool set_knob(const char* knob, const char* value) {
 
 const Tuning& tuning() {
     std::call_once(g_tuning_once, [] {
-        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_WAVES", "VPX_STREAM_KSPLIT", "VPX_MVN_FUSED"})
+        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_COLS", "VPX_CONV_WAVES", "VPX_STREAM_KSPLIT", "VPX_MVN_FUSED"})
             if (const char* v = std::getenv(k)) set_knob(k, v);
     });
     return g_tuning;
@@ -2957,13 +2973,12 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         const int cpt = (int)g.IC / 16;
         rg.S = (g.KY * g.KX * cpt + 1) / 2;
         rg.WS = rg.S * 32 + 16;
-        const int64_t PW = (g.OW - 1) * g.SX + g.KX;
         rg.m = g.SX * cpt;
-        rg.plane = (int)((PW * cpt + rg.m - 1) / rg.m);
-        const int64_t RB = (int64_t)rg.m * rg.plane * 16;
+        // bytes per patch row under CW output columns: m planes of chunks
+        auto row_bytes = [&](int64_t CW) { return (((CW - 1) * g.SX + g.KX) * cpt + rg.m - 1) / rg.m * rg.m * 16; };
         const int bn = g.OC <= 32 ? 32 : 64;  // channels per workgroup
         const size_t fixed = bn * (size_t)rg.WS + bn * sizeof(ChanPrep) + 2 * bn * sizeof(int) + 16 + (size_t)(2 * rg.S + 3) / 4 * 16;
-        auto need = [&](int64_t R) { return fixed + (size_t)((R - 1) * g.SY + g.KY) * (size_t)RB; };
+        auto need = [&](int64_t R, int64_t CW) { return fixed + (size_t)((R - 1) * g.SY + g.KY) * (size_t)row_bytes(CW); };
         int cus = 0;
         int rc = device_compute_units(&cus);
         if (rc) return rc;
@@ -2973,24 +2988,35 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         // each) plus the staging of the rows at about 64 bytes per clock; a workgroup's eight waves take a block each.
         const int S = rg.S;
         int best_r = 0, best_tm = 0;
+        int64_t best_cw = 0;
         double best = 0;
-        for (int64_t R = 1; R <= g.OH && need(R) <= kMaxDynLds; R++) {
-            const int64_t ntiles = g.N * ((g.OH + R - 1) / R);
-            const int64_t per_wg = (ntiles + slots - 1) / slots;
-            for (int tm = 2; tm <= 4; tm += 2) {
-                const int64_t blocks = (R * g.OW + 32 * tm - 1) / (32 * tm);
-                const double cost = (double)per_wg * ((double)((blocks + 7) / 8) * tm * (bn / 32) * (S * 32.0 + 400) * 2 +
-                                                      (double)((R - 1) * g.SY + g.KY) * (double)RB / 64 + 1500);
-                if (best_tm == 0 || cost < best || (cost == best && (int)R == best_r)) {  // (a tie between the block sizes of one height: the larger)
-                    best = cost;
-                    best_r = (int)R;
-                    best_tm = tm;
+        // (the whole width, or the width in 2 .. 32 column tiles: the rows under a band of a wide image do not fit LDS)
+        for (int tx = 1; tx <= 32 && (tx == 1 || best_tm == 0 || g.OW / tx >= 64); tx++) {
+            const int64_t CW = (g.OW + tx - 1) / tx, RB = row_bytes(CW);
+            if (tx > 1 && (g.OW + CW - 1) / CW != tx) continue;
+            for (int64_t R = 1; R <= g.OH && need(R, CW) <= kMaxDynLds; R++) {
+                const int64_t ntiles = g.N * ((g.OH + R - 1) / R) * tx;
+                const int64_t per_wg = (ntiles + slots - 1) / slots;
+                for (int tm = 2; tm <= 4; tm += 2) {
+                    const int64_t blocks = (R * CW + 32 * tm - 1) / (32 * tm);
+                    const double cost = (double)per_wg * ((double)((blocks + 7) / 8) * tm * (bn / 32) * (S * 32.0 + 400) * 2 +
+                                                          (double)((R - 1) * g.SY + g.KY) * (double)RB / 64 + 1500);
+                    if (best_tm == 0 || cost < best || (cost == best && (int)R == best_r && CW == best_cw)) {  // (a tie between the block sizes of one tile: the larger)
+                        best = cost;
+                        best_r = (int)R;
+                        best_cw = CW;
+                        best_tm = tm;
+                    }
                 }
             }
         }
         if (const int v = knobs.conv_rows.load()) {
-            if (v >= 1 && v <= g.OH && need(v) <= kMaxDynLds) best_r = v;
+            if (best_tm != 0 && v >= 1 && v <= g.OH && need(v, best_cw) <= kMaxDynLds) best_r = v;
         }
+        if (const int v = knobs.conv_cols.load()) {
+            if (best_tm != 0 && v >= 1 && v <= g.OW && need(best_r, v) <= kMaxDynLds) best_cw = v;
+        }
+        const int64_t RB = best_tm ? row_bytes(best_cw) : 0;
         if (best_tm != 0 && RB < (1 << 20)) {
             const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
             rc = rebias_weights();
@@ -3001,20 +3027,24 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             if (hi < tmin) hi = tmin;
             if (lo > hi) lo = hi;
             auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
-            const int tiles_y = (int)((g.OH + best_r - 1) / best_r);
+            const int tiles_y = (int)((g.OH + best_r - 1) / best_r), tiles_x = (int)((g.OW + best_cw - 1) / best_cw);
             rg.R = best_r;
+            rg.CW = (int)best_cw;
             rg.PH = (best_r - 1) * g.SY + g.KY;
             rg.RB = (int)RB;
-            rg.row_chunks = (int)(PW * cpt);
-            rg.ntiles = (int)(g.N * tiles_y);
+            rg.plane = (int)(RB / 16 / rg.m);
+            rg.row_chunks = (int)(((best_cw - 1) * g.SX + g.KX) * cpt);
+            rg.ntiles = (int)(g.N * tiles_y * tiles_x);
             rg.tiles_y = fd(tiles_y);
+            rg.tiles_x = fd(tiles_x);
+            rg.cw = fd(best_cw);
             rg.ow = fd(g.OW);
             rg.rc = fd(rg.row_chunks);
             rg.cpp = fd(cpt);
             rg.kc = fd(2 * rg.S);
             rg.fm = fd(rg.m);
             rg.rin = fd(g.KX * cpt);
-            const size_t lds = need(best_r);
+            const size_t lds = need(best_r, best_cw);
             const int64_t per_wg = (rg.ntiles + slots - 1) / slots;
             const dim3 grid((unsigned)((rg.ntiles + per_wg - 1) / per_wg), (unsigned)ocb);
             GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, t.zp_out, lo, hi, out_signed ? 1 : 0, rowterm};
