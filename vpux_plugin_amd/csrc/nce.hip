@@ -3017,7 +3017,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             if (best_tm != 0 && v >= 1 && v <= g.OW && need(best_r, v) <= kMaxDynLds) best_cw = v;
         }
         const int64_t RB = best_tm ? row_bytes(best_cw) : 0;
-        if (best_tm != 0 && RB < (1 << 20)) {
+        if (best_tm != 0 && RB < (1 << 20) && g.N * ((g.OH + best_r - 1) / best_r) * ((g.OW + best_cw - 1) / best_cw) < (1ll << 30)) {
             const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
             rc = rebias_weights();
             if (rc) return rc;
