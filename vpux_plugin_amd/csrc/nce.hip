@@ -202,17 +202,34 @@ __device__ __forceinline__ int ppe_fast(int acc, const ChanPrep& c, const PpeFas
     return t < p.hi ? t : p.hi;
 }
 
+// The same narrowing from the fixed-point value held as a double (an integer v standing for v * 2^-15; any magnitude).
+// v is first rounded to the eleven significant bits of an fp16 by adding and subtracting 2^(exponent of v + 42) with
+// v's sign: the sum's last place is then 2^(exponent - 10), the addition rounds to nearest even there and the
+// subtraction is exact.  What is left converts to single precision, scales by 2^-15 and converts to fp16 without
+// further rounding (|v| < 2 is exact as it is: multiples of 2^-15 are fp16 subnormals' multiples of 2^-24), and values
+// from 65520 on become infinite as in the direct conversion -- which is also what the 32-bit saturation of the
+// fixed-point stage ends in (2^31 - 1 stands for 65535.99997), so that stage needs no step of its own here.
+__device__ __forceinline__ uint16_t f16_from_scaled(double v, float lo, float hi) {
+    const unsigned top = (unsigned)(__builtin_bit_cast(unsigned long long, v) >> 32);
+    const unsigned mtop = ((top & 0x7ff00000u) + (42u << 20)) | (top & 0x80000000u);
+    const double big = __builtin_bit_cast(double, (unsigned long long)mtop << 32);
+    const double r = (v + big) - big;
+    const float x = (float)r * 0x1p-15f;
+    float y = x < lo ? lo : x;
+    y = x > hi ? hi : y;
+    return __builtin_bit_cast(uint16_t, (_Float16)y);
+}
+
 // fp16 output, fast form.  `c` comes from ppe_prepare with shift - 15, so b * f is the value in units of 2^-15;
-// the fused multiply-add rounds the exact product once to an integer (ties to even), the subtraction that
-// follows is exact, and the saturation to 32 bits absorbs products too large for that trick.
+// the fused multiply-add rounds the exact product once to an integer (ties to even) and the subtraction that
+// follows is exact (products too large for that trick stay far above the fp16 range).
 __device__ __forceinline__ uint16_t ppe_fast_f16(int acc, const ChanPrep& c, float lo, float hi) {
     const int b = (int)((unsigned)acc + (unsigned)c.bias);
     const bool neg = (b ^ c.sgn) < 0;
     const double f = neg ? c.f_neg : c.f_pos;
     constexpr double kMagic = 6755399441055744.0;  // 1.5 * 2^52
-    double v = __builtin_fma((double)b, f, kMagic) - kMagic;
-    v = v > 2147483647.0 ? 2147483647.0 : (v < -2147483648.0 ? -2147483648.0 : v);
-    return f16_from_s1715((int)v, lo, hi);
+    const double v = __builtin_fma((double)b, f, kMagic) - kMagic;
+    return f16_from_scaled(v, lo, hi);
 }
 
 // Four results of one output channel as four bytes.  Same arithmetic as ppe_fast with the tail
