@@ -526,6 +526,8 @@ F16_NONE = {"clamp_low": -(2 ** 31), "clamp_high": 2 ** 31 - 1}
 @pytest.mark.parametrize("geom,kernel,force", [
     (dict(N=1, H=700, W=1, IC=128, OC=520, KY=1, KX=1), "nce_gemm_mfma", "tile256"),     # 256 x 256 tiles, ragged edges
     (dict(N=1, H=130, W=1, IC=64, OC=200, KY=1, KX=1), "nce_gemm_mfma", None),           # 128 x 128 tiles
+    (dict(N=1, H=300, W=1, IC=128, OC=77, KY=1, KX=1), "nce_gemm_mfma", None),           # rows of an odd length: no 16-byte stores
+    (dict(N=1, H=333, W=1, IC=192, OC=301, KY=1, KX=1), "nce_gemm_mfma", "tile256"),     # the same with both halves of a 256-row tile ragged
     (dict(N=2, H=9, W=11, IC=64, OC=70, KY=3, KX=3), "nce_conv_mfma", None),             # convolution: gather kernel
     (dict(N=1, H=10, W=12, IC=48, OC=40, KY=3, KX=3), "nce_conv_mfma16", None),
     (dict(N=2, H=6, W=7, IC=5, OC=9, KY=3, KX=2), "nce_conv_naive", None),

@@ -787,22 +787,55 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
 
     // Epilogue.  Accumulator register r of lane l is C[8*(r/4) + 4*(l/32) + r%4][l%32] of its 32x32 tile.
     if constexpr (OUT == OUT_F16) {
-        // fp16 output: 16-bit values straight from the registers, 32 adjacent columns (64 bytes) per half-wavefront
+        // fp16 output: through the staging tile like the bytes below, half of a 256-row tile at a time (128 rows x 544
+        // bytes), so that the tile leaves in whole rows of 16-byte stores (two-byte stores straight from the registers,
+        // 64 bytes of a row per half-wavefront, cost the [4096 x 4096] . [4096 x 11008] matmul 60 us).
+        constexpr int PASSES = TILE == 256 ? 2 : 1, ROWS = BM / PASSES, STR = BN * 2 + 32;
+        static_assert(ROWS * STR <= NS * STAGE, "the fp16 staging tile fits the panel buffers");
         uint16_t* out16 = reinterpret_cast<uint16_t*>(out);
-#pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const uint32_t w2 = (uint32_t)w2r[j];
-            const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu) - 15,
-                                           (int)((unsigned)w3r[j] + (unsigned)(ppe.corr * csr[j])), ppe.prelu_mult, ppe.prelu_shift);
-            const int64_t n = n0 + wn0 + j * 32 + (lane & 31);
+        if (ppe.rowterm) {  // (padded past the last row: edge tiles may read ahead)
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int64_t m = m0 + wm0 + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
-                    const int extra = ppe.rowterm ? ppe.rowterm[m] : 0;
-                    if (m < M && n < N) out16[m * N + n] = ppe_fast_f16(acc[i][j][r] + extra, c, ppe.f16_lo, ppe.f16_hi);
+                for (int g = 0; g < 4; g++) {
+                    const i32x4 v = *reinterpret_cast<const i32x4*>(ppe.rowterm + m0 + wm0 + i * 32 + 8 * g + 4 * (lane >> 5));
+#pragma unroll
+                    for (int j = 0; j < TN; j++)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) acc[i][j][g * 4 + q] += v[q];
                 }
+        }
+        const bool vec_ok = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+#pragma unroll
+        for (int pass = 0; pass < PASSES; pass++) {
+            if (wm0 / ROWS == pass) {
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const uint32_t w2 = (uint32_t)w2r[j];
+                    const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu) - 15,
+                                                   (int)((unsigned)w3r[j] + (unsigned)(ppe.corr * csr[j])), ppe.prelu_mult, ppe.prelu_shift);
+                    uint8_t* const col = smem + (wm0 - pass * ROWS + 4 * (lane >> 5)) * STR + (wn0 + j * 32 + (lane & 31)) * 2;
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++)
+                            *reinterpret_cast<uint16_t*>(col + (i * 32 + 8 * (r / 4) + (r % 4)) * STR) = ppe_fast_f16(acc[i][j][r], c, ppe.f16_lo, ppe.f16_hi);
+                }
+            }
+            __syncthreads();
+            for (int it = 0; it < ROWS * (BN / 8) / NT; it++) {
+                const int cid = tid + NT * it;
+                const int row = cid / (BN / 8), c8 = cid % (BN / 8);
+                const int64_t m = m0 + pass * ROWS + row, n = n0 + c8 * 8;
+                if (m >= M || n >= N) continue;
+                const i32x4 v = *reinterpret_cast<const i32x4*>(smem + row * STR + c8 * 16);
+                if (vec_ok && n + 8 <= N) {
+                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(out16 + m * N + n));
+                } else {
+                    for (int e = 0; e < 8 && n + e < N; e++) out16[m * N + n + e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+                }
+            }
+            if (pass + 1 < PASSES) __syncthreads();  // the other half overwrites the staging tile
         }
         return;
     }
