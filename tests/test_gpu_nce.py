@@ -528,7 +528,12 @@ F16_NONE = {"clamp_low": -(2 ** 31), "clamp_high": 2 ** 31 - 1}
     (dict(N=1, H=130, W=1, IC=64, OC=200, KY=1, KX=1), "nce_gemm_mfma", None),           # 128 x 128 tiles
     (dict(N=1, H=300, W=1, IC=128, OC=77, KY=1, KX=1), "nce_gemm_mfma", None),           # rows of an odd length: no 16-byte stores
     (dict(N=1, H=333, W=1, IC=192, OC=301, KY=1, KX=1), "nce_gemm_mfma", "tile256"),     # the same with both halves of a 256-row tile ragged
-    (dict(N=2, H=9, W=11, IC=64, OC=70, KY=3, KX=3), "nce_conv_mfma", None),             # convolution: gather kernel
+    (dict(N=2, H=9, W=11, IC=64, OC=70, KY=3, KX=3), "nce_conv_tile", None),             # convolution: input patch in LDS, 128-byte staging rows
+    (dict(N=2, H=9, W=11, IC=64, OC=70, KY=3, KX=3), "nce_conv_mfma", "gather"),         # the gather kernel
+    (dict(N=2, H=13, W=10, IC=128, OC=136, KY=3, KX=3), "nce_conv_tile", None),
+    (dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3), "nce_conv_stream", None),           # streamed weights, K split over two groups of waves
+    (dict(N=3, H=7, W=7, IC=512, OC=72, KY=3, KX=3), "nce_conv_stream", None),           # ... over eight waves
+    (dict(N=2, H=30, W=33, IC=192, OC=40, KY=3, KX=3), "nce_conv_stream", None),         # ... one tile per wave
     (dict(N=1, H=10, W=12, IC=48, OC=40, KY=3, KX=3), "nce_conv_mfma16", None),
     (dict(N=2, H=6, W=7, IC=5, OC=9, KY=3, KX=2), "nce_conv_naive", None),
     (dict(N=1, H=40, W=1, IC=64, OC=96, KY=1, KX=1), "nce_conv_naive", "naive"),
@@ -561,6 +566,42 @@ def test_f16_output_s1715_path(rt, orc, dev, geom, kernel, force, mode):
             assert vals.min() >= 0.0
         if mode == "LRELUX":
             assert vals.max() <= 6.0 and (vals == 6.0).any()
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_f16_output_conv_random_geometries(rt, orc, dev, seed):
+    """fp16 outputs of convolutions whichever kernel the layer selects (tile and streamed-weights kernels stage 128 bytes
+    a position, the gather kernels store from registers): seeded draws of shape, kernel, stride, padding, channel counts
+    (odd ones: no 16-byte stores), zero points, PPE mode and fp16 clamp."""
+    rng = np.random.default_rng(seed)
+    for i in range(24):
+        IC = int(rng.choice([16, 32, 64, 64, 128, 128, 192, 256, 512]))
+        OC = int(rng.choice([8, 24, 63, 64, 72, 100, 128, 130]))
+        KY, KX = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        SY, SX = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        pl, pr, pt, pb = [int(v) for v in rng.integers(0, 2, 4)]
+        pl, pr, pt, pb = min(pl, KX - 1), min(pr, KX - 1), min(pt, KY - 1), min(pb, KY - 1)
+        H, W, N = int(rng.integers(KY, 30)), int(rng.integers(KX, 40)), int(rng.integers(1, 4))
+        in_u8 = bool(rng.integers(0, 2))
+        zp_in = int(rng.integers(0, 256)) if in_u8 else int(rng.integers(-128, 128))
+        w_u8, zp_w = False, 0
+        if rng.integers(0, 3) == 0:
+            w_u8 = bool(rng.integers(0, 2))
+            zp_w = int(rng.integers(0, 256)) if w_u8 else int(rng.integers(-128, 128))
+        mode = ["NOOP", "LPRELU", "LRELU", "LRELUX"][int(rng.integers(0, 4))]
+        kw = dict(F16_NONE, lrelu_mult=int(rng.integers(0, 2048)), lrelu_shift=int(rng.integers(8, 16)))
+        if mode == "LRELUX":
+            kw["clamp_high"] = orc.pack_clamp_f16(0.0, 6.0)
+        what = "seed %d case %d: N=%d H=%d W=%d IC=%d OC=%d K=%dx%d S=%dx%d pads=%s in_u8=%s zp_in=%d w_u8=%s zp_w=%d mode=%s" % (
+            seed, i, N, H, W, IC, OC, KY, KX, SY, SX, (pl, pr, pt, pb), in_u8, zp_in, w_u8, zp_w, mode)
+        print(what, flush=True)
+        inp, w, mults, shifts, bias = rand_case(rng, N, H, W, IC, OC, KY, KX, in_u8=in_u8, w_u8=w_u8, shift_lo=10, shift_hi=26)
+        if rng.integers(0, 2):
+            mults = np.where(rng.random(mults.shape) < 0.5, -mults, mults)
+        bias = (bias - np.int64(round(KY * KX * IC * (inp.mean() - zp_in) * (w.mean() - zp_w)))).astype(np.int32)
+        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, strides=(SY, SX),
+                                   pads=(pl, pr, pt, pb), mode=getattr(rt, "PPE_" + mode), out_f16=True)
+        assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))
 
 
 def test_f16_output_scale_is_weight_scale_times_input_scale(rt, orc, dev):

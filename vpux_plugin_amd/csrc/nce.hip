@@ -509,6 +509,7 @@ struct GemmPpe {
     int out_signed;               // output storage is i8
     const int32_t* rowterm;       // as in PpeFast; padded past the last position, so edge tiles may read ahead
     float f16_lo, f16_hi;         // fp16 output: clamp bounds
+    int out_f16;                  // the LDS-patch tile kernels: the output is fp16 (s17.15 narrowed), not bytes
 };
 
 // Where the rows of A sit: row m at byte m * K (a matrix, or a 1x1 stride-1 layer), or, for a 1x1 layer with a stride,
@@ -1061,6 +1062,44 @@ struct PatchGeom {
 
 constexpr int kPatchMaxMT = 14;
 constexpr int kPatchOutStride = 80;  // bytes per output position in the staging tile
+constexpr int kPatchOutStrideF16 = 144;  // the same for an fp16 output
+
+// fp16 output of the tile kernels below (a wave holds row blocks mi0, mi0 + mstep, ... of 32 positions x the 32 channels
+// of tile nj; accumulator register r of lane l is position 8*(r/4) + 4*(l/32) + r%4, channel l%32): values through the
+// staging tile, 128 bytes a position, then whole runs of eight channels per store.  All threads of the workgroup call
+// this after the barrier that frees the patch.
+template <int TMW, int NT>
+__device__ __forceinline__ void patch_epilogue_f16(i32x16 (&acc)[TMW], int mi0, int mstep, int nj, int MT, const ChanPrep& c,
+                                                   const GemmPpe& ppe, const int32_t* rt, uint8_t* stage, uint16_t* out16,
+                                                   int valid, int oc0, int OC) {
+    const int tid = threadIdx.x, lane = tid & 63;
+#pragma unroll
+    for (int i = 0; i < TMW; i++) {
+        const int mi = mi0 + i * mstep;
+        if (mi >= MT) continue;
+        uint8_t* const col = stage + (mi * 32 + 4 * (lane >> 5)) * kPatchOutStrideF16 + (nj * 32 + (lane & 31)) * 2;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int row = 8 * (r / 4) + (r % 4);
+            const int extra = rt ? rt[mi * 32 + 4 * (lane >> 5) + row] : 0;
+            *reinterpret_cast<uint16_t*>(col + row * kPatchOutStrideF16) = ppe_fast_f16(acc[i][r] + extra, c, ppe.f16_lo, ppe.f16_hi);
+        }
+    }
+    __syncthreads();
+    const bool vec_ok = (OC & 7) == 0 && (reinterpret_cast<uintptr_t>(out16) & 15) == 0;
+    for (int cid = tid; cid < valid * 8; cid += NT) {
+        const int row = cid >> 3, c8 = cid & 7;
+        const int n = oc0 + c8 * 8;
+        if (n >= OC) continue;
+        const i32x4 v = *reinterpret_cast<const i32x4*>(stage + row * kPatchOutStrideF16 + c8 * 16);
+        uint16_t* dst = out16 + ((int64_t)row * OC + n);
+        if (vec_ok && n + 8 <= OC) {
+            __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
+        } else {
+            for (int e = 0; e < 8 && n + e < OC; e++) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+        }
+    }
+}
 
 // SAME_F (template parameter of the kernels below): the PPE treats both signs alike (no PReLU stage),
 // which drops the per-value sign test.
@@ -1228,6 +1267,19 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
     __syncthreads();  // all waves are done with the patch: its LDS becomes the output staging tile
 
     // ---- epilogue
+    if (ppe.out_f16) {
+        int64_t n = oc0 + brow;
+        n = n < g.OC ? n : g.OC - 1;
+        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu) - 15,
+                                       (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * (ppe.corr != 0 ? csum[brow] : 0))),
+                                       ppe.prelu_mult, ppe.prelu_shift);
+        const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
+        const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
+        patch_epilogue_f16<TMW, NT>(acc, mi0, mstep, nj, pg.MT, c, ppe, ppe.rowterm ? ppe.rowterm + pos0 : nullptr, patch,
+                                    reinterpret_cast<uint16_t*>(out) + pos0 * g.OC, rows_here * (int)g.OW, oc0, (int)g.OC);
+        return;
+    }
     {
         int64_t n = oc0 + brow;
         n = n < g.OC ? n : g.OC - 1;
@@ -1777,6 +1829,19 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
     }
 
     // ---- epilogue (the last barrier of the loop has freed the patch)
+    if (ppe.out_f16) {
+        int64_t n = oc0 + brow;
+        n = n < g.OC ? n : g.OC - 1;
+        const uint32_t w2 = (uint32_t)wt[n * 4 + 2];
+        const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu) - 15,
+                                       (int)((unsigned)wt[n * 4 + 3] + (unsigned)(ppe.corr * (colsum ? colsum[n] : 0))), ppe.prelu_mult,
+                                       ppe.prelu_shift);
+        const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
+        const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
+        patch_epilogue_f16<TMW, NT>(acc, mi0, mstep, nj, pg.MT, c, ppe, ppe.rowterm ? ppe.rowterm + pos0 : nullptr, patch,
+                                    reinterpret_cast<uint16_t*>(out) + pos0 * g.OC, rows_here * (int)g.OW, oc0, (int)g.OC);
+        return;
+    }
     {
         int64_t n = oc0 + brow;
         n = n < g.OC ? n : g.OC - 1;
@@ -2731,7 +2796,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
 
         // Preferred: input patch in LDS, one launch.  R = output rows per workgroup.
         // (an fp16 output takes the gather kernel below: the tile kernels' epilogues stage bytes)
-        if (allow_lds && !out_f16 && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20) &&
+        if (allow_lds && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20) &&
             g.IC < (1 << 14) && g.W * g.SX < (1 << 14) && g.N * g.OH * g.OW < (1ll << 31)) {
             // IC of 64 or 128: the one-tile-per-workgroup kernel with padded LDS rows (a tap's fragments of more
             // channels do not fit the registers twice)
@@ -2746,7 +2811,9 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             // microsecond per workgroup, which pays from about 50 000 output positions on ([32,56,56,64] -> 64: 9.1 us
             // against 9.5 us; [4,224,224,64] -> 64: 13.9 against 29.2; [32,28,28,64] -> 64: 7.0 against 6.0; the same input
             // at stride 2: 7.5 against 7.1).
-            if (g.IC == 64 && g.KY == 3 && g.KX == 3 && (first < 0 || (first == 0 && g.N * g.OH * g.OW >= 50000))) {
+            const size_t out_stride = out_f16 ? kPatchOutStrideF16 : kPatchOutStride;  // staging bytes per position
+            // (the weights-in-registers kernel stores bytes straight from its registers: integer outputs only)
+            if (!out_f16 && g.IC == 64 && g.KY == 3 && g.KX == 3 && (first < 0 || (first == 0 && g.N * g.OH * g.OW >= 50000))) {
                 PatchGeom pg{};
                 const int64_t PS = g.IC + 16, WS = Ktot + 16;
                 auto need = [&](int R) {
@@ -2781,7 +2848,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     pg.ow = fd(g.OW);
                     const size_t lds = need(pg.R);
                     const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
-                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
+                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi, out_f16 ? 1 : 0};
                     const int pad_byte = t.zp_in & 0xff;
                     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
 #define VPX_REGW(U8, SAME)                                                                                            \
@@ -2807,7 +2874,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 const int64_t PS = g.IC + 16, WS = Ktot + 16;
                 auto need = [&](int R) {
                     const size_t patch = (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)PS;
-                    const size_t stage = (size_t)((R * g.OW + 31) / 32) * 32 * kPatchOutStride;
+                    const size_t stage = (size_t)((R * g.OW + 31) / 32) * 32 * out_stride;
                     return 64 * (size_t)WS + (patch > stage ? patch : stage);
                 };
                 int R = (int)(32 * kPatchMaxMT / g.OW);
@@ -2840,7 +2907,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     pg.ow = fd(g.OW);
                     const size_t lds = need(pg.R);
                     const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
-                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
+                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi, out_f16 ? 1 : 0};
                     const int pad_byte = t.zp_in & 0xff;
                     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
                     const int nw = knobs.conv_waves.load() == 4 ? 4 : 8;
@@ -2892,7 +2959,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 const int64_t PS = g.IC + 16;
                 auto need = [&](int R) {
                     const size_t patch = (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)PS;
-                    const size_t stage = (size_t)((R * g.OW + 31) / 32) * 32 * kPatchOutStride;
+                    const size_t stage = (size_t)((R * g.OW + 31) / 32) * 32 * out_stride;
                     return 2 * 64 * (size_t)(sg.ksl + 16) + (patch > stage ? patch : stage);
                 };
                 int R = (int)(32 * kPatchMaxMT / g.OW);
@@ -2930,7 +2997,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                     size_t lds = need(pg.R);
                     if (lds < (size_t)(ksplit_waves % 80) * 16384) lds = (size_t)(ksplit_waves % 80) * 16384;  // the partial sums
                     const dim3 grid((unsigned)(g.N * tiles_y), (unsigned)ocb);
-                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm};
+                    GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi, out_f16 ? 1 : 0};
                     const int pad_byte = t.zp_in & 0xff;
                     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
                     int32_t* colsum = nullptr;
