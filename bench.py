@@ -36,7 +36,7 @@ MEASURED_TRAFFIC = {
     "c1_fake_quantize": 888359, "c2_softmax": 134285956, "c3_mvn": 17028413, "c4_conv": 14908721,
     "c5_matmul": 339645868, "c5_dequantize": 135341729, "c5_eltwise_add": 270522802, "c5_nce_eltwise": 135260398,
     "calib_int_mm": 532970109, "x_mvn6_layernorm": 268490358, "x_activation_hswish": 180562131,
-    "x_mvn1_three_steps": 25324896, "x_stem_conv": 67487813,
+    "x_mvn1_three_steps": 25324896, "x_stem_conv": 67487813, "x_small_plane_conv": 20929448,
 }
 
 
@@ -203,6 +203,24 @@ def make_stem(rt):
     ops = 2 * N * (H // 2) * (H // 2) * OC * K * K * IC
     return Workload("x_stem_conv", "int8 Conv 7x7 s2 p3 NHWC [32,224,224,16] u8 zp128 x [64,7,7,16] i8, ReLU (not a BASELINE config)",
                     step, inp.numel() + out.numel() + w.numel() + wt.numel() * 4, ops, "mfma", "int8", "nce_conv_rows16")
+
+
+def make_small_plane_conv(rt):
+    """A late ResNet-50 layer, 3x3 over 7x7 planes of 512 channels: not a BASELINE config."""
+    import torch
+    N, H, IC, OC, K = 32, 7, 512, 512, 3
+    g = torch.Generator(device="cuda").manual_seed(10)
+    inp = torch.randint(0, 256, (N, H, H, IC), dtype=torch.uint8, device="cuda", generator=g)
+    w = torch.randint(-127, 128, (OC, K, K, IC), dtype=torch.int8, device="cuda", generator=g)
+    wt = _dev(rt.make_weights_table(np.full(OC, 20000), np.full(OC, 24), np.zeros(OC, np.int32), K * K * IC))
+    out = torch.empty((N, H, H, OC), dtype=torch.uint8, device="cuda")
+    ppe = rt.PpeInt(rt.PPE_LRELU, 0, 255, 1, 0)
+    task = _nce_task(rt, inp, w, wt, out, ppe, 128, 0, (1, 1), (1, 1, 1, 1))
+    step = _nce_step(rt, task)
+    step.keep = (inp, w, wt, out, task)
+    ops = 2 * N * H * H * OC * K * K * IC
+    return Workload("x_small_plane_conv", "int8 Conv 3x3 s1 p1 NHWC [32,7,7,512] u8 zp128 x [512,3,3,512] i8, ReLU (not a BASELINE config)",
+                    step, inp.numel() + out.numel() + w.numel() + wt.numel() * 4, ops, "mfma", "int8", "nce_conv_stream")
 
 
 _C5_CACHE = {}
@@ -421,6 +439,7 @@ MAKERS = {
     "x_activation_hswish": make_activation,
     "x_mvn1_three_steps": make_mvn_steps,
     "x_stem_conv": make_stem,
+    "x_small_plane_conv": make_small_plane_conv,
 }
 
 
@@ -592,7 +611,7 @@ NOTES = {
 
 HEADLINE = "c5_matmul"
 OTHER_CONFIGS = ["c1_fake_quantize", "c2_softmax", "c3_mvn", "c4_conv", "c5_dequantize", "c5_eltwise_add"]
-EXTRA_CONFIGS = ["c5_nce_eltwise", "x_mvn6_layernorm", "x_activation_hswish", "x_mvn1_three_steps", "x_stem_conv"]
+EXTRA_CONFIGS = ["c5_nce_eltwise", "x_mvn6_layernorm", "x_activation_hswish", "x_mvn1_three_steps", "x_stem_conv", "x_small_plane_conv"]
 
 
 def main():
