@@ -133,7 +133,7 @@ VPX_API const char* vpx_sw_kernel_name(uint32_t i);
  * t *= prelu_mult and shift += prelu_shift; r = round_half_even(t / 2^shift) + zp_out;
  * clamp to [clamp_low, clamp_high]; saturate to the output type.
  *
- * output_type VPX_NN_FP16 (CONV tasks; "INT32 s17.15 fixed-point convert to FP16",
+ * output_type VPX_NN_FP16 (CONV and ELTWISE tasks; "INT32 s17.15 fixed-point convert to FP16",
  * src/vpux_compiler/src/dialect/VPUMI37XX/ops/external/runtime_dpu_parser_imports.cpp.inc:546-574): the same
  * pipeline with the round stage keeping 15 fractional bits, fx = round_half_even(t / 2^(shift - 15)) saturated to
  * 32 bits; the output is fx * 2^-15 narrowed to fp16 with one round-to-nearest-even (infinity from 65520 up).
@@ -181,7 +181,7 @@ typedef struct vpx_nce_task_t {
     void* output;
     int32_t input_type;   /* VPX_NN_U8 or VPX_NN_I8 */
     int32_t weights_type; /* VPX_NN_U8 or VPX_NN_I8 */
-    int32_t output_type;  /* VPX_NN_U8, VPX_NN_I8, or VPX_NN_FP16 (CONV tasks) */
+    int32_t output_type;  /* VPX_NN_U8, VPX_NN_I8, or VPX_NN_FP16 */
     int64_t N, H, W, IC;  /* input shape */
     int64_t OC;
     int32_t kernel_size[2];    /* KY, KX */

@@ -402,11 +402,17 @@ def nce_conv(inp, w, wt, p, zp_in=0, zp_w=0, strides=(1, 1), pads=(0, 0, 0, 0), 
     return (out, acc) if want_acc else out
 
 
-def nce_eltwise(a, b, p, zp_a, zp_b, mult_a, mult_b, out_mult, out_shift, subtract=False, out_signed=False):
-    """Quantized add / subtract of two 8-bit tensors of the same shape (the NCE ELTWISE task)."""
+def nce_eltwise(a, b, p, zp_a, zp_b, mult_a, mult_b, out_mult, out_shift, subtract=False, out_signed=False, out_f16=False):
+    """Quantized add / subtract of two 8-bit tensors of the same shape (the NCE ELTWISE task); out_f16: fp16 bit patterns."""
     a = np.ascontiguousarray(a)
     b = np.ascontiguousarray(b)
     assert a.shape == b.shape
+    if out_f16:
+        out = np.zeros(a.shape, dtype=np.uint16)
+        lib().orc_nce_eltwise_f16(_p(a), C.c_int(int(a.dtype == np.int8)), _p(b), C.c_int(int(b.dtype == np.int8)), _p(out),
+                                  C.c_int64(a.size), C.c_int32(zp_a), C.c_int32(zp_b), C.c_int32(mult_a), C.c_int32(mult_b),
+                                  C.c_int(int(subtract)), C.c_int32(out_mult), C.c_int32(out_shift), C.byref(p))
+        return out
     out = np.zeros(a.shape, dtype=np.int8 if out_signed else np.uint8)
     lib().orc_nce_eltwise(_p(a), C.c_int(int(a.dtype == np.int8)), _p(b), C.c_int(int(b.dtype == np.int8)), _p(out),
                           C.c_int(int(out_signed)), C.c_int64(a.size), C.c_int32(zp_a), C.c_int32(zp_b),

@@ -599,3 +599,19 @@ void orc_nce_eltwise(const void* a, int a_signed, const void* b, int b_signed, v
         po[i] = (uint8_t)r;
     }
 }
+
+/* The same task with an fp16 output: the sum goes through the fixed-point PPE of orc_ppe_requant_f16 (no output zero
+ * point).  "parity unpinned" against silicon like that function. */
+void orc_nce_eltwise_f16(const void* a, int a_signed, const void* b, int b_signed, uint16_t* out, int64_t n, int32_t zp_a,
+                         int32_t zp_b, int32_t mult_a, int32_t mult_b, int subtract, int32_t out_mult, int32_t out_shift,
+                         const orc_ppe_t* ppe) {
+    const uint8_t* pa = (const uint8_t*)a;
+    const uint8_t* pb = (const uint8_t*)b;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        const int32_t va = (a_signed ? (int32_t)(int8_t)pa[i] : (int32_t)pa[i]) - zp_a;
+        const int32_t vb = (b_signed ? (int32_t)(int8_t)pb[i] : (int32_t)pb[i]) - zp_b;
+        const int32_t acc = va * mult_a + (subtract ? -1 : 1) * vb * mult_b;
+        out[i] = orc_ppe_requant_f16(acc, 0, out_mult, out_shift, ppe);
+    }
+}

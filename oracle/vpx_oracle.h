@@ -139,6 +139,11 @@ void orc_nce_eltwise(const void* a, int a_signed, const void* b, int b_signed, v
                      int32_t zp_a, int32_t zp_b, int32_t mult_a, int32_t mult_b, int subtract, int32_t out_mult,
                      int32_t out_shift, const orc_ppe_t* ppe);
 
+/* The same task with an fp16 output (the PPE of orc_ppe_requant_f16; no output zero point). */
+void orc_nce_eltwise_f16(const void* a, int a_signed, const void* b, int b_signed, uint16_t* out, int64_t n, int32_t zp_a,
+                         int32_t zp_b, int32_t mult_a, int32_t mult_b, int subtract, int32_t out_mult, int32_t out_shift,
+                         const orc_ppe_t* ppe);
+
 int orc_num_threads(void);
 void orc_set_num_threads(int n);
 

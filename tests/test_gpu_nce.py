@@ -731,6 +731,50 @@ def test_nce_eltwise(rt, orc, dev, subtract, mode):
         assert np.array_equal(got, want), "%s, negative multiplier: %d mismatches" % (shape, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("subtract", [False, True])
+@pytest.mark.parametrize("mode", ["NOOP", "LPRELU", "LRELU", "LRELUX"])
+def test_nce_eltwise_f16_output(rt, orc, dev, subtract, mode):
+    """The quantized add / subtract with an fp16 output (the sum through the s17.15 fixed-point PPE, no output zero point):
+    operand signedness, ragged sizes, an unaligned view, both signs of the output multiplier, an fp16 clamp."""
+    import torch
+    rng = np.random.default_rng(96)
+    in1_mult, in2_mult, out_mult, out_shift = rt.eltwise_quantization_approximation(0.02, 0.035, 0.05, 1 if subtract else 0)
+    md = getattr(rt, "PPE_" + mode)
+    hi = orc.pack_clamp_f16(0.0, 6.0) if mode == "LRELUX" else 2 ** 31 - 1
+    for a_signed, b_signed, zp1, zp2, shape, mult in ((False, True, 128, -3, (2, 9, 11, 64), out_mult), (True, True, 0, 5, (1, 7, 5, 33), -out_mult),
+                                                      (True, False, -7, 100, (3, 4, 4, 16), out_mult), (False, False, 3, 250, (1, 1, 1, 5), out_mult)):
+        a = rng.integers(-128, 128, shape).astype(np.int8) if a_signed else rng.integers(0, 256, shape, dtype=np.uint8)
+        b = rng.integers(-128, 128, shape).astype(np.int8) if b_signed else rng.integers(0, 256, shape, dtype=np.uint8)
+        ppe = rt.PpeInt(md, -(2 ** 31), hi, 1638, 14, mult, out_shift, in1_mult, in2_mult)
+        out = torch.full(shape, 99, dtype=torch.float16, device=dev)
+        rt.nce_eltwise(dev_t(a, dev), dev_t(b, dev), out, ppe, zp1, zp2, 0, subtract=subtract)
+        torch.cuda.synchronize()
+        assert rt.nce_last_kernel() == "nce_eltwise_kernel"
+        pm, ps = {"NOOP": (1, 0), "LPRELU": (1638, 14), "LRELU": (0, 0), "LRELUX": (0, 0)}[mode]
+        op = orc.ppe(pm, ps, 0, -(2 ** 31), hi)
+        want = orc.nce_eltwise(a, b, op, zp1, zp2, in1_mult, in2_mult, mult, out_shift, subtract=subtract, out_f16=True)
+        got = out.cpu().numpy().view(np.uint16)
+        assert np.array_equal(got, want), "%s: %d mismatches" % (shape, int((got != want).sum()))
+        vals = got.view(np.float16).astype(np.float32)
+        if mode in ("LRELU", "LRELUX"):
+            assert vals.min() >= 0.0
+        if mode == "LRELUX":
+            assert vals.max() <= 6.0
+    # an unaligned view: one value per lane
+    base = torch.zeros(1 + 2 * 5 * 3 * 16, dtype=torch.float16, device=dev)
+    view = base[1:].view(2, 5, 3, 16)
+    a = rng.integers(0, 256, (2, 5, 3, 16), dtype=np.uint8)
+    b = rng.integers(0, 256, (2, 5, 3, 16), dtype=np.uint8)
+    ppe = rt.PpeInt(md, -(2 ** 31), hi, 1638, 14, out_mult, out_shift, in1_mult, in2_mult)
+    rt.nce_eltwise(dev_t(a, dev), dev_t(b, dev), view, ppe, 120, 131, 0, subtract=subtract)
+    torch.cuda.synchronize()
+    pm, ps = {"NOOP": (1, 0), "LPRELU": (1638, 14), "LRELU": (0, 0), "LRELUX": (0, 0)}[mode]
+    want = orc.nce_eltwise(a, b, orc.ppe(pm, ps, 0, -(2 ** 31), hi), 120, 131, in1_mult, in2_mult, out_mult, out_shift, subtract=subtract,
+                           out_f16=True)
+    assert np.array_equal(view.cpu().numpy().view(np.uint16), want)
+    assert float(base[0]) == 0.0
+
+
 def test_nce_eltwise_full_size_residual(rt, orc, dev):
     """[4096, 11008] i8 + i8 -> i8, the quantized form of the C5 residual add, whole tensor against the oracle."""
     import torch

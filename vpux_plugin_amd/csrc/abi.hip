@@ -688,9 +688,9 @@ int vpx_nce_task(const vpx_nce_task_t* t, void* stream) {
     VPX_REQUIRE(t->groups >= 0 && (t->groups <= 1 || !eltwise), VPX_RESULT_ERROR_INVALID_ARGUMENT,
                 "NCE task: groups = %d (CONV tasks take 0, 1 or more; ELTWISE tasks 0 or 1)", t->groups);
     const auto is8 = [](int32_t ty) { return ty == VPX_NN_U8 || ty == VPX_NN_I8; };
-    const bool f16_out = t->output_type == VPX_NN_FP16 && !eltwise;
+    const bool f16_out = t->output_type == VPX_NN_FP16;
     VPX_REQUIRE(is8(t->input_type) && is8(t->weights_type) && (is8(t->output_type) || f16_out), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
-                "NCE task: U8/I8 input and weights with a U8/I8 output, or an FP16 output of a CONV task, are implemented (got %s, %s, %s)",
+                "NCE task: U8/I8 input and weights with a U8/I8 or FP16 output are implemented (got %s, %s, %s)",
                 dtype_name((uint32_t)t->input_type), dtype_name((uint32_t)t->weights_type), dtype_name((uint32_t)t->output_type));
     // a float output has no zero point (setupQuantInFloatOut programs none, runtime_dpu_parser_imports.cpp.inc:546-574)
     VPX_REQUIRE(!f16_out || t->zp_out == 0, VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: an FP16 output takes no zero point (got %d)",

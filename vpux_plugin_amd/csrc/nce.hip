@@ -1914,15 +1914,44 @@ struct EltParams {
     ChanPrep cp;
     PpePack pk;
     int general;
+    ChanPrep cp16;         // fp16 output: the factors with 15 fractional bits kept, plain form (see ppe_fast_f16)
+    float f16_lo, f16_hi;  // and its clamp bounds
 };
 
-template <bool A_SIGNED, bool B_SIGNED, bool SAME_F>
+// OUT_F16: sixteen sums leave as sixteen fp16 values (two 16-byte stores per lane).
+template <bool A_SIGNED, bool B_SIGNED, bool SAME_F, bool OUT_F16 = false>
 __global__ __launch_bounds__(256) void nce_eltwise_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
                                                           uint8_t* __restrict__ out, int64_t n_vec, int64_t n,
                                                           EltParams e) {
     auto val = [](unsigned word, int k, bool sgn) {
         return sgn ? (int)(int8_t)(word >> (8 * k)) : (int)((word >> (8 * k)) & 0xffu);
     };
+    if constexpr (OUT_F16) {
+        uint16_t* out16 = reinterpret_cast<uint16_t*>(out);
+        const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+        if (v < n_vec) {
+            const i32x4 qa = reinterpret_cast<const i32x4*>(a)[v];
+            const i32x4 qb = reinterpret_cast<const i32x4*>(b)[v];
+            i32x4 r[2] = {i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}};
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int acc = val((unsigned)qa[j], k, A_SIGNED) * e.m1 + val((unsigned)qb[j], k, B_SIGNED) * e.m2;
+                    const int idx = 4 * j + k;  // value idx of the sixteen: half (idx % 2) of dword idx / 2
+                    r[idx >> 3][(idx >> 1) & 3] |= (int)ppe_fast_f16(acc, e.cp16, e.f16_lo, e.f16_hi) << (16 * (idx & 1));
+                }
+            __builtin_nontemporal_store(r[0], reinterpret_cast<i32x4*>(out16) + 2 * v);
+            __builtin_nontemporal_store(r[1], reinterpret_cast<i32x4*>(out16) + 2 * v + 1);
+        }
+        if (blockIdx.x == gridDim.x - 1) {
+            for (int64_t i = n_vec * 16 + threadIdx.x; i < n; i += 256) {
+                const int acc = val(a[i], 0, A_SIGNED) * e.m1 + val(b[i], 0, B_SIGNED) * e.m2;
+                out16[i] = ppe_fast_f16(acc, e.cp16, e.f16_lo, e.f16_hi);
+            }
+        }
+        return;
+    }
     auto four = [&](unsigned wa, unsigned wb, auto general_c) {
         int acc[4];
 #pragma unroll
@@ -2401,6 +2430,7 @@ int set_dyn_lds(KernelT kernel, size_t bytes) {
 // PPE of one eltwise value on the host: decides which device variant is needed
 int launch_nce_eltwise(const vpx_nce_task_t& t, const Ppe& ppe, hipStream_t s, const char** kernel_name) {
     const bool a_signed = t.input_type == VPX_NN_I8, b_signed = t.weights_type == VPX_NN_I8, out_signed = t.output_type == VPX_NN_I8;
+    const bool out_f16 = t.output_type == VPX_NN_FP16;
     const int64_t n = t.N * t.H * t.W * t.IC;
     *kernel_name = "nce_eltwise_kernel";
     if (n == 0) return VPX_RESULT_SUCCESS;
@@ -2433,6 +2463,14 @@ int launch_nce_eltwise(const vpx_nce_task_t& t, const Ppe& ppe, hipStream_t s, c
     const int off = out_signed ? 128 : 0, z = t.zp_out + off;
     e.pk = PpePack{6755399441055744.0 + (double)(z & ~1), z & 1, lo + off, hi + off, out_signed ? 0x80808080u : 0u};
     e.general = (e.cp.bmax_pos != 0x7fffffff || e.cp.bmax_neg != 0x7fffffff || (z & 1)) ? 1 : 0;
+    // host copy of ppe_prepare with shift - 15 (an fp16 output keeps 15 fractional bits of the scaled value)
+    e.cp16.f_pos = std::ldexp((double)t.ppe.quant_mult, -(t.ppe.quant_shift - 15));
+    e.cp16.f_neg = std::ldexp((double)((long long)t.ppe.quant_mult * (long long)ppe.prelu_mult), -(t.ppe.quant_shift - 15 + ppe.prelu_shift));
+    e.cp16.bias = (int)bias;
+    e.cp16.sgn = t.ppe.quant_mult < 0 ? -1 : 0;
+    e.cp16.bmax_pos = e.cp16.bmax_neg = 0x7fffffff;
+    e.f16_lo = ppe.f16_lo;
+    e.f16_hi = ppe.f16_hi;
     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
     const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights) |
                            reinterpret_cast<uintptr_t>(t.output)) & 15) == 0;
@@ -2443,6 +2481,18 @@ int launch_nce_eltwise(const vpx_nce_task_t& t, const Ppe& ppe, hipStream_t s, c
 #define VPX_ELT(AS, BS, SF)                                                                                            \
     hipLaunchKernelGGL((nce_eltwise_kernel<AS, BS, SF>), grid, block, 0, s, (const uint8_t*)t.input,                   \
                        (const uint8_t*)t.weights, (uint8_t*)t.output, n_vec, n, e)
+#define VPX_ELT16(AS, BS)                                                                                              \
+    hipLaunchKernelGGL((nce_eltwise_kernel<AS, BS, false, true>), grid, block, 0, s, (const uint8_t*)t.input,          \
+                       (const uint8_t*)t.weights, (uint8_t*)t.output, n_vec, n, e)
+    if (out_f16) {
+        if (a_signed && b_signed) VPX_ELT16(true, true);
+        else if (a_signed) VPX_ELT16(true, false);
+        else if (b_signed) VPX_ELT16(false, true);
+        else VPX_ELT16(false, false);
+#undef VPX_ELT16
+        VPX_HIP_CHECK(hipGetLastError());
+        return VPX_RESULT_SUCCESS;
+    }
     const int sel = (a_signed ? 4 : 0) | (b_signed ? 2 : 0) | (same_f ? 1 : 0);
     switch (sel) {
     case 0: VPX_ELT(false, false, false); break;
