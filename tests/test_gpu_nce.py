@@ -534,7 +534,9 @@ F16_NONE = {"clamp_low": -(2 ** 31), "clamp_high": 2 ** 31 - 1}
     (dict(N=1, H=9, W=9, IC=256, OC=96, KY=3, KX=3), "nce_conv_stream", None),           # streamed weights, K split over two groups of waves
     (dict(N=3, H=7, W=7, IC=512, OC=72, KY=3, KX=3), "nce_conv_stream", None),           # ... over eight waves
     (dict(N=2, H=30, W=33, IC=192, OC=40, KY=3, KX=3), "nce_conv_stream", None),         # ... one tile per wave
-    (dict(N=1, H=10, W=12, IC=48, OC=40, KY=3, KX=3), "nce_conv_mfma16", None),
+    (dict(N=1, H=10, W=12, IC=48, OC=40, KY=3, KX=3), "nce_conv_rows16", None),          # input rows in LDS, two 16-byte stores per position and lane
+    (dict(N=2, H=31, W=40, IC=16, OC=72, KY=3, KX=3), "nce_conv_rows16", None),
+    (dict(N=1, H=10, W=12, IC=48, OC=40, KY=3, KX=3), "nce_conv_mfma16", "gather"),
     (dict(N=2, H=6, W=7, IC=5, OC=9, KY=3, KX=2), "nce_conv_naive", None),
     (dict(N=1, H=40, W=1, IC=64, OC=96, KY=1, KX=1), "nce_conv_naive", "naive"),
 ])

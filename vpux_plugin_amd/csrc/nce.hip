@@ -2109,8 +2109,8 @@ struct RowsGeom {
 };
 
 // TN: channel tiles of 32 per workgroup (1 for layers of up to 32 output channels).  MULTI: some workgroup takes more
-// than one tile.
-template <bool IN_U8, int TM, int TN, bool MULTI>
+// than one tile.  F16: the output is fp16 (the s17.15 PPE; sixteen channels of a position are two 16-byte stores).
+template <bool IN_U8, int TM, int TN, bool MULTI, bool F16 = false>
 __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                        const int32_t* __restrict__ wt, uint8_t* __restrict__ out, ConvGeom g,
                                                        RowsGeom rg, int pad_byte, GemmPpe ppe) {
@@ -2241,7 +2241,8 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
     const PpePack pk = make_ppe_pack(ppe.zp_out, ppe.lo, ppe.hi, ppe.out_signed != 0);
     if (tid < BN) {
         const uint32_t w2 = (uint32_t)wt2;
-        const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu),
+        // (an fp16 output keeps 15 fractional bits of the scaled value)
+        const ChanPrep c = ppe_prepare((int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu) - (F16 ? 15 : 0),
                                        (int)((unsigned)wt3 + (unsigned)(ppe.corr * csum[tid])), ppe.prelu_mult, ppe.prelu_shift);
         sprep[tid] = c;
         sbias[tid] = c.bias;
@@ -2277,9 +2278,10 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         uint8_t* const out0 = out + pos0 * OC;
 
         auto one_block = [&](int b, auto kind_c) {
-            // PPE kinds.  0: the general form; 1: two factors, the short form (see ppe_pack4_biased); 2: one factor
+            // PPE kinds.  0: the general form; 1: two factors, the short form (see ppe_pack4_biased); 2: one factor;
+            // 3: fp16 output (like the general form the accumulators start from zero and the PPE adds the bias)
             constexpr int KIND = decltype(kind_c)::value;
-            constexpr bool GENERAL = KIND == 0;
+            constexpr bool GENERAL = KIND == 0 || KIND == 3;
             const uint8_t* pl[TM];
             int pc[TM];  // the position's offset from the tile's first one in the output, -1 for none
 #pragma unroll
@@ -2353,6 +2355,40 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                         for (int r = 0; r < 16; r++) acc[i][j][r] += v;
                 }
             }
+            if constexpr (KIND == 3) {
+                uint16_t* const out16 = reinterpret_cast<uint16_t*>(out) + pos0 * OC;
+                const bool vec16_ok = (OC & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const int qc = q16 + 32 * j;
+#pragma unroll
+                    for (int half8 = 0; half8 < 2; half8++) {  // channels 0-7, then 8-15 of the lane's sixteen
+                        i32x4 o8[TM];
+#pragma unroll
+                        for (int i = 0; i < TM; i++) o8[i] = i32x4{0, 0, 0, 0};
+#pragma unroll
+                        for (int r8 = 0; r8 < 8; r8++) {
+                            const int r = half8 * 8 + r8;
+                            const ChanPrep c = sprep[32 * j + 16 * half + r];
+#pragma unroll
+                            for (int i = 0; i < TM; i++)
+                                o8[i][r8 >> 1] |= (int)ppe_fast_f16(acc[i][j][r], c, ppe.f16_lo, ppe.f16_hi) << (16 * (r8 & 1));
+                            __builtin_amdgcn_sched_barrier(0);  // (a channel at a time: hoisted, the parameters of all sixteen fill the register file)
+                        }
+#pragma unroll
+                        for (int i = 0; i < TM; i++) {
+                            if (pc[i] < 0 || qc + 8 * half8 >= OC) continue;
+                            uint16_t* dst = out16 + ((int64_t)pc[i] * OC + qc + 8 * half8);
+                            if (vec16_ok && qc + 8 * half8 + 8 <= OC) {
+                                __builtin_nontemporal_store(o8[i], reinterpret_cast<i32x4*>(dst));
+                            } else {
+                                for (int e = 0; e < 8 && qc + 8 * half8 + e < OC; e++) dst[e] = (uint16_t)(o8[i][e >> 1] >> (16 * (e & 1)));
+                            }
+                        }
+                    }
+                }
+                return;
+            }
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 i32x4 o[TM];
@@ -2361,7 +2397,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const ChanPrep* cpp = sprep + 32 * j + 16 * half + r;
-                    if constexpr (GENERAL) {
+                    if constexpr (KIND == 0) {
                         ChanPrep c = *cpp;  // the form ppe_one takes: sign flip in the bias, factors swapped for a negative multiplier
                         c.bias = (int)((unsigned)c.bias + 0x80000000u);
                         if (c.sgn) {
@@ -2395,7 +2431,9 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                 }
             }
         };
-        if (general) {
+        if constexpr (F16) {
+            for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 3>{});
+        } else if (general) {
             for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 0>{});
         } else if (same_f) {
             for (int b = wave; b < nblk; b += NW) one_block(b, std::integral_constant<int, 2>{});
@@ -3134,7 +3172,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
 
     // Channel counts that are a multiple of 16 but not of 32 (stem layers): the row-patch kernel where a band of input
     // rows and the weights fit LDS together, else the gather kernel below.
-    if (allow_lds && mfma_ok && aligned && !out_f16 && g.IC % 16 == 0 && g.IC % 32 != 0 && g.H * g.W * g.IC < (1ll << 31) &&
+    if (allow_lds && mfma_ok && aligned && g.IC % 16 == 0 && g.IC % 32 != 0 && g.H * g.W * g.IC < (1ll << 31) &&
         g.N * g.OH < (1ll << 30) && g.OC < (1 << 24) && g.KY * g.KX * g.IC < (1 << 16)) {
         RowsGeom rg{};
         const int cpt = (int)g.IC / 16;
@@ -3214,15 +3252,23 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             const size_t lds = need(best_r, best_cw);
             const int64_t per_wg = (rg.ntiles + slots - 1) / slots;
             const dim3 grid((unsigned)((rg.ntiles + per_wg - 1) / per_wg), (unsigned)ocb);
-            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, t.zp_out, lo, hi, out_signed ? 1 : 0, rowterm};
+            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, t.zp_out, lo, hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi, out_f16 ? 1 : 0};
             const int pad_byte = t.zp_in & 0xff;
 #define VPX_ROWS_T(U8, TNV, TMV, MULTIV)                                                                              \
     do {                                                                                                              \
-        auto kern = nce_conv_rows16<U8, TMV, TNV, MULTIV>;                                                            \
-        rc = set_dyn_lds(kern, lds);                                                                                  \
-        if (rc) return rc;                                                                                            \
-        hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, \
-                           (uint8_t*)t.output, g, rg, pad_byte, gp);                                                  \
+        if (out_f16) {                                                                                                \
+            auto kern = nce_conv_rows16<U8, TMV, TNV, MULTIV, true>;                                                  \
+            rc = set_dyn_lds(kern, lds);                                                                              \
+            if (rc) return rc;                                                                                        \
+            hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,       \
+                               t.weight_table, (uint8_t*)t.output, g, rg, pad_byte, gp);                              \
+        } else {                                                                                                      \
+            auto kern = nce_conv_rows16<U8, TMV, TNV, MULTIV, false>;                                                 \
+            rc = set_dyn_lds(kern, lds);                                                                              \
+            if (rc) return rc;                                                                                        \
+            hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,       \
+                               t.weight_table, (uint8_t*)t.output, g, rg, pad_byte, gp);                              \
+        }                                                                                                             \
     } while (0)
 #define VPX_ROWS(U8, TNV)                                                                                             \
     do {                                                                                                              \
