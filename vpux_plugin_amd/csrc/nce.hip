@@ -2810,6 +2810,129 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         wofs = wbytes + (rbytes + 255) / 256 * 256;
         return VPX_RESULT_SUCCESS;
     };
+    // Channel counts that are a multiple of 16 but not of 64 (stem layers; 32, 96, 160 ... channels): the row-patch kernel
+    // where a band of input rows and the weights fit LDS together, else the gather kernels below.  (Multiples of 32 have a
+    // gather kernel that takes any K: they come here while the weights leave most of LDS to the rows -- [32,112,112,32] ->
+    // 64 3x3: 27 us against 64 us, [32,14,14,160] -> 320 1x1: 9 against 19.5; 5x5 x 96 channels, 154 KiB of weights: 183 against 47.)
+    if (allow_lds && !use_gemm && mfma_ok && aligned && g.IC % 16 == 0 &&
+        (g.IC % 32 != 0 || (g.IC % 64 != 0 && (g.OC <= 32 ? 32 : 64) * ((g.KY * g.KX * (g.IC / 16) + 1) / 2 * 32 + 16) <= 100 * 1024)) &&
+        g.H * g.W * g.IC < (1ll << 31) &&
+        g.N * g.OH < (1ll << 30) && g.OC < (1 << 24) && g.KY * g.KX * g.IC < (1 << 16)) {
+        RowsGeom rg{};
+        const int cpt = (int)g.IC / 16;
+        rg.S = (g.KY * g.KX * cpt + 1) / 2;
+        rg.WS = rg.S * 32 + 16;
+        rg.m = g.SX * cpt;
+        // bytes per patch row under CW output columns: m planes of chunks
+        auto row_bytes = [&](int64_t CW) { return (((CW - 1) * g.SX + g.KX) * cpt + rg.m - 1) / rg.m * rg.m * 16; };
+        const int bn = g.OC <= 32 ? 32 : 64;  // channels per workgroup
+        const size_t fixed = bn * (size_t)rg.WS + bn * sizeof(ChanPrep) + 2 * bn * sizeof(int) + 16 + (size_t)(2 * rg.S + 3) / 4 * 16;
+        auto need = [&](int64_t R, int64_t CW) { return fixed + (size_t)((R - 1) * g.SY + g.KY) * (size_t)row_bytes(CW); };
+        int cus = 0;
+        int rc = device_compute_units(&cus);
+        if (rc) return rc;
+        const int64_t ocb = (g.OC + bn - 1) / bn;
+        const int64_t slots = cus / ocb > 0 ? cus / ocb : 1;  // workgroups per block of channels
+        // Tile height and positions per wave block: the cheapest of all that fit, counted in MFMA time (32 clocks
+        // each) plus the staging of the rows at about 64 bytes per clock; a workgroup's eight waves take a block each.
+        const int S = rg.S;
+        int best_r = 0, best_tm = 0;
+        int64_t best_cw = 0;
+        double best = 0;
+        // (the whole width, or the width in 2 .. 32 column tiles: the rows under a band of a wide image do not fit LDS)
+        for (int tx = 1; tx <= 32 && (tx == 1 || best_tm == 0 || g.OW / tx >= 64); tx++) {
+            const int64_t CW = (g.OW + tx - 1) / tx, RB = row_bytes(CW);
+            if (tx > 1 && (g.OW + CW - 1) / CW != tx) continue;
+            for (int64_t R = 1; R <= g.OH && need(R, CW) <= kMaxDynLds; R++) {
+                const int64_t ntiles = g.N * ((g.OH + R - 1) / R) * tx;
+                const int64_t per_wg = (ntiles + slots - 1) / slots;
+                for (int tm = 2; tm <= 4; tm += 2) {
+                    const int64_t blocks = (R * CW + 32 * tm - 1) / (32 * tm);
+                    const double cost = (double)per_wg * ((double)((blocks + 7) / 8) * tm * (bn / 32) * (S * 32.0 + 400) * 2 +
+                                                          (double)((R - 1) * g.SY + g.KY) * (double)RB / 64 + 1500);
+                    if (best_tm == 0 || cost < best || (cost == best && (int)R == best_r && CW == best_cw)) {  // (a tie between the block sizes of one tile: the larger)
+                        best = cost;
+                        best_r = (int)R;
+                        best_cw = CW;
+                        best_tm = tm;
+                    }
+                }
+            }
+        }
+        if (const int v = knobs.conv_rows.load()) {
+            if (best_tm != 0 && v >= 1 && v <= g.OH && need(v, best_cw) <= kMaxDynLds) best_r = v;
+        }
+        if (const int v = knobs.conv_cols.load()) {
+            if (best_tm != 0 && v >= 1 && v <= g.OW && need(best_r, v) <= kMaxDynLds) best_cw = v;
+        }
+        const int64_t RB = best_tm ? row_bytes(best_cw) : 0;
+        if (best_tm != 0 && RB < (1 << 20) && g.N * ((g.OH + best_r - 1) / best_r) * ((g.OW + best_cw - 1) / best_cw) < (1ll << 30)) {
+            const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
+            rc = rebias_weights();
+            if (rc) return rc;
+            const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
+            int lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin, hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
+            if (lo > tmax) lo = tmax;
+            if (hi < tmin) hi = tmin;
+            if (lo > hi) lo = hi;
+            auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
+            const int tiles_y = (int)((g.OH + best_r - 1) / best_r), tiles_x = (int)((g.OW + best_cw - 1) / best_cw);
+            rg.R = best_r;
+            rg.CW = (int)best_cw;
+            rg.PH = (best_r - 1) * g.SY + g.KY;
+            rg.RB = (int)RB;
+            rg.plane = (int)(RB / 16 / rg.m);
+            rg.row_chunks = (int)(((best_cw - 1) * g.SX + g.KX) * cpt);
+            rg.ntiles = (int)(g.N * tiles_y * tiles_x);
+            rg.tiles_y = fd(tiles_y);
+            rg.tiles_x = fd(tiles_x);
+            rg.cw = fd(best_cw);
+            rg.ow = fd(g.OW);
+            rg.rc = fd(rg.row_chunks);
+            rg.cpp = fd(cpt);
+            rg.kc = fd(2 * rg.S);
+            rg.fm = fd(rg.m);
+            rg.rin = fd(g.KX * cpt);
+            const size_t lds = need(best_r, best_cw);
+            const int64_t per_wg = (rg.ntiles + slots - 1) / slots;
+            const dim3 grid((unsigned)((rg.ntiles + per_wg - 1) / per_wg), (unsigned)ocb);
+            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, t.zp_out, lo, hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi, out_f16 ? 1 : 0};
+            const int pad_byte = t.zp_in & 0xff;
+#define VPX_ROWS_T(U8, TNV, TMV, MULTIV)                                                                              \
+    do {                                                                                                              \
+        if (out_f16) {                                                                                                \
+            auto kern = nce_conv_rows16<U8, TMV, TNV, MULTIV, true>;                                                  \
+            rc = set_dyn_lds(kern, lds);                                                                              \
+            if (rc) return rc;                                                                                        \
+            hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,       \
+                               t.weight_table, (uint8_t*)t.output, g, rg, pad_byte, gp);                              \
+        } else {                                                                                                      \
+            auto kern = nce_conv_rows16<U8, TMV, TNV, MULTIV, false>;                                                 \
+            rc = set_dyn_lds(kern, lds);                                                                              \
+            if (rc) return rc;                                                                                        \
+            hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,       \
+                               t.weight_table, (uint8_t*)t.output, g, rg, pad_byte, gp);                              \
+        }                                                                                                             \
+    } while (0)
+#define VPX_ROWS(U8, TNV)                                                                                             \
+    do {                                                                                                              \
+        if (best_tm == 4 && per_wg > 1) VPX_ROWS_T(U8, TNV, 4, true);                                                \
+        else if (best_tm == 4) VPX_ROWS_T(U8, TNV, 4, false);                                                        \
+        else if (per_wg > 1) VPX_ROWS_T(U8, TNV, 2, true);                                                           \
+        else VPX_ROWS_T(U8, TNV, 2, false);                                                                          \
+    } while (0)
+            if (in_u8 && bn == 32) VPX_ROWS(true, 1);
+            else if (in_u8) VPX_ROWS(true, 2);
+            else if (bn == 32) VPX_ROWS(false, 1);
+            else VPX_ROWS(false, 2);
+#undef VPX_ROWS
+#undef VPX_ROWS_T
+            VPX_HIP_CHECK(hipGetLastError());
+            *kernel_name = "nce_conv_rows16";
+            return VPX_RESULT_SUCCESS;
+        }
+    }
+
     if (allow_mfma && mfma_ok && aligned && (use_gemm || g.IC % 32 == 0)) {
         int rc = VPX_RESULT_SUCCESS;
         rc = rebias_weights();
@@ -3168,125 +3291,6 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         VPX_HIP_CHECK(hipGetLastError());
         *kernel_name = "nce_conv_mfma";
         return VPX_RESULT_SUCCESS;
-    }
-
-    // Channel counts that are a multiple of 16 but not of 32 (stem layers): the row-patch kernel where a band of input
-    // rows and the weights fit LDS together, else the gather kernel below.
-    if (allow_lds && mfma_ok && aligned && g.IC % 16 == 0 && g.IC % 32 != 0 && g.H * g.W * g.IC < (1ll << 31) &&
-        g.N * g.OH < (1ll << 30) && g.OC < (1 << 24) && g.KY * g.KX * g.IC < (1 << 16)) {
-        RowsGeom rg{};
-        const int cpt = (int)g.IC / 16;
-        rg.S = (g.KY * g.KX * cpt + 1) / 2;
-        rg.WS = rg.S * 32 + 16;
-        rg.m = g.SX * cpt;
-        // bytes per patch row under CW output columns: m planes of chunks
-        auto row_bytes = [&](int64_t CW) { return (((CW - 1) * g.SX + g.KX) * cpt + rg.m - 1) / rg.m * rg.m * 16; };
-        const int bn = g.OC <= 32 ? 32 : 64;  // channels per workgroup
-        const size_t fixed = bn * (size_t)rg.WS + bn * sizeof(ChanPrep) + 2 * bn * sizeof(int) + 16 + (size_t)(2 * rg.S + 3) / 4 * 16;
-        auto need = [&](int64_t R, int64_t CW) { return fixed + (size_t)((R - 1) * g.SY + g.KY) * (size_t)row_bytes(CW); };
-        int cus = 0;
-        int rc = device_compute_units(&cus);
-        if (rc) return rc;
-        const int64_t ocb = (g.OC + bn - 1) / bn;
-        const int64_t slots = cus / ocb > 0 ? cus / ocb : 1;  // workgroups per block of channels
-        // Tile height and positions per wave block: the cheapest of all that fit, counted in MFMA time (32 clocks
-        // each) plus the staging of the rows at about 64 bytes per clock; a workgroup's eight waves take a block each.
-        const int S = rg.S;
-        int best_r = 0, best_tm = 0;
-        int64_t best_cw = 0;
-        double best = 0;
-        // (the whole width, or the width in 2 .. 32 column tiles: the rows under a band of a wide image do not fit LDS)
-        for (int tx = 1; tx <= 32 && (tx == 1 || best_tm == 0 || g.OW / tx >= 64); tx++) {
-            const int64_t CW = (g.OW + tx - 1) / tx, RB = row_bytes(CW);
-            if (tx > 1 && (g.OW + CW - 1) / CW != tx) continue;
-            for (int64_t R = 1; R <= g.OH && need(R, CW) <= kMaxDynLds; R++) {
-                const int64_t ntiles = g.N * ((g.OH + R - 1) / R) * tx;
-                const int64_t per_wg = (ntiles + slots - 1) / slots;
-                for (int tm = 2; tm <= 4; tm += 2) {
-                    const int64_t blocks = (R * CW + 32 * tm - 1) / (32 * tm);
-                    const double cost = (double)per_wg * ((double)((blocks + 7) / 8) * tm * (bn / 32) * (S * 32.0 + 400) * 2 +
-                                                          (double)((R - 1) * g.SY + g.KY) * (double)RB / 64 + 1500);
-                    if (best_tm == 0 || cost < best || (cost == best && (int)R == best_r && CW == best_cw)) {  // (a tie between the block sizes of one tile: the larger)
-                        best = cost;
-                        best_r = (int)R;
-                        best_cw = CW;
-                        best_tm = tm;
-                    }
-                }
-            }
-        }
-        if (const int v = knobs.conv_rows.load()) {
-            if (best_tm != 0 && v >= 1 && v <= g.OH && need(v, best_cw) <= kMaxDynLds) best_r = v;
-        }
-        if (const int v = knobs.conv_cols.load()) {
-            if (best_tm != 0 && v >= 1 && v <= g.OW && need(best_r, v) <= kMaxDynLds) best_cw = v;
-        }
-        const int64_t RB = best_tm ? row_bytes(best_cw) : 0;
-        if (best_tm != 0 && RB < (1 << 20) && g.N * ((g.OH + best_r - 1) / best_r) * ((g.OW + best_cw - 1) / best_cw) < (1ll << 30)) {
-            const int corr = in_u8 ? 128 - t.zp_in : -t.zp_in;
-            rc = rebias_weights();
-            if (rc) return rc;
-            const int tmin = out_signed ? -128 : 0, tmax = out_signed ? 127 : 255;
-            int lo = ppe.clamp_lo > tmin ? ppe.clamp_lo : tmin, hi = ppe.clamp_hi < tmax ? ppe.clamp_hi : tmax;
-            if (lo > tmax) lo = tmax;
-            if (hi < tmin) hi = tmin;
-            if (lo > hi) lo = hi;
-            auto fd = [](int64_t d) { return FastDiv{(uint32_t)d, (uint32_t)(((1ull << 32) + (uint64_t)d - 1) / (uint64_t)d)}; };
-            const int tiles_y = (int)((g.OH + best_r - 1) / best_r), tiles_x = (int)((g.OW + best_cw - 1) / best_cw);
-            rg.R = best_r;
-            rg.CW = (int)best_cw;
-            rg.PH = (best_r - 1) * g.SY + g.KY;
-            rg.RB = (int)RB;
-            rg.plane = (int)(RB / 16 / rg.m);
-            rg.row_chunks = (int)(((best_cw - 1) * g.SX + g.KX) * cpt);
-            rg.ntiles = (int)(g.N * tiles_y * tiles_x);
-            rg.tiles_y = fd(tiles_y);
-            rg.tiles_x = fd(tiles_x);
-            rg.cw = fd(best_cw);
-            rg.ow = fd(g.OW);
-            rg.rc = fd(rg.row_chunks);
-            rg.cpp = fd(cpt);
-            rg.kc = fd(2 * rg.S);
-            rg.fm = fd(rg.m);
-            rg.rin = fd(g.KX * cpt);
-            const size_t lds = need(best_r, best_cw);
-            const int64_t per_wg = (rg.ntiles + slots - 1) / slots;
-            const dim3 grid((unsigned)((rg.ntiles + per_wg - 1) / per_wg), (unsigned)ocb);
-            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, t.zp_out, lo, hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi, out_f16 ? 1 : 0};
-            const int pad_byte = t.zp_in & 0xff;
-#define VPX_ROWS_T(U8, TNV, TMV, MULTIV)                                                                              \
-    do {                                                                                                              \
-        if (out_f16) {                                                                                                \
-            auto kern = nce_conv_rows16<U8, TMV, TNV, MULTIV, true>;                                                  \
-            rc = set_dyn_lds(kern, lds);                                                                              \
-            if (rc) return rc;                                                                                        \
-            hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,       \
-                               t.weight_table, (uint8_t*)t.output, g, rg, pad_byte, gp);                              \
-        } else {                                                                                                      \
-            auto kern = nce_conv_rows16<U8, TMV, TNV, MULTIV, false>;                                                 \
-            rc = set_dyn_lds(kern, lds);                                                                              \
-            if (rc) return rc;                                                                                        \
-            hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, (const int8_t*)t.input, (const int8_t*)wptr,       \
-                               t.weight_table, (uint8_t*)t.output, g, rg, pad_byte, gp);                              \
-        }                                                                                                             \
-    } while (0)
-#define VPX_ROWS(U8, TNV)                                                                                             \
-    do {                                                                                                              \
-        if (best_tm == 4 && per_wg > 1) VPX_ROWS_T(U8, TNV, 4, true);                                                \
-        else if (best_tm == 4) VPX_ROWS_T(U8, TNV, 4, false);                                                        \
-        else if (per_wg > 1) VPX_ROWS_T(U8, TNV, 2, true);                                                           \
-        else VPX_ROWS_T(U8, TNV, 2, false);                                                                          \
-    } while (0)
-            if (in_u8 && bn == 32) VPX_ROWS(true, 1);
-            else if (in_u8) VPX_ROWS(true, 2);
-            else if (bn == 32) VPX_ROWS(false, 1);
-            else VPX_ROWS(false, 2);
-#undef VPX_ROWS
-#undef VPX_ROWS_T
-            VPX_HIP_CHECK(hipGetLastError());
-            *kernel_name = "nce_conv_rows16";
-            return VPX_RESULT_SUCCESS;
-        }
     }
 
     if (allow_mfma && mfma_ok && aligned && g.IC % 16 == 0 && g.IC % 32 != 0 && ((Ktot + 31) / 32 * 32 + 16) * 64 <= 64 * 1024) {
