@@ -368,7 +368,7 @@ def test_row_patch_conv_random_geometries(rt, orc, dev, seed):
     rng = np.random.default_rng(seed)
     for i in range(24):
         IC = int(rng.choice([16, 16, 16, 48, 80, 112, 32, 96, 160]))
-        OC = int(rng.choice([1, 15, 16, 32, 40, 64, 64, 72, 100, 128, 130]))
+        OC = int(rng.choice([1, 15, 16, 32, 40, 64, 64, 72, 100, 128, 130, 250, 256]))  # (120 .. 128 of 128, 240 .. 256: blocks of 128 channels where K is short)
         KY, KX = int(rng.integers(1, 8)), int(rng.integers(1, 8))
         SY, SX = int(rng.integers(1, 4)), int(rng.integers(1, 4))
         pl, pr, pt, pb = [int(v) for v in rng.integers(0, 4, 4)]
@@ -408,7 +408,8 @@ def test_row_patch_conv_random_geometries(rt, orc, dev, seed):
         OW = (W + pl + pr - KX) // SX + 1
         steps, m = (KY * KX * IC // 16 + 1) // 2, SX * IC // 16
         row = -(-(((OW - 1) * SX + KX) * IC // 16) // m) * m * 16
-        bn = 32 if OC <= 32 else 64  # channels per workgroup
+        wide = OC > 64 and 128 * (steps * 32 + 16) <= 40 * 1024 and (-(-OC // 128) * 128 - OC) * 8 <= OC
+        bn = 32 if OC <= 32 else (128 if wide else 64)  # channels per workgroup
         lds = bn * (steps * 32 + 16) + bn * 32 + 2 * bn * 4 + 16 + (2 * steps + 3) // 4 * 16 + KY * row
         # (multiples of 32 have a gather kernel for any K: they take this one while the weights leave most of LDS to the rows)
         if lds <= 160 * 1024 - 512 and (IC % 32 != 0 or bn * (steps * 32 + 16) <= 100 * 1024):

@@ -2108,7 +2108,8 @@ struct RowsGeom {
     FastDiv tiles_y, ow, rc, cpp, kc, fm, rin;  // tiles per image, OW, row_chunks, chunks per pixel, 2 * S, m, chunks per kernel row
 };
 
-// TN: channel tiles of 32 per workgroup (1 for layers of up to 32 output channels).  MULTI: some workgroup takes more
+// TN: channel tiles of 32 per workgroup (1 for layers of up to 32 output channels; 4, with TM = 2, for short-K layers of
+// many output channels, whose input rows are then staged by half as many workgroups).  MULTI: some workgroup takes more
 // than one tile.  F16: the output is fp16 (the s17.15 PPE; sixteen channels of a position are two 16-byte stores).
 template <bool IN_U8, int TM, int TN, bool MULTI, bool F16 = false>
 __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
@@ -2133,7 +2134,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
 
     // ---- input rows -> LDS: patch row py is input row iy0 + py from pixel -PL on; padding and the sign flip applied here.
     // The first UPF chunks of every thread stay in registers from the load (issued a tile ahead) to the store.
-    constexpr int UPF = TM == 4 ? 6 : 9;  // (what the registers beside the accumulators allow)
+    constexpr int UPF = TM * TN >= 8 ? 6 : 9;  // (what the registers beside the accumulators allow)
     const int pad32 = (pad_byte & 0xff) * 0x01010101;
     const int total_chunks = rg.PH * rg.row_chunks;
     i32x4 qv[UPF];
@@ -2219,13 +2220,13 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         const int oc = oc0 + n < OC ? oc0 + n : OC - 1;  // channels past the end repeat the last one
         i32x4 v = i32x4{0, 0, 0, 0};
         if (c < nchunks) v = *reinterpret_cast<const i32x4*>(w + (int64_t)oc * Ktot + c * 16);
-        const int lrow = (n & 32) + 8 * ((n >> 2) & 3) + 4 * ((n >> 4) & 1) + (n & 3);
+        const int lrow = (n & ~31) + 8 * ((n >> 2) & 3) + 4 * ((n >> 4) & 1) + (n & 3);
         *reinterpret_cast<i32x4*>(wlds + lrow * rg.WS + c * 16) = v;
     }
     __syncthreads();
     if (tid < 4 * BN) {  // the sums of the weight rows, for the zero-point term
         const int n = tid >> 2, part = tid & 3;
-        const int lrow = (n & 32) + 8 * ((n >> 2) & 3) + 4 * ((n >> 4) & 1) + (n & 3);
+        const int lrow = (n & ~31) + 8 * ((n >> 2) & 3) + 4 * ((n >> 4) & 1) + (n & 3);
         int sum = 0;
         if (ppe.corr != 0)
             for (int c = part; c < kc; c += 4) {
@@ -2825,7 +2826,11 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         rg.m = g.SX * cpt;
         // bytes per patch row under CW output columns: m planes of chunks
         auto row_bytes = [&](int64_t CW) { return (((CW - 1) * g.SX + g.KX) * cpt + rg.m - 1) / rg.m * rg.m * 16; };
-        const int bn = g.OC <= 32 ? 32 : 64;  // channels per workgroup
+        // channels per workgroup: 128 where more than 64 are wanted, their weights are short (a quarter of LDS at most) and
+        // blocks of 128 leave at most an eighth of the last one empty ([32,28,28,96] -> 576 1x1: 21.6 -> 16.4 us; 192 channels,
+        // a third of two blocks empty: 21.7 -> 23.9 us, so those stay with blocks of 64)
+        const bool wide = g.OC > 64 && 128 * (size_t)rg.WS <= 40 * 1024 && ((g.OC + 127) / 128 * 128 - g.OC) * 8 <= g.OC;
+        const int bn = g.OC <= 32 ? 32 : (wide ? 128 : 64);
         const size_t fixed = bn * (size_t)rg.WS + bn * sizeof(ChanPrep) + 2 * bn * sizeof(int) + 16 + (size_t)(2 * rg.S + 3) / 4 * 16;
         auto need = [&](int64_t R, int64_t CW) { return fixed + (size_t)((R - 1) * g.SY + g.KY) * (size_t)row_bytes(CW); };
         int cus = 0;
@@ -2846,7 +2851,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             for (int64_t R = 1; R <= g.OH && need(R, CW) <= kMaxDynLds; R++) {
                 const int64_t ntiles = g.N * ((g.OH + R - 1) / R) * tx;
                 const int64_t per_wg = (ntiles + slots - 1) / slots;
-                for (int tm = 2; tm <= 4; tm += 2) {
+                for (int tm = 2; tm <= (bn == 128 ? 2 : 4); tm += 2) {
                     const int64_t blocks = (R * CW + 32 * tm - 1) / (32 * tm);
                     const double cost = (double)per_wg * ((double)((blocks + 7) / 8) * tm * (bn / 32) * (S * 32.0 + 400) * 2 +
                                                           (double)((R - 1) * g.SY + g.KY) * (double)RB / 64 + 1500);
@@ -2921,7 +2926,12 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         else if (per_wg > 1) VPX_ROWS_T(U8, TNV, 2, true);                                                           \
         else VPX_ROWS_T(U8, TNV, 2, false);                                                                          \
     } while (0)
-            if (in_u8 && bn == 32) VPX_ROWS(true, 1);
+            if (bn == 128) {  // (TM = 2 only: eight accumulator tiles a wave)
+                if (in_u8 && per_wg > 1) VPX_ROWS_T(true, 4, 2, true);
+                else if (in_u8) VPX_ROWS_T(true, 4, 2, false);
+                else if (per_wg > 1) VPX_ROWS_T(false, 4, 2, true);
+                else VPX_ROWS_T(false, 4, 2, false);
+            } else if (in_u8 && bn == 32) VPX_ROWS(true, 1);
             else if (in_u8) VPX_ROWS(true, 2);
             else if (bn == 32) VPX_ROWS(false, 1);
             else VPX_ROWS(false, 2);
