@@ -499,6 +499,35 @@ __device__ __forceinline__ unsigned quad_transpose_bytes(unsigned w, int lane) {
     return QuadTranspose(lane)(w);
 }
 
+// The first `count` (at most 16) bytes of `v` to a destination that is not known to be 16-byte aligned or that ends
+// early -- rows whose length is not a multiple of 16 bytes: whole 8- or 4-byte pieces where the row length and the
+// tensor's base allow (`align`: 8, 4, or less), single bytes for what is left.  (72-, 88-, 120-, 200-channel layers
+// are common in mobile networks; byte by byte their stores took three times the rest of the kernel.)
+__device__ __forceinline__ void store_tail16(uint8_t* dst, const i32x4& v, int count, int align) {
+    int e = 0;
+    if (align >= 8) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+            if (count >= 8 * h + 8) {
+                *reinterpret_cast<uint2*>(dst + 8 * h) = uint2{(unsigned)v[2 * h], (unsigned)v[2 * h + 1]};
+                e = 8 * h + 8;
+            }
+    } else if (align >= 4) {
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (count >= 4 * q + 4) {
+                *reinterpret_cast<unsigned*>(dst + 4 * q) = (unsigned)v[q];
+                e = 4 * q + 4;
+            }
+    }
+    for (; e < count; e++) dst[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+}
+// alignment (8, 4 or 1) shared by every 16-byte-chunk start of rows `row_bytes` long in a tensor at `base`
+__device__ __forceinline__ int row_align(const void* base, int64_t row_bytes) {
+    const unsigned bits = (unsigned)reinterpret_cast<uintptr_t>(base) | (unsigned)row_bytes;
+    return (bits & 7) == 0 ? 8 : ((bits & 3) == 0 ? 4 : 1);
+}
+
 constexpr int kOutStride = 288;  // bytes per row of the 256-column output staging tile in LDS
 constexpr int kGemmLdsHead = 1024;  // bytes in front of the matmul kernel's panel buffers (column sums of B)
 
@@ -833,7 +862,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                 if (vec_ok && n + 8 <= N) {
                     __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(out16 + m * N + n));
                 } else {
-                    for (int e = 0; e < 8 && n + e < N; e++) out16[m * N + n + e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+                    store_tail16(reinterpret_cast<uint8_t*>(out16 + m * N + n), v, (int)(N - n < 8 ? N - n : 8) * 2, row_align(out, 2 * N));
                 }
             }
             if (pass + 1 < PASSES) __syncthreads();  // the other half overwrites the staging tile
@@ -906,7 +935,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
         if (vec_ok && n + 16 <= N) {
             __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(out + m * N + n));
         } else {
-            for (int e = 0; e < 16 && n + e < N; e++) out[m * N + n + e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+            store_tail16(out + m * N + n, v, (int)(N - n < 16 ? N - n : 16), row_align(out, N));
         }
     }
 }
@@ -1096,7 +1125,7 @@ __device__ __forceinline__ void patch_epilogue_f16(i32x16 (&acc)[TMW], int mi0, 
         if (vec_ok && n + 8 <= OC) {
             __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
         } else {
-            for (int e = 0; e < 8 && n + e < OC; e++) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+            store_tail16(reinterpret_cast<uint8_t*>(dst), v, (OC - n < 8 ? OC - n : 8) * 2, row_align(out16, 2 * (int64_t)OC));
         }
     }
 }
@@ -1338,7 +1367,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
         if (vec_ok && n + 16 <= g.OC) {
             __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
         } else {
-            for (int e = 0; e < 16 && n + e < g.OC; e++) dst[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+            store_tail16(dst, v, (int)(g.OC - n < 16 ? g.OC - n : 16), row_align(out, g.OC));
         }
     }
 }
@@ -1552,7 +1581,7 @@ __global__ __launch_bounds__(512) void nce_conv_regw(const int8_t* __restrict__ 
             if (vec_ok && q16 + 16 <= OC) {
                 __builtin_nontemporal_store(o, reinterpret_cast<i32x4*>(dst));
             } else {
-                for (int e = 0; e < 16 && q16 + e < OC; e++) dst[e] = (uint8_t)(o[e >> 2] >> (8 * (e & 3)));
+                store_tail16(dst, o, OC - q16 < 16 ? OC - q16 : 16, row_align(out, OC));
             }
         }
     };
@@ -1900,7 +1929,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
         if (vec_ok && n + 16 <= g.OC) {
             __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
         } else {
-            for (int e = 0; e < 16 && n + e < g.OC; e++) dst[e] = (uint8_t)(v[e >> 2] >> (8 * (e & 3)));
+            store_tail16(dst, v, (int)(g.OC - n < 16 ? g.OC - n : 16), row_align(out, g.OC));
         }
     }
 }
@@ -2257,6 +2286,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
 
     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;  // no PReLU stage (or a slope of zero, which the host turns into a clamp)
     const bool vec_ok = (OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    const bool half_ok = (OC & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0;
     const uint8_t* const wl = wlds + (lane & 31) * rg.WS + half * 16;
     const int q16 = oc0 + half * 16;  // first of the 16 channels this lane stores in channel tile 0
 
@@ -2426,6 +2456,9 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                     uint8_t* dst = out0 + ((int64_t)pc[i] * OC + qc);
                     if (vec_ok && qc + 16 <= OC) {
                         __builtin_nontemporal_store(o[i], reinterpret_cast<i32x4*>(dst));
+                    } else if (half_ok && qc + 16 <= OC) {  // (rows a multiple of 8 bytes long: 72, 88, 120 channels)
+                        *reinterpret_cast<uint2*>(dst) = uint2{(unsigned)o[i][0], (unsigned)o[i][1]};
+                        *reinterpret_cast<uint2*>(dst + 8) = uint2{(unsigned)o[i][2], (unsigned)o[i][3]};
                     } else {
                         for (int e = 0; e < 16 && qc + e < OC; e++) dst[e] = (uint8_t)(o[i][e >> 2] >> (8 * (e & 3)));
                     }
