@@ -14,8 +14,9 @@ def dev_t(a, dev):
 
 
 def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0, zp_out=0, strides=(1, 1),
-             pads=(0, 0, 0, 0), out_signed=False, mode=None, force=None, rows=None, out_f16=False):
-    """pads = (left, right, top, bottom).  Returns (gpu_out, oracle_out, kernel_name)."""
+             pads=(0, 0, 0, 0), out_signed=False, mode=None, force=None, rows=None, out_f16=False, out_offset=None):
+    """pads = (left, right, top, bottom).  Returns (gpu_out, oracle_out, kernel_name).  With out_offset the output tensor
+    starts that many elements into a larger allocation, whose elements either side of it must come back untouched."""
     import torch
     OC, KY, KX, IC = w.shape
     wt = rt.make_weights_table(mults, shifts, bias, KY * KX * IC)
@@ -28,7 +29,12 @@ def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0,
     N, H, W, _ = inp.shape
     OH = (H + pads[2] + pads[3] - KY) // strides[0] + 1
     OW = (W + pads[0] + pads[1] - KX) // strides[1] + 1
-    out = torch.full((N, OH, OW, OC), 77, dtype=torch.float16 if out_f16 else (torch.int8 if out_signed else torch.uint8), device=dev)
+    odt = torch.float16 if out_f16 else (torch.int8 if out_signed else torch.uint8)
+    if out_offset is None:
+        out = torch.full((N, OH, OW, OC), 77, dtype=odt, device=dev)
+    else:
+        whole = torch.full((out_offset + N * OH * OW * OC + 64,), 77, dtype=odt, device=dev)
+        out = whole[out_offset:out_offset + N * OH * OW * OC].view(N, OH, OW, OC)
     if force in ("regw", "tile", "stream"):  # the LDS-patch kernels only, starting the choice at this one
         rt.set_tuning("VPX_CONV_KERNEL", force)
         rt.set_tuning("VPX_NCE_KERNEL", "conv")
@@ -44,6 +50,8 @@ def run_task(rt, orc, dev, inp, w, mults, shifts, bias, ppe_kw, zp_in=0, zp_w=0,
     want = orc.nce_conv(inp, w, wt, op, zp_in=zp_in, zp_w=zp_w, strides=strides,
                         pads=(pads[2], pads[0], pads[3], pads[1]), out_signed=out_signed, rows=rows, out_f16=out_f16)
     got = out.cpu().numpy()
+    if out_offset is not None:
+        assert bool((whole[:out_offset] == 77).all()) and bool((whole[out_offset + out.numel():] == 77).all()), "wrote outside the output"
     return (got.view(np.uint16) if out_f16 else got), want, rt.nce_last_kernel()
 
 
@@ -609,6 +617,35 @@ def test_f16_output_conv_random_geometries(rt, orc, dev, seed):
         got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=zp_in, zp_w=zp_w, strides=(SY, SX),
                                    pads=(pl, pr, pt, pb), mode=getattr(rt, "PPE_" + mode), out_f16=True)
         assert np.array_equal(got, want), "%s (%s): %d mismatches" % (what, name, int((got != want).sum()))
+
+
+@pytest.mark.parametrize("out_f16", [False, True])
+@pytest.mark.parametrize("geom,kernel,force", [
+    (dict(N=2, H=20, W=24, IC=64, KY=1, KX=1), "nce_gemm_mfma", None),
+    (dict(N=2, H=20, W=24, IC=64, KY=3, KX=3), "nce_conv_regw", "regw"),
+    (dict(N=2, H=20, W=24, IC=128, KY=3, KX=3), "nce_conv_tile", None),
+    (dict(N=3, H=7, W=7, IC=256, KY=3, KX=3), "nce_conv_stream", None),       # the K steps split over the waves
+    (dict(N=1, H=30, W=33, IC=192, KY=3, KX=3), "nce_conv_stream", None),     # one tile per wave
+    (dict(N=2, H=20, W=24, IC=48, KY=1, KX=1), "nce_conv_rows16", None),
+    (dict(N=2, H=20, W=24, IC=16, KY=3, KX=3), "nce_conv_rows16", None),
+    (dict(N=1, H=12, W=10, IC=64, KY=3, KX=3), "nce_conv_mfma", "gather"),
+    (dict(N=1, H=12, W=10, IC=48, KY=3, KX=3), "nce_conv_mfma16", "gather"),
+])
+def test_output_rows_that_are_not_whole_16_byte_pieces(rt, orc, dev, geom, kernel, force, out_f16):
+    """Channel counts whose output rows are a multiple of 8, 4, 2 or 1 bytes only, in tensors that start 0, 8, 4 or an odd
+    number of bytes past an aligned address: the kernels store such rows in the largest pieces row length and base allow,
+    and the elements either side of the tensor stay as they were."""
+    rng = np.random.default_rng(640 + geom["IC"] + geom["KY"])
+    pads = (1, 1, 1, 1) if geom["KY"] > 1 else (0, 0, 0, 0)
+    for OC, offset in ((72, 0), (72, 8), (72, 4), (100, 0), (100, 4), (120, 16), (200, 8), (36, 0), (70, 2), (37, 1), (72, 3), (88, 0)):
+        if out_f16:
+            offset = (offset + 1) // 2 if offset % 2 == 0 else offset  # elements of two bytes: 0, 8, 4, 2 bytes and odd element counts
+        inp, w, mults, shifts, bias = rand_case(rng, OC=OC, shift_lo=14, shift_hi=22, **geom)
+        kw = dict(F16_NONE if out_f16 else U8, lrelu_mult=1638, lrelu_shift=14)
+        got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, kw, zp_in=128, zp_out=0 if out_f16 else 3, pads=pads,
+                                   mode=rt.PPE_LPRELU, force=force, out_f16=out_f16, out_offset=offset)
+        assert name == ("nce_conv_tile" if out_f16 and kernel == "nce_conv_regw" else kernel)  # (no fp16 output from that one)
+        assert np.array_equal(got, want), "%s OC=%d offset=%d: %d mismatches" % (name, OC, offset, int((got != want).sum()))
 
 
 def test_f16_output_scale_is_weight_scale_times_input_scale(rt, orc, dev):
