@@ -2994,11 +2994,23 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         if (pf.lo > pf.hi) pf.lo = pf.hi;  // inverted window: max-then-min always ends at the upper bound
 
         if (use_gemm) {
-            // 256 x 256 tiles when they fill the chip and K is long enough to amortise their prologue and epilogue;
-            // else 128 x 128 (four times as many, two workgroups per CU): [25088 x 512 x 128] 14.1 -> 7.8 us,
-            // [100352 x 256 x 128] 23.8 -> 14.4 us, [512 x 4096 x 4096] 43 -> 24 us.  VPX_GEMM_TILE=128|256 overrides.
+            // 256 x 256 tiles (one workgroup per CU) or 128 x 128 (four times as many, two workgroups per CU): whichever
+            // leaves less of the chip idle, counting the padding of edge tiles and the empty part of the last round of
+            // workgroups; at equal use the large tile is about an eighth faster from K = 256 on (half the operand traffic per
+            // MFMA), about equal at K = 128 and slower at K = 64 (all epilogue).  [25088 x 512 x 128] 14.1 -> 7.8 us,
+            // [100352 x 256 x 128] 23.8 -> 14.4 us, [512 x 4096 x 4096] 43 -> 24 us with the small tile; [25088 x 256 x 512]
+            // 14.3 -> 11.4 us, [12544 x 1024 x 1024] 26.5 -> 21.1 us with the large one.  VPX_GEMM_TILE=128|256 overrides.
+            int cus_gemm = 0;
+            rc = device_compute_units(&cus_gemm);
+            if (rc) return rc;
+            const int64_t t256 = gemm_tiles * G, t128 = ((Mtot + 127) / 128) * ((g.OC + 127) / 128) * G;
+            const double work = (double)Mtot * (double)g.OC * (double)G;
+            const double use256 = work / ((double)((t256 + cus_gemm - 1) / cus_gemm) * cus_gemm * 65536.0);
+            const double use128 = work / ((double)((t128 + 2 * cus_gemm - 1) / (2 * cus_gemm)) * 2 * cus_gemm * 16384.0);
+            const bool large = g.IC >= 256 ? use256 * 1.12 > use128
+                                           : (g.IC >= 128 && t256 * 10 >= cus_gemm * 7 && t256 <= cus_gemm && use256 * 1.03 > use128);
             const int tile_knob = knobs.gemm_tile.load();
-            const int tile = tile_knob ? tile_knob : (gemm_tiles < 200 || g.IC <= 256 ? 128 : 256);
+            const int tile = tile_knob ? tile_knob : (large ? 256 : 128);
             const int tiles_m = (int)((Mtot + tile - 1) / tile), tiles_n = (int)((g.OC + tile - 1) / tile);
             const int per_xcd = (tiles_m * tiles_n + 7) / 8;
             // Eight waves (two per SIMD: one wave's reads and loads issue under the other's MFMAs) win at every K
