@@ -102,7 +102,7 @@ def test_conv_paths(rt, orc, dev, geom, force):
     other = gather if g["IC"] % 64 == 0 else "nce_conv_rows16"
     # (a 1x1 layer without padding is a matmul, with or without a stride, unless its few channels suit the 64-wide tiles better)
     M = g["N"] * ((g["H"] - 1) // strides[0] + 1) * ((g["W"] - 1) // strides[1] + 1)
-    matmul = (g["KY"], g["KX"]) == (1, 1) and pads == (0, 0, 0, 0) and g["IC"] % 64 == 0 and (g["OC"] > 64 or M < 1024)
+    matmul = (g["KY"], g["KX"]) == (1, 1) and pads == (0, 0, 0, 0) and g["IC"] % 64 == 0 and (g["OC"] > 64 or (g["OC"] > 48 and g["IC"] >= 192) or M < 1024)
     expect = {None: "nce_gemm_mfma" if matmul else ("nce_conv_tile" if tile else ("nce_conv_stream" if lds else other)),
               "regw": patch_kernel(g) if tile else ("nce_conv_stream" if lds else other),
               "stream": "nce_conv_stream" if lds else other,

@@ -2772,10 +2772,12 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const bool allow_lds = allow_gemm || force == NCE_CONV;
     const bool allow_mfma = allow_lds || force == NCE_GATHER;
 
-    // A 256-column matmul tile wastes three quarters of its MFMAs on 64 output channels: such 1x1 layers go
-    // to the convolution kernels, whose tiles are 64 channels wide (measured 7 us against 18 us at [100352 x 64 x 64]).
+    // A matmul tile wastes half (128 columns) or three quarters of its MFMAs on 64 output channels: such 1x1 layers go
+    // to the convolution kernels, whose tiles are 64 channels wide (7.5 us against 9.5 us at [100352 x 64 x 64]), unless K
+    // is long enough for the matmul kernel's deeper pipeline to make up for it (from 192 channels on: [100352 x 192 x 64]
+    // 13.8 -> 11.1 us, [25088 x 512 x 64] 8.6 -> 7.5 us, [6272 x 1024 x 64] 11.1 -> 9.0 us; 128 channels: even).
     const int64_t gemm_tiles = ((Mtot + 255) / 256) * ((g.OC + 255) / 256);
-    const bool use_gemm = allow_gemm && (is_gemm || is_strided_gemm) && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || Mtot < 1024);
+    const bool use_gemm = allow_gemm && (is_gemm || is_strided_gemm) && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || (g.OC > 48 && g.IC >= 192) || Mtot < 1024);
     // VPU.NCE.MatMul's groups: one launch of the matmul kernel when it serves the shape (the preparation passes then
     // walk all groups' weights / activations as one tensor), else one task after the other on the stream.
     const int64_t G = t.groups > 1 ? t.groups : 1;
