@@ -3009,8 +3009,11 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             const double work = (double)Mtot * (double)g.OC * (double)G;
             const double use256 = work / ((double)((t256 + cus_gemm - 1) / cus_gemm) * cus_gemm * 65536.0);
             const double use128 = work / ((double)((t128 + 2 * cus_gemm - 1) / (2 * cus_gemm)) * 2 * cus_gemm * 16384.0);
-            const bool large = g.IC >= 256 ? use256 * 1.12 > use128
-                                           : (g.IC >= 128 && t256 * 10 >= cus_gemm * 7 && t256 <= cus_gemm && use256 * 1.03 > use128);
+            // (fp16 outputs: the large tile's epilogue leaves in two passes and costs more than its main loop saves up to
+            // K = 1024 -- [32768 x 512 x 512] 26.6 us small, 30.4 us large; [32768 x 2048 x 512] 58.4 and 54.8)
+            const bool large = out_f16 ? (g.IC >= 2048 && use256 * 1.06 > use128)
+                               : g.IC >= 256 ? use256 * 1.12 > use128
+                                             : (g.IC >= 128 && t256 * 10 >= cus_gemm * 7 && t256 <= cus_gemm && use256 * 1.03 > use128);
             const int tile_knob = knobs.gemm_tile.load();
             const int tile = tile_knob ? tile_knob : (large ? 256 : 128);
             const int tiles_m = (int)((Mtot + tile - 1) / tile), tiles_n = (int)((g.OC + tile - 1) / tile);
