@@ -94,7 +94,10 @@ VPX_API int vpx_sw_kernel_launch_noalloc(const char* entry, const void* params, 
  * a capture, or to keep hipMalloc out of a serving loop).  vpx_workspace_release waits for the stream, then frees
  * its block, the blocks it outgrew and the per-axis tables cached for it; the next launch allocates afresh.
  * Blocks are keyed by the stream HANDLE: release before destroying a stream (a new stream may get the same
- * handle), and do not run one handle's work concurrently from several threads' per-thread streams. */
+ * handle), and do not run one handle's work concurrently from several threads' per-thread streams.  A graph captured
+ * on a stream records the addresses of that stream's block, counter area and cached tables: destroy such graphs
+ * before releasing the stream's workspace (and replay them on no other stream).  Every block is freed even when one
+ * hipFree fails; the first failure is what the call returns. */
 VPX_API int vpx_workspace_reserve(void* stream, size_t bytes);
 VPX_API int vpx_workspace_release(void* stream);
 
@@ -119,6 +122,7 @@ VPX_API const char* vpx_sw_kernel_name(uint32_t i);
  *       (src/vpux_compiler/src/NPU37XX/dialect/VPU/impl/nce_sparsity_converters.cpp:14-41);
  *       words 0 and 1 (weight / sparsity pointers) are NPU addresses and are ignored
  *   output  NHWC  [N][OH][OW][OC] u8 or i8
+ * input and output may be strided views of larger tensors (input_strides / output_strides below).
  * A matmul A[M][K] x B[N][K] -> [M][N] is the task N=1, H=M, W=1, IC=K, OC=N, 1x1 kernel.
  *
  * task_type ELTWISE (the quantized residual add of a network): `weights` is the second input,
@@ -196,6 +200,22 @@ typedef struct vpx_nce_task_t {
      * pointers.  0 and 1 both mean a single task.  A matmul the MFMA matmul kernel serves is one launch for all
      * groups (the group on the grid's second dimension). */
     int32_t groups;
+    /* Operand strides in ELEMENTS, in the order N, H, W, C: the strides of the operand's memref
+     * (src/vpux_compiler/tblgen/vpux/compiler/dialect/VPUIP/ops.td:651-700).  The NPU writes a task's output into the
+     * buffer its bit strides describe -- the ODU's te_dim_z is stride_x / stride_z, the channel pitch of the BUFFER, not
+     * the task's channel count (src/vpux_compiler/src/dialect/VPUMI37XX/ops/external/runtime_dpu_parser_imports.cpp.inc:
+     * 1031-1090) -- and reads its input out of the parent tensor's dimensions (:850-852); that is how the compiler
+     * elides Concat (a task writes channels [c0, c0 + OC) of a wider tensor) and tiles a layer over H or W (a task
+     * reads a window of a larger tensor).  Here the pointer names the operand's first element and the strides say how
+     * far apart its images, rows and pixels lie.  All four zero = dense NHWC (the default: every field an existing
+     * caller leaves zeroed).  Otherwise C must be 1 and the others must keep the operand's elements apart, outermost
+     * largest (W >= channels, H >= (width - 1) * W + channels, N likewise).  `weights_strides` describes the second
+     * input of an ELTWISE task; the weights of a CONV task are always dense.  Strides need groups <= 1.
+     * The MFMA kernels read 16 bytes at a time: an input whose base address or strides are not multiples of 16 bytes
+     * runs on the general kernel (correct, slow).  Outputs may sit anywhere. */
+    int64_t input_strides[4];
+    int64_t weights_strides[4];
+    int64_t output_strides[4];
 } vpx_nce_task_t;
 
 VPX_API int vpx_nce_task(const vpx_nce_task_t* task, void* stream);

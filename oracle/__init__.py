@@ -28,7 +28,8 @@ class _PPE(C.Structure):
 class _Conv(C.Structure):
     _fields_ = [(n, C.c_int64) for n in ("N", "H", "W", "IC", "OC", "KY", "KX", "stride_y", "stride_x", "pad_top",
                                           "pad_left", "pad_bottom", "pad_right")] + \
-               [(n, C.c_int32) for n in ("in_signed", "w_signed", "out_signed", "zp_in", "zp_w")] + [("ppe", _PPE)]
+               [(n, C.c_int32) for n in ("in_signed", "w_signed", "out_signed", "zp_in", "zp_w")] + [("ppe", _PPE)] + \
+               [("in_strides", C.c_int64 * 3), ("out_strides", C.c_int64 * 3)]
 
 
 _lib = None
@@ -379,12 +380,19 @@ def pack_clamp_f16(lo, hi):
     return v - (1 << 32) if v & 0x80000000 else v
 
 
+def _nhw_strides(x):
+    """N, H, W strides in elements of a 4-D array whose channels are contiguous (a view of a larger tensor)."""
+    assert x.ndim == 4 and (x.shape[3] == 1 or x.strides[3] == x.itemsize)
+    return tuple(int(v) // x.itemsize for v in x.strides[:3])
+
+
 def nce_conv(inp, w, wt, p, zp_in=0, zp_w=0, strides=(1, 1), pads=(0, 0, 0, 0), out_signed=False, rows=None,
-             want_acc=False, out_f16=False):
+             want_acc=False, out_f16=False, out=None):
     """inp NHWC int8/uint8, w [OC,KY,KX,IC] int8/uint8, wt [OC,4] int32; pads = (top,left,bottom,right).
 
-    rows=(row0,nrows) computes only those flattened output rows (the rest of the result is zero)."""
-    inp = np.ascontiguousarray(inp)
+    rows=(row0,nrows) computes only those flattened output rows (the rest of the result is zero).
+    inp may be a view of a larger array (channels contiguous): it is read in place through its strides.  `out`, when
+    given, is the array to write, likewise a view if wanted; elements of its parent outside the view are not touched."""
     w = np.ascontiguousarray(w)
     wt = np.ascontiguousarray(wt, dtype=np.int32)
     N, H, W, IC = inp.shape
@@ -394,7 +402,17 @@ def nce_conv(inp, w, wt, p, zp_in=0, zp_w=0, strides=(1, 1), pads=(0, 0, 0, 0), 
               int(inp.dtype == np.int8), int(w.dtype == np.int8), 2 if out_f16 else int(out_signed), zp_in, zp_w, p)
     OH = (H + pads[0] + pads[2] - KY) // strides[0] + 1
     OW = (W + pads[1] + pads[3] - KX) // strides[1] + 1
-    out = np.zeros((N, OH, OW, OC), dtype=np.uint16 if out_f16 else (np.int8 if out_signed else np.uint8))
+    odt = np.uint16 if out_f16 else (np.int8 if out_signed else np.uint8)
+    if not inp.flags.c_contiguous:
+        for i, v in enumerate(_nhw_strides(inp)):
+            d.in_strides[i] = v
+    if out is None:
+        out = np.zeros((N, OH, OW, OC), dtype=odt)
+    else:
+        assert out.shape == (N, OH, OW, OC) and out.dtype == odt
+        if not out.flags.c_contiguous:
+            for i, v in enumerate(_nhw_strides(out)):
+                d.out_strides[i] = v
     acc = np.zeros((N, OH, OW, OC), dtype=np.int32) if want_acc else None
     row0, nrows = rows if rows is not None else (0, N * OH * OW)
     lib().orc_nce_conv_rows(C.byref(d), _p(inp), _p(w), _p(wt), _p(out), _p(acc) if want_acc else None,
@@ -402,11 +420,22 @@ def nce_conv(inp, w, wt, p, zp_in=0, zp_w=0, strides=(1, 1), pads=(0, 0, 0, 0), 
     return (out, acc) if want_acc else out
 
 
-def nce_eltwise(a, b, p, zp_a, zp_b, mult_a, mult_b, out_mult, out_shift, subtract=False, out_signed=False, out_f16=False):
+def nce_eltwise(a, b, p, zp_a, zp_b, mult_a, mult_b, out_mult, out_shift, subtract=False, out_signed=False, out_f16=False,
+                out=None):
     """Quantized add / subtract of two 8-bit tensors of the same shape (the NCE ELTWISE task); out_f16: fp16 bit patterns."""
-    a = np.ascontiguousarray(a)
-    b = np.ascontiguousarray(b)
     assert a.shape == b.shape
+    if out is not None or not (a.flags.c_contiguous and b.flags.c_contiguous):
+        # views of larger arrays (channels contiguous), read and written in place
+        odt = np.uint16 if out_f16 else (np.int8 if out_signed else np.uint8)
+        if out is None:
+            out = np.zeros(a.shape, dtype=odt)
+        assert out.shape == a.shape and out.dtype == odt and a.ndim == 4
+        lib().orc_nce_eltwise_views(_p(a), C.c_int(int(a.dtype == np.int8)), _p(b), C.c_int(int(b.dtype == np.int8)), _p(out),
+                                    C.c_int(2 if out_f16 else int(out_signed)), _i64(a.shape), _i64(_nhw_strides(a)),
+                                    _i64(_nhw_strides(b)), _i64(_nhw_strides(out)), C.c_int32(zp_a), C.c_int32(zp_b),
+                                    C.c_int32(mult_a), C.c_int32(mult_b), C.c_int(int(subtract)), C.c_int32(out_mult),
+                                    C.c_int32(out_shift), C.byref(p))
+        return out
     if out_f16:
         out = np.zeros(a.shape, dtype=np.uint16)
         lib().orc_nce_eltwise_f16(_p(a), C.c_int(int(a.dtype == np.int8)), _p(b), C.c_int(int(b.dtype == np.int8)), _p(out),

@@ -525,11 +525,19 @@ void orc_nce_conv_rows(const orc_conv_t* d, const void* in, const void* w, const
     const int64_t OW = (d->W + d->pad_left + d->pad_right - d->KX) / d->stride_x + 1;
     const int64_t IC = d->IC, OC = d->OC;
     const int fast = d->in_signed == 0 && d->w_signed == 1;
+    /* dense unless strides are given */
+    const int in_view = (d->in_strides[0] | d->in_strides[1] | d->in_strides[2]) != 0;
+    const int out_view = (d->out_strides[0] | d->out_strides[1] | d->out_strides[2]) != 0;
+    const int64_t isw = in_view ? d->in_strides[2] : IC, ish = in_view ? d->in_strides[1] : d->W * IC,
+                  isn = in_view ? d->in_strides[0] : d->H * d->W * IC;
+    const int64_t osw = out_view ? d->out_strides[2] : OC, osh = out_view ? d->out_strides[1] : OW * OC,
+                  osn = out_view ? d->out_strides[0] : OH * OW * OC;
 #pragma omp parallel for schedule(dynamic, 16)
     for (int64_t row = row0; row < row0 + nrows; row++) {
         const int64_t n = row / (OH * OW);
         const int64_t oy = (row / OW) % OH;
         const int64_t ox = row % OW;
+        const int64_t obase = n * osn + oy * osh + ox * osw;
         for (int64_t oc = 0; oc < OC; oc++) {
             int32_t acc = 0;
             for (int64_t ky = 0; ky < d->KY; ky++) {
@@ -538,7 +546,7 @@ void orc_nce_conv_rows(const orc_conv_t* d, const void* in, const void* w, const
                 for (int64_t kx = 0; kx < d->KX; kx++) {
                     const int64_t ix = ox * d->stride_x + kx - d->pad_left;
                     if (ix < 0 || ix >= d->W) continue;
-                    const int64_t ibase = ((n * d->H + iy) * d->W + ix) * IC;
+                    const int64_t ibase = n * isn + iy * ish + ix * isw;
                     const int64_t wbase = ((oc * d->KY + ky) * d->KX + kx) * IC;
                     int32_t part = 0;
                     if (fast) {
@@ -563,15 +571,15 @@ void orc_nce_conv_rows(const orc_conv_t* d, const void* in, const void* w, const
             orc_wt_unpack_scale(wt[oc * 4 + 2], &mult, &shift);
             if (acc_out) acc_out[row * OC + oc] = acc;
             if (d->out_signed == 2) { /* fp16 output */
-                ((uint16_t*)out)[row * OC + oc] = orc_ppe_requant_f16(acc, wt[oc * 4 + 3], mult, shift, &d->ppe);
+                ((uint16_t*)out)[obase + oc] = orc_ppe_requant_f16(acc, wt[oc * 4 + 3], mult, shift, &d->ppe);
                 continue;
             }
             const int32_t r = orc_ppe_requant(acc, wt[oc * 4 + 3], mult, shift, &d->ppe);
             /* convert: saturate to the storage type */
             if (d->out_signed)
-                ((int8_t*)out)[row * OC + oc] = (int8_t)(r < -128 ? -128 : (r > 127 ? 127 : r));
+                ((int8_t*)out)[obase + oc] = (int8_t)(r < -128 ? -128 : (r > 127 ? 127 : r));
             else
-                ((uint8_t*)out)[row * OC + oc] = (uint8_t)(r < 0 ? 0 : (r > 255 ? 255 : r));
+                ((uint8_t*)out)[obase + oc] = (uint8_t)(r < 0 ? 0 : (r > 255 ? 255 : r));
         }
     }
 }
@@ -613,5 +621,27 @@ void orc_nce_eltwise_f16(const void* a, int a_signed, const void* b, int b_signe
         const int32_t vb = (b_signed ? (int32_t)(int8_t)pb[i] : (int32_t)pb[i]) - zp_b;
         const int32_t acc = va * mult_a + (subtract ? -1 : 1) * vb * mult_b;
         out[i] = orc_ppe_requant_f16(acc, 0, out_mult, out_shift, ppe);
+    }
+}
+
+/* The two eltwise functions above on views of larger tensors: one pixel's channels at a time, through the same
+ * per-value functions. */
+void orc_nce_eltwise_views(const void* a, int a_signed, const void* b, int b_signed, void* out, int out_kind,
+                           const int64_t dims[4], const int64_t a_strides[3], const int64_t b_strides[3],
+                           const int64_t out_strides[3], int32_t zp_a, int32_t zp_b, int32_t mult_a, int32_t mult_b,
+                           int subtract, int32_t out_mult, int32_t out_shift, const orc_ppe_t* ppe) {
+    const int64_t N = dims[0], H = dims[1], W = dims[2], Cn = dims[3];
+#pragma omp parallel for schedule(static)
+    for (int64_t pixel = 0; pixel < N * H * W; pixel++) {
+        const int64_t n = pixel / (H * W), y = (pixel / W) % H, x = pixel % W;
+        const uint8_t* pa = (const uint8_t*)a + n * a_strides[0] + y * a_strides[1] + x * a_strides[2];
+        const uint8_t* pb = (const uint8_t*)b + n * b_strides[0] + y * b_strides[1] + x * b_strides[2];
+        const int64_t o = n * out_strides[0] + y * out_strides[1] + x * out_strides[2];
+        if (out_kind == 2)
+            orc_nce_eltwise_f16(pa, a_signed, pb, b_signed, (uint16_t*)out + o, Cn, zp_a, zp_b, mult_a, mult_b, subtract, out_mult,
+                                out_shift, ppe);
+        else
+            orc_nce_eltwise(pa, a_signed, pb, b_signed, (uint8_t*)out + o, out_kind, Cn, zp_a, zp_b, mult_a, mult_b, subtract,
+                            out_mult, out_shift, ppe);
     }
 }

@@ -126,6 +126,12 @@ typedef struct {
     int32_t in_signed, w_signed, out_signed; /* out_signed: 0 = u8, 1 = i8, 2 = fp16 (16-bit output elements) */
     int32_t zp_in, zp_w;
     orc_ppe_t ppe;
+    /* Strides of the input and the output in elements, for images, rows and pixels (N, H, W; a pixel's channels are
+     * contiguous): the operands of a task may be views of larger tensors, as the NPU's are
+     * (VPUMI37XX/ops/external/runtime_dpu_parser_imports.cpp.inc:850-852, 1031-1090).  All three zero = dense NHWC.
+     * acc_out stays dense. */
+    int64_t in_strides[3];
+    int64_t out_strides[3];
 } orc_conv_t;
 void orc_nce_conv(const orc_conv_t* d, const void* in, const void* w, const int32_t* wt, void* out, int32_t* acc_out);
 /* only rows [row0,row0+nrows) of the flattened N*OH*OW output are produced (into out + row0*OC) */
@@ -143,6 +149,13 @@ void orc_nce_eltwise(const void* a, int a_signed, const void* b, int b_signed, v
 void orc_nce_eltwise_f16(const void* a, int a_signed, const void* b, int b_signed, uint16_t* out, int64_t n, int32_t zp_a,
                          int32_t zp_b, int32_t mult_a, int32_t mult_b, int subtract, int32_t out_mult, int32_t out_shift,
                          const orc_ppe_t* ppe);
+
+/* Both on views of larger tensors: dims = {N, H, W, C}; strides of a, b and out in elements for N, H, W (channels
+ * contiguous).  out_kind: 0 = u8, 1 = i8, 2 = fp16 (as orc_conv_t.out_signed). */
+void orc_nce_eltwise_views(const void* a, int a_signed, const void* b, int b_signed, void* out, int out_kind,
+                           const int64_t dims[4], const int64_t a_strides[3], const int64_t b_strides[3],
+                           const int64_t out_strides[3], int32_t zp_a, int32_t zp_b, int32_t mult_a, int32_t mult_b,
+                           int subtract, int32_t out_mult, int32_t out_shift, const orc_ppe_t* ppe);
 
 int orc_num_threads(void);
 void orc_set_num_threads(int n);

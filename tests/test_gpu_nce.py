@@ -482,6 +482,23 @@ def test_matmul_gemm_path(rt, orc, dev, gemm_waves, M, K, N):
         assert np.array_equal(got, want), "M=%d K=%d N=%d zp=%d: %d mismatches" % (M, K, N, zp, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("M,K,N", [(300, 128, 520), (513, 256, 77)])
+def test_matmul_gemm_path_f16_output(rt, orc, dev, gemm_waves, M, K, N):
+    """The wave-count knob does not reach the fp16-output matmul, which exists with eight waves per large tile only."""
+    rng = np.random.default_rng(71 + M)
+    for in_u8, zp in ((False, 3), (True, 128)):
+        a = rng.integers(0, 256, (M, K), dtype=np.uint8) if in_u8 else rng.integers(-128, 128, (M, K)).astype(np.int8)
+        b = rng.integers(-127, 128, (N, K)).astype(np.int8)
+        mults = rng.integers(2 ** 14, 2 ** 15, N)
+        shifts = rng.integers(18, 24, N)
+        bias = rng.integers(-2 ** 15, 2 ** 15, N).astype(np.int32)
+        kw = dict(F16_NONE, lrelu_mult=1638, lrelu_shift=14)
+        got, want, name = run_task(rt, orc, dev, a.reshape(1, M, 1, K), b.reshape(N, 1, 1, K), mults, shifts, bias, kw,
+                                   zp_in=zp, mode=rt.PPE_LPRELU, out_f16=True)
+        assert name == "nce_gemm_mfma"
+        assert np.array_equal(got, want), "M=%d K=%d N=%d zp=%d: %d mismatches" % (M, K, N, zp, int((got != want).sum()))
+
+
 @pytest.mark.parametrize("mode", ["NOOP", "LRELU", "LRELUX", "LPRELU"])
 def test_ppe_modes_and_rounding_edges(rt, orc, dev, mode):
     """Accumulators chosen to land on ties, on both signs, with shifts from 0 to 40 and output zero points."""

@@ -907,6 +907,37 @@ def test_mvn_one_launch_kernel_and_its_fallback(rt, orc, dev, shape):
     assert_close_f16_mvn(two, want, orc, "two launches %s" % (shape,))
 
 
+@pytest.mark.parametrize("shape", [(4, 64, 64, 64), (3, 5, 40, 104), (2, 3, 8, 8), (2, 70, 112, 112)])
+@pytest.mark.parametrize("fused", [None, "nowait"])
+def test_mvn_in_place(rt, orc, dev, shape, fused):
+    """Output tensor = input tensor.  Long groups then leave the one-launch kernel alone (a workgroup that recomputes
+    its group's moments would read slices other workgroups have already normalised): same bits as out of place."""
+    import torch
+    rng = np.random.default_rng(sum(shape) + 5)
+    xb = orc.f32_to_f16((rng.uniform(-8, 8, shape) + rng.normal(0, 2, (1, shape[1], 1, 1))).astype(np.float32))
+    rt.set_tuning("VPX_MVN_FUSED", "off")
+    try:
+        apart = _mvn(rt, dev, xb, True, True, 1e-9)
+        rt.set_tuning("VPX_MVN_FUSED", fused)
+        x = to_dev(xb, dev, True)
+        rt.mvn(x, x, True, True, 1e-9)
+        torch.cuda.synchronize()
+    finally:
+        rt.set_tuning("VPX_MVN_FUSED", None)
+    assert np.array_equal(f16_bits(x), apart)
+    assert_close_f16_mvn(apart, orc.mvn_f16(xb, True, True, 1e-9), orc, "in place %s" % (shape,))
+
+
+def test_mvn_rejects_partial_overlap(rt, dev):
+    import torch
+    buf = torch.zeros((2 * 4 * 64 * 64 + 64,), dtype=torch.float16, device=dev)
+    x = buf[:2 * 4 * 64 * 64].view(2, 4, 64, 64)
+    y = buf[64:].view(2, 4, 64, 64)
+    with pytest.raises(rt.VpxError) as e:
+        rt.mvn(x, y, True, True, 1e-9)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+
+
 def test_mvn_large_offset_and_constant(rt, orc, dev):
     rng = np.random.default_rng(42)
     x = (1000.0 + rng.normal(0, 1, (2, 4, 64, 64))).astype(np.float32)  # mean >> spread

@@ -440,6 +440,42 @@ def test_nce_conv_against_brute_force(orc):
     assert np.array_equal(part[2:6], out[2:6])
 
 
+def test_nce_operands_as_views_of_larger_tensors(orc):
+    """Strided operands: the result on views equals the dense result on packed copies, and nothing outside the
+    output view is written."""
+    rng = np.random.default_rng(9)
+    N, H, W, IC, OC, KY, KX = 2, 7, 6, 16, 5, 3, 3
+    parent = rng.integers(0, 256, (N, H + 3, W + 4, IC + 7), dtype=np.uint8)
+    inp = parent[:, 2:2 + H, 1:1 + W, 3:3 + IC]
+    w = rng.integers(-127, 128, (OC, KY, KX, IC)).astype(np.int8)
+    wt = orc.make_weights_table(rng.integers(2 ** 14, 2 ** 15, OC), rng.integers(12, 16, OC), rng.integers(-2 ** 15, 2 ** 15, OC).astype(np.int32),
+                                KY * KX * IC)
+    p = orc.ppe(1638, 14, 2, 0, 255)
+    for out_f16 in (False, True):
+        dense = orc.nce_conv(np.ascontiguousarray(inp), w, wt, p, zp_in=128, strides=(2, 1), pads=(1, 1, 0, 1), out_f16=out_f16)
+        oparent = np.full((N, dense.shape[1] + 2, dense.shape[2] + 3, OC + 9), 99, dtype=dense.dtype)
+        oview = oparent[:, 1:1 + dense.shape[1], 2:2 + dense.shape[2], 4:4 + OC]
+        got = orc.nce_conv(inp, w, wt, p, zp_in=128, strides=(2, 1), pads=(1, 1, 0, 1), out_f16=out_f16, out=oview)
+        assert got is oview and np.array_equal(oview, dense)
+        mask = np.ones(oparent.shape, bool)
+        mask[:, 1:1 + dense.shape[1], 2:2 + dense.shape[2], 4:4 + OC] = False
+        assert (oparent[mask] == 99).all()
+    # eltwise
+    a = parent[:, 0:H, 0:W, 0:IC].view(np.int8)
+    b = parent[:, 1:1 + H, 2:2 + W, 5:5 + IC]
+    pe = orc.ppe(1638, 14, 3, -128, 127)
+    for out_f16 in (False, True):
+        dense = orc.nce_eltwise(np.ascontiguousarray(a), np.ascontiguousarray(b), pe, 3, 120, 11000, 9000, 17000, 28, subtract=True,
+                                out_signed=True, out_f16=out_f16)
+        oparent = np.full((N, H + 1, W + 2, IC + 3), 99, dtype=dense.dtype)
+        oview = oparent[:, 1:, 1:1 + W, 2:2 + IC]
+        orc.nce_eltwise(a, b, pe, 3, 120, 11000, 9000, 17000, 28, subtract=True, out_signed=True, out_f16=out_f16, out=oview)
+        assert np.array_equal(oview, dense)
+        mask = np.ones(oparent.shape, bool)
+        mask[:, 1:, 1:1 + W, 2:2 + IC] = False
+        assert (oparent[mask] == 99).all()
+
+
 def test_nce_eltwise_against_exact_integers_and_real_arithmetic(orc):
     """The eltwise restatement against Python integers (round half even with fractions) and, loosely,
     against the real-valued sum it approximates; multipliers from the reference's golden case

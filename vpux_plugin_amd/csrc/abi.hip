@@ -183,18 +183,27 @@ int workspace_release(hipStream_t stream) {
     VPX_HIP_CHECK(hipStreamSynchronize(stream));
     int dev = 0;
     VPX_HIP_CHECK(hipGetDevice(&dev));
+    // Everything the stream holds is freed whatever an individual hipFree returns; the first failure is reported.
+    hipError_t first = hipSuccess;
+    const auto release = [&first](void* p) {
+        if (!p) return;
+        const hipError_t e = hipFree(p);
+        if (e != hipSuccess && first == hipSuccess) first = e;
+    };
     {
         std::lock_guard<std::mutex> lock(g_ws_mutex);
         const auto it = g_ws.find(std::make_pair(dev, stream));
         if (it != g_ws.end()) {
             Scratch sc = it->second;
             g_ws.erase(it);
-            for (void* p : sc.retired) VPX_HIP_CHECK(hipFree(p));
-            if (sc.ptr) VPX_HIP_CHECK(hipFree(sc.ptr));
-            if (sc.sync) VPX_HIP_CHECK(hipFree(sc.sync));
+            for (void* p : sc.retired) release(p);
+            release(sc.ptr);
+            release(sc.sync);
         }
     }
-    return release_axis_tables(dev, stream);
+    const int rc = release_axis_tables(dev, stream);
+    VPX_HIP_CHECK(first);
+    return rc;
 }
 
 // ---- blob parsing -----------------------------------------------------------------------------

@@ -403,7 +403,30 @@ __global__ __launch_bounds__(256) void nce_colsum_kernel(const int8_t* __restric
 struct ConvGeom {
     int64_t N, H, W, IC, OC, OH, OW;
     int KY, KX, SY, SX, PT, PL;
+    // Where the operands' images, rows and pixels lie: the input in bytes, the output in elements (a dense NHWC tensor
+    // has isw = IC, ish = W * isw, isn = H * ish and osw = OC, osh = OW * osw, osn = OH * osh; a view of a larger
+    // tensor -- a channel slice, a window in H or W -- has the parent's).
+    int64_t isn, ish, isw;
+    int64_t osn, osh, osw;
+    int out_flat;       // 2: output position m = (n, oy, ox) of N x OH x OW sits at m * osw; 1: that holds inside an image; 0: neither
+    unsigned out_bits;  // the output's base address and its strides in bytes, or-ed: the alignment every row start shares
 };
+
+// Element offset of output position m, counted over the dense N x OH x OW positions.
+__device__ __forceinline__ int64_t out_pos(const ConvGeom& g, int64_t m) {
+    if (g.out_flat == 2) return m * g.osw;
+    const int64_t ohow = g.OH * g.OW;
+    const int64_t n = m / ohow, rem = m - n * ohow, oy = rem / g.OW, ox = rem - oy * g.OW;
+    return n * g.osn + oy * g.osh + ox * g.osw;
+}
+// Byte offset of input pixel (n, iy, ix).
+__device__ __forceinline__ int64_t in_pos(const ConvGeom& g, int64_t n, int64_t iy, int64_t ix) {
+    return n * g.isn + iy * g.ish + ix * g.isw;
+}
+// Largest store (16, 8, 4 bytes, or 1) that every row start of the output is aligned to.
+__device__ __forceinline__ int out_align(unsigned bits) {
+    return (bits & 15) == 0 ? 16 : ((bits & 7) == 0 ? 8 : ((bits & 3) == 0 ? 4 : 1));
+}
 
 template <bool IN_SIGNED, bool W_SIGNED, int OUT>
 __global__ __launch_bounds__(256) void nce_conv_naive(const uint8_t* __restrict__ in, const uint8_t* __restrict__ w,
@@ -423,7 +446,7 @@ __global__ __launch_bounds__(256) void nce_conv_naive(const uint8_t* __restrict_
         for (int kx = 0; kx < g.KX; kx++) {
             const int64_t ix = ox * g.SX + kx - g.PL;
             if (ix < 0 || ix >= g.W) continue;
-            const uint8_t* pi = in + ((n * g.H + iy) * g.W + ix) * g.IC;
+            const uint8_t* pi = in + in_pos(g, n, iy, ix);
             const uint8_t* pw = w + ((oc * g.KY + ky) * g.KX + kx) * g.IC;
             for (int64_t ic = 0; ic < g.IC; ic++) {
                 const int a = IN_SIGNED ? (int)(int8_t)pi[ic] : (int)pi[ic];
@@ -434,8 +457,9 @@ __global__ __launch_bounds__(256) void nce_conv_naive(const uint8_t* __restrict_
     }
     const uint32_t w2 = (uint32_t)wt[oc * 4 + 2];
     ChanParams c{wt[oc * 4 + 3], (int)(int16_t)(w2 >> 16), (int)((w2 >> 8) & 0xffu)};
-    if (OUT == OUT_F16) reinterpret_cast<uint16_t*>(out)[idx] = ppe_requant_f16(acc, c, ppe);
-    else out[idx] = saturate8<OUT == OUT_I8>(ppe_requant(acc, c, ppe));
+    const int64_t o = n * g.osn + oy * g.osh + ox * g.osw + oc;
+    if (OUT == OUT_F16) reinterpret_cast<uint16_t*>(out)[o] = ppe_requant_f16(acc, c, ppe);
+    else out[o] = saturate8<OUT == OUT_I8>(ppe_requant(acc, c, ppe));
 }
 
 // ---------------------------------------------------------------- GEMM path
@@ -545,9 +569,24 @@ struct GemmPpe {
 // output position m = (n, oy, ox) at pixel (n, oy * sy, ox * sx) of the input tensor -- the matmul kernel's loads
 // take a byte offset per lane, so a strided 1x1 convolution is a matmul whose rows are picked from the input.
 struct GemmRows {
-    int strided;              // 0: dense rows
-    int ow, ohow, sx, sy;     // output width, positions per image, strides
-    int w, hw;                // input width, pixels per image
+    int strided;              // 0: row m at byte m * lda
+    int64_t lda;
+    int ow, ohow;             // output width, positions per image
+    unsigned px, py, pimg;    // bytes from one output column / row / image to the next in the input (strides folded in)
+};
+
+// Where the rows of the result go: row m at element m * ldc (a matrix, a dense tensor, or a channel slice of one), or
+// position m = (n, oy, ox) at n * sn + oy * sh + ox * sw (a window of a larger tensor).
+struct GemmOut {
+    int flat;                 // 1: row m at m * sw
+    int64_t sn, sh, sw;
+    int ow, ohow;
+    unsigned bits;            // base address and strides in bytes, or-ed (see ConvGeom::out_bits)
+    __device__ __forceinline__ int64_t row(int64_t m) const {
+        if (flat) return m * sw;
+        const unsigned mm = (unsigned)m, img = mm / (unsigned)ohow, rem = mm - img * (unsigned)ohow, oy = rem / (unsigned)ow, ox = rem - oy * (unsigned)ow;
+        return (int64_t)img * sn + (int64_t)oy * sh + (int64_t)ox * sw;
+    }
 };
 
 // A[M][K] x B[N][K]^T with the PPE fused; see the file header.  K must be a multiple of 64.
@@ -565,7 +604,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                                                      const int32_t* __restrict__ wt, const int32_t* __restrict__ colsum,
                                                      uint8_t* __restrict__ out,
                                                      int64_t M, int64_t N, int64_t K, int tiles_m, int tiles_n,
-                                                     GemmPpe ppe, GemmRows rows) {
+                                                     GemmPpe ppe, GemmRows rows, GemmOut dst) {
     // NW = 4: waves 2 x 2, 128 x 128 each, one per SIMD.  NW = 8: waves 2 x 4, 128 x 64 each, two per SIMD,
     // so that one wave's loads and address arithmetic issue while the other's MFMAs run.
     // TILE = 128 (four waves of 64 x 64, 64 KiB of LDS, two workgroups per CU) serves problems with too few 256 x 256 tiles.
@@ -628,14 +667,14 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
         int64_t m = m0 + r, n = n0 + r;
         m = m < M ? m : M - 1;  // rows past the edge repeat the last one; their outputs are not stored
         n = n < N ? n : N - 1;
-        oa[i] = (unsigned)((m - m0) * K + c * 16);
+        oa[i] = (unsigned)((m - m0) * rows.lda + c * 16);
         if (rows.strided) {  // (offsets from the tensor's first byte; the host has checked that they fit 32 bits)
             const int mm = (int)m, img = mm / rows.ohow, rem = mm - img * rows.ohow, oy = rem / rows.ow, ox = rem - oy * rows.ow;
-            oa[i] = (unsigned)(img * rows.hw + oy * rows.sy * rows.w + ox * rows.sx) * (unsigned)K + (unsigned)(c * 16);
+            oa[i] = (unsigned)img * rows.pimg + (unsigned)oy * rows.py + (unsigned)ox * rows.px + (unsigned)(c * 16);
         }
         ob[i] = (unsigned)((n - n0) * K + c * 16);
     }
-    const int8_t* abase = rows.strided ? A : A + m0 * K;
+    const int8_t* abase = rows.strided ? A : A + m0 * rows.lda;
     const int8_t* bbase = B + n0 * K;
     const unsigned lds0 = lds_address(smem);
     const int nk = (int)(K / BK);
@@ -835,7 +874,7 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                         for (int q = 0; q < 4; q++) acc[i][j][g * 4 + q] += v[q];
                 }
         }
-        const bool vec_ok = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+        const bool vec_ok = (dst.bits & 15) == 0;
 #pragma unroll
         for (int pass = 0; pass < PASSES; pass++) {
             if (wm0 / ROWS == pass) {
@@ -859,10 +898,11 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
                 const int64_t m = m0 + pass * ROWS + row, n = n0 + c8 * 8;
                 if (m >= M || n >= N) continue;
                 const i32x4 v = *reinterpret_cast<const i32x4*>(smem + row * STR + c8 * 16);
+                uint16_t* const to = out16 + dst.row(m) + n;
                 if (vec_ok && n + 8 <= N) {
-                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(out16 + m * N + n));
+                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(to));
                 } else {
-                    store_tail16(reinterpret_cast<uint8_t*>(out16 + m * N + n), v, (int)(N - n < 8 ? N - n : 8) * 2, row_align(out, 2 * N));
+                    store_tail16(reinterpret_cast<uint8_t*>(to), v, (int)(N - n < 8 ? N - n : 8) * 2, out_align(dst.bits));
                 }
             }
             if (pass + 1 < PASSES) __syncthreads();  // the other half overwrites the staging tile
@@ -925,17 +965,18 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
     else if (ppe.prelu_mult == 1 && ppe.prelu_shift == 0) requant_tile(std::integral_constant<int, 2>{});
     else requant_tile(std::integral_constant<int, 1>{});
     __syncthreads();
-    const bool vec_ok = (N & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    const bool vec_ok = (dst.bits & 15) == 0;
     for (int it = 0; it < BM * (BN / 16) / NT; it++) {
         const int cid = tid + NT * it;
         const int row = cid / (BN / 16), c16 = cid % (BN / 16);
         const int64_t m = m0 + row, n = n0 + c16 * 16;
         if (m >= M || n >= N) continue;
         const i32x4 v = *reinterpret_cast<const i32x4*>(smem + row * kOutStride + c16 * 16);
+        uint8_t* const to = out + dst.row(m) + n;
         if (vec_ok && n + 16 <= N) {
-            __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(out + m * N + n));
+            __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(to));
         } else {
-            store_tail16(out + m * N + n, v, (int)(N - n < 16 ? N - n : 16), row_align(out, N));
+            store_tail16(to, v, (int)(N - n < 16 ? N - n : 16), out_align(dst.bits));
         }
     }
 }
@@ -971,7 +1012,7 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
         m = m < Mtot ? m : Mtot - 1;
         ox[i] = (int)(m % g.OW);
         oy[i] = (int)((m / g.OW) % g.OH);
-        base_n[i] = (m / (g.OW * g.OH)) * g.H * g.W * g.IC;
+        base_n[i] = (m / (g.OW * g.OH)) * g.isn;
     }
     const int pad32 = (pad_byte & 0xff) * 0x01010101;
 
@@ -1014,7 +1055,7 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
                     const int iy = oy[i] * g.SY + ky - g.PT;
                     const int ix = ox[i] * g.SX + kx - g.PL;
                     inside[i] = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-                    pin[i] = in + base_n[i] + ((int64_t)(inside[i] ? iy : 0) * g.W + (inside[i] ? ix : 0)) * g.IC + ic0 + kgroup * 16;
+                    pin[i] = in + base_n[i] + (int64_t)(inside[i] ? iy : 0) * g.ish + (int64_t)(inside[i] ? ix : 0) * g.isw + ic0 + kgroup * 16;
                 }
                 for (int ic = 0; ic < icn; ic += 32) {
                     i32x4 fa[TM], fb[TN];
@@ -1054,8 +1095,9 @@ __global__ __launch_bounds__(256) void nce_conv_mfma(const int8_t* __restrict__ 
                 const int64_t m = m0 + wave * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
                 if (m >= Mtot) continue;
                 const int a = acc[i][j][r] + (ppe.rowterm ? ppe.rowterm[m] : 0);
-                if (OUT == OUT_F16) reinterpret_cast<uint16_t*>(out)[m * g.OC + oc] = ppe_fast_f16(a, cp, ppe.f16_lo, ppe.f16_hi);
-                else out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(a, cp, ppe);
+                const int64_t o = out_pos(g, m) + oc;
+                if (OUT == OUT_F16) reinterpret_cast<uint16_t*>(out)[o] = ppe_fast_f16(a, cp, ppe.f16_lo, ppe.f16_hi);
+                else out[o] = (uint8_t)ppe_fast<true>(a, cp, ppe);
             }
         }
     }
@@ -1089,6 +1131,13 @@ struct PatchGeom {
     FastDiv tiles_y, cpr, cpp, upr, ow;  // tiles per image, chunks per weight row / pixel, units per patch row, OW
 };
 
+// Element offset of the tile's position p = r * OW + ox from the tile's first output position (rows osh apart).
+__device__ __forceinline__ int64_t tile_out_pos(const ConvGeom& g, int p, FastDiv ow) {
+    if (g.out_flat) return (int64_t)p * g.osw;
+    const int r = fdiv(p, ow), ox = p - r * (int)ow.d;
+    return (int64_t)r * g.osh + (int64_t)ox * g.osw;
+}
+
 constexpr int kPatchMaxMT = 14;
 constexpr int kPatchOutStride = 80;  // bytes per output position in the staging tile
 constexpr int kPatchOutStrideF16 = 144;  // the same for an fp16 output
@@ -1100,7 +1149,7 @@ constexpr int kPatchOutStrideF16 = 144;  // the same for an fp16 output
 template <int TMW, int NT>
 __device__ __forceinline__ void patch_epilogue_f16(i32x16 (&acc)[TMW], int mi0, int mstep, int nj, int MT, const ChanPrep& c,
                                                    const GemmPpe& ppe, const int32_t* rt, uint8_t* stage, uint16_t* out16,
-                                                   int valid, int oc0, int OC) {
+                                                   int valid, int oc0, int OC, const ConvGeom& g, FastDiv ow) {
     const int tid = threadIdx.x, lane = tid & 63;
 #pragma unroll
     for (int i = 0; i < TMW; i++) {
@@ -1115,17 +1164,17 @@ __device__ __forceinline__ void patch_epilogue_f16(i32x16 (&acc)[TMW], int mi0, 
         }
     }
     __syncthreads();
-    const bool vec_ok = (OC & 7) == 0 && (reinterpret_cast<uintptr_t>(out16) & 15) == 0;
+    const bool vec_ok = (g.out_bits & 15) == 0;
     for (int cid = tid; cid < valid * 8; cid += NT) {
         const int row = cid >> 3, c8 = cid & 7;
         const int n = oc0 + c8 * 8;
         if (n >= OC) continue;
         const i32x4 v = *reinterpret_cast<const i32x4*>(stage + row * kPatchOutStrideF16 + c8 * 16);
-        uint16_t* dst = out16 + ((int64_t)row * OC + n);
+        uint16_t* dst = out16 + (tile_out_pos(g, row, ow) + n);
         if (vec_ok && n + 8 <= OC) {
             __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
         } else {
-            store_tail16(reinterpret_cast<uint8_t*>(dst), v, (OC - n < 8 ? OC - n : 8) * 2, row_align(out16, 2 * (int64_t)OC));
+            store_tail16(reinterpret_cast<uint8_t*>(dst), v, (OC - n < 8 ? OC - n : 8) * 2, out_align(g.out_bits));
         }
     }
 }
@@ -1169,7 +1218,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
         const int row_chunks = pg.PW * cpp;
         const int upr = (int)pg.upr.d, units = pg.PH * upr;
         const int pad32 = (pad_byte & 0xff) * 0x01010101;
-        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
+        const int8_t* img_base = in + (int64_t)img * g.isn;
         const int iy0 = oy0 * g.SY - g.PT;
         const bool full_rows = oc0 + BN <= g.OC;       // the 64 weight rows are one contiguous run
         for (int q0 = 0, u0 = 0; q0 < wchunks || u0 < units; q0 += NT * UW, u0 += NW * UP) {
@@ -1198,7 +1247,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
                 const int px = qi / cpp, cc = qi % cpp;
                 const int iy = iy0 + py, ix = px - g.PL;
                 const bool inside = ok && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-                const int64_t off = inside ? ((int64_t)iy * g.W + ix) * IC + cc * 16 : 0;
+                const int64_t off = inside ? (int64_t)iy * g.ish + (int64_t)ix * g.isw + cc * 16 : 0;
                 const i32x4 v = *reinterpret_cast<const i32x4*>(img_base + off);
                 qp[u] = inside ? v : i32x4{pad32, pad32, pad32, pad32};
                 dp[u] = ok ? (py * pg.PW + px) * PS + cc * 16 : -1;
@@ -1306,7 +1355,8 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
         const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
         const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
         patch_epilogue_f16<TMW, NT>(acc, mi0, mstep, nj, pg.MT, c, ppe, ppe.rowterm ? ppe.rowterm + pos0 : nullptr, patch,
-                                    reinterpret_cast<uint16_t*>(out) + pos0 * g.OC, rows_here * (int)g.OW, oc0, (int)g.OC);
+                                    reinterpret_cast<uint16_t*>(out) + ((int64_t)img * g.osn + (int64_t)oy0 * g.osh),
+                                    rows_here * (int)g.OW, oc0, (int)g.OC, g, pg.ow);
         return;
     }
     {
@@ -1356,18 +1406,18 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : (TMW <= 4 ? 2 : 1)) void nce
     __syncthreads();
     const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
     const int valid = rows_here * (int)g.OW;
-    const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
-    const bool vec_ok = (g.OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    uint8_t* const out0 = out + ((int64_t)img * g.osn + (int64_t)oy0 * g.osh);  // the tile's first output position
+    const bool vec_ok = (g.out_bits & 15) == 0;
     for (int cid = tid; cid < valid * 4; cid += NT) {
         const int row = cid >> 2, c16 = cid & 3;
         const int64_t n = oc0 + c16 * 16;
         if (n >= g.OC) continue;
         const i32x4 v = *reinterpret_cast<const i32x4*>(patch + row * kPatchOutStride + c16 * 16);
-        uint8_t* dst = out + (pos0 + row) * g.OC + n;
+        uint8_t* dst = out0 + tile_out_pos(g, row, pg.ow) + n;
         if (vec_ok && n + 16 <= g.OC) {
             __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
         } else {
-            store_tail16(dst, v, (int)(g.OC - n < 16 ? g.OC - n : 16), row_align(out, g.OC));
+            store_tail16(dst, v, (int)(g.OC - n < 16 ? g.OC - n : 16), out_align(g.out_bits));
         }
     }
 }
@@ -1421,8 +1471,9 @@ __global__ __launch_bounds__(512) void nce_conv_regw(const int8_t* __restrict__ 
         const int iy0 = oy0 * g.SY - g.PT;
         // patch pixel (py, px) is input pixel (iy0 + py, px - PL): byte offset py * W*IC + px * IC from `corner`, which
         // may lie outside the tensor; lanes whose pixel is padding read the first pixel of the tile's first real row
-        const int8_t* corner = in + (((int64_t)img * H + iy0) * W - g.PL) * IC;
-        const int safe_off = ((iy0 < 0 ? -iy0 : 0) * W + g.PL) * IC;
+        const int isw = (int)g.isw, ish = (int)g.ish;  // (the host sends layers here whose patch offsets fit 32 bits)
+        const int8_t* corner = in + ((int64_t)img * g.isn + (int64_t)iy0 * g.ish - (int64_t)g.PL * g.isw);
+        const int safe_off = (iy0 < 0 ? -iy0 : 0) * ish + g.PL * isw;
         const int8_t* wsrc = w + (int64_t)oc0 * Ktot;
         const bool full_rows = oc0 + BN <= OC;         // the 64 weight rows are one contiguous run
         i32x4 qw[UW], qp[UP];
@@ -1439,7 +1490,7 @@ __global__ __launch_bounds__(512) void nce_conv_regw(const int8_t* __restrict__ 
                 const int px = qi / cpp;
                 const int iy = iy0 + py;
                 const bool inside = ok && (unsigned)iy < (unsigned)H && (unsigned)(px - g.PL) < (unsigned)W;
-                const int off = inside ? py * (W * IC) + qi * 16 : safe_off;
+                const int off = inside ? py * ish + px * isw + (qi % cpp) * 16 : safe_off;
                 qp[u] = *reinterpret_cast<const i32x4*>(corner + off);
                 pin[u] = inside;
                 dp[u] = ok ? py * (pg.PW * PS) + px * PS + (qi % cpp) * 16 : -1;
@@ -1522,8 +1573,8 @@ __global__ __launch_bounds__(512) void nce_conv_regw(const int8_t* __restrict__ 
     const int nblk = (valid + 15) >> 4;
     const int64_t pos0 = ((int64_t)img * OH + oy0) * OW;
     const int32_t* rt = ppe.rowterm ? ppe.rowterm + pos0 : nullptr;
-    uint8_t* const out0 = out + pos0 * OC;  // the tile's first output position
-    const bool vec_ok = (OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    uint8_t* const out0 = out + ((int64_t)img * g.osn + (int64_t)oy0 * g.osh);  // the tile's first output position
+    const bool vec_ok = (g.out_bits & 15) == 0;
     const int q16 = oc0 + (n16 >> 2) * 16;  // first of the 16 channels this lane stores
     int soff[TAPS];
 #pragma unroll
@@ -1577,11 +1628,11 @@ __global__ __launch_bounds__(512) void nce_conv_regw(const int8_t* __restrict__ 
         }
         const int pi = b * 16 + 4 * c4 + (lane & 3);
         if (pi < valid && q16 < OC) {
-            uint8_t* dst = out0 + (pi * OC + q16);
+            uint8_t* dst = out0 + (tile_out_pos(g, pi, pg.ow) + q16);
             if (vec_ok && q16 + 16 <= OC) {
                 __builtin_nontemporal_store(o, reinterpret_cast<i32x4*>(dst));
             } else {
-                store_tail16(dst, o, OC - q16 < 16 ? OC - q16 : 16, row_align(out, OC));
+                store_tail16(dst, o, OC - q16 < 16 ? OC - q16 : 16, out_align(g.out_bits));
             }
         }
     };
@@ -1677,7 +1728,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
         const int row_chunks = pg.PW * cpp;
         const int upr = (int)pg.upr.d, units = pg.PH * upr;
         const int pad32 = (pad_byte & 0xff) * 0x01010101;
-        const int8_t* img_base = in + (int64_t)img * g.H * g.W * IC;
+        const int8_t* img_base = in + (int64_t)img * g.isn;
         const int iy0 = oy0 * g.SY - g.PT;
         for (int u0 = 0; u0 < units; u0 += NW * UP) {
             i32x4 qp[UP];
@@ -1691,7 +1742,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
                 const int px = fdiv(qi, pg.cpp), cc = qi - px * cpp;
                 const int iy = iy0 + py, ix = px - g.PL;
                 const bool inside = ok && iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-                const int64_t off = inside ? ((int64_t)iy * g.W + ix) * IC + cc * 16 : 0;
+                const int64_t off = inside ? (int64_t)iy * g.ish + (int64_t)ix * g.isw + cc * 16 : 0;
                 const i32x4 v = *reinterpret_cast<const i32x4*>(img_base + off);
                 qp[u] = inside ? v : i32x4{pad32, pad32, pad32, pad32};
                 dp[u] = ok ? (py * pg.PW + px) * PS + cc * 16 : -1;
@@ -1868,7 +1919,8 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
         const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
         const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
         patch_epilogue_f16<TMW, NT>(acc, mi0, mstep, nj, pg.MT, c, ppe, ppe.rowterm ? ppe.rowterm + pos0 : nullptr, patch,
-                                    reinterpret_cast<uint16_t*>(out) + pos0 * g.OC, rows_here * (int)g.OW, oc0, (int)g.OC);
+                                    reinterpret_cast<uint16_t*>(out) + ((int64_t)img * g.osn + (int64_t)oy0 * g.osh),
+                                    rows_here * (int)g.OW, oc0, (int)g.OC, g, pg.ow);
         return;
     }
     {
@@ -1918,18 +1970,18 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void nce_conv_stream(cons
     __syncthreads();
     const int rows_here = g.OH - oy0 < pg.R ? (int)(g.OH - oy0) : pg.R;
     const int valid = rows_here * (int)g.OW;
-    const int64_t pos0 = ((int64_t)img * g.OH + oy0) * g.OW;
-    const bool vec_ok = (g.OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+    uint8_t* const out0 = out + ((int64_t)img * g.osn + (int64_t)oy0 * g.osh);  // the tile's first output position
+    const bool vec_ok = (g.out_bits & 15) == 0;
     for (int cid = tid; cid < valid * 4; cid += NT) {
         const int row = cid >> 2, c16 = cid & 3;
         const int64_t n = oc0 + c16 * 16;
         if (n >= g.OC) continue;
         const i32x4 v = *reinterpret_cast<const i32x4*>(patch + row * kPatchOutStride + c16 * 16);
-        uint8_t* dst = out + (pos0 + row) * g.OC + n;
+        uint8_t* dst = out0 + tile_out_pos(g, row, pg.ow) + n;
         if (vec_ok && n + 16 <= g.OC) {
             __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst));
         } else {
-            store_tail16(dst, v, (int)(g.OC - n < 16 ? g.OC - n : 16), row_align(out, g.OC));
+            store_tail16(dst, v, (int)(g.OC - n < 16 ? g.OC - n : 16), out_align(g.out_bits));
         }
     }
 }
@@ -2010,6 +2062,75 @@ __global__ __launch_bounds__(256) void nce_eltwise_kernel(const uint8_t* __restr
     }
 }
 
+// The same task on operands that are views of larger tensors (strides per image, row and pixel; a pixel's channels
+// are contiguous): a lane takes up to sixteen channels of one pixel, in 16-byte accesses where the operand's base and
+// strides allow, else byte by byte.
+struct EltViews {
+    int64_t H, W, C;
+    int64_t asn, ash, asw, bsn, bsh, bsw, osn, osh, osw;  // a and b in bytes, the output in elements
+    int cpp;            // sixteen-channel chunks per pixel
+    int in_vec;         // both inputs: base and strides are multiples of 16 bytes
+    unsigned out_bits;  // the output's base address and strides in bytes, or-ed
+};
+
+template <bool A_SIGNED, bool B_SIGNED, bool SAME_F, bool OUT_F16>
+__global__ __launch_bounds__(256) void nce_eltwise_views_kernel(const uint8_t* __restrict__ a, const uint8_t* __restrict__ b,
+                                                                uint8_t* __restrict__ out, int64_t chunks, EltViews ev, EltParams e) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= chunks) return;
+    const int64_t pixel = t / ev.cpp;
+    const int c0 = (int)(t - pixel * ev.cpp) * 16;
+    const int64_t hw = ev.H * ev.W, n = pixel / hw, rem = pixel - n * hw, y = rem / ev.W, x = rem - y * ev.W;
+    const uint8_t* pa = a + (n * ev.asn + y * ev.ash + x * ev.asw + c0);
+    const uint8_t* pb = b + (n * ev.bsn + y * ev.bsh + x * ev.bsw + c0);
+    const int64_t o = n * ev.osn + y * ev.osh + x * ev.osw + c0;
+    const int count = ev.C - c0 < 16 ? (int)(ev.C - c0) : 16;
+    i32x4 qa = i32x4{0, 0, 0, 0}, qb = i32x4{0, 0, 0, 0};
+    if (ev.in_vec && count == 16) {
+        qa = *reinterpret_cast<const i32x4*>(pa);
+        qb = *reinterpret_cast<const i32x4*>(pb);
+    } else {
+        for (int k = 0; k < count; k++) {
+            qa[k >> 2] |= (int)pa[k] << (8 * (k & 3));
+            qb[k >> 2] |= (int)pb[k] << (8 * (k & 3));
+        }
+    }
+    auto val = [](unsigned word, int k, bool sgn) {
+        return sgn ? (int)(int8_t)(word >> (8 * k)) : (int)((word >> (8 * k)) & 0xffu);
+    };
+    if constexpr (OUT_F16) {
+        uint16_t* const po = reinterpret_cast<uint16_t*>(out) + o;
+        i32x4 r[2] = {i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}};
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int acc = val((unsigned)qa[j], k, A_SIGNED) * e.m1 + val((unsigned)qb[j], k, B_SIGNED) * e.m2;
+                const int idx = 4 * j + k;
+                r[idx >> 3][(idx >> 1) & 3] |= (int)ppe_fast_f16(acc, e.cp16, e.f16_lo, e.f16_hi) << (16 * (idx & 1));
+            }
+        if ((ev.out_bits & 15) == 0 && count == 16) {
+            __builtin_nontemporal_store(r[0], reinterpret_cast<i32x4*>(po));
+            __builtin_nontemporal_store(r[1], reinterpret_cast<i32x4*>(po) + 1);
+        } else {
+            const int al = out_align(ev.out_bits);
+            store_tail16(reinterpret_cast<uint8_t*>(po), r[0], (count < 8 ? count : 8) * 2, al);
+            if (count > 8) store_tail16(reinterpret_cast<uint8_t*>(po + 8), r[1], (count - 8) * 2, al);
+        }
+    } else {
+        i32x4 r;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            int acc[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) acc[k] = val((unsigned)qa[j], k, A_SIGNED) * e.m1 + val((unsigned)qb[j], k, B_SIGNED) * e.m2;
+            r[j] = (int)ppe_pack4<SAME_F, true>(acc[0], acc[1], acc[2], acc[3], e.cp, e.pk);
+        }
+        if ((ev.out_bits & 15) == 0 && count == 16) __builtin_nontemporal_store(r, reinterpret_cast<i32x4*>(out + o));
+        else store_tail16(out + o, r, count, out_align(ev.out_bits));
+    }
+}
+
 // ---------------------------------------------------------------- gather convolution, IC a multiple of 16
 // Stem layers (3 or 4 image channels padded to 16) and other channel counts that are a multiple of
 // 16 but not of 32.  K = KY*KX*IC is walked as a flat run of 16-byte chunks, two per MFMA step:
@@ -2047,7 +2168,7 @@ __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict_
         m = m < Mtot ? m : Mtot - 1;
         ox[i] = (int)(m % g.OW) * g.SX - g.PL;
         oy[i] = (int)((m / g.OW) % g.OH) * g.SY - g.PT;
-        base_n[i] = (m / (g.OW * g.OH)) * g.H * g.W * g.IC;
+        base_n[i] = (m / (g.OW * g.OH)) * g.isn;
     }
     const int pad32 = (pad_byte & 0xff) * 0x01010101;
     i32x16 acc[TM][TN];
@@ -2071,7 +2192,7 @@ __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict_
         for (int i = 0; i < TM; i++) {
             const int iy = oy[i] + ky, ix = ox[i] + kx;
             const bool inside = iy >= 0 && iy < g.H && ix >= 0 && ix < g.W;
-            const int64_t off = inside ? ((int64_t)iy * g.W + ix) * g.IC + cc * 16 : 0;
+            const int64_t off = inside ? (int64_t)iy * g.ish + (int64_t)ix * g.isw + cc * 16 : 0;
             i32x4 q = *reinterpret_cast<const i32x4*>(in + base_n[i] + off);
             if (!inside) q = i32x4{pad32, pad32, pad32, pad32};
             if (IN_U8) q ^= (int32_t)0x80808080;
@@ -2097,8 +2218,9 @@ __global__ __launch_bounds__(256) void nce_conv_mfma16(const int8_t* __restrict_
                 const int64_t m = m0 + wave * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
                 if (m >= Mtot) continue;
                 const int a = acc[i][j][r] + (ppe.rowterm ? ppe.rowterm[m] : 0);
-                if (OUT == OUT_F16) reinterpret_cast<uint16_t*>(out)[m * g.OC + oc] = ppe_fast_f16(a, cp, ppe.f16_lo, ppe.f16_hi);
-                else out[m * g.OC + oc] = (uint8_t)ppe_fast<true>(a, cp, ppe);
+                const int64_t o = out_pos(g, m) + oc;
+                if (OUT == OUT_F16) reinterpret_cast<uint16_t*>(out)[o] = ppe_fast_f16(a, cp, ppe.f16_lo, ppe.f16_hi);
+                else out[o] = (uint8_t)ppe_fast<true>(a, cp, ppe);
             }
         }
     }
@@ -2187,7 +2309,8 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         const TilePos tp = tile_pos(tile_);
         const int iy0 = tp.oy0 * g.SY - g.PT, ix0 = tp.ox0 * g.SX - g.PL;
         const int safe_row = iy0 < 0 ? 0 : (iy0 < H ? iy0 : H - 1);
-        return Origin{in + (((int64_t)tp.img * H + iy0) * W + ix0) * IC, iy0, ix0, ((safe_row - iy0) * W - ix0) * IC};
+        return Origin{in + ((int64_t)tp.img * g.isn + (int64_t)iy0 * g.ish + (int64_t)ix0 * g.isw), iy0, ix0,
+                      (safe_row - iy0) * (int)g.ish - ix0 * (int)g.isw};
     };
     auto chunk = [&](const Origin& o, int q) {
         Chunk c;
@@ -2196,7 +2319,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         const int py = fdiv(qq, rg.rc), qi = qq - py * rg.row_chunks;
         const int px = fdiv(qi, rg.cpp);
         c.inside = c.ok && (unsigned)(o.iy0 + py) < (unsigned)H && (unsigned)(o.ix0 + px) < (unsigned)W;
-        c.src = c.inside ? py * (W * IC) + qi * 16 : o.safe_off;
+        c.src = c.inside ? py * (int)g.ish + px * (int)g.isw + (qi - px * (int)rg.cpp.d) * 16 : o.safe_off;
         const int qd = fdiv(qi, rg.fm);
         c.dst = py * rg.RB + ((qi - qd * rg.m) * rg.plane + qd) * 16;
         return c;
@@ -2285,8 +2408,8 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
     // (the barrier after the first patch makes these visible)
 
     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;  // no PReLU stage (or a slope of zero, which the host turns into a clamp)
-    const bool vec_ok = (OC & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
-    const bool half_ok = (OC & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0;
+    const bool vec_ok = (g.out_bits & 15) == 0;
+    const bool half_ok = (g.out_bits & 7) == 0;
     const uint8_t* const wl = wlds + (lane & 31) * rg.WS + half * 16;
     const int q16 = oc0 + half * 16;  // first of the 16 channels this lane stores in channel tile 0
 
@@ -2306,7 +2429,14 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
         const int nblk = (rows_here * rg.CW + BP - 1) / BP;
         const int64_t pos0 = ((int64_t)img * OH + oy0) * OW + ox0;
         const int32_t* rt = ppe.rowterm ? ppe.rowterm + pos0 : nullptr;
-        uint8_t* const out0 = out + pos0 * OC;
+        const int64_t opos0 = (int64_t)img * g.osn + (int64_t)oy0 * g.osh + (int64_t)ox0 * g.osw;  // the tile's first output position
+        uint8_t* const out0 = out + opos0;
+        // element offset of the position r * OW + c from there
+        auto out_off = [&](int pcv) {
+            if (g.out_flat) return (int64_t)pcv * g.osw;
+            const int r = fdiv(pcv, rg.ow), c = pcv - r * OW;
+            return (int64_t)r * g.osh + (int64_t)c * g.osw;
+        };
 
         auto one_block = [&](int b, auto kind_c) {
             // PPE kinds.  0: the general form; 1: two factors, the short form (see ppe_pack4_biased); 2: one factor;
@@ -2387,8 +2517,8 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                 }
             }
             if constexpr (KIND == 3) {
-                uint16_t* const out16 = reinterpret_cast<uint16_t*>(out) + pos0 * OC;
-                const bool vec16_ok = (OC & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+                uint16_t* const out16 = reinterpret_cast<uint16_t*>(out) + opos0;
+                const bool vec16_ok = vec_ok;
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
                     const int qc = q16 + 32 * j;
@@ -2409,7 +2539,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
 #pragma unroll
                         for (int i = 0; i < TM; i++) {
                             if (pc[i] < 0 || qc + 8 * half8 >= OC) continue;
-                            uint16_t* dst = out16 + ((int64_t)pc[i] * OC + qc + 8 * half8);
+                            uint16_t* dst = out16 + (out_off(pc[i]) + qc + 8 * half8);
                             if (vec16_ok && qc + 8 * half8 + 8 <= OC) {
                                 __builtin_nontemporal_store(o8[i], reinterpret_cast<i32x4*>(dst));
                             } else {
@@ -2453,7 +2583,7 @@ __global__ __launch_bounds__(512) void nce_conv_rows16(const int8_t* __restrict_
                 for (int i = 0; i < TM; i++) {
                     if (pc[i] < 0 || qc >= OC) continue;
                     o[i] ^= (int)pk.flip;
-                    uint8_t* dst = out0 + ((int64_t)pc[i] * OC + qc);
+                    uint8_t* dst = out0 + (out_off(pc[i]) + qc);
                     if (vec_ok && qc + 16 <= OC) {
                         __builtin_nontemporal_store(o[i], reinterpret_cast<i32x4*>(dst));
                     } else if (half_ok && qc + 16 <= OC) {  // (rows a multiple of 8 bytes long: 72, 88, 120 channels)
@@ -2496,6 +2626,44 @@ int set_dyn_lds(KernelT kernel, size_t bytes) {
     if (g_lds_done.count({dev, fn})) return VPX_RESULT_SUCCESS;
     VPX_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxDynLds));
     g_lds_done.insert({dev, fn});
+    return VPX_RESULT_SUCCESS;
+}
+
+// An operand of an NCE task as a view: the strides of its images, rows and pixels in elements (channels contiguous).
+// All four task strides zero is the dense tensor.  Dimensions of size one take the stride that keeps the view as flat
+// as the others allow (their own is never used).
+struct View {
+    int64_t sn, sh, sw;
+    bool dense;   // the packed NHWC tensor
+    int flat;     // 2: position m of N x H x W at m * sw; 1: that holds inside an image; 0: neither
+    int64_t span; // elements from the first to one past the last
+};
+int operand_view(const int64_t st[4], int64_t N, int64_t H, int64_t W, int64_t C, const char* what, View* v) {
+    if ((st[0] | st[1] | st[2] | st[3]) == 0) {
+        *v = View{H * W * C, W * C, C, true, 2, N * H * W * C};
+        return VPX_RESULT_SUCCESS;
+    }
+    VPX_REQUIRE(st[3] == 1, VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: the %s's channel stride is %lld; channels must be contiguous (1)", what,
+                (long long)st[3]);
+    VPX_REQUIRE(st[0] >= 0 && st[1] >= 0 && st[2] >= 0, VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: the %s has a negative stride", what);
+    const int64_t ext_w = (W - 1) * st[2] + C;
+    VPX_REQUIRE(W <= 1 || st[2] >= C, VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: the %s's W stride %lld is below its %lld channels", what,
+                (long long)st[2], (long long)C);
+    VPX_REQUIRE(H <= 1 || st[1] >= ext_w, VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: the %s's H stride %lld is below the %lld elements a row spans",
+                what, (long long)st[1], (long long)ext_w);
+    const int64_t ext_h = (H - 1) * st[1] + ext_w;
+    VPX_REQUIRE(N <= 1 || st[0] >= ext_h, VPX_RESULT_ERROR_INVALID_ARGUMENT, "NCE task: the %s's N stride %lld is below the %lld elements an image spans",
+                what, (long long)st[0], (long long)ext_h);
+    int64_t sn = st[0], sh = st[1], sw = st[2];
+    if (W <= 1) sw = H > 1 ? sh : (N > 1 ? sn : C);
+    if (H <= 1) sh = N > 1 && W <= 1 ? sn : W * sw;
+    if (N <= 1) sn = H * sh;
+    v->sn = sn;
+    v->sh = sh;
+    v->sw = sw;
+    v->flat = sh == W * sw ? (sn == H * sh ? 2 : 1) : 0;
+    v->dense = v->flat == 2 && sw == C;
+    v->span = (N > 0 && H > 0 && W > 0) ? (N - 1) * sn + (H - 1) * sh + (W - 1) * sw + C : 0;
     return VPX_RESULT_SUCCESS;
 }
 
@@ -2544,6 +2712,46 @@ int launch_nce_eltwise(const vpx_nce_task_t& t, const Ppe& ppe, hipStream_t s, c
     e.f16_lo = ppe.f16_lo;
     e.f16_hi = ppe.f16_hi;
     const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
+    View va, vb, vo;
+    int vrc = operand_view(t.input_strides, t.N, t.H, t.W, t.IC, "first input", &va);
+    if (!vrc) vrc = operand_view(t.weights_strides, t.N, t.H, t.W, t.IC, "second input", &vb);
+    if (!vrc) vrc = operand_view(t.output_strides, t.N, t.H, t.W, t.IC, "output", &vo);
+    if (vrc) return vrc;
+    if (!(va.dense && vb.dense && vo.dense)) {
+        // views of larger tensors: up to sixteen channels of a pixel per lane
+        EltViews ev{};
+        ev.H = t.H; ev.W = t.W; ev.C = t.IC;
+        ev.asn = va.sn; ev.ash = va.sh; ev.asw = va.sw;
+        ev.bsn = vb.sn; ev.bsh = vb.sh; ev.bsw = vb.sw;
+        ev.osn = vo.sn; ev.osh = vo.sh; ev.osw = vo.sw;
+        ev.cpp = (int)((t.IC + 15) / 16);
+        ev.in_vec = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights) | (uintptr_t)(va.sn | va.sh | va.sw) |
+                      (uintptr_t)(vb.sn | vb.sh | vb.sw)) & 15) == 0 ? 1 : 0;
+        const int ob = out_f16 ? 2 : 1;
+        ev.out_bits = (unsigned)(reinterpret_cast<uintptr_t>(t.output) | (uintptr_t)((vo.sn | vo.sh | vo.sw) * ob));
+        VPX_REQUIRE(t.IC < (1ll << 31) - 16, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "NCE eltwise: %lld channels are too many", (long long)t.IC);
+        const int64_t chunks = t.N * t.H * t.W * ev.cpp;
+        const int64_t blocks = (chunks + 255) / 256;
+        VPX_REQUIRE(blocks < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "NCE eltwise: tensor of %lld elements is too large", (long long)n);
+#define VPX_ELTV(AS, BS, SF, F16)                                                                                      \
+    hipLaunchKernelGGL((nce_eltwise_views_kernel<AS, BS, SF, F16>), dim3((unsigned)blocks), dim3(256), 0, s,          \
+                       (const uint8_t*)t.input, (const uint8_t*)t.weights, (uint8_t*)t.output, chunks, ev, e)
+#define VPX_ELTV_S(AS, BS)                                                                                             \
+    do {                                                                                                               \
+        if (out_f16) VPX_ELTV(AS, BS, false, true);                                                                    \
+        else if (same_f) VPX_ELTV(AS, BS, true, false);                                                                \
+        else VPX_ELTV(AS, BS, false, false);                                                                           \
+    } while (0)
+        if (a_signed && b_signed) VPX_ELTV_S(true, true);
+        else if (a_signed) VPX_ELTV_S(true, false);
+        else if (b_signed) VPX_ELTV_S(false, true);
+        else VPX_ELTV_S(false, false);
+#undef VPX_ELTV_S
+#undef VPX_ELTV
+        VPX_HIP_CHECK(hipGetLastError());
+        *kernel_name = "nce_eltwise_views_kernel";
+        return VPX_RESULT_SUCCESS;
+    }
     const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights) |
                            reinterpret_cast<uintptr_t>(t.output)) & 15) == 0;
     const int64_t n_vec = aligned ? n / 16 : 0;
@@ -2588,14 +2796,20 @@ int launch_nce_eltwise(const vpx_nce_task_t& t, const Ppe& ppe, hipStream_t s, c
 // convolution kernels add the result to their accumulators before the PPE.  A 1x1, stride-1, unpadded layer
 // (a matmul) needs only the first, which then applies the factor itself.
 __global__ __launch_bounds__(256) void nce_pixel_sum_kernel(const uint8_t* __restrict__ in, int32_t* __restrict__ cs, int64_t pixels,
-                                                            int IC, int lpp, int flip, int offset, int factor) {
+                                                            int IC, int lpp, int flip, int offset, int factor, ConvGeom g, int in_flat) {
     // lpp lanes (a power of two, at most 64) share a pixel; each sums 16-byte chunks
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t pixel = t / lpp;
     const int sub = (int)(t % lpp);
     unsigned sum = 0;
     if (pixel < pixels) {
-        const i32x4* row = reinterpret_cast<const i32x4*>(in + pixel * IC);
+        // (pixels are counted over the dense N x H x W grid; a view of a larger tensor has them isw / ish / isn apart)
+        int64_t at = pixel * g.isw;
+        if (!in_flat) {
+            const int64_t hw = g.H * g.W, n = pixel / hw, rem = pixel - n * hw, y = rem / g.W;
+            at = in_pos(g, n, y, rem - y * g.W);
+        }
+        const i32x4* row = reinterpret_cast<const i32x4*>(in + at);
         for (int c = sub; c < IC / 16; c += lpp) {
             const i32x4 q = row[c];
 #pragma unroll
@@ -2748,6 +2962,21 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const int64_t Ktot = (int64_t)g.KY * g.KX * g.IC;
     if (Mtot == 0 || g.OC == 0) return VPX_RESULT_SUCCESS;
 
+    // Input and output as views (dense unless the task gives strides); the weights are always dense.
+    View vin, vout;
+    {
+        int rc = operand_view(t.input_strides, g.N, g.H, g.W, g.IC, "input", &vin);
+        if (!rc) rc = operand_view(t.output_strides, g.N, g.OH, g.OW, g.OC, "output", &vout);
+        if (rc) return rc;
+        VPX_REQUIRE(t.groups <= 1 || (vin.dense && vout.dense), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                    "NCE task: a grouped task takes dense operands (strides were given with groups = %d)", t.groups);
+    }
+    g.isn = vin.sn; g.ish = vin.sh; g.isw = vin.sw;
+    g.osn = vout.sn; g.osh = vout.sh; g.osw = vout.sw;
+    g.out_flat = vout.flat;
+    g.out_bits = (unsigned)(reinterpret_cast<uintptr_t>(t.output) | (uintptr_t)((vout.sn | vout.sh | vout.sw) * (out_f16 ? 2 : 1)));
+    const bool in_flat = vin.flat == 2;
+
     const bool zp_in_ok = in_u8 ? (t.zp_in >= 0 && t.zp_in <= 255) : (t.zp_in >= -128 && t.zp_in <= 127);
     // the fast epilogue adds the output zero point after limiting the scaled value to +-2^30
     const bool zp_out_ok = t.zp_out >= -(1 << 20) && t.zp_out <= (1 << 20);
@@ -2761,9 +2990,14 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     const bool is_1x1 = g.KY == 1 && g.KX == 1 && t.kernel_padding[0] == 0 && t.kernel_padding[1] == 0 &&
                         t.kernel_padding[2] == 0 && t.kernel_padding[3] == 0;
     const bool is_gemm = is_1x1 && g.SY == 1 && g.SX == 1;
-    // a 1x1 layer with a stride is a matmul over rows picked from the input (one group, tensor below 4 GiB)
-    const bool is_strided_gemm = is_1x1 && !is_gemm && t.groups <= 1 && g.N * g.H * g.W * g.IC < (1ll << 32);
-    const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights)) & 15) == 0;
+    // a 1x1 layer with a stride, or whose input pixels are not evenly spaced (a window of a larger tensor), is a matmul
+    // over rows picked from the input (one group, the view spanning less than 4 GiB)
+    const bool picks_rows = !(is_gemm && in_flat);
+    const bool is_strided_gemm = is_1x1 && picks_rows && t.groups <= 1 && vin.span < (1ll << 32);
+    const bool is_flat_gemm = is_gemm && in_flat && vin.sw < (1ll << 23);
+    // (the MFMA kernels read 16 bytes at a time from wherever a pixel starts)
+    const bool aligned = ((reinterpret_cast<uintptr_t>(t.input) | reinterpret_cast<uintptr_t>(t.weights) |
+                           (uintptr_t)(vin.sn | vin.sh | vin.sw)) & 15) == 0;
     // VPX_NCE_KERNEL=naive|gather|conv restricts the choice to the slower, more general paths (used by tests
     // to check the device paths against each other).
     const Tuning& knobs = tuning();
@@ -2777,7 +3011,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     // is long enough for the matmul kernel's deeper pipeline to make up for it (from 192 channels on: [100352 x 192 x 64]
     // 13.8 -> 11.1 us, [25088 x 512 x 64] 8.6 -> 7.5 us, [6272 x 1024 x 64] 11.1 -> 9.0 us; 128 channels: even).
     const int64_t gemm_tiles = ((Mtot + 255) / 256) * ((g.OC + 255) / 256);
-    const bool use_gemm = allow_gemm && (is_gemm || is_strided_gemm) && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || (g.OC > 48 && g.IC >= 192) || Mtot < 1024);
+    const bool use_gemm = allow_gemm && (is_flat_gemm || is_strided_gemm) && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || (g.OC > 48 && g.IC >= 192) || Mtot < 1024);
     // VPU.NCE.MatMul's groups: one launch of the matmul kernel when it serves the shape (the preparation passes then
     // walk all groups' weights / activations as one tensor), else one task after the other on the stream.
     const int64_t G = t.groups > 1 ? t.groups : 1;
@@ -2835,7 +3069,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                         (long long)pixels);
             hipLaunchKernelGGL(nce_pixel_sum_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const uint8_t*)t.input, cs, pixels,
                                (int)g.IC, lpp, in_u8 ? 0 : (int)0x80808080, (int)((in_u8 ? 0 : 128) * g.IC + t.zp_in * g.IC),
-                               direct ? wz_rest : 1);
+                               direct ? wz_rest : 1, g, in_flat ? 1 : 0);
             VPX_HIP_CHECK(hipGetLastError());
             if (!direct) {
                 hipLaunchKernelGGL(nce_window_sum_kernel, dim3((unsigned)((Mtot + 255) / 256)), dim3(256), 0, s, cs, rt, g, wz_rest, Mtot);
@@ -2852,7 +3086,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     // 64 3x3: 27 us against 64 us, [32,14,14,160] -> 320 1x1: 9 against 19.5; 5x5 x 96 channels, 154 KiB of weights: 183 against 47.)
     if (allow_lds && !use_gemm && mfma_ok && aligned && g.IC % 16 == 0 &&
         (g.IC % 32 != 0 || (g.IC % 64 != 0 && (g.OC <= 32 ? 32 : 64) * ((g.KY * g.KX * (g.IC / 16) + 1) / 2 * 32 + 16) <= 100 * 1024)) &&
-        g.H * g.W * g.IC < (1ll << 31) &&
+        g.H * g.ish < (1ll << 31) &&
         g.N * g.OH < (1ll << 30) && g.OC < (1 << 24) && g.KY * g.KX * g.IC < (1 << 16)) {
         RowsGeom rg{};
         const int cpt = (int)g.IC / 16;
@@ -3021,7 +3255,8 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             // Eight waves (two per SIMD: one wave's reads and loads issue under the other's MFMAs) win at every K
             // (8192^3: 466 us against 483 us with four waves of 128 x 128).  VPX_GEMM_WAVES=4|8 overrides.
             const int waves_knob = knobs.gemm_waves.load();
-            const int nw = tile == 128 ? 4 : (waves_knob ? waves_knob : 8);
+            // (an fp16 output exists in the eight-wave form of the large tile only: the knob does not apply to it)
+            const int nw = tile == 128 ? 4 : (out_f16 ? 8 : (waves_knob ? waves_knob : 8));
             const dim3 grid((unsigned)(per_xcd * 8), (unsigned)G), block(64 * nw);
             const int64_t nk = g.IC / 64;
             const bool shortk = tile == 128 && nk <= 3 && !out_f16;
@@ -3033,14 +3268,16 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             lds += kGemmLdsHead;
             GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi};
             const int32_t* colsum = nullptr;  // the kernel sums the columns of B itself, from the fragments it reads
-            const GemmRows rows{is_gemm ? 0 : 1, (int)g.OW, (int)(g.OH * g.OW), g.SX, g.SY, (int)g.W, (int)(g.H * g.W)};
+            const GemmRows rows{picks_rows ? 1 : 0, vin.sw, (int)g.OW, (int)(g.OH * g.OW), (unsigned)(g.SX * vin.sw), (unsigned)(g.SY * vin.sh),
+                                (unsigned)vin.sn};
+            const GemmOut dst{vout.flat == 2 ? 1 : 0, vout.sn, vout.sh, vout.sw, (int)g.OW, (int)(g.OH * g.OW), g.out_bits};
 #define VPX_GEMM_W(U8, SGN, NW, TILE, SHORTK)                                                                        \
     do {                                                                                                             \
         auto kern = nce_gemm_mfma<U8, SGN, NW, TILE, SHORTK>;                                                        \
         rc = set_dyn_lds(kern, lds);                                                                                 \
         if (rc) return rc;                                                                                           \
         hipLaunchKernelGGL(kern, grid, block, lds, s, (const int8_t*)t.input, (const int8_t*)wptr,              \
-                           t.weight_table, colsum, (uint8_t*)t.output, Mtot, g.OC, g.IC, tiles_m, tiles_n, gp, rows); \
+                           t.weight_table, colsum, (uint8_t*)t.output, Mtot, g.OC, g.IC, tiles_m, tiles_n, gp, rows, dst); \
     } while (0)
 #define VPX_GEMM(U8, SGN)                                                                                            \
     do {                                                                                                             \
@@ -3084,7 +3321,8 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             // at stride 2: 7.5 against 7.1).
             const size_t out_stride = out_f16 ? kPatchOutStrideF16 : kPatchOutStride;  // staging bytes per position
             // (the weights-in-registers kernel stores bytes straight from its registers: integer outputs only)
-            if (!out_f16 && g.IC == 64 && g.KY == 3 && g.KX == 3 && (first < 0 || (first == 0 && g.N * g.OH * g.OW >= 50000))) {
+            if (!out_f16 && g.IC == 64 && g.KY == 3 && g.KX == 3 && g.H * g.ish < (1ll << 31) &&
+                (first < 0 || (first == 0 && g.N * g.OH * g.OW >= 50000))) {
                 PatchGeom pg{};
                 const int64_t PS = g.IC + 16, WS = Ktot + 16;
                 auto need = [&](int R) {

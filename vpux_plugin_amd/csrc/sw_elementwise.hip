@@ -1952,15 +1952,19 @@ int dequantize_axis_impl(const MemRef& in, const MemRef& out, const double* scal
 }  // namespace
 
 int release_axis_tables(int dev, hipStream_t s) {
+    // every table of the stream leaves the cache and is freed; the first failure, if any, is what the call returns
     std::lock_guard<std::mutex> lock(g_axis_mutex);
+    hipError_t first = hipSuccess;
     for (auto it = g_axis_tables.begin(); it != g_axis_tables.end();) {
         if (it->second.dev == dev && it->second.stream == s) {
-            VPX_HIP_CHECK(hipFree(it->second.table));
+            const hipError_t e = hipFree(it->second.table);
+            if (e != hipSuccess && first == hipSuccess) first = e;
             it = g_axis_tables.erase(it);
         } else {
             ++it;
         }
     }
+    VPX_HIP_CHECK(first);
     return VPX_RESULT_SUCCESS;
 }
 

@@ -679,6 +679,14 @@ int launch_fused_groups(const half_t* in, half_t* out, int64_t groups, int64_t g
     int rc = device_compute_units(&cus);
     if (rc) return rc;
     if (groups > cus || groups > kFusedMaxGroups) return VPX_RESULT_SUCCESS;
+    // In place (or any overlap of the two tensors): a workgroup whose wait runs out reads its whole group again, and by
+    // then other workgroups may have stored their normalised slices over it.  The two-launch kernels finish every
+    // read of the statistics before the first store, so overlapping tensors go there.
+    {
+        const uintptr_t ib = reinterpret_cast<uintptr_t>(in), ob = reinterpret_cast<uintptr_t>(out);
+        const uintptr_t bytes = (uintptr_t)(groups * group_size) * sizeof(half_t);
+        if (ib < ob + bytes && ob < ib + bytes) return VPX_RESULT_SUCCESS;
+    }
     int64_t wpg = cus / groups;  // (two workgroups per compute unit measured 1.2 us slower at [4,256,64,64])
     if (wpg > kMergeInKernel) wpg = kMergeInKernel;
     const int64_t words = group_size / 8;
@@ -1409,6 +1417,12 @@ int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool n
     const half_t* pi = (const half_t*)in.data;
     half_t* po = (half_t*)out.data;
     const int nv = normalize_variance ? 1 : 0;
+    {   // in place is served (every kernel reads a value before it stores that value's result); any other overlap is not
+        const uintptr_t ib = reinterpret_cast<uintptr_t>(pi), ob = reinterpret_cast<uintptr_t>(po);
+        const uintptr_t bytes = (uintptr_t)total * sizeof(half_t);
+        VPX_REQUIRE(ib == ob || ib + bytes <= ob || ob + bytes <= ib, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "mvn1: input and output overlap without being the same tensor");
+    }
 
     int64_t groups, group_size;
     if (across_channels) {

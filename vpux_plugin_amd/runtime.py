@@ -71,7 +71,8 @@ class NceTask(C.Structure):
                 ("output_type", C.c_int32), ("N", C.c_int64), ("H", C.c_int64), ("W", C.c_int64), ("IC", C.c_int64),
                 ("OC", C.c_int64), ("kernel_size", C.c_int32 * 2), ("kernel_strides", C.c_int32 * 2),
                 ("kernel_padding", C.c_int32 * 4), ("zp_in", C.c_int32), ("zp_w", C.c_int32), ("zp_out", C.c_int32),
-                ("ppe", PpeInt), ("eltwise_type", C.c_int32), ("groups", C.c_int32)]
+                ("ppe", PpeInt), ("eltwise_type", C.c_int32), ("groups", C.c_int32),
+                ("input_strides", C.c_int64 * 4), ("weights_strides", C.c_int64 * 4), ("output_strides", C.c_int64 * 4)]
 
 
 NCE_CONV, NCE_ELTWISE = 0, 4
@@ -473,11 +474,20 @@ def softmax(x, out, axis, pad_size=0, order=None, packed=True, stream=None):
     return out
 
 
+def _view_strides(field, x):
+    """N, H, W, C strides (elements) of a 4-D tensor that is a view of a larger one; a contiguous tensor leaves the
+    field zeroed, which is the task's dense default."""
+    if not x.is_contiguous():
+        for i, v in enumerate(x.stride()[-4:]):
+            field[i] = v
+
+
 def nce_task(inp, weights, weight_table, out, ppe, zp_in=0, zp_w=0, zp_out=0, strides=(1, 1),
              pads=(0, 0, 0, 0), stream=None, groups=None):
     """inp NHWC, weights [OC,KY,KX,IC], weight_table [OC,4] int32 (device), out NHWC.
     pads = (left, right, top, bottom).  With groups=G every tensor carries a leading dimension of G
-    (dense), and the G tasks go down in one call."""
+    (dense), and the G tasks go down in one call.  inp and out may be views of larger tensors (a channel slice,
+    a window in H or W): their strides go into the task."""
     if groups is not None:
         assert inp.shape[0] == weights.shape[0] == weight_table.shape[0] == out.shape[0] == groups
         assert all(x.is_contiguous() for x in (inp, weights, weight_table, out))
@@ -496,6 +506,10 @@ def nce_task(inp, weights, weight_table, out, ppe, zp_in=0, zp_w=0, zp_out=0, st
         t.kernel_padding[i] = pads[i]
     t.zp_in, t.zp_w, t.zp_out = zp_in, zp_w, zp_out
     t.ppe = ppe
+    if groups is None:
+        assert weights.is_contiguous() and weight_table.is_contiguous()
+        _view_strides(t.input_strides, inp)
+        _view_strides(t.output_strides, out)
     check(lib().vpx_nce_task(C.byref(t), _stream_handle(stream)))
     return out
 
@@ -514,6 +528,9 @@ def nce_eltwise(in1, in2, out, ppe, zp_in1=0, zp_in2=0, zp_out=0, subtract=False
     t.kernel_size[0] = t.kernel_size[1] = t.kernel_strides[0] = t.kernel_strides[1] = 1
     t.zp_in, t.zp_w, t.zp_out = zp_in1, zp_in2, zp_out
     t.ppe = ppe
+    _view_strides(t.input_strides, in1)
+    _view_strides(t.weights_strides, in2)
+    _view_strides(t.output_strides, out)
     check(lib().vpx_nce_task(C.byref(t), _stream_handle(stream)))
     return out
 
