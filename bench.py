@@ -187,6 +187,25 @@ def make_c4(rt):
                     step, nbytes, ops, "mfma", "int8", "nce_conv_regw", cpu, (3136, 100352, "output positions"))
 
 
+def make_conv64(rt, name, N, H, W):
+    """3x3, 64 -> 64 channels, stride 1, padding 1, ReLU: the C4 layer at other sizes (not a BASELINE config)."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(17)
+    inp = torch.randint(0, 256, (N, H, W, 64), dtype=torch.uint8, device="cuda", generator=g)
+    w = torch.randint(-127, 128, (64, 3, 3, 64), dtype=torch.int8, device="cuda", generator=g)
+    rng = np.random.default_rng(17)
+    wt = _dev(rt.make_weights_table(rng.integers(2 ** 14, 2 ** 15, 64), rng.integers(20, 25, 64),
+                                    rng.integers(-2 ** 15, 2 ** 15, 64).astype(np.int32), 9 * 64))
+    out = torch.empty((N, H, W, 64), dtype=torch.uint8, device="cuda")
+    ppe = rt.PpeInt(rt.PPE_NOOP, 0, 255, 1, 0)
+    task = _nce_task(rt, inp, w, wt, out, ppe, 128, 0, (1, 1), (1, 1, 1, 1))
+    step = _nce_step(rt, task)
+    step.keep = (inp, w, wt, out, task)
+    ops = 2 * N * H * W * 64 * 9 * 64
+    return Workload(name, "int8 Conv 3x3 s1 p1 NHWC [%d,%d,%d,64] u8 zp128 x [64,3,3,64] i8, ReLU clamp (not a BASELINE config)" % (N, H, W),
+                    step, inp.numel() + out.numel() + w.numel() + wt.numel() * 4, ops, "mfma", "int8", "nce_conv_regw")
+
+
 def make_stem(rt):
     """The first layer of a ResNet-50 with the image channels padded to 16: not a BASELINE config."""
     import torch
@@ -439,6 +458,8 @@ MAKERS = {
     "x_activation_hswish": make_activation,
     "x_mvn1_three_steps": make_mvn_steps,
     "x_stem_conv": make_stem,
+    "x_large_conv": lambda rt: make_conv64(rt, "x_large_conv", 128, 56, 56),
+    "x_wide_conv": lambda rt: make_conv64(rt, "x_wide_conv", 32, 112, 112),
     "x_small_plane_conv": make_small_plane_conv,
 }
 
@@ -614,12 +635,38 @@ OTHER_CONFIGS = ["c1_fake_quantize", "c2_softmax", "c3_mvn", "c4_conv", "c5_dequ
 EXTRA_CONFIGS = ["c5_nce_eltwise", "x_mvn6_layernorm", "x_activation_hswish", "x_mvn1_three_steps", "x_stem_conv", "x_small_plane_conv"]
 
 
+def coissue_table(rt, iters=20000):
+    """vpx_calib_coissue over every vector instruction kind and both MFMA shapes: nanoseconds per round when every wave
+    multiplies, when every wave runs the vector instructions, when the two waves of a SIMD do one each, and when every
+    wave does both (four vector instructions behind each MFMA).  One JSON line."""
+    import torch
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty((cus * 8192,), device="cuda", dtype=torch.uint8)
+    rows = []
+    for wide in (1, 0):
+        for kind, name in enumerate(rt.COISSUE_KINDS):
+            ns = []
+            for mode in range(4):
+                rt.calib_coissue(kind, wide, mode, 200, sink)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                rt.calib_coissue(kind, wide, mode, iters, sink)
+                e1.record()
+                torch.cuda.synchronize()
+                ns.append(round(e0.elapsed_time(e1) * 1e6 / iters, 1))
+            rows.append({"mfma": "32x32x32" if wide else "16x16x64", "valu": name, "ns_per_round_all_mfma": ns[0], "ns_per_round_all_valu": ns[1],
+                         "ns_per_round_one_wave_each": ns[2], "ns_per_round_both_in_every_wave": ns[3]})
+    print(json.dumps({"workload": "calib_coissue", "round": "16 int8 MFMAs per multiplying wave, 64 vector instructions per vector wave, two waves per SIMD",
+                      "rows": rows}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default=HEADLINE, choices=sorted(MAKERS))
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(MAKERS) + ["calib_coissue"])
     ap.add_argument("--only", action="store_true", help="measure the headline workload only (no other_configs)")
     ap.add_argument("--extra", action="store_true", help="also measure the workloads beside the BASELINE configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
@@ -637,6 +684,9 @@ def main():
     rt.lib()
     torch.cuda.set_device(0)
 
+    if args.workload == "calib_coissue":
+        coissue_table(rt)
+        return
     t_start = time.perf_counter()
     w, rec = measure(args.workload, rt, args.steps, args.warmup, args.rotate, cpu=not args.no_cpu)
     line = {

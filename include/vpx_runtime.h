@@ -240,6 +240,15 @@ VPX_API int vpx_set_tuning(const char* knob, const char* value);
  * that receives the accumulators; `*ops` (may be NULL) is set to the integer operations the launch performs. */
 VPX_API int vpx_calib_mfma_i8(const void* operands, void* sink, int iters, int fragment_reads, int64_t* ops, void* stream);
 
+/* Measurement aid (no counterpart in the reference): whether vector-ALU instructions of one wave run under the MFMAs of
+ * the other wave of its SIMD.  One workgroup of eight waves (two per SIMD) per compute unit; a round is sixteen int8 MFMAs
+ * (`wide_mfma` non-zero: 32x32x32, else 16x16x64) for a wave that multiplies and sixty-four instructions of `valu_kind`
+ * (0 v_fma_f64, 1 v_fma_f32, 2 v_add_u32, 3 v_mul_lo_u32, 4 v_mad_u64_u32, 5 v_cvt_f64_i32) for a wave that does not.
+ * `mode` 0: every wave multiplies; 1: every wave runs the vector instructions; 2: waves 0-3 multiply while waves 4-7 run
+ * the vector instructions; 3: every wave does both, four vector instructions behind each MFMA.  `sink`: 8 KiB of device
+ * memory per compute unit.  The caller times the launch; time / iters is the length of a round. */
+VPX_API int vpx_calib_coissue(int valu_kind, int wide_mfma, int mode, int iters, void* sink, void* stream);
+
 /* Name of the device kernel the last successful vpx_nce_task on this thread dispatched to
  * ("" before the first); for tests and profiles. */
 VPX_API const char* vpx_nce_last_kernel(void);

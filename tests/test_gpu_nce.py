@@ -455,18 +455,21 @@ def test_row_patch_conv_wide_image(rt, orc, dev):
     assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
 
 
-@pytest.fixture(params=[("8", "256"), ("4", "256"), ("4", "128")], ids=["8w256", "4w256", "4w128"])
+@pytest.fixture(params=[("8", "256", None), ("8", "256", "on"), ("4", "256", None), ("4", "128", None)], ids=["8w256", "8w256pp", "4w256", "4w128"])
 def gemm_waves(request, rt):
-    """The shapes of the matmul kernel: 256 x 256 tiles with two waves per SIMD (128 x 64 each) or one (128 x 128), and
-    128 x 128 tiles (four waves of 64 x 64), which small problems select by themselves."""
+    """The shapes of the matmul kernel: 256 x 256 tiles with two waves per SIMD (128 x 64 each; "pp": the two taking turns
+    at the MFMAs, where K is a multiple of 256) or one (128 x 128), and 128 x 128 tiles (four waves of 64 x 64), which
+    small problems select by themselves."""
     rt.set_tuning("VPX_GEMM_WAVES", request.param[0])
     rt.set_tuning("VPX_GEMM_TILE", request.param[1])
+    rt.set_tuning("VPX_GEMM_PINGPONG", request.param[2])
     yield request.param
     rt.set_tuning("VPX_GEMM_WAVES", None)
     rt.set_tuning("VPX_GEMM_TILE", None)
+    rt.set_tuning("VPX_GEMM_PINGPONG", None)
 
 
-@pytest.mark.parametrize("M,K,N", [(256, 64, 256), (300, 128, 520), (1, 64, 1), (513, 256, 77), (1024, 512, 768)])
+@pytest.mark.parametrize("M,K,N", [(256, 64, 256), (300, 128, 520), (1, 64, 1), (513, 256, 77), (1024, 512, 768), (700, 1024, 300)])
 def test_matmul_gemm_path(rt, orc, dev, gemm_waves, M, K, N):
     rng = np.random.default_rng(70 + M)
     for in_u8, zp in ((False, 3), (True, 128), (False, 0), (True, 11)):

@@ -745,6 +745,11 @@ int vpx_calib_mfma_i8(const void* operands, void* sink, int iters, int fragment_
     return calib_mfma_i8(operands, sink, iters, fragment_reads, ops, static_cast<hipStream_t>(stream));
 }
 
+int vpx_calib_coissue(int valu_kind, int wide_mfma, int mode, int iters, void* sink, void* stream) {
+    last_error().clear();
+    return calib_coissue(valu_kind, wide_mfma, mode, iters, sink, static_cast<hipStream_t>(stream));
+}
+
 const char* vpx_nce_last_kernel(void) {
     return g_last_nce_kernel;
 }

@@ -69,7 +69,106 @@ __global__ __launch_bounds__(kCalibThreads) void calib_mfma_i8_kernel(const v4i*
     sink[(size_t)blockIdx.x * kCalibThreads + threadIdx.x] = s;
 }
 
+// Does the vector ALU work of one wave run under the MFMAs of the other wave of its SIMD?  Eight waves, two per SIMD.
+// A round is sixteen MFMAs for an MFMA wave and sixty-four instructions of one kind for a vector wave.
+//   mode 0: every wave multiplies; 1: every wave runs the vector instructions; 2: waves 0-3 multiply and waves 4-7 (their
+//   SIMD partners) run the vector instructions; 3: every wave does both, four vector instructions behind each MFMA.
+// If the two kinds overlap, mode 2 takes as long as the longer of the two alone on one wave (half of mode 0 or 1).
+enum { CO_FMA_F64 = 0, CO_FMA_F32, CO_ADD_U32, CO_MUL_LO_U32, CO_MAD_U64_U32, CO_CVT_F64_I32, CO_KINDS };
+
+template <int KIND>
+__device__ __forceinline__ void co_valu4(unsigned (&x)[8], unsigned long long (&y)[4], int base) {
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int i = (base + u) & 7, j = (base + u) & 3;
+        if (KIND == CO_FMA_F64) asm volatile("v_fma_f64 %0, %0, %1, %1" : "+v"(y[j]) : "v"(y[(j + 1) & 3]));
+        else if (KIND == CO_FMA_F32) asm volatile("v_fma_f32 %0, %0, %1, %1" : "+v"(x[i]) : "v"(x[(i + 1) & 7]));
+        else if (KIND == CO_ADD_U32) asm volatile("v_add_u32 %0, %0, %1" : "+v"(x[i]) : "v"(x[(i + 1) & 7]));
+        else if (KIND == CO_MUL_LO_U32) asm volatile("v_mul_lo_u32 %0, %0, %1" : "+v"(x[i]) : "v"(x[(i + 1) & 7]));
+        else if (KIND == CO_MAD_U64_U32) asm volatile("v_mad_u64_u32 %0, vcc, %1, %2, %0" : "+v"(y[j]) : "v"(x[i]), "v"(x[(i + 1) & 7]) : "vcc");
+        else asm volatile("v_cvt_f64_i32 %0, %1" : "=v"(y[j]) : "v"(x[i]));
+    }
+}
+
+template <int KIND, bool WIDE>
+__global__ __launch_bounds__(kCalibThreads) void calib_coissue_kernel(v4i* __restrict__ sink, int iters, int mode) {
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const bool do_mfma = mode == 0 || mode == 3 || (mode == 2 && wave < 4);
+    const bool do_valu = mode == 1 || (mode == 2 && wave >= 4);
+    v16i acc32[4];
+    v4i acc16[8];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) acc32[i][j] = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc16[i] = v4i{0, 0, 0, 0};
+    const v4i a = {(int)threadIdx.x * 0x01030507, 0x11223344, (int)threadIdx.x, 0x7f7f7f7f}, b = {0x01020304, (int)threadIdx.x * 77, 0x55aa55aa, 3};
+    unsigned x[8];
+    unsigned long long y[4];
+#pragma unroll
+    for (int i = 0; i < 8; i++) x[i] = threadIdx.x * 2654435761u + i;
+#pragma unroll
+    for (int i = 0; i < 4; i++) y[i] = 0x3ff0000000000000ull + threadIdx.x + i;  // doubles near 1
+    if (mode == 3) {
+        for (int it = 0; it < iters; it++)
+#pragma unroll
+            for (int m = 0; m < 16; m++) {
+                if (WIDE) acc32[m & 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc32[m & 3], 0, 0, 0);
+                else acc16[m & 7] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc16[m & 7], 0, 0, 0);
+                co_valu4<KIND>(x, y, 4 * m);
+            }
+    } else if (do_mfma) {
+        for (int it = 0; it < iters; it++)
+#pragma unroll
+            for (int m = 0; m < 16; m++) {
+                if (WIDE) acc32[m & 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc32[m & 3], 0, 0, 0);
+                else acc16[m & 7] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc16[m & 7], 0, 0, 0);
+            }
+    } else if (do_valu) {
+        for (int it = 0; it < iters; it++)
+#pragma unroll
+            for (int m = 0; m < 16; m++) co_valu4<KIND>(x, y, 4 * m);
+    }
+    v4i sres = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 16; j++) sres[j & 3] += acc32[i][j];
+#pragma unroll
+    for (int i = 0; i < 8; i++) sres += acc16[i];
+#pragma unroll
+    for (int i = 0; i < 8; i++) sres[i & 3] += (int)x[i];
+#pragma unroll
+    for (int i = 0; i < 4; i++) sres[i] += (int)(y[i] >> 20);
+    sink[(size_t)blockIdx.x * kCalibThreads + threadIdx.x] = sres;
+}
+
 }  // namespace
+
+int calib_coissue(int valu_kind, int wide_mfma, int mode, int iters, void* sink, hipStream_t s) {
+    if (!sink || iters < 1 || valu_kind < 0 || valu_kind >= CO_KINDS || mode < 0 || mode > 3)
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "calib_coissue: null buffer, iters < 1, or an unknown kind / mode");
+    int blocks = 0;
+    if (const int rc = device_compute_units(&blocks)) return rc;
+#define VPX_CO(K)                                                                                                      \
+    case K:                                                                                                            \
+        if (wide_mfma) hipLaunchKernelGGL((calib_coissue_kernel<K, true>), dim3(blocks), dim3(kCalibThreads), 0, s, static_cast<v4i*>(sink), iters, mode); \
+        else hipLaunchKernelGGL((calib_coissue_kernel<K, false>), dim3(blocks), dim3(kCalibThreads), 0, s, static_cast<v4i*>(sink), iters, mode); \
+        break
+    switch (valu_kind) {
+        VPX_CO(CO_FMA_F64);
+        VPX_CO(CO_FMA_F32);
+        VPX_CO(CO_ADD_U32);
+        VPX_CO(CO_MUL_LO_U32);
+        VPX_CO(CO_MAD_U64_U32);
+    default:
+        VPX_CO(CO_CVT_F64_I32);
+    }
+#undef VPX_CO
+    if (hipGetLastError() != hipSuccess) return fail(VPX_RESULT_ERROR_UNKNOWN, "calib_coissue: launch failed");
+    return VPX_RESULT_SUCCESS;
+}
 
 int calib_mfma_i8(const void* operands, void* sink, int iters, int fragment_reads, int64_t* ops, hipStream_t s) {
     if (!operands || !sink || iters < 1) return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "calib_mfma_i8: null buffer or iters < 1");

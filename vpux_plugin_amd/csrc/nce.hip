@@ -128,6 +128,8 @@ bool set_knob(const char* knob, const char* value) {
         g_tuning.gemm_tile = *v ? (std::atoi(v) == 128 ? 128 : 256) : 0;
     } else if (!std::strcmp(knob, "VPX_GEMM_WAVES")) {
         g_tuning.gemm_waves = *v ? (std::atoi(v) == 4 ? 4 : 8) : 0;
+    } else if (!std::strcmp(knob, "VPX_GEMM_PINGPONG")) {
+        g_tuning.gemm_pingpong = !std::strcmp(v, "on") ? 1 : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_KERNEL")) {
         g_tuning.conv_stream = !std::strcmp(v, "stream") ? 2 : (!std::strcmp(v, "tile") ? 1 : (!std::strcmp(v, "regw") ? -1 : 0));
     } else if (!std::strcmp(knob, "VPX_CONV_ROWS")) {
@@ -151,7 +153,7 @@ bool set_knob(const char* knob, const char* value) {
 
 const Tuning& tuning() {
     std::call_once(g_tuning_once, [] {
-        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_COLS", "VPX_CONV_WAVES", "VPX_STREAM_KSPLIT", "VPX_MVN_FUSED"})
+        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_GEMM_PINGPONG", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_COLS", "VPX_CONV_WAVES", "VPX_STREAM_KSPLIT", "VPX_MVN_FUSED"})
             if (const char* v = std::getenv(k)) set_knob(k, v);
     });
     return g_tuning;
@@ -496,7 +498,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                                 (unsigned)vin.sn};
             const GemmOut dst{vout.flat == 2 ? 1 : 0, vout.sn, vout.sh, vout.sw, (int)g.OW, (int)(g.OH * g.OW), g.out_bits};
             const GemmLaunch gl{(const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, (uint8_t*)t.output, Mtot, g.OC, g.IC, G,
-                                tile, nw, shortk, in_u8, out_f16 ? OUT_F16 : (out_signed ? OUT_I8 : OUT_U8), gp, rows, dst};
+                                tile, nw, shortk, in_u8, knobs.gemm_pingpong.load() != 0, out_f16 ? OUT_F16 : (out_signed ? OUT_I8 : OUT_U8), gp, rows, dst};
             rc = launch_gemm_mfma(gl, s);
             if (rc) return rc;
             *kernel_name = "nce_gemm_mfma";
@@ -504,7 +506,6 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
         }
 
         // Preferred: input patch in LDS, one launch.  R = output rows per workgroup.
-        // (an fp16 output takes the gather kernel below: the tile kernels' epilogues stage bytes)
         if (allow_lds && g.IC % 64 == 0 && g.OW <= 32 * kPatchMaxMT && g.N * g.OH < (1ll << 30) && Ktot < (1 << 20) &&
             g.IC < (1 << 14) && g.W * g.SX < (1 << 14) && g.N * g.OH * g.OW < (1ll << 31)) {
             // IC of 64 or 128: the one-tile-per-workgroup kernel with padded LDS rows (a tap's fragments of more

@@ -611,6 +611,7 @@ struct Tuning {
     std::atomic<int> nce_kernel{NCE_AUTO};  // VPX_NCE_KERNEL = naive | gather | conv: restrict the choice to slower, more general paths
     std::atomic<int> gemm_tile{0};          // VPX_GEMM_TILE = 128 | 256 (0: chosen from the shape)
     std::atomic<int> gemm_waves{0};         // VPX_GEMM_WAVES = 4 | 8
+    std::atomic<int> gemm_pingpong{0};      // VPX_GEMM_PINGPONG = on | off: the waves of a SIMD take turns at the MFMAs
     std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = regw | tile | stream: start the choice of LDS-patch kernel at this one (-1, 1, 2; 0: by size)
     std::atomic<int> conv_rows{0};          // VPX_CONV_ROWS = n: cap on the output rows per workgroup of the LDS-patch kernels
     std::atomic<int> conv_cols{0};          // VPX_CONV_COLS = n: output columns per tile of the row-patch kernel
@@ -640,7 +641,7 @@ struct GemmLaunch {
     uint8_t* out;
     int64_t M, N, K, G;
     int tile, waves;
-    bool shortk, in_u8;
+    bool shortk, in_u8, pingpong;
     int out_kind;  // OutKind
     GemmPpe ppe;
     GemmRows rows;

@@ -19,7 +19,13 @@ namespace {
 // so that the MFMAs of the second sub-step cover the first fragment reads of panel kt+1.  The column sums of B that the zero-point
 // term needs come from nce_colsum_kernel (only when that term is not zero), and the per-column PPE
 // parameters are unpacked from the weight table in the epilogue.
-template <bool IN_U8, int OUT, int NW, int TILE = 256, bool SHORTK = false>
+//
+// PP (eight waves, large tile, K a multiple of four panels): the two waves of a SIMD take turns.  While one runs the
+// sixteen MFMAs of a panel back to back at raised priority, the other issues everything else it has to -- the twelve
+// fragment reads of its next panel, its four panel loads, the column sums -- and at a workgroup barrier they swap,
+// twice per panel.  (With both waves running the same interleaved stream their loads and reads fall on the same
+// moments and the MFMA pipe waits for both.)
+template <bool IN_U8, int OUT, int NW, int TILE = 256, bool SHORTK = false, bool PP = false>
 __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restrict__ A, const int8_t* __restrict__ B,
                                                      const int32_t* __restrict__ wt, const int32_t* __restrict__ colsum,
                                                      uint8_t* __restrict__ out,
@@ -260,9 +266,92 @@ __global__ __launch_bounds__(64 * NW) void nce_gemm_mfma(const int8_t* __restric
             }
         }
     };
-    // (a matmul of at most three panels is all epilogue: there every wave sums its own columns and nothing is handed over)
-    if (SHORTK || wm0 == 0) main_loop(std::true_type{});
-    else main_loop(std::false_type{});
+    // Waves w and w + 4 share a SIMD.  Half-steps are counted from 0; in half-step h the first four waves (the tile's upper
+    // half) multiply panel h / 2 when h is even and do their memory work when it is odd, the other four the other way
+    // round, one half-step behind.  Panel p sits in buffer p % 4, and its loads are issued three panels ahead: by the
+    // lower waves in half-step 2 (p - 3), by the upper ones in 2 (p - 3) + 1; the buffer they write held panel p - 4, whose
+    // last fragment reads were consumed by MFMAs two half-steps earlier.  Before the barrier that ends an even
+    // half-step 2 k every wave waits for its own loads of panel k + 1, so behind that barrier the panel is complete.
+    auto pingpong_loop = [&]() {
+        static_assert(!PP || (NW == 8 && TILE == 256 && !SHORTK), "wave roles alternate on the eight-wave large tile");
+        auto read_panel = [&](auto stage_c) {
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int n = 0; n < TM + TN; n++) load_frag_static(stage_c, kk, kk, n);
+        };
+        auto dma_panel = [&](int p) {
+#pragma unroll
+            for (int d = 0; d < 2 * DMA_PER_WAVE; d++) dma_one(std::false_type{}, p, d);
+        };
+        auto mfma_panel = [&]() {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    i32x4 a = fa[kk][i];
+                    if (IN_U8) a ^= (int32_t)0x80808080;  // u8 -> s8 (value - 128)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, fb[kk][j], acc[i][j], 0, 0, 0);
+                }
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        auto sum_panel = [&]() {  // the column sums of B from the fragments of the panel just multiplied
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int d = 0; d < 4; d++) cs[j] = __builtin_amdgcn_sdot4(fb[kk][j][d], 0x01010101, cs[j], false);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+#pragma unroll
+        for (int p = 0; p < NS - 1; p++) dma_panel(p);
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * DMA_PER_WAVE) : "memory");  // panel 0 is in
+        // (two loops, one per role: the same number of barriers in each)
+        if (wm0 == 0) {
+            read_panel(std::integral_constant<int, 0>{});
+            auto one_panel = [&](auto u_c, int k) {
+                constexpr int u = decltype(u_c)::value;
+                mfma_panel();
+                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * DMA_PER_WAVE) : "memory");  // this wave's share of panel k + 1 is in
+                sum_panel();
+                if (k + 1 < nk) read_panel(std::integral_constant<int, (u + 1) & (NS - 1)>{});
+                dma_panel(k + NS - 1);
+                asm volatile("s_barrier" ::: "memory");
+            };
+            for (int k = 0; k < nk; k += NS) {
+                one_panel(std::integral_constant<int, 0>{}, k);
+                one_panel(std::integral_constant<int, 1>{}, k + 1);
+                one_panel(std::integral_constant<int, 2>{}, k + 2);
+                one_panel(std::integral_constant<int, 3>{}, k + 3);
+            }
+        } else {
+            auto one_panel = [&](auto u_c, int k) {
+                read_panel(u_c);
+                dma_panel(k + NS - 1);
+                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * DMA_PER_WAVE) : "memory");  // likewise, with panel k + 3 just asked for
+                mfma_panel();
+                asm volatile("s_barrier" ::: "memory");
+            };
+            for (int k = 0; k < nk; k += NS) {
+                one_panel(std::integral_constant<int, 0>{}, k);
+                one_panel(std::integral_constant<int, 1>{}, k + 1);
+                one_panel(std::integral_constant<int, 2>{}, k + 2);
+                one_panel(std::integral_constant<int, 3>{}, k + 3);
+            }
+        }
+    };
+    if constexpr (PP) {
+        pingpong_loop();
+    } else {
+        // (a matmul of at most three panels is all epilogue: there every wave sums its own columns and nothing is handed over)
+        if (SHORTK || wm0 == 0) main_loop(std::true_type{});
+        else main_loop(std::false_type{});
+    }
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         csr[j] = cs[j] + __shfl_xor(cs[j], 32, 64);  // every lane takes part
@@ -419,6 +508,8 @@ int launch_gemm_mfma(const GemmLaunch& a, hipStream_t s) {
     lds += kGemmLdsHead;
     const int32_t* colsum = nullptr;  // the kernel sums the columns of B itself, from the fragments it reads
     int rc = VPX_RESULT_SUCCESS;
+    // the form in which the waves of a SIMD take turns: K a whole number of panel-buffer rounds
+    const bool pingpong = a.pingpong && tile == 256 && nw == 8 && nk % 4 == 0 && nk >= 4 && !out_f16;
 #define VPX_GEMM_W(U8, SGN, NW, TILE, SHORTK)                                                                        \
     do {                                                                                                             \
         auto kern = nce_gemm_mfma<U8, SGN, NW, TILE, SHORTK>;                                                        \
@@ -427,11 +518,20 @@ int launch_gemm_mfma(const GemmLaunch& a, hipStream_t s) {
         hipLaunchKernelGGL(kern, grid, dim3(64 * NW), lds, s, a.A, a.B, a.wt, colsum, a.out, a.M, a.N, a.K, tiles_m,  \
                            tiles_n, a.ppe, a.rows, a.dst);                                                           \
     } while (0)
+#define VPX_GEMM_PP(U8, SGN)                                                                                         \
+    do {                                                                                                             \
+        auto kern = nce_gemm_mfma<U8, SGN, 8, 256, false, true>;                                                     \
+        rc = set_dyn_lds(kern, lds);                                                                                 \
+        if (rc) return rc;                                                                                           \
+        hipLaunchKernelGGL(kern, grid, dim3(512), lds, s, a.A, a.B, a.wt, colsum, a.out, a.M, a.N, a.K, tiles_m,      \
+                           tiles_n, a.ppe, a.rows, a.dst);                                                           \
+    } while (0)
 #define VPX_GEMM(U8, SGN)                                                                                            \
     do {                                                                                                             \
         if (shortk) VPX_GEMM_W(U8, SGN, 4, 128, true);                                                               \
         else if (tile == 128) VPX_GEMM_W(U8, SGN, 4, 128, false);                                                    \
         else if (nw == 4) VPX_GEMM_W(U8, SGN, 4, 256, false);                                                        \
+        else if (pingpong) VPX_GEMM_PP(U8, SGN);                                                                     \
         else VPX_GEMM_W(U8, SGN, 8, 256, false);                                                                     \
     } while (0)
     if (out_f16) {
@@ -444,6 +544,7 @@ int launch_gemm_mfma(const GemmLaunch& a, hipStream_t s) {
     else if (a.out_kind == OUT_I8) VPX_GEMM(false, OUT_I8);
     else VPX_GEMM(false, OUT_U8);
 #undef VPX_GEMM
+#undef VPX_GEMM_PP
 #undef VPX_GEMM_W
     (void)block;
     VPX_HIP_CHECK(hipGetLastError());

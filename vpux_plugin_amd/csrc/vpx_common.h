@@ -94,6 +94,7 @@ int release_axis_tables(int dev, hipStream_t stream);
 
 // Register-only int8 MFMA loop over every compute unit (calibration of the MFMA roofline); *ops = operations enqueued.
 int calib_mfma_i8(const void* operands, void* sink, int iters, int fragment_reads, int64_t* ops, hipStream_t s);
+int calib_coissue(int valu_kind, int wide_mfma, int mode, int iters, void* sink, hipStream_t s);
 
 // Dispatch override for tests and tuning (knob names are those of the VPX_* environment variables, read once).
 int set_tuning(const char* knob, const char* value);

@@ -81,7 +81,7 @@ ELTWISE_ADD, ELTWISE_SUBTRACT = 0, 1
 
 # every symbol include/vpx_runtime.h and include/vpx_compiler_utils.h declare
 EXPORTS = ["vpx_get_last_error", "vpx_get_version", "vpx_sw_kernel_launch", "vpx_sw_kernel_launch_noalloc", "vpx_sw_kernel_supported",
-           "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_set_tuning", "vpx_workspace_reserve", "vpx_workspace_release", "vpx_calib_mfma_i8", "vpx_approximate",
+           "vpx_sw_kernel_count", "vpx_sw_kernel_name", "vpx_nce_task", "vpx_nce_last_kernel", "vpx_set_tuning", "vpx_workspace_reserve", "vpx_workspace_release", "vpx_calib_mfma_i8", "vpx_calib_coissue", "vpx_approximate",
            "vpx_eltwise_quantization_approximation", "vpx_wt_get_scale", "vpx_wt_get_bias", "vpx_get_weights_table",
            "vpx_retrieve_ppe_int", "vpx_generate_softmax_attr", "vpx_get_quant_params_attr", "vpx_create_kernel_params", "vpx_get_kernel_info",
            "vpx_float_to_half_bits", "vpx_half_bits_to_float"]
@@ -561,6 +561,15 @@ def calib_mfma_i8(operands, sink, iters, fragment_reads=False, stream=None):
     check(lib().vpx_calib_mfma_i8(operands.data_ptr(), sink.data_ptr(), int(iters), int(bool(fragment_reads)), C.byref(ops),
                                   _stream_handle(stream)))
     return ops.value
+
+
+COISSUE_KINDS = ["v_fma_f64", "v_fma_f32", "v_add_u32", "v_mul_lo_u32", "v_mad_u64_u32", "v_cvt_f64_i32"]
+
+
+def calib_coissue(valu_kind, wide_mfma, mode, iters, sink, stream=None):
+    """Enqueue the co-issue calibration loop (vpx_calib_coissue; sink: 8 KiB per compute unit on the device)."""
+    check(lib().vpx_calib_coissue(int(valu_kind), int(bool(wide_mfma)), int(mode), int(iters), C.c_void_p(sink.data_ptr()),
+                                  _stream_handle(stream)))
 
 
 def workspace_reserve(nbytes, stream=None):
