@@ -8,9 +8,11 @@ metric's first clause (int8 TOP/s) is quoted on; the same run appends `other_con
 remaining BASELINE configurations (C1 FakeQuantize, C2 softmax, C3 MVN, C4 conv, C5 dequantize and
 C5 add), each with its own roofline and CPU baseline.
 
-Every configuration is timed over a rotation of separate buffer sets whose total exceeds the 256 MB
-Infinity Cache, so a step does not find its operands in cache; the same-buffers figure and a HIP-graph
-replay are reported beside it as named extras.
+Every configuration is timed over a rotation of separate buffer sets whose total is at least 1 GiB
+(four times the 256 MB Infinity Cache), so a step does not find its operands in cache; the same-buffers
+figure, a HIP-graph replay and a steady-state figure (200 launches after 50 ms of the same launches) are
+reported beside it as named extras.  The JSON line on stdout holds numbers; the descriptions and notes of
+the configurations go to stderr.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5_matmul] [--only] [--no-cpu] [--extra]
 """
@@ -501,17 +503,33 @@ def time_steps(step, steps, warmup, graph=False):
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps
 
 
+def steady_state(step, dev_ms, launches=200, lead_ms=50.0):
+    """Device ms per step of `launches` steps that follow at least `lead_ms` of the same steps without a pause: what a
+    long run settles at, where a short one still sees clocks and caches ramp."""
+    import torch
+    lead = int(min(200000, max(1, lead_ms / max(dev_ms, 1e-4)))) + 1
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    for _ in range(lead):
+        step()
+    e0.record()
+    for _ in range(launches):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / launches
+
+
 def roofline(w, dev_ms):
     traffic = MEASURED_TRAFFIC.get(w.name)
-    src = "profiles/%s__*.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run, not measured in this run)" % w.name
     if w.bound == "hbm":
         achieved = w.bytes / (dev_ms * 1e-3) / 1e9
         return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": src if traffic else None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "kernel": w.kernel, "algorithmic_bytes": w.bytes}
     achieved = w.ops / (dev_ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": round(achieved, 2), "peak": I8_PEAK_TOPS, "unit": "TOP/s",
-            "frac": round(achieved / I8_PEAK_TOPS, 4), "traffic": traffic, "traffic_source": src if traffic else None,
+            "frac": round(achieved / I8_PEAK_TOPS, 4), "traffic": traffic,
             "kernel": w.kernel, "algorithmic_ops": w.ops}
 
 
@@ -568,7 +586,8 @@ def cpu_baseline(w, budget_s=8.0, one_thread_s=2.5):
 
 
 CACHE_BYTES = 256 << 20   # Infinity Cache of the part
-MAX_SETS = 512
+ROTATION_BYTES = 4 * CACHE_BYTES  # what the buffer sets of a configuration add up to, at least
+MAX_SETS = 2048
 
 
 def footprint(w):
@@ -578,9 +597,9 @@ def footprint(w):
 
 def build_sets(name, rt, rotate):
     """The workload plus as many further copies on separate buffers as the rotation asks for: by default enough that
-    their total is at least 1.25 times the Infinity Cache, so that a set has left the cache when its turn comes again."""
+    their total is at least four times the Infinity Cache, so that a set has left the cache when its turn comes again."""
     w = MAKERS[name](rt)
-    n = rotate if rotate > 0 else min(MAX_SETS, max(2, -(-(CACHE_BYTES * 5 // 4) // footprint(w))))
+    n = rotate if rotate > 0 else min(MAX_SETS, max(2, -(-ROTATION_BYTES // footprint(w))))
     sets = [w] + [MAKERS[name](rt) for _ in range(n - 1)]
     ring = itertools.cycle([x.step for x in sets])
 
@@ -595,18 +614,19 @@ def measure(name, rt, steps, warmup, rotate, cpu, extras=True):
     w, sets, step = build_sets(name, rt, rotate)
     wall_ms, dev_ms = time_steps(step, steps, warmup)
     value, unit = value_of(w, wall_ms)
-    rec = {"value": round(value, 2), "unit": unit, "dtype": w.dtype, "description": w.desc, "steps": steps, "warmup": warmup,
+    rec = {"value": round(value, 2), "unit": unit, "dtype": w.dtype, "steps": steps, "warmup": warmup,
            "launch": "eager", "buffer_sets": len(sets), "buffer_bytes_total": len(sets) * footprint(w),
            "ms_per_step": round(wall_ms, 6), "device_ms_per_step": round(dev_ms, 6), "roofline": roofline(w, dev_ms)}
-    if name in NOTES:
-        rec["note"] = NOTES[name]
     if extras:
         _, same_ms = time_steps(w.step, steps, min(warmup, 5))
         _, graph_ms = time_steps(step, steps, 2, graph=True)
+        steady_ms = steady_state(step, dev_ms)
         rec["extras"] = {"same_buffers_device_ms_per_step": round(same_ms, 6),
                          "same_buffers_frac": roofline(w, same_ms)["frac"],
                          "graph_device_ms_per_step": round(graph_ms, 6),
-                         "graph_frac": roofline(w, graph_ms)["frac"]}
+                         "graph_frac": roofline(w, graph_ms)["frac"],
+                         "steady_state_device_ms_per_step": round(steady_ms, 6),
+                         "steady_state_frac": roofline(w, steady_ms)["frac"]}
     if cpu:
         rec["cpu_baseline"] = cpu_baseline(w)
     del sets, step
@@ -672,7 +692,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     ap.add_argument("--rotate", type=int, default=0, metavar="N",
                     help="number of separate buffer sets a workload cycles through (default 0: as many as make their "
-                         "total exceed 1.25 x the 256 MB Infinity Cache; 1: the same buffers every step)")
+                         "total reach 4 x the 256 MB Infinity Cache; 1: the same buffers every step)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on one GPU only (every kernel shards without exchange, so N GPUs would run N independent copies); "
@@ -689,18 +709,18 @@ def main():
         return
     t_start = time.perf_counter()
     w, rec = measure(args.workload, rt, args.steps, args.warmup, args.rotate, cpu=not args.no_cpu)
+    texts = {w.name: {"description": w.desc, "note": NOTES.get(w.name)}}
     line = {
         "metric": METRIC, "value": rec["value"], "unit": rec["unit"], "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": rec["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": w.dtype, "data": "synthetic",
-        "config": {"workload": w.name, "description": w.desc, "launch": "eager", "buffer_sets": rec["buffer_sets"],
+        "config": {"workload": w.name, "launch": "eager", "buffer_sets": rec["buffer_sets"],
                    "buffer_bytes_total": rec["buffer_bytes_total"]},
         "device_ms_per_step": rec["device_ms_per_step"],
         "roofline": rec["roofline"],
         "extras": rec.get("extras"),
+        "traffic_source": "roofline.traffic: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run (profiles/<workload>__*.md), not measured in this run",
     }
-    if "note" in rec:
-        line["config"]["note"] = rec["note"]
     if "cpu_baseline" in rec:
         line["cpu_baseline"] = rec["cpu_baseline"]
     if not args.only:
@@ -708,19 +728,36 @@ def main():
         names = [n for n in OTHER_CONFIGS + [HEADLINE] + (EXTRA_CONFIGS if args.extra else []) if n != args.workload]
         for name in names:
             steps = min(args.steps, 100) if name == "c5_matmul" else args.steps
-            _, r = measure(name, rt, steps, min(args.warmup, 10), args.rotate, cpu=not args.no_cpu)
+            ow, r = measure(name, rt, steps, min(args.warmup, 10), args.rotate, cpu=not args.no_cpu)
             others[name] = r
+            texts[name] = {"description": ow.desc, "note": NOTES.get(name)}
             sys.stderr.write("bench.py: %s done at %.0f s\n" % (name, time.perf_counter() - t_start))
             sys.stderr.flush()
         line["other_configs"] = others
-        # what the MFMA pipe sustains on this part today, beside the matmul it bounds (register-only loops, no global memory)
+        # configuration 5 end to end: the matmul, the dequantize of its result and the residual add, one after the other
+        parts = {n: (rec if n == args.workload else others.get(n)) for n in ("c5_matmul", "c5_dequantize", "c5_eltwise_add")}
+        if all(parts.values()):
+            line["c5_chain"] = {"device_ms": round(sum(p["device_ms_per_step"] for p in parts.values()), 6),
+                                "steady_state_device_ms": round(sum(p["extras"]["steady_state_device_ms_per_step"] for p in parts.values()), 6),
+                                "parts": list(parts)}
+        # what the part sustains today, beside the kernels it bounds: a plain copy for the HBM side (rotated like the
+        # configurations), register-only loops of the int8 MFMA for the matrix side
         calib = {}
+        hbm = {}
+        cw, cr = measure("calib_copy", rt, args.steps, min(args.warmup, 10), args.rotate, cpu=False, extras=False)
+        hbm["calib_copy"] = {"device_ms_per_step": cr["device_ms_per_step"], "achieved": cr["roofline"]["achieved"], "unit": "GB/s",
+                               "frac_of_peak": cr["roofline"]["frac"], "buffer_sets": cr["buffer_sets"]}
+        texts["calib_copy"] = {"description": cw.desc, "note": None}
         for name in ("calib_mfma_zero", "calib_mfma_random", "calib_mfma_random_lds"):
             cw = MAKERS[name](rt)
             _, ms = time_steps(cw.step, 50, 5)
-            calib[name] = {"description": cw.desc, "device_ms_per_step": round(ms, 6), "achieved": round(cw.ops / (ms * 1e-3) / 1e12, 1),
+            calib[name] = {"device_ms_per_step": round(ms, 6), "achieved": round(cw.ops / (ms * 1e-3) / 1e12, 1),
                            "unit": "TOP/s", "frac_of_peak": round(cw.ops / (ms * 1e-3) / 1e12 / I8_PEAK_TOPS, 4)}
+            texts[name] = {"description": cw.desc, "note": None}
+        line["hbm_calibration"] = hbm
         line["mfma_calibration"] = calib
+    sys.stderr.write("bench.py: descriptions %s\n" % json.dumps(texts))
+    sys.stderr.flush()
     print(json.dumps(line), flush=True)
 
 

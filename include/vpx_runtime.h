@@ -222,11 +222,13 @@ VPX_API int vpx_nce_task(const vpx_nce_task_t* task, void* stream);
 
 /* Testing and tuning hook (no counterpart in the reference): overrides how vpx_nce_task picks its device kernel.
  * `knob` is one of "VPX_NCE_KERNEL" (naive | gather | conv), "VPX_GEMM_TILE" (128 | 256), "VPX_GEMM_WAVES" (4 | 8),
+ * "VPX_GEMM_PINGPONG" (on: the two waves of a SIMD take turns at the MFMAs of the large matmul tile; measured slower, off by default),
  * "VPX_CONV_KERNEL" (regw | tile | stream), "VPX_CONV_ROWS" (n), "VPX_CONV_COLS" (n), "VPX_CONV_WAVES" (4 | 8), "VPX_STREAM_KSPLIT" (off: the streamed-weights
  * convolution kernel gives every wave a 32 x 32 tile also on small planes, instead of splitting K over the waves of a group),
  * "VPX_MVN_FUSED" (off: long MVN groups take
  * the two-launch kernels; nowait: the one-launch kernel's workgroups do not wait for each other and each recomputes its
- * group's statistics, the path taken when they are not all resident); `value` NULL or "" restores the default.
+ * group's statistics, the path taken when they are not all resident), "VPX_CALIB_BLOCKS" (n: workgroups of
+ * vpx_calib_mfma_i8, by default one per compute unit); `value` NULL or "" restores the default.
  * Environment variables of the same names give the initial values; they are read once, at the first NCE task or the
  * first call of this function, never during a launch.  Process-wide; results do not depend on any of them. */
 VPX_API int vpx_set_tuning(const char* knob, const char* value);

@@ -45,7 +45,7 @@ def build(verbose=True, jobs=8):
     subprocess.check_call(cmd)
     # the C++ host example: the C ABI driven without Python; it links the HIP runtime itself
     exe = os.path.join(HERE, "examples", "c_abi_host")
-    cmd = [hipcc, "-O2", "-std=c++17", "-I", os.path.join(ROOT, "include"), os.path.join(HERE, "examples", "c_abi_host.cpp"),
+    cmd = [hipcc, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I", os.path.join(ROOT, "include"), os.path.join(HERE, "examples", "c_abi_host.cpp"),
            "-L", HERE, "-lvpx_amd", "-Wl,-rpath,$ORIGIN/..", "-o", exe]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -209,8 +209,12 @@ int workspace_release(hipStream_t stream) {
 // ---- blob parsing -----------------------------------------------------------------------------
 namespace {
 
+constexpr int kMaxMemRefs = VPX_MAX_KERNEL_INPUTS + VPX_MAX_KERNEL_OUTPUTS;
+
+// The operands of one launch, on the caller's stack: a launch allocates nothing on the heap.
 struct Args {
-    std::vector<MemRef> mem;
+    MemRef mem[kMaxMemRefs];
+    int n_mem = 0;
     const uint8_t* attrs = nullptr;
     size_t attrs_size = 0;
 };
@@ -227,12 +231,13 @@ bool is_compact(const MemRef& m) {
 int parse_blob(const char* entry, int n_in, int n_out, const void* params, size_t params_size,
                const vpx_memref_addr_t* addrs, uint32_t num_addrs, Args& a) {
     const int n_mem = n_in + n_out;
+    VPX_REQUIRE(n_mem <= kMaxMemRefs, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: %d operands, at most %d are supported", entry, n_mem, kMaxMemRefs);
     VPX_REQUIRE((int)num_addrs == n_mem, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: expects %d memref addresses (%d in, %d out), got %u",
                 entry, n_mem, n_in, n_out, num_addrs);
     VPX_REQUIRE(params_size >= (size_t)n_mem * sizeof(vpx_memref_data_t), VPX_RESULT_ERROR_INVALID_ARGUMENT,
                 "%s: params blob of %zu bytes cannot hold %d MemRefData records", entry, params_size, n_mem);
     const uint8_t* p = (const uint8_t*)params;
-    a.mem.resize(n_mem);
+    a.n_mem = n_mem;
     size_t tail = 0;
     bool tail_needed = false;
     for (int i = 0; i < n_mem; i++) {
@@ -499,8 +504,16 @@ const Entry kEntries[] = {
 constexpr uint32_t kNumEntries = sizeof(kEntries) / sizeof(kEntries[0]);
 
 const Entry* find_entry(const char* name) {
+    // callers pass the same string again and again: the last pointer's entry is checked first (one comparison)
+    thread_local const char* last_name = nullptr;
+    thread_local const Entry* last_entry = nullptr;
+    if (name == last_name && last_entry != nullptr && strcmp(last_entry->name, name) == 0) return last_entry;
     for (uint32_t i = 0; i < kNumEntries; i++)
-        if (strcmp(kEntries[i].name, name) == 0) return &kEntries[i];
+        if (strcmp(kEntries[i].name, name) == 0) {
+            last_name = name;
+            last_entry = &kEntries[i];
+            return last_entry;
+        }
     return nullptr;
 }
 
@@ -568,16 +581,16 @@ static int sw_kernel_launch(const char* entry, const void* params, size_t params
         return launch_fake_quantize(a.mem[0], &a.mem[1], a.mem[5], levels, s);
     }
     case K_QUANT: {
-        std::vector<double> scales;
-        std::vector<int64_t> zps;
+        thread_local std::vector<double> scales;  // (their storage is kept from launch to launch)
+        thread_local std::vector<int64_t> zps;
         rc = read_quant_params(entry, a, a.mem[0].dtype, scales, zps);
         if (rc) return rc;
         if (scales.size() == 1) return launch_quantize(a.mem[0], a.mem[1], scales[0], zps[0], s);
         return launch_quantize_per_axis(a.mem[0], a.mem[1], scales.data(), zps.data(), (int64_t)scales.size(), s);
     }
     case K_DEQUANT: {
-        std::vector<double> scales;
-        std::vector<int64_t> zps;
+        thread_local std::vector<double> scales;  // (their storage is kept from launch to launch)
+        thread_local std::vector<int64_t> zps;
         rc = read_quant_params(entry, a, a.mem[1].dtype, scales, zps);
         if (rc) return rc;
         if (scales.size() == 1) return launch_dequantize(a.mem[0], a.mem[1], scales[0], zps[0], s);
@@ -613,9 +626,9 @@ static int sw_kernel_launch(const char* entry, const void* params, size_t params
     }
     case K_DYN_QUANT: return launch_dynamic_quantize(a.mem[0], a.mem[1], a.mem[2], a.mem[3], s);
     case K_DYN_DEQUANT: {
-        VPX_REQUIRE(a.mem.size() == 3 || a.mem.size() == 4, VPX_RESULT_ERROR_INVALID_ARGUMENT,
-                    "dynamic_dequantize: expects input, scale, an optional zero point and the output, got %zu memrefs", a.mem.size());
-        const bool has_zp = a.mem.size() == 4;
+        VPX_REQUIRE(a.n_mem == 3 || a.n_mem == 4, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "dynamic_dequantize: expects input, scale, an optional zero point and the output, got %d memrefs", a.n_mem);
+        const bool has_zp = a.n_mem == 4;
         return launch_dynamic_dequantize(a.mem[0], a.mem[1], has_zp ? &a.mem[2] : nullptr, a.mem[has_zp ? 3 : 2], s);
     }
     case K_MVN6: {
@@ -625,9 +638,9 @@ static int sw_kernel_launch(const char* entry, const void* params, size_t params
         VPX_REQUIRE(read_attr(a, 0, &marker) && read_attr(a, 8, &mask) && read_attr(a, 16, &normvar) && read_attr(a, 24, &eps_mode) &&
                             read_attr(a, 32, &eps) && read_attr(a, 36, &n_axes),
                     VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: params blob is too short for its attributes");
-        VPX_REQUIRE((mask & 9) == 9 && (mask & ~15ll) == 0 && 2 + ((mask >> 1) & 1) + ((mask >> 2) & 1) == (int64_t)a.mem.size(),
-                    VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: operand mask 0x%llx does not describe %zu memrefs",
-                    (unsigned long long)mask, a.mem.size());
+        VPX_REQUIRE((mask & 9) == 9 && (mask & ~15ll) == 0 && 2 + ((mask >> 1) & 1) + ((mask >> 2) & 1) == (int64_t)a.n_mem,
+                    VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: operand mask 0x%llx does not describe %d memrefs",
+                    (unsigned long long)mask, a.n_mem);
         VPX_REQUIRE(n_axes >= 1 && n_axes <= VPX_MAX_ND_DIMS, VPX_RESULT_ERROR_INVALID_ARGUMENT, "mvn6: %lld axes", (long long)n_axes);
         int64_t axes[VPX_MAX_ND_DIMS];
         for (int64_t i = 0; i < n_axes; i++)

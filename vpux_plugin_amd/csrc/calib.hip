@@ -175,6 +175,7 @@ int calib_mfma_i8(const void* operands, void* sink, int iters, int fragment_read
     int blocks = 0;
     if (const int rc = device_compute_units(&blocks)) return rc;
     if (blocks <= 0) return fail(VPX_RESULT_ERROR_UNKNOWN, "calib_mfma_i8: no compute units reported");
+    if (const int fewer = tuning_calib_blocks(); fewer > 0 && fewer < blocks) blocks = fewer;
     const auto kernel = fragment_reads ? calib_mfma_i8_kernel<true> : calib_mfma_i8_kernel<false>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kCalibLds) != hipSuccess)
         return fail(VPX_RESULT_ERROR_UNKNOWN, "calib_mfma_i8: cannot reserve 64 KiB of LDS");

@@ -23,10 +23,17 @@ std::set<std::pair<int, const void*>> g_lds_done;
 int set_dyn_lds_attribute(const void* fn) {
     int dev = 0;
     VPX_HIP_CHECK(hipGetDevice(&dev));
+    // the kernel this thread launched last needs no lock and no search
+    thread_local int last_dev = -1;
+    thread_local const void* last_fn = nullptr;
+    if (dev == last_dev && fn == last_fn) return VPX_RESULT_SUCCESS;
     std::lock_guard<std::mutex> lock(g_lds_mutex);
-    if (g_lds_done.count({dev, fn})) return VPX_RESULT_SUCCESS;
-    VPX_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxDynLds));
-    g_lds_done.insert({dev, fn});
+    if (!g_lds_done.count({dev, fn})) {
+        VPX_HIP_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxDynLds));
+        g_lds_done.insert({dev, fn});
+    }
+    last_dev = dev;
+    last_fn = fn;
     return VPX_RESULT_SUCCESS;
 }
 
@@ -142,6 +149,8 @@ bool set_knob(const char* knob, const char* value) {
         g_tuning.stream_ksplit = (!std::strcmp(v, "off") || !std::strcmp(v, "0")) ? 0 : 1;
     } else if (!std::strcmp(knob, "VPX_MVN_FUSED")) {
         g_tuning.mvn_fused = !std::strcmp(v, "off") ? 0 : (!std::strcmp(v, "nowait") ? 2 : 1);
+    } else if (!std::strcmp(knob, "VPX_CALIB_BLOCKS")) {
+        g_tuning.calib_blocks = std::atoi(v) > 0 ? std::atoi(v) : 0;
     } else {
         return false;
     }
@@ -153,7 +162,7 @@ bool set_knob(const char* knob, const char* value) {
 
 const Tuning& tuning() {
     std::call_once(g_tuning_once, [] {
-        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_GEMM_PINGPONG", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_COLS", "VPX_CONV_WAVES", "VPX_STREAM_KSPLIT", "VPX_MVN_FUSED"})
+        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_GEMM_PINGPONG", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_COLS", "VPX_CONV_WAVES", "VPX_STREAM_KSPLIT", "VPX_MVN_FUSED", "VPX_CALIB_BLOCKS"})
             if (const char* v = std::getenv(k)) set_knob(k, v);
     });
     return g_tuning;
@@ -166,6 +175,10 @@ using namespace nce;
 
 int tuning_mvn_fused() {
     return tuning().mvn_fused.load();
+}
+
+int tuning_calib_blocks() {
+    return tuning().calib_blocks.load();
 }
 
 int set_tuning(const char* knob, const char* value) {

@@ -618,6 +618,7 @@ struct Tuning {
     std::atomic<int> conv_waves{0};         // VPX_CONV_WAVES = 4 | 8
     std::atomic<int> stream_ksplit{1};      // VPX_STREAM_KSPLIT = off: the streamed-weights kernel never splits K over its waves
     std::atomic<int> mvn_fused{1};          // VPX_MVN_FUSED = off | nowait (see tuning_mvn_fused)
+    std::atomic<int> calib_blocks{0};       // VPX_CALIB_BLOCKS = n: workgroups of the MFMA calibration loop (0: one per compute unit)
 };
 const Tuning& tuning();
 

@@ -700,7 +700,7 @@ int launch_fused_groups(const half_t* in, half_t* out, int64_t groups, int64_t g
     void* sync = nullptr;
     rc = get_sync_area(s, &sync);
     if (rc) return rc;
-    const unsigned long long spin = mode == 2 ? 0ull : 500000ull;  // 5 ms of the 100 MHz counter
+    const unsigned long long spin = mode == 2 ? 0ull : 50000ull;  // 0.5 ms of the 100 MHz counter
     const dim3 grid((unsigned)(groups * wpg)), block(kThreads);
 #define VPX_FUSED(V)                                                                                                  \
     hipLaunchKernelGGL((mvn_fused_kernel<V>), grid, block, 0, s, in, out, group_size, (int)wpg, slice, (unsigned*)sync, \

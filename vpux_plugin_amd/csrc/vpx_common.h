@@ -101,6 +101,9 @@ int set_tuning(const char* knob, const char* value);
 // VPX_MVN_FUSED: 0 = never take the one-launch MVN kernel, 1 = default, 2 = its workgroups do not wait for each other
 // (every one recomputes the group's moments: the path a workgroup takes when the others are not resident)
 int tuning_mvn_fused();
+// VPX_CALIB_BLOCKS: workgroups of the MFMA calibration loop (0: one per compute unit); fewer leave compute units free
+// for whatever another stream launches beside it
+int tuning_calib_blocks();
 
 // ---- kernel launchers (defined in the .hip files) ------------------------------------------
 int launch_convert(const MemRef& in, const MemRef& out, hipStream_t s);

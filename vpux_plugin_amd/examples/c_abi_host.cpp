@@ -3,13 +3,19 @@
 // serialises the kernel parameters the way the compiler does, and enqueues
 //   (1) a `softmax` ACT-SHAVE kernel (fp16, last axis), and
 //   (2) an NCE matmul with the integer PPE followed by `dequantize`,
-// checking both against straightforward host arithmetic.  Exit code 0 = all checks passed.
+// checking both against straightforward host arithmetic, and
+//   (3) times what a call costs the host: 10 000 launches each of an empty kernel through hipLaunchKernelGGL, of
+//       `fake_quantize` ([1,64,56,56] fp16, per tensor) and of an NCE convolution ([32,56,56,64] -> 64, 3 x 3), on the
+//       same buffers, in batches of 500 with the stream drained between batches (the clock runs while calls are
+//       enqueued, not while the GPU catches up).
+// Exit code 0 = all checks passed.
 //
 // Build (the library leaves the HIP runtime to the process, so the host links it):
 //   hipcc -O2 -std=c++17 -I include vpux_plugin_amd/examples/c_abi_host.cpp -L vpux_plugin_amd -lvpx_amd
 //         -Wl,-rpath,$PWD/vpux_plugin_amd -o c_abi_host
 #include <hip/hip_runtime.h>
 
+#include <chrono>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -44,6 +50,31 @@ static std::vector<uint8_t> make_blob(const std::vector<vpx_tensor_desc_t>& in, 
     std::vector<uint8_t> blob(size);
     vpx_create_kernel_params(in.data(), (uint32_t)in.size(), out.data(), (uint32_t)out.size(), attrs, attrs_size, blob.data(), &size);
     return blob;
+}
+
+// an empty kernel with the argument block of a typical launch (seven pointers and three words)
+struct EmptyArgs {
+    const void* p[7];
+    int64_t n[3];
+};
+__global__ void empty_kernel(EmptyArgs a, int64_t n_vec, int64_t n) {
+    if (n < 0) *(int64_t*)a.p[0] = n_vec;  // (never: keeps the arguments alive)
+}
+
+// microseconds of host time per call of `call`, over `batches` batches of `per_batch` calls
+template <class F>
+static double host_us_per_call(F&& call, hipStream_t stream, int batches = 20, int per_batch = 500) {
+    for (int i = 0; i < 50; i++) call();
+    (void)hipStreamSynchronize(stream);
+    double total = 0;
+    for (int b = 0; b < batches; b++) {
+        const auto t0 = std::chrono::steady_clock::now();
+        for (int i = 0; i < per_batch; i++) call();
+        const auto t1 = std::chrono::steady_clock::now();
+        (void)hipStreamSynchronize(stream);
+        total += std::chrono::duration<double, std::micro>(t1 - t0).count();
+    }
+    return total / ((double)batches * per_batch);
 }
 
 int main() {
@@ -169,6 +200,70 @@ int main() {
             }
         std::printf("matmul %dx%dx%d + PPE + dequantize: %ld mismatches (bit-exact expected)\n", M, K, N, mismatches);
         if (mismatches) failures++;
+    }
+
+    // ---------------------------------------------------------------- what a call costs the host
+    {
+        const EmptyArgs ea{};
+        const double bare = host_us_per_call([&] { hipLaunchKernelGGL(empty_kernel, dim3(196), dim3(256), 0, stream, ea, (int64_t)1, (int64_t)1); }, stream);
+
+        // FakeQuantize fp16 NCHW [1,64,56,56], per tensor, 256 levels
+        const size_t n_fq = (size_t)64 * 56 * 56;
+        void *fx, *fy, *frange;
+        HIP_OK(hipMalloc(&fx, n_fq * 2));
+        HIP_OK(hipMalloc(&fy, n_fq * 2));
+        HIP_OK(hipMalloc(&frange, 4 * 2));
+        HIP_OK(hipMemset(fx, 0, n_fq * 2));
+        const uint16_t range[4] = {vpx_float_to_half_bits(-4.f), vpx_float_to_half_bits(4.f), vpx_float_to_half_bits(-4.f), vpx_float_to_half_bits(4.f)};
+        HIP_OK(hipMemcpy(frange, range, sizeof(range), hipMemcpyHostToDevice));
+        const int32_t xd[4] = {56, 56, 64, 1}, od[4] = {1, 1, 1, 1};
+        const int64_t xs[4] = {16, 16 * 56, 16 * 56 * 56, 16 * 56 * 56 * 64}, os[4] = {16, 16, 16, 16};
+        vpx_tensor_desc_t tx{4, xd, xs, VPX_NN_FP16, VPX_ORDER_NCHW, VPX_LOC_DDR}, t1{4, od, os, VPX_NN_FP16, VPX_ORDER_NCHW, VPX_LOC_DDR};
+        const int64_t levels = 256;
+        const std::vector<uint8_t> fq_blob = make_blob({tx, t1, t1, t1, t1}, {tx}, &levels, 8);
+        const vpx_memref_addr_t fq_addrs[6] = {{fx, nullptr, nullptr},
+                                               {(uint16_t*)frange + 0, nullptr, nullptr},
+                                               {(uint16_t*)frange + 1, nullptr, nullptr},
+                                               {(uint16_t*)frange + 2, nullptr, nullptr},
+                                               {(uint16_t*)frange + 3, nullptr, nullptr},
+                                               {fy, nullptr, nullptr}};
+        VPX_OK(vpx_sw_kernel_launch("fake_quantize", fq_blob.data(), fq_blob.size(), fq_addrs, 6, stream));
+        const double fq = host_us_per_call([&] { (void)vpx_sw_kernel_launch("fake_quantize", fq_blob.data(), fq_blob.size(), fq_addrs, 6, stream); }, stream);
+
+        // NCE convolution u8 [32,56,56,64] -> 64 channels, 3 x 3, pad 1
+        const size_t n_in = (size_t)32 * 56 * 56 * 64, n_w = (size_t)64 * 9 * 64;
+        void *ci, *cw, *cwt, *co;
+        HIP_OK(hipMalloc(&ci, n_in));
+        HIP_OK(hipMalloc(&cw, n_w));
+        HIP_OK(hipMalloc(&cwt, 64 * 16));
+        HIP_OK(hipMalloc(&co, n_in));
+        HIP_OK(hipMemset(ci, 0x80, n_in));
+        HIP_OK(hipMemset(cw, 1, n_w));
+        std::vector<int32_t> cwt_h(64 * 4);
+        for (int n = 0; n < 64; n++) {
+            cwt_h[n * 4 + 0] = 0;
+            cwt_h[n * 4 + 1] = 0xFFFFFF;
+            cwt_h[n * 4 + 2] = vpx_wt_get_scale(22, (int16_t)20000);
+            cwt_h[n * 4 + 3] = 100;
+        }
+        HIP_OK(hipMemcpy(cwt, cwt_h.data(), cwt_h.size() * 4, hipMemcpyHostToDevice));
+        vpx_nce_task_t c{};
+        c.task_type = VPX_NCE_CONV;
+        c.input = ci; c.weights = cw; c.weight_table = (const int32_t*)cwt; c.output = co;
+        c.input_type = VPX_NN_U8; c.weights_type = VPX_NN_I8; c.output_type = VPX_NN_U8;
+        c.N = 32; c.H = 56; c.W = 56; c.IC = 64; c.OC = 64;
+        c.kernel_size[0] = c.kernel_size[1] = 3;
+        c.kernel_strides[0] = c.kernel_strides[1] = 1;
+        c.kernel_padding[0] = c.kernel_padding[1] = c.kernel_padding[2] = c.kernel_padding[3] = 1;
+        c.zp_in = 128;
+        c.ppe.mode = VPX_PPE_LRELU;
+        c.ppe.clamp_low = 0; c.ppe.clamp_high = 255;
+        c.ppe.lrelu_mult = 1; c.ppe.lrelu_shift = 0;
+        VPX_OK(vpx_nce_task(&c, stream));
+        const char* conv_kernel = vpx_nce_last_kernel();
+        const double conv = host_us_per_call([&] { (void)vpx_nce_task(&c, stream); }, stream, 20, 100);
+        std::printf("host time per call: empty kernel through hipLaunchKernelGGL %.2f us; vpx_sw_kernel_launch(fake_quantize) %.2f us "
+                    "(+%.2f); vpx_nce_task(%s) %.2f us (+%.2f)\n", bare, fq, fq - bare, conv_kernel, conv, conv - bare);
     }
     std::printf(failures ? "FAILED\n" : "OK\n");
     return failures ? 1 : 0;
