@@ -138,6 +138,34 @@ def make_c3(rt):
                     (1, 4, "batch elements"))
 
 
+def make_softmax_outer(rt):
+    """Softmax over an outer axis too long for the register slabs: [32,2048,1024] fp16 over axis 1."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = (torch.randn((32, 2048, 1024), device="cuda", generator=g) * 3).half()
+    out = torch.empty_like(x)
+    ops = [rt.Operand(x), rt.Operand(out)]
+    dims = [int(d) for d in ops[0].dims]
+    st = [int(s) // 16 for s in ops[0].strides]
+    attrs = rt.generate_softmax_attr(dims, st, st, 1, 0).tobytes()  # axis counted from the innermost dimension
+    blob = rt.create_kernel_params(ops[:1], ops[1:], attrs)
+    return Workload("x_softmax_outer_axis", "Softmax fp16 [32,2048,1024] over axis 1 (2048 steps, rows of 1024 contiguous)",
+                    _prebuilt_sw_launch(rt, "softmax", blob, ops), x.numel() * 4, 0, "hbm", "f16", "softmax_cols")
+
+
+def make_mvn_nhwc(rt):
+    """MVN per channel on a channel-minor tensor: [16,112,112,256] fp16 stored NHWC."""
+    import torch
+    g = torch.Generator(device="cuda").manual_seed(12)
+    x = (torch.rand((16, 112, 112, 256), device="cuda", generator=g) * 16 - 8).half()
+    out = torch.empty_like(x)
+    ops = [rt.Operand(x, "NHWC"), rt.Operand(out, "NHWC")]  # (operands are indexed in memory order)
+    attrs = np.asarray([0, -1], dtype=np.int64).tobytes() + np.float32(1e-9).tobytes()
+    blob = rt.create_kernel_params(ops[:1], ops[1:], attrs)
+    return Workload("x_mvn_nhwc_per_channel", "MVN fp16 per channel, NHWC storage [16,112,112,256], normalize_variance",
+                    _prebuilt_sw_launch(rt, "mvn1", blob, ops), x.numel() * 4, 0, "hbm", "f16", "mvn_nhwc kernels")
+
+
 def _nce_step(rt, task):
     import torch
     L = rt.lib()
@@ -459,6 +487,8 @@ MAKERS = {
     "x_mvn6_layernorm": make_layernorm,
     "x_activation_hswish": make_activation,
     "x_mvn1_three_steps": make_mvn_steps,
+    "x_softmax_outer_axis": make_softmax_outer,
+    "x_mvn_nhwc_per_channel": make_mvn_nhwc,
     "x_stem_conv": make_stem,
     "x_large_conv": lambda rt: make_conv64(rt, "x_large_conv", 128, 56, 56),
     "x_wide_conv": lambda rt: make_conv64(rt, "x_wide_conv", 32, 112, 112),

@@ -539,7 +539,7 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             if (!out_f16 && g.IC == 64 && g.KY == 3 && g.KX == 3 && g.H * g.ish < (1ll << 31) &&
                 (first < 0 || (first == 0 && g.N * g.OH * g.OW >= 50000))) {
                 PatchGeom pg{};
-                const int64_t PS = g.IC + 16, WS = Ktot + 16;
+                const int64_t PS = g.IC + 32, WS = Ktot + 32;  // the kernel's LDS strides of a pixel and of a weight row
                 auto need = [&](int R) {
                     return 64 * (size_t)WS + (size_t)((R - 1) * g.SY + g.KY) * (size_t)((g.OW - 1) * g.SX + g.KX) * (size_t)PS;
                 };

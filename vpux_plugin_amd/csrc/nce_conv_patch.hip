@@ -268,10 +268,14 @@ template <bool IN_U8, bool SAME_F, int KY, int KX>
 __global__ __launch_bounds__(512) void nce_conv_regw(const int8_t* __restrict__ in, const int8_t* __restrict__ w,
                                                      const int32_t* __restrict__ wt, uint8_t* __restrict__ out, ConvGeom g,
                                                      PatchGeom pg, int pad_byte, GemmPpe ppe) {
-    constexpr int BN = 64, IC = 64, PS = IC + 16, NW = 8, NT = 64 * NW, TAPS = KY * KX, Ktot = TAPS * IC, WS = Ktot + 16;
+    // LDS strides of a pixel and of a weight row: a fragment read has sixteen lanes sixteen rows apart and four such
+    // groups one 16-byte chunk apart, which LDS serves without bank conflicts when the row stride is 2 mod 4 chunks
+    // (96 and 608 bytes; measured: 80 or 592 bytes take twice as long per read)
+    constexpr int BN = 64, IC = 64, PS = IC + 32, NW = 8, NT = 64 * NW, TAPS = KY * KX, Ktot = TAPS * IC, WS = Ktot + 32;
+    static_assert((PS / 16) % 4 == 2 && (WS / 16) % 4 == 2, "conflict-free fragment reads");
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    uint8_t* const wlds = smem;             // [64][Ktot + 16], rows in tile order
-    uint8_t* const patch = smem + BN * WS;  // [PH*PW][IC + 16]
+    uint8_t* const wlds = smem;             // [64][Ktot + 32], rows in tile order
+    uint8_t* const patch = smem + BN * WS;  // [PH*PW][IC + 32]
     __shared__ int csum[BN];                // weight sums, by LDS row
 
     // A launch of a few microseconds is bound by instructions as much as by anything else: all index arithmetic below
