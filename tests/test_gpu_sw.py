@@ -738,7 +738,9 @@ def _softmax(rt, dev, x_bits, axis, pad=0, packed=True, f32=False):
                                         ((1, 1000, 66), 1), ((1, 1024, 2, 64), 1), ((1, 1100, 64), 1), ((2, 2, 512, 512), 2),
                                         # outer axis past the slabs: wavefronts along the axis, lanes along the columns
                                         ((4, 2048, 128), 1), ((2, 1500, 70), 1), ((3, 1200, 5, 13), 1), ((2, 4000, 520), 1),
-                                        ((5000, 64), 0), ((1, 1030, 1024), 1)])
+                                        ((5000, 64), 0), ((1, 1030, 1024), 1),
+                                        # steps either side of 2048, 63 and 200 columns
+                                        ((2, 2047, 64), 1), ((1, 1025, 200), 1), ((2, 2049, 64), 1), ((1, 2048, 1, 63), 1)])
 def test_softmax_shapes_and_axes(rt, orc, dev, shape, axis):
     rng = np.random.default_rng(hash((shape, axis)) % 2 ** 32)
     x = rng.normal(0, 3, shape).astype(np.float32)

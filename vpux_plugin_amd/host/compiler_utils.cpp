@@ -111,7 +111,7 @@ int vpx_approximate(int bits, double target, int64_t* mult, int64_t* shift, int6
     *post_shift = a.postShift;
     if (a.postShift != 0)
         return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT,
-                    "Encountered an attempt to approximate %g as mult = %lld, shift = %lld, postShift = %lld, but postShift is not supported",
+                    "%g approximates to multiplier %lld >> %lld with a further post-shift of %lld; this path has no post-shift stage",
                     target, (long long)a.mult, (long long)a.shift, (long long)a.postShift);
     return VPX_RESULT_SUCCESS;
 }
@@ -177,7 +177,7 @@ int32_t vpx_wt_get_scale(uint8_t shift, int16_t mult) {
 int vpx_wt_get_bias(double real_val, int32_t* bias) {
     const double r = std::round(real_val);
     if (!(r > (double)std::numeric_limits<int32_t>::min() && r < (double)std::numeric_limits<int32_t>::max()))
-        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Rescaled bias value is out of range");
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "a bias divided by its rescale factor does not fit 32 bits");
     *bias = (int32_t)r;
     return VPX_RESULT_SUCCESS;
 }
@@ -200,7 +200,7 @@ int vpx_get_weights_table(double in_scale, double out_scale, const double* weigh
         const Approximation a = approximate(15, rescale);
         if (a.postShift != 0)
             return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT,
-                        "Encountered an attempt to approximate %g as mult = %lld, shift = %lld, postShift = %lld, but postShift is not supported",
+                        "%g approximates to multiplier %lld >> %lld with a further post-shift of %lld; this path has no post-shift stage",
                         rescale, (long long)a.mult, (long long)a.shift, (long long)a.postShift);
         if (a.shift > 255 || a.mult > 32767 || a.mult < -32768)
             return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "scale %g does not fit the multiplier / shift fields", rescale);
@@ -259,13 +259,18 @@ int vpx_retrieve_ppe_int(int post_op, double param0, double param1, const vpx_qu
             }
             return VPX_RESULT_SUCCESS;
         }
+        // the clamp bounds in quantized steps around the zero point, cut to what the storage type holds; a range that
+        // starts at the zero point and ends below the storage maximum is a ReLU-X
         const int64_t zp = out_type->zero_point;
-        const int64_t qMin = (int64_t)std::round(param0 / out_type->scale) + zp;
-        const int64_t qMax = (int64_t)std::round(param1 / out_type->scale) + zp;
-        const int64_t lo = std::max(out_type->storage_min, qMin), hi = std::min(out_type->storage_max, qMax);
-        ppe->clamp_low = (int32_t)lo;
-        ppe->clamp_high = (int32_t)hi;
-        if (lo - zp == 0 && hi - zp < out_type->storage_max) ppe->mode = VPX_PPE_LRELUX;
+        int64_t bound[2];
+        const double real[2] = {param0, param1};
+        for (int k = 0; k < 2; k++) bound[k] = zp + (int64_t)std::round(real[k] / out_type->scale);
+        if (bound[0] < out_type->storage_min) bound[0] = out_type->storage_min;
+        if (bound[1] > out_type->storage_max) bound[1] = out_type->storage_max;
+        ppe->clamp_low = (int32_t)bound[0];
+        ppe->clamp_high = (int32_t)bound[1];
+        const bool from_zero = bound[0] == zp, below_max = bound[1] - zp < out_type->storage_max;
+        if (from_zero && below_max) ppe->mode = VPX_PPE_LRELUX;
         return VPX_RESULT_SUCCESS;
     }
     case VPX_POSTOP_LEAKY_RELU: {
@@ -281,14 +286,14 @@ int vpx_retrieve_ppe_int(int post_op, double param0, double param1, const vpx_qu
             const Approximation a = approximate(11, alpha);
             if (a.postShift != 0)
                 return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT,
-                            "Encountered an attempt to approximate %g as mult = %lld, shift = %lld, postShift = %lld, but postShift is not supported",
+                            "%g approximates to multiplier %lld >> %lld with a further post-shift of %lld; this path has no post-shift stage",
                             alpha, (long long)a.mult, (long long)a.shift, (long long)a.postShift);
             ppe->lrelu_mult = (int32_t)a.mult;
             ppe->lrelu_shift = (int32_t)a.shift;
         }
         return VPX_RESULT_SUCCESS;
     }
-    default: return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Received unknown PPE PostOp: %d", post_op);
+    default: return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "post-op kind %d is not one of the VPX_POSTOP_* values", post_op);
     }
 }
 
@@ -351,7 +356,7 @@ int vpx_get_quant_params_attr(const double* scales, const int64_t* zero_points, 
                               uint64_t* words, uint32_t* n_words) {
     if (!scales || !zero_points || !words || !n_words) return fail(VPX_RESULT_ERROR_INVALID_NULL_HANDLE, "getQuantParamsAttr: null argument");
     if (float_type != VPX_NN_FP16 && float_type != VPX_NN_FP32)
-        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "Supported non-quantized type : f16/f32");
+        return fail(VPX_RESULT_ERROR_INVALID_ARGUMENT, "a tensor that is not quantized must be FP16 or FP32 here");
     const uint32_t per = float_type == VPX_NN_FP16 ? 4 : 2, width = 64 / per;
     uint32_t w = 0;
     words[w++] = n;
