@@ -114,7 +114,7 @@ def test_approximate_goldens_and_oracle(rt, orc):
     # exponent above the bit width needs a post shift, which the reference refuses
     with pytest.raises(rt.VpxError) as e:
         rt.approximate(15, 2.0 ** 20)
-    assert e.value.code == rt.ERROR_INVALID_ARGUMENT and "postShift" in e.value.text
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT and "post-shift" in e.value.text
 
 
 def test_eltwise_approximation_goldens(rt):
