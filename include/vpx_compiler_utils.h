@@ -85,6 +85,8 @@ typedef struct vpx_tensor_desc_t {
     uint32_t data_type;     /* vpx_data_type_t */
     uint64_t dims_order;    /* vpx_nd_order_t */
     uint32_t location;      /* vpx_location_t */
+    uint32_t dynamic_shape; /* non-zero: dims / strides are upper bounds, MemRefData::isStatic is written as 0 and the live
+                               values are read from device memory when the kernel runs (softmax only) */
 } vpx_tensor_desc_t;
 VPX_API int vpx_create_kernel_params(const vpx_tensor_desc_t* inputs, uint32_t n_inputs,
                                      const vpx_tensor_desc_t* outputs, uint32_t n_outputs, const void* attrs,

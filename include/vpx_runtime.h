@@ -65,6 +65,13 @@ typedef struct vpx_memref_addr_t {
     const int32_t* dims;    /* host memory, innermost first, or NULL */
     const int64_t* strides; /* host memory, bits, innermost first, or NULL */
 } vpx_memref_addr_t;
+/* A memref whose MemRefData has isStatic = 0 (a bounded dynamic shape; `softmax` / `softmaxFp32` with the
+ * [axis, padSize], [SoftmaxModeDynamic, rank] form of their parameters, update_sw_kernel_params.cpp:48-55): the blob's
+ * own dims and strides are the bounds, and `dims` / `strides` above must point at DEVICE memory holding the live
+ * values -- what MemRefData::dimsAddr / stridesAddr point at on the NPU, written by whatever produced the shape.
+ * They are read by the kernel, not during the call; elements outside the live shape are left untouched.  The SHAVE
+ * kernel's source is not public: that the live strides are taken as found (compact over the live shape or those of
+ * the bound buffer, whichever the producer wrote) is this library's reading. */
 
 VPX_API int vpx_sw_kernel_launch(const char* entry, const void* params, size_t params_size,
                                  const vpx_memref_addr_t* addrs, uint32_t num_addrs, void* stream);

@@ -806,6 +806,62 @@ def test_softmax_config_c2_full_size_properties(rt, orc, dev):
     assert_close_f16(f16_bits(out), orc.softmax_f16(c["x"], c["axis"]), orc, "C2 whole tensor")
 
 
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("bound,live,axis,pad,compact", [
+    ((4, 100, 64), (3, 77, 50), 2, 0, False), ((4, 100, 64), (3, 77, 50), 1, 0, False), ((4, 100, 64), (3, 77, 50), 0, 0, False),
+    ((4, 100, 64), (3, 77, 50), 2, 0, True), ((4, 100, 64), (3, 77, 50), 1, 5, True), ((2, 3, 40, 33), (2, 3, 40, 33), 3, 0, False),
+    ((2, 3, 40, 33), (1, 2, 17, 9), 2, 0, True), ((8, 700), (5, 513), 1, 13, False), ((600,), (257,), 0, 0, False)])
+def test_softmax_bounded_dynamic_shape(rt, orc, dev, dtype, bound, live, axis, pad, compact):
+    """SoftmaxModeDynamic: the kernel takes the shape from the memrefs' dims and strides in device memory.  The live tensor
+    equals the oracle's softmax of the same values; every element outside it keeps the guard value.  (Parity with the
+    SHAVE kernel itself is unpinned: its source is not public.)"""
+    import torch
+    rng = np.random.default_rng(hash((bound, live, axis)) % 2 ** 32)
+    xf = rng.normal(0, 3, bound).astype(np.float32)
+    live_sl = tuple(slice(0, n) for n in live)
+    if dtype == "f16":
+        xb = orc.f32_to_f16(xf)
+        x = to_dev(xb, dev, True)
+        out = torch.full(bound, 7.0, dtype=torch.float16, device=dev)
+    else:
+        x = torch.from_numpy(xf).to(dev)
+        out = torch.full(bound, 7.0, dtype=torch.float32, device=dev)
+    if compact:  # the live tensor lies compactly at the start of both buffers
+        n_live = int(np.prod(live))
+        src = (xb if dtype == "f16" else xf)[live_sl].reshape(-1).copy()
+        flat = x.view(-1)
+        flat[:n_live] = to_dev(src, dev, True) if dtype == "f16" else torch.from_numpy(src).to(dev)
+    keep = rt.softmax_dynamic(x, out, live, axis, pad, compact=compact)
+    torch.cuda.synchronize()
+    del keep
+    valid = live[axis] - pad
+    src_live = (xb if dtype == "f16" else xf)[live_sl]
+    cut = tuple(slice(0, valid) if d == axis else slice(None) for d in range(len(live)))
+    if dtype == "f16":
+        want = np.zeros(live, dtype=np.uint16)
+        want[cut] = orc.softmax_f16(np.ascontiguousarray(src_live[cut]), axis)
+        got_all = f16_bits(out)
+        guard = np.uint16(0x4700)
+    else:
+        want = np.zeros(live, dtype=np.float32)
+        want[cut] = orc.softmax_f32(np.ascontiguousarray(src_live[cut]), axis)
+        got_all = out.cpu().numpy()
+        guard = np.float32(7.0)
+    if compact:
+        n_live = int(np.prod(live))
+        got = got_all.reshape(-1)[:n_live].reshape(live)
+        assert np.all(got_all.reshape(-1)[n_live:] == guard)
+    else:
+        got = got_all[live_sl]
+        mask = np.ones(bound, dtype=bool)
+        mask[live_sl] = False
+        assert np.all(got_all[mask] == guard)
+    if dtype == "f16":
+        assert_close_f16(got, want, orc, "dynamic softmax %s of %s axis %d" % (live, bound, axis))
+    else:
+        assert np.allclose(got, want, rtol=2e-3, atol=1e-7)
+
+
 def test_softmax_rejects_bad_arguments(rt, dev):
     import torch
     x = torch.zeros((4, 8), dtype=torch.float16, device=dev)
@@ -814,6 +870,22 @@ def test_softmax_rejects_bad_arguments(rt, dev):
     assert e.value.code == rt.ERROR_INVALID_ARGUMENT
     with pytest.raises(rt.VpxError) as e:
         rt.softmax(x, torch.empty_like(x), 1, pad_size=8, packed=False)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    # dynamic-shape parameters with static memrefs, and a dynamic memref on a kernel that takes none
+    ops = [rt.Operand(x), rt.Operand(torch.empty_like(x))]
+    dyn_words = np.asarray([0, 0 | (2 << 32)], dtype=np.uint64).tobytes()
+    with pytest.raises(rt.VpxError) as e:
+        rt.sw_kernel_launch("softmax", rt.create_kernel_params(ops[:1], ops[1:], dyn_words), ops)
+    assert e.value.code == rt.ERROR_INVALID_ARGUMENT
+    dyn = [rt.Operand(x, None, dynamic=True), rt.Operand(torch.empty_like(x), None, dynamic=True)]
+    for o in dyn:
+        o.live_dims = torch.tensor([8, 4], dtype=torch.int32, device=dev)
+        o.live_strides = torch.tensor([16, 128], dtype=torch.int64, device=dev)
+    with pytest.raises(rt.VpxError) as e:
+        rt.sw_kernel_launch("convert", rt.create_kernel_params(dyn[:1], dyn[1:]), dyn)
+    assert e.value.code == rt.ERROR_UNSUPPORTED_FEATURE
+    with pytest.raises(rt.VpxError) as e:  # static form of the parameters with dynamic memrefs
+        rt.sw_kernel_launch("softmax", rt.create_kernel_params(dyn[:1], dyn[1:], np.asarray([0, 0], dtype=np.int64).tobytes()), dyn)
     assert e.value.code == rt.ERROR_INVALID_ARGUMENT
 
 

@@ -229,7 +229,7 @@ bool is_compact(const MemRef& m) {
 }
 
 int parse_blob(const char* entry, int n_in, int n_out, const void* params, size_t params_size,
-               const vpx_memref_addr_t* addrs, uint32_t num_addrs, Args& a) {
+               const vpx_memref_addr_t* addrs, uint32_t num_addrs, bool dynamic_ok, Args& a) {
     const int n_mem = n_in + n_out;
     VPX_REQUIRE(n_mem <= kMaxMemRefs, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: %d operands, at most %d are supported", entry, n_mem, kMaxMemRefs);
     VPX_REQUIRE((int)num_addrs == n_mem, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: expects %d memref addresses (%d in, %d out), got %u",
@@ -254,9 +254,18 @@ int parse_blob(const char* entry, int n_in, int n_out, const void* params, size_
                     dtype_name(md.dataType), md.dataType);
         VPX_REQUIRE((addrs[i].dims == nullptr) == (addrs[i].strides == nullptr), VPX_RESULT_ERROR_INVALID_ARGUMENT,
                     "%s: memref %d must give both dims and strides or neither", entry, i);
+        if (md.isStatic == 0) {
+            // bounded dynamic shape: the side pointers are device memory with the live values, the blob holds the bounds
+            VPX_REQUIRE(dynamic_ok, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE,
+                        "%s: memref %d has a dynamic shape (isStatic = 0), which only softmax / softmaxFp32 take", entry, i);
+            VPX_REQUIRE(addrs[i].dims != nullptr, VPX_RESULT_ERROR_INVALID_NULL_HANDLE,
+                        "%s: memref %d has a dynamic shape: its dims and strides must point at the live values in device memory", entry, i);
+            m.live_dims = addrs[i].dims;
+            m.live_strides = addrs[i].strides;
+        }
         m.data = addrs[i].data;
         tail += (size_t)m.nd * (sizeof(int32_t) + sizeof(int64_t));
-        if (addrs[i].dims == nullptr) tail_needed = true;
+        if (addrs[i].dims == nullptr || md.isStatic == 0) tail_needed = true;  // (a dynamic shape's bounds are in the blob)
     }
     size_t body = params_size - (size_t)n_mem * sizeof(vpx_memref_data_t);
     if (tail_needed) {
@@ -285,7 +294,7 @@ int parse_blob(const char* entry, int n_in, int n_out, const void* params, size_
         for (int d = 0; d < m.nd; d++) {
             int32_t dim;
             int64_t stride_bits;
-            if (addrs[i].dims) {
+            if (addrs[i].dims && m.live_dims == nullptr) {
                 dim = addrs[i].dims[d];
                 stride_bits = addrs[i].strides[d];
             } else {
@@ -409,6 +418,8 @@ int run_softmax(const char* entry, const Args& a, hipStream_t s) {
     SoftmaxPlan p{};
     if ((w1 >> 32) == 0) {
         // first form: int64 axis, int64 padSize
+        VPX_REQUIRE(in.live_dims == nullptr && out.live_dims == nullptr, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: memrefs with isStatic = 0 need the dynamic-shape form of the parameters", entry);
         const int64_t axis = (int64_t)w0, pad = (int64_t)w1;
         VPX_REQUIRE(axis >= 0 && axis < in.nd, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: axis %lld outside rank %d", entry,
                     (long long)axis, in.nd);
@@ -419,7 +430,19 @@ int run_softmax(const char* entry, const Args& a, hipStream_t s) {
         // packed form
         const int64_t axis = (int64_t)(w0 & 0xffffffffu), pad = (int64_t)(w0 >> 32);
         const int64_t mode = (int64_t)(w1 & 0xffffffffu), nd = (int64_t)(w1 >> 32);
-        VPX_REQUIRE(mode != VPX_SOFTMAX_DYNAMIC, VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "%s: dynamic-shape parameters are not supported", entry);
+        if (mode == VPX_SOFTMAX_DYNAMIC) {
+            // [axis, padSize], [SoftmaxModeDynamic, rank] and nothing else (update_sw_kernel_params.cpp:48-55): the shape is
+            // whatever the memrefs' dims and strides in device memory say when the kernel runs
+            VPX_REQUIRE(in.live_dims != nullptr && out.live_dims != nullptr, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                        "%s: dynamic-shape parameters need memrefs with isStatic = 0 and their live dims / strides in device memory", entry);
+            VPX_REQUIRE(nd == in.nd && axis >= 0 && axis < nd, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                        "%s: dynamic-shape parameters name axis %lld of %lld dimensions, the memrefs have %d", entry, (long long)axis,
+                        (long long)nd, in.nd);
+            VPX_REQUIRE(pad >= 0 && pad < (1ll << 31), VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: padSize %lld", entry, (long long)pad);
+            return launch_softmax_dynamic(in, out, (int)axis, (int)pad, s);
+        }
+        VPX_REQUIRE(in.live_dims == nullptr && out.live_dims == nullptr, VPX_RESULT_ERROR_INVALID_ARGUMENT,
+                    "%s: memrefs with isStatic = 0 need the dynamic-shape form of the parameters", entry);
         VPX_REQUIRE(mode >= 1 && mode <= 3, VPX_RESULT_ERROR_INVALID_ARGUMENT, "%s: unknown mode %lld", entry, (long long)mode);
         VPX_REQUIRE(nd >= 1 && nd <= VPX_MAX_ND_DIMS && axis < nd, VPX_RESULT_ERROR_INVALID_ARGUMENT,
                     "%s: packed parameters name axis %lld of %lld dimensions", entry, (long long)axis, (long long)nd);
@@ -569,7 +592,7 @@ static int sw_kernel_launch(const char* entry, const void* params, size_t params
                     "%s: the memref list must hold 2..4 records and end at the marker word", entry);
         n_in = n_mem - e->n_out;
     }
-    int rc = parse_blob(entry, n_in, e->n_out, params, params_size, addrs, num_addrs, a);
+    int rc = parse_blob(entry, n_in, e->n_out, params, params_size, addrs, num_addrs, e->kind == K_SOFTMAX, a);
     if (rc) return rc;
     hipStream_t s = (hipStream_t)stream;
     switch (e->kind) {

@@ -1040,7 +1040,79 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
     return VPX_RESULT_SUCCESS;
 }
 
+// ---------------------------------------------------------------- bounded dynamic shapes
+// The compiler leaves a softmax over a tensor whose shape is only bounded at compile time two parameter words -- [axis,
+// padSize] and [SoftmaxModeDynamic, rank] (update_sw_kernel_params.cpp:48-55) -- and the kernel takes the shape from the
+// memrefs' dims and strides in memory when it runs.  Here: one workgroup per row of the BOUND shape (every combination
+// of the other coordinates); each reads the live dims, leaves if its row lies outside them, and otherwise walks the
+// axis three times with the strides it finds (in bits, as MemRefData holds them).  Elements outside the live shape are
+// not touched.  The last `pad` positions of the axis are written as zeros, as in the static kernels.
+struct DynDims {
+    const int32_t* dims;      // live dims of the input, innermost first (device memory)
+    const int64_t* in_bits;   // live strides of the input, bits
+    const int64_t* out_bits;  // live strides of the output, bits
+    int nd, axis, pad, elem_bits;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_dynamic_kernel(const T* __restrict__ in, T* __restrict__ out, DynDims dd) {
+    __shared__ float smem[4];
+    // the row's coordinates over the live dims (the axis left out), innermost first
+    int64_t r = blockIdx.x, ioff = 0, ooff = 0, len = 1;
+    bool inside = true;
+    for (int d = 0; d < dd.nd; d++) {
+        const int64_t n = dd.dims[d];
+        if (d == dd.axis) {
+            len = n;
+            continue;
+        }
+        if (n <= 0) {
+            inside = false;
+            break;
+        }
+        const int64_t c = r % n;
+        r /= n;
+        ioff += c * (dd.in_bits[d] / dd.elem_bits);
+        ooff += c * (dd.out_bits[d] / dd.elem_bits);
+    }
+    if (!inside || r != 0) return;  // (wave-uniform: the row is the workgroup's)
+    const int64_t in_es = dd.in_bits[dd.axis] / dd.elem_bits, out_es = dd.out_bits[dd.axis] / dd.elem_bits;
+    const int64_t valid = len - dd.pad > 0 ? len - dd.pad : 0;
+    const T* px = in + ioff;
+    T* py = out + ooff;
+    float m = -INFINITY;
+    for (int64_t i = threadIdx.x; i < valid; i += 256) m = fmaxf(m, (float)px[i * in_es]);
+    m = block_allreduce_max(m, smem);
+    float sum = 0.f;
+    for (int64_t i = threadIdx.x; i < valid; i += 256) sum += fast_exp((float)px[i * in_es] - m);
+    sum = block_allreduce_sum(sum, smem);
+    const float inv = 1.0f / sum;
+    for (int64_t i = threadIdx.x; i < len; i += 256)
+        py[i * out_es] = (T)(i < valid ? fast_exp((float)px[i * in_es] - m) * inv : 0.f);
+}
+
 }  // namespace
+
+int launch_softmax_dynamic(const MemRef& in, const MemRef& out, int axis, int pad, hipStream_t s) {
+    VPX_REQUIRE(in.live_dims && in.live_strides && out.live_strides, VPX_RESULT_ERROR_INVALID_NULL_HANDLE,
+                "softmax: a dynamic shape needs its live dims and strides in device memory");
+    int64_t rows = 1;
+    for (int d = 0; d < in.nd; d++)
+        if (d != axis) rows *= in.dims[d];  // the bound shape
+    VPX_REQUIRE(rows < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "softmax: %lld rows in the bound shape exceed the launch limit",
+                (long long)rows);
+    if (rows == 0 || in.dims[axis] == 0) return VPX_RESULT_SUCCESS;
+    const DynDims dd{in.live_dims, in.live_strides, out.live_strides, in.nd, axis, pad, in.elem_bits};
+    if (in.dtype == VPX_NN_FP16) {
+        hipLaunchKernelGGL(softmax_dynamic_kernel<half_t>, dim3((unsigned)rows), dim3(256), 0, s, (const half_t*)in.data, (half_t*)out.data, dd);
+    } else if (in.dtype == VPX_NN_FP32) {
+        hipLaunchKernelGGL(softmax_dynamic_kernel<float>, dim3((unsigned)rows), dim3(256), 0, s, (const float*)in.data, (float*)out.data, dd);
+    } else {
+        return fail(VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "softmax: element type %s is not implemented", dtype_name(in.dtype));
+    }
+    VPX_HIP_CHECK(hipGetLastError());
+    return VPX_RESULT_SUCCESS;
+}
 
 int launch_softmax(const SoftmaxPlan& p, uint32_t dtype, const void* in, void* out, hipStream_t s) {
     VPX_REQUIRE(p.nd >= 1 && p.nd <= VPX_MAX_ND_DIMS && p.axis >= 0 && p.axis < p.nd, VPX_RESULT_ERROR_INVALID_ARGUMENT,

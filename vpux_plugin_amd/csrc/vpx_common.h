@@ -42,6 +42,11 @@ struct MemRef {
     int64_t strides[VPX_MAX_ND_DIMS] = {};  // in elements, innermost first
     int elem_bits = 0;
     bool compact = false;
+    // A memref whose MemRefData says isStatic = 0 (a bounded dynamic shape): dims / strides above are the bounds the blob
+    // holds; the live ones sit in device memory (int32 dims, int64 strides in bits, innermost first), where the producer
+    // of the shape wrote them, and only a kernel can read them.
+    const int32_t* live_dims = nullptr;
+    const int64_t* live_strides = nullptr;
 
     int64_t numel() const {
         int64_t n = 1;
@@ -126,6 +131,9 @@ struct SoftmaxPlan {
     int64_t out_stride[VPX_MAX_ND_DIMS];
 };
 int launch_softmax(const SoftmaxPlan& p, uint32_t dtype, const void* in, void* out, hipStream_t s);
+// bounded dynamic shapes (SoftmaxModeDynamic): the live dims and strides are read on the device; `axis` counts from the
+// innermost dimension of the memrefs as they are (no packing)
+int launch_softmax_dynamic(const MemRef& in, const MemRef& out, int axis, int pad, hipStream_t s);
 
 int launch_mvn(const MemRef& in, const MemRef& out, bool across_channels, bool normalize_variance, float eps,
                hipStream_t s);

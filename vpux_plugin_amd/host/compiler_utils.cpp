@@ -533,7 +533,7 @@ int vpx_create_kernel_params(const vpx_tensor_desc_t* inputs, uint32_t n_inputs,
         m.dimsOrder = t.dims_order;
         m.dataType = t.data_type;
         m.location = t.location;
-        m.isStatic = 1;
+        m.isStatic = t.dynamic_shape ? 0 : 1;
         append(&m, sizeof(m));
     };
     for (uint32_t i = 0; i < n_inputs; i++) add_memref(inputs[i]);

@@ -41,7 +41,7 @@ class MemRefAddr(C.Structure):
 
 class TensorDesc(C.Structure):
     _fields_ = [("num_dims", C.c_uint32), ("dims", C.POINTER(C.c_int32)), ("strides", C.POINTER(C.c_int64)),
-                ("data_type", C.c_uint32), ("dims_order", C.c_uint64), ("location", C.c_uint32)]
+                ("data_type", C.c_uint32), ("dims_order", C.c_uint64), ("location", C.c_uint32), ("dynamic_shape", C.c_uint32)]
 
 
 class PpeInt(C.Structure):
@@ -275,7 +275,7 @@ class Operand:
     """A device tensor seen as a memref: `t` is indexed in MEMORY order (outermost first); its torch
     strides may describe a sub-view.  `order` is the NDOrder code / name of the logical layout."""
 
-    def __init__(self, t, order=None):
+    def __init__(self, t, order=None, dynamic=False):
         self.t = t
         nd = t.dim()
         if order is None:
@@ -287,7 +287,8 @@ class Operand:
         bits = t.element_size() * 8
         self.dims = (C.c_int32 * nd)(*[int(s) for s in reversed(t.shape)])
         self.strides = (C.c_int64 * nd)(*[int(s) * bits for s in reversed(t.stride())])
-        self.desc = TensorDesc(nd, self.dims, self.strides, _torch_dtype_code(t), order, LOC_DDR)
+        self.desc = TensorDesc(nd, self.dims, self.strides, _torch_dtype_code(t), order, LOC_DDR, 1 if dynamic else 0)
+        self.live_dims = self.live_strides = None  # dynamic shapes: device tensors (int32 dims, int64 strides in bits)
 
 
 def create_kernel_params(inputs, outputs, attrs=b""):
@@ -317,7 +318,10 @@ def sw_kernel_launch(entry, blob, operands, stream=None, side_dims=False, noallo
     addrs = (MemRefAddr * len(operands))()
     for i, o in enumerate(operands):
         addrs[i].data = o.t.data_ptr()
-        if side_dims:
+        if o.live_dims is not None:
+            addrs[i].dims = C.cast(C.c_void_p(o.live_dims.data_ptr()), C.POINTER(C.c_int32))
+            addrs[i].strides = C.cast(C.c_void_p(o.live_strides.data_ptr()), C.POINTER(C.c_int64))
+        elif side_dims:
             addrs[i].dims = C.cast(o.dims, C.POINTER(C.c_int32))
             addrs[i].strides = C.cast(o.strides, C.POINTER(C.c_int64))
     fn = lib().vpx_sw_kernel_launch_noalloc if noalloc else lib().vpx_sw_kernel_launch
@@ -472,6 +476,37 @@ def softmax(x, out, axis, pad_size=0, order=None, packed=True, stream=None):
     entry = "softmaxFp32" if _torch_dtype_code(x) == NN_FP32 else "softmax"
     sw_kernel_launch(entry, create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
     return out
+
+
+def softmax_dynamic(x, out, live_shape, axis, pad_size=0, compact=False, stream=None):
+    """Softmax over a tensor whose shape is only bounded at compile time: x / out are the buffers of the bound shape,
+    `live_shape` (memory order, like x.shape) the shape at run time.  The live dims and strides are put in device memory
+    and the kernel reads them there; compact=True lays the live tensor out compactly at the start of the buffers,
+    otherwise it keeps the bound buffer's strides.  Returns the (dims, in strides, out strides) device tensors."""
+    import torch
+    nd = x.dim()
+    axis = axis % nd
+    ops = [Operand(x, None, dynamic=True), Operand(out, None, dynamic=True)]
+    bits = x.element_size() * 8
+    dims = [int(d) for d in reversed(live_shape)]
+    held = []
+    for o in ops:
+        if compact:
+            st, acc = [], 1
+            for d in dims:
+                st.append(acc * bits)
+                acc *= d
+        else:
+            st = [int(v) for v in o.strides]
+        o.live_dims = torch.tensor(dims, dtype=torch.int32, device=x.device)
+        o.live_strides = torch.tensor(st, dtype=torch.int64, device=x.device)
+        held += [o.live_dims, o.live_strides]
+    w0 = (nd - 1 - axis) | (int(pad_size) << 32)
+    w1 = 0 | (nd << 32)  # SoftmaxModeDynamic = 0
+    attrs = np.asarray([w0, w1], dtype=np.uint64).tobytes()
+    entry = "softmaxFp32" if _torch_dtype_code(x) == NN_FP32 else "softmax"
+    sw_kernel_launch(entry, create_kernel_params(ops[:1], ops[1:], attrs), ops, stream)
+    return held
 
 
 def _view_strides(field, x):
