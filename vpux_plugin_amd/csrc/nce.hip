@@ -547,12 +547,27 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
                 rc = device_compute_units(&cus);
                 if (rc) return rc;
                 const int64_t ocb = (g.OC + 63) / 64;
-                // one workgroup per compute unit where the layer allows: rows per tile from the rows there are
-                int R = (int)((g.N * g.OH * ocb + cus - 1) / cus);
+                // Rows per tile: a workgroup costs about 2.9 us whatever its tile (launch, the fetch of its weights and rows,
+                // the register copies) and 0.0106 us per output position, and the workgroups run in rounds of one per compute
+                // unit -- the plane is cut into the number of tiles for which rounds x (fixed + positions) is smallest
+                // ([128,56,56,64]: 512 tiles of 14 rows, two full rounds, 22.5 us; the 384 tiles of 19 rows that one
+                // workgroup per compute unit and LDS allowed took 26.4 us, a round and a half; [32,112,112,64]: 7 rows,
+                // 23.0 against 26.3 us)
                 const int rmin = (int)((128 + g.OW - 1) / g.OW);  // eight waves want eight blocks of 16 positions
-                if (R < rmin) R = rmin;
-                if (R > g.OH) R = (int)g.OH;
-                while (R > 1 && need(R) > kMaxDynLds) R--;
+                int R = 0;
+                double best = 0;
+                for (int64_t ty = 1; ty <= g.OH; ty++) {
+                    const int64_t r = (g.OH + ty - 1) / ty;
+                    if (r < rmin && ty > 1) break;
+                    if (need((int)r) > kMaxDynLds) continue;
+                    const int64_t rounds = (g.N * ty * ocb + cus - 1) / cus;
+                    const double cost = (double)rounds * (2.9 + 0.0106 * (double)(r * g.OW));
+                    if (R == 0 || cost < best) {
+                        best = cost;
+                        R = (int)r;
+                    }
+                }
+                if (R == 0) R = 1;
                 if (const int v = knobs.conv_rows.load()) {
                     if (v >= 1 && v <= R) R = v;
                 }
