@@ -862,6 +862,22 @@ def test_softmax_bounded_dynamic_shape(rt, orc, dev, dtype, bound, live, axis, p
         assert np.allclose(got, want, rtol=2e-3, atol=1e-7)
 
 
+def test_softmax_dynamic_shape_larger_than_its_bound_is_cut(rt, orc, dev):
+    """Live dims beyond the bound (a producer's mistake) never make the kernel leave the buffers: each is cut to its bound."""
+    import torch
+    rng = np.random.default_rng(77)
+    xb = orc.f32_to_f16(rng.normal(0, 3, (3, 40, 24)).astype(np.float32))
+    x = to_dev(xb, dev, True)
+    pad_before = torch.full((4096,), 5.0, dtype=torch.float16, device=dev)
+    out = torch.full((3, 40, 24), 7.0, dtype=torch.float16, device=dev)
+    pad_after = torch.full((4096,), 5.0, dtype=torch.float16, device=dev)
+    keep = rt.softmax_dynamic(x, out, (5, 41, 99), 2)
+    torch.cuda.synchronize()
+    del keep
+    assert_close_f16(f16_bits(out), orc.softmax_f16(xb, 2), orc, "dynamic softmax cut to its bound")
+    assert bool((pad_before == 5.0).all()) and bool((pad_after == 5.0).all())
+
+
 def test_softmax_rejects_bad_arguments(rt, dev):
     import torch
     x = torch.zeros((4, 8), dtype=torch.float16, device=dev)

@@ -1046,12 +1046,14 @@ int softmax_typed(const SoftmaxPlan& p, const T* in, T* out, hipStream_t s) {
 // memrefs' dims and strides in memory when it runs.  Here: one workgroup per row of the BOUND shape (every combination
 // of the other coordinates); each reads the live dims, leaves if its row lies outside them, and otherwise walks the
 // axis three times with the strides it finds (in bits, as MemRefData holds them).  Elements outside the live shape are
-// not touched.  The last `pad` positions of the axis are written as zeros, as in the static kernels.
+// not touched, and a live dimension larger than its bound is cut to the bound.  The last `pad` positions of the axis
+// are written as zeros, as in the static kernels.
 struct DynDims {
     const int32_t* dims;      // live dims of the input, innermost first (device memory)
     const int64_t* in_bits;   // live strides of the input, bits
     const int64_t* out_bits;  // live strides of the output, bits
     int nd, axis, pad, elem_bits;
+    int32_t bound[VPX_MAX_ND_DIMS];  // the dims the blob holds: a live dimension is never taken to be larger
 };
 
 template <typename T>
@@ -1061,7 +1063,8 @@ __global__ __launch_bounds__(256) void softmax_dynamic_kernel(const T* __restric
     int64_t r = blockIdx.x, ioff = 0, ooff = 0, len = 1;
     bool inside = true;
     for (int d = 0; d < dd.nd; d++) {
-        const int64_t n = dd.dims[d];
+        const int64_t live = dd.dims[d];
+        const int64_t n = live < dd.bound[d] ? live : dd.bound[d];  // (the buffers were sized for the bound)
         if (d == dd.axis) {
             len = n;
             continue;
@@ -1102,7 +1105,8 @@ int launch_softmax_dynamic(const MemRef& in, const MemRef& out, int axis, int pa
     VPX_REQUIRE(rows < (1ll << 31), VPX_RESULT_ERROR_UNSUPPORTED_FEATURE, "softmax: %lld rows in the bound shape exceed the launch limit",
                 (long long)rows);
     if (rows == 0 || in.dims[axis] == 0) return VPX_RESULT_SUCCESS;
-    const DynDims dd{in.live_dims, in.live_strides, out.live_strides, in.nd, axis, pad, in.elem_bits};
+    DynDims dd{in.live_dims, in.live_strides, out.live_strides, in.nd, axis, pad, in.elem_bits, {}};
+    for (int d = 0; d < in.nd; d++) dd.bound[d] = (int32_t)in.dims[d];
     if (in.dtype == VPX_NN_FP16) {
         hipLaunchKernelGGL(softmax_dynamic_kernel<half_t>, dim3((unsigned)rows), dim3(256), 0, s, (const half_t*)in.data, (half_t*)out.data, dd);
     } else if (in.dtype == VPX_NN_FP32) {
