@@ -39,7 +39,7 @@ MEASURED_TRAFFIC = {
     "c5_matmul": 339731998, "c5_dequantize": 135262411, "c5_eltwise_add": 270552950, "c5_nce_eltwise": 135260008,
     "calib_copy": 134217728, "calib_int_mm": 534882288, "x_mvn6_layernorm": 268523883, "x_activation_hswish": 180471319,
     "x_mvn1_three_steps": 25341653, "x_stem_conv": 67131551, "x_small_plane_conv": 20886567, "x_large_conv": 54593192,
-    "x_wide_conv": 58724921, "x_softmax_outer_axis": 402620437, "x_mvn_nhwc_per_channel": 317063410,
+    "x_wide_conv": 58724921, "x_pointwise_conv": 36897809, "x_softmax_outer_axis": 402620437, "x_mvn_nhwc_per_channel": 317063410,
 }
 
 
@@ -235,6 +235,27 @@ def make_conv64(rt, name, N, H, W):
     ops = 2 * N * H * W * 64 * 9 * 64
     return Workload(name, "int8 Conv 3x3 s1 p1 NHWC [%d,%d,%d,64] u8 zp128 x [64,3,3,64] i8, ReLU clamp (not a BASELINE config)" % (N, H, W),
                     step, inp.numel() + out.numel() + w.numel() + wt.numel() * 4, ops, "mfma", "int8", "nce_conv_regw")
+
+
+def make_pointwise(rt):
+    """1x1, 64 -> 256 channels (the expansion layer of a ResNet-50 stage-2 block): bound by its 26 MB of output
+    (not a BASELINE config)."""
+    import torch
+    N, H, W, IC, OC = 32, 56, 56, 64, 256
+    g = torch.Generator(device="cuda").manual_seed(19)
+    inp = torch.randint(0, 256, (N, H, W, IC), dtype=torch.uint8, device="cuda", generator=g)
+    w = torch.randint(-127, 128, (OC, 1, 1, IC), dtype=torch.int8, device="cuda", generator=g)
+    rng = np.random.default_rng(19)
+    wt = _dev(rt.make_weights_table(rng.integers(2 ** 14, 2 ** 15, OC), rng.integers(18, 23, OC),
+                                    rng.integers(-2 ** 15, 2 ** 15, OC).astype(np.int32), IC))
+    out = torch.empty((N, H, W, OC), dtype=torch.uint8, device="cuda")
+    ppe = rt.PpeInt(rt.PPE_NOOP, 0, 255, 1, 0)
+    task = _nce_task(rt, inp, w, wt, out, ppe, 128, 0, (1, 1), (0, 0, 0, 0))
+    step = _nce_step(rt, task)
+    step.keep = (inp, w, wt, out, task)
+    ops = 2 * N * H * W * IC * OC
+    return Workload("x_pointwise_conv", "int8 Conv 1x1 NHWC [32,56,56,64] u8 zp128 x [256,1,1,64] i8, ReLU clamp (not a BASELINE config)",
+                    step, inp.numel() + out.numel() + w.numel() + wt.numel() * 4, ops, "hbm", "int8", "nce_gemm_regb")
 
 
 def make_stem(rt):
@@ -491,6 +512,7 @@ MAKERS = {
     "x_softmax_outer_axis": make_softmax_outer,
     "x_mvn_nhwc_per_channel": make_mvn_nhwc,
     "x_stem_conv": make_stem,
+    "x_pointwise_conv": make_pointwise,
     "x_large_conv": lambda rt: make_conv64(rt, "x_large_conv", 128, 56, 56),
     "x_wide_conv": lambda rt: make_conv64(rt, "x_wide_conv", 32, 112, 112),
     "x_small_plane_conv": make_small_plane_conv,

@@ -229,6 +229,8 @@ VPX_API int vpx_nce_task(const vpx_nce_task_t* task, void* stream);
 
 /* Testing and tuning hook (no counterpart in the reference): overrides how vpx_nce_task picks its device kernel.
  * `knob` is one of "VPX_NCE_KERNEL" (naive | gather | conv), "VPX_GEMM_TILE" (128 | 256), "VPX_GEMM_WAVES" (4 | 8),
+ * "VPX_GEMM_REGB" (on | wide | off: the weights-in-registers matmul for a K of 64, 128 or 256, which by itself serves layers of
+ * many rows; wide: with as many channel blocks per wave as it otherwise takes from some hundreds of thousands of rows on),
  * "VPX_GEMM_PINGPONG" (on: the two waves of a SIMD take turns at the MFMAs of the large matmul tile; measured slower, off by default),
  * "VPX_CONV_KERNEL" (regw | tile | stream), "VPX_CONV_ROWS" (n), "VPX_CONV_COLS" (n), "VPX_CONV_WAVES" (4 | 8), "VPX_STREAM_KSPLIT" (off: the streamed-weights
  * convolution kernel gives every wave a 32 x 32 tile also on small planes, instead of splitting K over the waves of a group),

@@ -178,7 +178,15 @@ def test_large_nce_eltwise_and_matmul(rt, orc, dev):
     wt = rt.make_weights_table(rng.integers(2 ** 14, 2 ** 15, N), rng.integers(18, 24, N), rng.integers(-2 ** 15, 2 ** 15, N).astype(np.int32), K)
     wtd = torch.from_numpy(wt).to(dev)
     p = rt.PpeInt(rt.PPE_LPRELU, -128, 127, 1638, 14)
-    out = _whole_and_parts(lambda o, lo, hi: rt.nce_matmul(A[lo:hi], B, wtd, o[lo:hi], p, zp_a=3), (M, N), torch.int8, dev, M)
-    assert rt.nce_last_kernel() == "nce_gemm_mfma"
     want = orc.nce_matmul(A[-64:].cpu().numpy(), B.cpu().numpy(), wt, orc.ppe(1638, 14, 0, -128, 127), zp_a=3)
-    assert np.array_equal(out[-64:].cpu().numpy(), want)
+    # so many rows of a short K take the weights-in-registers kernel by themselves; the tile kernel when that is switched off
+    for knob, kernel in ((None, "nce_gemm_regb"), ("off", "nce_gemm_mfma")):
+        rt.set_tuning("VPX_GEMM_REGB", knob)
+        try:
+            out = _whole_and_parts(lambda o, lo, hi: rt.nce_matmul(A[lo:hi], B, wtd, o[lo:hi], p, zp_a=3), (M, N), torch.int8, dev, M)
+        finally:
+            rt.set_tuning("VPX_GEMM_REGB", None)
+        assert rt.nce_last_kernel() == kernel
+        assert np.array_equal(out[-64:].cpu().numpy(), want)
+        del out
+        torch.cuda.empty_cache()

@@ -485,6 +485,76 @@ def test_matmul_gemm_path(rt, orc, dev, gemm_waves, M, K, N):
         assert np.array_equal(got, want), "M=%d K=%d N=%d zp=%d: %d mismatches" % (M, K, N, zp, int((got != want).sum()))
 
 
+@pytest.fixture(params=["on", "wide"])
+def regb_on(rt, request):
+    """The weights-in-registers matmul, which by itself serves a short K from some tens of thousands of rows on; "wide":
+    with as many channel blocks per wave as it takes from some hundreds of thousands of rows on."""
+    rt.set_tuning("VPX_GEMM_REGB", request.param)
+    yield request.param
+    rt.set_tuning("VPX_GEMM_REGB", None)
+
+
+@pytest.mark.parametrize("M,K,N", [(4096, 64, 256), (1000, 64, 64), (517, 128, 208), (33, 256, 80), (1, 64, 16), (2050, 256, 528),
+                                   (16, 128, 64), (700, 64, 192), (900, 64, 512), (333, 64, 128), (650, 128, 512), (300, 64, 384)])
+def test_matmul_weights_in_registers(rt, orc, dev, regb_on, M, K, N):
+    """Every PPE form (short with and without a slope, the general integer one through clipping scales, an odd zero
+    point and a slope above one), both input types, row and channel counts that end inside a block."""
+    rng = np.random.default_rng(170 + M + N)
+    cases = [
+        (False, 3, dict(I8, lrelu_mult=1638, lrelu_shift=14), rt.PPE_LPRELU, True, 0, (18, 24)),
+        (True, 128, dict(U8), rt.PPE_NOOP, False, 0, (16, 22)),
+        (True, 11, dict(U8, lrelu_mult=3, lrelu_shift=1), rt.PPE_LPRELU, False, 4, (16, 22)),   # slope 1.5: general
+        (False, 0, dict(I8), rt.PPE_LRELU, True, 7, (16, 22)),                                  # odd zero point: general
+        (True, 128, dict(clamp_low=10, clamp_high=200), rt.PPE_NOOP, False, 0, (8, 13)),        # scales above 1/2: clipping
+    ]
+    for in_u8, zp, kw, mode, out_signed, zp_out, (slo, shi) in cases:
+        a = rng.integers(0, 256, (M, K), dtype=np.uint8) if in_u8 else rng.integers(-128, 128, (M, K)).astype(np.int8)
+        b = rng.integers(-127, 128, (N, K)).astype(np.int8)
+        mults = rng.integers(2 ** 14, 2 ** 15, N)
+        shifts = rng.integers(slo, shi, N)
+        bias = rng.integers(-2 ** 15, 2 ** 15, N).astype(np.int32)
+        got, want, name = run_task(rt, orc, dev, a.reshape(1, M, 1, K), b.reshape(N, 1, 1, K), mults, shifts, bias, kw,
+                                   zp_in=zp, zp_out=zp_out, out_signed=out_signed, mode=mode)
+        assert name == "nce_gemm_regb"
+        assert np.array_equal(got, want), "M=%d K=%d N=%d zp=%d mode=%s: %d mismatches" % (M, K, N, zp, mode, int((got != want).sum()))
+
+
+@pytest.mark.parametrize("M,K,N,w_u8,zp_w", [(900, 64, 256, True, 128), (530, 128, 144, True, 117), (300, 256, 64, False, -5)])
+def test_matmul_weights_in_registers_weight_zero_points(rt, orc, dev, regb_on, M, K, N, w_u8, zp_w):
+    rng = np.random.default_rng(180 + M)
+    a = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    b = rng.integers(0, 256, (N, K), dtype=np.uint8) if w_u8 else rng.integers(-127, 128, (N, K)).astype(np.int8)
+    mults = rng.integers(2 ** 14, 2 ** 15, N)
+    shifts = rng.integers(18, 24, N)
+    bias = rng.integers(-2 ** 15, 2 ** 15, N).astype(np.int32)
+    got, want, name = run_task(rt, orc, dev, a.reshape(1, M, 1, K), b.reshape(N, 1, 1, K), mults, shifts, bias, dict(U8),
+                               zp_in=121, zp_w=zp_w, out_offset=48)
+    assert name == "nce_gemm_regb"
+    assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
+
+
+def test_matmul_weights_in_registers_leaves_ragged_rows_to_the_tile_kernel(rt, orc, dev, regb_on):
+    """Channel counts that are not a multiple of 16 (rows of the result that do not end on a 16-byte piece) and a K it
+    does not serve."""
+    rng = np.random.default_rng(185)
+    for M, K, N in ((300, 64, 77), (300, 192, 128)):
+        a = rng.integers(-128, 128, (M, K)).astype(np.int8)
+        b = rng.integers(-127, 128, (N, K)).astype(np.int8)
+        got, want, name = run_task(rt, orc, dev, a.reshape(1, M, 1, K), b.reshape(N, 1, 1, K), rng.integers(2 ** 14, 2 ** 15, N),
+                                   rng.integers(18, 24, N), rng.integers(-2 ** 15, 2 ** 15, N).astype(np.int32), dict(I8), out_signed=True)
+        assert name == "nce_gemm_mfma"
+        assert np.array_equal(got, want)
+
+
+def test_1x1_layer_takes_the_weights_in_registers_matmul_by_itself(rt, orc, dev):
+    """[8,112,112,64] -> 256, 1x1: 100 352 rows of 64."""
+    rng = np.random.default_rng(190)
+    inp, w, mults, shifts, bias = rand_case(rng, 8, 112, 112, 64, 256, 1, 1, shift_lo=18, shift_hi=22)
+    got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, dict(U8), zp_in=128)
+    assert name == "nce_gemm_regb"
+    assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())
+
+
 @pytest.mark.parametrize("M,K,N", [(300, 128, 520), (513, 256, 77)])
 def test_matmul_gemm_path_f16_output(rt, orc, dev, gemm_waves, M, K, N):
     """The wave-count knob does not reach the fp16-output matmul, which exists with eight waves per large tile only."""

@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB = os.path.join(HERE, "libvpx_amd.so")
 
-HIP_SOURCES = ["csrc/abi.hip", "csrc/sw_elementwise.hip", "csrc/sw_softmax.hip", "csrc/sw_mvn.hip", "csrc/nce.hip", "csrc/nce_gemm.hip",
+HIP_SOURCES = ["csrc/abi.hip", "csrc/sw_elementwise.hip", "csrc/sw_softmax.hip", "csrc/sw_mvn.hip", "csrc/nce.hip", "csrc/nce_gemm.hip", "csrc/nce_gemm_regb.hip",
                "csrc/nce_conv_patch.hip", "csrc/nce_conv_rows.hip", "csrc/nce_conv_gather.hip", "csrc/nce_eltwise.hip", "csrc/calib.hip"]
 HOST_SOURCES = ["host/compiler_utils.cpp"]
 

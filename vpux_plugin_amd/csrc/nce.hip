@@ -1,5 +1,5 @@
 // NCE cluster task on CDNA4: the dispatcher from a vpx_nce_task_t to a device kernel, the tuning knobs, the operand
-// views and the small kernels that prepare a weight zero point.  The kernels live in nce_gemm.hip, nce_conv_patch.hip,
+// views and the small kernels that prepare a weight zero point.  The kernels live in nce_gemm.hip, nce_gemm_regb.hip, nce_conv_patch.hip,
 // nce_conv_rows.hip, nce_conv_gather.hip and nce_eltwise.hip; nce_common.h says what each serves.
 #include <mutex>
 #include <set>
@@ -135,6 +135,8 @@ bool set_knob(const char* knob, const char* value) {
         g_tuning.gemm_tile = *v ? (std::atoi(v) == 128 ? 128 : 256) : 0;
     } else if (!std::strcmp(knob, "VPX_GEMM_WAVES")) {
         g_tuning.gemm_waves = *v ? (std::atoi(v) == 4 ? 4 : 8) : 0;
+    } else if (!std::strcmp(knob, "VPX_GEMM_REGB")) {
+        g_tuning.gemm_regb = !std::strcmp(v, "on") ? 1 : (!std::strcmp(v, "wide") ? 2 : (!std::strcmp(v, "off") ? -1 : 0));
     } else if (!std::strcmp(knob, "VPX_GEMM_PINGPONG")) {
         g_tuning.gemm_pingpong = !std::strcmp(v, "on") ? 1 : 0;
     } else if (!std::strcmp(knob, "VPX_CONV_KERNEL")) {
@@ -162,7 +164,7 @@ bool set_knob(const char* knob, const char* value) {
 
 const Tuning& tuning() {
     std::call_once(g_tuning_once, [] {
-        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_GEMM_PINGPONG", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_COLS", "VPX_CONV_WAVES", "VPX_STREAM_KSPLIT", "VPX_MVN_FUSED", "VPX_CALIB_BLOCKS"})
+        for (const char* k : {"VPX_NCE_KERNEL", "VPX_GEMM_TILE", "VPX_GEMM_WAVES", "VPX_GEMM_REGB", "VPX_GEMM_PINGPONG", "VPX_CONV_KERNEL", "VPX_CONV_ROWS", "VPX_CONV_COLS", "VPX_CONV_WAVES", "VPX_STREAM_KSPLIT", "VPX_MVN_FUSED", "VPX_CALIB_BLOCKS"})
             if (const char* v = std::getenv(k)) set_knob(k, v);
     });
     return g_tuning;
@@ -488,6 +490,40 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             int cus_gemm = 0;
             rc = device_compute_units(&cus_gemm);
             if (rc) return rc;
+            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi};
+            const GemmRows rows{picks_rows ? 1 : 0, vin.sw, (int)g.OW, (int)(g.OH * g.OW), (unsigned)(g.SX * vin.sw), (unsigned)(g.SY * vin.sh),
+                                (unsigned)vin.sn};
+            const GemmOut dst{vout.flat == 2 ? 1 : 0, vout.sn, vout.sh, vout.sw, (int)g.OW, (int)(g.OH * g.OW), g.out_bits};
+            // A short K and many rows: the weights of a 64-channel block stay in the registers of a wave that walks
+            // blocks of 16 rows (nce_gemm_regb.hip).  VPX_GEMM_REGB=on|off overrides.
+            const int regb_knob = knobs.gemm_regb.load();
+            if (!out_f16 && G == 1 && !picks_rows && (g.IC == 64 || g.IC == 128 || g.IC == 256) && regb_knob >= 0 && Mtot < (1ll << 31) &&
+                dst.flat && g.OC % 16 == 0 && (g.out_bits & 15) == 0) {
+                const int64_t nblk = (Mtot + 15) / 16;
+                int cbw = 1, gw = 1;
+                gemm_regb_shape(Mtot, g.OC, g.IC, cus_gemm, regb_knob == 2, &cbw, &gw);
+                const int64_t supers = (g.OC + 63) / 64 / cbw / gw;  // workgroups come in multiples of this
+                // workgroups of four waves, as many as are resident at once
+                const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
+                int64_t wgs = (int64_t)cus_gemm * gemm_regb_workgroups_per_cu(same_f, g.IC, cbw);
+                wgs = (wgs + supers - 1) / supers * supers;
+                const int64_t per_wg = 4 / gw, streams = wgs / supers * per_wg;  // row streams
+                // Measured against the tile kernel (us, rotating buffers): [100352 x 64] . [64 x 256] 10.3 / 15.2,
+                // [401408 x 64] . [64 x 256] 30.8 / 42.9, [100352 x 256] . [256 x 64] 12.3 / 17.6, [25088 x 64] . [64 x 256]
+                // 6.2 / 6.4; about equal at K = 128 ([100352 x 128] . [128 x 256] 17.5 / 17.8, [25088 x 128] . [128 x 512]
+                // 10.3 / 10.5); behind it at K = 256 with more than 64 channels ([25088 x 256] . [256 x 128] 8.9 / 8.0,
+                // [25088 x 256] . [256 x 512] 15.5 / 12.8).
+                const bool pays = nblk * cbw >= (g.IC == 128 ? 4 : 2) * streams && (g.IC < 256 || g.OC <= 64);
+                if (regb_knob > 0 || pays) {
+                    if (nblk < streams) wgs = (nblk + per_wg - 1) / per_wg * supers;
+                    const GemmLaunch gl{(const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, (uint8_t*)t.output, Mtot, g.OC, g.IC, G,
+                                        0, 8, false, in_u8, false, out_signed ? OUT_I8 : OUT_U8, gp, rows, dst};
+                    rc = launch_gemm_regb(gl, cbw, gw, (int)wgs, s);
+                    if (rc) return rc;
+                    *kernel_name = "nce_gemm_regb";
+                    return VPX_RESULT_SUCCESS;
+                }
+            }
             const int64_t t256 = gemm_tiles * G, t128 = ((Mtot + 127) / 128) * ((g.OC + 127) / 128) * G;
             const double work = (double)Mtot * (double)g.OC * (double)G;
             const double use256 = work / ((double)((t256 + cus_gemm - 1) / cus_gemm) * cus_gemm * 65536.0);
@@ -506,10 +542,6 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             const int nw = tile == 128 ? 4 : (out_f16 ? 8 : (waves_knob ? waves_knob : 8));
             const int64_t nk = g.IC / 64;
             const bool shortk = tile == 128 && nk <= 3 && !out_f16;
-            GemmPpe gp{ppe.prelu_mult, ppe.prelu_shift, corr, pf.zp_out, pf.lo, pf.hi, out_signed ? 1 : 0, rowterm, ppe.f16_lo, ppe.f16_hi};
-            const GemmRows rows{picks_rows ? 1 : 0, vin.sw, (int)g.OW, (int)(g.OH * g.OW), (unsigned)(g.SX * vin.sw), (unsigned)(g.SY * vin.sh),
-                                (unsigned)vin.sn};
-            const GemmOut dst{vout.flat == 2 ? 1 : 0, vout.sn, vout.sh, vout.sw, (int)g.OW, (int)(g.OH * g.OW), g.out_bits};
             const GemmLaunch gl{(const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, (uint8_t*)t.output, Mtot, g.OC, g.IC, G,
                                 tile, nw, shortk, in_u8, knobs.gemm_pingpong.load() != 0, out_f16 ? OUT_F16 : (out_signed ? OUT_I8 : OUT_U8), gp, rows, dst};
             rc = launch_gemm_mfma(gl, s);

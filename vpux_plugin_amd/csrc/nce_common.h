@@ -4,6 +4,7 @@
 //
 //   nce.hip             the dispatcher (vpx_nce_task -> kernel), tuning knobs, operand views, preparation kernels
 //   nce_gemm.hip        nce_gemm_mfma: 1x1 layers and NCE.MatMul
+//   nce_gemm_regb.hip   nce_gemm_regb: the same with a short K and many rows, weights in registers
 //   nce_conv_patch.hip  nce_conv_regw / nce_conv_tile / nce_conv_stream: input rows of a tile in LDS
 //   nce_conv_rows.hip   nce_conv_rows16: channel counts that are a multiple of 16 only
 //   nce_conv_gather.hip nce_conv_mfma / nce_conv_mfma16 / nce_conv_naive: the general fallbacks
@@ -611,6 +612,7 @@ struct Tuning {
     std::atomic<int> nce_kernel{NCE_AUTO};  // VPX_NCE_KERNEL = naive | gather | conv: restrict the choice to slower, more general paths
     std::atomic<int> gemm_tile{0};          // VPX_GEMM_TILE = 128 | 256 (0: chosen from the shape)
     std::atomic<int> gemm_waves{0};         // VPX_GEMM_WAVES = 4 | 8
+    std::atomic<int> gemm_regb{0};          // VPX_GEMM_REGB = on | wide | off: weights-in-registers matmul for K of 64, 128 or 256 (1, 2: with the most channel blocks per wave, -1; 0: chosen from the shape)
     std::atomic<int> gemm_pingpong{0};      // VPX_GEMM_PINGPONG = on | off: the waves of a SIMD take turns at the MFMAs
     std::atomic<int> conv_stream{0};        // VPX_CONV_KERNEL = regw | tile | stream: start the choice of LDS-patch kernel at this one (-1, 1, 2; 0: by size)
     std::atomic<int> conv_rows{0};          // VPX_CONV_ROWS = n: cap on the output rows per workgroup of the LDS-patch kernels
@@ -649,6 +651,12 @@ struct GemmLaunch {
     GemmOut dst;
 };
 int launch_gemm_mfma(const GemmLaunch& a, hipStream_t s);
+// nce_gemm_regb.hip: K of 64, 128 or 256, rows of A and of the result at a fixed pitch, 16-byte aligned, N a multiple of
+// 16, one group, byte output; `workgroups` x 4 waves, a multiple of
+// (64-channel blocks / `cbw` / `gw`).
+int launch_gemm_regb(const GemmLaunch& a, int cbw, int gw, int workgroups, hipStream_t s);
+void gemm_regb_shape(int64_t M, int64_t N, int64_t K, int cus, bool widest, int* cbw, int* gw);  // 64-channel blocks per wave, groups of them per workgroup
+int gemm_regb_workgroups_per_cu(bool same_f, int64_t K, int cbw);                   // resident workgroups the kernel's registers allow
 
 // nce_conv_patch.hip: one workgroup per tile of `pg.R` output rows x 64 channels.
 struct PatchLaunch {
