@@ -546,10 +546,11 @@ def test_matmul_weights_in_registers_leaves_ragged_rows_to_the_tile_kernel(rt, o
         assert np.array_equal(got, want)
 
 
-def test_1x1_layer_takes_the_weights_in_registers_matmul_by_itself(rt, orc, dev):
-    """[8,112,112,64] -> 256, 1x1: 100 352 rows of 64."""
-    rng = np.random.default_rng(190)
-    inp, w, mults, shifts, bias = rand_case(rng, 8, 112, 112, 64, 256, 1, 1, shift_lo=18, shift_hi=22)
+@pytest.mark.parametrize("IC,OC", [(64, 256), (64, 48), (128, 64), (256, 64)])
+def test_1x1_layer_takes_the_weights_in_registers_matmul_by_itself(rt, orc, dev, IC, OC):
+    """[8,112,112,IC] -> OC, 1x1: 100 352 rows of a short K, also where the channels are fewer than a matmul tile is wide."""
+    rng = np.random.default_rng(190 + OC)
+    inp, w, mults, shifts, bias = rand_case(rng, 8, 112, 112, IC, OC, 1, 1, shift_lo=18, shift_hi=22)
     got, want, name = run_task(rt, orc, dev, inp, w, mults, shifts, bias, dict(U8), zp_in=128)
     assert name == "nce_gemm_regb"
     assert np.array_equal(got, want), "%d mismatches" % int((got != want).sum())

@@ -293,7 +293,45 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
     // is long enough for the matmul kernel's deeper pipeline to make up for it (from 192 channels on: [100352 x 192 x 64]
     // 13.8 -> 11.1 us, [25088 x 512 x 64] 8.6 -> 7.5 us, [6272 x 1024 x 64] 11.1 -> 9.0 us; 128 channels: even).
     const int64_t gemm_tiles = ((Mtot + 255) / 256) * ((g.OC + 255) / 256);
-    const bool use_gemm = allow_gemm && (is_flat_gemm || is_strided_gemm) && g.IC % 64 == 0 && g.IC < (1 << 24) && (g.OC > 64 || (g.OC > 48 && g.IC >= 192) || Mtot < 1024);
+    // A short K and many rows: the weights of 64-channel blocks stay in the registers of waves that walk blocks of 16
+    // rows (nce_gemm_regb.hip; its units are 64 channels wide, so it serves the narrow layers too).  VPX_GEMM_REGB=on|
+    // wide|off overrides.  Measured against the tile kernel (us, rotating buffers): [100352 x 64] . [64 x 256] 10.3 / 15.2,
+    // [401408 x 64] . [64 x 256] 30.8 / 42.9, [100352 x 256] . [256 x 64] 12.3 / 17.6, [25088 x 64] . [64 x 256] 6.2 / 6.4;
+    // about equal at K = 128 ([100352 x 128] . [128 x 256] 17.5 / 17.8, [25088 x 128] . [128 x 512] 10.3 / 10.5); behind it
+    // at K = 256 with more than 64 channels ([25088 x 256] . [256 x 128] 8.9 / 8.0, [25088 x 256] . [256 x 512] 15.5 / 12.8).
+    // Against the convolution kernels on 64 channels and fewer: [100352 x 64] . [64 x 64] 6.4 / 7.9, [100352 x 128] . [128 x 64]
+    // 9.1 / 14.1, [401408 x 64] . [64 x 64] 14.4 / 30.3, [25088 x 64] . [64 x 64] 6.4 / 6.3.
+    int regb_cbw = 0, regb_gw = 0;
+    int64_t regb_wgs = 0;
+    {
+        const int regb_knob = knobs.gemm_regb.load();
+        if (allow_gemm && is_flat_gemm && !out_f16 && t.groups <= 1 && (g.IC == 64 || g.IC == 128 || g.IC == 256) && regb_knob >= 0 &&
+            Mtot < (1ll << 31) && vout.flat == 2 && g.OC % 16 == 0 && (g.out_bits & 15) == 0) {
+            int cus = 0;
+            const int rc = device_compute_units(&cus);
+            if (rc) return rc;
+            int cbw = 1, gw = 1;
+            gemm_regb_shape(Mtot, g.OC, g.IC, cus, regb_knob == 2, &cbw, &gw);
+            const int64_t nblk = (Mtot + 15) / 16;
+            const int64_t supers = (g.OC + 63) / 64 / cbw / gw;  // workgroups come in multiples of this
+            // workgroups of four waves, as many as are resident at once
+            const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
+            int64_t wgs = (int64_t)cus * gemm_regb_workgroups_per_cu(same_f, g.IC, cbw);
+            wgs = (wgs + supers - 1) / supers * supers;
+            const int64_t per_wg = 4 / gw, streams = wgs / supers * per_wg;  // row streams
+            // units of 16 rows x 64 channels per wave: from one and a half on, three where the tile kernel is the alternative at K = 128
+            const int64_t units = nblk * ((g.OC + 63) / 64), waves = wgs * 4;
+            const bool pays = (g.OC <= 64 || g.IC == 64 ? 2 * units >= 3 * waves : units >= 3 * waves) && (g.IC < 256 || g.OC <= 64);
+            if (regb_knob > 0 || pays) {
+                if (nblk < streams) wgs = (nblk + per_wg - 1) / per_wg * supers;
+                regb_cbw = cbw;
+                regb_gw = gw;
+                regb_wgs = wgs;
+            }
+        }
+    }
+    const bool use_gemm = allow_gemm && (is_flat_gemm || is_strided_gemm) && g.IC % 64 == 0 && g.IC < (1 << 24) &&
+                          (g.OC > 64 || (g.OC > 48 && g.IC >= 192) || Mtot < 1024 || regb_cbw != 0);
     // VPU.NCE.MatMul's groups: one launch of the matmul kernel when it serves the shape (the preparation passes then
     // walk all groups' weights / activations as one tensor), else one task after the other on the stream.
     const int64_t G = t.groups > 1 ? t.groups : 1;
@@ -494,35 +532,13 @@ int launch_nce(const vpx_nce_task_t& t, hipStream_t s, const char** kernel_name)
             const GemmRows rows{picks_rows ? 1 : 0, vin.sw, (int)g.OW, (int)(g.OH * g.OW), (unsigned)(g.SX * vin.sw), (unsigned)(g.SY * vin.sh),
                                 (unsigned)vin.sn};
             const GemmOut dst{vout.flat == 2 ? 1 : 0, vout.sn, vout.sh, vout.sw, (int)g.OW, (int)(g.OH * g.OW), g.out_bits};
-            // A short K and many rows: the weights of a 64-channel block stay in the registers of a wave that walks
-            // blocks of 16 rows (nce_gemm_regb.hip).  VPX_GEMM_REGB=on|off overrides.
-            const int regb_knob = knobs.gemm_regb.load();
-            if (!out_f16 && G == 1 && !picks_rows && (g.IC == 64 || g.IC == 128 || g.IC == 256) && regb_knob >= 0 && Mtot < (1ll << 31) &&
-                dst.flat && g.OC % 16 == 0 && (g.out_bits & 15) == 0) {
-                const int64_t nblk = (Mtot + 15) / 16;
-                int cbw = 1, gw = 1;
-                gemm_regb_shape(Mtot, g.OC, g.IC, cus_gemm, regb_knob == 2, &cbw, &gw);
-                const int64_t supers = (g.OC + 63) / 64 / cbw / gw;  // workgroups come in multiples of this
-                // workgroups of four waves, as many as are resident at once
-                const bool same_f = ppe.prelu_mult == 1 && ppe.prelu_shift == 0;
-                int64_t wgs = (int64_t)cus_gemm * gemm_regb_workgroups_per_cu(same_f, g.IC, cbw);
-                wgs = (wgs + supers - 1) / supers * supers;
-                const int64_t per_wg = 4 / gw, streams = wgs / supers * per_wg;  // row streams
-                // Measured against the tile kernel (us, rotating buffers): [100352 x 64] . [64 x 256] 10.3 / 15.2,
-                // [401408 x 64] . [64 x 256] 30.8 / 42.9, [100352 x 256] . [256 x 64] 12.3 / 17.6, [25088 x 64] . [64 x 256]
-                // 6.2 / 6.4; about equal at K = 128 ([100352 x 128] . [128 x 256] 17.5 / 17.8, [25088 x 128] . [128 x 512]
-                // 10.3 / 10.5); behind it at K = 256 with more than 64 channels ([25088 x 256] . [256 x 128] 8.9 / 8.0,
-                // [25088 x 256] . [256 x 512] 15.5 / 12.8).
-                const bool pays = nblk * cbw >= (g.IC == 128 ? 4 : 2) * streams && (g.IC < 256 || g.OC <= 64);
-                if (regb_knob > 0 || pays) {
-                    if (nblk < streams) wgs = (nblk + per_wg - 1) / per_wg * supers;
-                    const GemmLaunch gl{(const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, (uint8_t*)t.output, Mtot, g.OC, g.IC, G,
-                                        0, 8, false, in_u8, false, out_signed ? OUT_I8 : OUT_U8, gp, rows, dst};
-                    rc = launch_gemm_regb(gl, cbw, gw, (int)wgs, s);
-                    if (rc) return rc;
-                    *kernel_name = "nce_gemm_regb";
-                    return VPX_RESULT_SUCCESS;
-                }
+            if (regb_cbw != 0) {
+                const GemmLaunch gl{(const int8_t*)t.input, (const int8_t*)wptr, t.weight_table, (uint8_t*)t.output, Mtot, g.OC, g.IC, G,
+                                    0, 4, false, in_u8, false, out_signed ? OUT_I8 : OUT_U8, gp, rows, dst};
+                rc = launch_gemm_regb(gl, regb_cbw, regb_gw, (int)regb_wgs, s);
+                if (rc) return rc;
+                *kernel_name = "nce_gemm_regb";
+                return VPX_RESULT_SUCCESS;
             }
             const int64_t t256 = gemm_tiles * G, t128 = ((Mtot + 127) / 128) * ((g.OC + 127) / 128) * G;
             const double work = (double)Mtot * (double)g.OC * (double)G;
