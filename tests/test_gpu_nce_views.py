@@ -146,6 +146,22 @@ def test_views_on_every_kernel(rt, orc, dev, family, in_kind, out_kind):
         assert name == kernel
 
 
+@pytest.mark.parametrize("knob", ["on", "wide"])
+@pytest.mark.parametrize("N,in_kind,out_kind,kernel", [
+    (2, "chan16", "chan16", "nce_gemm_regb"), (2, "dense", "chan16", "nce_gemm_regb"), (2, "chan16", "dense", "nce_gemm_regb"),
+    (1, "rows", "rows", "nce_gemm_regb"),
+    # rows that are not a fixed pitch apart, or that do not start on 16 bytes: the tile kernel
+    (2, "window", "chan16", "nce_gemm_mfma"), (2, "chan16", "window", "nce_gemm_mfma"), (2, "chan16", "chan_odd", "nce_gemm_mfma")])
+def test_views_on_the_weights_in_registers_matmul(rt, orc, dev, knob, N, in_kind, out_kind, kernel):
+    """It serves operands whose rows are a fixed pitch apart (channel slices, a band of rows of one image)."""
+    rng = np.random.default_rng(seed("regb", knob, N, in_kind, out_kind))
+    for IC, OC in ((64, 208), (128, 128), (256, 64)):
+        g = dict(N=N, H=20, W=16, IC=IC, OC=OC, KY=1, KX=1)
+        for in_u8, out_signed in ((True, False), (False, True)):
+            name = run_views(rt, orc, dev, rng, g, in_kind, out_kind, in_u8=in_u8, out_signed=out_signed, tuning=(("VPX_GEMM_REGB", knob),))
+            assert name == kernel
+
+
 @pytest.mark.parametrize("in_kind,out_kind", [("chan16", "chan_odd"), ("window_chan", "window_chan"), ("window", "chan16")])
 @pytest.mark.parametrize("family", ["gemm256", "gemm128", "tile", "stream", "rows16", "rows16_48", "gather", "gather16", "naive"])
 def test_views_with_an_fp16_output(rt, orc, dev, family, in_kind, out_kind):
